@@ -1,0 +1,94 @@
+"""Builds cumo_amd/libcumo_hip.so (gfx950) from cumo_amd/csrc with hipcc.
+
+One hipcc invocation per translation unit, run in parallel, then one link. The
+library is kept in-tree next to this file; nothing is installed.
+
+    python -m cumo_amd.build [-j N] [--force]
+"""
+import argparse
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libcumo_hip.so")
+
+ARCH = "gfx950"
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+COMMON = [
+    "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=default",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+    "-Wall", "-Wno-unused-function", "-Wno-deprecated-declarations",
+]
+# device code: no packed FP32 forms
+DEVICE = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def sources():
+    out = []
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith(".hip") or name.endswith(".cpp"):
+            out.append(os.path.join(CSRC, name))
+    return out
+
+
+def headers_mtime():
+    newest = 0.0
+    for d in (CSRC, os.path.join(ROOT, "include")):
+        for name in os.listdir(d):
+            if name.endswith((".h", ".inc")):
+                newest = max(newest, os.path.getmtime(os.path.join(d, name)))
+    return newest
+
+
+def compile_one(src, force, hdr_mtime):
+    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+    if not force and os.path.exists(obj):
+        m = os.path.getmtime(obj)
+        if m > os.path.getmtime(src) and m > hdr_mtime:
+            return obj, "", 0
+    if src.endswith(".hip"):
+        cmd = [HIPCC] + DEVICE + COMMON + ["-c", "-x", "hip", src, "-o", obj]
+    else:
+        cmd = [HIPCC] + COMMON + ["-x", "hip", "--offload-arch=" + ARCH, "-c", src, "-o", obj]
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    log = "\n".join(l for l in p.stdout.splitlines() if "packed-fp32-ops' is not a recognized feature" not in l)
+    return obj, log, p.returncode
+
+
+def build(jobs=None, force=False, verbose=True):
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    hdr = headers_mtime()
+    srcs = sources()
+    objs = []
+    failed = False
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        futs = {ex.submit(compile_one, s, force, hdr): s for s in srcs}
+        for f in concurrent.futures.as_completed(futs):
+            obj, log, rc = f.result()
+            if verbose and (log.strip() or rc):
+                print("== %s (rc=%d)\n%s" % (os.path.basename(futs[f]), rc, log), flush=True)
+            if rc:
+                failed = True
+            objs.append(obj)
+    if failed:
+        raise RuntimeError("hipcc failed")
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o", LIB] + sorted(objs)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode:
+        print(p.stdout)
+        raise RuntimeError("link failed")
+    return LIB
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("-j", type=int, default=None)
+    ap.add_argument("--force", action="store_true")
+    a = ap.parse_args()
+    print(build(a.j, a.force))

@@ -1,0 +1,304 @@
+// Bit (1 bit per element, LSB first in 32-bit words) kernels: logical ops,
+// count_true / count_false, Bit -> number.
+//
+// Replaces ext/cumo/narray/gen/tmpl_bit/{binary,unary,bit_count}_kernel.cu and
+// narray/gen/tmpl/store_bit_kernel.cu of the reference. count_* there is one
+// thread per bit and one 64-bit global atomicAdd per set bit
+// (tmpl_bit/bit_count_kernel.cu:15-24); here a contiguous run is counted by
+// popcount over whole words, reduced across the wave with shuffles and across
+// the block through LDS, and each block adds its total once. Integer addition
+// commutes, so the answer does not depend on the order the blocks arrive in.
+#include "common.h"
+#include "plan.h"
+
+#include <cstring>
+
+using namespace cumo_hip;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr unsigned kGridCap = kNumCU * 8;
+
+__device__ __forceinline__ uint32_t low_bits(unsigned n) { return n >= 32 ? 0xffffffffu : ((1u << n) - 1u); }
+
+// 32 bits of `a` starting at absolute bit position q (q may be negative at the
+// front edge or run past the end; bits outside [0, 32*nw) read as 0)
+__device__ __forceinline__ uint32_t bits_at(const CUMO_BIT_DIGIT* a, int64_t q, uint64_t nw) {
+    const int64_t w = q >> 5;  // floor
+    const unsigned sh = (unsigned)(q & 31);
+    uint32_t lo = (w >= 0 && (uint64_t)w < nw) ? a[w] : 0u;
+    if (sh == 0) return lo;
+    uint32_t hi = (w + 1 >= 0 && (uint64_t)(w + 1) < nw) ? a[w + 1] : 0u;
+    return (lo >> sh) | (hi << (32 - sh));
+}
+
+enum { B_AND, B_OR, B_XOR, B_EQ, B_COPY, B_NOT };
+
+template <int OP>
+__device__ __forceinline__ uint32_t bit_apply(uint32_t x, uint32_t y) {
+    switch (OP) {
+    case B_AND: return x & y;
+    case B_OR: return x | y;
+    case B_XOR: return x ^ y;
+    case B_EQ: return ~(x ^ y);
+    case B_COPY: return x;
+    default: return ~x;
+    }
+}
+
+// z[p3 + i] = op(x[p1 + i], y[p2 + i]) for i in [0, n): one output word per thread
+template <int OP, bool BINARY>
+__global__ __launch_bounds__(kBlock) void bit_contiguous_kernel(const CUMO_BIT_DIGIT* a1, uint64_t p1, const CUMO_BIT_DIGIT* a2,
+                                                                uint64_t p2, CUMO_BIT_DIGIT* a3, uint64_t p3, uint64_t n) {
+    const uint64_t nw1 = (p1 + n + 31) >> 5, nw2 = (p2 + n + 31) >> 5, nw3 = (p3 + n + 31) >> 5;
+    for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < nw3; w += (uint64_t)gridDim.x * kBlock) {
+        // element index of bit 0 of this output word (negative inside the first word)
+        const int64_t e0 = (int64_t)(w << 5) - (int64_t)p3;
+        const uint32_t x = bits_at(a1, e0 + (int64_t)p1, nw1);
+        const uint32_t y = BINARY ? bits_at(a2, e0 + (int64_t)p2, nw2) : 0u;
+        const uint32_t z = bit_apply<OP>(x, y);
+        const unsigned lo = (w == 0) ? (unsigned)p3 : 0u;
+        const uint64_t endbit = p3 + n;
+        const unsigned hi = ((w + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (w << 5));
+        const uint32_t mask = low_bits(hi) & ~low_bits(lo);
+        // one thread owns a word, so the shared edge words need no atomic
+        if (mask == 0xffffffffu) a3[w] = z;
+        else a3[w] = (z & mask) | (a3[w] & ~mask);
+    }
+}
+
+struct BitNd {
+    int ndim;
+    uint64_t total;
+    uint64_t shape[kMaxDim];
+};
+
+// bit position / byte offset of flat element i of an operand that is strided or
+// indexed per dimension
+__device__ __forceinline__ int64_t stridx_offset(const cumo_stridx_t* sdx, const BitNd& nd, uint64_t i) {
+    int64_t off = 0;
+    for (int d = nd.ndim - 1; d >= 0; --d) {
+        uint64_t k;
+        if (d == 0) {
+            k = i;
+        } else {
+            const uint64_t q = i / nd.shape[d];
+            k = i - q * nd.shape[d];
+            i = q;
+        }
+        const cumo_stridx_t s = sdx[d];
+        if (s.stride & 1) off += (s.stride >> 1) * (int64_t)k;
+        else off += (int64_t)s.index[k];
+    }
+    return off;
+}
+
+__device__ __forceinline__ uint32_t load_bit(const CUMO_BIT_DIGIT* a, uint64_t pos) { return (a[pos >> 5] >> (pos & 31)) & 1u; }
+
+__device__ __forceinline__ void store_bit_atomic(CUMO_BIT_DIGIT* a, uint64_t pos, uint32_t v) {
+    const uint32_t bit = 1u << (pos & 31);
+    if (v) atomicOr(&a[pos >> 5], bit);
+    else atomicAnd(&a[pos >> 5], ~bit);
+}
+
+template <int OP, bool BINARY>
+__global__ __launch_bounds__(kBlock) void bit_generic_kernel(cumo_na_bit_iarray_stridx_t a1, cumo_na_bit_iarray_stridx_t a2,
+                                                             cumo_na_bit_iarray_stridx_t a3, BitNd nd) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < nd.total; i += (uint64_t)gridDim.x * kBlock) {
+        const uint32_t x = load_bit(a1.ptr, a1.pos + (uint64_t)stridx_offset(a1.stridx, nd, i));
+        const uint32_t y = BINARY ? load_bit(a2.ptr, a2.pos + (uint64_t)stridx_offset(a2.stridx, nd, i)) : 0u;
+        store_bit_atomic(a3.ptr, a3.pos + (uint64_t)stridx_offset(a3.stridx, nd, i), bit_apply<OP>(x, y) & 1u);
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void store_bit_kernel(cumo_na_iarray_stridx_t dst, cumo_na_bit_iarray_stridx_t src, BitNd nd) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < nd.total; i += (uint64_t)gridDim.x * kBlock) {
+        const uint32_t x = load_bit(src.ptr, src.pos + (uint64_t)stridx_offset(src.stridx, nd, i));
+        *reinterpret_cast<T*>(dst.ptr + stridx_offset(dst.stridx, nd, i)) = (T)x;
+    }
+}
+
+// ---- counting -------------------------------------------------------------------
+__device__ __forceinline__ uint64_t block_sum_u64(uint64_t v) {
+    __shared__ uint64_t wave_sum[kBlock / 64];
+    for (unsigned d = 32; d > 0; d >>= 1) {
+        const uint32_t lo = __shfl_down((uint32_t)v, d);
+        const uint32_t hi = __shfl_down((uint32_t)(v >> 32), d);
+        v += ((uint64_t)hi << 32) | lo;
+    }
+    if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = v;
+    __syncthreads();
+    uint64_t t = 0;
+    if (threadIdx.x == 0) {
+        for (int w = 0; w < kBlock / 64; ++w) t += wave_sum[w];
+    }
+    return t;  // valid in thread 0
+}
+
+// bits [p1, p1 + n) of a, step 1: whole words, edges masked
+template <bool COUNT_FALSE>
+__global__ __launch_bounds__(kBlock) void bit_count_words_kernel(const CUMO_BIT_DIGIT* a, uint64_t p1, uint64_t n, unsigned long long* out) {
+    const uint64_t w0 = p1 >> 5;
+    const uint64_t endbit = p1 + n;
+    const uint64_t w1 = (endbit + 31) >> 5;
+    uint64_t c = 0;
+    for (uint64_t w = w0 + (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < w1; w += (uint64_t)gridDim.x * kBlock) {
+        uint32_t x = a[w];
+        if (COUNT_FALSE) x = ~x;
+        const unsigned lo = (w == w0) ? (unsigned)(p1 & 31) : 0u;
+        const unsigned hi = ((w + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (w << 5));
+        x &= low_bits(hi) & ~low_bits(lo);
+        c += (uint64_t)__popc(x);
+    }
+    const uint64_t t = block_sum_u64(c);
+    if (threadIdx.x == 0 && t) atomicAdd(out, (unsigned long long)t);
+}
+
+// any stride or an index array, all into one counter
+template <bool COUNT_FALSE>
+__global__ __launch_bounds__(kBlock) void bit_count_gather_kernel(const CUMO_BIT_DIGIT* a, uint64_t p1, int64_t s1, const size_t* idx1,
+                                                                  uint64_t n, unsigned long long* out) {
+    uint64_t c = 0;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) {
+        const uint64_t pos = idx1 ? (p1 + idx1[i]) : (uint64_t)((int64_t)p1 + (int64_t)i * s1);
+        const uint32_t x = load_bit(a, pos);
+        c += COUNT_FALSE ? (x == 0) : (x != 0);
+    }
+    const uint64_t t = block_sum_u64(c);
+    if (threadIdx.x == 0 && t) atomicAdd(out, (unsigned long long)t);
+}
+
+// element i goes to its own counter at p2 + i*s2 (s2 != 0), so nothing is shared
+template <bool COUNT_FALSE>
+__global__ __launch_bounds__(kBlock) void bit_count_scatter_kernel(const CUMO_BIT_DIGIT* a, uint64_t p1, int64_t s1, const size_t* idx1,
+                                                                   char* p2, int64_t s2, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) {
+        const uint64_t pos = idx1 ? (p1 + idx1[i]) : (uint64_t)((int64_t)p1 + (int64_t)i * s1);
+        const uint32_t x = load_bit(a, pos);
+        if (COUNT_FALSE ? (x == 0) : (x != 0)) *reinterpret_cast<uint64_t*>(p2 + (int64_t)i * s2) += 1;
+    }
+}
+
+unsigned grid_for(uint64_t items) {
+    uint64_t g = (items + kBlock - 1) / kBlock;
+    if (g > kGridCap) g = kGridCap;
+    if (g == 0) g = 1;
+    return (unsigned)g;
+}
+
+BitNd make_nd(const cumo_na_indexer_t* indexer) {
+    BitNd nd;
+    std::memset(&nd, 0, sizeof(nd));
+    nd.ndim = indexer->ndim;
+    nd.total = indexer->total_size;
+    for (int d = 0; d < indexer->ndim; ++d) nd.shape[d] = indexer->shape[d];
+    return nd;
+}
+
+template <int OP, bool BINARY>
+void launch_contiguous(CUMO_BIT_DIGIT* a1, size_t p1, CUMO_BIT_DIGIT* a2, size_t p2, CUMO_BIT_DIGIT* a3, size_t p3, uint64_t n) {
+    if (n == 0) return;
+    const uint64_t nw3 = (p3 + n + 31) >> 5;
+    hipLaunchKernelGGL((bit_contiguous_kernel<OP, BINARY>), dim3(grid_for(nw3)), dim3(kBlock), 0, current_stream(), a1, (uint64_t)p1, a2,
+                       (uint64_t)p2, a3, (uint64_t)p3, n);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+bool flat_stride1(const cumo_na_bit_iarray_stridx_t* a, int ndim) {
+    return ndim == 1 && CUMO_SDX_IS_STRIDE(a->stridx[0]) && CUMO_SDX_GET_STRIDE(a->stridx[0]) == 1;
+}
+
+template <int OP, bool BINARY>
+void launch_generic(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_bit_iarray_stridx_t* a3,
+                    cumo_na_indexer_t* indexer) {
+    if (indexer->total_size == 0) return;
+    // the host iterator already routes the flat case to the word kernel
+    // (tmpl_bit/binary.c:17-31); do the same for callers that do not
+    if (flat_stride1(a1, indexer->ndim) && (!BINARY || flat_stride1(a2, indexer->ndim)) && flat_stride1(a3, indexer->ndim)) {
+        launch_contiguous<OP, BINARY>(a1->ptr + a1->pos / 32, a1->pos % 32, BINARY ? a2->ptr + a2->pos / 32 : nullptr,
+                                      BINARY ? a2->pos % 32 : 0, a3->ptr + a3->pos / 32, a3->pos % 32, indexer->total_size);
+        return;
+    }
+    BitNd nd = make_nd(indexer);
+    hipLaunchKernelGGL((bit_generic_kernel<OP, BINARY>), dim3(grid_for(nd.total)), dim3(kBlock), 0, current_stream(), *a1,
+                       BINARY ? *a2 : *a1, *a3, nd);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+template <bool COUNT_FALSE>
+void launch_count(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, ssize_t s1, size_t* idx1, ssize_t s2, uint64_t n) {
+    if (n == 0) return;
+    hipStream_t st = current_stream();
+    if (s2 != 0) {
+        hipLaunchKernelGGL((bit_count_scatter_kernel<COUNT_FALSE>), dim3(grid_for(n)), dim3(kBlock), 0, st, a1, (uint64_t)p1, (int64_t)s1, idx1,
+                           p2, (int64_t)s2, n);
+    } else if (!idx1 && s1 == 1) {
+        hipLaunchKernelGGL((bit_count_words_kernel<COUNT_FALSE>), dim3(grid_for((n + 31) / 32 + 1)), dim3(kBlock), 0, st, a1, (uint64_t)p1, n,
+                           (unsigned long long*)p2);
+    } else {
+        hipLaunchKernelGGL((bit_count_gather_kernel<COUNT_FALSE>), dim3(grid_for(n)), dim3(kBlock), 0, st, a1, (uint64_t)p1, (int64_t)s1, idx1,
+                           n, (unsigned long long*)p2);
+    }
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+}  // namespace
+
+#define CUMO_DEF_BIT_BINARY(name, OP)                                                                                         \
+    extern "C" void cumo_iter_bit_##name##_kernel_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2,    \
+                                                         cumo_na_bit_iarray_stridx_t* a3, cumo_na_indexer_t* indexer) {       \
+        launch_generic<OP, true>(a1, a2, a3, indexer);                                                                        \
+    }                                                                                                                         \
+    extern "C" void cumo_iter_bit_##name##_contiguous_kernel_launch(CUMO_BIT_DIGIT* a1, size_t p1, CUMO_BIT_DIGIT* a2,        \
+                                                                    size_t p2, CUMO_BIT_DIGIT* a3, size_t p3, uint64_t n) {   \
+        launch_contiguous<OP, true>(a1, p1, a2, p2, a3, p3, n);                                                               \
+    }
+#define CUMO_DEF_BIT_UNARY(name, OP)                                                                                          \
+    extern "C" void cumo_iter_bit_##name##_kernel_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a3,    \
+                                                         cumo_na_indexer_t* indexer) {                                        \
+        launch_generic<OP, false>(a1, nullptr, a3, indexer);                                                                  \
+    }                                                                                                                         \
+    extern "C" void cumo_iter_bit_##name##_contiguous_kernel_launch(CUMO_BIT_DIGIT* a1, size_t p1, CUMO_BIT_DIGIT* a3,        \
+                                                                    size_t p3, uint64_t n) {                                  \
+        launch_contiguous<OP, false>(a1, p1, nullptr, 0, a3, p3, n);                                                          \
+    }
+CUMO_DEF_BIT_BINARY(and, B_AND)
+CUMO_DEF_BIT_BINARY(or, B_OR)
+CUMO_DEF_BIT_BINARY(xor, B_XOR)
+CUMO_DEF_BIT_BINARY(eq, B_EQ)
+CUMO_DEF_BIT_UNARY(copy, B_COPY)
+CUMO_DEF_BIT_UNARY(not, B_NOT)
+
+#define CUMO_DEF_BIT_COUNT(name, CF)                                                                                          \
+    extern "C" void cumo_iter_bit_##name##_index_kernel_launch(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, size_t* idx1,         \
+                                                               uint64_t n) {                                                  \
+        launch_count<CF>(p1, p2, a1, 0, idx1, 0, n);                                                                          \
+    }                                                                                                                         \
+    extern "C" void cumo_iter_bit_##name##_stride_kernel_launch(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, ssize_t s1,          \
+                                                                uint64_t n) {                                                 \
+        launch_count<CF>(p1, p2, a1, s1, nullptr, 0, n);                                                                      \
+    }                                                                                                                         \
+    extern "C" void cumo_iter_bit_##name##_index_stride_kernel_launch(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, size_t* idx1,  \
+                                                                      ssize_t s2, uint64_t n) {                               \
+        launch_count<CF>(p1, p2, a1, 0, idx1, s2, n);                                                                         \
+    }                                                                                                                         \
+    extern "C" void cumo_iter_bit_##name##_stride_stride_kernel_launch(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, ssize_t s1,   \
+                                                                       ssize_t s2, uint64_t n) {                              \
+        launch_count<CF>(p1, p2, a1, s1, nullptr, s2, n);                                                                     \
+    }
+CUMO_DEF_BIT_COUNT(count_true, false)
+CUMO_DEF_BIT_COUNT(count_false, true)
+
+#define CUMO_DEF_STORE_BIT(t, c)                                                                                              \
+    extern "C" void cumo_iter_##t##_store_bit_kernel_launch(cumo_na_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2,     \
+                                                            cumo_na_indexer_t* indexer) {                                     \
+        if (indexer->total_size == 0) return;                                                                                 \
+        BitNd nd = make_nd(indexer);                                                                                          \
+        hipLaunchKernelGGL((store_bit_kernel<c>), dim3(grid_for(nd.total)), dim3(kBlock), 0, current_stream(), *a1, *a2, nd); \
+        cumo_cuda_runtime_check_kernel_launch();                                                                              \
+    }
+CUMO_DEF_STORE_BIT(sfloat, float)
+CUMO_DEF_STORE_BIT(dfloat, double)
+CUMO_DEF_STORE_BIT(int32, int32_t)

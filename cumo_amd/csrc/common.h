@@ -1,0 +1,29 @@
+// Shared host-side plumbing of the library: error reporting, the per-thread
+// stream, and the launch-check helper every launcher ends with.
+#ifndef CUMO_HIP_COMMON_H
+#define CUMO_HIP_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "cumo_hip.h"
+
+namespace cumo_hip {
+
+// Reports an error to the installed handler (which may not return) or latches
+// it for cumo_hip_last_error. Callers must hold no C++ object with a
+// destructor when they call it: a Ruby handler raises with longjmp.
+void report_error(int kind, int hip_status, const char* message);
+void report_hip_error(hipError_t status, const char* what);
+
+hipStream_t current_stream();
+
+static inline bool hip_ok(hipError_t status, const char* what) {
+    if (status == hipSuccess) return true;
+    report_hip_error(status, what);
+    return false;
+}
+
+}  // namespace cumo_hip
+
+#endif

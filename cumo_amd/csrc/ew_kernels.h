@@ -1,0 +1,505 @@
+// Elementwise kernels for gfx950 and the launcher template that drives them.
+//
+// These replace every expansion of the reference's elementwise templates
+// (ext/cumo/narray/gen/tmpl/{binary,unary,unary2,unary_s,binary_s,cond_binary,
+// cond_unary,store_from,fill}_kernel.cu). The reference expands each template
+// once per ndim 0..8 and decomposes a flat index with 64-bit divides per
+// element; here there are two kernels:
+//
+//  ew_rows_kernel       lanes run along the one dimension every operand walks
+//                       fastest (or is broadcast along); the other dimensions
+//                       are decomposed once per row per thread, never per
+//                       element. With one dimension left it is the plain
+//                       streaming kernel. 128-bit accesses when the planner
+//                       found every operand aligned for them.
+//  ew_transpose_kernel  an input walks a different dimension fastest than the
+//                       output does (a transposed view): a 64-wide tile goes
+//                       through LDS so that both the read and the write are
+//                       along memory.
+//
+// A Bit result is written by whole 32-bit words assembled across lanes;
+// only words shared with a neighbouring row fall back to atomics
+// (the reference does two atomics per element: include/cumo/template_kernel.h:26-35).
+#ifndef CUMO_HIP_EW_KERNELS_H
+#define CUMO_HIP_EW_KERNELS_H
+
+#include "common.h"
+#include "plan.h"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace cumo_hip {
+
+constexpr int kEwBlock = 256;
+constexpr int kEwUnroll = 4;
+
+struct EwKParams {
+    uint64_t inner;      // extent of the fast dim
+    uint64_t rows;       // product of the other dims
+    uint64_t col_tiles;  // tiles along the fast dim
+    uint64_t n_tiles;
+    int nouter;
+    int tx_bits;         // 2^tx_bits lanes along the fast dim, the rest of the block along rows
+    int use_scalar;      // 0: both inputs are arrays, 1: y = sv, 2: x = sv
+    int small_rows;      // rows < 2^32: decompose with 32-bit divides
+    int* flag;           // pinned host word for rejected elements (may be NULL)
+    uint64_t out_bitpos; // Bit output: position of element 0
+    uint64_t oshape[kMaxDim - 1];
+    int64_t ostep[3][kMaxDim - 1];  // [in1, in2, out]; bits for a Bit output
+    int64_t istep[3];
+    char* ptr[3];
+};
+
+template <class T, int N>
+struct alignas((sizeof(T) * N) > 16 ? 16 : (sizeof(T) * N)) VecT {
+    T v[N];
+};
+
+template <class T, int VEC>
+__device__ __forceinline__ void ew_load(const char* base, int64_t istep, int64_t col, T (&out)[VEC]) {
+    if (istep == 0) {
+        T v = *reinterpret_cast<const T*>(base);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = v;
+    } else if (VEC > 1) {
+        const VecT<T, VEC> v = *reinterpret_cast<const VecT<T, VEC>*>(base + col * (int64_t)sizeof(T));
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = v.v[j];
+    } else {
+        out[0] = *reinterpret_cast<const T*>(base + col * istep);
+    }
+}
+
+// Stores the VEC result bits of every lane of the wave. Every lane of the
+// wave must call it (inactive lanes with active == false).
+//   P      bit position of the lane's first bit
+//   bits   the lane's results, bit j = element j
+//   vmask  which of them exist
+template <int VEC>
+__device__ __forceinline__ void ew_store_bits(CUMO_BIT_DIGIT* base, uint64_t P, uint32_t bits, uint32_t vmask, bool active) {
+    constexpr unsigned G = 32 / VEC;  // lanes per word
+    const unsigned lane = __lane_id();
+    const unsigned want_sh = (lane % G) * VEC;
+    const uint64_t actmask = __ballot(active);
+    if (actmask == 0) return;
+    const uint64_t word = P >> 5;
+    const unsigned gbase = lane & ~(G - 1);
+    const uint64_t gmask = (actmask >> gbase) & ((1ull << G) - 1);
+    const int leader = gmask ? (int)(gbase + __builtin_ctzll(gmask)) : (int)lane;
+    const uint32_t lw_lo = __shfl((uint32_t)word, leader);
+    const uint32_t lw_hi = __shfl((uint32_t)(word >> 32), leader);
+    const bool fits = !active || (((unsigned)(P & 31) == want_sh) && lw_lo == (uint32_t)word && lw_hi == (uint32_t)(word >> 32));
+    const bool fast = __ballot(!fits) == 0;
+    if (fast) {
+        uint32_t w = active ? ((bits & vmask) << want_sh) : 0u;
+        uint32_t m = active ? (vmask << want_sh) : 0u;
+#pragma unroll
+        for (unsigned d = 1; d < G; d <<= 1) {
+            w |= __shfl_xor(w, d);
+            m |= __shfl_xor(m, d);
+        }
+        if (active && (int)lane == leader) {
+            if (m == 0xffffffffu) {
+                base[word] = w;
+            } else {
+                // the rest of the word belongs to a neighbouring row or to elements
+                // outside the view
+                atomicAnd(&base[word], ~m);
+                atomicOr(&base[word], w);
+            }
+        }
+    } else if (active) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            if ((vmask >> j) & 1u) {
+                const uint64_t q = P + j;
+                const uint32_t bit = 1u << (q & 31);
+                if ((bits >> j) & 1u) atomicOr(&base[q >> 5], bit);
+                else atomicAnd(&base[q >> 5], ~bit);
+            }
+        }
+    }
+}
+
+template <int NOPS>
+__device__ __forceinline__ void ew_row_offsets(const EwKParams& p, uint64_t row, int64_t (&off)[3]) {
+    off[0] = off[1] = off[2] = 0;
+    if (p.nouter == 0) return;
+    if (p.small_rows) {
+        uint32_t r = (uint32_t)row;
+        for (int d = p.nouter - 1; d >= 1; --d) {
+            const uint32_t n = (uint32_t)p.oshape[d];
+            const uint32_t q = r / n;
+            const uint32_t i = r - q * n;
+            r = q;
+            off[0] += (int64_t)i * p.ostep[0][d];
+            if (NOPS > 2) off[1] += (int64_t)i * p.ostep[1][d];
+            off[2] += (int64_t)i * p.ostep[2][d];
+        }
+        off[0] += (int64_t)r * p.ostep[0][0];
+        if (NOPS > 2) off[1] += (int64_t)r * p.ostep[1][0];
+        off[2] += (int64_t)r * p.ostep[2][0];
+    } else {
+        uint64_t r = row;
+        for (int d = p.nouter - 1; d >= 1; --d) {
+            const uint64_t n = p.oshape[d];
+            const uint64_t q = r / n;
+            const uint64_t i = r - q * n;
+            r = q;
+            off[0] += (int64_t)i * p.ostep[0][d];
+            if (NOPS > 2) off[1] += (int64_t)i * p.ostep[1][d];
+            off[2] += (int64_t)i * p.ostep[2][d];
+        }
+        off[0] += (int64_t)r * p.ostep[0][0];
+        if (NOPS > 2) off[1] += (int64_t)r * p.ostep[1][0];
+        off[2] += (int64_t)r * p.ostep[2][0];
+    }
+}
+
+// Op contract:
+//   typedef A, B (input element types), R (output element type; uint32_t 0/1 for BIT_OUT), S (scalar type)
+//   static constexpr int NIN (0, 1 or 2); static constexpr bool BIT_OUT, CHECKED
+//   __device__ bool operator()(A x, B y, R& z) const   -- false: reject the element (do not store, raise flag)
+template <class Op, int VEC>
+__global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, typename Op::S sv) {
+    typedef typename Op::A A;
+    typedef typename Op::B B;
+    typedef typename Op::R R;
+    constexpr int NIN = Op::NIN;
+    constexpr bool TWO = (NIN == 2);
+
+    const unsigned TX = 1u << p.tx_bits;
+    const unsigned TY = kEwBlock >> p.tx_bits;
+    const unsigned tx = threadIdx.x & (TX - 1);
+    const unsigned ty = threadIdx.x >> p.tx_bits;
+    const uint64_t tile_cols = (uint64_t)TX * VEC * kEwUnroll;
+    const int64_t inner = (int64_t)p.inner;
+    const bool two_arrays = TWO && p.use_scalar == 0;
+
+    for (uint64_t tile = blockIdx.x; tile < p.n_tiles; tile += gridDim.x) {
+        uint64_t rt, ct;
+        if (p.col_tiles == 1) {
+            rt = tile;
+            ct = 0;
+        } else {
+            rt = tile / p.col_tiles;
+            ct = tile - rt * p.col_tiles;
+        }
+        const uint64_t row = rt * TY + ty;
+        const bool row_ok = row < p.rows;
+        int64_t off[3];
+        ew_row_offsets<TWO ? 3 : 2>(p, row_ok ? row : 0, off);
+
+        int64_t lead = 0;
+        if (Op::BIT_OUT && VEC == 1) lead = (int64_t)((p.out_bitpos + (uint64_t)off[2]) & 31);
+        const int64_t col0 = (int64_t)(ct * tile_cols) + (int64_t)tx * VEC - lead;
+
+        const char* b0 = p.ptr[0] + off[0];
+        const char* b1 = p.ptr[1] + off[1];
+
+        A xv[kEwUnroll][VEC];
+        B yv[kEwUnroll][VEC];
+        int nval[kEwUnroll];  // how many of the VEC elements exist
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; ++u) {
+            const int64_t col = col0 + (int64_t)u * TX * VEC;
+            int nv = 0;
+            if (row_ok && col >= 0 && col < inner) nv = (col + VEC <= inner) ? VEC : (int)(inner - col);
+            nval[u] = nv;
+            if (nv == VEC) {
+                if (NIN >= 1) ew_load<A, VEC>(b0, p.istep[0], col, xv[u]);
+                if (two_arrays) ew_load<B, VEC>(b1, p.istep[1], col, yv[u]);
+            } else if (nv > 0) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    if (j < nv) {
+                        if (NIN >= 1) xv[u][j] = *reinterpret_cast<const A*>(b0 + (col + j) * p.istep[0]);
+                        if (two_arrays) yv[u][j] = *reinterpret_cast<const B*>(b1 + (col + j) * p.istep[1]);
+                    }
+                }
+            }
+        }
+
+#pragma unroll
+        for (int u = 0; u < kEwUnroll; ++u) {
+            const int64_t col = col0 + (int64_t)u * TX * VEC;
+            const int nv = nval[u];
+            R zv[VEC];
+            uint32_t okmask = 0;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if (j < nv) {
+                    A x = (NIN >= 1) ? xv[u][j] : A();
+                    B y = B();
+                    if (TWO) {
+                        if (p.use_scalar == 0) y = yv[u][j];
+                        else if (p.use_scalar == 1) y = (B)sv;
+                        else { y = (B)x; x = (A)sv; }
+                    }
+                    R z = R();
+                    if (op(x, y, z)) okmask |= 1u << j;
+                    zv[j] = z;
+                }
+            }
+            if (Op::BIT_OUT) {
+                uint32_t bits = 0;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) if (j < nv && zv[j]) bits |= 1u << j;
+                const uint64_t P = p.out_bitpos + (uint64_t)off[2] + (uint64_t)(col * p.istep[2]);
+                ew_store_bits<VEC>(reinterpret_cast<CUMO_BIT_DIGIT*>(p.ptr[2]), P, bits, (nv >= VEC) ? ((1u << VEC) - 1u) : ((1u << nv) - 1u), nv > 0);
+            } else if (nv > 0) {
+                char* o = p.ptr[2] + off[2];
+                const uint32_t full = (1u << VEC) - 1u;
+                if (Op::CHECKED && okmask != ((nv >= VEC) ? full : ((1u << nv) - 1u))) {
+                    if (p.flag) *p.flag = 1;
+                }
+                if (VEC > 1 && nv == VEC && okmask == full && p.istep[2] != 0) {
+                    VecT<R, VEC> v;
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) v.v[j] = zv[j];
+                    *reinterpret_cast<VecT<R, VEC>*>(o + col * (int64_t)sizeof(R)) = v;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        if (j < nv && ((okmask >> j) & 1u)) *reinterpret_cast<R*>(o + (col + j) * p.istep[2]) = zv[j];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Transposed-operand kernel. Dims: outer..., G (second last), F (last, the
+// output's fast dim). An input whose step along G is smaller than along F is
+// read with lanes along G into LDS and picked up transposed.
+// ---------------------------------------------------------------------------
+struct EwTParams {
+    uint64_t nf, ng;          // extents of F and G
+    uint64_t f_tiles, g_tiles, n_tiles;
+    int nouter;
+    int use_scalar;
+    int tr[2];                // input k goes through LDS
+    int* flag;
+    uint64_t oshape[kMaxDim - 2];
+    int64_t ostep[3][kMaxDim - 2];
+    int64_t fstep[3], gstep[3];
+    char* ptr[3];
+};
+
+template <class Op, int TG>
+__global__ __launch_bounds__(kEwBlock) void ew_transpose_kernel(EwTParams p, Op op, typename Op::S sv) {
+    typedef typename Op::A A;
+    typedef typename Op::B B;
+    typedef typename Op::R R;
+    constexpr int NIN = Op::NIN;
+    constexpr bool TWO = (NIN == 2);
+    constexpr int TF = 64;
+    __shared__ A tile_a[TG][TF + 1];
+    __shared__ B tile_b[TWO ? TG : 1][TF + 1];
+
+    const bool two_arrays = TWO && p.use_scalar == 0;
+    for (uint64_t tile = blockIdx.x; tile < p.n_tiles; tile += gridDim.x) {
+        uint64_t t = tile;
+        const uint64_t ft = t % p.f_tiles; t /= p.f_tiles;
+        const uint64_t gt = t % p.g_tiles; t /= p.g_tiles;
+        int64_t off[3] = {0, 0, 0};
+        for (int d = p.nouter - 1; d >= 0; --d) {
+            const uint64_t n = p.oshape[d];
+            const uint64_t i = (d == 0) ? t : (t % n);
+            t = (d == 0) ? 0 : (t / n);
+            off[0] += (int64_t)i * p.ostep[0][d];
+            off[1] += (int64_t)i * p.ostep[1][d];
+            off[2] += (int64_t)i * p.ostep[2][d];
+        }
+        const uint64_t f0 = ft * TF, g0 = gt * TG;
+
+        // phase 1: transposed inputs, lanes along G
+        {
+            const unsigned lg = threadIdx.x % TG;
+            const unsigned lf0 = threadIdx.x / TG;
+            constexpr unsigned FSTEP = kEwBlock / TG;
+            const uint64_t g = g0 + lg;
+            if (p.tr[0]) {
+#pragma unroll 4
+                for (unsigned lf = lf0; lf < TF; lf += FSTEP) {
+                    const uint64_t f = f0 + lf;
+                    if (g < p.ng && f < p.nf)
+                        tile_a[lg][lf] = *reinterpret_cast<const A*>(p.ptr[0] + off[0] + (int64_t)g * p.gstep[0] + (int64_t)f * p.fstep[0]);
+                }
+            }
+            if (two_arrays && p.tr[1]) {
+#pragma unroll 4
+                for (unsigned lf = lf0; lf < TF; lf += FSTEP) {
+                    const uint64_t f = f0 + lf;
+                    if (g < p.ng && f < p.nf)
+                        tile_b[TWO ? lg : 0][lf] = *reinterpret_cast<const B*>(p.ptr[1] + off[1] + (int64_t)g * p.gstep[1] + (int64_t)f * p.fstep[1]);
+                }
+            }
+        }
+        __syncthreads();
+        // phase 2: lanes along F
+        {
+            const unsigned lf = threadIdx.x % TF;
+            const unsigned lg0 = threadIdx.x / TF;
+            constexpr unsigned GSTEP = kEwBlock / TF;
+            const uint64_t f = f0 + lf;
+#pragma unroll 4
+            for (unsigned lg = lg0; lg < TG; lg += GSTEP) {
+                const uint64_t g = g0 + lg;
+                if (g < p.ng && f < p.nf) {
+                    A x = A();
+                    B y = B();
+                    if (NIN >= 1) {
+                        x = p.tr[0] ? tile_a[lg][lf]
+                                    : *reinterpret_cast<const A*>(p.ptr[0] + off[0] + (int64_t)g * p.gstep[0] + (int64_t)f * p.fstep[0]);
+                    }
+                    if (TWO) {
+                        if (p.use_scalar == 0) {
+                            y = p.tr[1] ? tile_b[TWO ? lg : 0][lf]
+                                        : *reinterpret_cast<const B*>(p.ptr[1] + off[1] + (int64_t)g * p.gstep[1] + (int64_t)f * p.fstep[1]);
+                        } else if (p.use_scalar == 1) {
+                            y = (B)sv;
+                        } else {
+                            y = (B)x;
+                            x = (A)sv;
+                        }
+                    }
+                    R z = R();
+                    if (op(x, y, z)) {
+                        *reinterpret_cast<R*>(p.ptr[2] + off[2] + (int64_t)g * p.gstep[2] + (int64_t)f * p.fstep[2]) = z;
+                    } else if (p.flag) {
+                        *p.flag = 1;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+static inline unsigned ew_grid_cap() {
+    static unsigned cap = 0;
+    if (cap == 0) {
+        const char* e = std::getenv("CUMO_HIP_EW_GRID_CAP");
+        cap = e ? (unsigned)std::strtoul(e, nullptr, 10) : 0;
+        if (cap == 0) cap = (unsigned)kNumCU * 16;
+    }
+    return cap;
+}
+
+// in1/in2 may be NULL (NIN < 2 or the scalar form). out_bit is non-NULL for a
+// Bit result, in which case out is ignored.
+template <class Op>
+static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t* in2, const cumo_na_iarray_t* out,
+                      const cumo_na_bit_iarray_t* out_bit, const cumo_na_indexer_t* indexer, typename Op::S sv, int use_scalar,
+                      int* flag) {
+    typedef typename Op::A A;
+    typedef typename Op::B B;
+    typedef typename Op::R R;
+    EwOperand ops[3];
+    int slot[3];
+    int nops = 0;
+    if (Op::NIN >= 1 && in1) { ops[nops] = EwOperand{in1->ptr, in1->step, (int)sizeof(A), 0}; slot[nops++] = 0; }
+    if (Op::NIN >= 2 && in2 && use_scalar == 0) { ops[nops] = EwOperand{in2->ptr, in2->step, (int)sizeof(B), 0}; slot[nops++] = 1; }
+    if (Op::BIT_OUT) {
+        ops[nops] = EwOperand{(const char*)out_bit->ptr, out_bit->step, 0, out_bit->pos};
+    } else {
+        ops[nops] = EwOperand{out->ptr, out->step, (int)sizeof(R), 0};
+    }
+    slot[nops++] = 2;
+
+    EwPlan plan;
+    plan_elementwise(indexer->ndim, indexer->shape, nops, ops, &plan);
+    if (plan.kind == EW_EMPTY) return;
+    hipStream_t stream = current_stream();
+
+    if (plan.kind == EW_TRANSPOSE) {
+        EwTParams tp;
+        std::memset(&tp, 0, sizeof(tp));
+        const int n = plan.ndim;
+        tp.nf = plan.shape[n - 1];
+        tp.ng = plan.shape[n - 2];
+        tp.nouter = n - 2;
+        tp.use_scalar = use_scalar;
+        tp.flag = flag;
+        constexpr int TG = (sizeof(A) >= 8 || sizeof(B) >= 8) ? 32 : 64;
+        tp.f_tiles = (tp.nf + 63) / 64;
+        tp.g_tiles = (tp.ng + TG - 1) / TG;
+        uint64_t outer = 1;
+        for (int d = 0; d < n - 2; ++d) { tp.oshape[d] = plan.shape[d]; outer *= plan.shape[d]; }
+        tp.n_tiles = tp.f_tiles * tp.g_tiles * outer;
+        for (int o = 0; o < nops; ++o) {
+            const int s = slot[o];
+            tp.ptr[s] = const_cast<char*>(ops[o].ptr);
+            tp.fstep[s] = plan.step[o][n - 1];
+            tp.gstep[s] = plan.step[o][n - 2];
+            for (int d = 0; d < n - 2; ++d) tp.ostep[s][d] = plan.step[o][d];
+            if (s < 2) {
+                const uint64_t gs = tp.gstep[s] < 0 ? -tp.gstep[s] : tp.gstep[s];
+                const uint64_t fs = tp.fstep[s] < 0 ? -tp.fstep[s] : tp.fstep[s];
+                tp.tr[s] = (gs != 0 && fs != 0 && gs < fs) ? 1 : 0;
+            }
+        }
+        uint64_t grid = tp.n_tiles;
+        if (grid > 0x7fffffffull) grid = 0x7fffffffull;
+        hipLaunchKernelGGL((ew_transpose_kernel<Op, TG>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, tp, op, sv);
+        cumo_cuda_runtime_check_kernel_launch();
+        return;
+    }
+
+    EwKParams kp;
+    std::memset(&kp, 0, sizeof(kp));
+    const int n = plan.ndim;
+    kp.inner = plan.shape[n - 1];
+    kp.rows = plan.total / kp.inner;
+    kp.nouter = n - 1;
+    kp.use_scalar = use_scalar;
+    kp.flag = flag;
+    kp.small_rows = kp.rows < 0xffffffffull ? 1 : 0;
+    for (int d = 0; d < n - 1; ++d) kp.oshape[d] = plan.shape[d];
+    for (int o = 0; o < nops; ++o) {
+        const int s = slot[o];
+        kp.ptr[s] = const_cast<char*>(ops[o].ptr);
+        kp.istep[s] = plan.step[o][n - 1];
+        for (int d = 0; d < n - 1; ++d) kp.ostep[s][d] = plan.step[o][d];
+    }
+    if (Op::BIT_OUT) kp.out_bitpos = out_bit->pos;
+
+    const int vec = plan.vec;
+    const bool shift = Op::BIT_OUT && vec == 1;
+    const uint64_t span = kp.inner + (shift ? 31 : 0);
+    uint64_t lanes_needed = (span + vec - 1) / vec;
+    int tx_bits = 0;
+    while (tx_bits < 8 && (1ull << tx_bits) < lanes_needed) ++tx_bits;
+    if (kp.rows == 1) tx_bits = 8;
+    kp.tx_bits = tx_bits;
+    const uint64_t tile_cols = (1ull << tx_bits) * vec * kEwUnroll;
+    const uint64_t TY = (uint64_t)kEwBlock >> tx_bits;
+    kp.col_tiles = (span + tile_cols - 1) / tile_cols;
+    const uint64_t row_tiles = (kp.rows + TY - 1) / TY;
+    kp.n_tiles = kp.col_tiles * row_tiles;
+    uint64_t grid = kp.n_tiles;
+    if (grid > ew_grid_cap()) grid = ew_grid_cap();
+
+    switch (vec) {
+    case 4:
+        hipLaunchKernelGGL((ew_rows_kernel<Op, 4>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, kp, op, sv);
+        break;
+    case 2:
+        hipLaunchKernelGGL((ew_rows_kernel<Op, 2>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, kp, op, sv);
+        break;
+    default:
+        hipLaunchKernelGGL((ew_rows_kernel<Op, 1>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, kp, op, sv);
+        break;
+    }
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+}  // namespace cumo_hip
+
+#endif

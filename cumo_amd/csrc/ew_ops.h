@@ -1,0 +1,165 @@
+// Element functors for the elementwise kernels.
+//
+// Semantics follow the reference's device macros
+// (ext/cumo/include/cumo/types/float_macro_kernel.h:28-123,
+// xint_macro_kernel.h:15-42, int_macro_kernel.h:8-27) with one deliberate
+// difference: for SFloat, every libm function is evaluated in double and
+// rounded once, which is what the host macros (types/float_macro.h:84-118)
+// compile to on the CPU that Numo runs on, instead of the device's float
+// overload. The kernels are bandwidth bound, so the wider evaluation is free.
+#ifndef CUMO_HIP_EW_OPS_H
+#define CUMO_HIP_EW_OPS_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <float.h>
+
+namespace cumo_hip {
+
+#define CUMO_HIP_OP_COMMON(TA, TB, TR, NIN_, BIT_, CHK_) \
+    typedef TA A; typedef TB B; typedef TR R; typedef TA S; \
+    static constexpr int NIN = NIN_; static constexpr bool BIT_OUT = BIT_; static constexpr bool CHECKED = CHK_;
+
+// ---- binary, float ---------------------------------------------------------
+#define CUMO_HIP_FBIN(NAME, EXPR) \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) \
+        __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (T)(EXPR); return true; } };
+CUMO_HIP_FBIN(OpAdd, x + y)
+CUMO_HIP_FBIN(OpSub, x - y)
+CUMO_HIP_FBIN(OpMul, x * y)
+CUMO_HIP_FBIN(OpDiv, x / y)
+CUMO_HIP_FBIN(OpFMod, fmod((double)x, (double)y))
+CUMO_HIP_FBIN(OpCopysign, copysign((double)x, (double)y))
+CUMO_HIP_FBIN(OpAtan2, atan2((double)x, (double)y))
+CUMO_HIP_FBIN(OpHypot, hypot((double)x, (double)y))
+
+// ---- binary, int32 (wrapping arithmetic done in unsigned) -------------------
+#define CUMO_HIP_IBIN(NAME, EXPR) \
+    struct NAME { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 2, false, false) \
+        __device__ __forceinline__ bool operator()(int32_t x, int32_t y, int32_t& z) const { z = (int32_t)(EXPR); return true; } };
+CUMO_HIP_IBIN(OpIAdd, (uint32_t)x + (uint32_t)y)
+CUMO_HIP_IBIN(OpISub, (uint32_t)x - (uint32_t)y)
+CUMO_HIP_IBIN(OpIMul, (uint32_t)x * (uint32_t)y)
+CUMO_HIP_IBIN(OpIAnd, x & y)
+CUMO_HIP_IBIN(OpIOr, x | y)
+CUMO_HIP_IBIN(OpIXor, x ^ y)
+CUMO_HIP_IBIN(OpIShl, (uint32_t)x << (y & 31))
+CUMO_HIP_IBIN(OpIShr, x >> (y & 31))
+
+// division by zero rejects the element and raises the flag
+// (reference: narray/gen/tmpl/binary_kernel.cu:3-8)
+struct OpIDiv { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 2, false, true)
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t y, int32_t& z) const {
+        if (y == 0) return false;
+        z = (x == INT32_MIN && y == -1) ? INT32_MIN : x / y;
+        return true; } };
+struct OpIMod { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 2, false, true)
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t y, int32_t& z) const {
+        if (y == 0) return false;
+        z = (y == -1) ? 0 : x % y;
+        return true; } };
+
+// ---- unary -----------------------------------------------------------------
+#define CUMO_HIP_FUN(NAME, EXPR) \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const { z = (T)(EXPR); return true; } };
+CUMO_HIP_FUN(OpMinus, -x)
+CUMO_HIP_FUN(OpReciprocal, 1 / x)
+CUMO_HIP_FUN(OpSquare, x * x)
+CUMO_HIP_FUN(OpSign, (x == 0) ? 0.0 : ((x > 0) ? 1.0 : ((x < 0) ? -1.0 : (double)x)))
+CUMO_HIP_FUN(OpFAbs, fabs((double)x))
+CUMO_HIP_FUN(OpFloor, floor((double)x))
+CUMO_HIP_FUN(OpRound, round((double)x))
+CUMO_HIP_FUN(OpCeil, ceil((double)x))
+CUMO_HIP_FUN(OpTrunc, trunc((double)x))
+CUMO_HIP_FUN(OpRint, rint((double)x))
+// NMath (reference list: narray/gen/spec.rb:427-457)
+CUMO_HIP_FUN(OpSqrt, sqrt((double)x))
+CUMO_HIP_FUN(OpCbrt, cbrt((double)x))
+CUMO_HIP_FUN(OpLog, log((double)x))
+CUMO_HIP_FUN(OpLog2, log2((double)x))
+CUMO_HIP_FUN(OpLog10, log10((double)x))
+CUMO_HIP_FUN(OpExp, exp((double)x))
+CUMO_HIP_FUN(OpExp2, exp2((double)x))
+CUMO_HIP_FUN(OpExp10, exp10((double)x))
+CUMO_HIP_FUN(OpSin, sin((double)x))
+CUMO_HIP_FUN(OpCos, cos((double)x))
+CUMO_HIP_FUN(OpTan, tan((double)x))
+CUMO_HIP_FUN(OpAsin, asin((double)x))
+CUMO_HIP_FUN(OpAcos, acos((double)x))
+CUMO_HIP_FUN(OpAtan, atan((double)x))
+CUMO_HIP_FUN(OpSinh, sinh((double)x))
+CUMO_HIP_FUN(OpCosh, cosh((double)x))
+CUMO_HIP_FUN(OpTanh, tanh((double)x))
+CUMO_HIP_FUN(OpAsinh, asinh((double)x))
+CUMO_HIP_FUN(OpAcosh, acosh((double)x))
+CUMO_HIP_FUN(OpAtanh, atanh((double)x))
+// the host macro guards x == 0 (types/float_macro.h:113); the reference's device
+// macro does not and answers NaN there, which Numo does not
+CUMO_HIP_FUN(OpSinc, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
+CUMO_HIP_FUN(OpErf, erf((double)x))
+CUMO_HIP_FUN(OpErfc, erfc((double)x))
+CUMO_HIP_FUN(OpLog1p, log1p((double)x))
+CUMO_HIP_FUN(OpExpm1, expm1((double)x))
+
+#define CUMO_HIP_IUN(NAME, EXPR) \
+    struct NAME { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false) \
+        __device__ __forceinline__ bool operator()(int32_t x, int32_t, int32_t& z) const { z = (int32_t)(EXPR); return true; } };
+CUMO_HIP_IUN(OpIMinus, 0u - (uint32_t)x)
+CUMO_HIP_IUN(OpISquare, (uint32_t)x * (uint32_t)x)
+CUMO_HIP_IUN(OpISign, (x == 0) ? 0 : ((x > 0) ? 1 : -1))
+CUMO_HIP_IUN(OpINot, ~x)
+// reference: types/int_macro_kernel.h:12-24 and narray/gen/tmpl/unary_kernel.cu:4-9
+struct OpIReciprocal { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, true)
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t, int32_t& z) const {
+        if (x == 0) return false;
+        z = (x == 1) ? 1 : ((x == -1) ? -1 : 0);
+        return true; } };
+// reference: narray/gen/tmpl/unary2_kernel.cu:4-9
+struct OpIAbs { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, true)
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t, int32_t& z) const {
+        if (x == INT32_MIN) return false;
+        z = (x < 0) ? -x : x;
+        return true; } };
+
+// ---- comparisons into Bit ---------------------------------------------------
+#define CUMO_HIP_CMP(NAME, EXPR) \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, uint32_t, 2, true, false) \
+        __device__ __forceinline__ bool operator()(T x, T y, uint32_t& z) const { z = (EXPR) ? 1u : 0u; return true; } };
+CUMO_HIP_CMP(OpEq, x == y)
+CUMO_HIP_CMP(OpNe, x != y)
+CUMO_HIP_CMP(OpGt, x > y)
+CUMO_HIP_CMP(OpGe, x >= y)
+CUMO_HIP_CMP(OpLt, x < y)
+CUMO_HIP_CMP(OpLe, x <= y)
+// reference: types/sfloat_kernel.h:9, dfloat_kernel.h (the float form does the
+// subtraction in float and everything else in double)
+template <class T> struct OpNearlyEq { CUMO_HIP_OP_COMMON(T, T, uint32_t, 2, true, false)
+    __device__ __forceinline__ bool operator()(T x, T y, uint32_t& z) const {
+        const double eps = (sizeof(T) == 4) ? (double)FLT_EPSILON : DBL_EPSILON;
+        z = (fabs((double)(T)(x - y)) <= (fabs((double)x) + fabs((double)y)) * eps * 2) ? 1u : 0u;
+        return true; } };
+
+#define CUMO_HIP_CND(NAME, EXPR) \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, uint32_t, 1, true, false) \
+        __device__ __forceinline__ bool operator()(T x, T, uint32_t& z) const { z = (EXPR) ? 1u : 0u; return true; } };
+CUMO_HIP_CND(OpIsNan, x != x)
+CUMO_HIP_CND(OpIsInf, isinf(x))
+CUMO_HIP_CND(OpIsPosInf, isinf(x) && !signbit(x))
+CUMO_HIP_CND(OpIsNegInf, isinf(x) && signbit(x))
+CUMO_HIP_CND(OpIsFinite, isfinite(x))
+CUMO_HIP_CND(OpSignbit, signbit(x))
+
+// ---- store/cast, fill --------------------------------------------------------
+// dst = (dst type)src, the plain C conversion of the reference's device macros
+// (types/float_macro_kernel.h:21-27, xint_macro_kernel.h:7-13)
+template <class TD, class TS> struct OpCast { CUMO_HIP_OP_COMMON(TS, TS, TD, 1, false, false)
+    __device__ __forceinline__ bool operator()(TS x, TS, TD& z) const { z = (TD)x; return true; } };
+
+template <class T> struct OpFill { CUMO_HIP_OP_COMMON(T, T, T, 0, false, false)
+    T value;
+    __device__ __forceinline__ bool operator()(T, T, T& z) const { z = value; return true; } };
+
+}  // namespace cumo_hip
+
+#endif

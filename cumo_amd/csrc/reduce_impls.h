@@ -1,0 +1,258 @@
+// Reduction semantics: what each reduction folds and how accumulators merge.
+//
+// The rules are the reference's impl structs
+// (ext/cumo/narray/gen/tmpl/real_accum_kernel.cu:11-157,
+// float_accum_kernel.cu:15-146, accum_arg_kernel.cu:15-112,
+// accum_index_kernel.cu:15-112), which in turn restate Numo's sequential loops
+// (ext/cumo/include/cumo/types/real_accum.h:25-441): NaN skipping, all-NaN
+// answers, lowest index on ties, Int32 sums widening to 64 bits.
+//
+// Every combine() is insensitive to the order in which accumulators arrive,
+// so the kernels are free to interleave lanes. Where Numo's answer depends on
+// order -- which of two equal elements min/max keep, i.e. the sign of a zero --
+// the accumulator carries the index and the earlier element wins, as the
+// reference's tests require (test/narray_test.rb:667-672).
+#ifndef CUMO_HIP_REDUCE_IMPLS_H
+#define CUMO_HIP_REDUCE_IMPLS_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <float.h>
+
+namespace cumo_hip {
+
+template <class T> struct is_float_t { static constexpr bool value = false; };
+template <> struct is_float_t<float> { static constexpr bool value = true; };
+template <> struct is_float_t<double> { static constexpr bool value = true; };
+
+template <class T> __device__ __forceinline__ bool isnan_t(T x) { return x != x; }
+template <> __device__ __forceinline__ bool isnan_t<int32_t>(int32_t) { return false; }
+
+// what an accumulator of min/max starts from: `skip` loses to every element
+// (NaN for floats), `lowest`/`highest` lose to every element but a NaN
+template <class T> struct Lim;
+template <> struct Lim<float> {
+    static __device__ __forceinline__ float skip() { return __int_as_float(0x7fc00000); }
+    static __device__ __forceinline__ float highest() { return __int_as_float(0x7f800000); }
+    static __device__ __forceinline__ float lowest() { return __int_as_float(0xff800000); }
+};
+template <> struct Lim<double> {
+    static __device__ __forceinline__ double skip() { return __longlong_as_double(0x7ff8000000000000ll); }
+    static __device__ __forceinline__ double highest() { return __longlong_as_double(0x7ff0000000000000ll); }
+    static __device__ __forceinline__ double lowest() { return __longlong_as_double(0xfff0000000000000ll); }
+};
+template <> struct Lim<int32_t> {
+    static __device__ __forceinline__ int32_t skip() { return 0; }
+    static __device__ __forceinline__ int32_t highest() { return INT32_MAX; }
+    static __device__ __forceinline__ int32_t lowest() { return INT32_MIN; }
+};
+
+template <class T> __device__ __forceinline__ T spread(T hi, T lo) { return hi - lo; }
+template <> __device__ __forceinline__ int32_t spread<int32_t>(int32_t hi, int32_t lo) { return (int32_t)((uint32_t)hi - (uint32_t)lo); }
+
+// ---- sum / prod / mean -------------------------------------------------------
+// TA: accumulator type (the input type for floats, int64 for Int32:
+// narray/gen/spec.rb:308-319). divisor != 0 turns the sum into a mean
+// (float_accum_kernel.cu:42-50).
+template <class T, class TA, bool PROD, bool SKIP_NAN>
+struct SumImpl {
+    typedef T In;
+    typedef TA Acc;
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 1;
+    TA divisor;
+    __device__ __forceinline__ Acc identity() const { return PROD ? (TA)1 : (TA)0; }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
+        if (SKIP_NAN && isnan_t(x)) return;
+        if (PROD) acc = (TA)x * acc; else acc = (TA)x + acc;
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        if (PROD) acc = next * acc; else acc = next + acc;
+    }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
+        *reinterpret_cast<TA*>(out) = (divisor != (TA)0) ? (TA)(acc / divisor) : acc;
+    }
+};
+
+// mean(nan: true): the count of what was left rides along (float_accum_kernel.cu:86-101)
+template <class T>
+struct MeanNanImpl {
+    typedef T In;
+    struct Acc { T sum; int64_t n; };
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 1;
+    __device__ __forceinline__ Acc identity() const { return Acc{(T)0, 0}; }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
+        if (isnan_t(x)) return;
+        acc.sum = x + acc.sum;
+        acc.n += 1;
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { acc.sum = next.sum + acc.sum; acc.n += next.n; }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const { *reinterpret_cast<T*>(out) = acc.sum / (T)acc.n; }
+};
+
+// ---- rms ----------------------------------------------------------------------
+// count: the length of the reduce axis, known to the launcher
+// (float_accum_kernel.cu:52-58); the nan form counts what it kept (:103-116).
+template <class T, bool SKIP_NAN>
+struct RmsImpl {
+    typedef T In;
+    struct Acc { T sum; int64_t n; };
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 1;
+    T count;
+    __device__ __forceinline__ Acc identity() const { return Acc{(T)0, 0}; }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
+        if (SKIP_NAN) {
+            if (isnan_t(x)) return;
+            acc.n += 1;
+        }
+        acc.sum += x * x;
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { acc.sum += next.sum; acc.n += next.n; }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
+        const T n = SKIP_NAN ? (T)acc.n : count;
+        *reinterpret_cast<T*>(out) = (T)sqrt((double)(acc.sum / n));
+    }
+};
+
+// ---- var / stddev: Welford per element, Chan between accumulators ---------------
+// (float_accum_kernel.cu:10-40,102-125). Numo takes two passes with the exact
+// mean (types/real_accum.h:114-131); the two agree to rounding.
+template <class T, bool SKIP_NAN>
+struct MomentsImpl {
+    typedef T In;
+    struct Acc { T n; T mean; T m2; };
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 1;
+    int take_sqrt;
+    __device__ __forceinline__ Acc identity() const { return Acc{(T)0, (T)0, (T)0}; }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
+        if (SKIP_NAN && isnan_t(x)) return;
+        acc.n += (T)1;
+        const T delta = x - acc.mean;
+        acc.mean += delta / acc.n;
+        acc.m2 += delta * (x - acc.mean);
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        if (next.n == (T)0) return;
+        if (acc.n == (T)0) { acc = next; return; }
+        const T n = acc.n + next.n;
+        const T delta = next.mean - acc.mean;
+        acc.mean = acc.mean + delta * (next.n / n);
+        acc.m2 += next.m2 + delta * delta * acc.n * next.n / n;
+        acc.n = n;
+    }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
+        // every element NaN leaves no count; Numo answers +0 there (float_accum_kernel.cu:74-84)
+        T v = (SKIP_NAN && acc.n == (T)0) ? (T)0 : acc.m2 / (acc.n - (T)1);
+        if (take_sqrt) v = (T)sqrt((double)v);
+        *reinterpret_cast<T*>(out) = v;
+    }
+};
+
+// ---- kahan_sum (DFloat): Neumaier partials (float_accum_kernel.cu:116-146) ------
+template <class T, bool SKIP_NAN>
+struct KahanImpl {
+    typedef T In;
+    struct Acc { T sum; T comp; };
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 1;
+    __device__ __forceinline__ Acc identity() const { return Acc{(T)0, (T)0}; }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        const T t = acc.sum + next.sum;
+        const T c = (fabs(acc.sum) >= fabs(next.sum)) ? (acc.sum - t) + next.sum : (next.sum - t) + acc.sum;
+        acc.comp += next.comp + c;
+        acc.sum = t;
+    }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
+        if (SKIP_NAN && isnan_t(x)) return;
+        combine(Acc{x, (T)0}, acc);
+    }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const { *reinterpret_cast<T*>(out) = acc.sum + acc.comp; }
+};
+
+// ---- min / max / argmin / argmax / min_index / max_index -------------------------
+// One accumulator for all of them: the value and the index it was seen at.
+// NAN_WINS = false: a NaN loses to anything, every element NaN answers the first
+// (accum_arg_kernel.cu:15-37). NAN_WINS = true (nan: true): the first NaN wins
+// outright (accum_arg_kernel.cu:40-61). Equal values: lower index.
+// out_mode: 0 store the value (min/max), 4 / 8 store the index as int32 / int64.
+template <class T, bool IS_MAX, bool NAN_WINS>
+struct ArgImpl {
+    typedef T In;
+    struct Acc { T value; int64_t index; };
+    static constexpr bool USES_INDEX = true;
+    static constexpr int NOUT = 1;
+    int out_mode;
+    __device__ __forceinline__ Acc identity() const {
+        if (is_float_t<T>::value && !NAN_WINS) return Acc{Lim<T>::skip(), INT64_MAX};
+        return Acc{IS_MAX ? Lim<T>::lowest() : Lim<T>::highest(), INT64_MAX};
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        if (is_float_t<T>::value) {
+            const bool an = isnan_t(acc.value), nn = isnan_t(next.value);
+            if (an || nn) {
+                if (NAN_WINS) {
+                    if (nn && (!an || next.index < acc.index)) acc = next;
+                } else {
+                    if (an && (!nn || next.index < acc.index)) acc = next;
+                }
+                return;
+            }
+        }
+        const bool better = IS_MAX ? (acc.value < next.value) : (acc.value > next.value);
+        if (better || (acc.value == next.value && next.index < acc.index)) acc = next;
+    }
+    __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{x, idx}, acc); }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
+        if (out_mode == 0) *reinterpret_cast<T*>(out) = acc.value;
+        else if (out_mode == 4) *reinterpret_cast<int32_t*>(out) = (int32_t)acc.index;
+        else *reinterpret_cast<int64_t*>(out) = acc.index;
+    }
+};
+
+// ---- minmax / ptp ------------------------------------------------------------------
+// Both ends at once, each with its index so that minmax answers exactly what min
+// and max answer (real_accum_kernel.cu:54-84,139-157).
+// out_mode: 0 = two outputs (minmax), 1 = max - min (ptp).
+template <class T, bool NAN_WINS>
+struct MinMaxImpl {
+    typedef T In;
+    typedef typename ArgImpl<T, false, NAN_WINS>::Acc One;
+    struct Acc { One lo; One hi; };
+    static constexpr bool USES_INDEX = true;
+    static constexpr int NOUT = 2;
+    int out_mode;
+    __device__ __forceinline__ Acc identity() const {
+        ArgImpl<T, false, NAN_WINS> a{0};
+        ArgImpl<T, true, NAN_WINS> b{0};
+        const typename ArgImpl<T, true, NAN_WINS>::Acc h = b.identity();
+        return Acc{a.identity(), One{h.value, h.index}};
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        ArgImpl<T, false, NAN_WINS> a{0};
+        ArgImpl<T, true, NAN_WINS> b{0};
+        a.combine(next.lo, acc.lo);
+        typename ArgImpl<T, true, NAN_WINS>::Acc h{acc.hi.value, acc.hi.index};
+        b.combine(typename ArgImpl<T, true, NAN_WINS>::Acc{next.hi.value, next.hi.index}, h);
+        acc.hi = One{h.value, h.index};
+    }
+    __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{One{x, idx}, One{x, idx}}, acc); }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const {
+        if (out_mode == 0) {
+            *reinterpret_cast<T*>(out) = acc.lo.value;
+            *reinterpret_cast<T*>(out2) = acc.hi.value;
+        } else {
+            // (+0) - (-0) and the like: Numo keeps one element for both ends, so a
+            // zero spread is +0 (types/real_accum.h:406-441)
+            T d = spread<T>(acc.hi.value, acc.lo.value);
+            if (d == (T)0) d = (T)0;
+            *reinterpret_cast<T*>(out) = d;
+        }
+    }
+};
+
+}  // namespace cumo_hip
+
+#endif

@@ -1,0 +1,430 @@
+// Reduction engine for gfx950.
+//
+// Replaces ext/cumo/include/cumo/reduce_kernel.h of the reference (address
+// planner, reduction_kernel / _arg_ / _pair_ / _partial_kernel and the
+// cumo_reduce* orchestration). The reference runs 512-thread blocks that
+// combine through a nine-level shared-memory tree with a barrier per level.
+// Here:
+//
+//  red_row_kernel  the reduce axis runs along memory. 2^k lanes (1..64, or a
+//                  whole 256-thread block for long axes) share one output;
+//                  each lane strides over the axis with 128-bit loads, lanes
+//                  combine with wave64 shuffles (no LDS, no barrier, up to a
+//                  wave), four waves combine through 4 LDS slots.
+//  red_col_kernel  the output axis runs along memory. Each lane owns VEC
+//                  neighbouring outputs and walks the reduce axis itself, so
+//                  loads are 128-bit and coalesced across lanes and nothing
+//                  is combined across lanes at all.
+//
+// Either kernel can run as the first pass of a split reduction: the reduce
+// axis is cut into n_split chunks, accumulators go to
+// partial[i_out * n_split + i_split], and a second red_row_kernel launch
+// combines them in a fixed order. Both passes are deterministic (fixed
+// shuffle order, no atomics), like the reference's.
+//
+// Impl contract (all __device__):
+//   typedef In, Acc;  static constexpr bool USES_INDEX; static constexpr int NOUT (1 or 2)
+//   Acc identity() const
+//   void accumulate(In x, int64_t idx, Acc& acc) const     -- fold one input element
+//   void combine(const Acc& next, Acc& acc) const          -- fold an accumulator of LATER elements into acc
+//   void store(const Acc& acc, char* out, char* out2) const
+#ifndef CUMO_HIP_REDUCE_KERNELS_H
+#define CUMO_HIP_REDUCE_KERNELS_H
+
+#include "common.h"
+#include "plan.h"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace cumo_hip {
+
+constexpr int kRedBlock = 256;
+constexpr int kRedUnroll = 4;
+
+struct RedKParams {
+    int out_ndim, red_ndim;
+    int tpr_bits;        // row kernel: 2^tpr_bits lanes per output
+    int index_mode;      // what accumulate() gets as idx: 1 = position along the flattened reduce axes, 2 = element offset from in
+    int small;           // totals fit 32 bits
+    uint64_t out_total, red_total;
+    uint64_t n_split, chunk;
+    uint64_t out_shape[kMaxDim], red_shape[kMaxDim];
+    int64_t in_out_step[kMaxDim], in_red_step[kMaxDim], out_step[kMaxDim], out2_step[kMaxDim];
+    char* in;
+    char* out;
+    char* out2;
+};
+
+template <class T>
+__device__ __forceinline__ T shfl_down_any(const T& v, unsigned delta) {
+    static_assert(sizeof(T) % 4 == 0, "accumulator must be a whole number of 32-bit words");
+    constexpr int W = sizeof(T) / 4;
+    union U {
+        T t;
+        uint32_t w[W];
+        __device__ U() {}
+    } a, b;
+    a.t = v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) b.w[i] = __shfl_down(a.w[i], delta);
+    return b.t;
+}
+
+template <class T, int N>
+struct alignas((sizeof(T) * N) > 16 ? 16 : (sizeof(T) * N)) RedVec {
+    T v[N];
+};
+
+// offset of flat index i over dims [0, nd) with the given steps
+__device__ __forceinline__ int64_t red_decompose(uint64_t i, int nd, const uint64_t* shape, const int64_t* step, int small) {
+    int64_t off = 0;
+    if (nd == 1) return (int64_t)i * step[0];
+    if (small) {
+        uint32_t r = (uint32_t)i;
+        for (int d = nd - 1; d >= 1; --d) {
+            const uint32_t n = (uint32_t)shape[d];
+            const uint32_t q = r / n;
+            off += (int64_t)(r - q * n) * step[d];
+            r = q;
+        }
+        if (nd > 0) off += (int64_t)r * step[0];
+    } else {
+        uint64_t r = i;
+        for (int d = nd - 1; d >= 1; --d) {
+            const uint64_t n = shape[d];
+            const uint64_t q = r / n;
+            off += (int64_t)(r - q * n) * step[d];
+            r = q;
+        }
+        if (nd > 0) off += (int64_t)r * step[0];
+    }
+    return off;
+}
+
+template <class Impl, int VEC, bool PARTIAL>
+__global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    __shared__ Acc wave_acc[kRedBlock / 64];
+
+    const unsigned TPR = 1u << p.tpr_bits;
+    const unsigned RPB = kRedBlock >> p.tpr_bits;
+    const unsigned lane_r = threadIdx.x & (TPR - 1);
+    const unsigned row_in_block = threadIdx.x >> p.tpr_bits;
+    const uint64_t n_rows = p.out_total * p.n_split;
+    const uint64_t n_blocks = (n_rows + RPB - 1) / RPB;
+    const int64_t rstep = p.in_red_step[p.red_ndim > 0 ? p.red_ndim - 1 : 0];
+    const uint64_t stride = (uint64_t)TPR * VEC;
+
+    for (uint64_t rb = blockIdx.x; rb < n_blocks; rb += gridDim.x) {
+        const uint64_t vrow = rb * RPB + row_in_block;
+        const bool ok = vrow < n_rows;
+        uint64_t i_out = 0, i_split = 0;
+        if (ok) {
+            if (p.n_split == 1) {
+                i_out = vrow;
+            } else {
+                i_out = vrow / p.n_split;
+                i_split = vrow - i_out * p.n_split;
+            }
+        }
+        Acc acc = impl.identity();
+        if (ok) {
+            const uint64_t begin = i_split * p.chunk;
+            uint64_t end = begin + p.chunk;
+            if (end > p.red_total) end = p.red_total;
+            const int64_t in_off = red_decompose(i_out, p.out_ndim, p.out_shape, p.in_out_step, p.small);
+            const char* base = p.in + in_off;
+            for (uint64_t i0 = begin + (uint64_t)lane_r * VEC; i0 < end; i0 += stride * kRedUnroll) {
+                In x[kRedUnroll][VEC];
+                int64_t eoff[kRedUnroll];
+#pragma unroll
+                for (int u = 0; u < kRedUnroll; ++u) {
+                    const uint64_t i = i0 + (uint64_t)u * stride;
+                    if (i < end) {
+                        const int64_t off = (p.red_ndim <= 1) ? (int64_t)i * rstep
+                                                              : red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
+                        eoff[u] = in_off + off;
+                        if constexpr (VEC > 1) {
+                            const RedVec<In, VEC> v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
+                        } else {
+                            x[u][0] = *reinterpret_cast<const In*>(base + off);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kRedUnroll; ++u) {
+                    const uint64_t i = i0 + (uint64_t)u * stride;
+                    if (i < end) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            int64_t idx = 0;
+                            if (Impl::USES_INDEX) {
+                                idx = (p.index_mode == 2) ? (eoff[u] / (int64_t)sizeof(In) + j) : (int64_t)(i + j);
+                            }
+                            impl.accumulate(x[u][j], idx, acc);
+                        }
+                    }
+                }
+            }
+        }
+        // lanes of one output combine; lane 0 of the group ends up with everything,
+        // later lanes folded into earlier ones in a fixed order
+        const unsigned wave_span = TPR < 64 ? TPR : 64;
+        for (unsigned d = wave_span >> 1; d > 0; d >>= 1) {
+            const Acc other = shfl_down_any(acc, d);
+            impl.combine(other, acc);
+        }
+        if (TPR > 64) {
+            const unsigned wave = threadIdx.x >> 6;
+            if ((threadIdx.x & 63) == 0) wave_acc[wave] = acc;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                for (unsigned w = 1; w < kRedBlock / 64; ++w) impl.combine(wave_acc[w], acc);
+            }
+            __syncthreads();
+        }
+        if (ok && lane_r == 0) {
+            if (PARTIAL) {
+                partial[vrow] = acc;
+            } else {
+                const int64_t o1 = red_decompose(i_out, p.out_ndim, p.out_shape, p.out_step, p.small);
+                const int64_t o2 = (Impl::NOUT > 1) ? red_decompose(i_out, p.out_ndim, p.out_shape, p.out2_step, p.small) : 0;
+                impl.store(acc, p.out + o1, (Impl::NOUT > 1) ? (p.out2 + o2) : nullptr);
+            }
+        }
+    }
+}
+
+template <class Impl, int VEC, bool PARTIAL>
+__global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    const uint64_t groups = p.out_total / VEC;  // planner guarantees divisibility of the innermost out dim
+    const uint64_t n_items = groups * p.n_split;
+    const int L = p.out_ndim - 1;
+
+    for (uint64_t g = (uint64_t)blockIdx.x * kRedBlock + threadIdx.x; g < n_items; g += (uint64_t)gridDim.x * kRedBlock) {
+        uint64_t i_split = 0, cg = g;
+        if (p.n_split > 1) {
+            i_split = g / groups;
+            cg = g - i_split * groups;
+        }
+        const uint64_t i_out0 = cg * VEC;
+        const int64_t in_off = red_decompose(i_out0, p.out_ndim, p.out_shape, p.in_out_step, p.small);
+        const int64_t ostep_in = p.in_out_step[L];
+        const char* base = p.in + in_off;
+        const uint64_t begin = i_split * p.chunk;
+        uint64_t end = begin + p.chunk;
+        if (end > p.red_total) end = p.red_total;
+
+        Acc acc[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = impl.identity();
+
+        for (uint64_t i0 = begin; i0 < end; i0 += kRedUnroll) {
+            In x[kRedUnroll][VEC];
+            int64_t roff[kRedUnroll];
+#pragma unroll
+            for (int u = 0; u < kRedUnroll; ++u) {
+                const uint64_t i = i0 + u;
+                if (i < end) {
+                    const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
+                    roff[u] = off;
+                    if constexpr (VEC > 1) {
+                        const RedVec<In, VEC> v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
+                    } else {
+                        x[u][0] = *reinterpret_cast<const In*>(base + off);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kRedUnroll; ++u) {
+                const uint64_t i = i0 + u;
+                if (i < end) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        int64_t idx = 0;
+                        if (Impl::USES_INDEX) {
+                            idx = (p.index_mode == 2) ? ((in_off + roff[u] + (int64_t)j * ostep_in) / (int64_t)sizeof(In)) : (int64_t)i;
+                        }
+                        impl.accumulate(x[u][j], idx, acc[j]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const uint64_t i_out = i_out0 + j;
+            if (PARTIAL) {
+                partial[i_out * p.n_split + i_split] = acc[j];
+            } else {
+                const int64_t o1 = red_decompose(i_out, p.out_ndim, p.out_shape, p.out_step, p.small);
+                const int64_t o2 = (Impl::NOUT > 1) ? red_decompose(i_out, p.out_ndim, p.out_shape, p.out2_step, p.small) : 0;
+                impl.store(acc[j], p.out + o1, (Impl::NOUT > 1) ? (p.out2 + o2) : nullptr);
+            }
+        }
+    }
+}
+
+// Second pass of a split reduction: the input is accumulators.
+template <class Impl>
+struct CombineImpl {
+    typedef typename Impl::Acc In;
+    typedef typename Impl::Acc Acc;
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = Impl::NOUT;
+    Impl impl;
+    __device__ __forceinline__ Acc identity() const { return impl.identity(); }
+    __device__ __forceinline__ void accumulate(const In& x, int64_t, Acc& acc) const { impl.combine(x, acc); }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { impl.combine(next, acc); }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const { impl.store(acc, out, out2); }
+};
+
+static inline unsigned red_grid_cap() {
+    static unsigned cap = 0;
+    if (cap == 0) {
+        const char* e = std::getenv("CUMO_HIP_RED_GRID_CAP");
+        cap = e ? (unsigned)std::strtoul(e, nullptr, 10) : 0;
+        if (cap == 0) cap = (unsigned)kNumCU * 32;
+    }
+    return cap;
+}
+
+static inline void red_fill_params(RedKParams* kp, const ReducePlan& plan, const cumo_na_reduction_arg_t* arg,
+                                   const cumo_na_iarray_t* out2, int index_mode) {
+    std::memset(kp, 0, sizeof(*kp));
+    kp->out_ndim = plan.out_ndim;
+    kp->red_ndim = plan.red_ndim;
+    kp->index_mode = index_mode;
+    kp->out_total = plan.out_total;
+    kp->red_total = plan.red_total;
+    kp->n_split = 1;
+    kp->chunk = plan.red_total;
+    for (int d = 0; d < kMaxDim; ++d) {
+        kp->out_shape[d] = plan.out_shape[d];
+        kp->red_shape[d] = plan.red_shape[d];
+        kp->in_out_step[d] = plan.in_out_step[d];
+        kp->in_red_step[d] = plan.in_red_step[d];
+        kp->out_step[d] = plan.out_step[d];
+        kp->out2_step[d] = plan.out2_step[d];
+    }
+    kp->in = arg->in.ptr;
+    kp->out = arg->out.ptr;
+    kp->out2 = out2 ? out2->ptr : nullptr;
+    kp->small = (arg->in_indexer.total_size < 0xffffffffull) ? 1 : 0;
+}
+
+template <class Impl, bool PARTIAL, bool SCALAR_ONLY = false>
+static void red_launch_row(const RedKParams& kp, int vec, Impl impl, typename Impl::Acc* partial, hipStream_t stream) {
+    constexpr int kMaxVec = SCALAR_ONLY ? 1 : (int)(16 / sizeof(typename Impl::In));
+    const uint64_t n_rows = kp.out_total * kp.n_split;
+    const uint64_t rpb = (uint64_t)kRedBlock >> kp.tpr_bits;
+    uint64_t grid = (n_rows + rpb - 1) / rpb;
+    if (grid > red_grid_cap()) grid = red_grid_cap();
+    if (grid == 0) return;
+    const dim3 g((unsigned)grid), b(kRedBlock);
+    if constexpr (kMaxVec >= 4) {
+        if (vec == 4) { hipLaunchKernelGGL((red_row_kernel<Impl, 4, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
+    }
+    if constexpr (kMaxVec >= 2) {
+        if (vec == 2) { hipLaunchKernelGGL((red_row_kernel<Impl, 2, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
+    }
+    hipLaunchKernelGGL((red_row_kernel<Impl, 1, PARTIAL>), g, b, 0, stream, kp, impl, partial);
+}
+
+template <class Impl, bool PARTIAL>
+static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Impl::Acc* partial, hipStream_t stream) {
+    constexpr int kMaxVec = (int)(16 / sizeof(typename Impl::In));
+    const uint64_t items = (kp.out_total / vec) * kp.n_split;
+    uint64_t grid = (items + kRedBlock - 1) / kRedBlock;
+    if (grid > red_grid_cap()) grid = red_grid_cap();
+    if (grid == 0) return;
+    const dim3 g((unsigned)grid), b(kRedBlock);
+    if constexpr (kMaxVec >= 4) {
+        if (vec == 4) { hipLaunchKernelGGL((red_col_kernel<Impl, 4, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
+    }
+    if constexpr (kMaxVec >= 2) {
+        if (vec == 2) { hipLaunchKernelGGL((red_col_kernel<Impl, 2, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
+    }
+    hipLaunchKernelGGL((red_col_kernel<Impl, 1, PARTIAL>), g, b, 0, stream, kp, impl, partial);
+}
+
+// index_mode: 1 for arg reductions, 2 for *_index reductions, ignored by impls
+// that do not use the index. The scratch of a split reduction comes from the
+// pool and goes back right after the second launch is queued: the next owner
+// can only touch it from work queued later on the same stream
+// (reference: include/cumo/reduce_kernel.h:493-496).
+template <class Impl>
+static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Impl impl, int index_mode) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    if (arg->out_indexer.total_size == 0) return;  // reference: reduce_kernel.h:444-446
+    ReducePlan plan;
+    plan_reduce(arg, out2, (int)sizeof(In), (int)sizeof(Acc), &plan);
+    if (plan.kind == RED_EMPTY) return;
+    hipStream_t stream = current_stream();
+    RedKParams kp;
+    red_fill_params(&kp, plan, arg, out2, index_mode);
+    kp.tpr_bits = 0;
+    while ((1 << kp.tpr_bits) < plan.threads_per_row) ++kp.tpr_bits;
+
+    if (plan.n_split <= 1) {
+        if (plan.kind == RED_COL) red_launch_col<Impl, false>(kp, plan.vec, impl, nullptr, stream);
+        else red_launch_row<Impl, false>(kp, plan.vec, impl, nullptr, stream);
+        cumo_cuda_runtime_check_kernel_launch();
+        return;
+    }
+
+    // first pass
+    const uint64_t ns = (uint64_t)plan.n_split;
+    uint64_t chunk = (plan.red_total + ns - 1) / ns;
+    if (plan.kind == RED_ROW) {
+        // whole vectors per lane: chunks start on a multiple of the vector width
+        const uint64_t q = (uint64_t)plan.vec;
+        chunk = ((chunk + q - 1) / q) * q;
+    }
+    kp.n_split = (plan.red_total + chunk - 1) / chunk;
+    kp.chunk = chunk;
+    const uint64_t n_partial = plan.out_total * kp.n_split;
+    Acc* partial = reinterpret_cast<Acc*>(cumo_cuda_runtime_malloc(sizeof(Acc) * n_partial));
+    if (!partial) return;
+    if (plan.kind == RED_COL) red_launch_col<Impl, true>(kp, plan.vec, impl, partial, stream);
+    else red_launch_row<Impl, true>(kp, plan.vec, impl, partial, stream);
+    cumo_cuda_runtime_check_kernel_launch();
+
+    // second pass over partial[out_total][n_split]
+    RedKParams k2 = kp;
+    k2.in = reinterpret_cast<char*>(partial);
+    k2.red_ndim = 1;
+    k2.red_shape[0] = kp.n_split;
+    k2.in_red_step[0] = (int64_t)sizeof(Acc);
+    k2.red_total = kp.n_split;
+    k2.n_split = 1;
+    k2.chunk = kp.n_split;
+    int64_t s = (int64_t)sizeof(Acc) * (int64_t)kp.n_split;
+    for (int d = plan.out_ndim - 1; d >= 0; --d) {
+        k2.in_out_step[d] = s;
+        s *= (int64_t)plan.out_shape[d];
+    }
+    k2.small = (n_partial < 0xffffffffull && plan.out_total < 0xffffffffull) ? 1 : 0;
+    int tpr = 1;
+    while (tpr < 64 && (uint64_t)tpr * 4 < kp.n_split) tpr <<= 1;
+    if (kp.n_split > 1024) tpr = 256;
+    k2.tpr_bits = 0;
+    while ((1 << k2.tpr_bits) < tpr) ++k2.tpr_bits;
+    CombineImpl<Impl> cimpl;
+    cimpl.impl = impl;
+    red_launch_row<CombineImpl<Impl>, false, true>(k2, 1, cimpl, nullptr, stream);
+    cumo_cuda_runtime_check_kernel_launch();
+    cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
+}
+
+}  // namespace cumo_hip
+
+#endif

@@ -1,0 +1,140 @@
+// Runtime glue: error reporting, stream selection, the pinned error flag the
+// Int32 division and abs kernels write through, and the synchronous copies the
+// host uses to read results back.
+//
+// Replaces ext/cumo/cuda/runtime.c:16-68 of the reference. That file raises a
+// Ruby exception from cumo_cuda_runtime_check_kernel_launch; this one cannot
+// include ruby.h, so it calls the handler the host installed instead.
+#include "common.h"
+
+#include <cstdio>
+#include <cstring>
+#include <atomic>
+
+namespace cumo_hip {
+
+static std::atomic<cumo_hip_error_handler_t> g_handler{nullptr};
+
+struct LastError {
+    int kind = 0;
+    int status = 0;
+    char message[512] = {0};
+};
+static thread_local LastError t_last;
+static thread_local hipStream_t t_stream = nullptr;
+
+void report_error(int kind, int hip_status, const char* message) {
+    cumo_hip_error_handler_t h = g_handler.load();
+    if (h) {
+        h(kind, hip_status, message);  // may longjmp
+        return;
+    }
+    // keep the first error until somebody reads it
+    if (t_last.kind == 0) {
+        t_last.kind = kind;
+        t_last.status = hip_status;
+        std::snprintf(t_last.message, sizeof(t_last.message), "%s", message ? message : "");
+    }
+}
+
+void report_hip_error(hipError_t status, const char* what) {
+    char buf[384];
+    std::snprintf(buf, sizeof(buf), "%s: %s (error=%d)", what ? what : "hip", hipGetErrorString(status), (int)status);
+    report_error(status == hipErrorOutOfMemory ? CUMO_HIP_ERROR_OUT_OF_MEMORY : CUMO_HIP_ERROR_RUNTIME, (int)status, buf);
+}
+
+hipStream_t current_stream() { return t_stream; }
+
+}  // namespace cumo_hip
+
+using namespace cumo_hip;
+
+extern "C" {
+
+void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler) { g_handler.store(handler); }
+
+int cumo_hip_last_error(const char** message) {
+    static thread_local char copy[512];
+    int kind = t_last.kind;
+    if (message) {
+        std::memcpy(copy, t_last.message, sizeof(copy));
+        *message = copy;
+    }
+    t_last.kind = 0;
+    t_last.status = 0;
+    t_last.message[0] = 0;
+    return kind;
+}
+
+void cumo_hip_set_stream(void* hip_stream) { t_stream = (hipStream_t)hip_stream; }
+void* cumo_hip_get_stream(void) { return (void*)t_stream; }
+
+int cumo_hip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+void cumo_hip_synchronize(void) { hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize"); }
+
+void cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n) {
+    if (n == 0) return;
+    if (!hip_ok(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, t_stream), "hipMemcpyAsync(h2d)")) return;
+    hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+
+void cumo_hip_memcpy_d2h(void* dst, const void* src, size_t n) {
+    if (n == 0) return;
+    if (!hip_ok(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, t_stream), "hipMemcpyAsync(d2h)")) return;
+    hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+
+// reference: cuda/runtime.c:16-20
+void cumo_cuda_runtime_check_kernel_launch(void) {
+    hipError_t st = hipGetLastError();
+    if (st != hipSuccess) report_hip_error(st, "kernel launch");
+}
+
+// Pinned, device-mapped host words a kernel writes through when it rejects an
+// element (reference: cuda/runtime.c:22-68). hipHostMalloc, not registration of
+// existing memory.
+static int* alloc_pinned_word(size_t bytes) {
+    void* p = nullptr;
+    if (!hip_ok(hipHostMalloc(&p, bytes, hipHostMallocMapped | hipHostMallocPortable), "hipHostMalloc")) return nullptr;
+    std::memset(p, 0, bytes);
+    return (int*)p;
+}
+
+int* cumo_cuda_runtime_error_flag_ptr(void) {
+    static int* flag = nullptr;
+    if (flag == nullptr) flag = alloc_pinned_word(sizeof(int));
+    return flag;
+}
+
+int* cumo_cuda_runtime_error_flag_new(void) {
+    int* flag = cumo_cuda_runtime_error_flag_ptr();
+    if (flag) *flag = 0;
+    return flag;
+}
+
+bool cumo_cuda_runtime_error_flag_get(int* flag) {
+    if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return false;
+    return flag && (*(volatile int*)flag != 0);
+}
+
+size_t* cumo_cuda_runtime_error_item_ptr(void) {
+    static size_t* item = nullptr;
+    if (item == nullptr) item = (size_t*)alloc_pinned_word(sizeof(size_t));
+    return item;
+}
+
+size_t* cumo_cuda_runtime_error_item_new(void) {
+    size_t* item = cumo_cuda_runtime_error_item_ptr();
+    if (item) *item = 0;
+    return item;
+}
+
+}  // extern "C"

@@ -1,0 +1,390 @@
+/*
+ * cumo_hip.h -- the C-ABI of the MI355X (gfx950) array-compute library.
+ *
+ * Everything in this header is `extern "C"`, plain pointers and sizes. The
+ * first half reproduces, byte for byte, the launch descriptors and launcher
+ * entry points that the Cumo Ruby extension's generated host iterators bind
+ * (the reference file:line each one replaces is cited beside it), so that the
+ * extension can link this library in place of its own kernel translation
+ * units. The second half (`cumo_hip_*`) is what this library adds: the error
+ * hook that stands in for the extension's raise, stream selection, the memory
+ * pool's C interface, the launch planner's introspection calls and the host
+ * launch layer (ndloop) that builds the descriptors from array views.
+ */
+#ifndef CUMO_HIP_H
+#define CUMO_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+#include <stdbool.h>
+#include <sys/types.h>
+
+#if defined(__cplusplus)
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------
+ * 1. Launch descriptors (reference: ext/cumo/include/cumo/indexer.h:16-68,
+ *    ext/cumo/include/cumo/narray.h:236-240,489-496).
+ * ---------------------------------------------------------------------- */
+#define CUMO_NA_MAX_DIMENSION 12            /* narray.h:489 */
+typedef unsigned int CUMO_BIT_DIGIT;        /* narray.h:492 */
+#define CUMO_NB (sizeof(CUMO_BIT_DIGIT)*8)  /* narray.h:494 */
+
+/* stride or index array of one dimension (narray.h:236-240,324-330): a stride
+ * is stored as (stride<<1)|1, anything with bit 0 clear is a device pointer to
+ * size_t offsets. */
+typedef union {
+    ssize_t stride;
+    size_t *index;
+} cumo_stridx_t;
+#define CUMO_SDX_IS_STRIDE(x) ((x).stride&0x1)
+#define CUMO_SDX_IS_INDEX(x)  (!CUMO_SDX_IS_STRIDE(x))
+#define CUMO_SDX_GET_STRIDE(x) ((x).stride>>1)
+#define CUMO_SDX_GET_INDEX(x)  ((x).index)
+#define CUMO_SDX_SET_STRIDE(x,s) ((x).stride=((s)<<1)|0x1)
+#define CUMO_SDX_SET_INDEX(x,idx) ((x).index=idx)
+
+/* indexer.h:16-22 (216 bytes). index[] and raw_index are scratch the
+ * reference's kernels write per element; this library never touches them. */
+typedef struct {
+    unsigned char ndim;
+    size_t total_size;
+    size_t shape[CUMO_NA_MAX_DIMENSION];
+    uint64_t index[CUMO_NA_MAX_DIMENSION];
+    uint64_t raw_index;
+} cumo_na_indexer_t;
+
+/* indexer.h:28-31 (104 bytes). ptr already includes the view offset; step is a
+ * signed byte stride per dimension, 0 for a broadcast dimension. */
+typedef struct {
+    char* ptr;
+    ssize_t step[CUMO_NA_MAX_DIMENSION];
+} cumo_na_iarray_t;
+
+/* indexer.h:40-44 (112 bytes). pos and step are in bits. */
+typedef struct {
+    CUMO_BIT_DIGIT* ptr;
+    size_t pos;
+    ssize_t step[CUMO_NA_MAX_DIMENSION];
+} cumo_na_bit_iarray_t;
+
+/* indexer.h:46-49 */
+typedef struct {
+    char* ptr;
+    cumo_stridx_t stridx[CUMO_NA_MAX_DIMENSION];
+} cumo_na_iarray_stridx_t;
+
+/* indexer.h:57-61 */
+typedef struct {
+    CUMO_BIT_DIGIT* ptr;
+    size_t pos;
+    cumo_stridx_t stridx[CUMO_NA_MAX_DIMENSION];
+} cumo_na_bit_iarray_stridx_t;
+
+/* indexer.h:63-68 (640 bytes). The first out_indexer.ndim dimensions of `in`
+ * are the output dimensions, the rest are reduced (indexer.h:189-220). */
+typedef struct {
+    cumo_na_iarray_t in;
+    cumo_na_iarray_t out;
+    cumo_na_indexer_t in_indexer;
+    cumo_na_indexer_t out_indexer;
+} cumo_na_reduction_arg_t;
+
+/* ------------------------------------------------------------------------
+ * 2. Runtime glue and device memory (reference:
+ *    ext/cumo/include/cumo/cuda/memory_pool.h:15-24,
+ *    ext/cumo/include/cumo/template_kernel.h:83-90,
+ *    ext/cumo/include/cumo/cuda/runtime.h:59-65, ext/cumo/cuda/runtime.c:16-68).
+ *    In the reference these raise a Ruby exception on failure; here a failure
+ *    goes to the handler installed with cumo_hip_set_error_handler (which may
+ *    longjmp/raise), or is latched for cumo_hip_last_error when none is set.
+ * ---------------------------------------------------------------------- */
+char* cumo_cuda_runtime_malloc(size_t size);
+void  cumo_cuda_runtime_free(char *ptr);
+void  cumo_cuda_runtime_free_no_raise(char *ptr);
+void  cumo_cuda_runtime_check_kernel_launch(void);
+int*  cumo_cuda_runtime_error_flag_ptr(void);
+int*  cumo_cuda_runtime_error_flag_new(void);
+bool  cumo_cuda_runtime_error_flag_get(int *flag);
+size_t* cumo_cuda_runtime_error_item_ptr(void);
+size_t* cumo_cuda_runtime_error_item_new(void);
+
+/* ------------------------------------------------------------------------
+ * 3. Elementwise launchers. The lists below are expanded into declarations
+ *    here and into definitions in the library, so the two cannot drift.
+ *    T(type_name, c_type)
+ * ---------------------------------------------------------------------- */
+#define CUMO_HIP_FLOAT_TYPES(T) T(sfloat, float) T(dfloat, double)
+#define CUMO_HIP_INT_TYPES(T)   T(int32, int32_t)
+
+/* binary ops with a scalar form: narray/gen/tmpl/binary_kernel.cu:11,52-81,
+ * host declaration narray/gen/tmpl/binary.c:12-15; op list narray/gen/spec.rb:199-207,249-256,268-271 */
+#define CUMO_HIP_BINARY_OPS_ALL(X, t, c)   X(t, c, add) X(t, c, sub) X(t, c, mul) X(t, c, div) X(t, c, mod)
+#define CUMO_HIP_BINARY_OPS_FLOAT(X, t, c) X(t, c, copysign)
+#define CUMO_HIP_BINARY_OPS_INT(X, t, c)   X(t, c, bit_and) X(t, c, bit_or) X(t, c, bit_xor) X(t, c, left_shift) X(t, c, right_shift)
+
+#define CUMO_HIP_DECL_BINARY(t, c, op) \
+    void cumo_iter_##t##_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer, int* divzero); \
+    void cumo_iter_##t##_##op##_s_kernel_launch(cumo_na_iarray_t* a1, c sv, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer, int* divzero, int scalar_is_left);
+
+/* unary ops: narray/gen/tmpl/unary_kernel.cu:14-42, host narray/gen/tmpl/unary.c:3;
+ * op list narray/gen/spec.rb:216-219,259,272-277 */
+#define CUMO_HIP_UNARY_OPS_ALL(X, t, c)   X(t, c, minus) X(t, c, reciprocal) X(t, c, sign) X(t, c, square)
+#define CUMO_HIP_UNARY_OPS_FLOAT(X, t, c) X(t, c, floor) X(t, c, round) X(t, c, ceil) X(t, c, trunc) X(t, c, rint)
+#define CUMO_HIP_UNARY_OPS_INT(X, t, c)   X(t, c, bit_not)
+
+#define CUMO_HIP_DECL_UNARY(t, c, op) \
+    void cumo_iter_##t##_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer, int* divzero);
+
+/* abs: narray/gen/tmpl/unary2_kernel.cu:15-41, host narray/gen/tmpl/unary2.c:3 */
+#define CUMO_HIP_DECL_ABS(t, c) \
+    void cumo_iter_##t##_abs_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer, int* intmin);
+
+/* NMath one-argument functions: narray/gen/tmpl/unary_s_kernel.cu:3-29, host
+ * narray/gen/tmpl/unary_s.c:2; list narray/gen/spec.rb:427-457 */
+#define CUMO_HIP_MATH_OPS(X, t, c) \
+    X(t, c, sqrt) X(t, c, cbrt) X(t, c, log) X(t, c, log2) X(t, c, log10) X(t, c, exp) X(t, c, exp2) X(t, c, exp10) \
+    X(t, c, sin) X(t, c, cos) X(t, c, tan) X(t, c, asin) X(t, c, acos) X(t, c, atan) \
+    X(t, c, sinh) X(t, c, cosh) X(t, c, tanh) X(t, c, asinh) X(t, c, acosh) X(t, c, atanh) \
+    X(t, c, sinc) X(t, c, erf) X(t, c, erfc) X(t, c, log1p) X(t, c, expm1)
+
+#define CUMO_HIP_DECL_MATH(t, c, op) \
+    void cumo_iter_##t##_math_s_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer);
+
+/* NMath two-argument functions: narray/gen/tmpl/binary_s_kernel.cu:7-52, host
+ * narray/gen/tmpl/binary_s.c:2-3 */
+#define CUMO_HIP_MATH2_OPS(X, t, c) X(t, c, atan2) X(t, c, hypot)
+
+#define CUMO_HIP_DECL_MATH2(t, c, op) \
+    void cumo_iter_##t##_math_s_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_math_s_##op##_s_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer, c sv, int scalar_is_left);
+
+/* comparisons into Bit: narray/gen/tmpl/cond_binary_kernel.cu:7-53, host
+ * narray/gen/tmpl/cond_binary.c:2-3 */
+#define CUMO_HIP_COND_OPS_ALL(X, t, c)   X(t, c, eq) X(t, c, ne) X(t, c, gt) X(t, c, ge) X(t, c, lt) X(t, c, le)
+#define CUMO_HIP_COND_OPS_FLOAT(X, t, c) X(t, c, nearly_eq)
+
+#define CUMO_HIP_DECL_COND(t, c, op) \
+    void cumo_iter_##t##_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_bit_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_##op##_s_kernel_launch(cumo_na_iarray_t* a1, c sv, cumo_na_bit_iarray_t* a3, cumo_na_indexer_t* indexer, int scalar_is_left);
+
+/* float classification into Bit: narray/gen/tmpl/cond_unary_kernel.cu:3-29,
+ * host narray/gen/tmpl/cond_unary.c:2 */
+#define CUMO_HIP_COND_UNARY_OPS(X, t, c) X(t, c, isnan) X(t, c, isinf) X(t, c, isposinf) X(t, c, isneginf) X(t, c, isfinite) X(t, c, signbit)
+
+#define CUMO_HIP_DECL_COND_UNARY(t, c, op) \
+    void cumo_iter_##t##_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_bit_iarray_t* a2, cumo_na_indexer_t* indexer);
+
+/* fill and 0-dim construction: narray/gen/tmpl/fill_kernel.cu:3-27 (host
+ * fill.c:2), narray/gen/tmpl/new_dim0_kernel.cu:2-10 (host new_dim0.c:2);
+ * Bit -> number: narray/gen/tmpl/store_bit_kernel.cu:3-30 (host store_bit.c:2) */
+#define CUMO_HIP_DECL_FILL(t, c) \
+    void cumo_iter_##t##_fill_kernel_launch(cumo_na_iarray_t* a1, cumo_na_indexer_t* indexer, c val); \
+    void cumo_##t##_new_dim0_kernel_launch(c *ptr, c x); \
+    void cumo_iter_##t##_store_bit_kernel_launch(cumo_na_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_indexer_t* indexer);
+
+CUMO_HIP_BINARY_OPS_ALL(CUMO_HIP_DECL_BINARY, sfloat, float)
+CUMO_HIP_BINARY_OPS_ALL(CUMO_HIP_DECL_BINARY, dfloat, double)
+CUMO_HIP_BINARY_OPS_ALL(CUMO_HIP_DECL_BINARY, int32, int32_t)
+CUMO_HIP_BINARY_OPS_FLOAT(CUMO_HIP_DECL_BINARY, sfloat, float)
+CUMO_HIP_BINARY_OPS_FLOAT(CUMO_HIP_DECL_BINARY, dfloat, double)
+CUMO_HIP_BINARY_OPS_INT(CUMO_HIP_DECL_BINARY, int32, int32_t)
+
+CUMO_HIP_UNARY_OPS_ALL(CUMO_HIP_DECL_UNARY, sfloat, float)
+CUMO_HIP_UNARY_OPS_ALL(CUMO_HIP_DECL_UNARY, dfloat, double)
+CUMO_HIP_UNARY_OPS_ALL(CUMO_HIP_DECL_UNARY, int32, int32_t)
+CUMO_HIP_UNARY_OPS_FLOAT(CUMO_HIP_DECL_UNARY, sfloat, float)
+CUMO_HIP_UNARY_OPS_FLOAT(CUMO_HIP_DECL_UNARY, dfloat, double)
+CUMO_HIP_UNARY_OPS_INT(CUMO_HIP_DECL_UNARY, int32, int32_t)
+
+CUMO_HIP_DECL_ABS(sfloat, float)
+CUMO_HIP_DECL_ABS(dfloat, double)
+CUMO_HIP_DECL_ABS(int32, int32_t)
+
+CUMO_HIP_MATH_OPS(CUMO_HIP_DECL_MATH, sfloat, float)
+CUMO_HIP_MATH_OPS(CUMO_HIP_DECL_MATH, dfloat, double)
+CUMO_HIP_MATH2_OPS(CUMO_HIP_DECL_MATH2, sfloat, float)
+CUMO_HIP_MATH2_OPS(CUMO_HIP_DECL_MATH2, dfloat, double)
+
+CUMO_HIP_COND_OPS_ALL(CUMO_HIP_DECL_COND, sfloat, float)
+CUMO_HIP_COND_OPS_ALL(CUMO_HIP_DECL_COND, dfloat, double)
+CUMO_HIP_COND_OPS_ALL(CUMO_HIP_DECL_COND, int32, int32_t)
+CUMO_HIP_COND_OPS_FLOAT(CUMO_HIP_DECL_COND, sfloat, float)
+CUMO_HIP_COND_OPS_FLOAT(CUMO_HIP_DECL_COND, dfloat, double)
+
+CUMO_HIP_COND_UNARY_OPS(CUMO_HIP_DECL_COND_UNARY, sfloat, float)
+CUMO_HIP_COND_UNARY_OPS(CUMO_HIP_DECL_COND_UNARY, dfloat, double)
+
+CUMO_HIP_DECL_FILL(sfloat, float)
+CUMO_HIP_DECL_FILL(dfloat, double)
+CUMO_HIP_DECL_FILL(int32, int32_t)
+
+/* typed store / cast, dst = (dst type)src: narray/gen/tmpl/store_from_kernel.cu:3-53,
+ * host narray/gen/tmpl/store_from.c:2; pairs narray/gen/spec.rb:122-142.
+ * a1 is the destination, a2 the source. int64 appears because Int32#sum
+ * answers Int64 (narray/gen/spec.rb:308-319). */
+#define CUMO_HIP_STORE_PAIRS(X) \
+    X(sfloat, sfloat) X(sfloat, dfloat) X(sfloat, int32) X(sfloat, int64) \
+    X(dfloat, sfloat) X(dfloat, dfloat) X(dfloat, int32) X(dfloat, int64) \
+    X(int32, sfloat)  X(int32, dfloat)  X(int32, int32)  X(int32, int64)
+#define CUMO_HIP_DECL_STORE(dst, src) \
+    void cumo_iter_##dst##_store_##src##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer);
+CUMO_HIP_STORE_PAIRS(CUMO_HIP_DECL_STORE)
+
+/* copy of any view, a1 = source, a2 = destination:
+ * narray/data_kernel.cu:47-132, host narray/data.c:56,84-92 */
+void cumo_iter_copy_bytes_indexer_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer, ssize_t elmsz);
+
+/* ------------------------------------------------------------------------
+ * 4. Reduction launchers: narray/gen/tmpl/real_accum_kernel.cu:166-226,
+ *    float_accum_kernel.cu:155-206, accum_arg_kernel.cu:117-142,
+ *    accum_index_kernel.cu:117-142; host declarations accum.c:8, minmax.c:2-4,
+ *    accum_arg.c:5, accum_index.c:5.
+ * ---------------------------------------------------------------------- */
+#define CUMO_HIP_DECL_REDUCE(t, name) \
+    void cumo_##t##_##name##_kernel_launch(cumo_na_reduction_arg_t* arg);
+#define CUMO_HIP_DECL_REDUCE_PAIR(t, name) \
+    void cumo_##t##_##name##_kernel_launch(cumo_na_reduction_arg_t* arg, cumo_na_iarray_t* out2);
+
+#define CUMO_HIP_REDUCE_OPS_ALL(X, t)   X(t, sum) X(t, prod) X(t, min) X(t, max) X(t, ptp)
+#define CUMO_HIP_REDUCE_OPS_FLOAT(X, t) \
+    X(t, sum_nan) X(t, prod_nan) X(t, min_nan) X(t, max_nan) X(t, ptp_nan) \
+    X(t, mean) X(t, var) X(t, stddev) X(t, rms) \
+    X(t, mean_nan) X(t, var_nan) X(t, stddev_nan) X(t, rms_nan)
+#define CUMO_HIP_REDUCE_OPS_DOUBLE(X, t) X(t, kahan_sum) X(t, kahan_sum_nan)
+#define CUMO_HIP_ARG_OPS_ALL(X, t) \
+    X(t, argmin_int32) X(t, argmin_int64) X(t, argmax_int32) X(t, argmax_int64) \
+    X(t, min_index_int32) X(t, min_index_int64) X(t, max_index_int32) X(t, max_index_int64)
+#define CUMO_HIP_ARG_OPS_FLOAT(X, t) \
+    X(t, argmin_nan_int32) X(t, argmin_nan_int64) X(t, argmax_nan_int32) X(t, argmax_nan_int64) \
+    X(t, min_index_nan_int32) X(t, min_index_nan_int64) X(t, max_index_nan_int32) X(t, max_index_nan_int64)
+
+CUMO_HIP_REDUCE_OPS_ALL(CUMO_HIP_DECL_REDUCE, sfloat)
+CUMO_HIP_REDUCE_OPS_ALL(CUMO_HIP_DECL_REDUCE, dfloat)
+CUMO_HIP_REDUCE_OPS_ALL(CUMO_HIP_DECL_REDUCE, int32)
+CUMO_HIP_REDUCE_OPS_FLOAT(CUMO_HIP_DECL_REDUCE, sfloat)
+CUMO_HIP_REDUCE_OPS_FLOAT(CUMO_HIP_DECL_REDUCE, dfloat)
+CUMO_HIP_REDUCE_OPS_DOUBLE(CUMO_HIP_DECL_REDUCE, dfloat)
+CUMO_HIP_ARG_OPS_ALL(CUMO_HIP_DECL_REDUCE, sfloat)
+CUMO_HIP_ARG_OPS_ALL(CUMO_HIP_DECL_REDUCE, dfloat)
+CUMO_HIP_ARG_OPS_ALL(CUMO_HIP_DECL_REDUCE, int32)
+CUMO_HIP_ARG_OPS_FLOAT(CUMO_HIP_DECL_REDUCE, sfloat)
+CUMO_HIP_ARG_OPS_FLOAT(CUMO_HIP_DECL_REDUCE, dfloat)
+CUMO_HIP_DECL_REDUCE_PAIR(sfloat, minmax)
+CUMO_HIP_DECL_REDUCE_PAIR(dfloat, minmax)
+CUMO_HIP_DECL_REDUCE_PAIR(int32, minmax)
+CUMO_HIP_DECL_REDUCE_PAIR(sfloat, minmax_nan)
+CUMO_HIP_DECL_REDUCE_PAIR(dfloat, minmax_nan)
+
+/* ------------------------------------------------------------------------
+ * 5. Bit launchers: narray/gen/tmpl_bit/binary_kernel.cu:1-52 (host
+ *    tmpl_bit/binary.c:1-2), tmpl_bit/unary_kernel.cu (host tmpl_bit/unary.c),
+ *    tmpl_bit/bit_count_kernel.cu:4-78 (host tmpl_bit/bit_count.c:4-7).
+ *    count_* ADD onto the uint64 the output pointer names, as the reference's
+ *    atomicAdd does; ndloop pre-fills it with 0 (narray/ndloop.c:853-860).
+ * ---------------------------------------------------------------------- */
+#define CUMO_HIP_BIT_BINARY_OPS(X) X(and) X(or) X(xor) X(eq)
+#define CUMO_HIP_BIT_UNARY_OPS(X)  X(copy) X(not)
+#define CUMO_HIP_DECL_BIT_BINARY(op) \
+    void cumo_iter_bit_##op##_kernel_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_bit_iarray_stridx_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_bit_##op##_contiguous_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, CUMO_BIT_DIGIT *a2, size_t p2, CUMO_BIT_DIGIT *a3, size_t p3, uint64_t n);
+#define CUMO_HIP_DECL_BIT_UNARY(op) \
+    void cumo_iter_bit_##op##_kernel_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_bit_##op##_contiguous_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, CUMO_BIT_DIGIT *a3, size_t p3, uint64_t n);
+#define CUMO_HIP_DECL_BIT_COUNT(name) \
+    void cumo_iter_bit_##name##_index_kernel_launch(size_t p1, char *p2, CUMO_BIT_DIGIT *a1, size_t *idx1, uint64_t n); \
+    void cumo_iter_bit_##name##_stride_kernel_launch(size_t p1, char *p2, CUMO_BIT_DIGIT *a1, ssize_t s1, uint64_t n); \
+    void cumo_iter_bit_##name##_index_stride_kernel_launch(size_t p1, char *p2, CUMO_BIT_DIGIT *a1, size_t *idx1, ssize_t s2, uint64_t n); \
+    void cumo_iter_bit_##name##_stride_stride_kernel_launch(size_t p1, char *p2, CUMO_BIT_DIGIT *a1, ssize_t s1, ssize_t s2, uint64_t n);
+
+CUMO_HIP_BIT_BINARY_OPS(CUMO_HIP_DECL_BIT_BINARY)
+CUMO_HIP_BIT_UNARY_OPS(CUMO_HIP_DECL_BIT_UNARY)
+CUMO_HIP_DECL_BIT_COUNT(count_true)
+CUMO_HIP_DECL_BIT_COUNT(count_false)
+
+/* ------------------------------------------------------------------------
+ * 6. What this library adds (no counterpart symbol in the reference).
+ * ---------------------------------------------------------------------- */
+
+/* Error reporting. The reference raises from inside the launcher
+ * (cuda/runtime.c:16-20, cuda/memory_pool.cpp:64-96). A host that can raise
+ * installs a handler; it is called with kind and message and may not return
+ * (longjmp). With no handler the error is latched per thread. */
+enum {
+    CUMO_HIP_OK = 0,
+    CUMO_HIP_ERROR_RUNTIME = 1,        /* Cumo::CUDA::RuntimeError */
+    CUMO_HIP_ERROR_OUT_OF_MEMORY = 2,  /* Cumo::CUDA::OutOfMemoryError */
+    CUMO_HIP_ERROR_ARGUMENT = 3        /* ArgumentError / ShapeError raised by the host layer */
+};
+typedef void (*cumo_hip_error_handler_t)(int kind, int hip_status, const char* message);
+void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler);
+/* Returns the latched error kind (0 if none) and clears it; message, if not
+ * NULL, receives a pointer to a thread-local string. */
+int cumo_hip_last_error(const char** message);
+
+/* The stream every launcher and the pool use from this host thread. The
+ * reference only ever uses the default stream (cuda/memory_pool.cpp:43-44). */
+void  cumo_hip_set_stream(void* hip_stream);
+void* cumo_hip_get_stream(void);
+int   cumo_hip_device_count(void);
+void  cumo_hip_synchronize(void);
+/* synchronous copies for host read-back/ingest (extract_cpu, to_a, from_binary) */
+void  cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n);
+void  cumo_hip_memcpy_d2h(void* dst, const void* src, size_t n);
+void  cumo_hip_memset(void* dst, int byte, size_t n);
+
+/* Memory pool (replaces cumo::internal::MemoryPool, cuda/memory_pool_impl.hpp:160-435).
+ * Returns CUMO_HIP_OK or an error kind; never raises. */
+int    cumo_hip_pool_malloc(size_t size, void* hip_stream, void** ptr);
+int    cumo_hip_pool_free(void* ptr);                       /* CUMO_HIP_ERROR_ARGUMENT if the pool does not own ptr */
+void   cumo_hip_pool_free_all_blocks(void);
+void   cumo_hip_pool_free_all_blocks_stream(void* hip_stream);
+size_t cumo_hip_pool_n_free_blocks(void);
+size_t cumo_hip_pool_used_bytes(void);
+size_t cumo_hip_pool_free_bytes(void);
+size_t cumo_hip_pool_total_bytes(void);
+/* bytes and calls that went to hipMalloc since the process started */
+size_t cumo_hip_pool_device_malloc_calls(void);
+int    cumo_hip_pool_enable(int on);                        /* returns previous state; CUMO_MEMORY_POOL env sets the default */
+/* test hook: cap what the pool may hold from the device (0 = no cap), so that
+ * the out-of-memory path can be driven from the host without exhausting HBM */
+void   cumo_hip_pool_set_limit(size_t bytes);
+/* test hook: back the pool with the host heap (1) or the device (0) so that
+ * split/merge/accounting can be exercised without a GPU; only while the pool
+ * holds nothing */
+int    cumo_hip_pool_use_host_backend(int on);
+
+/* Launch planner introspection: what the elementwise/reduction launchers
+ * decide for a given set of descriptors, without launching. Host-only. */
+typedef struct {
+    int kind;           /* 0 empty, 1 rows (threads along the common fast dim), 2 transpose (LDS tile), 3 generic */
+    int ndim;           /* dimensions left after dropping size-1 and merging */
+    int vec;            /* elements per 128-bit access, 1 if not vectorised */
+    int fast_dim;       /* collapsed dim the threads run along */
+    int tr_dim;         /* second tile dim for kind 2, else -1 */
+    uint64_t shape[CUMO_NA_MAX_DIMENSION];
+    int64_t step[4][CUMO_NA_MAX_DIMENSION];
+} cumo_hip_ew_plan_t;
+/* elmsz[i] = element size of operand i in bytes, 0 for a Bit operand (steps in bits). */
+int cumo_hip_plan_elementwise(const cumo_na_indexer_t* indexer, int n_operands,
+                              const cumo_na_iarray_t* const* operands, const int* elmsz,
+                              const size_t* bitpos, cumo_hip_ew_plan_t* plan);
+
+typedef struct {
+    int kind;           /* 0 empty, 1 row (reduce axis along memory), 2 column (output axis along memory), 3 generic */
+    int vec;
+    int threads_per_row;     /* kind 1: lanes that share one output */
+    int n_split;             /* >1: two-pass, partial accumulators then combine */
+    int out_ndim, red_ndim;  /* after merging */
+    uint64_t out_total, red_total;
+    uint64_t out_shape[CUMO_NA_MAX_DIMENSION], red_shape[CUMO_NA_MAX_DIMENSION];
+    int64_t in_out_step[CUMO_NA_MAX_DIMENSION], in_red_step[CUMO_NA_MAX_DIMENSION], out_step[CUMO_NA_MAX_DIMENSION];
+} cumo_hip_reduce_plan_t;
+int cumo_hip_plan_reduce(const cumo_na_reduction_arg_t* arg, int in_elmsz, int accum_bytes, cumo_hip_reduce_plan_t* plan);
+
+#if defined(__cplusplus)
+}
+#endif
+
+#endif /* CUMO_HIP_H */
