@@ -1,0 +1,148 @@
+"""ctypes binding of libcumo_hip.so (the C-ABI declared in include/cumo_hip.h).
+
+There is no fallback: if the library has not been built, importing this module
+raises. Every call goes through `call`, which turns an error latched by the
+library into the exception the reference's Ruby extension would have raised.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libcumo_hip.so")
+
+MAX_DIM = 12  # CUMO_NA_MAX_DIMENSION
+
+
+class RuntimeError_(RuntimeError):
+    """Cumo::CUDA::RuntimeError (reference: ext/cumo/cuda/runtime.c:16-20)."""
+
+
+class OutOfMemoryError(MemoryError):
+    """Cumo::CUDA::OutOfMemoryError (reference: ext/cumo/cuda/memory_pool.cpp:90-92)."""
+
+
+class ShapeError(ValueError):
+    """Cumo::NArray::ShapeError (reference: ext/cumo/narray/ndloop.c:508-512)."""
+
+
+class Indexer(C.Structure):
+    # reference: ext/cumo/include/cumo/indexer.h:16-22
+    _fields_ = [("ndim", C.c_ubyte), ("total_size", C.c_size_t), ("shape", C.c_size_t * MAX_DIM),
+                ("index", C.c_uint64 * MAX_DIM), ("raw_index", C.c_uint64)]
+
+
+class IArray(C.Structure):
+    # reference: indexer.h:28-31
+    _fields_ = [("ptr", C.c_void_p), ("step", C.c_ssize_t * MAX_DIM)]
+
+
+class BitIArray(C.Structure):
+    # reference: indexer.h:40-44
+    _fields_ = [("ptr", C.c_void_p), ("pos", C.c_size_t), ("step", C.c_ssize_t * MAX_DIM)]
+
+
+class IArrayStridx(C.Structure):
+    # reference: indexer.h:46-49; a stride s is stored as (s << 1) | 1
+    _fields_ = [("ptr", C.c_void_p), ("stridx", C.c_ssize_t * MAX_DIM)]
+
+
+class BitIArrayStridx(C.Structure):
+    # reference: indexer.h:57-61
+    _fields_ = [("ptr", C.c_void_p), ("pos", C.c_size_t), ("stridx", C.c_ssize_t * MAX_DIM)]
+
+
+class ReductionArg(C.Structure):
+    # reference: indexer.h:63-68
+    _fields_ = [("in_", IArray), ("out", IArray), ("in_indexer", Indexer), ("out_indexer", Indexer)]
+
+
+class EwPlan(C.Structure):
+    _fields_ = [("kind", C.c_int), ("ndim", C.c_int), ("vec", C.c_int), ("fast_dim", C.c_int), ("tr_dim", C.c_int),
+                ("shape", C.c_uint64 * MAX_DIM), ("step", (C.c_int64 * MAX_DIM) * 4)]
+
+
+class ReducePlan(C.Structure):
+    _fields_ = [("kind", C.c_int), ("vec", C.c_int), ("threads_per_row", C.c_int), ("n_split", C.c_int),
+                ("out_ndim", C.c_int), ("red_ndim", C.c_int), ("out_total", C.c_uint64), ("red_total", C.c_uint64),
+                ("out_shape", C.c_uint64 * MAX_DIM), ("red_shape", C.c_uint64 * MAX_DIM),
+                ("in_out_step", C.c_int64 * MAX_DIM), ("in_red_step", C.c_int64 * MAX_DIM),
+                ("out_step", C.c_int64 * MAX_DIM)]
+
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "cumo_amd: %s is missing. Build it with `python -m cumo_amd.build` (needs hipcc); "
+        "there is no CPU fallback." % LIB_PATH)
+
+lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+
+P = C.POINTER
+_sig = {
+    "cumo_cuda_runtime_malloc": (C.c_void_p, [C.c_size_t]),
+    "cumo_cuda_runtime_free": (None, [C.c_void_p]),
+    "cumo_cuda_runtime_free_no_raise": (None, [C.c_void_p]),
+    "cumo_cuda_runtime_check_kernel_launch": (None, []),
+    "cumo_cuda_runtime_error_flag_ptr": (P(C.c_int), []),
+    "cumo_cuda_runtime_error_flag_new": (P(C.c_int), []),
+    "cumo_cuda_runtime_error_flag_get": (C.c_bool, [P(C.c_int)]),
+    "cumo_hip_last_error": (C.c_int, [P(C.c_char_p)]),
+    "cumo_hip_set_stream": (None, [C.c_void_p]),
+    "cumo_hip_get_stream": (C.c_void_p, []),
+    "cumo_hip_device_count": (C.c_int, []),
+    "cumo_hip_synchronize": (None, []),
+    "cumo_hip_memcpy_h2d": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "cumo_hip_memcpy_d2h": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "cumo_hip_memset": (None, [C.c_void_p, C.c_int, C.c_size_t]),
+    "cumo_hip_pool_malloc": (C.c_int, [C.c_size_t, C.c_void_p, P(C.c_void_p)]),
+    "cumo_hip_pool_free": (C.c_int, [C.c_void_p]),
+    "cumo_hip_pool_free_all_blocks": (None, []),
+    "cumo_hip_pool_free_all_blocks_stream": (None, [C.c_void_p]),
+    "cumo_hip_pool_n_free_blocks": (C.c_size_t, []),
+    "cumo_hip_pool_used_bytes": (C.c_size_t, []),
+    "cumo_hip_pool_free_bytes": (C.c_size_t, []),
+    "cumo_hip_pool_total_bytes": (C.c_size_t, []),
+    "cumo_hip_pool_device_malloc_calls": (C.c_size_t, []),
+    "cumo_hip_pool_enable": (C.c_int, [C.c_int]),
+    "cumo_hip_pool_set_limit": (None, [C.c_size_t]),
+    "cumo_hip_pool_use_host_backend": (C.c_int, [C.c_int]),
+    "cumo_hip_plan_elementwise": (C.c_int, [P(Indexer), C.c_int, P(P(IArray)), P(C.c_int), P(C.c_size_t), P(EwPlan)]),
+    "cumo_hip_plan_reduce": (C.c_int, [P(ReductionArg), C.c_int, C.c_int, P(ReducePlan)]),
+}
+for _name, (_res, _args) in _sig.items():
+    _f = getattr(lib, _name)
+    _f.restype = _res
+    _f.argtypes = _args
+
+CTYPE = {"sfloat": C.c_float, "dfloat": C.c_double, "int32": C.c_int32}
+
+
+def fn(name, restype=None, argtypes=None):
+    """Looks a launcher up by its C name; fails loudly when the symbol is missing."""
+    try:
+        f = getattr(lib, name)
+    except AttributeError:
+        raise NotImplementedError("libcumo_hip.so does not export %s" % name)
+    if argtypes is not None:
+        f.argtypes = argtypes
+    f.restype = restype
+    return f
+
+
+def check():
+    """Raises what the Ruby extension would have raised for a latched error."""
+    msg = C.c_char_p()
+    kind = lib.cumo_hip_last_error(C.byref(msg))
+    if kind == 0:
+        return
+    text = msg.value.decode("utf-8", "replace") if msg.value else ""
+    if kind == 2:
+        raise OutOfMemoryError(text)
+    if kind == 3:
+        raise ValueError(text)
+    raise RuntimeError_(text)
+
+
+def call(f, *args):
+    r = f(*args)
+    check()
+    return r

@@ -174,11 +174,11 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
     const uint64_t out_total = arg->out_indexer.total_size;
     const uint64_t in_total = arg->in_indexer.total_size;
     plan->out_total = out_total;
-    if (out_total == 0 || in_total == 0) {
+    if (out_total == 0) {
         plan->kind = RED_EMPTY;
-        plan->red_total = (out_total == 0) ? 0 : in_total / out_total;
         return;
     }
+    // an empty reduce axis still answers the identity for every output
     plan->red_total = in_total / out_total;
 
     // output dims: drop size 1, merge where input, output (and second output) agree

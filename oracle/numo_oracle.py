@@ -1,0 +1,315 @@
+"""ctypes front end of the CPU oracle (oracle/numo_oracle.c). TEST INFRASTRUCTURE:
+only tests/, the smoke check and the cpu_baseline leg of bench.py import it.
+
+Operands are numpy arrays (any strides, views welcome); broadcasting is resolved
+here with numpy's own stride-0 views so that the C side sees exactly the
+shape/steps descriptors the launch layer hands to the device.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB = os.path.join(HERE, "libnumo_oracle.so")
+REF_LIB = os.path.join(HERE, "_ref", "libref_accum.so")
+
+T_SFLOAT, T_DFLOAT, T_INT32, T_INT64, T_UINT64 = 0, 1, 2, 3, 4
+_TCODE = {np.dtype(np.float32): T_SFLOAT, np.dtype(np.float64): T_DFLOAT, np.dtype(np.int32): T_INT32,
+          np.dtype(np.int64): T_INT64, np.dtype(np.uint64): T_UINT64}
+
+
+def build():
+    """Compiles the oracle (and oracle/_ref where the reference tree exists)."""
+    subprocess.run(["make", "-C", HERE], check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+
+
+def _load():
+    if not os.path.exists(LIB):
+        build()
+    return C.CDLL(LIB)
+
+
+lib = _load()
+SZ = C.c_size_t
+SSZ = C.c_ssize_t
+lib.numo_binary.restype = C.c_int
+lib.numo_unary.restype = C.c_int
+lib.numo_compare.restype = C.c_int
+lib.numo_cond_unary.restype = C.c_int
+lib.numo_store.restype = C.c_int
+lib.numo_store_bit.restype = C.c_int
+lib.numo_copy_bytes.restype = C.c_int
+lib.numo_fill.restype = C.c_int
+lib.numo_bit_binary.restype = C.c_int
+lib.numo_bit_count.restype = C.c_uint64
+lib.numo_bit_count.argtypes = [C.c_void_p, SZ, SSZ, C.c_uint64, C.c_int]
+lib.numo_reduce.restype = C.c_int
+lib.numo_sfloat_f.restype = C.c_float
+lib.numo_sfloat_f.argtypes = [C.c_char_p, SZ, C.c_void_p]
+lib.numo_dfloat_f.restype = C.c_double
+lib.numo_dfloat_f.argtypes = [C.c_char_p, SZ, C.c_void_p]
+lib.numo_sfloat_index_f.restype = C.c_int64
+lib.numo_sfloat_index_f.argtypes = [C.c_char_p, SZ, C.c_void_p]
+lib.numo_dfloat_index_f.restype = C.c_int64
+lib.numo_dfloat_index_f.argtypes = [C.c_char_p, SZ, C.c_void_p]
+
+
+def _desc(a, shape):
+    """(pointer, steps) of `a` broadcast to `shape`."""
+    b = np.broadcast_to(a, shape)
+    steps = (SSZ * max(1, len(shape)))(*[int(s) for s in b.strides])
+    return C.c_void_p(b.__array_interface__["data"][0]), steps
+
+
+def _shape(shape):
+    return (SZ * max(1, len(shape)))(*[int(s) for s in shape])
+
+
+def _tcode(a):
+    return _TCODE[np.dtype(a.dtype)]
+
+
+class FlagError(Exception):
+    """The operation rejected an element (division by zero, abs(INT_MIN))."""
+
+    def __init__(self, result):
+        super().__init__("flag raised")
+        self.result = result
+
+
+def binary(op, x, y, scalar_is_left=False, out=None):
+    """x op y. Either side may be a Python number (the scalar form)."""
+    if isinstance(x, np.ndarray) and isinstance(y, np.ndarray):
+        shape = np.broadcast_shapes(x.shape, y.shape)
+        res = np.zeros(shape, dtype=x.dtype) if out is None else out
+        p1, s1 = _desc(x, shape)
+        p2, s2 = _desc(y, shape)
+        p3, s3 = _desc(res, shape)
+        rc = lib.numo_binary(op.encode(), _tcode(x), len(shape), _shape(shape), p1, s1, p2, s2, p3, s3, C.c_double(0), 0)
+    else:
+        arr, sv = (y, x) if scalar_is_left else (x, y)
+        shape = arr.shape
+        res = np.zeros(shape, dtype=arr.dtype) if out is None else out
+        p1, s1 = _desc(arr, shape)
+        p3, s3 = _desc(res, shape)
+        rc = lib.numo_binary(op.encode(), _tcode(arr), len(shape), _shape(shape), p1, s1, None, None, p3, s3,
+                             C.c_double(float(sv)), 1 if scalar_is_left else 0)
+    if rc < 0:
+        raise ValueError("oracle: unknown op %s" % op)
+    if rc == 1:
+        raise FlagError(res)
+    return res
+
+
+def unary(op, x, out=None):
+    res = np.zeros(x.shape, dtype=x.dtype) if out is None else out
+    p1, s1 = _desc(x, x.shape)
+    p2, s2 = _desc(res, x.shape)
+    rc = lib.numo_unary(op.encode(), _tcode(x), x.ndim, _shape(x.shape), p1, s1, p2, s2)
+    if rc < 0:
+        raise ValueError("oracle: unknown op %s" % op)
+    if rc == 1:
+        raise FlagError(res)
+    return res
+
+
+def _bit_words(nbits):
+    return np.zeros((nbits + 31) // 32 + 1, dtype=np.uint32)
+
+
+def unpack(words, pos, shape, steps=None):
+    """Bits of a packed word array as a uint8 array of `shape`."""
+    n = int(np.prod(shape)) if len(shape) else 1
+    bits = np.unpackbits(words.view(np.uint8), bitorder="little")
+    if steps is None:
+        return bits[pos:pos + n].reshape(shape).astype(np.uint8)
+    idx = np.full(shape, pos, dtype=np.int64)
+    for d, (s, st) in enumerate(zip(shape, steps)):
+        sh = [1] * len(shape)
+        sh[d] = s
+        idx = idx + (np.arange(s, dtype=np.int64) * st).reshape(sh)
+    return bits[idx].astype(np.uint8)
+
+
+def pack(bits):
+    """uint8 0/1 array -> packed uint32 words (contiguous, position 0)."""
+    flat = np.ascontiguousarray(bits).reshape(-1) != 0
+    w = np.zeros(((flat.size + 31) // 32) * 4, dtype=np.uint8)
+    p = np.packbits(flat, bitorder="little")
+    w[:p.size] = p
+    return w.view(np.uint32)
+
+
+def compare(op, x, y, scalar_is_left=False):
+    """Returns the result as an unpacked uint8 array (0/1)."""
+    if isinstance(x, np.ndarray) and isinstance(y, np.ndarray):
+        shape = np.broadcast_shapes(x.shape, y.shape)
+        arr = x
+    else:
+        arr, sv = (y, x) if scalar_is_left else (x, y)
+        shape = arr.shape
+    n = int(np.prod(shape)) if len(shape) else 1
+    words = _bit_words(n)
+    bs = (SSZ * max(1, len(shape)))(*[int(s // 1) for s in (np.empty(shape, dtype=np.uint8).strides or (1,))])
+    if isinstance(x, np.ndarray) and isinstance(y, np.ndarray):
+        p1, s1 = _desc(x, shape)
+        p2, s2 = _desc(y, shape)
+        rc = lib.numo_compare(op.encode(), _tcode(x), len(shape), _shape(shape), p1, s1, p2, s2,
+                              words.ctypes.data_as(C.c_void_p), SZ(0), bs, C.c_double(0), 0)
+    else:
+        p1, s1 = _desc(arr, shape)
+        rc = lib.numo_compare(op.encode(), _tcode(arr), len(shape), _shape(shape), p1, s1, None, None,
+                              words.ctypes.data_as(C.c_void_p), SZ(0), bs, C.c_double(float(sv)), 1 if scalar_is_left else 0)
+    if rc < 0:
+        raise ValueError("oracle: unknown op %s" % op)
+    return unpack(words, 0, shape)
+
+
+def cond_unary(op, x):
+    shape = x.shape
+    n = int(np.prod(shape)) if len(shape) else 1
+    words = _bit_words(n)
+    bs = (SSZ * max(1, len(shape)))(*[int(s) for s in (np.empty(shape, dtype=np.uint8).strides or (1,))])
+    p1, s1 = _desc(x, shape)
+    rc = lib.numo_cond_unary(op.encode(), _tcode(x), len(shape), _shape(shape), p1, s1,
+                             words.ctypes.data_as(C.c_void_p), SZ(0), bs)
+    if rc < 0:
+        raise ValueError("oracle: unknown op %s" % op)
+    return unpack(words, 0, shape)
+
+
+def store(dst_dtype, src):
+    res = np.zeros(src.shape, dtype=dst_dtype)
+    pd, sd = _desc(res, src.shape)
+    ps, ss = _desc(src, src.shape)
+    rc = lib.numo_store(_TCODE[np.dtype(dst_dtype)], _tcode(src), src.ndim, _shape(src.shape), pd, sd, ps, ss)
+    if rc < 0:
+        raise ValueError("oracle: unsupported store")
+    return res
+
+
+def copy(src):
+    res = np.zeros(src.shape, dtype=src.dtype)
+    pd, sd = _desc(res, src.shape)
+    ps, ss = _desc(src, src.shape)
+    lib.numo_copy_bytes(SZ(src.dtype.itemsize), src.ndim, _shape(src.shape), ps, ss, pd, sd)
+    return res
+
+
+def fill(dtype, shape, value):
+    res = np.zeros(shape, dtype=dtype)
+    pd, sd = _desc(res, shape)
+    lib.numo_fill(_TCODE[np.dtype(dtype)], len(shape), _shape(shape), pd, sd, C.c_double(float(value)))
+    return res
+
+
+def bit_binary(op, x, y=None):
+    """x, y: uint8 0/1 arrays (broadcastable). Packs, runs the per-bit loop, unpacks."""
+    shape = x.shape if y is None else np.broadcast_shapes(x.shape, y.shape)
+    xb = pack(np.broadcast_to(x, shape))
+    yb = pack(np.broadcast_to(y, shape)) if y is not None else None
+    n = int(np.prod(shape)) if len(shape) else 1
+    words = _bit_words(n)
+    bs = (SSZ * max(1, len(shape)))(*[int(s) for s in (np.empty(shape, dtype=np.uint8).strides or (1,))])
+    rc = lib.numo_bit_binary(op.encode(), len(shape), _shape(shape), xb.ctypes.data_as(C.c_void_p), SZ(0), bs,
+                             yb.ctypes.data_as(C.c_void_p) if yb is not None else None, SZ(0), bs,
+                             words.ctypes.data_as(C.c_void_p), SZ(0), bs)
+    if rc < 0:
+        raise ValueError("oracle: unknown bit op %s" % op)
+    return unpack(words, 0, shape)
+
+
+def bit_count(words, pos, step, n, count_false=False):
+    return int(lib.numo_bit_count(words.ctypes.data_as(C.c_void_p), pos, step, n, 1 if count_false else 0))
+
+
+def store_bit(dst_dtype, bits):
+    w = pack(bits)
+    shape = bits.shape
+    res = np.zeros(shape, dtype=dst_dtype)
+    pd, sd = _desc(res, shape)
+    bs = (SSZ * max(1, len(shape)))(*[int(s) for s in (np.empty(shape, dtype=np.uint8).strides or (1,))])
+    lib.numo_store_bit(_TCODE[np.dtype(dst_dtype)], len(shape), _shape(shape), pd, sd, w.ctypes.data_as(C.c_void_p), SZ(0), bs)
+    return res
+
+
+_OUT_DTYPE = {"sum": {T_INT32: np.int64}, "prod": {T_INT32: np.int64}}
+
+
+def reduce(op, x, axis=None, keepdims=False, nan=False, index_dtype=np.int32):
+    """The reduction `op` of x over `axis` (None = all) the way Numo answers it."""
+    nd = x.ndim
+    if axis is None:
+        axes = tuple(range(nd))
+    elif isinstance(axis, (int, np.integer)):
+        axes = (int(axis) % nd,)
+    else:
+        axes = tuple(sorted(int(a) % nd for a in axis))
+    keep = [d for d in range(nd) if d not in axes]
+    order = keep + list(axes)
+    xt = x.transpose(order) if nd else x
+    shape = xt.shape
+    steps = (SSZ * max(1, nd))(*[int(s) for s in xt.strides])
+    out_shape = tuple(x.shape[d] for d in keep)
+    name = op + ("_nan" if nan and x.dtype.kind == "f" else "")
+    is_idx = op.startswith("arg") or op.endswith("_index")
+    if is_idx:
+        odt = np.dtype(index_dtype)
+    else:
+        odt = np.dtype(_OUT_DTYPE.get(op, {}).get(_tcode(x), x.dtype))
+    res = np.zeros(out_shape, dtype=odt)
+    so = (SSZ * max(1, len(out_shape)))(*[int(s) for s in res.strides])
+    n_red = int(np.prod([x.shape[d] for d in axes])) if axes else 1
+    scratch = np.zeros(max(1, n_red), dtype=x.dtype)
+    rc = lib.numo_reduce(name.encode(), _tcode(x), nd, len(keep), _shape(shape),
+                         C.c_void_p(xt.__array_interface__["data"][0]), steps,
+                         res.ctypes.data_as(C.c_void_p), so, odt.itemsize, scratch.ctypes.data_as(C.c_void_p))
+    if rc < 0:
+        raise ValueError("oracle: unknown reduction %s" % name)
+    if keepdims:
+        res = res.reshape([x.shape[d] if d in keep else 1 for d in range(nd)])
+    return res
+
+
+def f1d(op, x):
+    """The sequential 1-d loop f_<op> on a contiguous 1-d array."""
+    x = np.ascontiguousarray(x)
+    if op.endswith("_index") or op.endswith("_index_nan") or op.startswith("arg"):
+        f = lib.numo_sfloat_index_f if x.dtype == np.float32 else lib.numo_dfloat_index_f
+        return int(f(op.encode(), x.size, x.ctypes.data_as(C.c_void_p)))
+    f = lib.numo_sfloat_f if x.dtype == np.float32 else lib.numo_dfloat_f
+    return f(op.encode(), x.size, x.ctypes.data_as(C.c_void_p))
+
+
+# ---- oracle/_ref: the reference's own real_accum.h ---------------------------------
+def ref_available():
+    return os.path.exists(REF_LIB)
+
+
+_ref = None
+
+
+def _ref_lib():
+    global _ref
+    if _ref is None:
+        _ref = C.CDLL(REF_LIB)
+        for t in ("sfloat", "dfloat"):
+            f = getattr(_ref, t + "_ref_f")
+            f.restype = C.c_double
+            f.argtypes = [C.c_char_p, SZ, C.c_void_p, SSZ]
+            g = getattr(_ref, t + "_ref_index_f")
+            g.restype = C.c_int64
+            g.argtypes = [C.c_char_p, SZ, C.c_void_p, SSZ]
+    return _ref
+
+
+def ref_f1d(op, x):
+    """f_<op> of the reference's real_accum.h on a 1-d array (any stride)."""
+    r = _ref_lib()
+    t = "sfloat" if x.dtype == np.float32 else "dfloat"
+    p = C.c_void_p(x.__array_interface__["data"][0])
+    if op.endswith("_index") or op.endswith("_index_nan"):
+        return int(getattr(r, t + "_ref_index_f")(op.encode(), x.size, p, x.strides[0]))
+    return getattr(r, t + "_ref_f")(op.encode(), x.size, p, x.strides[0])

@@ -1,0 +1,98 @@
+"""Bit parity: packing, logical ops, count_true/count_false, Bit -> number.
+Everything here is bit-exact (test/bit_test.rb:19-72, test/narray_test.rb:2667-2860)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+import numo_oracle as oracle  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def test_bit_test_rb_literals():
+    # test/bit_test.rb:19-72
+    import cumo_amd
+    a = cumo_amd.Bit.cast([0, 1, 1, 0, 1, 0, 0, 1])
+    assert a.to_numpy().tolist() == [0, 1, 1, 0, 1, 0, 0, 1]
+    assert int(a.count_true()) == 4
+    assert int(a.count_false()) == 4
+    assert (~a).to_numpy().tolist() == [1, 0, 0, 1, 0, 1, 1, 0]
+    b = cumo_amd.Bit.cast([0, 0, 1, 1, 0, 0, 1, 1])
+    assert (a & b).to_numpy().tolist() == [0, 0, 1, 0, 0, 0, 0, 1]
+    assert (a | b).to_numpy().tolist() == [0, 1, 1, 1, 1, 0, 1, 1]
+    assert (a ^ b).to_numpy().tolist() == [0, 1, 0, 1, 1, 0, 1, 0]
+    assert a.eq(b).to_numpy().tolist() == [1, 0, 1, 0, 0, 1, 0, 0]
+    m = cumo_amd.Bit.cast([[0, 1, 1, 0], [1, 0, 0, 1]])
+    assert m.count_true(axis=0).to_numpy().tolist() == [1, 1, 1, 1]
+    assert m.count_true(axis=1).to_numpy().tolist() == [2, 2]
+    assert m.count_false(axis=1).to_numpy().tolist() == [2, 2]
+
+
+@pytest.mark.parametrize("n", [1, 5, 31, 32, 33, 63, 64, 65, 200, 1000, 100003, 1 << 20])
+def test_long_arrays_and_views(n):
+    import cumo_amd
+    rng = np.random.default_rng(300 + n)
+    ha = rng.integers(0, 2, size=n).astype(np.uint8)
+    hb = rng.integers(0, 2, size=n).astype(np.uint8)
+    a, b = cumo_amd.Bit.cast(ha), cumo_amd.Bit.cast(hb)
+    assert (a.to_numpy() == ha).all()
+    assert ((a & b).to_numpy() == oracle.bit_binary("and", ha, hb)).all()
+    assert ((a | b).to_numpy() == oracle.bit_binary("or", ha, hb)).all()
+    assert ((a ^ b).to_numpy() == oracle.bit_binary("xor", ha, hb)).all()
+    assert (a.eq(b).to_numpy() == oracle.bit_binary("eq", ha, hb)).all()
+    assert ((~a).to_numpy() == oracle.bit_binary("not", ha)).all()
+    assert int(a.count_true()) == int(ha.sum())
+    assert int(a.count_false()) == int(n - ha.sum())
+    w = oracle.pack(ha)
+    if n > 40:
+        # views that start inside a word, skip, and run backwards
+        for sl in (slice(3, None), slice(5, n - 7), slice(None, None, 2), slice(1, None, 3), slice(None, None, -1), slice(n - 2, 3, -5)):
+            va, vb = a[sl], b[sl]
+            assert (va.to_numpy() == ha[sl]).all(), sl
+            assert int(va.count_true()) == int(ha[sl].sum()), sl
+            assert int(va.count_false()) == int((1 - ha[sl]).sum()), sl
+            start, stop, step = sl.indices(n)
+            cnt = len(range(start, stop, step))
+            assert int(va.count_true()) == oracle.bit_count(w, start, step, cnt), sl
+            assert ((va & vb).to_numpy() == (ha[sl] & hb[sl])).all(), sl
+            assert ((~va).to_numpy() == 1 - ha[sl]).all(), sl
+            assert (va.copy().to_numpy() == ha[sl]).all(), sl
+
+
+def test_count_along_axes_and_2d_views():
+    import cumo_amd
+    rng = np.random.default_rng(301)
+    h = rng.integers(0, 2, size=(13, 70, 9)).astype(np.uint8)
+    d = cumo_amd.Bit.cast(h)
+    for axis in [0, 1, 2, (0, 1), (1, 2), (0, 2), None]:
+        got = d.count_true(axis=axis)
+        got = got.to_numpy() if hasattr(got, "to_numpy") else got
+        assert (np.asarray(got) == h.sum(axis=axis)).all(), axis
+    t = d.transpose()
+    assert (t.count_true(axis=0).to_numpy() == h.transpose().sum(axis=0)).all()
+    assert (d[::2, 1::3].count_false(axis=1).to_numpy() == (1 - h[::2, 1::3]).sum(axis=1)).all()
+    assert d.count_true(axis=1, keepdims=True).shape == (13, 1, 9)
+    # logical ops on views that cannot be flattened (test/narray_test.rb:3500-3605)
+    a, b = d[:, ::2], d[:, 1::2]
+    assert ((a & b).to_numpy() == (h[:, ::2] & h[:, 1::2])).all()
+    assert ((a.transpose() | b.transpose()).to_numpy() == (h[:, ::2] | h[:, 1::2]).transpose()).all()
+    assert ((d & d[0]).to_numpy() == (h & h[0])).all()
+
+
+def test_compare_then_count_matches_popcount():
+    import cumo_amd
+    rng = np.random.default_rng(302)
+    h = rng.standard_normal((300, 1000)).astype(np.float32)
+    d = cumo_amd.SFloat.cast(h)
+    mask = d > 0.5
+    assert int(mask.count_true()) == int((h > 0.5).sum())
+    assert (mask.count_true(axis=1).to_numpy() == (h > 0.5).sum(axis=1)).all()
+    tm = d.transpose() > 0.5
+    assert int(tm.count_true()) == int((h > 0.5).sum())
+    assert (tm.to_numpy() == (h.T > 0.5)).all()
+    nums = mask._store_into(cumo_amd.Int32)
+    assert (nums.to_numpy() == (h > 0.5)).all()
+    assert (mask._store_into(cumo_amd.DFloat).to_numpy() == oracle.store_bit(np.float64, (h > 0.5).astype(np.uint8))).all()

@@ -1,0 +1,310 @@
+"""Elementwise parity: the HIP path through the C-ABI against the CPU oracle on the
+same seeded inputs. Bit-exact for arithmetic that is a single IEEE operation, for
+Int32 and for Bit results; <= 1 ulp for libm functions."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+import numo_oracle as oracle  # noqa: E402
+
+from helpers import assert_bits_equal, assert_ulp  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = [("sfloat", np.float32), ("dfloat", np.float64)]
+PYOP = {"add": "__add__", "sub": "__sub__", "mul": "__mul__", "div": "__truediv__", "mod": "__mod__"}
+RPYOP = {"add": "__radd__", "sub": "__rsub__", "mul": "__rmul__", "div": "__rtruediv__", "mod": "__rmod__"}
+
+
+def cls_of(name):
+    import cumo_amd
+    return {"sfloat": cumo_amd.SFloat, "dfloat": cumo_amd.DFloat, "int32": cumo_amd.Int32}[name]
+
+
+def views_of(shape_kind, host, dev):
+    """Pairs (numpy view, device view) built by the same slicing."""
+    if shape_kind == "contig":
+        return host, dev
+    if shape_kind == "colslice":
+        return host[..., 1::2], dev[..., 1::2]
+    if shape_kind == "rowslice":
+        return host[::3], dev[::3]
+    if shape_kind == "transpose":
+        return host.T, dev.transpose()
+    if shape_kind == "reverse":
+        return host[::-1, ::-1], dev[::-1, ::-1]
+    if shape_kind == "offset":
+        return host[1:, 3:], dev[1:, 3:]
+    raise ValueError(shape_kind)
+
+
+VIEW_KINDS = ["contig", "colslice", "rowslice", "transpose", "reverse", "offset"]
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "mod"])
+@pytest.mark.parametrize("kind", VIEW_KINDS)
+def test_float_binary_over_views(tname, dt, op, kind):
+    rng = np.random.default_rng(100)
+    cls = cls_of(tname)
+    hx = rng.standard_normal((96, 200)).astype(dt)
+    hy = (rng.standard_normal((96, 200)) + 0.5).astype(dt)
+    hx[2, 5] = np.nan
+    hy[4, 7] = 0.0
+    dx, dy = cls.cast(hx), cls.cast(hy)
+    vx, wx = views_of(kind, hx, dx)
+    vy, wy = views_of(kind, hy, dy)
+    with np.errstate(all="ignore"):
+        want = oracle.binary(op, vx, vy)
+    got = getattr(wx, PYOP[op])(wy).to_numpy()
+    assert_bits_equal(got, want, "%s %s %s" % (tname, op, kind))
+    # scalar on either side
+    with np.errstate(all="ignore"):
+        assert_bits_equal(getattr(wx, PYOP[op])(2.5).to_numpy(), oracle.binary(op, vx, 2.5), "scalar right")
+        assert_bits_equal(getattr(wx, RPYOP[op])(2.5).to_numpy(), oracle.binary(op, 2.5, vx, scalar_is_left=True), "scalar left")
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_broadcast_shapes(tname, dt):
+    rng = np.random.default_rng(101)
+    cls = cls_of(tname)
+    a = rng.standard_normal((33, 64)).astype(dt)
+    for other_shape in [(1, 64), (64,), (33, 1), (1, 1), (1,)]:
+        b = rng.standard_normal(other_shape).astype(dt)
+        assert_bits_equal((cls.cast(a) + cls.cast(b)).to_numpy(), oracle.binary("add", a, b), str(other_shape))
+        assert_bits_equal((cls.cast(b) - cls.cast(a)).to_numpy(), oracle.binary("sub", b, a), str(other_shape))
+    # more dims, both sides broadcasting
+    p = rng.standard_normal((5, 1, 7, 1)).astype(dt)
+    q = rng.standard_normal((4, 1, 9)).astype(dt)
+    assert_bits_equal((cls.cast(p) * cls.cast(q)).to_numpy(), oracle.binary("mul", p, q))
+    import cumo_amd
+    with pytest.raises(cumo_amd.ShapeError):
+        cls.cast(a) + cls.cast(np.zeros((32, 64), dtype=dt))
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_many_dims_and_permuted_views(tname, dt):
+    # past the reference's specialised accessors (ndim 5..8: test/narray_test.rb:41-51)
+    rng = np.random.default_rng(102)
+    cls = cls_of(tname)
+    for nd in (5, 6, 8):
+        shape = tuple(rng.integers(2, 4, size=nd))
+        h = rng.standard_normal(shape).astype(dt)
+        perm = tuple(rng.permutation(nd))
+        d = cls.cast(h)
+        got = (d.transpose(*perm) * 2.0 + d.transpose(*perm)).to_numpy()
+        want = oracle.binary("add", oracle.binary("mul", h.transpose(perm), 2.0), h.transpose(perm))
+        assert_bits_equal(got, want, "nd=%d" % nd)
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("n", [0, 1, 3, 31, 32, 33, 255, 256, 257, 1023, 4097, 100003])
+def test_sizes_and_tails(tname, dt, n):
+    rng = np.random.default_rng(103 + n)
+    cls = cls_of(tname)
+    hx = rng.standard_normal(n).astype(dt)
+    hy = rng.standard_normal(n).astype(dt)
+    got = (cls.cast(hx) * 2.5 + cls.cast(hy)).to_numpy()
+    want = oracle.binary("add", oracle.binary("mul", hx, 2.5), hy) if n else np.zeros(0, dtype=dt)
+    assert_bits_equal(got, want)
+    # unaligned start: a view one element in
+    if n > 4:
+        got = (cls.cast(hx)[1:] + cls.cast(hy)[:-1]).to_numpy()
+        assert_bits_equal(got, oracle.binary("add", hx[1:], hy[:-1]))
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_unary_and_rounding(tname, dt):
+    rng = np.random.default_rng(104)
+    cls = cls_of(tname)
+    h = (rng.standard_normal((40, 50)) * 7).astype(dt)
+    h[0, :6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 2.5]
+    d = cls.cast(h)
+    for view in ("contig", "transpose", "colslice"):
+        hv, dv = views_of(view, h, d)
+        for name in ["minus", "square", "sign", "floor", "round", "ceil", "trunc", "rint", "abs", "reciprocal"]:
+            with np.errstate(all="ignore"):
+                want = oracle.unary(name, hv)
+            assert_bits_equal(getattr(dv, name)().to_numpy(), want, "%s %s" % (name, view))
+
+
+MATH1 = ["sqrt", "cbrt", "log", "log2", "log10", "exp", "exp2", "exp10", "sin", "cos", "tan", "asin", "acos", "atan", "sinh",
+         "cosh", "tanh", "asinh", "acosh", "atanh", "sinc", "erf", "erfc", "log1p", "expm1"]
+
+
+def _math_domain(name, rng, dt):
+    x = rng.standard_normal(20000).astype(dt) * 3
+    if name in ("sqrt", "log", "log2", "log10"):
+        x = np.abs(x) + dt(1e-3)
+    elif name in ("asin", "acos", "atanh"):
+        x = np.clip(x / 4, -0.99, 0.99).astype(dt)
+    elif name == "acosh":
+        x = np.abs(x) + dt(1)
+    elif name == "log1p":
+        x = np.abs(x)
+    elif name in ("exp10",):
+        x = x * 2
+    return x
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("name", MATH1)
+def test_nmath(tname, dt, name):
+    """SFloat: the function is evaluated in double and rounded once, like the host
+    macro, so it lands within 1 ulp of the oracle (double rounding of two double
+    libms that differ in the last bit). DFloat: device libm against glibc, both
+    within 1 ulp of the true value for these functions, so within 2 of each other;
+    the last ulp of glibc on another machine is not pinned by anything."""
+    import cumo_amd
+    rng = np.random.default_rng(105)
+    cls = cls_of(tname)
+    x = _math_domain(name, rng, dt)
+    got = getattr(cumo_amd.NMath, name)(cls.cast(x)).to_numpy()
+    want = oracle.unary(name, x)
+    assert_ulp(got, want, 1 if dt == np.float32 else 2, "%s %s" % (tname, name))
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_nmath_two_args(tname, dt):
+    import cumo_amd
+    rng = np.random.default_rng(106)
+    cls = cls_of(tname)
+    x = rng.standard_normal((50, 40)).astype(dt)
+    y = rng.standard_normal((50, 40)).astype(dt)
+    for name in ("atan2", "hypot"):
+        f = getattr(cumo_amd.NMath, name)
+        assert_ulp(f(cls.cast(x), cls.cast(y)).to_numpy(), oracle.binary(name, x, y), 1 if dt == np.float32 else 2, name)
+        assert_ulp(f(cls.cast(x), 0.5).to_numpy(), oracle.binary(name, x, 0.5), 1 if dt == np.float32 else 2, name)
+        assert_ulp(f(0.5, cls.cast(x)).to_numpy(), oracle.binary(name, 0.5, x, scalar_is_left=True), 1 if dt == np.float32 else 2, name)
+    assert_bits_equal(cls.cast(x).copysign(cls.cast(y)).to_numpy(), oracle.binary("copysign", x, y))
+
+
+def test_int32_arithmetic():
+    rng = np.random.default_rng(107)
+    cls = cls_of("int32")
+    hx = rng.integers(-100000, 100000, size=(70, 90), dtype=np.int32)
+    hy = rng.integers(1, 300, size=(70, 90), dtype=np.int32) * rng.choice(np.array([-1, 1], dtype=np.int32), size=(70, 90))
+    dx, dy = cls.cast(hx), cls.cast(hy)
+    for kind in ("contig", "transpose", "colslice", "reverse"):
+        vx, wx = views_of(kind, hx, dx)
+        vy, wy = views_of(kind, hy, dy)
+        for op in ("add", "sub", "mul", "div", "mod"):
+            assert_bits_equal(getattr(wx, PYOP[op])(wy).to_numpy(), oracle.binary(op, vx, vy), "%s %s" % (op, kind))
+            assert_bits_equal(getattr(wx, PYOP[op])(7).to_numpy(), oracle.binary(op, vx, 7), "%s scalar" % op)
+        assert_bits_equal((wx & wy).to_numpy(), oracle.binary("bit_and", vx, vy))
+        assert_bits_equal((wx | wy).to_numpy(), oracle.binary("bit_or", vx, vy))
+        assert_bits_equal((wx ^ wy).to_numpy(), oracle.binary("bit_xor", vx, vy))
+        assert_bits_equal((~wx).to_numpy(), oracle.unary("bit_not", vx))
+        assert_bits_equal((-wx).to_numpy(), oracle.unary("minus", vx))
+        assert_bits_equal(wx.abs().to_numpy(), oracle.unary("abs", vx))
+        assert_bits_equal(wx.square().to_numpy(), oracle.unary("square", vx))
+        assert_bits_equal(wx.sign().to_numpy(), oracle.unary("sign", vx))
+    sh = cls.cast((np.abs(hy) % 31).astype(np.int32))
+    assert_bits_equal((dx >> sh).to_numpy(), oracle.binary("right_shift", hx, (np.abs(hy) % 31).astype(np.int32)))
+    small = (np.abs(hx) % 1000).astype(np.int32)
+    sh2 = (np.abs(hy) % 20).astype(np.int32)
+    assert_bits_equal((cls.cast(small) << cls.cast(sh2)).to_numpy(), oracle.binary("left_shift", small, sh2))
+    # scalar on the left of a non-commutative op
+    assert_bits_equal((7000 - dx).to_numpy(), oracle.binary("sub", 7000, hx, scalar_is_left=True))
+    assert_bits_equal((7000 / dy).to_numpy(), oracle.binary("div", 7000, hy, scalar_is_left=True))
+    # Float on Int32 upcasts to DFloat (reference: gen/def/int32.rb:22-23)
+    import cumo_amd
+    r = dx * 0.5
+    assert isinstance(r, cumo_amd.DFloat)
+    assert_bits_equal(r.to_numpy(), hx.astype(np.float64) * 0.5)
+
+
+def test_int32_error_flags():
+    # reference: test/narray_test.rb:4887-4905 -- the flag raises, also through views,
+    # and the rejected element is left alone
+    cls = cls_of("int32")
+    x = cls.cast(np.array([[6, 7, 8], [9, 10, 11]], dtype=np.int32))
+    y = cls.cast(np.array([[2, 0, 4], [3, 5, 1]], dtype=np.int32))
+    with pytest.raises(ZeroDivisionError):
+        x / y
+    with pytest.raises(ZeroDivisionError):
+        x % y
+    with pytest.raises(ZeroDivisionError):
+        x.transpose() / y.transpose()
+    with pytest.raises(ZeroDivisionError):
+        x / 0
+    assert (x / y[:, 2:]).to_numpy().tolist() == [[1, 1, 2], [9, 10, 11]]
+    with pytest.raises(ValueError):
+        cls.cast(np.array([1, -2**31], dtype=np.int32)).abs()
+    with pytest.raises(ZeroDivisionError):
+        cls.cast(np.array([1, 0], dtype=np.int32)).reciprocal()
+    assert cls.cast(np.array([1, -1, 5], dtype=np.int32)).reciprocal().to_numpy().tolist() == [1, -1, 0]
+
+
+@pytest.mark.parametrize("src,dst", [("sfloat", "dfloat"), ("dfloat", "sfloat"), ("int32", "sfloat"), ("int32", "dfloat"),
+                                     ("sfloat", "int32"), ("dfloat", "int32"), ("sfloat", "sfloat"), ("int32", "int32")])
+def test_casts_and_copies(src, dst):
+    rng = np.random.default_rng(108)
+    npdt = {"sfloat": np.float32, "dfloat": np.float64, "int32": np.int32}
+    h = (rng.standard_normal((64, 48)) * 1000).astype(npdt[src])
+    d = cls_of(src).cast(h)
+    for kind in ("contig", "transpose", "colslice", "rowslice"):
+        hv, dv = views_of(kind, h, d)
+        assert_bits_equal(cls_of(dst).cast(dv).to_numpy(), oracle.store(npdt[dst], hv), "%s->%s %s" % (src, dst, kind))
+        assert_bits_equal(dv.copy().to_numpy(), oracle.copy(hv))
+    # mixed-type binary op upcasts (reference: gen/def/*.rb upcast tables)
+    if src != dst:
+        a, b = cls_of(src).cast(h), cls_of(dst).cast(h.astype(npdt[dst]))
+        r = a + b
+        rank = {"int32": 0, "sfloat": 1, "dfloat": 2}
+        assert r.type_name == (src if rank[src] > rank[dst] else dst)
+
+
+def test_fill_and_store_into_views():
+    cls = cls_of("sfloat")
+    a = cls.zeros(6, 8)
+    a[::2, 1::3].fill(7.5)
+    want = np.zeros((6, 8), dtype=np.float32)
+    want[::2, 1::3] = 7.5
+    assert_bits_equal(a.to_numpy(), want)
+    b = cls_of("dfloat").cast(np.arange(8, dtype=np.float64))
+    a[1].store(b)
+    want[1] = np.arange(8)
+    assert_bits_equal(a.to_numpy(), want)
+    i = cls_of("int32").zeros(5).fill(-3)
+    assert i.to_numpy().tolist() == [-3] * 5
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+@pytest.mark.parametrize("op", ["eq", "ne", "gt", "ge", "lt", "le"])
+def test_compare_into_bit(tname, dt, op):
+    rng = np.random.default_rng(109)
+    cls = cls_of(tname)
+    for shape in [(1,), (31,), (32,), (33,), (64,), (1000,), (5, 67), (7, 64), (3, 5, 96), (129, 33)]:
+        hx = rng.integers(-3, 4, size=shape).astype(dt)
+        hy = rng.integers(-3, 4, size=shape).astype(dt)
+        if dt != np.int32:
+            hx.reshape(-1)[0] = np.nan
+        dx, dy = cls.cast(hx), cls.cast(hy)
+        assert (getattr(dx, op)(dy).to_numpy() == oracle.compare(op, hx, hy)).all(), (shape, op)
+        assert (getattr(dx, op)(1).to_numpy() == oracle.compare(op, hx, 1)).all(), (shape, op, "scalar")
+        if len(shape) == 2:
+            assert (getattr(dx.transpose(), op)(dy.transpose()).to_numpy() == oracle.compare(op, hx.T, hy.T)).all(), (shape, op, "T")
+            assert (getattr(dx[:, ::2], op)(0).to_numpy() == oracle.compare(op, hx[:, ::2], 0)).all()
+            assert (getattr(dx, op)(dy[0]).to_numpy() == oracle.compare(op, hx, hy[0])).all(), (shape, op, "bcast")
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_float_classification(tname, dt):
+    cls = cls_of(tname)
+    rng = np.random.default_rng(110)
+    h = rng.standard_normal(5000).astype(dt)
+    h[::7] = np.nan
+    h[1::11] = np.inf
+    h[2::13] = -np.inf
+    h[3::17] = -0.0
+    d = cls.cast(h)
+    for name in ("isnan", "isinf", "isposinf", "isneginf", "isfinite", "signbit"):
+        assert (getattr(d, name)().to_numpy() == oracle.cond_unary(name, h)).all(), name
+        assert (getattr(d[5::3], name)().to_numpy() == oracle.cond_unary(name, h[5::3])).all(), name
+    x = np.array([1.0, 1.0 + 1e-7, 1.001, 0.0], dtype=dt)
+    y = np.array([1.0, 1.0, 1.0, 0.0], dtype=dt)
+    assert (cls.cast(x).nearly_eq(cls.cast(y)).to_numpy() == oracle.compare("nearly_eq", x, y)).all()

@@ -1,0 +1,186 @@
+"""Reduction parity: the HIP reduction engine through the C-ABI against the CPU
+oracle. Integer results, min/max values and every index are bit-exact; float sums
+and moments are within rel 1e-5*log2(n) (SFloat) / 1e-12*log2(n) (DFloat) of the
+oracle's sequential answer, scaled by sum(|x|) because a sum of signed values has
+no scale of its own."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+import numo_oracle as oracle  # noqa: E402
+
+from helpers import assert_bits_equal, assert_reduction_close  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = [("sfloat", np.float32), ("dfloat", np.float64)]
+
+
+def cls_of(name):
+    import cumo_amd
+    return {"sfloat": cumo_amd.SFloat, "dfloat": cumo_amd.DFloat, "int32": cumo_amd.Int32}[name]
+
+
+def red_n(shape, axis):
+    if axis is None:
+        return int(np.prod(shape))
+    ax = (axis,) if isinstance(axis, int) else axis
+    return int(np.prod([shape[a] for a in ax]))
+
+
+def abs_sum(h, axis, keepdims=False):
+    return np.abs(h.astype(np.float64)).sum(axis=axis, keepdims=keepdims)
+
+
+VIEWS = {
+    "contig": lambda a: a,
+    "colslice": lambda a: a[..., 1::2],
+    "rowslice": lambda a: a[::2],
+    "transpose": lambda a: a.transpose(),
+    "reverse": lambda a: a[::-1],
+    "middle": lambda a: a[:, 1:-1] if a.ndim > 1 else a[1:-1],
+}
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("view", list(VIEWS))
+def test_float_reductions_every_axis(tname, dt, view):
+    # the pattern of test/narray_test.rb:3449-3486,4329-4363: every reduction over every
+    # axis of several kinds of view
+    rng = np.random.default_rng(200)
+    cls = cls_of(tname)
+    h = (rng.integers(-64, 64, size=(12, 20, 36)) / 16.0).astype(dt)  # multiples of 1/16: many ties
+    d = cls.cast(h)
+    hv, dv = VIEWS[view](h), VIEWS[view](d)
+    for axis in [None, 0, 1, 2, -1, (0, 1), (1, 2), (0, 2)]:
+        n = red_n(hv.shape, axis if axis != -1 else 2)
+        for name in ("min", "max", "ptp"):
+            assert_bits_equal(getattr(dv, name)(axis=axis).to_numpy(), oracle.reduce(name, hv, axis=axis), "%s %s %r" % (name, view, axis))
+        for name in ("argmin", "argmax"):
+            assert_bits_equal(getattr(dv, name)(axis=axis).to_numpy(), oracle.reduce(name, hv, axis=axis), "%s %s %r" % (name, view, axis))
+        # sums of multiples of 1/16 this small are exact in any order
+        assert_bits_equal(dv.sum(axis=axis).to_numpy(), oracle.reduce("sum", hv, axis=axis), "sum %s %r" % (view, axis))
+        assert_reduction_close(dv.mean(axis=axis).to_numpy(), oracle.reduce("mean", hv, axis=axis), n, abs_sum(hv, axis) / n, "mean")
+        for name in ("var", "stddev", "rms"):
+            want = oracle.reduce(name, hv, axis=axis)
+            assert_reduction_close(getattr(dv, name)(axis=axis).to_numpy(), want, n, np.abs(want) + 1e-30, "%s %s %r" % (name, view, axis))
+        lo, hi = dv.minmax(axis=axis)
+        assert_bits_equal(lo.to_numpy(), oracle.reduce("min", hv, axis=axis))
+        assert_bits_equal(hi.to_numpy(), oracle.reduce("max", hv, axis=axis))
+    # keepdims
+    assert dv.sum(axis=1, keepdims=True).shape == tuple(1 if k == 1 else s for k, s in enumerate(hv.shape))
+    assert_bits_equal(dv.max(axis=(0, 2), keepdims=True).to_numpy(), oracle.reduce("max", hv, axis=(0, 2), keepdims=True))
+    # max_index / min_index answer positions in the view's own flattening
+    assert_bits_equal(dv.max_index(axis=1).to_numpy(), oracle.reduce("max_index", np.ascontiguousarray(hv), axis=1))
+    assert_bits_equal(dv.min_index().to_numpy(), oracle.reduce("min_index", np.ascontiguousarray(hv)))
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("shape,axis", [((1000003,), None), ((7, 100000), 1), ((100000, 7), 0), ((3, 40000, 5), 1),
+                                        ((64, 64, 64), (0, 2)), ((2, 3), None), ((1,), None), ((70000, 3), 1),
+                                        ((5, 8192), 1), ((4096, 33), 0), ((33, 4096), 0)])
+def test_random_float_sums(tname, dt, shape, axis):
+    rng = np.random.default_rng(201)
+    cls = cls_of(tname)
+    h = rng.uniform(-1, 1, size=shape).astype(dt)
+    d = cls.cast(h)
+    n = red_n(shape, axis)
+    sc = abs_sum(h, axis)
+    assert_reduction_close(d.sum(axis=axis).to_numpy(), oracle.reduce("sum", h, axis=axis), n, sc, "sum")
+    assert_reduction_close(d.mean(axis=axis).to_numpy(), oracle.reduce("mean", h, axis=axis), n, sc / n, "mean")
+    want = oracle.reduce("var", h, axis=axis)
+    if n > 1:
+        assert_reduction_close(d.var(axis=axis).to_numpy(), want, n, np.abs(want), "var")
+        want = oracle.reduce("stddev", h, axis=axis)
+        assert_reduction_close(d.stddev(axis=axis).to_numpy(), want, n, np.abs(want), "stddev")
+    want = oracle.reduce("rms", h, axis=axis)
+    assert_reduction_close(d.rms(axis=axis).to_numpy(), want, n, np.abs(want), "rms")
+    assert_bits_equal(d.max(axis=axis).to_numpy(), oracle.reduce("max", h, axis=axis))
+    assert_bits_equal(d.min(axis=axis).to_numpy(), oracle.reduce("min", h, axis=axis))
+    assert_bits_equal(d.argmax(axis=axis).to_numpy(), oracle.reduce("argmax", h, axis=axis))
+    assert_bits_equal(d.argmin(axis=axis).to_numpy(), oracle.reduce("argmin", h, axis=axis))
+    p = oracle.reduce("prod", (h[..., :20] if h.ndim > 1 else h[:20]) * 1.5, axis=-1)
+    dp = cls.cast(np.ascontiguousarray((h[..., :20] if h.ndim > 1 else h[:20]) * dt(1.5)))
+    assert_reduction_close(dp.prod(axis=-1).to_numpy(), p, 20, np.abs(p), "prod")
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_nan_rules(tname, dt):
+    rng = np.random.default_rng(202)
+    cls = cls_of(tname)
+    h = rng.standard_normal((9, 3000)).astype(dt)
+    h[0, 5] = np.nan          # one NaN
+    h[1, :] = np.nan          # a whole row
+    h[2, 0] = np.nan          # leading
+    h[3, -1] = np.nan         # trailing
+    h[4, ::2] = np.nan        # half
+    h[5, 100] = np.inf
+    h[6, 200] = -np.inf
+    d = cls.cast(h)
+    for nan in (False, True):
+        for name in ("min", "max", "ptp", "argmin", "argmax"):
+            assert_bits_equal(getattr(d, name)(axis=1, nan=nan).to_numpy(), oracle.reduce(name, h, axis=1, nan=nan), "%s nan=%s" % (name, nan))
+            assert_bits_equal(getattr(d, name)(axis=0, nan=nan).to_numpy(), oracle.reduce(name, h, axis=0, nan=nan), "%s nan=%s axis0" % (name, nan))
+        for name in ("sum", "mean", "rms"):
+            want = oracle.reduce(name, h, axis=1, nan=nan)
+            got = getattr(d, name)(axis=1, nan=nan).to_numpy()
+            fin = np.isfinite(want)
+            assert (np.isnan(got) == np.isnan(want)).all(), name
+            assert_reduction_close(got[fin], want[fin], 3000, np.nansum(np.abs(h[fin].astype(np.float64)), axis=1) if name == "sum" else np.abs(want[fin]) + 1e-3, name)
+        for name in ("var", "stddev"):
+            want = oracle.reduce(name, h[:5], axis=1, nan=nan)
+            got = getattr(d[:5], name)(axis=1, nan=nan).to_numpy()
+            assert (np.isnan(got) == np.isnan(want)).all(), name
+            fin = np.isfinite(want)
+            assert_reduction_close(got[fin], want[fin], 3000, np.abs(want[fin]), name)
+    lo, hi = d.minmax(axis=1, nan=True)
+    assert_bits_equal(lo.to_numpy(), oracle.reduce("min", h, axis=1, nan=True))
+    assert_bits_equal(hi.to_numpy(), oracle.reduce("max", h, axis=1, nan=True))
+    # signed zeros: the earlier of two equal elements (test/narray_test.rb:667-672), also across lanes
+    z = np.zeros(5000, dtype=dt)
+    z[1::2] = -0.0
+    for arr in (z, -z, z[::-1].copy()):
+        dz = cls.cast(arr)
+        assert_bits_equal(dz.min().to_numpy(), oracle.reduce("min", arr))
+        assert_bits_equal(dz.max().to_numpy(), oracle.reduce("max", arr))
+
+
+def test_int32_reductions():
+    rng = np.random.default_rng(203)
+    cls = cls_of("int32")
+    h = rng.integers(-2**30, 2**30, size=(17, 33, 20), dtype=np.int32)
+    d = cls.cast(h)
+    for view in VIEWS:
+        hv, dv = VIEWS[view](h), VIEWS[view](d)
+        for axis in [None, 0, 1, 2, (0, 2)]:
+            for name in ("sum", "min", "max", "ptp", "argmin", "argmax"):
+                assert_bits_equal(getattr(dv, name)(axis=axis).to_numpy(), oracle.reduce(name, hv, axis=axis), "%s %s %r" % (name, view, axis))
+    small = rng.integers(-3, 4, size=(6, 12), dtype=np.int32)
+    assert_bits_equal(cls.cast(small).prod(axis=1).to_numpy(), oracle.reduce("prod", small, axis=1))
+    lo, hi = d.minmax(axis=1)
+    assert_bits_equal(lo.to_numpy(), h.min(axis=1))
+    assert_bits_equal(hi.to_numpy(), h.max(axis=1))
+    big = rng.integers(-2**31, 2**31 - 1, size=3000001, dtype=np.int32)
+    assert int(cls.cast(big).sum()) == int(big.astype(np.int64).sum())
+    assert cls.cast(big).sum().to_numpy().dtype == np.int64
+
+
+def test_empty_and_degenerate():
+    import cumo_amd
+    a = cumo_amd.SFloat.zeros(0, 5)
+    assert a.sum(axis=0).to_numpy().tolist() == [0.0] * 5   # reducing an empty axis leaves the identity... and
+    assert cumo_amd.SFloat.zeros(4, 0).sum(axis=0).shape == (0,)
+    with pytest.raises(ValueError):
+        cumo_amd.SFloat.zeros(0).max()
+    one = cumo_amd.DFloat.cast(np.array([[3.5]]))
+    assert float(one.sum()) == 3.5 and float(one.max(axis=0).to_numpy()[0]) == 3.5
+    assert int(one.argmax()) == 0
+
+
+def test_dfloat_kahan_sum():
+    import cumo_amd
+    h = np.array([1e16, 1.0, -1e16, 1.0] * 1000)
+    assert float(cumo_amd.DFloat.cast(h).kahan_sum()) == 2000.0
