@@ -1,0 +1,316 @@
+#!/usr/bin/env python3
+"""Benchmark of the array hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all-configs] [--no-cpu]
+
+Prints ONE JSON line. A "step" is one pass of the headline workload (BASELINE.json
+configs[1]: DFloat broadcast add + row reductions) with the inputs already resident
+in HBM: C = A + r; C.sum(axis:1); C.max(axis:1) -- three launches through the
+C-ABI. `value` is algorithmic bytes per step / seconds per step in GB/s, where
+algorithmic bytes count every distinct input element once and every output element
+once (the reference's own convention, bench/cumo_probe.rb:74-232).
+
+`roofline` covers the dominant kernel of the step (the broadcast add, 256 MiB of
+the step's 512 MiB), timed per launch with HIP events on the stream the launchers
+use. `cpu_baseline` times the Numo-shaped single-thread C loops of the oracle on the
+same workload on this machine's host cores. `per_config` lists every op of the five
+BASELINE configs (filled with --all-configs, which the default run also does with
+few iterations).
+
+Everything runs on one GPU; --gpus N with N > 1 exits with a message.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+METRIC = "achieved HBM GB/s (% of MI355X peak) and GElem/s vs Numo CPU, per config"
+MIB = 1 << 20
+
+
+# ---------------------------------------------------------------------------
+# synthetic inputs (host generated, seeded; neither library's own rand is usable
+# because Cumo draws from Philox and Numo from SFMT)
+# ---------------------------------------------------------------------------
+def inputs_c1(n=1 << 20):
+    rng = np.random.default_rng(0)
+    return {"x": rng.uniform(-1, 1, n).astype(np.float32), "b": rng.uniform(-1, 1, n).astype(np.float32)}
+
+
+def inputs_c2(n=4096):
+    rng = np.random.default_rng(1)
+    return {"A": rng.standard_normal((n, n)), "r": rng.standard_normal((1, n))}
+
+
+def inputs_c3(shape=(64, 512, 1024)):
+    rng = np.random.default_rng(2)
+    u = rng.random(shape, dtype=np.float32)
+    return {"T": (np.floor(u * 128) / 16 - 4).astype(np.float32)}  # multiples of 1/16 in [-4, 4): ties
+
+
+def inputs_c4(n=8192):
+    rng = np.random.default_rng(3)
+    m = rng.standard_normal((n, n), dtype=np.float32)
+    i = np.random.default_rng(4).integers(0, 1000, size=(n, n), dtype=np.int32)
+    return {"M": m, "I": i}
+
+
+def inputs_c5(s_shape=(32, 16, 512, 512), x_shape=(8192, 4096)):
+    rng = np.random.default_rng(4)
+    s = rng.standard_normal(s_shape, dtype=np.float32) * np.float32(2.0)  # N(0,2) read as sigma = 2
+    x = rng.standard_normal(x_shape, dtype=np.float32)
+    return {"S": s, "X": x}
+
+
+# ---------------------------------------------------------------------------
+# the five configs as chains of ops; every entry: (label, fn(env) -> result stored under label, bytes, elements)
+# ---------------------------------------------------------------------------
+def config_ops(name, cumo, host):
+    """Returns (env, ops). env holds the device-resident inputs; ops is a list of
+    (label, callable(env), algorithmic_bytes, elements)."""
+    NM = cumo.NMath
+    if name in ("c1", "c1_large"):
+        n = host["x"].size
+        env = {"x": cumo.SFloat.cast(host["x"]), "b": cumo.SFloat.cast(host["b"])}
+        return env, [
+            ("t=2.5*x", lambda e: e.__setitem__("t", 2.5 * e["x"]), 8 * n, n),
+            ("y=t+b", lambda e: e.__setitem__("y", e["t"] + e["b"]), 12 * n, n),
+            ("s=y.sum", lambda e: e.__setitem__("s", e["y"].sum()), 4 * n + 4, n),
+        ]
+    if name == "c2":
+        n = host["A"].shape[0]
+        env = {"A": cumo.DFloat.cast(host["A"]), "r": cumo.DFloat.cast(host["r"])}
+        full, vec = 8 * n * n, 8 * n
+        return env, [
+            ("C=A+r", lambda e: e.__setitem__("C", e["A"] + e["r"]), 2 * full + vec, n * n),
+            ("C.sum(axis:1)", lambda e: e.__setitem__("sum", e["C"].sum(axis=1)), full + vec, n * n),
+            ("C.max(axis:1)", lambda e: e.__setitem__("max", e["C"].max(axis=1)), full + vec, n * n),
+        ]
+    if name == "c3":
+        t = host["T"]
+        env = {"T": cumo.SFloat.cast(t)}
+        nb, n = t.nbytes, t.size
+        ops = []
+        for red in ("sum", "mean", "max", "min"):
+            for axis, out in ((0, t.shape[1] * t.shape[2]), (2, t.shape[0] * t.shape[1]), (None, 1)):
+                label = "T.%s(%s)" % (red, "axis:%d" % axis if axis is not None else "")
+                ops.append((label, (lambda r, a, l: lambda e: e.__setitem__(l, getattr(e["T"], r)(axis=a)))(red, axis, label), nb + 4 * out, n))
+        for red in ("argmax", "argmin"):
+            label = "T.%s(axis:2)" % red
+            ops.append((label, (lambda r, l: lambda e: e.__setitem__(l, getattr(e["T"], r)(axis=2)))(red, label), nb + 4 * t.shape[0] * t.shape[1], n))
+        return env, ops
+    if name == "c4":
+        m, i = host["M"], host["I"]
+        env = {"M": cumo.SFloat.cast(m), "I": cumo.Int32.cast(i)}
+        env["V"] = env["M"].transpose()[:, ::2]   # V = M.transpose[true, (0..-1).step(2)]: V[i,j] = M[2j,i]
+        nv = env["V"].size
+        rows = len(range(0, i.shape[0], 3))
+        return env, [
+            ("E0=NMath.exp(V)", lambda e: e.__setitem__("E0", NM.exp(e["V"])), 8 * nv, nv),
+            ("E=E0-1.0", lambda e: e.__setitem__("E", e["E0"] - 1.0), 8 * nv, nv),
+            ("mask=E>0.5", lambda e: e.__setitem__("mask", e["E"] > 0.5), 4 * nv + nv // 8, nv),
+            ("mask.count_true", lambda e: e.__setitem__("cnt", e["mask"].count_true()), nv // 8 + 8, nv),
+            ("I[(0..-1).step(3),true].copy", lambda e: e.__setitem__("Ic", e["I"][::3].copy()), 2 * 4 * rows * i.shape[1], rows * i.shape[1]),
+        ]
+    if name == "c5":
+        s, x = host["S"], host["X"]
+        env = {"S": cumo.SFloat.cast(s), "X": cumo.SFloat.cast(x)}
+        ns, nx = s.size, x.size
+        rs, rx = ns // s.shape[-1], x.shape[0]
+        return env, [
+            ("m=S.max(axis:-1,keepdims)", lambda e: e.__setitem__("m", e["S"].max(axis=-1, keepdims=True)), 4 * ns + 4 * rs, ns),
+            ("d=S-m", lambda e: e.__setitem__("d", e["S"] - e["m"]), 8 * ns + 4 * rs, ns),
+            ("e=NMath.exp(d)", lambda e: e.__setitem__("e", NM.exp(e["d"])), 8 * ns, ns),
+            ("z=e.sum(axis:-1,keepdims)", lambda e: e.__setitem__("z", e["e"].sum(axis=-1, keepdims=True)), 4 * ns + 4 * rs, ns),
+            ("p=e/z", lambda e: e.__setitem__("p", e["e"] / e["z"]), 8 * ns + 4 * rs, ns),
+            ("mean=X.mean(axis:-1,keepdims)", lambda e: e.__setitem__("mean", e["X"].mean(axis=-1, keepdims=True)), 4 * nx + 4 * rx, nx),
+            ("var=X.var(axis:-1,keepdims)", lambda e: e.__setitem__("var", e["X"].var(axis=-1, keepdims=True)), 4 * nx + 4 * rx, nx),
+            ("c=X-mean", lambda e: e.__setitem__("c", e["X"] - e["mean"]), 8 * nx + 4 * rx, nx),
+            ("v=var+1e-5", lambda e: e.__setitem__("v", e["var"] + 1e-5), 8 * rx, rx),
+            ("sd=NMath.sqrt(v)", lambda e: e.__setitem__("sd", NM.sqrt(e["v"])), 8 * rx, rx),
+            ("n=c/sd", lambda e: e.__setitem__("n", e["c"] / e["sd"]), 8 * nx + 4 * rx, nx),
+        ]
+    raise ValueError(name)
+
+
+HOST_INPUTS = {
+    "c1": inputs_c1, "c1_large": lambda: inputs_c1(1 << 26), "c2": inputs_c2, "c3": inputs_c3, "c4": inputs_c4, "c5": inputs_c5,
+}
+WORKLOAD_TEXT = {
+    "c1": "C1 SFloat axpy + full sum, n=2^20",
+    "c1_large": "C1 at n=2^26 (256 MiB per array)",
+    "c2": "C2 DFloat broadcast add + row reduce: A f64 [4096,4096] + r [1,4096]; C.sum(axis:1); C.max(axis:1)",
+    "c3": "C3 SFloat axis reductions on [64,512,1024]",
+    "c4": "C4 strided/transposed views on SFloat [8192,8192] + Int32 stride-3 row slice copy",
+    "c5": "C5 softmax [32,16,512,512] + layernorm statistics [8192,4096] composed from array ops",
+}
+
+
+class Timer:
+    def __init__(self, lib):
+        self.lib = lib
+        self.e0 = lib.cumo_hip_event_create()
+        self.e1 = lib.cumo_hip_event_create()
+
+    def time(self, fn):
+        self.lib.cumo_hip_event_record(self.e0)
+        fn()
+        self.lib.cumo_hip_event_record(self.e1)
+        return self.lib.cumo_hip_event_elapsed_ms(self.e0, self.e1)
+
+    def close(self):
+        self.lib.cumo_hip_event_destroy(self.e0)
+        self.lib.cumo_hip_event_destroy(self.e1)
+
+
+def measure_config(name, cumo, lib, iters, warmup):
+    host = HOST_INPUTS[name]()
+    env, ops = config_ops(name, cumo, host)
+    del host
+    timer = Timer(lib)
+    rows = []
+    for label, fn, nbytes, nelem in ops:
+        for _ in range(warmup):
+            fn(env)
+        ts = [timer.time(lambda: fn(env)) for _ in range(iters)]
+        ts.sort()
+        med = ts[len(ts) // 2]
+        best = ts[0]
+        rows.append({
+            "op": label, "bytes": int(nbytes), "ms_median": round(med, 5), "ms_best": round(best, 5),
+            "gbps": round(nbytes / (med * 1e-3) / 1e9, 1), "frac_of_peak": round(nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "gelem_s": round(nelem / (med * 1e-3) / 1e9, 2),
+        })
+    timer.close()
+    env.clear()
+    cumo.MemoryPool.free_all_blocks()
+    return rows
+
+
+def cpu_baseline_c2(budget_s=12.0):
+    """Numo-shaped single-thread C loops (the oracle's row loops) on the same C2
+    workload, on this machine's host cores. A bounded number of passes."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numo_oracle as oracle
+    lib = oracle.lib
+    h = inputs_c2()
+    a, r = h["A"], h["r"]
+    n = a.shape[0]
+    c = np.empty_like(a)
+    s = np.empty(n)
+    m = np.empty(n)
+    vp = lambda x: C.c_void_p(x.ctypes.data)
+    SZ, SSZ = C.c_size_t, C.c_ssize_t
+    lib.numo_rows_binary.restype = C.c_int
+    lib.numo_rows_reduce.restype = C.c_int
+
+    def one_pass():
+        lib.numo_rows_binary(b"add", 1, SZ(n), SZ(n), vp(a), SSZ(8 * n), SSZ(8), vp(r), SSZ(0), SSZ(8), vp(c), SSZ(8 * n), SSZ(8))
+        lib.numo_rows_reduce(b"sum", 1, SZ(n), SZ(n), vp(c), SSZ(8 * n), vp(s))
+        lib.numo_rows_reduce(b"max", 1, SZ(n), SZ(n), vp(c), SSZ(8 * n), vp(m))
+
+    one_pass()
+    t0 = time.perf_counter()
+    passes = 0
+    while passes < 2 or (time.perf_counter() - t0 < budget_s and passes < 200):
+        one_pass()
+        passes += 1
+    dt = (time.perf_counter() - t0) / passes
+    nbytes = 4 * 8 * n * n + 3 * 8 * n
+    return {
+        "value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": "%d passes of the full C2 step (A+r, row sum, row max on 4096x4096 f64), Numo-shaped single-thread C loops "
+                  "(oracle/numo_oracle.c numo_rows_*), gcc -O2, 1 of %d host cores; %.1f ms per pass" % (passes, os.cpu_count() or 0, dt * 1e3),
+        "ms_per_step": round(dt * 1e3, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--all-configs", action="store_true", help="measure every op of all five configs with full iteration counts")
+    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c3,c4,c5)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-per-config", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path has no cross-GPU stage)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import cumo_amd
+    from cumo_amd import _lib
+    lib = _lib.lib
+    if cumo_amd.device_count() < 1:
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+
+    # ---- headline step: C2 -------------------------------------------------------
+    host = inputs_c2()
+    env, ops = config_ops("c2", cumo_amd, host)
+    step_bytes = sum(o[2] for o in ops)
+
+    def step():
+        for _, fn, _, _ in ops:
+            fn(env)
+
+    for _ in range(args.warmup):
+        step()
+    cumo_amd.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    cumo_amd.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = step_bytes / (wall / args.steps) / 1e9
+
+    # dominant kernel, per launch, HIP events on the launch stream
+    timer = Timer(lib)
+    add_label, add_fn, add_bytes, _ = ops[0]
+    ts = sorted(timer.time(lambda: add_fn(env)) for _ in range(max(20, args.steps)))
+    timer.close()
+    avg_ms = sum(ts) / len(ts)
+    achieved = add_bytes / (avg_ms * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm", "kernel": "ew_rows_kernel<OpAdd<double>, 2> (C = A + r, f64 4096x4096 + 1x4096)",
+        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "bytes_per_launch": int(add_bytes), "avg_launch_ms": round(avg_ms, 5), "median_launch_ms": round(ts[len(ts) // 2], 5),
+        "traffic": None,
+    }
+    env.clear()
+    cumo_amd.MemoryPool.free_all_blocks()
+
+    per_config = {}
+    if not args.no_per_config:
+        names = [c for c in args.configs.split(",") if c] or ["c1", "c1_large", "c2", "c3", "c4", "c5"]
+        iters, warm = (30, 5) if args.all_configs else (7, 2)
+        for name in names:
+            per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm)}
+
+    out = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": WORKLOAD_TEXT["c2"], "bytes_per_step": int(step_bytes), "launches_per_step": 3,
+                   "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "gelem_per_s": round(3 * 4096 * 4096 / (wall / args.steps) / 1e9, 2)},
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_c2()
+    if per_config:
+        out["per_config"] = per_config
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -71,7 +71,7 @@ class ReducePlan(C.Structure):
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
-        "cumo_amd: %s is missing. Build it with `python -m cumo_amd.build` (needs hipcc); "
+        "cumo_amd: %s is missing. Build it with `python cumo_amd/build.py` (needs hipcc); "
         "there is no CPU fallback." % LIB_PATH)
 
 lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
@@ -90,6 +90,10 @@ _sig = {
     "cumo_hip_get_stream": (C.c_void_p, []),
     "cumo_hip_device_count": (C.c_int, []),
     "cumo_hip_synchronize": (None, []),
+    "cumo_hip_event_create": (C.c_void_p, []),
+    "cumo_hip_event_record": (None, [C.c_void_p]),
+    "cumo_hip_event_elapsed_ms": (C.c_float, [C.c_void_p, C.c_void_p]),
+    "cumo_hip_event_destroy": (None, [C.c_void_p]),
     "cumo_hip_memcpy_h2d": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_memcpy_d2h": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_memset": (None, [C.c_void_p, C.c_int, C.c_size_t]),

@@ -3,7 +3,9 @@
 One hipcc invocation per translation unit, run in parallel, then one link. The
 library is kept in-tree next to this file; nothing is installed.
 
-    python -m cumo_amd.build [-j N] [--force]
+    python cumo_amd/build.py [-j N] [--force]
+
+(run as a script, not with -m: importing the package loads the library)
 """
 import argparse
 import concurrent.futures

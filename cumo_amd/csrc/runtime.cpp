@@ -138,3 +138,29 @@ size_t* cumo_cuda_runtime_error_item_new(void) {
 }
 
 }  // extern "C"
+
+// Events on the stream the launchers use, for callers that time kernels
+// (the benchmark): create, record on the current stream, elapsed (waits for
+// the second event), destroy.
+extern "C" {
+
+void* cumo_hip_event_create(void) {
+    hipEvent_t ev = nullptr;
+    if (!hip_ok(hipEventCreate(&ev), "hipEventCreate")) return nullptr;
+    return (void*)ev;
+}
+
+void cumo_hip_event_record(void* ev) { hip_ok(hipEventRecord((hipEvent_t)ev, t_stream), "hipEventRecord"); }
+
+float cumo_hip_event_elapsed_ms(void* start, void* stop) {
+    float ms = 0.f;
+    if (!hip_ok(hipEventSynchronize((hipEvent_t)stop), "hipEventSynchronize")) return -1.f;
+    if (!hip_ok(hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime")) return -1.f;
+    return ms;
+}
+
+void cumo_hip_event_destroy(void* ev) {
+    if (ev) (void)hipEventDestroy((hipEvent_t)ev);
+}
+
+}  // extern "C"

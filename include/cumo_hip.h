@@ -329,6 +329,11 @@ void  cumo_hip_set_stream(void* hip_stream);
 void* cumo_hip_get_stream(void);
 int   cumo_hip_device_count(void);
 void  cumo_hip_synchronize(void);
+/* events on the current stream, for callers that time launches */
+void* cumo_hip_event_create(void);
+void  cumo_hip_event_record(void* event);
+float cumo_hip_event_elapsed_ms(void* start, void* stop);   /* waits for stop */
+void  cumo_hip_event_destroy(void* event);
 /* synchronous copies for host read-back/ingest (extract_cpu, to_a, from_binary) */
 void  cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n);
 void  cumo_hip_memcpy_d2h(void* dst, const void* src, size_t n);

@@ -704,7 +704,19 @@ int numo_reduce(const char *op, int dtype, int in_ndim, int out_ndim,
                 else j = (int64_t)i32_f_max_index(n, p);
             }
             if (j < 0) return -1;
-            if (is_index) j += (int64_t)(in_off / (ssize_t)elmsz);
+            if (is_index) {
+                /* position in the slice -> offset of that element from the start of
+                 * the array, in elements (tmpl/accum_index.c: the answer indexes the
+                 * flattened array) */
+                ssize_t off = in_off;
+                int64_t r = j;
+                for (int d = rnd; --d >= 0;) {
+                    int64_t nd_ = (int64_t)shape[out_ndim + d];
+                    off += (ssize_t)(r % nd_) * sin[out_ndim + d];
+                    r /= nd_;
+                }
+                j = (int64_t)(off / (ssize_t)elmsz);
+            }
             if (idx_bytes == 4) *(int32_t *)o = (int32_t)j; else *(int64_t *)o = j;
         } else if (dtype == T_SFLOAT) {
             float r = numo_sfloat_f(op, n, (const float *)scratch);
@@ -722,5 +734,60 @@ int numo_reduce(const char *op, int dtype, int in_ndim, int out_ndim,
             else return -1;
         }
     } while (iter_next(&it));
+    return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* Row loops for the CPU baseline timing. Numo's ndloop walks the outer */
+/* dimensions on the host and hands each innermost run to the iterator, */
+/* whose loop shapes are those of narray/gen/tmpl/binary.c:38-97: an    */
+/* indexed loop when every step is the element size, a pointer-bumping  */
+/* loop otherwise, the right operand read once when its step is 0.      */
+/* The benchmark times these, not the generic N-d driver above.         */
+/* ------------------------------------------------------------------ */
+#define ROW_LOOP(T, EXPR)                                                        \
+    for (size_t r = 0; r < nrows; ++r) {                                         \
+        const char *a = p1 + (ssize_t)r * r1, *b = p2 + (ssize_t)r * r2;         \
+        char *c = p3 + (ssize_t)r * r3;                                          \
+        if (s1 == (ssize_t)sizeof(T) && s2 == (ssize_t)sizeof(T) && s3 == (ssize_t)sizeof(T)) { \
+            const T *x_ = (const T *)a, *y_ = (const T *)b; T *z_ = (T *)c;      \
+            for (size_t i = 0; i < n; ++i) { T x = x_[i], y = y_[i]; z_[i] = (EXPR); } \
+        } else if (s2 == 0 && s1 == (ssize_t)sizeof(T) && s3 == (ssize_t)sizeof(T)) { \
+            const T *x_ = (const T *)a; T y = *(const T *)b; T *z_ = (T *)c;     \
+            for (size_t i = 0; i < n; ++i) { T x = x_[i]; z_[i] = (EXPR); }      \
+        } else {                                                                 \
+            for (size_t i = 0; i < n; ++i) {                                     \
+                T x = *(const T *)a, y = *(const T *)b;                          \
+                *(T *)c = (EXPR);                                                \
+                a += s1; b += s2; c += s3;                                       \
+            }                                                                    \
+        }                                                                        \
+    }
+
+#define ROWS_BY_OP(T)                                                            \
+    if (!strcmp(op, "add")) { ROW_LOOP(T, x + y) return 0; }                     \
+    if (!strcmp(op, "sub")) { ROW_LOOP(T, x - y) return 0; }                     \
+    if (!strcmp(op, "mul")) { ROW_LOOP(T, x * y) return 0; }                     \
+    if (!strcmp(op, "div")) { ROW_LOOP(T, x / y) return 0; }
+
+int numo_rows_binary(const char *op, int dtype, size_t nrows, size_t n,
+                     const char *p1, ssize_t r1, ssize_t s1,
+                     const char *p2, ssize_t r2, ssize_t s2,
+                     char *p3, ssize_t r3, ssize_t s3)
+{
+    if (dtype == T_SFLOAT) { ROWS_BY_OP(float) }
+    else if (dtype == T_DFLOAT) { ROWS_BY_OP(double) }
+    return -1;
+}
+
+/* one f_<op> per contiguous row (types/real_accum.h), result per row */
+int numo_rows_reduce(const char *op, int dtype, size_t nrows, size_t n,
+                     const char *p, ssize_t row_step, char *out)
+{
+    for (size_t r = 0; r < nrows; ++r) {
+        if (dtype == T_SFLOAT) ((float *)out)[r] = numo_sfloat_f(op, n, (const float *)(p + (ssize_t)r * row_step));
+        else if (dtype == T_DFLOAT) ((double *)out)[r] = numo_dfloat_f(op, n, (const double *)(p + (ssize_t)r * row_step));
+        else return -1;
+    }
     return 0;
 }

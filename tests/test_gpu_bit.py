@@ -24,7 +24,7 @@ def test_bit_test_rb_literals():
     assert (a & b).to_numpy().tolist() == [0, 0, 1, 0, 0, 0, 0, 1]
     assert (a | b).to_numpy().tolist() == [0, 1, 1, 1, 1, 0, 1, 1]
     assert (a ^ b).to_numpy().tolist() == [0, 1, 0, 1, 1, 0, 1, 0]
-    assert a.eq(b).to_numpy().tolist() == [1, 0, 1, 0, 0, 1, 0, 0]
+    assert a.eq(b).to_numpy().tolist() == [1, 0, 1, 0, 0, 1, 0, 1]
     m = cumo_amd.Bit.cast([[0, 1, 1, 0], [1, 0, 0, 1]])
     assert m.count_true(axis=0).to_numpy().tolist() == [1, 1, 1, 1]
     assert m.count_true(axis=1).to_numpy().tolist() == [2, 2]

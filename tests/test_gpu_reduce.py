@@ -35,6 +35,24 @@ def abs_sum(h, axis, keepdims=False):
     return np.abs(h.astype(np.float64)).sum(axis=axis, keepdims=keepdims)
 
 
+def exact_reduce(name, h, axis):
+    """The reduction in extended precision (x87 long double: 64-bit mantissa)."""
+    x = h.astype(np.longdouble)
+    if name == "sum":
+        r = x.sum(axis=axis)
+    elif name == "mean":
+        r = x.mean(axis=axis)
+    elif name == "var":
+        r = x.var(axis=axis, ddof=1)
+    elif name == "stddev":
+        r = np.sqrt(x.var(axis=axis, ddof=1))
+    elif name == "rms":
+        r = np.sqrt((x * x).mean(axis=axis))
+    else:
+        raise ValueError(name)
+    return np.asarray(r, dtype=np.float64)
+
+
 VIEWS = {
     "contig": lambda a: a,
     "colslice": lambda a: a[..., 1::2],
@@ -88,16 +106,20 @@ def test_random_float_sums(tname, dt, shape, axis):
     h = rng.uniform(-1, 1, size=shape).astype(dt)
     d = cls.cast(h)
     n = red_n(shape, axis)
-    sc = abs_sum(h, axis)
-    assert_reduction_close(d.sum(axis=axis).to_numpy(), oracle.reduce("sum", h, axis=axis), n, sc, "sum")
-    assert_reduction_close(d.mean(axis=axis).to_numpy(), oracle.reduce("mean", h, axis=axis), n, sc / n, "mean")
-    want = oracle.reduce("var", h, axis=axis)
-    if n > 1:
-        assert_reduction_close(d.var(axis=axis).to_numpy(), want, n, np.abs(want), "var")
-        want = oracle.reduce("stddev", h, axis=axis)
-        assert_reduction_close(d.stddev(axis=axis).to_numpy(), want, n, np.abs(want), "stddev")
-    want = oracle.reduce("rms", h, axis=axis)
-    assert_reduction_close(d.rms(axis=axis).to_numpy(), want, n, np.abs(want), "rms")
+    # Numo folds a float32 axis sequentially, so over 10^6 elements its own answer
+    # carries up to n*eps/2 of rounding (var of 10^6 uniform values is 3.7e-4 off
+    # the exact value). The device is held to the stated tolerance against the
+    # EXACT value (extended precision), and the oracle is shown to sit within its
+    # a-priori sequential bound of the same value: the two agree to that.
+    names = ["sum", "mean", "rms"] + (["var", "stddev"] if n > 1 else [])
+    for name in names:
+        want = exact_reduce(name, h, axis)
+        scale = {"sum": abs_sum(h, axis), "mean": abs_sum(h, axis) / n}.get(name, np.abs(want))
+        got = getattr(d, name)(axis=axis).to_numpy()
+        assert_reduction_close(got, want.astype(dt), n, scale, name)
+        ora = oracle.reduce(name, h, axis=axis).astype(np.float64)
+        eps = np.finfo(dt).eps
+        assert (np.abs(ora - want) <= (2 * n * eps) * np.asarray(scale, dtype=np.float64) + 1e-300).all(), "oracle %s" % name
     assert_bits_equal(d.max(axis=axis).to_numpy(), oracle.reduce("max", h, axis=axis))
     assert_bits_equal(d.min(axis=axis).to_numpy(), oracle.reduce("min", h, axis=axis))
     assert_bits_equal(d.argmax(axis=axis).to_numpy(), oracle.reduce("argmax", h, axis=axis))

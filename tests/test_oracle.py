@@ -265,6 +265,14 @@ def test_arg_reductions_brute_force():
     mi = oracle.reduce("max_index", x, axis=2)
     assert (x.reshape(-1)[mi] == x.max(axis=2)).all()
     assert (mi == np.argmax(x, axis=2) + np.arange(45).reshape(5, 9) * 6).all()
+    # ... also when the axis is not the innermost one, and over two axes
+    m1 = oracle.reduce("max_index", x, axis=1)
+    assert (m1 == np.arange(5).reshape(5, 1) * 54 + np.argmax(x, axis=1) * 6 + np.arange(6)).all()
+    m02 = oracle.reduce("min_index", x, axis=(0, 2))
+    for j in range(9):
+        sl = x[:, j, :]
+        i, k = np.unravel_index(np.argmin(sl), sl.shape)
+        assert m02[j] == i * 54 + j * 6 + k
     # NaN: skipped unless nan: true, where the first NaN wins
     y = np.array([2.0, np.nan, 5.0, np.nan, 5.0])
     assert oracle.reduce("argmax", y) == 2
