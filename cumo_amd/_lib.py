@@ -146,7 +146,38 @@ def check():
     raise RuntimeError_(text)
 
 
+_recording = None
+
+
 def call(f, *args):
+    if _recording is not None and (f.__name__.endswith("_kernel_launch") or f.__name__ == "cumo_hip_memset"):
+        _recording.append((f, args))
     r = f(*args)
     check()
     return r
+
+
+class record:
+    """Collects the launcher calls (function, arguments) made inside the block, so
+    that a caller can issue exactly the same launches again without the host-side
+    work of building them: `with record() as calls: y = a + b`, then
+    `replay(calls)`. The arrays the launches write into must be kept alive."""
+
+    def __enter__(self):
+        global _recording
+        self._prev = _recording
+        _recording = []
+        self.calls = _recording
+        return self.calls
+
+    def __exit__(self, *exc):
+        global _recording
+        _recording = self._prev
+        return False
+
+
+def replay(calls, times=1):
+    for _ in range(times):
+        for f, args in calls:
+            f(*args)
+    check()

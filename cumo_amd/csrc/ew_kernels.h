@@ -43,6 +43,7 @@ struct EwKParams {
     int tx_bits;         // 2^tx_bits lanes along the fast dim, the rest of the block along rows
     int use_scalar;      // 0: both inputs are arrays, 1: y = sv, 2: x = sv
     int small_rows;      // rows < 2^32: decompose with 32-bit divides
+    int nt;              // bit 0: non-temporal loads, bit 1: non-temporal stores
     int* flag;           // pinned host word for rejected elements (may be NULL)
     uint64_t out_bitpos; // Bit output: position of element 0
     uint64_t oshape[kMaxDim - 1];
@@ -56,16 +57,85 @@ struct alignas((sizeof(T) * N) > 16 ? 16 : (sizeof(T) * N)) VecT {
     T v[N];
 };
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// VEC elements of T as raw 128/64/32-bit accesses. NT marks the access
+// non-temporal: streamed data that is touched once should not displace what the
+// caches hold.
+template <class T, int VEC, bool NT>
+__device__ __forceinline__ void raw_load(const char* p, T (&out)[VEC]) {
+    constexpr int BYTES = (int)sizeof(T) * VEC;
+    union U {
+        T t[VEC];
+        u32x4 q[BYTES >= 16 ? BYTES / 16 : 1];
+        u32x2 d;
+        uint32_t w;
+        __device__ U() {}
+    } u;
+    if constexpr (BYTES % 16 == 0) {
+#pragma unroll
+        for (int k = 0; k < BYTES / 16; ++k) {
+            const u32x4* src = reinterpret_cast<const u32x4*>(p) + k;
+            u.q[k] = NT ? __builtin_nontemporal_load(src) : *src;
+        }
+    } else if constexpr (BYTES == 8) {
+        const u32x2* src = reinterpret_cast<const u32x2*>(p);
+        u.d = NT ? __builtin_nontemporal_load(src) : *src;
+    } else if constexpr (BYTES == 4) {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(p);
+        u.w = NT ? __builtin_nontemporal_load(src) : *src;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) u.t[j] = reinterpret_cast<const T*>(p)[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) out[j] = u.t[j];
+}
+
+template <class T, int VEC, bool NT>
+__device__ __forceinline__ void raw_store(char* p, const T (&in)[VEC]) {
+    constexpr int BYTES = (int)sizeof(T) * VEC;
+    union U {
+        T t[VEC];
+        u32x4 q[BYTES >= 16 ? BYTES / 16 : 1];
+        u32x2 d;
+        uint32_t w;
+        __device__ U() {}
+    } u;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) u.t[j] = in[j];
+    if constexpr (BYTES % 16 == 0) {
+#pragma unroll
+        for (int k = 0; k < BYTES / 16; ++k) {
+            u32x4* dst = reinterpret_cast<u32x4*>(p) + k;
+            if (NT) __builtin_nontemporal_store(u.q[k], dst);
+            else *dst = u.q[k];
+        }
+    } else if constexpr (BYTES == 8) {
+        u32x2* dst = reinterpret_cast<u32x2*>(p);
+        if (NT) __builtin_nontemporal_store(u.d, dst);
+        else *dst = u.d;
+    } else if constexpr (BYTES == 4) {
+        uint32_t* dst = reinterpret_cast<uint32_t*>(p);
+        if (NT) __builtin_nontemporal_store(u.w, dst);
+        else *dst = u.w;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) reinterpret_cast<T*>(p)[j] = u.t[j];
+    }
+}
+
 template <class T, int VEC>
-__device__ __forceinline__ void ew_load(const char* base, int64_t istep, int64_t col, T (&out)[VEC]) {
+__device__ __forceinline__ void ew_load(const char* base, int64_t istep, int64_t col, T (&out)[VEC], int nt) {
     if (istep == 0) {
         T v = *reinterpret_cast<const T*>(base);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = v;
     } else if (VEC > 1) {
-        const VecT<T, VEC> v = *reinterpret_cast<const VecT<T, VEC>*>(base + col * (int64_t)sizeof(T));
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) out[j] = v.v[j];
+        const char* p = base + col * (int64_t)sizeof(T);
+        if (nt & 1) raw_load<T, VEC, true>(p, out);
+        else raw_load<T, VEC, false>(p, out);
     } else {
         out[0] = *reinterpret_cast<const T*>(base + col * istep);
     }
@@ -120,6 +190,22 @@ __device__ __forceinline__ void ew_store_bits(CUMO_BIT_DIGIT* base, uint64_t P, 
             }
         }
     }
+}
+
+// The vector form of a Bit row. The launcher only picks it when every row starts
+// on a word boundary and a word's 32/VEC lanes sit in one row. Lane k of a group of
+// 32/VEC lanes holds bits [k*VEC, k*VEC+VEC) of the group's word; the word is
+// gathered into the group's first lane with DPP row shifts (lane i reads lane i+d
+// of its 16-lane row): plain vector ALU, no trip through LDS.
+template <int VEC>
+__device__ __forceinline__ uint32_t ew_gather_word(uint32_t bits) {
+    constexpr unsigned G = 32 / VEC;
+    uint32_t w = bits;
+    w |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0x101, 0xf, 0xf, true) << VEC;
+    w |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0x102, 0xf, 0xf, true) << (2 * VEC);
+    w |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0x104, 0xf, 0xf, true) << (4 * VEC);
+    if constexpr (G > 8) w |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0x108, 0xf, 0xf, true) << (8 * VEC);
+    return w;
 }
 
 template <int NOPS>
@@ -193,7 +279,15 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
 
         int64_t lead = 0;
         if (Op::BIT_OUT && VEC == 1) lead = (int64_t)((p.out_bitpos + (uint64_t)off[2]) & 31);
-        const int64_t col0 = (int64_t)(ct * tile_cols) + (int64_t)tx * VEC - lead;
+        // Typed results: a wave's lanes sit side by side, unroll steps a whole lane
+        // row apart. Vector Bit results: the 32/VEC lanes of a word sit side by side
+        // and the unroll steps are the NEXT words, so that a group's first lane ends
+        // up with kEwUnroll consecutive words and stores them as one 128-bit access.
+        constexpr bool BITVEC = Op::BIT_OUT && VEC > 1;
+        constexpr int64_t G = BITVEC ? 32 / VEC : 1;
+        const int64_t col0 = BITVEC ? (int64_t)(ct * tile_cols) + (int64_t)(tx / G) * (32 * kEwUnroll) + (int64_t)(tx % G) * VEC
+                                    : (int64_t)(ct * tile_cols) + (int64_t)tx * VEC - lead;
+        const int64_t ustep = BITVEC ? 32 : (int64_t)TX * VEC;
 
         const char* b0 = p.ptr[0] + off[0];
         const char* b1 = p.ptr[1] + off[1];
@@ -203,13 +297,13 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
         int nval[kEwUnroll];  // how many of the VEC elements exist
 #pragma unroll
         for (int u = 0; u < kEwUnroll; ++u) {
-            const int64_t col = col0 + (int64_t)u * TX * VEC;
+            const int64_t col = col0 + (int64_t)u * ustep;
             int nv = 0;
             if (row_ok && col >= 0 && col < inner) nv = (col + VEC <= inner) ? VEC : (int)(inner - col);
             nval[u] = nv;
             if (nv == VEC) {
-                if (NIN >= 1) ew_load<A, VEC>(b0, p.istep[0], col, xv[u]);
-                if (two_arrays) ew_load<B, VEC>(b1, p.istep[1], col, yv[u]);
+                if (NIN >= 1) ew_load<A, VEC>(b0, p.istep[0], col, xv[u], p.nt);
+                if (two_arrays) ew_load<B, VEC>(b1, p.istep[1], col, yv[u], p.nt);
             } else if (nv > 0) {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
@@ -221,9 +315,10 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
             }
         }
 
+        uint32_t words[kEwUnroll];
 #pragma unroll
         for (int u = 0; u < kEwUnroll; ++u) {
-            const int64_t col = col0 + (int64_t)u * TX * VEC;
+            const int64_t col = col0 + (int64_t)u * ustep;
             const int nv = nval[u];
             R zv[VEC];
             uint32_t okmask = 0;
@@ -247,7 +342,11 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) if (j < nv && zv[j]) bits |= 1u << j;
                 const uint64_t P = p.out_bitpos + (uint64_t)off[2] + (uint64_t)(col * p.istep[2]);
-                ew_store_bits<VEC>(reinterpret_cast<CUMO_BIT_DIGIT*>(p.ptr[2]), P, bits, (nv >= VEC) ? ((1u << VEC) - 1u) : ((1u << nv) - 1u), nv > 0);
+                if constexpr (VEC > 1) {
+                    words[u] = ew_gather_word<VEC>(bits);
+                } else {
+                    ew_store_bits<VEC>(reinterpret_cast<CUMO_BIT_DIGIT*>(p.ptr[2]), P, bits, nv > 0 ? 1u : 0u, nv > 0);
+                }
             } else if (nv > 0) {
                 char* o = p.ptr[2] + off[2];
                 const uint32_t full = (1u << VEC) - 1u;
@@ -255,14 +354,37 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
                     if (p.flag) *p.flag = 1;
                 }
                 if (VEC > 1 && nv == VEC && okmask == full && p.istep[2] != 0) {
-                    VecT<R, VEC> v;
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j) v.v[j] = zv[j];
-                    *reinterpret_cast<VecT<R, VEC>*>(o + col * (int64_t)sizeof(R)) = v;
+                    if (p.nt & 2) raw_store<R, VEC, true>(o + col * (int64_t)sizeof(R), zv);
+                    else raw_store<R, VEC, false>(o + col * (int64_t)sizeof(R), zv);
                 } else {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
                         if (j < nv && ((okmask >> j) & 1u)) *reinterpret_cast<R*>(o + (col + j) * p.istep[2]) = zv[j];
+                    }
+                }
+            }
+        }
+        if constexpr (BITVEC) {
+            // the first lane of each group holds kEwUnroll consecutive words
+            if ((tx % G) == 0 && nval[0] > 0) {
+                CUMO_BIT_DIGIT* base = reinterpret_cast<CUMO_BIT_DIGIT*>(p.ptr[2]);
+                const uint64_t P0 = p.out_bitpos + (uint64_t)off[2] + (uint64_t)col0;
+                const int64_t left0 = inner - col0;  // elements of this row from the group's first bit on
+                CUMO_BIT_DIGIT* dst = base + (P0 >> 5);
+                if (left0 >= 32 * kEwUnroll && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                    *reinterpret_cast<u32x4*>(dst) = u32x4{words[0], words[1], words[2], words[3]};
+                } else {
+#pragma unroll
+                    for (int u = 0; u < kEwUnroll; ++u) {
+                        const int64_t left = left0 - 32 * u;
+                        if (left >= 32) {
+                            dst[u] = words[u];
+                        } else if (left > 0) {
+                            // a row's last, partly used word: its other bits are not ours
+                            const uint32_t m = (1u << left) - 1u;
+                            atomicAnd(&dst[u], ~m);
+                            atomicOr(&dst[u], words[u] & m);
+                        }
                     }
                 }
             }
@@ -281,6 +403,7 @@ struct EwTParams {
     int nouter;
     int use_scalar;
     int tr[2];                // input k goes through LDS
+    int order;                // how block index maps to tiles: 0 F fastest, 1 G fastest, 2 8x8 super-tiles
     int* flag;
     uint64_t oshape[kMaxDim - 2];
     int64_t ostep[3][kMaxDim - 2];
@@ -302,8 +425,22 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_kernel(EwTParams p, Op 
     const bool two_arrays = TWO && p.use_scalar == 0;
     for (uint64_t tile = blockIdx.x; tile < p.n_tiles; tile += gridDim.x) {
         uint64_t t = tile;
-        const uint64_t ft = t % p.f_tiles; t /= p.f_tiles;
-        const uint64_t gt = t % p.g_tiles; t /= p.g_tiles;
+        uint64_t ft, gt;
+        if (p.order == 1) {
+            gt = t % p.g_tiles; t /= p.g_tiles;
+            ft = t % p.f_tiles; t /= p.f_tiles;
+        } else if (p.order == 2) {
+            // 8 x 8 super-tiles (both tile counts are multiples of 8)
+            const uint64_t per_plane = p.f_tiles * p.g_tiles;
+            const uint64_t q = t % per_plane; t /= per_plane;
+            const uint64_t st = q >> 6, w = q & 63;
+            const uint64_t sf = p.f_tiles >> 3;
+            ft = (st % sf) * 8 + (w & 7);
+            gt = (st / sf) * 8 + (w >> 3);
+        } else {
+            ft = t % p.f_tiles; t /= p.f_tiles;
+            gt = t % p.g_tiles; t /= p.g_tiles;
+        }
         int64_t off[3] = {0, 0, 0};
         for (int d = p.nouter - 1; d >= 0; --d) {
             const uint64_t n = p.oshape[d];
@@ -387,9 +524,18 @@ static inline unsigned ew_grid_cap() {
     if (cap == 0) {
         const char* e = std::getenv("CUMO_HIP_EW_GRID_CAP");
         cap = e ? (unsigned)std::strtoul(e, nullptr, 10) : 0;
-        if (cap == 0) cap = (unsigned)kNumCU * 16;
+        if (cap == 0) cap = (unsigned)kNumCU * 64;  // measured: more, shorter blocks stream better than a long grid-stride loop
     }
     return cap;
+}
+
+static inline int ew_nt_mode() {
+    static int mode = -1;
+    if (mode < 0) {
+        const char* e = std::getenv("CUMO_HIP_NT");
+        mode = e ? std::atoi(e) : 0;
+    }
+    return mode;
 }
 
 // in1/in2 may be NULL (NIN < 2 or the scalar form). out_bit is non-NULL for a
@@ -427,12 +573,21 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         tp.nouter = n - 2;
         tp.use_scalar = use_scalar;
         tp.flag = flag;
+        {
+            static int order = -1;
+            if (order < 0) {
+                const char* e = std::getenv("CUMO_HIP_TR_ORDER");
+                order = e ? std::atoi(e) : 0;
+            }
+            tp.order = order;
+        }
         constexpr int TG = (sizeof(A) >= 8 || sizeof(B) >= 8) ? 32 : 64;
         tp.f_tiles = (tp.nf + 63) / 64;
         tp.g_tiles = (tp.ng + TG - 1) / TG;
         uint64_t outer = 1;
         for (int d = 0; d < n - 2; ++d) { tp.oshape[d] = plan.shape[d]; outer *= plan.shape[d]; }
         tp.n_tiles = tp.f_tiles * tp.g_tiles * outer;
+        if (tp.order == 2 && ((tp.f_tiles & 7) || (tp.g_tiles & 7))) tp.order = 0;
         for (int o = 0; o < nops; ++o) {
             const int s = slot[o];
             tp.ptr[s] = const_cast<char*>(ops[o].ptr);
@@ -469,8 +624,16 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         for (int d = 0; d < n - 1; ++d) kp.ostep[s][d] = plan.step[o][d];
     }
     if (Op::BIT_OUT) kp.out_bitpos = out_bit->pos;
+    kp.nt = ew_nt_mode();
 
-    const int vec = plan.vec;
+    int vec = plan.vec;
+    // the vector form of a Bit row needs the 32/vec lanes of a word inside one row
+    if (Op::BIT_OUT && vec > 1 && kp.inner < 32) vec = 1;
+    {
+        static int force1 = -1;
+        if (force1 < 0) force1 = std::getenv("CUMO_HIP_FORCE_VEC1") ? 1 : 0;
+        if (force1) vec = 1;
+    }
     const bool shift = Op::BIT_OUT && vec == 1;
     const uint64_t span = kp.inner + (shift ? 31 : 0);
     uint64_t lanes_needed = (span + vec - 1) / vec;

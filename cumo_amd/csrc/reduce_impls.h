@@ -50,6 +50,33 @@ template <> struct Lim<int32_t> {
 template <class T> __device__ __forceinline__ T spread(T hi, T lo) { return hi - lo; }
 template <> __device__ __forceinline__ int32_t spread<int32_t>(int32_t hi, int32_t lo) { return (int32_t)((uint32_t)hi - (uint32_t)lo); }
 
+// the plain element-by-element form of accumulate_n
+#define CUMO_HIP_ACCUMULATE_N_BY_ELEMENT                                                          \
+    template <int N>                                                                              \
+    __device__ __forceinline__ void accumulate_n(const In (&x)[N], int64_t idx0, Acc& acc) const { \
+        _Pragma("unroll") for (int k = 0; k < N; ++k) accumulate(x[k], idx0 + k, acc);            \
+    }
+
+template <class T> __device__ __forceinline__ T max_skipping_nan(T a, T b);
+template <> __device__ __forceinline__ float max_skipping_nan<float>(float a, float b) { return __builtin_fmaxf(a, b); }
+template <> __device__ __forceinline__ double max_skipping_nan<double>(double a, double b) { return __builtin_fmax(a, b); }
+template <> __device__ __forceinline__ int32_t max_skipping_nan<int32_t>(int32_t a, int32_t b) { return a > b ? a : b; }
+template <class T> __device__ __forceinline__ T min_skipping_nan(T a, T b);
+template <> __device__ __forceinline__ float min_skipping_nan<float>(float a, float b) { return __builtin_fminf(a, b); }
+template <> __device__ __forceinline__ double min_skipping_nan<double>(double a, double b) { return __builtin_fmin(a, b); }
+template <> __device__ __forceinline__ int32_t min_skipping_nan<int32_t>(int32_t a, int32_t b) { return a < b ? a : b; }
+
+// true if any of the N values is a NaN (a sum is NaN then; inf - inf also trips
+// it, which only costs the slow path)
+template <class T, int N>
+__device__ __forceinline__ bool maybe_nan(const T (&x)[N]) {
+    if (!is_float_t<T>::value) return false;
+    T s = x[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) s = s + x[k];
+    return s != s;
+}
+
 // ---- sum / prod / mean -------------------------------------------------------
 // TA: accumulator type (the input type for floats, int64 for Int32:
 // narray/gen/spec.rb:308-319). divisor != 0 turns the sum into a mean
@@ -66,6 +93,7 @@ struct SumImpl {
         if (SKIP_NAN && isnan_t(x)) return;
         if (PROD) acc = (TA)x * acc; else acc = (TA)x + acc;
     }
+    CUMO_HIP_ACCUMULATE_N_BY_ELEMENT
     __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
         if (PROD) acc = next * acc; else acc = next + acc;
     }
@@ -87,6 +115,7 @@ struct MeanNanImpl {
         acc.sum = x + acc.sum;
         acc.n += 1;
     }
+    CUMO_HIP_ACCUMULATE_N_BY_ELEMENT
     __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { acc.sum = next.sum + acc.sum; acc.n += next.n; }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const { *reinterpret_cast<T*>(out) = acc.sum / (T)acc.n; }
 };
@@ -109,6 +138,7 @@ struct RmsImpl {
         }
         acc.sum += x * x;
     }
+    CUMO_HIP_ACCUMULATE_N_BY_ELEMENT
     __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { acc.sum += next.sum; acc.n += next.n; }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
         const T n = SKIP_NAN ? (T)acc.n : count;
@@ -139,9 +169,33 @@ struct MomentsImpl {
         if (acc.n == (T)0) { acc = next; return; }
         const T n = acc.n + next.n;
         const T delta = next.mean - acc.mean;
-        acc.mean = acc.mean + delta * (next.n / n);
-        acc.m2 += next.m2 + delta * delta * acc.n * next.n / n;
+        const T w = next.n / n;
+        acc.mean = acc.mean + delta * w;
+        acc.m2 += next.m2 + delta * delta * acc.n * w;
         acc.n = n;
+    }
+    // N elements at once: their own mean and squared deviations in two passes over
+    // registers (no division: N is a power of two), then one Chan merge. One
+    // division per N elements instead of one per element, and the block statistics
+    // are as accurate as Numo's own two-pass form.
+    template <int N>
+    __device__ __forceinline__ void accumulate_n(const T (&x)[N], int64_t idx0, Acc& acc) const {
+        if (N == 1 || (N & (N - 1)) != 0 || (SKIP_NAN && maybe_nan<T, N>(x))) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) accumulate(x[k], idx0 + k, acc);
+            return;
+        }
+        T s = x[0];
+#pragma unroll
+        for (int k = 1; k < N; ++k) s = s + x[k];
+        const T mb = s * ((T)1 / (T)N);
+        T m2 = (T)0;
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            const T d = x[k] - mb;
+            m2 = m2 + d * d;
+        }
+        combine(Acc{(T)N, mb, m2}, acc);
     }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
         // every element NaN leaves no count; Numo answers +0 there (float_accum_kernel.cu:74-84)
@@ -169,6 +223,7 @@ struct KahanImpl {
         if (SKIP_NAN && isnan_t(x)) return;
         combine(Acc{x, (T)0}, acc);
     }
+    CUMO_HIP_ACCUMULATE_N_BY_ELEMENT
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const { *reinterpret_cast<T*>(out) = acc.sum + acc.comp; }
 };
 
@@ -205,6 +260,48 @@ struct ArgImpl {
         if (better || (acc.value == next.value && next.index < acc.index)) acc = next;
     }
     __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{x, idx}, acc); }
+    // N later elements at once. The block's extreme costs one max/min per element;
+    // only a block that beats the accumulator is looked at again, to find where its
+    // extreme first occurs, and then merged with one combine. An equal value never
+    // replaces, because everything in the block is later than what the accumulator
+    // holds.
+    template <int N>
+    __device__ __forceinline__ void accumulate_n(const T (&x)[N], int64_t idx0, Acc& acc) const {
+        if (N == 1) {
+            accumulate(x[0], idx0, acc);
+            return;
+        }
+        T m = x[0];
+#pragma unroll
+        for (int k = 1; k < N; ++k) m = IS_MAX ? max_skipping_nan<T>(m, x[k]) : min_skipping_nan<T>(m, x[k]);
+        bool look = IS_MAX ? (m > acc.value) : (m < acc.value);
+        look = look || acc.index == INT64_MAX;
+        if (is_float_t<T>::value) {
+            if (NAN_WINS) {
+                if (isnan_t(acc.value)) return;  // an earlier NaN already won
+                if (maybe_nan<T, N>(x)) {         // rare: let the exact rule sort it out
+#pragma unroll
+                    for (int k = 0; k < N; ++k) accumulate(x[k], idx0 + k, acc);
+                    return;
+                }
+            } else {
+                look = look || isnan_t(acc.value);  // nothing but NaN so far
+            }
+        }
+        if (!look) return;
+        // first position holding the extreme; if every element is a NaN, m is one and
+        // nothing compares equal, which leaves the block's first element
+        // (the value is taken from that position too: of +0 and -0 the earlier counts)
+        int first = 0;
+        T v = is_float_t<T>::value ? x[0] : m;
+#pragma unroll
+        for (int k = N - 1; k >= 0; --k) {
+            const bool hit = x[k] == m;
+            first = hit ? k : first;
+            v = hit ? x[k] : v;
+        }
+        combine(Acc{v, idx0 + first}, acc);
+    }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
         if (out_mode == 0) *reinterpret_cast<T*>(out) = acc.value;
         else if (out_mode == 4) *reinterpret_cast<int32_t*>(out) = (int32_t)acc.index;
@@ -239,6 +336,16 @@ struct MinMaxImpl {
         acc.hi = One{h.value, h.index};
     }
     __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{One{x, idx}, One{x, idx}}, acc); }
+    template <int N>
+    __device__ __forceinline__ void accumulate_n(const T (&x)[N], int64_t idx0, Acc& acc) const {
+        // each end runs its own block rule
+        ArgImpl<T, false, NAN_WINS> a{0};
+        ArgImpl<T, true, NAN_WINS> b{0};
+        a.template accumulate_n<N>(x, idx0, acc.lo);
+        typename ArgImpl<T, true, NAN_WINS>::Acc h{acc.hi.value, acc.hi.index};
+        b.template accumulate_n<N>(x, idx0, h);
+        acc.hi = One{h.value, h.index};
+    }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const {
         if (out_mode == 0) {
             *reinterpret_cast<T*>(out) = acc.lo.value;

@@ -26,7 +26,11 @@
 //   typedef In, Acc;  static constexpr bool USES_INDEX; static constexpr int NOUT (1 or 2)
 //   Acc identity() const
 //   void accumulate(In x, int64_t idx, Acc& acc) const     -- fold one input element
-//   void combine(const Acc& next, Acc& acc) const          -- fold an accumulator of LATER elements into acc
+//   void accumulate_n<N>(const In (&x)[N], int64_t idx0, Acc& acc) const
+//                                                          -- fold N elements at consecutive positions idx0..idx0+N-1,
+//                                                             later than anything this accumulator has seen
+//   void combine(const Acc& next, Acc& acc) const          -- merge two accumulators; must not depend on the order
+//                                                             in which accumulators arrive
 //   void store(const Acc& acc, char* out, char* out2) const
 #ifndef CUMO_HIP_REDUCE_KERNELS_H
 #define CUMO_HIP_REDUCE_KERNELS_H
@@ -159,14 +163,10 @@ __global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl i
                 for (int u = 0; u < kRedUnroll; ++u) {
                     const uint64_t i = i0 + (uint64_t)u * stride;
                     if (i < end) {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) {
-                            int64_t idx = 0;
-                            if (Impl::USES_INDEX) {
-                                idx = (p.index_mode == 2) ? (eoff[u] / (int64_t)sizeof(In) + j) : (int64_t)(i + j);
-                            }
-                            impl.accumulate(x[u][j], idx, acc);
-                        }
+                        // the VEC elements of one access are consecutive along the axis
+                        int64_t idx = 0;
+                        if (Impl::USES_INDEX) idx = (p.index_mode == 2) ? (eoff[u] / (int64_t)sizeof(In)) : (int64_t)i;
+                        impl.template accumulate_n<VEC>(x[u], idx, acc);
                     }
                 }
             }
@@ -243,17 +243,28 @@ __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl i
                     }
                 }
             }
+            if (i0 + kRedUnroll <= end && p.index_mode != 2) {
+                // a whole block of consecutive positions along the axis for each output
 #pragma unroll
-            for (int u = 0; u < kRedUnroll; ++u) {
-                const uint64_t i = i0 + u;
-                if (i < end) {
+                for (int j = 0; j < VEC; ++j) {
+                    In t[kRedUnroll];
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) {
-                        int64_t idx = 0;
-                        if (Impl::USES_INDEX) {
-                            idx = (p.index_mode == 2) ? ((in_off + roff[u] + (int64_t)j * ostep_in) / (int64_t)sizeof(In)) : (int64_t)i;
+                    for (int u = 0; u < kRedUnroll; ++u) t[u] = x[u][j];
+                    impl.template accumulate_n<kRedUnroll>(t, (int64_t)i0, acc[j]);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < kRedUnroll; ++u) {
+                    const uint64_t i = i0 + u;
+                    if (i < end) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            int64_t idx = 0;
+                            if (Impl::USES_INDEX) {
+                                idx = (p.index_mode == 2) ? ((in_off + roff[u] + (int64_t)j * ostep_in) / (int64_t)sizeof(In)) : (int64_t)i;
+                            }
+                            impl.accumulate(x[u][j], idx, acc[j]);
                         }
-                        impl.accumulate(x[u][j], idx, acc[j]);
                     }
                 }
             }
@@ -282,6 +293,11 @@ struct CombineImpl {
     Impl impl;
     __device__ __forceinline__ Acc identity() const { return impl.identity(); }
     __device__ __forceinline__ void accumulate(const In& x, int64_t, Acc& acc) const { impl.combine(x, acc); }
+    template <int N>
+    __device__ __forceinline__ void accumulate_n(const In (&x)[N], int64_t, Acc& acc) const {
+#pragma unroll
+        for (int k = 0; k < N; ++k) impl.combine(x[k], acc);
+    }
     __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { impl.combine(next, acc); }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const { impl.store(acc, out, out2); }
 };
