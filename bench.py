@@ -32,6 +32,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the C2 broadcast add, from two rocprofv3 --pmc runs of this
+# file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by the same
+# counter's reading for --pmc-calibration's plain 256 MiB copy (FETCH_SIZE x 1.9992,
+# WRITE_SIZE x 1.0000): 131294 KiB fetched + 131072 KiB written. The figures and
+# the commands are in profiles/ew_rows_add_f64_c2_hbm_traffic.txt.
+C2_ADD_TRAFFIC_BYTES = 268662587
 METRIC = "achieved HBM GB/s (% of MI355X peak) and GElem/s vs Numo CPU, per config"
 MIB = 1 << 20
 
@@ -249,6 +255,9 @@ def main():
     ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c3,c4,c5)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also launch a plain contiguous copy of known size (256 MiB in, 256 MiB out) five times, so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command can scale its counters by it")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path has no cross-GPU stage)" % args.gpus, file=sys.stderr)
@@ -326,10 +335,18 @@ def main():
         "bound": "hbm", "kernel": "ew_rows_kernel<OpAdd<double>, 2> (C = A + r, f64 4096x4096 + 1x4096)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
         "bytes_per_launch": int(add_bytes), "avg_launch_ms": round(avg_ms, 5), "median_launch_ms": round(ts[len(ts) // 2], 5),
-        "traffic": None,
+        "traffic": C2_ADD_TRAFFIC_BYTES,
     }
     env.clear()
     cumo_amd.MemoryPool.free_all_blocks()
+
+    if args.pmc_calibration:
+        src = cumo_amd.SFloat.zeros(1 << 26)
+        for _ in range(5):
+            dst = src.copy()  # ew_rows_kernel<OpCast<unsigned int, unsigned int>, 4>: reads 256 MiB, writes 256 MiB
+        cumo_amd.synchronize()
+        del src, dst
+        cumo_amd.MemoryPool.free_all_blocks()
 
     per_config = {}
     if not args.no_per_config:

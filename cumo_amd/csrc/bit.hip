@@ -19,6 +19,9 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr unsigned kGridCap = kNumCU * 8;
+// counting ends in one atomic add per block on a single word, so fewer, longer
+// blocks: one per compute unit
+constexpr unsigned kCountGridCap = kNumCU;
 
 __device__ __forceinline__ uint32_t low_bits(unsigned n) { return n >= 32 ? 0xffffffffu : ((1u << n) - 1u); }
 
@@ -181,9 +184,9 @@ __global__ __launch_bounds__(kBlock) void bit_count_scatter_kernel(const CUMO_BI
     }
 }
 
-unsigned grid_for(uint64_t items) {
+unsigned grid_for(uint64_t items, unsigned cap = kGridCap) {
     uint64_t g = (items + kBlock - 1) / kBlock;
-    if (g > kGridCap) g = kGridCap;
+    if (g > cap) g = cap;
     if (g == 0) g = 1;
     return (unsigned)g;
 }
@@ -235,11 +238,11 @@ void launch_count(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, ssize_t s1, size_t* i
         hipLaunchKernelGGL((bit_count_scatter_kernel<COUNT_FALSE>), dim3(grid_for(n)), dim3(kBlock), 0, st, a1, (uint64_t)p1, (int64_t)s1, idx1,
                            p2, (int64_t)s2, n);
     } else if (!idx1 && s1 == 1) {
-        hipLaunchKernelGGL((bit_count_words_kernel<COUNT_FALSE>), dim3(grid_for((n + 31) / 32 + 1)), dim3(kBlock), 0, st, a1, (uint64_t)p1, n,
+        hipLaunchKernelGGL((bit_count_words_kernel<COUNT_FALSE>), dim3(grid_for((n + 31) / 32 + 1, kCountGridCap)), dim3(kBlock), 0, st, a1, (uint64_t)p1, n,
                            (unsigned long long*)p2);
     } else {
-        hipLaunchKernelGGL((bit_count_gather_kernel<COUNT_FALSE>), dim3(grid_for(n)), dim3(kBlock), 0, st, a1, (uint64_t)p1, (int64_t)s1, idx1,
-                           n, (unsigned long long*)p2);
+        hipLaunchKernelGGL((bit_count_gather_kernel<COUNT_FALSE>), dim3(grid_for(n, kCountGridCap * 4)), dim3(kBlock), 0, st, a1, (uint64_t)p1,
+                           (int64_t)s1, idx1, n, (unsigned long long*)p2);
     }
     cumo_cuda_runtime_check_kernel_launch();
 }

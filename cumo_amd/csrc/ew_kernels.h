@@ -411,7 +411,10 @@ struct EwTParams {
     char* ptr[3];
 };
 
-template <class Op, int TG>
+// VT: every operand tolerates 128-bit accesses along its own fast dimension (the
+// launcher checks alignment and divisibility), so both the reads along G and the
+// writes along F move 16 bytes per lane.
+template <class Op, int TG, bool VT>
 __global__ __launch_bounds__(kEwBlock) void ew_transpose_kernel(EwTParams p, Op op, typename Op::S sv) {
     typedef typename Op::A A;
     typedef typename Op::B B;
@@ -453,7 +456,44 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_kernel(EwTParams p, Op 
         const uint64_t f0 = ft * TF, g0 = gt * TG;
 
         // phase 1: transposed inputs, lanes along G
-        {
+        if constexpr (VT) {
+            constexpr int V = 16 / (int)sizeof(A);
+            constexpr unsigned GV = TG / V;          // 128-bit slots along G
+            constexpr unsigned FP = kEwBlock / GV;   // F positions per pass
+            constexpr unsigned NP = TF / FP;
+            const unsigned gv = threadIdx.x % GV, lf0 = threadIdx.x / GV;
+            const uint64_t g = g0 + (uint64_t)gv * V;
+            if (p.tr[0] && g < p.ng) {
+                const char* src = p.ptr[0] + off[0] + (int64_t)g * (int64_t)sizeof(A) + (int64_t)(f0 + lf0) * p.fstep[0];
+                A v[NP][V];
+#pragma unroll
+                for (unsigned k = 0; k < NP; ++k) {
+                    if (f0 + lf0 + k * FP < p.nf) raw_load<A, V, false>(src + (int64_t)(k * FP) * p.fstep[0], v[k]);
+                }
+#pragma unroll
+                for (unsigned k = 0; k < NP; ++k) {
+                    if (f0 + lf0 + k * FP < p.nf) {
+#pragma unroll
+                        for (int q = 0; q < V; ++q) tile_a[gv * V + q][lf0 + k * FP] = v[k][q];
+                    }
+                }
+            }
+            if (two_arrays && p.tr[1] && g < p.ng) {
+                const char* src = p.ptr[1] + off[1] + (int64_t)g * (int64_t)sizeof(B) + (int64_t)(f0 + lf0) * p.fstep[1];
+                B v[NP][V];
+#pragma unroll
+                for (unsigned k = 0; k < NP; ++k) {
+                    if (f0 + lf0 + k * FP < p.nf) raw_load<B, V, false>(src + (int64_t)(k * FP) * p.fstep[1], v[k]);
+                }
+#pragma unroll
+                for (unsigned k = 0; k < NP; ++k) {
+                    if (f0 + lf0 + k * FP < p.nf) {
+#pragma unroll
+                        for (int q = 0; q < V; ++q) tile_b[TWO ? gv * V + q : 0][lf0 + k * FP] = v[k][q];
+                    }
+                }
+            }
+        } else {
             const unsigned lg = threadIdx.x % TG;
             const unsigned lf0 = threadIdx.x / TG;
             constexpr unsigned FSTEP = kEwBlock / TG;
@@ -477,7 +517,73 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_kernel(EwTParams p, Op 
         }
         __syncthreads();
         // phase 2: lanes along F
-        {
+        if constexpr (VT) {
+            constexpr int V = 16 / (int)sizeof(A);
+            constexpr unsigned FV = TF / V;          // 128-bit slots along F
+            constexpr unsigned GP = kEwBlock / FV;   // G positions per pass
+            constexpr unsigned NP = TG / GP;
+            const unsigned fv = threadIdx.x % FV, lg0 = threadIdx.x / FV;
+            const uint64_t f = f0 + (uint64_t)fv * V;
+            if (f < p.nf) {
+#pragma unroll
+                for (unsigned k = 0; k < NP; ++k) {
+                    const unsigned lg = lg0 + k * GP;
+                    const uint64_t g = g0 + lg;
+                    if (g >= p.ng) continue;
+                    A x[V];
+                    B y[V];
+                    if (NIN >= 1) {
+                        if (p.tr[0]) {
+#pragma unroll
+                            for (int q = 0; q < V; ++q) x[q] = tile_a[lg][fv * V + q];
+                        } else {
+                            ew_load<A, V>(p.ptr[0] + off[0] + (int64_t)g * p.gstep[0], p.fstep[0], (int64_t)f, x, 0);
+                        }
+                    }
+                    if (two_arrays) {
+                        if (p.tr[1]) {
+#pragma unroll
+                            for (int q = 0; q < V; ++q) y[q] = tile_b[TWO ? lg : 0][fv * V + q];
+                        } else {
+                            ew_load<B, V>(p.ptr[1] + off[1] + (int64_t)g * p.gstep[1], p.fstep[1], (int64_t)f, y, 0);
+                        }
+                    }
+                    R z[V];
+                    bool ok = true;
+#pragma unroll
+                    for (int q = 0; q < V; ++q) {
+                        A xa = (NIN >= 1) ? x[q] : A();
+                        B yb = B();
+                        if (TWO) {
+                            if (p.use_scalar == 0) yb = y[q];
+                            else if (p.use_scalar == 1) yb = (B)sv;
+                            else { yb = (B)xa; xa = (A)sv; }
+                        }
+                        z[q] = R();
+                        ok = op(xa, yb, z[q]) && ok;
+                    }
+                    char* dst = p.ptr[2] + off[2] + (int64_t)g * p.gstep[2] + (int64_t)f * (int64_t)sizeof(R);
+                    if (!Op::CHECKED || ok) {
+                        raw_store<R, V, false>(dst, z);
+                    } else {
+                        // some element was rejected: store the others one by one
+                        if (p.flag) *p.flag = 1;
+#pragma unroll
+                        for (int q = 0; q < V; ++q) {
+                            A xa = (NIN >= 1) ? x[q] : A();
+                            B yb = B();
+                            if (TWO) {
+                                if (p.use_scalar == 0) yb = y[q];
+                                else if (p.use_scalar == 1) yb = (B)sv;
+                                else { yb = (B)xa; xa = (A)sv; }
+                            }
+                            R zz = R();
+                            if (op(xa, yb, zz)) reinterpret_cast<R*>(dst)[q] = zz;
+                        }
+                    }
+                }
+            }
+        } else {
             const unsigned lf = threadIdx.x % TF;
             const unsigned lg0 = threadIdx.x / TF;
             constexpr unsigned GSTEP = kEwBlock / TF;
@@ -577,7 +683,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             static int order = -1;
             if (order < 0) {
                 const char* e = std::getenv("CUMO_HIP_TR_ORDER");
-                order = e ? std::atoi(e) : 0;
+                order = e ? std::atoi(e) : 1;  // measured on the transposed-view case: tiles along the inputs' fast dim first
             }
             tp.order = order;
         }
@@ -602,7 +708,23 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         }
         uint64_t grid = tp.n_tiles;
         if (grid > 0x7fffffffull) grid = 0x7fffffffull;
-        hipLaunchKernelGGL((ew_transpose_kernel<Op, TG>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, tp, op, sv);
+        // 128-bit form: same element size everywhere, whole vectors in both tile
+        // directions, every operand aligned along the dimension it is walked in
+        constexpr int V = 16 / (int)sizeof(A);
+        bool vt = sizeof(A) == sizeof(R) && (Op::NIN < 2 || sizeof(B) == sizeof(A)) && (16 % sizeof(A)) == 0 && sizeof(A) >= 4 &&
+                  (tp.ng % V) == 0 && (tp.nf % V) == 0;
+        for (int o = 0; o < nops && vt; ++o) {
+            const int sl = slot[o];
+            const int64_t es = (int64_t)sizeof(A);
+            const bool through_lds = sl < 2 && tp.tr[sl];
+            const int64_t along = through_lds ? tp.gstep[sl] : tp.fstep[sl];
+            const int64_t across = through_lds ? tp.fstep[sl] : tp.gstep[sl];
+            if (sl < 2 && !through_lds && along == 0) continue;  // broadcast along F: scalar loads
+            vt = along == es && (across % 16) == 0 && ((uintptr_t)tp.ptr[sl] % 16) == 0;
+            for (int d = 0; d < n - 2 && vt; ++d) vt = (tp.ostep[sl][d] % 16) == 0;
+        }
+        if (vt) hipLaunchKernelGGL((ew_transpose_kernel<Op, TG, true>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, tp, op, sv);
+        else hipLaunchKernelGGL((ew_transpose_kernel<Op, TG, false>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, tp, op, sv);
         cumo_cuda_runtime_check_kernel_launch();
         return;
     }
