@@ -186,10 +186,11 @@ def measure_config(name, cumo, lib, iters, warmup):
     rows = []
     batch = 10
     for label, fn, nbytes, nelem in ops:
-        # the op runs once through the host mirror, which records the launcher calls
-        # it makes; the timed region issues exactly those C-ABI calls again, `batch`
-        # times back to back between two events on the launch stream, so the figure
-        # is the kernel's and not the Python host's
+        # the op runs once through the host mirror, which records the library calls
+        # it makes; the timed region issues exactly those C-ABI calls again (into the
+        # result the first call allocated), `batch` times back to back between two
+        # events on the launch stream, so the figure is the library's and not the
+        # Python mirror's
         with _lib.record() as calls:
             fn(env)
         _lib.replay(calls, warmup)
@@ -277,24 +278,27 @@ def main():
     env, ops = config_ops("c2", cumo_amd, host)
     step_bytes = sum(o[2] for o in ops)
 
-    # One step through the host mirror records the launcher calls it makes. The
-    # timed step issues those same C-ABI calls, plus the pool round trip the
-    # extension's host side makes for each result (allocate before the launch,
-    # release afterwards), so it is the path the drop-in runs minus the Ruby VM.
-    step_calls = []
-    for _, fn, _, _ in ops:
-        with _lib.record() as calls:
-            fn(env)
-        step_calls.append(calls)
-    result_bytes = [8 * n * n, 8 * n, 8 * n]
-    pool_malloc, pool_free = lib.cumo_cuda_runtime_malloc, lib.cumo_cuda_runtime_free
+    # The timed step is the chain as the extension's C host side runs it: three
+    # calls into the library's host launch layer (broadcast, result allocation
+    # from the pool, descriptors, launch), each result released again once the
+    # chain is done. Only the Ruby VM above it is missing.
+    NA = _lib.NArrayDesc
+    dA, dr = env["A"]._desc(), env["r"]._desc()
+    na_binary, na_reduce, na_free = lib.cumo_hip_na_binary, lib.cumo_hip_na_reduce, lib.cumo_cuda_runtime_free
+    ref = C.byref
 
     def step():
-        for calls, nb in zip(step_calls, result_bytes):
-            p = pool_malloc(nb)
-            for f, a in calls:
-                f(*a)
-            pool_free(p)
+        zc, zs, zm = NA(), NA(), NA()
+        na_binary(b"add", ref(dA), ref(dr), ref(zc))
+        na_reduce(b"sum", ref(zc), 2, 0, 0, ref(zs), None)
+        na_reduce(b"max", ref(zc), 2, 0, 0, ref(zm), None)
+        na_free(zs.ptr)
+        na_free(zm.ptr)
+        na_free(zc.ptr)
+
+    # per-launch timing of the dominant kernel replays the recorded call of the add
+    with _lib.record() as add_calls:
+        ops[0][1](env)
 
     for _ in range(args.warmup):
         step()
@@ -325,7 +329,7 @@ def main():
     # dominant kernel, per launch: HIP events on the launch stream around batches of
     # back-to-back launches
     timer = Timer(lib)
-    add_calls, add_bytes = step_calls[0], ops[0][2]
+    add_bytes = ops[0][2]
     batch = 10
     ts = sorted(timer.time(lambda: _lib.replay(add_calls, batch)) / batch for _ in range(max(20, args.steps)))
     timer.close()

@@ -25,6 +25,10 @@ class ShapeError(ValueError):
     """Cumo::NArray::ShapeError (reference: ext/cumo/narray/ndloop.c:508-512)."""
 
 
+class DimensionError(ValueError):
+    """Cumo::NArray::DimensionError (reference: ext/cumo/narray/narray.c:1757-1759)."""
+
+
 class Indexer(C.Structure):
     # reference: ext/cumo/include/cumo/indexer.h:16-22
     _fields_ = [("ndim", C.c_ubyte), ("total_size", C.c_size_t), ("shape", C.c_size_t * MAX_DIM),
@@ -54,6 +58,37 @@ class BitIArrayStridx(C.Structure):
 class ReductionArg(C.Structure):
     # reference: indexer.h:63-68
     _fields_ = [("in_", IArray), ("out", IArray), ("in_indexer", Indexer), ("out_indexer", Indexer)]
+
+
+class NArrayDesc(C.Structure):
+    """cumo_hip_narray_t (include/cumo_hip_ndloop.h): a view of device memory."""
+    _fields_ = [("type", C.c_int), ("ndim", C.c_int), ("ptr", C.c_void_p), ("offset", C.c_ssize_t),
+                ("shape", C.c_size_t * MAX_DIM), ("stride", C.c_ssize_t * MAX_DIM)]
+
+
+class LoopArgs(C.Structure):
+    """cumo_hip_loop_args_t"""
+    _fields_ = [("type", C.c_int), ("elmsz", C.c_ssize_t), ("ptr", C.c_void_p), ("bitpos", C.c_size_t),
+                ("step", C.c_ssize_t * MAX_DIM)]
+
+
+class Loop(C.Structure):
+    """cumo_hip_loop_t"""
+    _fields_ = [("narg", C.c_int), ("ndim", C.c_int), ("n", C.c_size_t * MAX_DIM), ("args", LoopArgs * 4),
+                ("reduce_dim", C.c_int), ("opt_ptr", C.c_void_p), ("status", C.c_int)]
+
+
+ITER_FUNC = C.CFUNCTYPE(None, C.POINTER(Loop))
+
+
+class NdFunc(C.Structure):
+    """cumo_hip_ndfunc_t"""
+    _fields_ = [("func", ITER_FUNC), ("flag", C.c_uint), ("nin", C.c_int), ("nout", C.c_int), ("out_type", C.c_int * 2)]
+
+
+NDF_FLAT_REDUCE = 1 << 6
+NDF_KEEP_DIM = 1 << 3
+TYPE_CODE = {"sfloat": 0, "dfloat": 1, "int32": 2, "int64": 3, "uint64": 4, "bit": 5}
 
 
 class EwPlan(C.Structure):
@@ -111,6 +146,33 @@ _sig = {
     "cumo_hip_pool_use_host_backend": (C.c_int, [C.c_int]),
     "cumo_hip_plan_elementwise": (C.c_int, [P(Indexer), C.c_int, P(P(IArray)), P(C.c_int), P(C.c_size_t), P(EwPlan)]),
     "cumo_hip_plan_reduce": (C.c_int, [P(ReductionArg), C.c_int, C.c_int, P(ReducePlan)]),
+    # host launch layer (include/cumo_hip_ndloop.h)
+    "cumo_hip_na_storage_bytes": (C.c_size_t, [C.c_int, C.c_size_t]),
+    "cumo_hip_na_alloc": (C.c_int, [P(NArrayDesc), C.c_int, C.c_int, P(C.c_size_t)]),
+    "cumo_hip_na_ndloop": (C.c_int, [P(NdFunc), P(P(NArrayDesc)), P(P(NArrayDesc)), C.c_uint, C.c_void_p]),
+    "cumo_hip_na_ndloop_prepare": (C.c_int, [P(NdFunc), P(P(NArrayDesc)), P(P(NArrayDesc)), C.c_uint, P(Loop)]),
+    "cumo_hip_make_indexer": (None, [P(Loop), P(Indexer)]),
+    "cumo_hip_make_iarray": (None, [P(Loop), C.c_int, P(IArray)]),
+    "cumo_hip_make_bit_iarray": (None, [P(Loop), C.c_int, P(BitIArray)]),
+    "cumo_hip_make_iarray_stridx": (None, [P(Loop), C.c_int, P(IArrayStridx)]),
+    "cumo_hip_make_bit_iarray_stridx": (None, [P(Loop), C.c_int, P(BitIArrayStridx)]),
+    "cumo_hip_make_reduction_arg": (None, [P(Loop), P(ReductionArg)]),
+    "cumo_hip_na_binary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_binary_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_math": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_math2": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_math2_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_compare": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_compare_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_cond_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_store": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_copy": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_fill": (C.c_int, [P(NArrayDesc), C.c_double]),
+    "cumo_hip_na_reduce": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_uint, C.c_int, C.c_int, P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_bit_binary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_bit_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_bit_count": (C.c_int, [P(NArrayDesc), C.c_uint, C.c_int, C.c_int, P(NArrayDesc)]),
 }
 for _name, (_res, _args) in _sig.items():
     _f = getattr(lib, _name)
@@ -141,8 +203,16 @@ def check():
     text = msg.value.decode("utf-8", "replace") if msg.value else ""
     if kind == 2:
         raise OutOfMemoryError(text)
-    if kind == 3:
+    if kind in (3, 7):
         raise ValueError(text)
+    if kind == 4:
+        raise ShapeError(text)
+    if kind == 5:
+        raise ZeroDivisionError(text)
+    if kind == 6:
+        raise TypeError(text)
+    if kind == 8:
+        raise DimensionError(text)
     raise RuntimeError_(text)
 
 
@@ -150,7 +220,8 @@ _recording = None
 
 
 def call(f, *args):
-    if _recording is not None and (f.__name__.endswith("_kernel_launch") or f.__name__ == "cumo_hip_memset"):
+    if _recording is not None and (f.__name__.endswith("_kernel_launch") or f.__name__.startswith("cumo_hip_na_")
+                                   or f.__name__ == "cumo_hip_memset"):
         _recording.append((f, args))
     r = f(*args)
     check()
@@ -158,10 +229,12 @@ def call(f, *args):
 
 
 class record:
-    """Collects the launcher calls (function, arguments) made inside the block, so
-    that a caller can issue exactly the same launches again without the host-side
-    work of building them: `with record() as calls: y = a + b`, then
-    `replay(calls)`. The arrays the launches write into must be kept alive."""
+    """Collects the library calls (function, arguments) that launch work inside the
+    block, so that a caller can issue exactly the same calls again without the
+    Python-side work of building them: `with record() as calls: y = a + b`, then
+    `replay(calls)`. A recorded host-layer call carries its result descriptor with
+    the memory the first call allocated, so a replay writes into the same array;
+    the arrays involved must be kept alive."""
 
     def __enter__(self):
         global _recording

@@ -1,0 +1,1149 @@
+// The host launch layer: array views in, launch descriptors out, one launcher
+// call per operation.
+//
+// Replaces, for the stride-view operands of the array hot path,
+//   ext/cumo/narray/ndloop.c:339-452,493-595,749-863,870-1168,1459-1616
+//     (broadcast, reduce dimensions moved last, result allocation, loop
+//     contraction, the single call of the user iterator),
+//   ext/cumo/include/cumo/indexer.h:114-220 (cumo_na_make_*), and
+//   the host iterators / method bodies the reference generates per type from
+//   ext/cumo/narray/gen/tmpl/{binary,unary,unary2,unary_s,binary_s,cond_binary,
+//   cond_unary,store_from,store_bit,fill,accum,minmax,accum_arg,accum_index}.c
+//   and gen/tmpl_bit/{binary,unary,bit_count}.c.
+//
+// The reference prepares a loop with one xmalloc and a handful of Ruby calls
+// per operation and decomposes nothing itself; the per-element index
+// arithmetic is left to the kernels. Here the loop lives in a fixed-size struct
+// on the caller's stack, dimensions are merged before the launcher sees them,
+// and the per-type method bodies are tables of launcher pointers looked up by
+// operation name.
+//
+// No function here keeps a C++ object with a destructor alive across a call
+// that may report an error: the installed handler may leave with longjmp.
+#include <cstdio>
+#include <cstring>
+
+#include "common.h"
+#include "cumo_hip_ndloop.h"
+
+namespace {
+
+using cumo_hip::report_error;
+
+typedef cumo_na_iarray_t IA;
+typedef cumo_na_bit_iarray_t BIA;
+typedef cumo_na_indexer_t IX;
+typedef cumo_hip_narray_t NA;
+typedef cumo_hip_loop_t LP;
+
+const int kElmsz[CUMO_HIP_N_TYPES] = {4, 8, 4, 8, 8, 0};
+const int kMaxDim = CUMO_NA_MAX_DIMENSION;
+
+int fail(int kind, const char* msg) {
+    report_error(kind, 0, msg);
+    return kind;
+}
+
+inline bool valid_type(int t) { return t >= 0 && t < CUMO_HIP_N_TYPES; }
+inline bool is_arith(int t) { return t == CUMO_HIP_SFLOAT || t == CUMO_HIP_DFLOAT || t == CUMO_HIP_INT32; }
+inline bool is_float(int t) { return t == CUMO_HIP_SFLOAT || t == CUMO_HIP_DFLOAT; }
+
+size_t total_of(const NA* a) {
+    size_t n = 1;
+    for (int d = 0; d < a->ndim; d++) n *= a->shape[d];
+    return n;
+}
+
+// a view whose elements sit in row-major order without gaps (any offset)
+bool is_contiguous(const NA* a) {
+    ssize_t unit = a->type == CUMO_HIP_BIT ? 1 : kElmsz[a->type];
+    ssize_t s = unit;
+    for (int d = a->ndim - 1; d >= 0; d--) {
+        if (a->shape[d] != 1 && a->stride[d] != s) return false;
+        s *= (ssize_t)a->shape[d];
+    }
+    return true;
+}
+
+int check_view(const NA* a, const char* what) {
+    if (!a) return fail(CUMO_HIP_ERROR_ARGUMENT, "ndloop: missing array argument");
+    if (!valid_type(a->type)) return fail(CUMO_HIP_ERROR_TYPE, "ndloop: unknown element type");
+    if (a->ndim < 0 || a->ndim > kMaxDim) return fail(CUMO_HIP_ERROR_DIMENSION, "ndloop: too many dimensions");
+    if (a->type == CUMO_HIP_BIT && a->offset < 0) return fail(CUMO_HIP_ERROR_ARGUMENT, "ndloop: negative bit offset");
+    (void)what;
+    return CUMO_HIP_OK;
+}
+
+// Merges and drops loop dimensions inside [lo, hi) and appends what is left at
+// position `at`; returns the new end. Two neighbours merge when every argument
+// walks them as one run: step[outer] == step[inner] * n[inner]
+// (reference: cumo_ndfunc_contract_loop, ndloop.c:870-940; like it, reduce and
+// kept dimensions never merge with each other).
+int contract_range(LP* lp, const size_t* n, const ssize_t (*step)[kMaxDim], int lo, int hi, int at, bool keep_one) {
+    int first = at;
+    for (int d = lo; d < hi; d++) {
+        if (n[d] == 1) continue;
+        if (at > first) {
+            int p = at - 1;
+            bool merge = true;
+            for (int j = 0; j < lp->narg && merge; j++)
+                merge = lp->args[j].step[p] == step[j][d] * (ssize_t)n[d];
+            if (merge) {
+                lp->n[p] *= n[d];
+                for (int j = 0; j < lp->narg; j++) lp->args[j].step[p] = step[j][d];
+                continue;
+            }
+        }
+        lp->n[at] = n[d];
+        for (int j = 0; j < lp->narg; j++) lp->args[j].step[at] = step[j][d];
+        at++;
+    }
+    if (at == first && keep_one) {
+        lp->n[at] = 1;
+        for (int j = 0; j < lp->narg; j++) lp->args[j].step[at] = 0;
+        at++;
+    }
+    return at;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t cumo_hip_na_storage_bytes(int type, size_t n) {
+    if (!valid_type(type)) return 0;
+    if (type == CUMO_HIP_BIT) return ((n + 31) / 32) * 4;
+    return n * (size_t)kElmsz[type];
+}
+
+int cumo_hip_na_alloc(cumo_hip_narray_t* a, int type, int ndim, const size_t* shape) {
+    if (!a || !valid_type(type) || ndim < 0 || ndim > kMaxDim) return fail(CUMO_HIP_ERROR_ARGUMENT, "na_alloc: bad arguments");
+    a->type = type;
+    a->ndim = ndim;
+    a->offset = 0;
+    a->ptr = NULL;
+    ssize_t s = type == CUMO_HIP_BIT ? 1 : kElmsz[type];
+    size_t n = 1;
+    for (int d = ndim - 1; d >= 0; d--) {
+        a->shape[d] = shape[d];
+        a->stride[d] = s;
+        s *= (ssize_t)shape[d];
+        n *= shape[d];
+    }
+    size_t bytes = cumo_hip_na_storage_bytes(type, n);
+    if (bytes) {
+        a->ptr = cumo_cuda_runtime_malloc(bytes);  // reports the failure itself
+        if (!a->ptr) return CUMO_HIP_ERROR_OUT_OF_MEMORY;
+    }
+    return CUMO_HIP_OK;
+}
+
+int cumo_hip_na_ndloop_prepare(const cumo_hip_ndfunc_t* nf, const cumo_hip_narray_t* const* in,
+                               cumo_hip_narray_t* const* out, unsigned int reduce, cumo_hip_loop_t* lp) {
+    if (!nf || !lp || nf->nin < 1 || nf->nout < 0 || nf->nout > 2 || nf->nin + nf->nout > CUMO_HIP_NDLOOP_MAX_ARGS)
+        return fail(CUMO_HIP_ERROR_ARGUMENT, "ndloop: bad ndfunc");
+    const int nin = nf->nin, nout = nf->nout;
+    std::memset(lp, 0, sizeof(*lp));
+    lp->narg = nin + nout;
+
+    // the loop's rank and shape: operands are aligned at their last dimension
+    // and a dimension of size 1 repeats (ndloop.c:493-516)
+    int nd = 0;
+    for (int j = 0; j < nin; j++) {
+        int rc = check_view(in[j], "input");
+        if (rc) return rc;
+        if (in[j]->ndim > nd) nd = in[j]->ndim;
+    }
+    size_t bshape[kMaxDim];
+    for (int i = 0; i < nd; i++) bshape[i] = 1;
+    for (int j = 0; j < nin; j++) {
+        int off = nd - in[j]->ndim;
+        for (int k = 0; k < in[j]->ndim; k++) {
+            size_t n = in[j]->shape[k];
+            if (n == 1) continue;
+            if (bshape[off + k] == 1) {
+                bshape[off + k] = n;
+            } else if (bshape[off + k] != n) {
+                char msg[128];
+                std::snprintf(msg, sizeof(msg), "shape1[%d](=%zu) != shape2[%d](=%zu)", off + k, bshape[off + k], k, n);
+                return fail(CUMO_HIP_ERROR_SHAPE, msg);
+            }
+        }
+    }
+
+    // reduce dimensions go last: array [*,+,*,+,*] => loop [*,*,*,+,+] (ndloop.c:421-451)
+    if (reduce && !(nf->flag & CUMO_HIP_NDF_FLAT_REDUCE)) return fail(CUMO_HIP_ERROR_ARGUMENT, "ndloop: this operation does not reduce");
+    if (nd < 32 && (reduce >> nd)) return fail(CUMO_HIP_ERROR_DIMENSION, "dimension is out of range");
+    int trans_map[kMaxDim];
+    int nkeep = 0;
+    for (int i = 0; i < nd; i++)
+        if (!((reduce >> i) & 1u)) trans_map[i] = nkeep++;
+    {
+        int j = nkeep;
+        for (int i = 0; i < nd; i++)
+            if ((reduce >> i) & 1u) trans_map[i] = j++;
+    }
+    size_t n[kMaxDim];
+    ssize_t step[CUMO_HIP_NDLOOP_MAX_ARGS][kMaxDim];
+    std::memset(step, 0, sizeof(step));
+    for (int i = 0; i < nd; i++) n[trans_map[i]] = bshape[i];
+
+    // inputs (ndloop.c:519-595)
+    for (int j = 0; j < nin; j++) {
+        const NA* a = in[j];
+        cumo_hip_loop_args_t* la = &lp->args[j];
+        la->type = a->type;
+        la->elmsz = kElmsz[a->type];
+        if (a->type == CUMO_HIP_BIT) {
+            la->ptr = a->ptr;
+            la->bitpos = (size_t)a->offset;
+        } else {
+            la->ptr = a->ptr + a->offset;
+        }
+        int off = nd - a->ndim;
+        for (int k = 0; k < a->ndim; k++) step[j][trans_map[off + k]] = a->shape[k] == 1 ? 0 : a->stride[k];
+    }
+
+    // results: the loop's shape without the reduced dimensions, or with them
+    // at size 1 under KEEP_DIM (ndloop.c:750-863)
+    const bool keep = (nf->flag & CUMO_HIP_NDF_KEEP_DIM) != 0;
+    size_t rshape[kMaxDim];
+    int rmap[kMaxDim];
+    int rnd = 0;
+    for (int i = 0; i < nd; i++) {
+        bool red = (reduce >> i) & 1u;
+        if (red && !keep) {
+            rmap[i] = -1;
+        } else {
+            rshape[rnd] = red ? 1 : bshape[i];
+            rmap[i] = rnd++;
+        }
+    }
+    for (int j = 0; j < nout; j++) {
+        NA* o = out[j];
+        const int type = nf->out_type[j];
+        if (!o) return fail(CUMO_HIP_ERROR_ARGUMENT, "ndloop: missing result argument");
+        if (o->ptr == NULL) {
+            int rc = cumo_hip_na_alloc(o, type, rnd, rshape);
+            if (rc) return rc;
+        } else {
+            int rc = check_view(o, "result");
+            if (rc) return rc;
+            if (o->type != type) return fail(CUMO_HIP_ERROR_TYPE, "ndloop: result array has the wrong element type");
+            bool same = o->ndim == rnd;
+            for (int d = 0; same && d < rnd; d++) same = o->shape[d] == rshape[d];
+            if (!same) return fail(CUMO_HIP_ERROR_SHAPE, "ndloop: result array has the wrong shape");
+        }
+        cumo_hip_loop_args_t* la = &lp->args[nin + j];
+        la->type = type;
+        la->elmsz = kElmsz[type];
+        if (type == CUMO_HIP_BIT) {
+            la->ptr = o->ptr;
+            la->bitpos = (size_t)o->offset;
+        } else {
+            la->ptr = o->ptr + o->offset;
+        }
+        for (int i = 0; i < nd; i++) {
+            bool red = (reduce >> i) & 1u;
+            step[nin + j][trans_map[i]] = (red || rmap[i] < 0 || o->shape[rmap[i]] == 1) ? 0 : o->stride[rmap[i]];
+        }
+    }
+
+    // contraction, separately for the kept and the reduced dimensions
+    int at = contract_range(lp, n, step, 0, nkeep, 0, false);
+    int nkept = at;
+    // a reducing operation always keeps one reduce dimension, of size 1 if need be
+    at = contract_range(lp, n, step, nkeep, nd, at, (nf->flag & CUMO_HIP_NDF_FLAT_REDUCE) != 0);
+    lp->reduce_dim = at - nkept;
+    if (at == 0) {  // a single element
+        lp->n[0] = 1;
+        at = 1;
+    }
+    lp->ndim = at;
+    return CUMO_HIP_OK;
+}
+
+int cumo_hip_na_ndloop(const cumo_hip_ndfunc_t* nf, const cumo_hip_narray_t* const* in,
+                       cumo_hip_narray_t* const* out, unsigned int reduce, void* opt_ptr) {
+    cumo_hip_loop_t lp;
+    int rc = cumo_hip_na_ndloop_prepare(nf, in, out, reduce, &lp);
+    if (rc) return rc;
+    lp.opt_ptr = opt_ptr;
+    size_t out_total = 1;
+    for (int d = 0; d < lp.ndim - lp.reduce_dim; d++) out_total *= lp.n[d];
+    if (out_total == 0) return CUMO_HIP_OK;  // nothing to write (template_kernel.h:76-81)
+    nf->func(&lp);
+    return lp.status;
+}
+
+void cumo_hip_make_indexer(const cumo_hip_loop_t* lp, cumo_na_indexer_t* ix) {
+    std::memset(ix, 0, sizeof(*ix));
+    ix->ndim = (unsigned char)lp->ndim;
+    size_t t = 1;
+    for (int d = 0; d < lp->ndim; d++) {
+        ix->shape[d] = lp->n[d];
+        t *= lp->n[d];
+    }
+    ix->total_size = t;
+}
+
+void cumo_hip_make_iarray(const cumo_hip_loop_t* lp, int j, cumo_na_iarray_t* a) {
+    std::memset(a, 0, sizeof(*a));
+    a->ptr = lp->args[j].ptr;
+    for (int d = 0; d < lp->ndim; d++) a->step[d] = lp->args[j].step[d];
+}
+
+void cumo_hip_make_bit_iarray(const cumo_hip_loop_t* lp, int j, cumo_na_bit_iarray_t* a) {
+    std::memset(a, 0, sizeof(*a));
+    a->ptr = (CUMO_BIT_DIGIT*)lp->args[j].ptr;
+    a->pos = lp->args[j].bitpos;
+    for (int d = 0; d < lp->ndim; d++) a->step[d] = lp->args[j].step[d];
+}
+
+void cumo_hip_make_iarray_stridx(const cumo_hip_loop_t* lp, int j, cumo_na_iarray_stridx_t* a) {
+    std::memset(a, 0, sizeof(*a));
+    a->ptr = lp->args[j].ptr;
+    for (int d = 0; d < kMaxDim; d++) CUMO_SDX_SET_STRIDE(a->stridx[d], d < lp->ndim ? lp->args[j].step[d] : 0);
+}
+
+void cumo_hip_make_bit_iarray_stridx(const cumo_hip_loop_t* lp, int j, cumo_na_bit_iarray_stridx_t* a) {
+    std::memset(a, 0, sizeof(*a));
+    a->ptr = (CUMO_BIT_DIGIT*)lp->args[j].ptr;
+    a->pos = lp->args[j].bitpos;
+    for (int d = 0; d < kMaxDim; d++) CUMO_SDX_SET_STRIDE(a->stridx[d], d < lp->ndim ? lp->args[j].step[d] : 0);
+}
+
+void cumo_hip_make_reduction_arg(const cumo_hip_loop_t* lp, cumo_na_reduction_arg_t* arg) {
+    std::memset(arg, 0, sizeof(*arg));
+    cumo_hip_make_iarray(lp, 0, &arg->in);
+    cumo_hip_make_indexer(lp, &arg->in_indexer);
+    const int ond = lp->ndim - lp->reduce_dim;
+    arg->out.ptr = lp->args[1].ptr;
+    arg->out_indexer.ndim = (unsigned char)ond;
+    size_t t = 1;
+    for (int d = 0; d < ond; d++) {
+        arg->out.step[d] = lp->args[1].step[d];
+        arg->out_indexer.shape[d] = lp->n[d];
+        t *= lp->n[d];
+    }
+    arg->out_indexer.total_size = t;
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// Operation tables: what the reference generates as one C function per type
+// and method (gen/spec.rb:199-277,427-457) is one row per method here.
+// ---------------------------------------------------------------------------
+namespace {
+
+template <class C>
+struct BinFns {
+    void (*f)(IA*, IA*, IA*, IX*, int*);
+    void (*fs)(IA*, C, IA*, IX*, int*, int);
+};
+struct BinaryRow {
+    const char* op;
+    BinFns<float> sf;
+    BinFns<double> df;
+    BinFns<int32_t> i32;
+};
+#define BIN_FNS(t, op) {cumo_iter_##t##_##op##_kernel_launch, cumo_iter_##t##_##op##_s_kernel_launch}
+#define BIN_ROW_ALL(t, c, op) {#op, BIN_FNS(sfloat, op), BIN_FNS(dfloat, op), BIN_FNS(int32, op)},
+#define BIN_ROW_FLT(t, c, op) {#op, BIN_FNS(sfloat, op), BIN_FNS(dfloat, op), {nullptr, nullptr}},
+#define BIN_ROW_INT(t, c, op) {#op, {nullptr, nullptr}, {nullptr, nullptr}, BIN_FNS(int32, op)},
+const BinaryRow kBinary[] = {
+    CUMO_HIP_BINARY_OPS_ALL(BIN_ROW_ALL, _, _)
+    CUMO_HIP_BINARY_OPS_FLOAT(BIN_ROW_FLT, _, _)
+    CUMO_HIP_BINARY_OPS_INT(BIN_ROW_INT, _, _)
+};
+
+typedef void (*UnaryFn)(IA*, IA*, IX*, int*);
+struct UnaryRow {
+    const char* op;
+    UnaryFn f[3];  // sfloat, dfloat, int32
+};
+#define UN_ROW_ALL(t, c, op) {#op, {cumo_iter_sfloat_##op##_kernel_launch, cumo_iter_dfloat_##op##_kernel_launch, cumo_iter_int32_##op##_kernel_launch}},
+#define UN_ROW_FLT(t, c, op) {#op, {cumo_iter_sfloat_##op##_kernel_launch, cumo_iter_dfloat_##op##_kernel_launch, nullptr}},
+#define UN_ROW_INT(t, c, op) {#op, {nullptr, nullptr, cumo_iter_int32_##op##_kernel_launch}},
+const UnaryRow kUnary[] = {
+    CUMO_HIP_UNARY_OPS_ALL(UN_ROW_ALL, _, _)
+    CUMO_HIP_UNARY_OPS_FLOAT(UN_ROW_FLT, _, _)
+    CUMO_HIP_UNARY_OPS_INT(UN_ROW_INT, _, _)
+    UN_ROW_ALL(_, _, abs)
+};
+
+typedef void (*MathFn)(IA*, IA*, IX*);
+struct MathRow {
+    const char* op;
+    MathFn f[2];
+};
+#define MATH_ROW(t, c, op) {#op, {cumo_iter_sfloat_math_s_##op##_kernel_launch, cumo_iter_dfloat_math_s_##op##_kernel_launch}},
+const MathRow kMath[] = {CUMO_HIP_MATH_OPS(MATH_ROW, _, _)};
+
+struct Math2Row {
+    const char* op;
+    void (*sf)(IA*, IA*, IA*, IX*);
+    void (*sfs)(IA*, IA*, IX*, float, int);
+    void (*df)(IA*, IA*, IA*, IX*);
+    void (*dfs)(IA*, IA*, IX*, double, int);
+};
+#define MATH2_ROW(t, c, op) {#op, cumo_iter_sfloat_math_s_##op##_kernel_launch, cumo_iter_sfloat_math_s_##op##_s_kernel_launch, \
+                             cumo_iter_dfloat_math_s_##op##_kernel_launch, cumo_iter_dfloat_math_s_##op##_s_kernel_launch},
+const Math2Row kMath2[] = {CUMO_HIP_MATH2_OPS(MATH2_ROW, _, _)};
+
+template <class C>
+struct CondFns {
+    void (*f)(IA*, IA*, BIA*, IX*);
+    void (*fs)(IA*, C, BIA*, IX*, int);
+};
+struct CondRow {
+    const char* op;
+    CondFns<float> sf;
+    CondFns<double> df;
+    CondFns<int32_t> i32;
+};
+#define COND_ROW_ALL(t, c, op) {#op, BIN_FNS(sfloat, op), BIN_FNS(dfloat, op), BIN_FNS(int32, op)},
+#define COND_ROW_FLT(t, c, op) {#op, BIN_FNS(sfloat, op), BIN_FNS(dfloat, op), {nullptr, nullptr}},
+const CondRow kCond[] = {
+    CUMO_HIP_COND_OPS_ALL(COND_ROW_ALL, _, _)
+    CUMO_HIP_COND_OPS_FLOAT(COND_ROW_FLT, _, _)
+};
+
+typedef void (*CondUnaryFn)(IA*, BIA*, IX*);
+struct CondUnaryRow {
+    const char* op;
+    CondUnaryFn f[2];
+};
+#define CONDU_ROW(t, c, op) {#op, {cumo_iter_sfloat_##op##_kernel_launch, cumo_iter_dfloat_##op##_kernel_launch}},
+const CondUnaryRow kCondUnary[] = {CUMO_HIP_COND_UNARY_OPS(CONDU_ROW, _, _)};
+
+typedef void (*StoreFn)(IA*, IA*, IX*);
+// [dst: sfloat dfloat int32][src: sfloat dfloat int32 int64]
+#define STORE_ROW(d) {cumo_iter_##d##_store_sfloat_kernel_launch, cumo_iter_##d##_store_dfloat_kernel_launch, \
+                      cumo_iter_##d##_store_int32_kernel_launch, cumo_iter_##d##_store_int64_kernel_launch}
+const StoreFn kStore[3][4] = {STORE_ROW(sfloat), STORE_ROW(dfloat), STORE_ROW(int32)};
+
+typedef void (*StoreBitFn)(cumo_na_iarray_stridx_t*, cumo_na_bit_iarray_stridx_t*, IX*);
+const StoreBitFn kStoreBit[3] = {cumo_iter_sfloat_store_bit_kernel_launch, cumo_iter_dfloat_store_bit_kernel_launch,
+                                 cumo_iter_int32_store_bit_kernel_launch};
+
+typedef void (*ReduceFn)(cumo_na_reduction_arg_t*);
+typedef void (*ReducePairFn)(cumo_na_reduction_arg_t*, IA*);
+struct ReduceRow {
+    const char* op;
+    ReduceFn f[3];      // sfloat, dfloat, int32
+    ReduceFn f_nan[3];
+    int result;         // 0 same type, 1 the type sum answers (Int32 -> Int64)
+};
+#define RED3(name) {cumo_sfloat_##name##_kernel_launch, cumo_dfloat_##name##_kernel_launch, cumo_int32_##name##_kernel_launch}
+#define RED2(name) {cumo_sfloat_##name##_kernel_launch, cumo_dfloat_##name##_kernel_launch, nullptr}
+const ReduceRow kReduce[] = {
+    {"sum", RED3(sum), RED2(sum_nan), 1},
+    {"prod", RED3(prod), RED2(prod_nan), 1},
+    {"min", RED3(min), RED2(min_nan), 0},
+    {"max", RED3(max), RED2(max_nan), 0},
+    {"ptp", RED3(ptp), RED2(ptp_nan), 0},
+    {"mean", RED2(mean), RED2(mean_nan), 0},
+    {"var", RED2(var), RED2(var_nan), 0},
+    {"stddev", RED2(stddev), RED2(stddev_nan), 0},
+    {"rms", RED2(rms), RED2(rms_nan), 0},
+    {"kahan_sum", {nullptr, cumo_dfloat_kahan_sum_kernel_launch, nullptr}, {nullptr, cumo_dfloat_kahan_sum_nan_kernel_launch, nullptr}, 0},
+};
+struct ArgRow {
+    const char* op;
+    ReduceFn f32[3], f64[3], f32_nan[3], f64_nan[3];
+    bool memory_index;  // min_index/max_index: the answer indexes the operand's own flattening
+};
+#define ARG_ROW(name, mi) {#name, RED3(name##_int32), RED3(name##_int64), RED2(name##_nan_int32), RED2(name##_nan_int64), mi}
+const ArgRow kArg[] = {ARG_ROW(argmin, false), ARG_ROW(argmax, false), ARG_ROW(min_index, true), ARG_ROW(max_index, true)};
+const ReducePairFn kMinmax[3] = {cumo_sfloat_minmax_kernel_launch, cumo_dfloat_minmax_kernel_launch, cumo_int32_minmax_kernel_launch};
+const ReducePairFn kMinmaxNan[3] = {cumo_sfloat_minmax_nan_kernel_launch, cumo_dfloat_minmax_nan_kernel_launch, nullptr};
+
+typedef cumo_na_bit_iarray_stridx_t BSX;
+struct BitBinaryRow {
+    const char* op;
+    void (*f)(BSX*, BSX*, BSX*, IX*);
+    void (*fc)(CUMO_BIT_DIGIT*, size_t, CUMO_BIT_DIGIT*, size_t, CUMO_BIT_DIGIT*, size_t, uint64_t);
+};
+#define BITB_ROW(op) {#op, cumo_iter_bit_##op##_kernel_launch, cumo_iter_bit_##op##_contiguous_kernel_launch},
+const BitBinaryRow kBitBinary[] = {CUMO_HIP_BIT_BINARY_OPS(BITB_ROW)};
+struct BitUnaryRow {
+    const char* op;
+    void (*f)(BSX*, BSX*, IX*);
+    void (*fc)(CUMO_BIT_DIGIT*, size_t, CUMO_BIT_DIGIT*, size_t, uint64_t);
+};
+#define BITU_ROW(op) {#op, cumo_iter_bit_##op##_kernel_launch, cumo_iter_bit_##op##_contiguous_kernel_launch},
+const BitUnaryRow kBitUnary[] = {CUMO_HIP_BIT_UNARY_OPS(BITU_ROW)};
+
+template <class Row, size_t N>
+const Row* find_row(const Row (&rows)[N], const char* op) {
+    if (!op) return nullptr;
+    for (size_t i = 0; i < N; i++)
+        if (std::strcmp(rows[i].op, op) == 0) return &rows[i];
+    return nullptr;
+}
+
+int no_method(const char* op) {
+    char msg[96];
+    std::snprintf(msg, sizeof(msg), "undefined operation '%s' for this element type", op ? op : "(null)");
+    return fail(CUMO_HIP_ERROR_TYPE, msg);
+}
+
+// the higher of two arithmetic types: Int32 < SFloat < DFloat
+// (the upcast tables of gen/def/{int32,sfloat,dfloat}.rb)
+int upcast(int a, int b) {
+    static const int rank[3] = {1, 2, 0};  // indexed by type: sfloat, dfloat, int32
+    return rank[a] >= rank[b] ? a : b;
+}
+
+void free_tmp(NA* t) {
+    if (t->ptr) {
+        cumo_cuda_runtime_free(t->ptr);
+        t->ptr = NULL;
+    }
+}
+
+// ---- iterators ---------------------------------------------------------------
+struct StoreOpt {
+    StoreFn f;
+};
+void iter_store(LP* lp) {  // args: dst, src (gen/tmpl/store_from.c)
+    IA a1, a2;
+    IX ix;
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    cumo_hip_make_indexer(lp, &ix);
+    ((StoreOpt*)lp->opt_ptr)->f(&a1, &a2, &ix);
+}
+
+// *use = x itself, or a contiguous copy of x in `type` held by tmp
+int cast_operand(const NA* x, int type, NA* tmp, const NA** use) {
+    tmp->ptr = NULL;
+    if (x->type == type) {
+        *use = x;
+        return CUMO_HIP_OK;
+    }
+    int rc = cumo_hip_na_alloc(tmp, type, x->ndim, x->shape);
+    if (rc) return rc;
+    *use = tmp;
+    if (total_of(x) == 0) return CUMO_HIP_OK;
+    StoreOpt opt = {kStore[type][x->type]};
+    cumo_hip_ndfunc_t nf = {iter_store, 0, 2, 0, {0, 0}};
+    const NA* in[2] = {tmp, x};
+    return cumo_hip_na_ndloop(&nf, in, NULL, 0, &opt);
+}
+
+struct BinaryOpt {
+    const BinaryRow* row;
+    int type;
+    bool scalar;
+    double sv;
+    int left;
+    bool checked;   // the launcher reports a data error through the pinned flag
+    bool flagged;
+};
+void iter_binary(LP* lp) {
+    BinaryOpt* o = (BinaryOpt*)lp->opt_ptr;
+    IA a1, a2, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    int* flag = o->checked ? cumo_cuda_runtime_error_flag_new() : NULL;
+    if (o->scalar) {
+        cumo_hip_make_iarray(lp, 1, &a3);
+        switch (o->type) {
+            case CUMO_HIP_SFLOAT: o->row->sf.fs(&a1, (float)o->sv, &a3, &ix, flag, o->left); break;
+            case CUMO_HIP_DFLOAT: o->row->df.fs(&a1, o->sv, &a3, &ix, flag, o->left); break;
+            default: o->row->i32.fs(&a1, (int32_t)o->sv, &a3, &ix, flag, o->left); break;
+        }
+    } else {
+        cumo_hip_make_iarray(lp, 1, &a2);
+        cumo_hip_make_iarray(lp, 2, &a3);
+        switch (o->type) {
+            case CUMO_HIP_SFLOAT: o->row->sf.f(&a1, &a2, &a3, &ix, flag); break;
+            case CUMO_HIP_DFLOAT: o->row->df.f(&a1, &a2, &a3, &ix, flag); break;
+            default: o->row->i32.f(&a1, &a2, &a3, &ix, flag); break;
+        }
+    }
+    // the caller reads the flag with a stream synchronisation (gen/tmpl/binary.c:120-126)
+    if (flag && cumo_cuda_runtime_error_flag_get(flag)) o->flagged = true;
+}
+
+bool binary_has(const BinaryRow* r, int type, bool scalar) {
+    switch (type) {
+        case CUMO_HIP_SFLOAT: return scalar ? r->sf.fs != nullptr : r->sf.f != nullptr;
+        case CUMO_HIP_DFLOAT: return scalar ? r->df.fs != nullptr : r->df.f != nullptr;
+        default: return scalar ? r->i32.fs != nullptr : r->i32.f != nullptr;
+    }
+}
+
+struct UnaryOpt {
+    UnaryFn f;
+    bool checked, flagged;
+};
+void iter_unary(LP* lp) {
+    UnaryOpt* o = (UnaryOpt*)lp->opt_ptr;
+    IA a1, a2;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    int* flag = o->checked ? cumo_cuda_runtime_error_flag_new() : NULL;
+    o->f(&a1, &a2, &ix, flag);
+    if (flag && cumo_cuda_runtime_error_flag_get(flag)) o->flagged = true;
+}
+
+void iter_math(LP* lp) {
+    IA a1, a2;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    ((MathFn)lp->opt_ptr)(&a1, &a2, &ix);
+}
+
+struct Math2Opt {
+    const Math2Row* row;
+    int type;
+    bool scalar;
+    double sv;
+    int left;
+};
+void iter_math2(LP* lp) {
+    Math2Opt* o = (Math2Opt*)lp->opt_ptr;
+    IA a1, a2, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    if (o->scalar) {
+        cumo_hip_make_iarray(lp, 1, &a3);
+        if (o->type == CUMO_HIP_SFLOAT) o->row->sfs(&a1, &a3, &ix, (float)o->sv, o->left);
+        else o->row->dfs(&a1, &a3, &ix, o->sv, o->left);
+    } else {
+        cumo_hip_make_iarray(lp, 1, &a2);
+        cumo_hip_make_iarray(lp, 2, &a3);
+        if (o->type == CUMO_HIP_SFLOAT) o->row->sf(&a1, &a2, &a3, &ix);
+        else o->row->df(&a1, &a2, &a3, &ix);
+    }
+}
+
+struct CondOpt {
+    const CondRow* row;
+    int type;
+    bool scalar;
+    double sv;
+    int left;
+};
+void iter_cond(LP* lp) {
+    CondOpt* o = (CondOpt*)lp->opt_ptr;
+    IA a1, a2;
+    BIA a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    if (o->scalar) {
+        cumo_hip_make_bit_iarray(lp, 1, &a3);
+        switch (o->type) {
+            case CUMO_HIP_SFLOAT: o->row->sf.fs(&a1, (float)o->sv, &a3, &ix, o->left); break;
+            case CUMO_HIP_DFLOAT: o->row->df.fs(&a1, o->sv, &a3, &ix, o->left); break;
+            default: o->row->i32.fs(&a1, (int32_t)o->sv, &a3, &ix, o->left); break;
+        }
+    } else {
+        cumo_hip_make_iarray(lp, 1, &a2);
+        cumo_hip_make_bit_iarray(lp, 2, &a3);
+        switch (o->type) {
+            case CUMO_HIP_SFLOAT: o->row->sf.f(&a1, &a2, &a3, &ix); break;
+            case CUMO_HIP_DFLOAT: o->row->df.f(&a1, &a2, &a3, &ix); break;
+            default: o->row->i32.f(&a1, &a2, &a3, &ix); break;
+        }
+    }
+}
+bool cond_has(const CondRow* r, int type) {
+    switch (type) {
+        case CUMO_HIP_SFLOAT: return r->sf.f != nullptr;
+        case CUMO_HIP_DFLOAT: return r->df.f != nullptr;
+        default: return r->i32.f != nullptr;
+    }
+}
+
+void iter_cond_unary(LP* lp) {
+    IA a1;
+    BIA a2;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_bit_iarray(lp, 1, &a2);
+    ((CondUnaryFn)lp->opt_ptr)(&a1, &a2, &ix);
+}
+
+void iter_store_bit(LP* lp) {  // args: dst (number), src (Bit)  (gen/tmpl/store_bit.c)
+    cumo_na_iarray_stridx_t a1;
+    BSX a2;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray_stridx(lp, 0, &a1);
+    cumo_hip_make_bit_iarray_stridx(lp, 1, &a2);
+    ((StoreBitFn)lp->opt_ptr)(&a1, &a2, &ix);
+}
+
+void iter_copy_bytes(LP* lp) {  // args: src, dst  (narray/data.c:84-92)
+    IA a1, a2;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    cumo_iter_copy_bytes_indexer_kernel_launch(&a1, &a2, &ix, lp->args[0].elmsz);
+}
+
+struct FillOpt {
+    double value;
+};
+void iter_fill(LP* lp) {
+    IA a1;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    double v = ((FillOpt*)lp->opt_ptr)->value;
+    switch (lp->args[0].type) {
+        case CUMO_HIP_SFLOAT: cumo_iter_sfloat_fill_kernel_launch(&a1, &ix, (float)v); break;
+        case CUMO_HIP_DFLOAT: cumo_iter_dfloat_fill_kernel_launch(&a1, &ix, v); break;
+        default: cumo_iter_int32_fill_kernel_launch(&a1, &ix, (int32_t)v); break;
+    }
+}
+
+struct ReduceOpt {
+    ReduceFn f;
+    ReducePairFn fp;
+};
+void iter_reduce(LP* lp) {  // gen/tmpl/accum.c:41-45, minmax.c
+    ReduceOpt* o = (ReduceOpt*)lp->opt_ptr;
+    cumo_na_reduction_arg_t arg;
+    cumo_hip_make_reduction_arg(lp, &arg);
+    if (o->fp) {
+        IA out2;
+        std::memset(&out2, 0, sizeof(out2));
+        out2.ptr = lp->args[2].ptr;
+        for (int d = 0; d < lp->ndim - lp->reduce_dim; d++) out2.step[d] = lp->args[2].step[d];
+        o->fp(&arg, &out2);
+    } else {
+        o->f(&arg);
+    }
+}
+
+// The flat bit run [pos, pos + n) with step 1 can go to the word kernels.
+bool flat_bits(const LP* lp) {
+    if (lp->ndim != 1) return false;
+    for (int j = 0; j < lp->narg; j++)
+        if (lp->args[j].step[0] != 1) return false;
+    return true;
+}
+inline CUMO_BIT_DIGIT* word_ptr(const cumo_hip_loop_args_t& a) { return (CUMO_BIT_DIGIT*)a.ptr + a.bitpos / 32; }
+
+void iter_bit_binary(LP* lp) {  // gen/tmpl_bit/binary.c:17-60
+    const BitBinaryRow* r = (const BitBinaryRow*)lp->opt_ptr;
+    if (flat_bits(lp)) {
+        r->fc(word_ptr(lp->args[0]), lp->args[0].bitpos % 32, word_ptr(lp->args[1]), lp->args[1].bitpos % 32,
+              word_ptr(lp->args[2]), lp->args[2].bitpos % 32, lp->n[0]);
+        return;
+    }
+    BSX a1, a2, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_bit_iarray_stridx(lp, 0, &a1);
+    cumo_hip_make_bit_iarray_stridx(lp, 1, &a2);
+    cumo_hip_make_bit_iarray_stridx(lp, 2, &a3);
+    r->f(&a1, &a2, &a3, &ix);
+}
+
+void iter_bit_unary(LP* lp) {  // gen/tmpl_bit/unary.c
+    const BitUnaryRow* r = (const BitUnaryRow*)lp->opt_ptr;
+    if (flat_bits(lp)) {
+        r->fc(word_ptr(lp->args[0]), lp->args[0].bitpos % 32, word_ptr(lp->args[1]), lp->args[1].bitpos % 32, lp->n[0]);
+        return;
+    }
+    BSX a1, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_bit_iarray_stridx(lp, 0, &a1);
+    cumo_hip_make_bit_iarray_stridx(lp, 1, &a3);
+    r->f(&a1, &a3, &ix);
+}
+
+// count_true / count_false: the innermost loop dimension is one launch, the
+// outer ones are walked here (gen/tmpl_bit/bit_count.c:9-36 under the
+// host-walked loop of ndloop.c:1569-1613).
+struct CountOpt {
+    bool count_false;
+};
+void count_walk(const LP* lp, int level, size_t pos, char* optr, bool count_false) {
+    const cumo_hip_loop_args_t& in = lp->args[0];
+    const cumo_hip_loop_args_t& out = lp->args[1];
+    if (level == lp->ndim - 1) {
+        const ssize_t s1 = in.step[level], s2 = out.step[level];
+        CUMO_BIT_DIGIT* a = (CUMO_BIT_DIGIT*)in.ptr;
+        size_t p = pos;
+        if (s1 >= 0) {  // CUMO_INIT_PTR_BIT_IDX rebases the word pointer (template.h:41-62)
+            a += pos / 32;
+            p = pos % 32;
+        }
+        const uint64_t n = lp->n[level];
+        if (s2 == 0) {
+            if (count_false) cumo_iter_bit_count_false_stride_kernel_launch(p, optr, a, s1, n);
+            else cumo_iter_bit_count_true_stride_kernel_launch(p, optr, a, s1, n);
+        } else {
+            if (count_false) cumo_iter_bit_count_false_stride_stride_kernel_launch(p, optr, a, s1, s2, n);
+            else cumo_iter_bit_count_true_stride_stride_kernel_launch(p, optr, a, s1, s2, n);
+        }
+        return;
+    }
+    for (size_t i = 0; i < lp->n[level]; i++)
+        count_walk(lp, level + 1, pos + (size_t)((ssize_t)i * in.step[level]), optr + (ssize_t)i * out.step[level], count_false);
+}
+void iter_bit_count(LP* lp) { count_walk(lp, 0, lp->args[0].bitpos, lp->args[1].ptr, ((CountOpt*)lp->opt_ptr)->count_false); }
+
+int check_arith(const NA* x) {
+    int rc = check_view(x, "operand");
+    if (rc) return rc;
+    if (!is_arith(x->type)) return fail(CUMO_HIP_ERROR_TYPE, "operand is not SFloat, DFloat or Int32");
+    return CUMO_HIP_OK;
+}
+
+unsigned all_dims(const NA* x) { return x->ndim ? ((1u << x->ndim) - 1u) : 0u; }
+
+}  // namespace
+
+extern "C" {
+
+int cumo_hip_na_binary(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    const BinaryRow* row = find_row(kBinary, op);
+    const int up = upcast(x->type, y->type);
+    if (!row || !binary_has(row, up, false)) return no_method(op);
+    NA tx, ty;
+    const NA *ux, *uy;
+    rc = cast_operand(x, up, &tx, &ux);
+    if (!rc) rc = cast_operand(y, up, &ty, &uy);
+    else ty.ptr = NULL;
+    if (!rc) {
+        BinaryOpt opt = {row, up, false, 0.0, 0, up == CUMO_HIP_INT32 && (!std::strcmp(op, "div") || !std::strcmp(op, "mod")), false};
+        cumo_hip_ndfunc_t nf = {iter_binary, 0, 2, 1, {up, 0}};
+        const NA* in[2] = {ux, uy};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+        if (!rc && opt.flagged) rc = CUMO_HIP_ERROR_ZERO_DIVISION;
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    if (rc == CUMO_HIP_ERROR_ZERO_DIVISION) return fail(rc, "error in NArray operation");
+    return rc;
+}
+
+int cumo_hip_na_binary_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    const BinaryRow* row = find_row(kBinary, op);
+    if (!row || !binary_has(row, x->type, true)) return no_method(op);
+    BinaryOpt opt = {row, x->type, true, sv, scalar_is_left ? 1 : 0,
+                     x->type == CUMO_HIP_INT32 && (!std::strcmp(op, "div") || !std::strcmp(op, "mod")), false};
+    cumo_hip_ndfunc_t nf = {iter_binary, 0, 1, 1, {x->type, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    if (!rc && opt.flagged) return fail(CUMO_HIP_ERROR_ZERO_DIVISION, "error in NArray operation");
+    return rc;
+}
+
+int cumo_hip_na_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    const UnaryRow* row = find_row(kUnary, op);
+    if (!row || !row->f[x->type]) return no_method(op);
+    const bool is_abs = !std::strcmp(op, "abs");
+    UnaryOpt opt = {row->f[x->type], x->type == CUMO_HIP_INT32 && (is_abs || !std::strcmp(op, "reciprocal")), false};
+    cumo_hip_ndfunc_t nf = {iter_unary, 0, 1, 1, {x->type, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    if (!rc && opt.flagged)
+        return is_abs ? fail(CUMO_HIP_ERROR_VALUE, "error in NArray operation") : fail(CUMO_HIP_ERROR_ZERO_DIVISION, "error in NArray operation");
+    return rc;
+}
+
+int cumo_hip_na_math(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    const MathRow* row = find_row(kMath, op);
+    if (!row) return no_method(op);
+    // an Int32 argument is computed in DFloat (narray/math.c:60-110 picks the math module by upcast)
+    const int type = is_float(x->type) ? x->type : CUMO_HIP_DFLOAT;
+    NA tx;
+    const NA* ux;
+    rc = cast_operand(x, type, &tx, &ux);
+    if (!rc) {
+        cumo_hip_ndfunc_t nf = {iter_math, 0, 1, 1, {type, 0}};
+        const NA* in[1] = {ux};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, (void*)row->f[type]);
+    }
+    free_tmp(&tx);
+    return rc;
+}
+
+int cumo_hip_na_math2(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    const Math2Row* row = find_row(kMath2, op);
+    if (!row) return no_method(op);
+    int up = upcast(x->type, y->type);
+    if (!is_float(up)) up = CUMO_HIP_DFLOAT;
+    NA tx, ty;
+    const NA *ux, *uy;
+    rc = cast_operand(x, up, &tx, &ux);
+    if (!rc) rc = cast_operand(y, up, &ty, &uy);
+    else ty.ptr = NULL;
+    if (!rc) {
+        Math2Opt opt = {row, up, false, 0.0, 0};
+        cumo_hip_ndfunc_t nf = {iter_math2, 0, 2, 1, {up, 0}};
+        const NA* in[2] = {ux, uy};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    return rc;
+}
+
+int cumo_hip_na_math2_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    const Math2Row* row = find_row(kMath2, op);
+    if (!row) return no_method(op);
+    const int type = is_float(x->type) ? x->type : CUMO_HIP_DFLOAT;
+    NA tx;
+    const NA* ux;
+    rc = cast_operand(x, type, &tx, &ux);
+    if (!rc) {
+        Math2Opt opt = {row, type, true, sv, scalar_is_left ? 1 : 0};
+        cumo_hip_ndfunc_t nf = {iter_math2, 0, 1, 1, {type, 0}};
+        const NA* in[1] = {ux};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    }
+    free_tmp(&tx);
+    return rc;
+}
+
+int cumo_hip_na_compare(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    const CondRow* row = find_row(kCond, op);
+    const int up = upcast(x->type, y->type);
+    if (!row || !cond_has(row, up)) return no_method(op);
+    NA tx, ty;
+    const NA *ux, *uy;
+    rc = cast_operand(x, up, &tx, &ux);
+    if (!rc) rc = cast_operand(y, up, &ty, &uy);
+    else ty.ptr = NULL;
+    if (!rc) {
+        CondOpt opt = {row, up, false, 0.0, 0};
+        cumo_hip_ndfunc_t nf = {iter_cond, 0, 2, 1, {CUMO_HIP_BIT, 0}};
+        const NA* in[2] = {ux, uy};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    return rc;
+}
+
+int cumo_hip_na_compare_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    const CondRow* row = find_row(kCond, op);
+    if (!row || !cond_has(row, x->type)) return no_method(op);
+    CondOpt opt = {row, x->type, true, sv, scalar_is_left ? 1 : 0};
+    cumo_hip_ndfunc_t nf = {iter_cond, 0, 1, 1, {CUMO_HIP_BIT, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+}
+
+int cumo_hip_na_cond_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    const CondUnaryRow* row = find_row(kCondUnary, op);
+    if (!row || !is_float(x->type)) return no_method(op);
+    cumo_hip_ndfunc_t nf = {iter_cond_unary, 0, 1, 1, {CUMO_HIP_BIT, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, (void*)row->f[x->type]);
+}
+
+int cumo_hip_na_store(cumo_hip_narray_t* dst, const cumo_hip_narray_t* src) {
+    int rc = check_view(dst, "destination");
+    if (!rc) rc = check_view(src, "source");
+    if (rc) return rc;
+    if (!dst->ptr && total_of(dst)) return fail(CUMO_HIP_ERROR_ARGUMENT, "store: destination has no memory");
+    cumo_hip_ndfunc_t nf = {NULL, 0, 2, 0, {0, 0}};
+    void* opt = NULL;
+    StoreOpt sopt;
+    if (dst->type == CUMO_HIP_BIT) {
+        if (src->type != CUMO_HIP_BIT) return fail(CUMO_HIP_ERROR_TYPE, "store: only Bit can be stored into Bit on this path");
+        const BitUnaryRow* row = find_row(kBitUnary, "copy");
+        nf.func = iter_bit_unary;  // args: src, dst
+        opt = (void*)row;
+    } else if (!is_arith(dst->type)) {
+        return fail(CUMO_HIP_ERROR_TYPE, "store: destination must be SFloat, DFloat, Int32 or Bit");
+    } else if (src->type == CUMO_HIP_BIT) {
+        nf.func = iter_store_bit;
+        opt = (void*)kStoreBit[dst->type];
+    } else if (src->type <= CUMO_HIP_INT64) {
+        nf.func = iter_store;
+        sopt.f = kStore[dst->type][src->type];
+        opt = &sopt;
+    } else {
+        return fail(CUMO_HIP_ERROR_TYPE, "store: unsupported source type");
+    }
+    // the loop must have the destination's shape: the source may repeat, the destination may not
+    cumo_hip_loop_t lp;
+    const NA* in[2] = {dst, src};
+    if (nf.func == iter_bit_unary) {
+        in[0] = src;
+        in[1] = dst;
+    }
+    rc = cumo_hip_na_ndloop_prepare(&nf, in, NULL, 0, &lp);
+    if (rc) return rc;
+    size_t total = 1, dtotal = total_of(dst);
+    for (int d = 0; d < lp.ndim; d++) total *= lp.n[d];
+    if (total != dtotal || src->ndim > dst->ndim) return fail(CUMO_HIP_ERROR_SHAPE, "store: source cannot be broadcast to the destination");
+    if (total == 0) return CUMO_HIP_OK;
+    lp.opt_ptr = opt;
+    nf.func(&lp);
+    return lp.status;
+}
+
+int cumo_hip_na_copy(const cumo_hip_narray_t* src, cumo_hip_narray_t* dst) {
+    int rc = check_view(src, "source");
+    if (rc) return rc;
+    const NA* in[1] = {src};
+    NA* out[1] = {dst};
+    if (src->type == CUMO_HIP_BIT) {
+        cumo_hip_ndfunc_t nf = {iter_bit_unary, 0, 1, 1, {CUMO_HIP_BIT, 0}};
+        return cumo_hip_na_ndloop(&nf, in, out, 0, (void*)find_row(kBitUnary, "copy"));
+    }
+    cumo_hip_ndfunc_t nf = {iter_copy_bytes, 0, 1, 1, {src->type, 0}};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, NULL);
+}
+
+int cumo_hip_na_fill(cumo_hip_narray_t* dst, double value) {
+    int rc = check_arith(dst);
+    if (rc) return rc;
+    FillOpt opt = {value};
+    cumo_hip_ndfunc_t nf = {iter_fill, 0, 1, 0, {0, 0}};
+    const NA* in[1] = {dst};
+    return cumo_hip_na_ndloop(&nf, in, NULL, 0, &opt);
+}
+
+int cumo_hip_na_reduce(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, int nan,
+                       cumo_hip_narray_t* z, cumo_hip_narray_t* z2) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    if (!op) return no_method(op);
+    // narray/narray.c:1704-1716
+    if (total_of(x) == 0) return fail(CUMO_HIP_ERROR_SHAPE, "cannot reduce empty NArray");
+    if (x->ndim < 32 && (reduce >> x->ndim)) return fail(CUMO_HIP_ERROR_DIMENSION, "dimension is out of range");
+    if (!reduce) reduce = all_dims(x);
+    const bool use_nan = nan && is_float(x->type);
+    const unsigned flag = CUMO_HIP_NDF_FLAT_REDUCE | (keepdims ? CUMO_HIP_NDF_KEEP_DIM : 0u);
+    ReduceOpt opt = {nullptr, nullptr};
+    int out_type = x->type;
+    const NA* src = x;
+    NA tmp;
+    tmp.ptr = NULL;
+    int nout = 1;
+
+    if (!std::strcmp(op, "minmax")) {
+        opt.fp = use_nan ? kMinmaxNan[x->type] : kMinmax[x->type];
+        if (!opt.fp || !z2) return no_method(op);
+        nout = 2;
+    } else if (const ArgRow* arow = find_row(kArg, op)) {
+        // an Int64 answer only when Int32 cannot hold every index (gen/tmpl/accum_arg.c:92-110)
+        const bool wide = total_of(x) > 0xffffffffull;
+        out_type = wide ? CUMO_HIP_INT64 : CUMO_HIP_INT32;
+        opt.f = use_nan ? (wide ? arow->f64_nan : arow->f32_nan)[x->type] : (wide ? arow->f64 : arow->f32)[x->type];
+        if (!opt.f) return no_method(op);
+        if (arow->memory_index && !is_contiguous(x)) {
+            // the answer counts along the view's own row-major order: work on a
+            // contiguous copy (gen/tmpl/accum_index.c:118-126)
+            rc = cumo_hip_na_copy(x, &tmp);
+            if (rc) return rc;
+            src = &tmp;
+        }
+    } else if (const ReduceRow* row = find_row(kReduce, op)) {
+        opt.f = use_nan ? row->f_nan[x->type] : row->f[x->type];
+        if (!opt.f) return no_method(op);
+        if (row->result == 1 && x->type == CUMO_HIP_INT32) out_type = CUMO_HIP_INT64;  // gen/spec.rb:308-319
+    } else {
+        return no_method(op);
+    }
+    cumo_hip_ndfunc_t nf = {iter_reduce, flag, 1, nout, {out_type, out_type}};
+    const NA* in[1] = {src};
+    NA* out[2] = {z, z2};
+    rc = cumo_hip_na_ndloop(&nf, in, out, reduce, &opt);
+    free_tmp(&tmp);
+    return rc;
+}
+
+int cumo_hip_na_bit_binary(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {
+    int rc = check_view(x, "operand");
+    if (!rc) rc = check_view(y, "operand");
+    if (rc) return rc;
+    const BitBinaryRow* row = find_row(kBitBinary, op);
+    if (!row || x->type != CUMO_HIP_BIT || y->type != CUMO_HIP_BIT) return no_method(op);
+    cumo_hip_ndfunc_t nf = {iter_bit_binary, 0, 2, 1, {CUMO_HIP_BIT, 0}};
+    const NA* in[2] = {x, y};
+    NA* out[1] = {z};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, (void*)row);
+}
+
+int cumo_hip_na_bit_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
+    int rc = check_view(x, "operand");
+    if (rc) return rc;
+    const BitUnaryRow* row = find_row(kBitUnary, op);
+    if (!row || x->type != CUMO_HIP_BIT) return no_method(op);
+    cumo_hip_ndfunc_t nf = {iter_bit_unary, 0, 1, 1, {CUMO_HIP_BIT, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, (void*)row);
+}
+
+int cumo_hip_na_bit_count(const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, int count_false, cumo_hip_narray_t* z) {
+    int rc = check_view(x, "operand");
+    if (rc) return rc;
+    if (x->type != CUMO_HIP_BIT) return no_method(count_false ? "count_false" : "count_true");
+    if (x->ndim < 32 && (reduce >> x->ndim)) return fail(CUMO_HIP_ERROR_DIMENSION, "dimension is out of range");
+    if (!reduce) reduce = all_dims(x);
+    const unsigned flag = CUMO_HIP_NDF_FLAT_REDUCE | (keepdims ? CUMO_HIP_NDF_KEEP_DIM : 0u);
+    cumo_hip_ndfunc_t nf = {iter_bit_count, flag, 1, 1, {CUMO_HIP_UINT64, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    if (z && z->ptr && !is_contiguous(z)) return fail(CUMO_HIP_ERROR_ARGUMENT, "bit count: the result array must be contiguous");
+    cumo_hip_loop_t lp;
+    rc = cumo_hip_na_ndloop_prepare(&nf, in, out, reduce, &lp);
+    if (rc) return rc;
+    // the launchers add onto the result: start from 0 (ndloop.c:853-860)
+    size_t zbytes = total_of(z) * 8;
+    if (zbytes) cumo_hip_memset(z->ptr + z->offset, 0, zbytes);
+    if (total_of(x) == 0) return CUMO_HIP_OK;
+    CountOpt opt = {count_false != 0};
+    lp.opt_ptr = &opt;
+    iter_bit_count(&lp);
+    return lp.status;
+}
+
+}  // extern "C"

@@ -8,8 +8,9 @@
  * extension can link this library in place of its own kernel translation
  * units. The second half (`cumo_hip_*`) is what this library adds: the error
  * hook that stands in for the extension's raise, stream selection, the memory
- * pool's C interface, the launch planner's introspection calls and the host
- * launch layer (ndloop) that builds the descriptors from array views.
+ * pool's C interface and the launch planner's introspection calls. The host
+ * launch layer (ndloop) that builds the descriptors from array views is
+ * declared in cumo_hip_ndloop.h.
  */
 #ifndef CUMO_HIP_H
 #define CUMO_HIP_H
@@ -315,7 +316,13 @@ enum {
     CUMO_HIP_OK = 0,
     CUMO_HIP_ERROR_RUNTIME = 1,        /* Cumo::CUDA::RuntimeError */
     CUMO_HIP_ERROR_OUT_OF_MEMORY = 2,  /* Cumo::CUDA::OutOfMemoryError */
-    CUMO_HIP_ERROR_ARGUMENT = 3        /* ArgumentError / ShapeError raised by the host layer */
+    CUMO_HIP_ERROR_ARGUMENT = 3,       /* ArgumentError */
+    /* raised by the host launch layer (cumo_hip_ndloop.h) */
+    CUMO_HIP_ERROR_SHAPE = 4,          /* Cumo::NArray::ShapeError (narray/ndloop.c:508-512, narray/narray.c:1704-1716) */
+    CUMO_HIP_ERROR_ZERO_DIVISION = 5,  /* ZeroDivisionError (narray/gen/tmpl/binary.c:120-126) */
+    CUMO_HIP_ERROR_TYPE = 6,           /* TypeError / NoMethodError: no such operation for this element type */
+    CUMO_HIP_ERROR_VALUE = 7,          /* Cumo::NArray::ValueError (narray/gen/tmpl/unary2.c:61-66) */
+    CUMO_HIP_ERROR_DIMENSION = 8       /* Cumo::NArray::DimensionError (narray/narray.c:1757-1759) */
 };
 typedef void (*cumo_hip_error_handler_t)(int kind, int hip_status, const char* message);
 void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler);

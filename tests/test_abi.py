@@ -1,6 +1,6 @@
 """The drop-in boundary, checked without a GPU: descriptor layouts match the
 reference's structs byte for byte, the library loads, and every symbol that
-include/cumo_hip.h declares is exported."""
+the headers under include/ declare is exported."""
 import ctypes as C
 import os
 import re
@@ -9,7 +9,7 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "cumo_hip.h")
+HEADERS = sorted(os.path.join(ROOT, "include", n) for n in os.listdir(os.path.join(ROOT, "include")) if n.endswith(".h"))
 
 
 def test_descriptor_layouts():
@@ -47,8 +47,10 @@ def test_header_layouts_compile_to_the_same_numbers(tmp_path):
 
 def declared_symbols():
     """Function names in the preprocessed header."""
-    txt = subprocess.run(["gcc", "-E", "-P", "-I", os.path.join(ROOT, "include"), HEADER], check=True, stdout=subprocess.PIPE, text=True).stdout
-    names = set(re.findall(r"\b(cumo_[a-z0-9_]+)\s*\(", txt))
+    names = set()
+    for header in HEADERS:
+        txt = subprocess.run(["gcc", "-E", "-P", "-I", os.path.join(ROOT, "include"), header], check=True, stdout=subprocess.PIPE, text=True).stdout
+        names |= set(re.findall(r"\b(cumo_[a-z0-9_]+)\s*\(", txt))
     names.discard("cumo_hip_error_handler_t")
     return sorted(names)
 

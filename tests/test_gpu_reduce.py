@@ -192,11 +192,15 @@ def test_int32_reductions():
 
 def test_empty_and_degenerate():
     import cumo_amd
-    a = cumo_amd.SFloat.zeros(0, 5)
-    assert a.sum(axis=0).to_numpy().tolist() == [0.0] * 5   # reducing an empty axis leaves the identity... and
-    assert cumo_amd.SFloat.zeros(4, 0).sum(axis=0).shape == (0,)
+    # reference: narray/narray.c:1704-1716 -- "cannot reduce empty NArray", whatever the axis
+    for empty in (cumo_amd.SFloat.zeros(0, 5), cumo_amd.SFloat.zeros(4, 0), cumo_amd.SFloat.zeros(0)):
+        for op in ("sum", "max", "argmax", "mean"):
+            with pytest.raises(cumo_amd.ShapeError):
+                getattr(empty, op)(axis=0)
     with pytest.raises(ValueError):
-        cumo_amd.SFloat.zeros(0).max()
+        cumo_amd.SFloat.zeros(3, 4).sum(axis=2)   # DimensionError: dimension is out of range
+    one0 = cumo_amd.DFloat.cast(np.array(2.5))    # a 0-dimensional array reduces to itself
+    assert float(one0.sum()) == 2.5 and int(one0.argmax()) == 0
     one = cumo_amd.DFloat.cast(np.array([[3.5]]))
     assert float(one.sum()) == 3.5 and float(one.max(axis=0).to_numpy()[0]) == 3.5
     assert int(one.argmax()) == 0
