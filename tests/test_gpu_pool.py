@@ -1,0 +1,91 @@
+"""The memory pool over real device memory (the host-heap tests cover the
+bookkeeping): blocks come from hipMalloc, are reused without a device call,
+reuse is ordered by the stream, and the out-of-memory path raises what the
+reference raises (ext/cumo/cuda/memory_pool.cpp:64-96,
+test/cuda/memory_pool_test.rb:16-72)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def clean_pool():
+    import cumo_amd
+    cumo_amd.synchronize()
+    cumo_amd.MemoryPool.free_all_blocks()
+    yield
+    from cumo_amd import _lib
+    _lib.lib.cumo_hip_pool_set_limit(0)
+    cumo_amd.MemoryPool.free_all_blocks()
+
+
+def test_reuse_without_device_call_and_counters():
+    import cumo_amd
+    from cumo_amd import _lib
+    L = _lib.lib
+    base_used = L.cumo_hip_pool_used_bytes()
+    a = cumo_amd.SFloat.new(1000)                 # 4000 bytes -> 4096
+    assert L.cumo_hip_pool_used_bytes() - base_used == 4096
+    p = a._buf.ptr
+    calls = L.cumo_hip_pool_device_malloc_calls()
+    del a
+    assert L.cumo_hip_pool_used_bytes() == base_used and L.cumo_hip_pool_free_bytes() >= 4096
+    b = cumo_amd.SFloat.new(1024)
+    assert b._buf.ptr == p and L.cumo_hip_pool_device_malloc_calls() == calls
+    del b
+    cumo_amd.MemoryPool.free_all_blocks()
+    assert L.cumo_hip_pool_total_bytes() == base_used
+
+
+def test_stream_ordered_reuse_keeps_results_right():
+    import cumo_amd
+    n = 1 << 22
+    x = cumo_amd.SFloat.cast(np.arange(n, dtype=np.float32))
+    ptrs = set()
+    for k in range(20):
+        t = x + float(k)          # result block
+        u = t * 2.0               # second block; t is released right after the launch that reads it
+        ptrs.add(t._buf.ptr)
+        del t
+        got = u.to_numpy()
+        assert got[12345] == np.float32((12345 + k) * 2.0) and got[-1] == np.float32((n - 1 + k) * 2.0)
+        del u
+    assert len(ptrs) <= 2, "blocks are expected to be reused"
+
+
+def test_out_of_memory_raises_like_the_reference():
+    import cumo_amd
+    from cumo_amd import _lib
+    L = _lib.lib
+    L.cumo_hip_pool_set_limit(L.cumo_hip_pool_total_bytes() + (1 << 20))
+    with pytest.raises(cumo_amd.OutOfMemoryError) as ei:
+        cumo_amd.SFloat.new(1 << 20)              # 4 MiB over a 1 MiB allowance
+    assert "out of memory to allocate 4194304 bytes" in str(ei.value)
+    small = cumo_amd.SFloat.new(1 << 10)          # still serviceable
+    assert small._buf.ptr
+    # the failure inside a launch-layer call leaves nothing allocated behind
+    used = L.cumo_hip_pool_used_bytes()
+    x = cumo_amd.SFloat.new(1 << 17)              # 512 KiB fits
+    with pytest.raises(cumo_amd.OutOfMemoryError):
+        x + x + x                                  # needs two more 512 KiB blocks at once; the allowance holds one
+    del x
+    assert L.cumo_hip_pool_used_bytes() == used
+
+
+def test_pool_disabled_goes_straight_to_the_device():
+    import cumo_amd
+    from cumo_amd import _lib
+    L = _lib.lib
+    assert cumo_amd.MemoryPool.enabled()
+    cumo_amd.MemoryPool.disable()
+    try:
+        total = L.cumo_hip_pool_total_bytes()
+        a = cumo_amd.DFloat.cast(np.ones(1000))
+        assert L.cumo_hip_pool_total_bytes() == total
+        assert float((a + a).sum()) == 2000.0
+        del a
+    finally:
+        cumo_amd.MemoryPool.enable()
