@@ -57,13 +57,33 @@ template <> __device__ __forceinline__ int32_t spread<int32_t>(int32_t hi, int32
         _Pragma("unroll") for (int k = 0; k < N; ++k) accumulate(x[k], idx0 + k, acc);            \
     }
 
+// The hardware's max/min: of a number and a quiet NaN the number is kept. One
+// instruction each; the C library's fmax/fmin cost three here, because the
+// compiler quiets both operands first. A signalling NaN comes out as a NaN, which
+// the callers treat as "look at this block element by element".
 template <class T> __device__ __forceinline__ T max_skipping_nan(T a, T b);
-template <> __device__ __forceinline__ float max_skipping_nan<float>(float a, float b) { return __builtin_fmaxf(a, b); }
-template <> __device__ __forceinline__ double max_skipping_nan<double>(double a, double b) { return __builtin_fmax(a, b); }
+template <> __device__ __forceinline__ float max_skipping_nan<float>(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+template <> __device__ __forceinline__ double max_skipping_nan<double>(double a, double b) {
+    double r;
+    asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 template <> __device__ __forceinline__ int32_t max_skipping_nan<int32_t>(int32_t a, int32_t b) { return a > b ? a : b; }
 template <class T> __device__ __forceinline__ T min_skipping_nan(T a, T b);
-template <> __device__ __forceinline__ float min_skipping_nan<float>(float a, float b) { return __builtin_fminf(a, b); }
-template <> __device__ __forceinline__ double min_skipping_nan<double>(double a, double b) { return __builtin_fmin(a, b); }
+template <> __device__ __forceinline__ float min_skipping_nan<float>(float a, float b) {
+    float r;
+    asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+template <> __device__ __forceinline__ double min_skipping_nan<double>(double a, double b) {
+    double r;
+    asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 template <> __device__ __forceinline__ int32_t min_skipping_nan<int32_t>(int32_t a, int32_t b) { return a < b ? a : b; }
 
 // true if any of the N values is a NaN (a sum is NaN then; inf - inf also trips
@@ -274,21 +294,29 @@ struct ArgImpl {
         T m = x[0];
 #pragma unroll
         for (int k = 1; k < N; ++k) m = IS_MAX ? max_skipping_nan<T>(m, x[k]) : min_skipping_nan<T>(m, x[k]);
-        bool look = IS_MAX ? (m > acc.value) : (m < acc.value);
-        look = look || acc.index == INT64_MAX;
-        if (is_float_t<T>::value) {
-            if (NAN_WINS) {
+        if (is_float_t<T>::value && !NAN_WINS) {
+            // One ordered comparison settles the common case. It is false, and the
+            // block gets looked at, when the block's extreme is better, when the
+            // accumulator holds nothing but NaN so far, and when m came out a NaN.
+            if (IS_MAX ? (m <= acc.value) : (m >= acc.value)) return;
+            if (isnan_t(m)) {  // all NaN, or a signalling NaN poisoned m: exact rule, element by element
+#pragma unroll
+                for (int k = 0; k < N; ++k) accumulate(x[k], idx0 + k, acc);
+                return;
+            }
+        } else {
+            bool look = IS_MAX ? (m > acc.value) : (m < acc.value);
+            look = look || acc.index == INT64_MAX;
+            if (is_float_t<T>::value) {  // NAN_WINS
                 if (isnan_t(acc.value)) return;  // an earlier NaN already won
                 if (maybe_nan<T, N>(x)) {         // rare: let the exact rule sort it out
 #pragma unroll
                     for (int k = 0; k < N; ++k) accumulate(x[k], idx0 + k, acc);
                     return;
                 }
-            } else {
-                look = look || isnan_t(acc.value);  // nothing but NaN so far
             }
+            if (!look) return;
         }
-        if (!look) return;
         // first position holding the extreme; if every element is a NaN, m is one and
         // nothing compares equal, which leaves the block's first element
         // (the value is taken from that position too: of +0 and -0 the earlier counts)
@@ -302,11 +330,66 @@ struct ArgImpl {
         }
         combine(Acc{v, idx0 + first}, acc);
     }
+    // U blocks of N at once (all later than what the accumulator holds): when no
+    // element of any of them can change the accumulator, one comparison says so.
+    static constexpr bool GROUPED = true;
+    template <int U, int N>
+    __device__ __forceinline__ void accumulate_group(const T (&x)[U][N], const int64_t (&idx)[U], Acc& acc) const {
+        if (!is_float_t<T>::value || !NAN_WINS) {
+            T m = x[0][0];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int k = 0; k < N; ++k) m = IS_MAX ? max_skipping_nan<T>(m, x[u][k]) : min_skipping_nan<T>(m, x[u][k]);
+            }
+            // false for a NaN on either side, which sends the blocks down the exact path
+            if (IS_MAX ? (m <= acc.value) : (m >= acc.value)) {
+                if (is_float_t<T>::value || acc.index != INT64_MAX) return;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) accumulate_n<N>(x[u], idx[u], acc);
+    }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
         if (out_mode == 0) *reinterpret_cast<T*>(out) = acc.value;
         else if (out_mode == 4) *reinterpret_cast<int32_t*>(out) = (int32_t)acc.index;
         else *reinterpret_cast<int64_t*>(out) = acc.index;
     }
+};
+
+// ---- min / max, value only ---------------------------------------------------------
+// The answer of min/max is a value, and an index is needed for it in one case only:
+// when the extreme is a zero and zeros of both signs may be present, Numo's
+// sequential loop keeps the one that came first (real_accum.h:217-278). So the
+// fold keeps just the value, with the library's NaN-skipping max/min, and where it
+// ends on a zero the kernels fold that output once more with the exact rule.
+// An output that is all NaN stays NaN.
+template <class T, bool IS_MAX>
+struct ValueExtremeImpl {
+    typedef T In;
+    typedef T Acc;
+    typedef ArgImpl<T, IS_MAX, false> Exact;
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 1;
+    static constexpr bool HAS_EXACT = is_float_t<T>::value;
+    static __device__ __forceinline__ float pick(float a, float b) { return IS_MAX ? __builtin_fmaxf(a, b) : __builtin_fminf(a, b); }
+    static __device__ __forceinline__ double pick(double a, double b) { return IS_MAX ? __builtin_fmax(a, b) : __builtin_fmin(a, b); }
+    static __device__ __forceinline__ int32_t pick(int32_t a, int32_t b) { return IS_MAX ? (a > b ? a : b) : (a < b ? a : b); }
+    __device__ __forceinline__ Acc identity() const {
+        if (is_float_t<T>::value) return Lim<T>::skip();
+        return IS_MAX ? Lim<T>::lowest() : Lim<T>::highest();
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { acc = pick(acc, next); }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const { acc = pick(acc, x); }
+    template <int N>
+    __device__ __forceinline__ void accumulate_n(const T (&x)[N], int64_t, Acc& acc) const {
+#pragma unroll
+        for (int k = 0; k < N; ++k) acc = pick(acc, x[k]);
+    }
+    __device__ __forceinline__ bool needs_exact(const Acc& acc) const { return acc == (T)0; }
+    __host__ __device__ __forceinline__ Exact exact() const { return Exact{0}; }
+    __device__ __forceinline__ Acc from_exact(const typename Exact::Acc& e) const { return e.value; }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const { *reinterpret_cast<T*>(out) = acc; }
 };
 
 // ---- minmax / ptp ------------------------------------------------------------------

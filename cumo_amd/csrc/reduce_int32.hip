@@ -12,8 +12,8 @@ typedef int32_t T;
 
 CUMO_RED(sum) { reduce_launch(arg, nullptr, SumImpl<T, int64_t, false, false>{0}, 0); }
 CUMO_RED(prod) { reduce_launch(arg, nullptr, SumImpl<T, int64_t, true, false>{0}, 0); }
-CUMO_RED(min) { reduce_launch(arg, nullptr, ArgImpl<T, false, false>{0}, 1); }
-CUMO_RED(max) { reduce_launch(arg, nullptr, ArgImpl<T, true, false>{0}, 1); }
+CUMO_RED(min) { reduce_launch(arg, nullptr, ValueExtremeImpl<T, false>{}, 1); }
+CUMO_RED(max) { reduce_launch(arg, nullptr, ValueExtremeImpl<T, true>{}, 1); }
 CUMO_RED(ptp) { reduce_launch(arg, nullptr, MinMaxImpl<T, false>{1}, 1); }
 CUMO_RED(argmin_int32) { reduce_launch(arg, nullptr, ArgImpl<T, false, false>{4}, 1); }
 CUMO_RED(argmin_int64) { reduce_launch(arg, nullptr, ArgImpl<T, false, false>{8}, 1); }

@@ -32,6 +32,9 @@
 //   void combine(const Acc& next, Acc& acc) const          -- merge two accumulators; must not depend on the order
 //                                                             in which accumulators arrive
 //   void store(const Acc& acc, char* out, char* out2) const
+// Optional: GROUPED + accumulate_group<U,N> (several blocks offered at once);
+// HAS_EXACT + Exact/exact()/needs_exact()/from_exact() (a cheap fold with an exact
+// second fold of the same elements where the cheap one cannot decide).
 #ifndef CUMO_HIP_REDUCE_KERNELS_H
 #define CUMO_HIP_REDUCE_KERNELS_H
 
@@ -75,6 +78,16 @@ __device__ __forceinline__ T shfl_down_any(const T& v, unsigned delta) {
     return b.t;
 }
 
+// Impls whose fast fold leaves a question only an exact fold can answer declare
+// HAS_EXACT = true, a type Exact (an Impl over the same In), exact(),
+// needs_exact(acc) and from_exact(exact_acc).
+template <class I, class = void> struct has_exact { static constexpr bool value = false; };
+template <class I> struct has_exact<I, decltype((void)I::HAS_EXACT)> { static constexpr bool value = I::HAS_EXACT; };
+
+// Impls that can take several blocks at once declare GROUPED and accumulate_group.
+template <class I, class = void> struct has_group { static constexpr bool value = false; };
+template <class I> struct has_group<I, decltype((void)I::GROUPED)> { static constexpr bool value = true; };
+
 template <class T, int N>
 struct alignas((sizeof(T) * N) > 16 ? 16 : (sizeof(T) * N)) RedVec {
     T v[N];
@@ -106,20 +119,93 @@ __device__ __forceinline__ int64_t red_decompose(uint64_t i, int nd, const uint6
     return off;
 }
 
-template <class Impl, int VEC, bool PARTIAL>
-__global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
+// One output's share of the reduce axis, [begin, end), folded by the 2^tpr_bits
+// lanes that share the output. The result is complete in the group's first lane
+// (thread 0 of the block when a whole block shares the output). Every lane of the
+// wave must call it; lanes whose group has no output pass ok == false.
+template <class Impl, int VEC>
+__device__ __forceinline__ typename Impl::Acc red_row_scan(const RedKParams& p, const Impl& impl, bool ok, const char* base,
+                                                           int64_t in_off, uint64_t begin, uint64_t end) {
     typedef typename Impl::In In;
     typedef typename Impl::Acc Acc;
     __shared__ Acc wave_acc[kRedBlock / 64];
+    const unsigned TPR = 1u << p.tpr_bits;
+    const unsigned lane_r = threadIdx.x & (TPR - 1);
+    const int64_t rstep = p.in_red_step[p.red_ndim > 0 ? p.red_ndim - 1 : 0];
+    const uint64_t stride = (uint64_t)TPR * VEC;
 
+    Acc acc = impl.identity();
+    if (ok) {
+        for (uint64_t i0 = begin + (uint64_t)lane_r * VEC; i0 < end; i0 += stride * kRedUnroll) {
+            In x[kRedUnroll][VEC];
+            int64_t eoff[kRedUnroll];
+#pragma unroll
+            for (int u = 0; u < kRedUnroll; ++u) {
+                const uint64_t i = i0 + (uint64_t)u * stride;
+                if (i < end) {
+                    const int64_t off = (p.red_ndim <= 1) ? (int64_t)i * rstep
+                                                          : red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
+                    eoff[u] = in_off + off;
+                    if constexpr (VEC > 1) {
+                        const RedVec<In, VEC> v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
+                    } else {
+                        x[u][0] = *reinterpret_cast<const In*>(base + off);
+                    }
+                }
+            }
+            if constexpr (has_group<Impl>::value) {
+                if (i0 + (uint64_t)(kRedUnroll - 1) * stride < end) {
+                    // every access of the unrolled step is inside the row: offer them together
+                    int64_t idx[kRedUnroll];
+#pragma unroll
+                    for (int u = 0; u < kRedUnroll; ++u)
+                        idx[u] = (p.index_mode == 2) ? (eoff[u] / (int64_t)sizeof(In)) : (int64_t)(i0 + (uint64_t)u * stride);
+                    impl.template accumulate_group<kRedUnroll, VEC>(x, idx, acc);
+                    continue;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kRedUnroll; ++u) {
+                const uint64_t i = i0 + (uint64_t)u * stride;
+                if (i < end) {
+                    // the VEC elements of one access are consecutive along the axis
+                    int64_t idx = 0;
+                    if (Impl::USES_INDEX) idx = (p.index_mode == 2) ? (eoff[u] / (int64_t)sizeof(In)) : (int64_t)i;
+                    impl.template accumulate_n<VEC>(x[u], idx, acc);
+                }
+            }
+        }
+    }
+    // lanes of one output combine; lane 0 of the group ends up with everything,
+    // later lanes folded into earlier ones in a fixed order
+    const unsigned wave_span = TPR < 64 ? TPR : 64;
+    for (unsigned d = wave_span >> 1; d > 0; d >>= 1) {
+        const Acc other = shfl_down_any(acc, d);
+        impl.combine(other, acc);
+    }
+    if (TPR > 64) {
+        const unsigned wave = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0) wave_acc[wave] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (unsigned w = 1; w < kRedBlock / 64; ++w) impl.combine(wave_acc[w], acc);
+        }
+        __syncthreads();
+    }
+    return acc;
+}
+
+template <class Impl, int VEC, bool PARTIAL>
+__global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
+    typedef typename Impl::Acc Acc;
     const unsigned TPR = 1u << p.tpr_bits;
     const unsigned RPB = kRedBlock >> p.tpr_bits;
     const unsigned lane_r = threadIdx.x & (TPR - 1);
     const unsigned row_in_block = threadIdx.x >> p.tpr_bits;
     const uint64_t n_rows = p.out_total * p.n_split;
     const uint64_t n_blocks = (n_rows + RPB - 1) / RPB;
-    const int64_t rstep = p.in_red_step[p.red_ndim > 0 ? p.red_ndim - 1 : 0];
-    const uint64_t stride = (uint64_t)TPR * VEC;
 
     for (uint64_t rb = blockIdx.x; rb < n_blocks; rb += gridDim.x) {
         const uint64_t vrow = rb * RPB + row_in_block;
@@ -133,59 +219,39 @@ __global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl i
                 i_split = vrow - i_out * p.n_split;
             }
         }
-        Acc acc = impl.identity();
+        uint64_t begin = 0, end = 0;
+        int64_t in_off = 0;
         if (ok) {
-            const uint64_t begin = i_split * p.chunk;
-            uint64_t end = begin + p.chunk;
+            begin = i_split * p.chunk;
+            end = begin + p.chunk;
             if (end > p.red_total) end = p.red_total;
-            const int64_t in_off = red_decompose(i_out, p.out_ndim, p.out_shape, p.in_out_step, p.small);
-            const char* base = p.in + in_off;
-            for (uint64_t i0 = begin + (uint64_t)lane_r * VEC; i0 < end; i0 += stride * kRedUnroll) {
-                In x[kRedUnroll][VEC];
-                int64_t eoff[kRedUnroll];
-#pragma unroll
-                for (int u = 0; u < kRedUnroll; ++u) {
-                    const uint64_t i = i0 + (uint64_t)u * stride;
-                    if (i < end) {
-                        const int64_t off = (p.red_ndim <= 1) ? (int64_t)i * rstep
-                                                              : red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
-                        eoff[u] = in_off + off;
-                        if constexpr (VEC > 1) {
-                            const RedVec<In, VEC> v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
-#pragma unroll
-                            for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
-                        } else {
-                            x[u][0] = *reinterpret_cast<const In*>(base + off);
-                        }
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < kRedUnroll; ++u) {
-                    const uint64_t i = i0 + (uint64_t)u * stride;
-                    if (i < end) {
-                        // the VEC elements of one access are consecutive along the axis
-                        int64_t idx = 0;
-                        if (Impl::USES_INDEX) idx = (p.index_mode == 2) ? (eoff[u] / (int64_t)sizeof(In)) : (int64_t)i;
-                        impl.template accumulate_n<VEC>(x[u], idx, acc);
-                    }
-                }
-            }
+            in_off = red_decompose(i_out, p.out_ndim, p.out_shape, p.in_out_step, p.small);
         }
-        // lanes of one output combine; lane 0 of the group ends up with everything,
-        // later lanes folded into earlier ones in a fixed order
-        const unsigned wave_span = TPR < 64 ? TPR : 64;
-        for (unsigned d = wave_span >> 1; d > 0; d >>= 1) {
-            const Acc other = shfl_down_any(acc, d);
-            impl.combine(other, acc);
-        }
-        if (TPR > 64) {
-            const unsigned wave = threadIdx.x >> 6;
-            if ((threadIdx.x & 63) == 0) wave_acc[wave] = acc;
-            __syncthreads();
-            if (threadIdx.x == 0) {
-                for (unsigned w = 1; w < kRedBlock / 64; ++w) impl.combine(wave_acc[w], acc);
+        const char* base = p.in + in_off;
+        Acc acc = red_row_scan<Impl, VEC>(p, impl, ok, base, in_off, begin, end);
+
+        if constexpr (has_exact<Impl>::value) {
+            // The fast fold cannot tell which of two equal-valued elements came first.
+            // Where that matters for the answer (the impl says so), the lanes of the
+            // output fold their share again with the exact rule. The verdict comes
+            // from the group's first lane, so the whole group takes the same way.
+            __shared__ int s_need;
+            bool need;
+            if (TPR > 64) {
+                if (threadIdx.x == 0) s_need = impl.needs_exact(acc) ? 1 : 0;
+                __syncthreads();
+                need = s_need != 0;
+                __syncthreads();
+            } else {
+                const int mine = impl.needs_exact(acc) ? 1 : 0;
+                need = __shfl(mine, (int)((threadIdx.x & 63u) & ~(TPR - 1))) != 0;
             }
-            __syncthreads();
+            if (need) {
+                typedef typename Impl::Exact Exact;
+                const Exact ex = impl.exact();
+                const typename Exact::Acc eacc = red_row_scan<Exact, VEC>(p, ex, ok, base, in_off, begin, end);
+                acc = impl.from_exact(eacc);
+            }
         }
         if (ok && lane_r == 0) {
             if (PARTIAL) {
@@ -266,6 +332,23 @@ __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl i
                             impl.accumulate(x[u][j], idx, acc[j]);
                         }
                     }
+                }
+            }
+        }
+        if constexpr (has_exact<Impl>::value) {
+            // this thread walked the axis in order, but its fast fold may still have lost
+            // which of two equal elements came first: walk that output again, exactly
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if (impl.needs_exact(acc[j])) {
+                    typedef typename Impl::Exact Exact;
+                    const Exact ex = impl.exact();
+                    typename Exact::Acc e = ex.identity();
+                    for (uint64_t i = begin; i < end; ++i) {
+                        const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
+                        ex.accumulate(*reinterpret_cast<const In*>(base + off + (int64_t)j * ostep_in), (int64_t)i, e);
+                    }
+                    acc[j] = impl.from_exact(e);
                 }
             }
         }
@@ -434,9 +517,16 @@ static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     if (kp.n_split > 1024) tpr = 256;
     k2.tpr_bits = 0;
     while ((1 << k2.tpr_bits) < tpr) ++k2.tpr_bits;
-    CombineImpl<Impl> cimpl;
-    cimpl.impl = impl;
-    red_launch_row<CombineImpl<Impl>, false, true>(k2, 1, cimpl, nullptr, stream);
+    if constexpr (has_exact<Impl>::value) {
+        // the partials are plain values in axis order: fold them with the exact rule
+        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
+        k2.index_mode = 1;
+        red_launch_row<typename Impl::Exact, false, true>(k2, 1, impl.exact(), nullptr, stream);
+    } else {
+        CombineImpl<Impl> cimpl;
+        cimpl.impl = impl;
+        red_launch_row<CombineImpl<Impl>, false, true>(k2, 1, cimpl, nullptr, stream);
+    }
     cumo_cuda_runtime_check_kernel_launch();
     cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
 }

@@ -210,3 +210,36 @@ def test_dfloat_kahan_sum():
     import cumo_amd
     h = np.array([1e16, 1.0, -1e16, 1.0] * 1000)
     assert float(cumo_amd.DFloat.cast(h).kahan_sum()) == 2000.0
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("shape,axis", [((300, 77), 1), ((300, 77), 0), ((5, 20000), 1), ((20000, 5), 0), ((3000001,), None),
+                                        ((64, 33, 40), (0, 2)), ((6, 70000), 1), ((2, 3, 4096), 2)])
+def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
+    # Numo's sequential loop only replaces on a strict comparison (real_accum.h:217-278), so of
+    # +0 and -0 the earlier one is the answer. Every output here ends on a zero, with both signs
+    # present at seeded positions, through the row, column, block-wide and split kernels.
+    rng = np.random.default_rng(411)
+    cls = cls_of(tname)
+    sign = rng.integers(0, 2, size=shape).astype(bool)
+    zero = rng.random(shape) < 0.05
+    mag = rng.random(shape).astype(dt) + dt(0.5)
+    for name, away in (("max", -1.0), ("min", 1.0)):
+        h = (mag * dt(away)).astype(dt)
+        h[zero] = 0.0
+        h[zero & sign] = -0.0
+        d = cls.cast(h)
+        want = oracle.reduce(name, h, axis=axis)
+        got = getattr(d, name)(axis=axis).to_numpy()
+        assert_bits_equal(got, want, "%s %r axis %r" % (name, shape, axis))
+        if want.size >= 100:
+            zeros = want[want == 0]
+            assert np.signbit(zeros).any() and not np.signbit(zeros).all(), "the inputs are meant to produce both signs"
+    # NaN in the mix: skipped unless the output holds nothing else
+    h = (mag * dt(-1.0)).astype(dt)
+    h[zero] = np.nan
+    h[..., 0] = np.nan
+    d = cls.cast(h)
+    assert_bits_equal(d.max(axis=axis).to_numpy(), oracle.reduce("max", h, axis=axis), "max with NaN")
+    alln = np.full(shape, np.nan, dtype=dt)
+    assert np.isnan(cls.cast(alln).max(axis=axis).to_numpy()).all()
