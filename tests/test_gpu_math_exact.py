@@ -1,0 +1,61 @@
+"""SFloat exp answers the double-precision exp rounded to float once, which is what
+Numo's host macro computes (types/float_macro.h:84-97), for every input: the
+DFloat launcher followed by the DFloat -> SFloat store is that value, made on the
+device by another route. Against the CPU oracle ((float)exp((double)x) with
+glibc) the bar is <= 1 ulp."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+import numo_oracle as oracle  # noqa: E402
+
+from helpers import assert_bits_equal, assert_ulp  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def exp_both_ways(h):
+    import cumo_amd
+    x = cumo_amd.SFloat.cast(h)
+    fast = cumo_amd.NMath.exp(x).to_numpy()
+    wide = cumo_amd.SFloat.cast(cumo_amd.NMath.exp(cumo_amd.DFloat.cast(x))).to_numpy()
+    return fast, wide
+
+
+def test_exp_equals_the_double_exp_rounded_once_everywhere():
+    rng = np.random.default_rng(99)
+    parts = [
+        rng.uniform(-104, 89, size=1 << 22),               # the whole range with finite, non-zero answers
+        rng.uniform(-20, 5, size=1 << 22),                 # where softmax inputs live
+        rng.standard_normal(1 << 21) * 1e-3,               # around 1
+        np.array([0.0, -0.0, 87.0, -87.0, 87.000001, -87.000001, 88.72283, 88.72284, 89.0, -87.33655, -103.97, -103.98,
+                  -110.0, 1e-45, -1e-45, np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5, 1e-8]),
+    ]
+    h = np.concatenate(parts).astype(np.float32)
+    fast, wide = exp_both_ways(h)
+    assert_bits_equal(fast, wide, "SFloat exp vs DFloat exp rounded once")
+    assert_ulp(fast, oracle.unary("exp", h), 1, "SFloat exp vs the CPU oracle")
+
+
+def test_exp_every_exponent_and_dense_bit_patterns():
+    # every 1021st float bit pattern in [-87.5, 88.8]: all binades, all mantissa phases
+    b = np.arange(0, 1 << 32, 1021, dtype=np.uint64).astype(np.uint32)
+    h = b.view(np.float32)
+    h = h[np.isfinite(h) & (h > -105) & (h < 90)]
+    fast, wide = exp_both_ways(h)
+    assert_bits_equal(fast, wide, "SFloat exp vs DFloat exp rounded once")
+
+
+def test_exp_on_strided_and_transposed_views():
+    import cumo_amd
+    rng = np.random.default_rng(100)
+    h = rng.uniform(-30, 30, size=(130, 257)).astype(np.float32)
+    d = cumo_amd.SFloat.cast(h)
+    for hv, dv in ((h.T, d.transpose()), (h[::3, 1::2], d[::3, 1::2]), (h.T[:, ::2], d.transpose()[:, ::2])):
+        got = cumo_amd.NMath.exp(dv).to_numpy()
+        wide = cumo_amd.SFloat.cast(cumo_amd.NMath.exp(cumo_amd.DFloat.cast(dv))).to_numpy()
+        assert_bits_equal(got, wide)
+        assert_ulp(got, oracle.unary("exp", np.ascontiguousarray(hv)), 1)
