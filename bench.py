@@ -34,10 +34,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the C2 broadcast add, from two rocprofv3 --pmc runs of this
 # file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by the same
-# counter's reading for --pmc-calibration's plain 256 MiB copy (FETCH_SIZE x 1.9992,
-# WRITE_SIZE x 1.0000): 131294 KiB fetched + 131072 KiB written. The figures and
-# the commands are in profiles/ew_rows_add_f64_c2_hbm_traffic.txt.
-C2_ADD_TRAFFIC_BYTES = 268662587
+# counter's reading for --pmc-calibration's plain 256 MiB copy (FETCH_SIZE x 1.9998,
+# WRITE_SIZE x 0.9997): 131128 KiB fetched + 131030 KiB written. The figures and
+# the commands are in profiles/ew_rows2_add_f64_c2_hbm_traffic.txt.
+C2_ADD_TRAFFIC_BYTES = 268450055
 METRIC = "achieved HBM GB/s (% of MI355X peak) and GElem/s vs Numo CPU, per config"
 MIB = 1 << 20
 
@@ -336,7 +336,7 @@ def main():
     avg_ms = sum(ts) / len(ts)
     achieved = add_bytes / (avg_ms * 1e-3) / 1e9
     roofline = {
-        "bound": "hbm", "kernel": "ew_rows_kernel<OpAdd<double>, 2> (C = A + r, f64 4096x4096 + 1x4096)",
+        "bound": "hbm", "kernel": "ew_rows2_kernel<OpAdd<double>, 2, false> (C = A + r, f64 4096x4096 + 1x4096)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
         "bytes_per_launch": int(add_bytes), "avg_launch_ms": round(avg_ms, 5), "median_launch_ms": round(ts[len(ts) // 2], 5),
         "traffic": C2_ADD_TRAFFIC_BYTES,
@@ -347,7 +347,7 @@ def main():
     if args.pmc_calibration:
         src = cumo_amd.SFloat.zeros(1 << 26)
         for _ in range(5):
-            dst = src.copy()  # ew_rows_kernel<OpCast<unsigned int, unsigned int>, 4>: reads 256 MiB, writes 256 MiB
+            dst = src.copy()  # ew_flat_kernel<OpCast<unsigned int, unsigned int>, 4, true>: reads 256 MiB, writes 256 MiB
         cumo_amd.synchronize()
         del src, dst
         cumo_amd.MemoryPool.free_all_blocks()
