@@ -73,34 +73,76 @@ CUMO_HIP_FUN(OpRound, round((double)x))
 CUMO_HIP_FUN(OpCeil, ceil((double)x))
 CUMO_HIP_FUN(OpTrunc, trunc((double)x))
 CUMO_HIP_FUN(OpRint, rint((double)x))
-// NMath (reference list: narray/gen/spec.rb:427-457)
+// NMath (reference list: narray/gen/spec.rb:427-457). HEAVY: many instructions per element.
+#define CUMO_HIP_FUN_H(NAME, EXPR) \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true; \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const { z = (T)(EXPR); return true; } };
 CUMO_HIP_FUN(OpSqrt, sqrt((double)x))
-CUMO_HIP_FUN(OpCbrt, cbrt((double)x))
-CUMO_HIP_FUN(OpLog, log((double)x))
-CUMO_HIP_FUN(OpLog2, log2((double)x))
-CUMO_HIP_FUN(OpLog10, log10((double)x))
-CUMO_HIP_FUN(OpExp, exp((double)x))
-CUMO_HIP_FUN(OpExp2, exp2((double)x))
-CUMO_HIP_FUN(OpExp10, exp10((double)x))
-CUMO_HIP_FUN(OpSin, sin((double)x))
-CUMO_HIP_FUN(OpCos, cos((double)x))
-CUMO_HIP_FUN(OpTan, tan((double)x))
-CUMO_HIP_FUN(OpAsin, asin((double)x))
-CUMO_HIP_FUN(OpAcos, acos((double)x))
-CUMO_HIP_FUN(OpAtan, atan((double)x))
-CUMO_HIP_FUN(OpSinh, sinh((double)x))
-CUMO_HIP_FUN(OpCosh, cosh((double)x))
-CUMO_HIP_FUN(OpTanh, tanh((double)x))
-CUMO_HIP_FUN(OpAsinh, asinh((double)x))
-CUMO_HIP_FUN(OpAcosh, acosh((double)x))
-CUMO_HIP_FUN(OpAtanh, atanh((double)x))
+CUMO_HIP_FUN_H(OpCbrt, cbrt((double)x))
+CUMO_HIP_FUN_H(OpLog, log((double)x))
+CUMO_HIP_FUN_H(OpLog2, log2((double)x))
+CUMO_HIP_FUN_H(OpLog10, log10((double)x))
+// SFloat exp: the double-precision exp of the argument, rounded to float once.
+// The argument has 24 significant bits, so k = rint(x / ln 2) times the upper part
+// of ln 2 is exact; exp(r) on |r| <= ln(2)/2 is the Taylor polynomial of degree 13
+// (truncation below 2^-57), scaled by 2^k. Only full-rate instructions besides the
+// two conversions: k is rounded by adding 1.5 * 2^52 (its integer value is then
+// the low word of the sum), and 2^k is applied by adding k to the exponent field,
+// which is safe because the clamp keeps the result a normal double. Outside
+// [-105, 89] the float answer is already 0 or inf. No branch anywhere, so the
+// elements of a vector are evaluated side by side: NaN goes through the clamp
+// (the comparisons are false) and comes back in through xc - xc at the end,
+// which is +0 for every other argument.
+__device__ __forceinline__ float exp_float_rounded_once(float xf) {
+    float xc = (xf < -105.0f) ? -105.0f : xf;
+    xc = (xc > 89.0f) ? 89.0f : xc;
+    const double x = (double)xc;
+    const double big = 6755399441055744.0;  // 1.5 * 2^52
+    const double t = __builtin_fma(x, 1.44269504088896338700e+00, big);
+    const double k = t - big;
+    const int ki = (int)(uint32_t)__double_as_longlong(t);
+    double r = __builtin_fma(k, -6.93147180369123816490e-01, x);  // ln 2, upper 32 bits
+    r = __builtin_fma(k, -1.90821492927058770002e-10, r);         // ln 2, the rest
+    const double c[12] = {
+        1.60590438368216133e-10 /* 1/13! */, 2.08767569878681002e-09 /* 1/12! */, 2.50521083854417202e-08 /* 1/11! */,
+        2.75573192239858883e-07 /* 1/10! */, 2.75573192239858925e-06 /* 1/9! */,  2.48015873015873016e-05 /* 1/8! */,
+        1.98412698412698413e-04 /* 1/7! */,  1.38888888888888894e-03 /* 1/6! */,  8.33333333333333322e-03 /* 1/5! */,
+        4.16666666666666644e-02 /* 1/4! */,  1.66666666666666657e-01 /* 1/3! */,  5.00000000000000000e-01 /* 1/2! */};
+    double p = c[0];
+#pragma unroll
+    for (int i = 1; i < 12; ++i) p = __builtin_fma(p, r, c[i]);
+    p = __builtin_fma(p, r, 1.0);
+    p = __builtin_fma(p, r, 1.0);
+    const int hi = __double2hiint(p) + (ki << 20);
+    const float y = (float)__hiloint2double(hi, __double2loint(p));
+    return y + (xc - xc);
+}
+template <class T> struct OpExp { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
+    __device__ __forceinline__ bool operator()(T x, T, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)exp_float_rounded_once((float)x);
+        else z = (T)exp((double)x);
+        return true; } };
+CUMO_HIP_FUN_H(OpExp2, exp2((double)x))
+CUMO_HIP_FUN_H(OpExp10, exp10((double)x))
+CUMO_HIP_FUN_H(OpSin, sin((double)x))
+CUMO_HIP_FUN_H(OpCos, cos((double)x))
+CUMO_HIP_FUN_H(OpTan, tan((double)x))
+CUMO_HIP_FUN_H(OpAsin, asin((double)x))
+CUMO_HIP_FUN_H(OpAcos, acos((double)x))
+CUMO_HIP_FUN_H(OpAtan, atan((double)x))
+CUMO_HIP_FUN_H(OpSinh, sinh((double)x))
+CUMO_HIP_FUN_H(OpCosh, cosh((double)x))
+CUMO_HIP_FUN_H(OpTanh, tanh((double)x))
+CUMO_HIP_FUN_H(OpAsinh, asinh((double)x))
+CUMO_HIP_FUN_H(OpAcosh, acosh((double)x))
+CUMO_HIP_FUN_H(OpAtanh, atanh((double)x))
 // the host macro guards x == 0 (types/float_macro.h:113); the reference's device
 // macro does not and answers NaN there, which Numo does not
-CUMO_HIP_FUN(OpSinc, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
-CUMO_HIP_FUN(OpErf, erf((double)x))
-CUMO_HIP_FUN(OpErfc, erfc((double)x))
-CUMO_HIP_FUN(OpLog1p, log1p((double)x))
-CUMO_HIP_FUN(OpExpm1, expm1((double)x))
+CUMO_HIP_FUN_H(OpSinc, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
+CUMO_HIP_FUN_H(OpErf, erf((double)x))
+CUMO_HIP_FUN_H(OpErfc, erfc((double)x))
+CUMO_HIP_FUN_H(OpLog1p, log1p((double)x))
+CUMO_HIP_FUN_H(OpExpm1, expm1((double)x))
 
 #define CUMO_HIP_IUN(NAME, EXPR) \
     struct NAME { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false) \
