@@ -480,6 +480,83 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
 }
 
 // ---------------------------------------------------------------------------
+// Flat kernel for a Bit result: every input is one contiguous run (or the scalar)
+// and the result's first bit is the first bit of a 128-bit unit. The 32/VEC lanes
+// of a group take four consecutive words: per step each lane loads one vector, the
+// group's word is gathered in its first lane with DPP row shifts, and the first
+// lane stores the four words as one access. Nothing between the four loads of a
+// lane depends on data, so they go out back to back. Only the run's last group can
+// be ragged; it sets or clears its bits one by one.
+// ---------------------------------------------------------------------------
+template <class Op, int VEC, bool NT>
+__global__ __launch_bounds__(kEwBlock) void ew_flat_bit_kernel(const char* __restrict__ px, const char* __restrict__ py,
+                                                               CUMO_BIT_DIGIT* __restrict__ pz, uint64_t n, int use_scalar, Op op,
+                                                               typename Op::S sv) {
+    typedef typename Op::A A;
+    typedef typename Op::B B;
+    constexpr int NIN = Op::NIN;
+    constexpr bool TWO = (NIN == 2);
+    constexpr int UNR = 4;
+    constexpr unsigned G = 32 / VEC;
+    const uint64_t lane = (uint64_t)blockIdx.x * kEwBlock + threadIdx.x;
+    const uint64_t group = lane / G;
+    const unsigned k = (unsigned)(lane % G);
+    const uint64_t first = group * (32 * UNR);  // the group's first element
+    if (first >= n) return;
+    const bool two_arrays = TWO && use_scalar == 0;
+    const uint64_t e0 = first + (uint64_t)k * VEC;
+    if (first + 32 * UNR <= n) {
+        A xv[UNR][VEC];
+        B yv[UNR][VEC];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            if (NIN >= 1) raw_load<A, VEC, NT>(px + (e0 + 32 * u) * sizeof(A), xv[u]);
+            if (two_arrays) raw_load<B, VEC, NT>(py + (e0 + 32 * u) * sizeof(B), yv[u]);
+        }
+        uint32_t words[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            uint32_t bits = 0;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                A x = (NIN >= 1) ? xv[u][j] : A();
+                B y = B();
+                if (TWO) {
+                    if (use_scalar == 0) y = yv[u][j];
+                    else if (use_scalar == 1) y = (B)sv;
+                    else { y = (B)x; x = (A)sv; }
+                }
+                uint32_t z = 0;
+                op(x, y, z);
+                bits |= (z ? 1u : 0u) << j;
+            }
+            words[u] = ew_gather_word<VEC>(bits);
+        }
+        if (k == 0) *reinterpret_cast<u32x4*>(pz + group * UNR) = u32x4{words[0], words[1], words[2], words[3]};
+        return;
+    }
+    // the ragged end: at most 32 * UNR - 1 elements in the whole launch
+    for (int u = 0; u < UNR; ++u) {
+        for (int j = 0; j < VEC; ++j) {
+            const uint64_t e = e0 + 32 * u + j;
+            if (e >= n) continue;
+            A x = (NIN >= 1) ? reinterpret_cast<const A*>(px)[e] : A();
+            B y = B();
+            if (TWO) {
+                if (use_scalar == 0) y = reinterpret_cast<const B*>(py)[e];
+                else if (use_scalar == 1) y = (B)sv;
+                else { y = (B)x; x = (A)sv; }
+            }
+            uint32_t z = 0;
+            op(x, y, z);
+            const uint32_t bit = 1u << (e & 31);
+            if (z) atomicOr(&pz[e >> 5], bit);
+            else atomicAnd(&pz[e >> 5], ~bit);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Two-dimensional kernel for typed results: rows x inner, every operand either
 // walks the inner dimension contiguously or is constant along it (a column
 // vector, or the scalar), and may repeat along rows (a row vector). 32-bit
@@ -1078,6 +1155,33 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         if (force1) vec = 1;
     }
     const dim3 b(kEwBlock);
+
+    // A Bit result over flat inputs, starting on a 128-bit unit: the lean Bit kernel
+    // (measured on 2^25 SFloat > scalar: see the notes at the kernel).
+    if constexpr (Op::BIT_OUT) {
+        constexpr int VB = 16 / (int)sizeof(A);
+        bool flat = n == 1 && vec == VB && (Op::NIN < 2 || sizeof(B) == sizeof(A)) && plan.step[nops - 1][0] == 1 &&
+                    (out_bit->pos % 128) == 0 && ((uintptr_t)out_bit->ptr % 16) == 0;
+        for (int o = 0; o + 1 < nops && flat; ++o) {
+            const int sl = slot[o];
+            const int64_t es = sl == 0 ? (int64_t)sizeof(A) : (int64_t)sizeof(B);
+            flat = plan.step[o][0] == es;
+        }
+        if constexpr (VB == 4 || VB == 2) {
+            const uint64_t groups = (kp.inner + 127) / 128;
+            const uint64_t blocks = (groups * (32 / VB) + kEwBlock - 1) / kEwBlock;
+            if (flat && blocks <= ew_grid_max()) {
+                const int mode = ew_nt_mode();
+                const bool nt = mode < 0 ? kp.inner * sizeof(A) * (uint64_t)(nops - 1) > kEwNtBytes : mode != 0;
+                CUMO_BIT_DIGIT* dst = reinterpret_cast<CUMO_BIT_DIGIT*>(const_cast<char*>(ops[nops - 1].ptr)) + out_bit->pos / 32;
+                const dim3 g((unsigned)blocks);
+                if (nt) hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], dst, kp.inner, use_scalar, op, sv);
+                else hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], dst, kp.inner, use_scalar, op, sv);
+                cumo_cuda_runtime_check_kernel_launch();
+                return;
+            }
+        }
+    }
 
     // Typed results through 128-bit accesses have two lean kernels: one access per
     // lane, one 4 KiB tile per block, 32-bit index arithmetic. Measured on 1 GiB

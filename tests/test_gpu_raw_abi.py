@@ -168,6 +168,62 @@ def test_compare_into_bits_at_a_bit_offset():
     free(px, pw, pc)
 
 
+@pytest.mark.parametrize("pos", [0, 128, 256 + 128, 96, 5])
+@pytest.mark.parametrize("n", [1, 127, 128, 129, 255, 1000, 128 * 300, 128 * 300 + 77])
+def test_flat_compare_into_bits_positions_and_ragged_ends(pos, n):
+    """One contiguous run compared into a Bit run that starts on a 128-bit unit (the
+    lean kernel) or anywhere else (the general one): every bit before and after the
+    run must keep its value, whichever kernel stores the ragged last words."""
+    from cumo_amd import _lib
+    rng = np.random.default_rng(1000 + pos + n)
+    x = rng.integers(-3, 4, size=n).astype(np.float32)
+    y = rng.integers(-3, 4, size=n).astype(np.float32)
+    x[rng.integers(0, n)] = np.nan
+    px, py = dev(x), dev(y)
+    nwords = (pos + n + 31) // 32 + 8
+    for fillv in (0xFFFFFFFF, 0):
+        pw = dev(np.full(nwords, fillv, dtype=np.uint32))
+        a1, a2 = iarray(px, (4,)), iarray(py, (4,))
+        a3 = _lib.BitIArray()
+        a3.ptr, a3.pos = pw, pos
+        a3.step[0] = 1
+        ix = indexer((n,))
+        f = _lib.fn("cumo_iter_sfloat_le_kernel_launch", None, [P(_lib.IArray), P(_lib.IArray), P(_lib.BitIArray), P(_lib.Indexer)])
+        _lib.call(f, C.byref(a1), C.byref(a2), C.byref(a3), C.byref(ix))
+        bits = np.unpackbits(fetch(pw, (nwords,), np.uint32).view(np.uint8), bitorder="little")
+        want = np.full(nwords * 32, 1 if fillv else 0, dtype=np.uint8)
+        with np.errstate(invalid="ignore"):
+            want[pos:pos + n] = x <= y
+        assert (bits == want).all(), (pos, n, fillv, "array <= array")
+        # scalar on the left: 1 > x
+        fs = _lib.fn("cumo_iter_sfloat_gt_s_kernel_launch", None,
+                     [P(_lib.IArray), C.c_float, P(_lib.BitIArray), P(_lib.Indexer), C.c_int])
+        _lib.call(fs, C.byref(a1), C.c_float(1.0), C.byref(a3), C.byref(ix), 1)
+        bits = np.unpackbits(fetch(pw, (nwords,), np.uint32).view(np.uint8), bitorder="little")
+        with np.errstate(invalid="ignore"):
+            want[pos:pos + n] = np.float32(1.0) > x
+        assert (bits == want).all(), (pos, n, fillv, "scalar > array")
+        free(pw)
+    # DFloat: two elements per lane, sixteen lanes per word
+    xd = x.astype(np.float64)
+    pd = dev(xd)
+    pw = dev(np.full(nwords, 0xFFFFFFFF, dtype=np.uint32))
+    a1 = iarray(pd, (8,))
+    a3 = _lib.BitIArray()
+    a3.ptr, a3.pos = pw, pos
+    a3.step[0] = 1
+    ix = indexer((n,))
+    fd = _lib.fn("cumo_iter_dfloat_lt_s_kernel_launch", None,
+                 [P(_lib.IArray), C.c_double, P(_lib.BitIArray), P(_lib.Indexer), C.c_int])
+    _lib.call(fd, C.byref(a1), C.c_double(0.5), C.byref(a3), C.byref(ix), 0)
+    bits = np.unpackbits(fetch(pw, (nwords,), np.uint32).view(np.uint8), bitorder="little")
+    want = np.ones(nwords * 32, dtype=np.uint8)
+    with np.errstate(invalid="ignore"):
+        want[pos:pos + n] = xd < 0.5
+    assert (bits == want).all(), (pos, n, "dfloat")
+    free(px, py, pd, pw)
+
+
 def test_int32_divide_by_zero_sets_the_pinned_flag_and_skips_the_store():
     from cumo_amd import _lib
     x = np.array([7, 8, 9, 10], dtype=np.int32)
