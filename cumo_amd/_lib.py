@@ -29,6 +29,10 @@ class DimensionError(ValueError):
     """Cumo::NArray::DimensionError (reference: ext/cumo/narray/narray.c:1757-1759)."""
 
 
+class OperationError(ValueError):
+    """Cumo::NArray::OperationError (reference: ext/cumo/narray/gen/tmpl/clip.c:48-51,222)."""
+
+
 class Indexer(C.Structure):
     # reference: ext/cumo/include/cumo/indexer.h:16-22
     _fields_ = [("ndim", C.c_ubyte), ("total_size", C.c_size_t), ("shape", C.c_size_t * MAX_DIM),
@@ -160,6 +164,11 @@ _sig = {
     "cumo_hip_na_binary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_binary_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
     "cumo_hip_na_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_pow": (C.c_int, [P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_pow_s": (C.c_int, [P(NArrayDesc), C.c_double, C.c_int, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_ewcomp": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_clip": (C.c_int, [P(NArrayDesc), C.c_int, C.c_double, P(NArrayDesc), C.c_int, C.c_double, P(NArrayDesc),
+                                   P(NArrayDesc)]),
     "cumo_hip_na_math": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_math2": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_math2_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
@@ -213,6 +222,8 @@ def check():
         raise TypeError(text)
     if kind == 8:
         raise DimensionError(text)
+    if kind == 9:
+        raise OperationError(text)
     raise RuntimeError_(text)
 
 

@@ -164,6 +164,104 @@ struct OpIAbs { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, true)
         z = (x < 0) ? -x : x;
         return true; } };
 
+// ---- pow, maximum/minimum, clip ----------------------------------------------
+// Float ** float: the host macro's pow in double, rounded once
+// (reference: types/float_macro.h m_pow; device types/float_macro_kernel.h:36).
+template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) static constexpr bool HEAVY = true;
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (T)pow((double)x, (double)y); return true; } };
+
+// Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
+// element type for small exponents, pow() beyond 64, the reciprocal for negative ones.
+template <class T>
+__device__ __forceinline__ T pow_float_int(T x, int32_t p) {
+    const bool neg = p < 0;
+    uint32_t q = neg ? (0u - (uint32_t)p) : (uint32_t)p;
+    T r = 1;
+    switch (q) {
+        case 0: r = 1; break;
+        case 1: r = x; break;
+        case 2: r = x * x; break;
+        case 3: r = x * x * x; break;
+        case 4: x = x * x; r = x * x; break;
+        default:
+            if (q > 64) {
+                r = (T)pow((double)x, (double)q);
+            } else {
+                while (q) {
+                    if (q & 1u) r *= x;
+                    x *= x;
+                    q >>= 1;
+                }
+            }
+    }
+    return neg ? (T)1 / r : r;
+}
+template <class T> struct OpPowInt { typedef T A; typedef int32_t B; typedef T R; typedef T S;
+    static constexpr int NIN = 2; static constexpr bool BIT_OUT = false; static constexpr bool CHECKED = false;
+    __device__ __forceinline__ bool operator()(T x, int32_t y, T& z) const { z = pow_float_int<T>(x, y); return true; } };
+// the exponent is one Int32 for the whole launch
+template <class T> struct OpPowIntS { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false)
+    int32_t p;
+    __device__ __forceinline__ bool operator()(T x, T, T& z) const { z = pow_float_int<T>(x, p); return true; } };
+// the base is one number for the whole launch, the exponents are an Int32 array
+template <class T> struct OpPowIntLeft { typedef int32_t A; typedef int32_t B; typedef T R; typedef int32_t S;
+    static constexpr int NIN = 1; static constexpr bool BIT_OUT = false; static constexpr bool CHECKED = false;
+    T base;
+    __device__ __forceinline__ bool operator()(int32_t y, int32_t, T& z) const { z = pow_float_int<T>(base, y); return true; } };
+
+// Int32 ** Int32 (reference: types/int_macro_kernel.h:26-42): wrapping products, 0 for a negative exponent
+__device__ __forceinline__ int32_t pow_int32(int32_t x, int32_t p) {
+    uint32_t ux = (uint32_t)x, r = 1u;
+    switch (p) {
+        case 0: return 1;
+        case 1: return x;
+        case 2: return (int32_t)(ux * ux);
+        case 3: return (int32_t)(ux * ux * ux);
+    }
+    if (p < 0) return 0;
+    uint32_t q = (uint32_t)p;
+    while (q) {
+        if (q & 1u) r *= ux;
+        ux *= ux;
+        q >>= 1;
+    }
+    return (int32_t)r;
+}
+struct OpIPow { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 2, false, false)
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t y, int32_t& z) const { z = pow_int32(x, y); return true; } };
+struct OpIPowS { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false)
+    int32_t p;
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t, int32_t& z) const { z = pow_int32(x, p); return true; } };
+struct OpIPowLeft { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false)
+    int32_t base;
+    __device__ __forceinline__ bool operator()(int32_t y, int32_t, int32_t& z) const { z = pow_int32(base, y); return true; } };
+
+// maximum / minimum of two arrays (reference: types/real_accum_kernel.h:28-70,
+// xint_macro_kernel.h:54-68). The plain form answers the other operand when one
+// is NaN; the _nan form answers the NaN.
+template <class T> struct OpMaximum { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (x >= y) ? x : ((y == y) ? y : x); return true; } };
+template <class T> struct OpMaximumNan { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (x >= y) ? x : ((x != x) ? x : y); return true; } };
+template <class T> struct OpMinimum { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (x <= y) ? x : ((y == y) ? y : x); return true; } };
+template <class T> struct OpMinimumNan { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (x <= y) ? x : ((x != x) ? x : y); return true; } };
+
+// clip against one bound that is an array or the scalar, and against two scalar
+// bounds (reference: narray/gen/tmpl/clip_kernel.cu:7-44)
+template <class T> struct OpClipMin { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T lo, T& z) const { z = (x < lo) ? lo : x; return true; } };
+template <class T> struct OpClipMax { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T hi, T& z) const { z = (x > hi) ? hi : x; return true; } };
+template <class T> struct OpClipS { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false)
+    T lo, hi;
+    __device__ __forceinline__ bool operator()(T x, T, T& z) const {
+        if (x < lo) x = lo;
+        if (x > hi) x = hi;
+        z = x;
+        return true; } };
+
 // ---- comparisons into Bit ---------------------------------------------------
 #define CUMO_HIP_CMP(NAME, EXPR) \
     template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, uint32_t, 2, true, false) \

@@ -802,6 +802,100 @@ void count_walk(const LP* lp, int level, size_t pos, char* optr, bool count_fals
 }
 void iter_bit_count(LP* lp) { count_walk(lp, 0, lp->args[0].bitpos, lp->args[1].ptr, ((CountOpt*)lp->opt_ptr)->count_false); }
 
+
+// ---- pow, maximum/minimum, clip (gen/tmpl/pow.c, ewcomp.c, clip.c) ---------------
+typedef void (*Arr3Fn)(IA*, IA*, IA*, IX*);
+struct PowFns {
+    Arr3Fn pow, pow_int32;
+};
+#define POW_FNS(t) {cumo_iter_##t##_pow_kernel_launch, cumo_iter_##t##_pow_int32_kernel_launch}
+const PowFns kPow[3] = {POW_FNS(sfloat), POW_FNS(dfloat), POW_FNS(int32)};
+
+void iter_arr3(LP* lp) {  // two inputs, one result, no flag
+    IA a1, a2, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    cumo_hip_make_iarray(lp, 2, &a3);
+    ((Arr3Fn)lp->opt_ptr)(&a1, &a2, &a3, &ix);
+}
+
+struct PowSOpt {
+    int type;      // element type of the launcher family
+    int form;      // 0: x ** sv, 1: sv ** x, 2: x ** (Int32)sv, 3: sv ** (Int32 array)x
+    double sv;
+};
+void iter_pow_s(LP* lp) {
+    const PowSOpt* o = (const PowSOpt*)lp->opt_ptr;
+    IA a1, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a3);
+    switch (o->type) {
+        case CUMO_HIP_SFLOAT:
+            if (o->form <= 1) cumo_iter_sfloat_pow_s_kernel_launch(&a1, (float)o->sv, &a3, &ix, o->form);
+            else if (o->form == 2) cumo_iter_sfloat_pow_int32_s_kernel_launch(&a1, (int32_t)o->sv, &a3, &ix);
+            else cumo_iter_sfloat_pow_int32_s_left_kernel_launch((float)o->sv, &a1, &a3, &ix);
+            break;
+        case CUMO_HIP_DFLOAT:
+            if (o->form <= 1) cumo_iter_dfloat_pow_s_kernel_launch(&a1, o->sv, &a3, &ix, o->form);
+            else if (o->form == 2) cumo_iter_dfloat_pow_int32_s_kernel_launch(&a1, (int32_t)o->sv, &a3, &ix);
+            else cumo_iter_dfloat_pow_int32_s_left_kernel_launch(o->sv, &a1, &a3, &ix);
+            break;
+        default:
+            if (o->form <= 1) cumo_iter_int32_pow_s_kernel_launch(&a1, (int32_t)o->sv, &a3, &ix, o->form);
+            else if (o->form == 2) cumo_iter_int32_pow_int32_s_kernel_launch(&a1, (int32_t)o->sv, &a3, &ix);
+            else cumo_iter_int32_pow_int32_s_left_kernel_launch((int32_t)o->sv, &a1, &a3, &ix);
+            break;
+    }
+}
+
+struct EwcompRow {
+    const char* op;
+    Arr3Fn f[3], fnan[3];
+};
+const EwcompRow kEwcomp[] = {
+    {"maximum", {cumo_sfloat_maximum_kernel_launch, cumo_dfloat_maximum_kernel_launch, cumo_int32_maximum_kernel_launch},
+     {cumo_sfloat_maximum_nan_kernel_launch, cumo_dfloat_maximum_nan_kernel_launch, nullptr}},
+    {"minimum", {cumo_sfloat_minimum_kernel_launch, cumo_dfloat_minimum_kernel_launch, cumo_int32_minimum_kernel_launch},
+     {cumo_sfloat_minimum_nan_kernel_launch, cumo_dfloat_minimum_nan_kernel_launch, nullptr}},
+};
+
+struct ClipOpt {
+    int type;
+    int form;      // 0: two scalars, 1: scalar min, 2: scalar max, 3: array min, 4: array max, 5: two arrays
+    double lo, hi;
+    bool flagged;
+};
+void iter_clip(LP* lp) {
+    ClipOpt* o = (ClipOpt*)lp->opt_ptr;
+    IA a[4];
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    for (int j = 0; j < lp->narg; ++j) cumo_hip_make_iarray(lp, j, &a[j]);
+#define CLIP_CASES(t, c)                                                                              \
+    switch (o->form) {                                                                                \
+        case 0: cumo_iter_##t##_clip_s_kernel_launch(&a[0], (c)o->lo, (c)o->hi, &a[1], &ix); break;   \
+        case 1: cumo_iter_##t##_clip_min_s_kernel_launch(&a[0], (c)o->lo, &a[1], &ix); break;         \
+        case 2: cumo_iter_##t##_clip_max_s_kernel_launch(&a[0], (c)o->hi, &a[1], &ix); break;         \
+        case 3: cumo_iter_##t##_clip_min_kernel_launch(&a[0], &a[1], &a[2], &ix); break;              \
+        case 4: cumo_iter_##t##_clip_max_kernel_launch(&a[0], &a[1], &a[2], &ix); break;              \
+        default: {                                                                                    \
+            int* flag = cumo_cuda_runtime_error_flag_new();                                           \
+            cumo_iter_##t##_clip_kernel_launch(&a[0], &a[1], &a[2], &a[3], &ix, flag);                \
+            if (flag && cumo_cuda_runtime_error_flag_get(flag)) o->flagged = true;                    \
+        }                                                                                             \
+    }
+    switch (o->type) {
+        case CUMO_HIP_SFLOAT: CLIP_CASES(sfloat, float) break;
+        case CUMO_HIP_DFLOAT: CLIP_CASES(dfloat, double) break;
+        default: CLIP_CASES(int32, int32_t) break;
+    }
+#undef CLIP_CASES
+}
+
 int check_arith(const NA* x) {
     int rc = check_view(x, "operand");
     if (rc) return rc;
@@ -853,6 +947,155 @@ int cumo_hip_na_binary_s(const char* op, const cumo_hip_narray_t* x, double sv, 
     NA* out[1] = {z};
     rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
     if (!rc && opt.flagged) return fail(CUMO_HIP_ERROR_ZERO_DIVISION, "error in NArray operation");
+    return rc;
+}
+
+// x ** y for two arrays (gen/tmpl/pow.c:117-190,200-215): the result has the higher
+// type of the two; an Int32 exponent array takes the repeated-product form.
+int cumo_hip_na_pow(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    const int up = upcast(x->type, y->type);
+    NA tx, ty;
+    const NA *ux, *uy;
+    ty.ptr = NULL;
+    rc = cast_operand(x, up, &tx, &ux);
+    Arr3Fn f;
+    if (y->type == CUMO_HIP_INT32) {
+        uy = y;
+        f = kPow[up].pow_int32;
+    } else {
+        if (!rc) rc = cast_operand(y, up, &ty, &uy);
+        f = kPow[up].pow;
+    }
+    if (!rc) {
+        cumo_hip_ndfunc_t nf = {iter_arr3, 0, 2, 1, {up, 0}};
+        const NA* in[2] = {ux, uy};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, (void*)f);
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    return rc;
+}
+
+// x ** sv, or sv ** x when scalar_is_left. An integer sv takes the Int32 form as a
+// Ruby Integer does (gen/tmpl/pow.c:160-175); a non-integer base over an Int32 array
+// answers DFloat, the class a Ruby Float upcasts to.
+int cumo_hip_na_pow_s(const cumo_hip_narray_t* x, double sv, int sv_is_integer, int scalar_is_left, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    PowSOpt opt = {x->type, 0, sv};
+    int out_type = x->type;
+    if (!scalar_is_left) {
+        if (sv_is_integer) opt.form = 2;
+        else if (x->type == CUMO_HIP_INT32) return fail(CUMO_HIP_ERROR_TYPE, "Int32 ** Float: cast the array to DFloat first");
+        else opt.form = 0;
+    } else if (x->type == CUMO_HIP_INT32) {
+        opt.form = 3;
+        if (!sv_is_integer) {
+            opt.type = CUMO_HIP_DFLOAT;
+            out_type = CUMO_HIP_DFLOAT;
+        }
+    } else {
+        opt.form = 1;
+    }
+    cumo_hip_ndfunc_t nf = {iter_pow_s, 0, 1, 1, {out_type, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+}
+
+// Cumo::<T>.maximum / minimum (gen/tmpl/ewcomp.c:40-75)
+int cumo_hip_na_ewcomp(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, int nan, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    const EwcompRow* row = find_row(kEwcomp, op);
+    const int up = upcast(x->type, y->type);
+    if (!row) return no_method(op);
+    Arr3Fn f = (nan && is_float(up)) ? row->fnan[up] : row->f[up];
+    NA tx, ty;
+    const NA *ux, *uy;
+    ty.ptr = NULL;
+    rc = cast_operand(x, up, &tx, &ux);
+    if (!rc) rc = cast_operand(y, up, &ty, &uy);
+    if (!rc) {
+        cumo_hip_ndfunc_t nf = {iter_arr3, 0, 2, 1, {up, 0}};
+        const NA* in[2] = {ux, uy};
+        NA* out[1] = {z};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, (void*)f);
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    return rc;
+}
+
+// x.clip(min, max) (gen/tmpl/clip.c:199-254). lo_kind / hi_kind: 0 absent, 1 the
+// scalar, 2 the array. The result has x's type; array bounds are cast to it, and a
+// scalar bound beside an array bound becomes a 0-dimensional array, as there.
+int cumo_hip_na_clip(const cumo_hip_narray_t* x, int lo_kind, double lo_s, const cumo_hip_narray_t* lo_a, int hi_kind,
+                     double hi_s, const cumo_hip_narray_t* hi_a, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    if (lo_kind == 0 && hi_kind == 0) return fail(CUMO_HIP_ERROR_ARGUMENT, "min and max are not given");
+    const int t = x->type;
+    ClipOpt opt = {t, 0, lo_s, hi_s, false};
+    NA* out[1] = {z};
+    if (lo_kind != 2 && hi_kind != 2) {
+        if (lo_kind == 1 && hi_kind == 1) {
+            // compared in the element type, as the caller there does after m_num_to_data
+            bool bad;
+            if (t == CUMO_HIP_SFLOAT) bad = (float)lo_s > (float)hi_s;
+            else if (t == CUMO_HIP_DFLOAT) bad = lo_s > hi_s;
+            else bad = (int32_t)lo_s > (int32_t)hi_s;
+            if (bad) return fail(CUMO_HIP_ERROR_OPERATION, "min is greater than max");
+            opt.form = 0;
+        } else {
+            opt.form = lo_kind == 1 ? 1 : 2;
+        }
+        cumo_hip_ndfunc_t nf = {iter_clip, 0, 1, 1, {t, 0}};
+        const NA* in[1] = {x};
+        return cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    }
+    NA tlo, thi;
+    tlo.ptr = thi.ptr = NULL;
+    const NA *ulo = NULL, *uhi = NULL;
+    if (lo_kind == 2) {
+        rc = check_arith(lo_a);
+        if (!rc) rc = cast_operand(lo_a, t, &tlo, &ulo);
+    } else if (lo_kind == 1) {
+        rc = cumo_hip_na_alloc(&tlo, t, 0, NULL);
+        if (!rc) rc = cumo_hip_na_fill(&tlo, lo_s);
+        ulo = &tlo;
+    }
+    if (!rc) {
+        if (hi_kind == 2) {
+            rc = check_arith(hi_a);
+            if (!rc) rc = cast_operand(hi_a, t, &thi, &uhi);
+        } else if (hi_kind == 1) {
+            rc = cumo_hip_na_alloc(&thi, t, 0, NULL);
+            if (!rc) rc = cumo_hip_na_fill(&thi, hi_s);
+            uhi = &thi;
+        }
+    }
+    if (!rc) {
+        if (ulo && uhi) {
+            opt.form = 5;
+            cumo_hip_ndfunc_t nf = {iter_clip, 0, 3, 1, {t, 0}};
+            const NA* in[3] = {x, ulo, uhi};
+            rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+        } else {
+            opt.form = ulo ? 3 : 4;
+            cumo_hip_ndfunc_t nf = {iter_clip, 0, 2, 1, {t, 0}};
+            const NA* in[2] = {x, ulo ? ulo : uhi};
+            rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+        }
+    }
+    free_tmp(&tlo);
+    free_tmp(&thi);
+    if (!rc && opt.flagged) return fail(CUMO_HIP_ERROR_OPERATION, "min is greater than max");
     return rc;
 }
 

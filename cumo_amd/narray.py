@@ -369,6 +369,65 @@ class _Numeric(NArray):
     def __mod__(self, o): return self._binary(o, "mod")
     def __rmod__(self, o): return self._binary(o, "mod", True)
 
+    # -- pow, clip, maximum / minimum -------------------------------------------
+    def __pow__(self, other):
+        """reference: gen/tmpl/pow.c:117-215. An Integer exponent takes the
+        repeated-product form, a Float exponent pow(); a Float exponent over an
+        Int32 array moves the array to DFloat first."""
+        z = NArrayDesc()
+        if isinstance(other, numbers.Number):
+            is_int = isinstance(other, numbers.Integral)
+            x = (self if is_int else self._scalar_operand(float(other)))._desc()
+            return _run(_L.cumo_hip_na_pow_s, C.byref(x), float(other), 1 if is_int else 0, 0, C.byref(z), results=(z,))
+        if not isinstance(other, _Numeric):
+            return NotImplemented
+        x, y = self._desc(), other._desc()
+        return _run(_L.cumo_hip_na_pow, C.byref(x), C.byref(y), C.byref(z), results=(z,))
+
+    def __rpow__(self, other):
+        if not isinstance(other, numbers.Number):
+            return NotImplemented
+        z = NArrayDesc()
+        x = self._desc()
+        return _run(_L.cumo_hip_na_pow_s, C.byref(x), float(other), 1 if isinstance(other, numbers.Integral) else 0, 1,
+                    C.byref(z), results=(z,))
+
+    def pow(self, other): return self.__pow__(other)
+
+    def clip(self, min=None, max=None):
+        """reference: gen/tmpl/clip.c:199-254"""
+        def bound(b):
+            if b is None:
+                return 0, 0.0, None
+            if isinstance(b, numbers.Number):
+                return 1, float(b), None
+            if not isinstance(b, _Numeric):
+                b = type(self).cast(b)
+            return 2, 0.0, b._desc()
+        lk, ls, la = bound(min)
+        hk, hs, ha = bound(max)
+        z = NArrayDesc()
+        x = self._desc()
+        return _run(_L.cumo_hip_na_clip, C.byref(x), lk, ls, C.byref(la) if la is not None else None, hk, hs,
+                    C.byref(ha) if ha is not None else None, C.byref(z), results=(z,))
+
+    @classmethod
+    def _ewcomp(cls, op, a, b, nan):
+        a = a if isinstance(a, _Numeric) else cls.cast(a)
+        b = b if isinstance(b, _Numeric) else cls.cast(b)
+        z = NArrayDesc()
+        x, y = a._desc(), b._desc()
+        return _run(_L.cumo_hip_na_ewcomp, op.encode(), C.byref(x), C.byref(y), 1 if nan else 0, C.byref(z), results=(z,))
+
+    @classmethod
+    def maximum(cls, a, b, nan=False):
+        """reference: gen/tmpl/ewcomp.c:40-75"""
+        return cls._ewcomp("maximum", a, b, nan)
+
+    @classmethod
+    def minimum(cls, a, b, nan=False):
+        return cls._ewcomp("minimum", a, b, nan)
+
     # -- unary ----------------------------------------------------------------
     def _unary(self, op):
         x, z = self._desc(), NArrayDesc()

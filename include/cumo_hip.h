@@ -221,6 +221,49 @@ CUMO_HIP_DECL_FILL(sfloat, float)
 CUMO_HIP_DECL_FILL(dfloat, double)
 CUMO_HIP_DECL_FILL(int32, int32_t)
 
+/* pow: narray/gen/tmpl/pow_kernel.cu:6-36,58-113, host narray/gen/tmpl/pow.c:2-6.
+ * A numeric exponent or base rides in as sv; an Int32 exponent takes the
+ * repeated-product form (types/float_macro_kernel.h:125-149, int_macro_kernel.h:26-42). */
+#define CUMO_HIP_DECL_POW(t, c) \
+    void cumo_iter_##t##_pow_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_pow_s_kernel_launch(cumo_na_iarray_t* a1, c sv, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer, int scalar_is_left); \
+    void cumo_iter_##t##_pow_int32_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_pow_int32_s_kernel_launch(cumo_na_iarray_t* a1, int32_t sv, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_pow_int32_s_left_kernel_launch(c sv_base, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
+
+/* maximum / minimum of two arrays: narray/gen/tmpl/ewcomp_kernel.cu:5-32, host
+ * narray/gen/tmpl/ewcomp.c:18; semantics types/real_accum_kernel.h:28-70,
+ * xint_macro_kernel.h:54-68 (no iter_ in these names) */
+#define CUMO_HIP_DECL_EWCOMP(t, name) \
+    void cumo_##t##_##name##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
+
+/* clip: narray/gen/tmpl/clip_kernel.cu:7-44,65-136, host narray/gen/tmpl/clip.c:2-7.
+ * The array-bounds form leaves an element with min > max unwritten and sets *invalid. */
+#define CUMO_HIP_DECL_CLIP(t, c) \
+    void cumo_iter_##t##_clip_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_iarray_t* a4, cumo_na_indexer_t* indexer, int* invalid); \
+    void cumo_iter_##t##_clip_s_kernel_launch(cumo_na_iarray_t* a1, c sv_min, c sv_max, cumo_na_iarray_t* a4, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_clip_min_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_clip_min_s_kernel_launch(cumo_na_iarray_t* a1, c sv, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_clip_max_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_clip_max_s_kernel_launch(cumo_na_iarray_t* a1, c sv, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
+
+CUMO_HIP_DECL_POW(sfloat, float)
+CUMO_HIP_DECL_POW(dfloat, double)
+CUMO_HIP_DECL_POW(int32, int32_t)
+CUMO_HIP_DECL_EWCOMP(sfloat, maximum)
+CUMO_HIP_DECL_EWCOMP(sfloat, maximum_nan)
+CUMO_HIP_DECL_EWCOMP(sfloat, minimum)
+CUMO_HIP_DECL_EWCOMP(sfloat, minimum_nan)
+CUMO_HIP_DECL_EWCOMP(dfloat, maximum)
+CUMO_HIP_DECL_EWCOMP(dfloat, maximum_nan)
+CUMO_HIP_DECL_EWCOMP(dfloat, minimum)
+CUMO_HIP_DECL_EWCOMP(dfloat, minimum_nan)
+CUMO_HIP_DECL_EWCOMP(int32, maximum)
+CUMO_HIP_DECL_EWCOMP(int32, minimum)
+CUMO_HIP_DECL_CLIP(sfloat, float)
+CUMO_HIP_DECL_CLIP(dfloat, double)
+CUMO_HIP_DECL_CLIP(int32, int32_t)
+
 /* typed store / cast, dst = (dst type)src: narray/gen/tmpl/store_from_kernel.cu:3-53,
  * host narray/gen/tmpl/store_from.c:2; pairs narray/gen/spec.rb:122-142.
  * a1 is the destination, a2 the source. int64 appears because Int32#sum
@@ -322,7 +365,8 @@ enum {
     CUMO_HIP_ERROR_ZERO_DIVISION = 5,  /* ZeroDivisionError (narray/gen/tmpl/binary.c:120-126) */
     CUMO_HIP_ERROR_TYPE = 6,           /* TypeError / NoMethodError: no such operation for this element type */
     CUMO_HIP_ERROR_VALUE = 7,          /* Cumo::NArray::ValueError (narray/gen/tmpl/unary2.c:61-66) */
-    CUMO_HIP_ERROR_DIMENSION = 8       /* Cumo::NArray::DimensionError (narray/narray.c:1757-1759) */
+    CUMO_HIP_ERROR_DIMENSION = 8,      /* Cumo::NArray::DimensionError (narray/narray.c:1757-1759) */
+    CUMO_HIP_ERROR_OPERATION = 9       /* Cumo::NArray::OperationError (narray/gen/tmpl/clip.c:48-51,222) */
 };
 typedef void (*cumo_hip_error_handler_t)(int kind, int hip_status, const char* message);
 void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler);

@@ -159,6 +159,23 @@ int cumo_hip_na_binary_s(const char* op, const cumo_hip_narray_t* x, double sv, 
  * Int32 reciprocal / abs report CUMO_HIP_ERROR_ZERO_DIVISION / CUMO_HIP_ERROR_ARGUMENT
  * for 1/0 and |INT_MIN| (reference: gen/tmpl/unary.c:76-119, unary2.c). */
 int cumo_hip_na_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
+/* z = x ** y (reference: gen/tmpl/pow.c:117-215): the result has the higher type of
+ * the two; an Int32 y takes the repeated-product form. pow_s: x ** sv, or sv ** x
+ * when scalar_is_left; sv_is_integer selects the Int32 form as a Ruby Integer does.
+ * Int32 ** non-integer reports CUMO_HIP_ERROR_TYPE (cast x first); a non-integer
+ * base over an Int32 x answers DFloat. */
+int cumo_hip_na_pow(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
+int cumo_hip_na_pow_s(const cumo_hip_narray_t* x, double sv, int sv_is_integer, int scalar_is_left, cumo_hip_narray_t* z);
+/* Cumo::<T>.maximum / minimum of two arrays; nan selects the NaN-propagating form
+ * (reference: gen/tmpl/ewcomp.c, types/real_accum_kernel.h:28-70). */
+int cumo_hip_na_ewcomp(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, int nan, cumo_hip_narray_t* z);
+/* x.clip(min, max) (reference: gen/tmpl/clip.c:199-254). lo_kind / hi_kind: 0 absent,
+ * 1 the scalar lo_s / hi_s, 2 the array lo_a / hi_a. min > max reports
+ * CUMO_HIP_ERROR_OPERATION (two scalars: before anything is written; arrays: after
+ * the launch, elements with min > max left unwritten); no bound at all
+ * CUMO_HIP_ERROR_ARGUMENT. */
+int cumo_hip_na_clip(const cumo_hip_narray_t* x, int lo_kind, double lo_s, const cumo_hip_narray_t* lo_a, int hi_kind,
+                     double hi_s, const cumo_hip_narray_t* hi_a, cumo_hip_narray_t* z);
 /* Cumo::NMath functions of one and two arguments (reference: gen/tmpl/unary_s.c, binary_s.c). */
 int cumo_hip_na_math(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
 int cumo_hip_na_math2(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);

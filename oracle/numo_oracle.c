@@ -120,6 +120,14 @@ static int T##_binary(const char *op, T x, T y, T *z)                          \
         *z = (x >= y) ? x : ((y == y) ? y : x); return 1; }                    \
     if (!strcmp(op, "minimum")) { /* types/real_accum.h:466-475 */             \
         *z = (x <= y) ? x : ((y == y) ? y : x); return 1; }                    \
+    if (!strcmp(op, "maximum_nan")) { /* types/real_accum.h:455-464 */         \
+        *z = (x >= y) ? x : ((x != x) ? x : y); return 1; }                    \
+    if (!strcmp(op, "minimum_nan")) { /* types/real_accum.h:477-486 */         \
+        *z = (x <= y) ? x : ((x != x) ? x : y); return 1; }                    \
+    if (!strcmp(op, "pow")) { *z = (T)pow(x, y); return 1; } /* float_macro.h:33 */ \
+    /* narray/gen/tmpl/clip.c:74-75,106-107: one-sided clip */                 \
+    if (!strcmp(op, "clip_min")) { *z = (x < y) ? y : x; return 1; }           \
+    if (!strcmp(op, "clip_max")) { *z = (x > y) ? y : x; return 1; }           \
     return 0;                                                                  \
 }
 FLOAT_BINARY(float)
@@ -223,6 +231,19 @@ static int i32_binary(const char *op, int32_t x, int32_t y, int32_t *z, int *fla
     if (!strcmp(op, "right_shift")) { *z = x >> (y & 31); return 1; }
     if (!strcmp(op, "maximum")) { *z = (x >= y) ? x : y; return 1; }
     if (!strcmp(op, "minimum")) { *z = (x <= y) ? x : y; return 1; }
+    if (!strcmp(op, "clip_min")) { *z = (x < y) ? y : x; return 1; }
+    if (!strcmp(op, "clip_max")) { *z = (x > y) ? y : x; return 1; }
+    if (!strcmp(op, "pow")) { /* types/int_macro_kernel.h:26-42 (the host copy in int_macro.h:26-42 is commented out) */
+        uint32_t ux = (uint32_t)x, r = 1u; int32_t p = y;
+        switch (p) {
+        case 0: *z = 1; return 1;
+        case 1: *z = x; return 1;
+        case 2: *z = (int32_t)(ux * ux); return 1;
+        case 3: *z = (int32_t)(ux * ux * ux); return 1;
+        }
+        if (p < 0) { *z = 0; return 1; }
+        while (p) { if (p & 1) r *= ux; ux *= ux; p >>= 1; }
+        *z = (int32_t)r; return 1; }
     return 0;
 }
 
@@ -787,6 +808,42 @@ int numo_rows_reduce(const char *op, int dtype, size_t nrows, size_t n,
     for (size_t r = 0; r < nrows; ++r) {
         if (dtype == T_SFLOAT) ((float *)out)[r] = numo_sfloat_f(op, n, (const float *)(p + (ssize_t)r * row_step));
         else if (dtype == T_DFLOAT) ((double *)out)[r] = numo_dfloat_f(op, n, (const double *)(p + (ssize_t)r * row_step));
+        else return -1;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* Float ** Int32: types/float_macro.h:125-144 (pow_int). Products in  */
+/* the element type up to an exponent of 64, pow() beyond, 1/.. for a  */
+/* negative exponent. Flat arrays of n elements; p_step 0 repeats one  */
+/* exponent, x_step 0 one base.                                        */
+/* ------------------------------------------------------------------ */
+#define POW_INT(T)                                                             \
+static T T##_pow_int(T x, int p)                                               \
+{                                                                              \
+    T r = 1;                                                                   \
+    switch (p) {                                                               \
+    case 0: return 1;                                                          \
+    case 1: return x;                                                          \
+    case 2: return x * x;                                                      \
+    case 3: return x * x * x;                                                  \
+    case 4: x = x * x; return x * x;                                           \
+    }                                                                          \
+    if (p < 0) return 1 / T##_pow_int(x, (int)(0u - (unsigned)p));             \
+    if (p > 64) return (T)pow(x, p);                                           \
+    while (p) { if (p & 1) r *= x; x *= x; p >>= 1; }                          \
+    return r;                                                                  \
+}
+POW_INT(float)
+POW_INT(double)
+
+int numo_pow_int(int dtype, size_t n, const void *x, ssize_t x_step, const int32_t *p, ssize_t p_step, void *out)
+{
+    for (size_t i = 0; i < n; ++i) {
+        const int32_t e = p[(ssize_t)i * p_step];
+        if (dtype == T_SFLOAT) ((float *)out)[i] = float_pow_int(((const float *)x)[(ssize_t)i * x_step], e);
+        else if (dtype == T_DFLOAT) ((double *)out)[i] = double_pow_int(((const double *)x)[(ssize_t)i * x_step], e);
         else return -1;
     }
     return 0;

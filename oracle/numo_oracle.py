@@ -44,6 +44,8 @@ lib.numo_copy_bytes.restype = C.c_int
 lib.numo_fill.restype = C.c_int
 lib.numo_bit_binary.restype = C.c_int
 lib.numo_bit_count.restype = C.c_uint64
+lib.numo_pow_int.argtypes = [C.c_int, SZ, C.c_void_p, SSZ, C.c_void_p, SSZ, C.c_void_p]
+lib.numo_pow_int.restype = C.c_int
 lib.numo_bit_count.argtypes = [C.c_void_p, SZ, SSZ, C.c_uint64, C.c_int]
 lib.numo_reduce.restype = C.c_int
 lib.numo_sfloat_f.restype = C.c_float
@@ -113,6 +115,44 @@ def unary(op, x, out=None):
     if rc == 1:
         raise FlagError(res)
     return res
+
+
+def pow_int(x, p):
+    """Float array (or one float) ** Int32 array (or one integer): the repeated-product
+    form of types/float_macro.h:125-144. Operands are broadcast; x fixes the type."""
+    xa = np.asarray(x)
+    pa = np.asarray(p, dtype=np.int32)
+    shape = np.broadcast_shapes(xa.shape, pa.shape)
+    xf = np.ascontiguousarray(np.broadcast_to(xa, shape)).reshape(-1)
+    pf = np.ascontiguousarray(np.broadcast_to(pa, shape)).reshape(-1)
+    out = np.zeros(xf.shape, dtype=xf.dtype)
+    rc = lib.numo_pow_int(_tcode(xf), xf.size, C.c_void_p(xf.ctypes.data), 1, C.c_void_p(pf.ctypes.data), 1,
+                          C.c_void_p(out.ctypes.data))
+    if rc:
+        raise ValueError("oracle: pow_int of a non-float type")
+    return out.reshape(shape)
+
+
+def clip(x, lo=None, hi=None):
+    """x.clip(lo, hi) (narray/gen/tmpl/clip.c:23-33,199-254); bounds are numbers, arrays
+    of x's type, or None. Raises FlagError when a lower bound exceeds its upper bound
+    (the elements concerned keep the zeros of the fresh result)."""
+    res = x.copy()
+    if lo is not None and hi is not None:
+        lo_a = np.broadcast_to(np.asarray(lo, dtype=x.dtype), x.shape)
+        hi_a = np.broadcast_to(np.asarray(hi, dtype=x.dtype), x.shape)
+        with np.errstate(invalid="ignore"):
+            bad = lo_a > hi_a
+        res = binary("clip_max", binary("clip_min", x, np.ascontiguousarray(lo_a)), np.ascontiguousarray(hi_a))
+        if bad.any():
+            res[bad] = 0
+            raise FlagError(res)
+        return res
+    if lo is not None:
+        return binary("clip_min", x, lo if not isinstance(lo, np.ndarray) else lo.astype(x.dtype))
+    if hi is not None:
+        return binary("clip_max", x, hi if not isinstance(hi, np.ndarray) else hi.astype(x.dtype))
+    raise ValueError("min and max are not given")
 
 
 def _bit_words(nbits):
