@@ -1,0 +1,209 @@
+// mulsum: the sum of products of two runs (the inner product under Cumo's dot).
+//
+// Replaces narray/gen/tmpl/accum_binary_kernel.cu of the reference (a grid of up to
+// 1024 blocks of 512 threads with a nine-level LDS tree each, then one block over
+// the partials). Here a block takes one contiguous chunk of the run, lanes read 128
+// bits from both operands when both are contiguous and keep four independent
+// accumulators, lanes combine with wave64 shuffles and the four waves through LDS;
+// the partials of the blocks are folded in index order by a second launch, which
+// also adds onto what the result already holds, as the reference does
+// (accum_binary_kernel.cu:46-47,63). No atomics: the answer does not depend on
+// scheduling. Products and sums are in the element type, unfused, as the macros
+// write them (types/real_accum_kernel.h:6-10, xint_macro_kernel.h:44).
+#include "common.h"
+
+namespace cumo_hip {
+namespace {
+
+constexpr int kMsBlock = 256;
+constexpr int kMsMaxGrid = 2048;
+
+template <class T> struct ms_is_int { static constexpr bool value = false; };
+template <> struct ms_is_int<int32_t> { static constexpr bool value = true; };
+
+template <class T, bool NANF>
+__device__ __forceinline__ void ms_fold(T x, T y, T& acc) {
+    if constexpr (ms_is_int<T>::value) {
+        acc = (T)((uint32_t)acc + (uint32_t)x * (uint32_t)y);
+    } else {
+        if (NANF && (x != x || y != y)) return;
+        acc = x * y + acc;
+    }
+}
+template <class T>
+__device__ __forceinline__ T ms_add(T a, T b) {
+    if constexpr (ms_is_int<T>::value) return (T)((uint32_t)a + (uint32_t)b);
+    else return a + b;
+}
+
+template <class T>
+__device__ __forceinline__ T ms_shfl_down(T v, unsigned d) {
+    if constexpr (sizeof(T) == 8) {
+        union { T t; uint32_t w[2]; } a, b;
+        a.t = v;
+        b.w[0] = __shfl_down(a.w[0], d);
+        b.w[1] = __shfl_down(a.w[1], d);
+        return b.t;
+    } else {
+        union { T t; uint32_t w; } a, b;
+        a.t = v;
+        b.w = __shfl_down(a.w, d);
+        return b.t;
+    }
+}
+
+// the block's total in thread 0
+template <class T>
+__device__ __forceinline__ T ms_block_sum(T acc) {
+    __shared__ T wave_acc[kMsBlock / 64];
+    for (unsigned d = 32; d > 0; d >>= 1) acc = ms_add(acc, ms_shfl_down(acc, d));
+    if ((threadIdx.x & 63) == 0) wave_acc[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kMsBlock / 64; ++w) acc = ms_add(acc, wave_acc[w]);
+    }
+    return acc;
+}
+
+// VEC > 1: both runs contiguous and 16-byte aligned at every chunk start
+template <class T, bool NANF, int VEC>
+__global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1, const char* p2, int64_t s1, int64_t s2, uint64_t n,
+                                                                  uint64_t chunk, T* partial, T* out) {
+    const uint64_t begin = (uint64_t)blockIdx.x * chunk;
+    uint64_t end = begin + chunk;
+    if (end > n) end = n;
+    T acc[4] = {T(), T(), T(), T()};
+    if constexpr (VEC > 1) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        union V { u4 q; T t[VEC]; __device__ V() {} };
+        const uint64_t stride = (uint64_t)kMsBlock * VEC;
+        uint64_t i = begin + (uint64_t)threadIdx.x * VEC;
+        // whole vectors, four per lane and operand in flight
+        for (; i + 3 * stride + VEC <= end; i += 4 * stride) {
+            V a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a[u].q = *reinterpret_cast<const u4*>(p1 + (i + u * stride) * sizeof(T));
+                b[u].q = *reinterpret_cast<const u4*>(p2 + (i + u * stride) * sizeof(T));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) ms_fold<T, NANF>(a[u].t[j], b[u].t[j], acc[u]);
+        }
+        for (; i < end; i += stride) {
+            if (i + VEC <= end) {
+                V a, b;
+                a.q = *reinterpret_cast<const u4*>(p1 + i * sizeof(T));
+                b.q = *reinterpret_cast<const u4*>(p2 + i * sizeof(T));
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) ms_fold<T, NANF>(a.t[j], b.t[j], acc[0]);
+            } else {
+                for (uint64_t k = i; k < end; ++k)
+                    ms_fold<T, NANF>(reinterpret_cast<const T*>(p1)[k], reinterpret_cast<const T*>(p2)[k], acc[0]);
+            }
+        }
+    } else {
+        uint64_t i = begin + threadIdx.x;
+        for (; i + 3 * kMsBlock < end; i += 4 * kMsBlock) {
+            T a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a[u] = *reinterpret_cast<const T*>(p1 + (int64_t)(i + u * kMsBlock) * s1);
+                b[u] = *reinterpret_cast<const T*>(p2 + (int64_t)(i + u * kMsBlock) * s2);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ms_fold<T, NANF>(a[u], b[u], acc[u]);
+        }
+        for (; i < end; i += kMsBlock)
+            ms_fold<T, NANF>(*reinterpret_cast<const T*>(p1 + (int64_t)i * s1), *reinterpret_cast<const T*>(p2 + (int64_t)i * s2), acc[0]);
+    }
+    T tot = ms_add(ms_add(acc[0], acc[1]), ms_add(acc[2], acc[3]));
+    tot = ms_block_sum<T>(tot);
+    if (threadIdx.x == 0) {
+        if (partial) partial[blockIdx.x] = tot;
+        else *out = ms_add(*out, tot);
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(kMsBlock) void mulsum_combine_kernel(const T* partial, uint64_t n, T* out) {
+    T acc = T();
+    for (uint64_t i = threadIdx.x; i < n; i += kMsBlock) acc = ms_add(acc, partial[i]);
+    acc = ms_block_sum<T>(acc);
+    if (threadIdx.x == 0) *out = ms_add(*out, acc);
+}
+
+template <class T, bool NANF>
+__global__ __launch_bounds__(kMsBlock) void mulsum_elementwise_kernel(const char* p1, const char* p2, char* p3, int64_t s1, int64_t s2, int64_t s3,
+                                                                      uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kMsBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kMsBlock) {
+        T* z = reinterpret_cast<T*>(p3 + (int64_t)i * s3);
+        T acc = *z;
+        ms_fold<T, NANF>(*reinterpret_cast<const T*>(p1 + (int64_t)i * s1), *reinterpret_cast<const T*>(p2 + (int64_t)i * s2), acc);
+        *z = acc;
+    }
+}
+
+template <class T, bool NANF>
+void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, uint64_t n) {
+    hipStream_t stream = current_stream();
+    constexpr int VEC = 16 / (int)sizeof(T);
+    // a block's chunk: at least 16 KiB per operand, a whole number of 4-vector rounds
+    const uint64_t round = (uint64_t)kMsBlock * VEC * 4;
+    uint64_t grid = (n + 4 * round - 1) / (4 * round);
+    if (grid == 0) grid = 1;
+    if (grid > (uint64_t)kMsMaxGrid) grid = kMsMaxGrid;
+    uint64_t chunk = (n + grid - 1) / grid;
+    chunk = ((chunk + round - 1) / round) * round;
+    grid = n ? (n + chunk - 1) / chunk : 1;
+    const bool vec = s1 == (ssize_t)sizeof(T) && s2 == (ssize_t)sizeof(T) && ((uintptr_t)p1 % 16) == 0 && ((uintptr_t)p2 % 16) == 0;
+    T* partial = nullptr;
+    if (grid > 1) {
+        partial = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * grid));
+        if (!partial) return;
+    }
+    if (vec)
+        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n,
+                           chunk, partial, reinterpret_cast<T*>(p3));
+    else
+        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n,
+                           chunk, partial, reinterpret_cast<T*>(p3));
+    if (partial) {
+        hipLaunchKernelGGL((mulsum_combine_kernel<T>), dim3(1), dim3(kMsBlock), 0, stream, (const T*)partial, grid, reinterpret_cast<T*>(p3));
+        cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
+    }
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+template <class T, bool NANF>
+void mulsum_elementwise_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, ssize_t s3, uint64_t n) {
+    if (n == 0) return;
+    uint64_t grid = (n + kMsBlock - 1) / kMsBlock;
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL((mulsum_elementwise_kernel<T, NANF>), dim3((unsigned)grid), dim3(kMsBlock), 0, current_stream(), p1, p2, p3, (int64_t)s1,
+                       (int64_t)s2, (int64_t)s3, n);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+}  // namespace
+}  // namespace cumo_hip
+
+using namespace cumo_hip;
+
+extern "C" {
+
+#define CUMO_DEF_MULSUM(t, c, name, NANF)                                                                                  \
+    void cumo_##t##_##name##_reduce_kernel_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, uint64_t n) {      \
+        mulsum_reduce_launch<c, NANF>(p1, p2, p3, s1, s2, n);                                                              \
+    }                                                                                                                      \
+    void cumo_##t##_##name##_kernel_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, ssize_t s3, uint64_t n) { \
+        mulsum_elementwise_launch<c, NANF>(p1, p2, p3, s1, s2, s3, n);                                                     \
+    }
+CUMO_DEF_MULSUM(sfloat, float, mulsum, false)
+CUMO_DEF_MULSUM(sfloat, float, mulsum_nan, true)
+CUMO_DEF_MULSUM(dfloat, double, mulsum, false)
+CUMO_DEF_MULSUM(dfloat, double, mulsum_nan, true)
+CUMO_DEF_MULSUM(int32, int32_t, mulsum, false)
+
+}  // extern "C"

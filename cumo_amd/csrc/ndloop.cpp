@@ -896,6 +896,40 @@ void iter_clip(LP* lp) {
 #undef CLIP_CASES
 }
 
+
+// ---- mulsum (gen/tmpl/accum_binary.c:8-60): the innermost loop dimension is one
+// launch, the others are walked here, as the reference's host-walked loop does.
+typedef void (*MulsumReduceFn)(char*, char*, char*, ssize_t, ssize_t, uint64_t);
+typedef void (*MulsumEwFn)(char*, char*, char*, ssize_t, ssize_t, ssize_t, uint64_t);
+struct MulsumFns {
+    MulsumReduceFn red, red_nan;
+    MulsumEwFn ew, ew_nan;
+};
+const MulsumFns kMulsum[3] = {
+    {cumo_sfloat_mulsum_reduce_kernel_launch, cumo_sfloat_mulsum_nan_reduce_kernel_launch, cumo_sfloat_mulsum_kernel_launch,
+     cumo_sfloat_mulsum_nan_kernel_launch},
+    {cumo_dfloat_mulsum_reduce_kernel_launch, cumo_dfloat_mulsum_nan_reduce_kernel_launch, cumo_dfloat_mulsum_kernel_launch,
+     cumo_dfloat_mulsum_nan_kernel_launch},
+    {cumo_int32_mulsum_reduce_kernel_launch, nullptr, cumo_int32_mulsum_kernel_launch, nullptr},
+};
+struct MulsumOpt {
+    int type;
+    bool nan;
+};
+void mulsum_walk(const LP* lp, int level, char* p1, char* p2, char* p3, const MulsumOpt* o) {
+    const int last = lp->ndim - 1;
+    if (level == last) {
+        const MulsumFns& f = kMulsum[o->type];
+        const ssize_t s1 = lp->args[0].step[last], s2 = lp->args[1].step[last], s3 = lp->args[2].step[last];
+        if (s3 == 0) (o->nan && f.red_nan ? f.red_nan : f.red)(p1, p2, p3, s1, s2, lp->n[last]);
+        else (o->nan && f.ew_nan ? f.ew_nan : f.ew)(p1, p2, p3, s1, s2, s3, lp->n[last]);
+        return;
+    }
+    for (size_t i = 0; i < lp->n[level]; ++i)
+        mulsum_walk(lp, level + 1, p1 + (ssize_t)i * lp->args[0].step[level], p2 + (ssize_t)i * lp->args[1].step[level],
+                    p3 + (ssize_t)i * lp->args[2].step[level], o);
+}
+
 int check_arith(const NA* x) {
     int rc = check_view(x, "operand");
     if (rc) return rc;
@@ -1096,6 +1130,192 @@ int cumo_hip_na_clip(const cumo_hip_narray_t* x, int lo_kind, double lo_s, const
     free_tmp(&tlo);
     free_tmp(&thi);
     if (!rc && opt.flagged) return fail(CUMO_HIP_ERROR_OPERATION, "min is greater than max");
+    return rc;
+}
+
+// x.mulsum(y, axis:, keepdims:, nan:) (gen/tmpl/accum_binary.c:62-110): the sum of the
+// products over the reduced dimensions, started from 0. With more inner runs than
+// is sensible to launch one by one, the products go through an array of their own
+// and the reduction engine (for nan: true that skips a product that is NaN though
+// neither factor is, inf * 0, where the run launcher would add it).
+int cumo_hip_na_mulsum(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, unsigned int reduce, int keepdims, int nan,
+                       cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    const int up = upcast(x->type, y->type);
+    const int nd = x->ndim > y->ndim ? x->ndim : y->ndim;
+    if (reduce == 0) reduce = nd ? ((1u << nd) - 1u) : 0u;
+    NA tx, ty;
+    const NA *ux, *uy;
+    ty.ptr = NULL;
+    rc = cast_operand(x, up, &tx, &ux);
+    if (!rc) rc = cast_operand(y, up, &ty, &uy);
+    if (!rc) {
+        cumo_hip_ndfunc_t nf = {NULL, CUMO_HIP_NDF_FLAT_REDUCE | (keepdims ? CUMO_HIP_NDF_KEEP_DIM : 0u), 2, 1, {up, 0}};
+        const NA* in[2] = {ux, uy};
+        NA* out[1] = {z};
+        LP lp;
+        const bool fresh = z->ptr == NULL;
+        rc = cumo_hip_na_ndloop_prepare(&nf, in, out, reduce, &lp);
+        size_t launches = 1, total = 1;
+        for (int d = 0; !rc && d < lp.ndim; ++d) {
+            total *= lp.n[d];
+            if (d < lp.ndim - 1) launches *= lp.n[d];
+        }
+        if (!rc && total_of(z) != 0) {
+            if (launches <= 1024 || total == 0) {
+                rc = cumo_hip_na_fill(z, 0.0);
+                if (!rc && total != 0) {
+                    MulsumOpt opt = {up, nan != 0 && is_float(up)};
+                    mulsum_walk(&lp, 0, lp.args[0].ptr, lp.args[1].ptr, lp.args[2].ptr, &opt);
+                }
+            } else {
+                NA prod;
+                prod.ptr = NULL;
+                rc = cumo_hip_na_binary("mul", ux, uy, &prod);
+                if (!rc) {
+                    // the product has the broadcast shape, so the same dimensions are reduced
+                    NA zs = *z;
+                    NA sum64;
+                    sum64.ptr = NULL;
+                    if (up == CUMO_HIP_INT32) {
+                        // Int32#sum answers Int64; mulsum stays Int32 (wrapping), so narrow it
+                        rc = cumo_hip_na_reduce("sum", &prod, reduce, keepdims, 0, &sum64, NULL);
+                        if (!rc) rc = cumo_hip_na_store(&zs, &sum64);
+                        free_tmp(&sum64);
+                    } else {
+                        rc = cumo_hip_na_reduce("sum", &prod, reduce, keepdims, nan && is_float(up), &zs, NULL);
+                    }
+                }
+                free_tmp(&prod);
+            }
+        }
+        if (rc && fresh) free_tmp(z);
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    return rc;
+}
+
+// x.cumsum / x.cumprod (axis:, nan:) (gen/tmpl/cum.c:48-80): the running sum or
+// product along the given dimensions taken together in row-major order (all of them
+// when reduce is 0); the result has x's shape and type.
+int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int nan, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    int prod;
+    if (op && !std::strcmp(op, "cumsum")) prod = 0;
+    else if (op && !std::strcmp(op, "cumprod")) prod = 1;
+    else return no_method(op);
+    const int nd = x->ndim;
+    if (nd < 32 && (reduce >> nd)) return fail(CUMO_HIP_ERROR_DIMENSION, "dimension is out of range");
+    if (reduce == 0) reduce = nd ? ((1u << nd) - 1u) : 0u;
+    const bool fresh = z->ptr == NULL;
+    if (fresh) {
+        rc = cumo_hip_na_alloc(z, x->type, nd, x->shape);
+        if (rc) return rc;
+    } else {
+        rc = check_view(z, "result");
+        if (rc) return rc;
+        bool same = z->type == x->type && z->ndim == nd;
+        for (int d = 0; same && d < nd; ++d) same = z->shape[d] == x->shape[d];
+        if (!same) return fail(CUMO_HIP_ERROR_SHAPE, "cum: result array has the wrong shape or type");
+    }
+    if (total_of(x) == 0) return CUMO_HIP_OK;
+    const ssize_t es = kElmsz[x->type];
+
+    // the scanned dimensions as one run: each walks its successor's whole extent
+    bool one_run = true;
+    ssize_t s_in = es, s_out = es;
+    size_t n = 1;
+    {
+        bool first = true;
+        for (int d = nd - 1; d >= 0; --d) {
+            if (!((reduce >> d) & 1u) || x->shape[d] == 1) continue;
+            if (first) {
+                s_in = x->stride[d];
+                s_out = z->stride[d];
+                first = false;
+            } else if (x->stride[d] != s_in * (ssize_t)n || z->stride[d] != s_out * (ssize_t)n) {
+                one_run = false;
+            }
+            n *= x->shape[d];
+        }
+    }
+    const NA* src = x;
+    NA* dst = z;
+    NA tx, tz, zperm;
+    tx.ptr = tz.ptr = NULL;
+    unsigned int red = reduce;
+    if (!one_run) {
+        // bring the scanned dimensions together at the end of a contiguous copy, scan
+        // that into a contiguous result, and store it back through the same permutation
+        NA xperm = *x;
+        zperm = *z;
+        int k = 0;
+        for (int pass = 0; pass < 2; ++pass)
+            for (int d = 0; d < nd; ++d)
+                if ((((reduce >> d) & 1u) != 0) == (pass == 1)) {
+                    xperm.shape[k] = x->shape[d];
+                    xperm.stride[k] = x->stride[d];
+                    zperm.shape[k] = z->shape[d];
+                    zperm.stride[k] = z->stride[d];
+                    ++k;
+                }
+        int nred = 0;
+        for (int d = 0; d < nd; ++d) nred += (reduce >> d) & 1u;
+        red = ((1u << nred) - 1u) << (nd - nred);
+        rc = cumo_hip_na_copy(&xperm, &tx);
+        if (!rc) rc = cumo_hip_na_alloc(&tz, x->type, nd, xperm.shape);
+        if (rc) {
+            free_tmp(&tx);
+            if (fresh) free_tmp(z);
+            return rc;
+        }
+        src = &tx;
+        dst = &tz;
+        n = 1;
+        for (int d = nd - nred; d < nd; ++d) n *= src->shape[d];
+        s_in = s_out = es;
+    }
+    cumo_hip_scan_rows_t runs;
+    std::memset(&runs, 0, sizeof(runs));
+    runs.rows = 1;
+    for (int d = 0; d < nd; ++d) {
+        if (((red >> d) & 1u) || src->shape[d] == 1) continue;
+        runs.oshape[runs.nouter] = src->shape[d];
+        runs.ostep_in[runs.nouter] = src->stride[d];
+        runs.ostep_out[runs.nouter] = dst->stride[d];
+        runs.rows *= src->shape[d];
+        ++runs.nouter;
+    }
+    runs.n = n;
+    runs.s_in = s_in;
+    runs.s_out = s_out;
+    runs.in = src->ptr + src->offset;
+    runs.out = dst->ptr + dst->offset;
+    const bool use_nan = nan && is_float(x->type);
+    if (runs.rows == 1 && n > (1u << 16)) {
+        // one long run: the three-launch form
+        typedef int (*RunFn)(char*, char*, ssize_t, ssize_t, uint64_t);
+        static const RunFn fns[3][4] = {
+            {cumo_sfloat_cumsum_kernel_launch, cumo_sfloat_cumsum_nan_kernel_launch, cumo_sfloat_cumprod_kernel_launch, cumo_sfloat_cumprod_nan_kernel_launch},
+            {cumo_dfloat_cumsum_kernel_launch, cumo_dfloat_cumsum_nan_kernel_launch, cumo_dfloat_cumprod_kernel_launch, cumo_dfloat_cumprod_nan_kernel_launch},
+            {cumo_int32_cumsum_kernel_launch, cumo_int32_cumsum_kernel_launch, cumo_int32_cumprod_kernel_launch, cumo_int32_cumprod_kernel_launch},
+        };
+        const int st = fns[x->type][prod * 2 + (use_nan ? 1 : 0)](runs.in, runs.out, s_in, s_out, n);
+        if (st != 0) {
+            cumo_hip::report_hip_error((hipError_t)st, "cumsum/cumprod launch");
+            rc = CUMO_HIP_ERROR_RUNTIME;
+        }
+    } else {
+        cumo_hip_scan_rows_kernel_launch(x->type, prod, use_nan ? 1 : 0, &runs);
+    }
+    if (!rc && !one_run) rc = cumo_hip_na_store(&zperm, &tz);
+    free_tmp(&tx);
+    free_tmp(&tz);
+    if (rc && fresh) free_tmp(z);
     return rc;
 }
 

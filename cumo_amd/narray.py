@@ -428,6 +428,29 @@ class _Numeric(NArray):
     def minimum(cls, a, b, nan=False):
         return cls._ewcomp("minimum", a, b, nan)
 
+    # -- mulsum, cumsum / cumprod ---------------------------------------------------
+    def mulsum(self, other, axis=None, keepdims=False, nan=False):
+        """reference: gen/tmpl/accum_binary.c:62-110"""
+        if not isinstance(other, _Numeric):
+            other = type(self).cast(other)
+        nd = max(self.ndim, other.ndim)
+        z = NArrayDesc()
+        x, y = self._desc(), other._desc()
+        return _run(_L.cumo_hip_na_mulsum, C.byref(x), C.byref(y), _reduce_mask(nd, axis), 1 if keepdims else 0,
+                    1 if nan else 0, C.byref(z), results=(z,))
+
+    def _cum(self, op, axis, nan):
+        z = NArrayDesc()
+        x = self._desc()
+        return _run(_L.cumo_hip_na_cum, op.encode(), C.byref(x), _reduce_mask(self.ndim, axis), 1 if nan else 0, C.byref(z),
+                    results=(z,))
+
+    def cumsum(self, axis=None, nan=False):
+        """reference: gen/tmpl/cum.c:48-80"""
+        return self._cum("cumsum", axis, nan)
+
+    def cumprod(self, axis=None, nan=False): return self._cum("cumprod", axis, nan)
+
     # -- unary ----------------------------------------------------------------
     def _unary(self, op):
         x, z = self._desc(), NArrayDesc()

@@ -264,6 +264,34 @@ CUMO_HIP_DECL_CLIP(sfloat, float)
 CUMO_HIP_DECL_CLIP(dfloat, double)
 CUMO_HIP_DECL_CLIP(int32, int32_t)
 
+/* cumsum / cumprod along one run of n elements with byte steps s1 (input) and s2
+ * (result): narray/gen/tmpl/cum_kernel.cu:51-76, host narray/gen/tmpl/cum.c:3.
+ * Returns 0 or the runtime's error code, as the reference returns cudaError_t. */
+#define CUMO_HIP_DECL_CUM(t, name) \
+    int cumo_##t##_##name##_kernel_launch(char *p1, char *p2, ssize_t s1, ssize_t s2, uint64_t n);
+CUMO_HIP_DECL_CUM(sfloat, cumsum)
+CUMO_HIP_DECL_CUM(sfloat, cumsum_nan)
+CUMO_HIP_DECL_CUM(sfloat, cumprod)
+CUMO_HIP_DECL_CUM(sfloat, cumprod_nan)
+CUMO_HIP_DECL_CUM(dfloat, cumsum)
+CUMO_HIP_DECL_CUM(dfloat, cumsum_nan)
+CUMO_HIP_DECL_CUM(dfloat, cumprod)
+CUMO_HIP_DECL_CUM(dfloat, cumprod_nan)
+CUMO_HIP_DECL_CUM(int32, cumsum)
+CUMO_HIP_DECL_CUM(int32, cumprod)
+
+/* mulsum: narray/gen/tmpl/accum_binary_kernel.cu:32-110, host
+ * narray/gen/tmpl/accum_binary.c:4-5. The reduce form ADDS the sum of the n
+ * products onto *p3; the other form does p3[i] += p1[i] * p2[i]. Steps in bytes. */
+#define CUMO_HIP_DECL_MULSUM(t, name) \
+    void cumo_##t##_##name##_reduce_kernel_launch(char *p1, char *p2, char *p3, ssize_t s1, ssize_t s2, uint64_t n); \
+    void cumo_##t##_##name##_kernel_launch(char *p1, char *p2, char *p3, ssize_t s1, ssize_t s2, ssize_t s3, uint64_t n);
+CUMO_HIP_DECL_MULSUM(sfloat, mulsum)
+CUMO_HIP_DECL_MULSUM(sfloat, mulsum_nan)
+CUMO_HIP_DECL_MULSUM(dfloat, mulsum)
+CUMO_HIP_DECL_MULSUM(dfloat, mulsum_nan)
+CUMO_HIP_DECL_MULSUM(int32, mulsum)
+
 /* typed store / cast, dst = (dst type)src: narray/gen/tmpl/store_from_kernel.cu:3-53,
  * host narray/gen/tmpl/store_from.c:2; pairs narray/gen/spec.rb:122-142.
  * a1 is the destination, a2 the source. int64 appears because Int32#sum
@@ -373,6 +401,22 @@ void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler);
 /* Returns the latched error kind (0 if none) and clears it; message, if not
  * NULL, receives a pointer to a thread-local string. */
 int cumo_hip_last_error(const char** message);
+
+/* Many scan runs in one launch (no counterpart in the reference, which calls the
+ * run launcher once per run from a loop on the host, narray/gen/tmpl/cum.c:12-46).
+ * Run r starts at in + sum_k i_k * ostep_in[k] where (i_0 .. i_{nouter-1}) is r
+ * decomposed over oshape, row-major; elements of a run are s_in / s_out bytes apart.
+ * type: 0 SFloat, 1 DFloat, 2 Int32. */
+typedef struct {
+    int      nouter;
+    uint64_t rows, n;
+    size_t   oshape[CUMO_NA_MAX_DIMENSION];
+    ssize_t  ostep_in[CUMO_NA_MAX_DIMENSION], ostep_out[CUMO_NA_MAX_DIMENSION];
+    ssize_t  s_in, s_out;
+    char*    in;
+    char*    out;
+} cumo_hip_scan_rows_t;
+void cumo_hip_scan_rows_kernel_launch(int type, int prod, int nan, const cumo_hip_scan_rows_t* runs);
 
 /* The stream every launcher and the pool use from this host thread. The
  * reference only ever uses the default stream (cuda/memory_pool.cpp:43-44). */

@@ -204,6 +204,16 @@ int cumo_hip_na_fill(cumo_hip_narray_t* dst, double value);
 int cumo_hip_na_reduce(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, int nan,
                        cumo_hip_narray_t* z, cumo_hip_narray_t* z2);
 
+/* z = sum over the reduced dimensions of x * y, started from 0 (reference:
+ * gen/tmpl/accum_binary.c:62-110); reduce / keepdims / nan as for cumo_hip_na_reduce.
+ * The result has the higher type of the two (Int32 stays Int32, wrapping). */
+int cumo_hip_na_mulsum(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, unsigned int reduce, int keepdims, int nan,
+                       cumo_hip_narray_t* z);
+/* op "cumsum" or "cumprod": the running value along the dimensions in `reduce` taken
+ * together in row-major order (0 = all); z has x's shape and type (reference:
+ * gen/tmpl/cum.c:48-80). nan: NaN elements are skipped (leading ones stay NaN). */
+int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int nan, cumo_hip_narray_t* z);
+
 /* Bit logic: and or xor eq / copy not (reference: gen/tmpl_bit/binary.c, unary.c). */
 int cumo_hip_na_bit_binary(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
 int cumo_hip_na_bit_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);

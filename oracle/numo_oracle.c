@@ -848,3 +848,77 @@ int numo_pow_int(int dtype, size_t n, const void *x, ssize_t x_step, const int32
     }
     return 0;
 }
+
+/* ------------------------------------------------------------------ */
+/* cumsum / cumprod along one run: the host loop of                    */
+/* narray/gen/tmpl/cum.c:32-45 with the operators of                   */
+/* types/real_accum.h:9-23 and xint_macro.h:46-47. The first element   */
+/* is copied through; each later one updates the running value.        */
+/* ------------------------------------------------------------------ */
+#define CUM_RUN(T, ISNAN)                                                      \
+static void T##_cum_run(int prod, int nan, size_t n, const char *p1, ssize_t s1, char *p2, ssize_t s2) \
+{                                                                              \
+    if (n == 0) return;                                                        \
+    T x = *(const T *)p1;                                                      \
+    *(T *)p2 = x;                                                              \
+    for (size_t i = 1; i < n; ++i) {                                           \
+        const T y = *(const T *)(p1 + (ssize_t)i * s1);                        \
+        if (nan) {                                                             \
+            if (ISNAN(x)) x = y;                                               \
+            else if (!ISNAN(y)) x = prod ? x * y : x + y;                      \
+        } else {                                                               \
+            x = prod ? x * y : x + y;                                          \
+        }                                                                      \
+        *(T *)(p2 + (ssize_t)i * s2) = x;                                      \
+    }                                                                          \
+}
+#define FISNAN(v) ((v) != (v))
+CUM_RUN(float, FISNAN)
+CUM_RUN(double, FISNAN)
+
+int numo_cum_run(int prod, int dtype, int nan, size_t n, const char *p1, ssize_t s1, char *p2, ssize_t s2)
+{
+    if (dtype == T_SFLOAT) float_cum_run(prod, nan, n, p1, s1, p2, s2);
+    else if (dtype == T_DFLOAT) double_cum_run(prod, nan, n, p1, s1, p2, s2);
+    else if (dtype == T_INT32) {
+        if (n == 0) return 0;
+        uint32_t x = *(const uint32_t *)p1;
+        *(uint32_t *)p2 = x;
+        for (size_t i = 1; i < n; ++i) {
+            const uint32_t y = *(const uint32_t *)(p1 + (ssize_t)i * s1);
+            x = prod ? x * y : x + y;   /* wrapping, done in unsigned */
+            *(uint32_t *)(p2 + (ssize_t)i * s2) = x;
+        }
+    } else return -1;
+    return 0;
+}
+
+/* mulsum over one run, added onto *acc: narray/gen/tmpl/accum_binary.c:27-38   */
+/* with types/real_accum.h:3-7 and xint_macro.h:44. Product and sum are two     */
+/* roundings in the element type (this file is built with -ffp-contract=off).   */
+int numo_mulsum_run(int dtype, int nan, size_t n, const char *p1, ssize_t s1, const char *p2, ssize_t s2, void *acc)
+{
+    if (dtype == T_SFLOAT) {
+        float z = *(float *)acc;
+        for (size_t i = 0; i < n; ++i) {
+            const float x = *(const float *)(p1 + (ssize_t)i * s1), y = *(const float *)(p2 + (ssize_t)i * s2);
+            if (nan && (x != x || y != y)) continue;
+            z = x * y + z;
+        }
+        *(float *)acc = z;
+    } else if (dtype == T_DFLOAT) {
+        double z = *(double *)acc;
+        for (size_t i = 0; i < n; ++i) {
+            const double x = *(const double *)(p1 + (ssize_t)i * s1), y = *(const double *)(p2 + (ssize_t)i * s2);
+            if (nan && (x != x || y != y)) continue;
+            z = x * y + z;
+        }
+        *(double *)acc = z;
+    } else if (dtype == T_INT32) {
+        uint32_t z = *(uint32_t *)acc;
+        for (size_t i = 0; i < n; ++i)
+            z += *(const uint32_t *)(p1 + (ssize_t)i * s1) * *(const uint32_t *)(p2 + (ssize_t)i * s2);
+        *(uint32_t *)acc = z;
+    } else return -1;
+    return 0;
+}

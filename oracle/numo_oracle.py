@@ -44,6 +44,10 @@ lib.numo_copy_bytes.restype = C.c_int
 lib.numo_fill.restype = C.c_int
 lib.numo_bit_binary.restype = C.c_int
 lib.numo_bit_count.restype = C.c_uint64
+lib.numo_cum_run.argtypes = [C.c_int, C.c_int, C.c_int, SZ, C.c_void_p, SSZ, C.c_void_p, SSZ]
+lib.numo_cum_run.restype = C.c_int
+lib.numo_mulsum_run.argtypes = [C.c_int, C.c_int, SZ, C.c_void_p, SSZ, C.c_void_p, SSZ, C.c_void_p]
+lib.numo_mulsum_run.restype = C.c_int
 lib.numo_pow_int.argtypes = [C.c_int, SZ, C.c_void_p, SSZ, C.c_void_p, SSZ, C.c_void_p]
 lib.numo_pow_int.restype = C.c_int
 lib.numo_bit_count.argtypes = [C.c_void_p, SZ, SSZ, C.c_uint64, C.c_int]
@@ -153,6 +157,64 @@ def clip(x, lo=None, hi=None):
     if hi is not None:
         return binary("clip_max", x, hi if not isinstance(hi, np.ndarray) else hi.astype(x.dtype))
     raise ValueError("min and max are not given")
+
+
+def _axes(ndim, axis):
+    if axis is None:
+        return tuple(range(ndim))
+    if isinstance(axis, (int, np.integer)):
+        axis = (axis,)
+    return tuple(sorted(a + ndim if a < 0 else a for a in axis))
+
+
+def cum(op, x, axis=None, nan=False):
+    """x.cumsum / x.cumprod (narray/gen/tmpl/cum.c:12-80): the running value along
+    the given axes taken together in row-major order, all of them by default."""
+    prod = {"cumsum": 0, "cumprod": 1}[op]
+    ax = _axes(x.ndim, axis)
+    keep = tuple(d for d in range(x.ndim) if d not in ax)
+    xt = np.ascontiguousarray(np.transpose(x, keep + ax))
+    n = int(np.prod([x.shape[d] for d in ax])) if ax else 1
+    rows = xt.size // n if n else 0
+    flat = xt.reshape(rows, n) if n else xt.reshape(0, 0)
+    out = np.zeros_like(flat)
+    es = flat.dtype.itemsize
+    for r in range(rows):
+        rc = lib.numo_cum_run(prod, _tcode(flat), 1 if nan else 0, n, C.c_void_p(flat[r].ctypes.data), es,
+                              C.c_void_p(out[r].ctypes.data), es)
+        if rc:
+            raise ValueError("oracle: cum of an unsupported type")
+    res = out.reshape(xt.shape)
+    return np.ascontiguousarray(np.transpose(res, np.argsort(keep + ax)))
+
+
+def mulsum(x, y, axis=None, keepdims=False, nan=False):
+    """x.mulsum(y) (narray/gen/tmpl/accum_binary.c:27-38,62-110): the sum of the
+    products over the given axes, sequentially in row-major order, started from 0.
+    Operands are broadcast and must have one type."""
+    assert x.dtype == y.dtype
+    shape = np.broadcast_shapes(x.shape, y.shape)
+    ax = _axes(len(shape), axis)
+    keep = tuple(d for d in range(len(shape)) if d not in ax)
+    perm = keep + ax
+    xt = np.ascontiguousarray(np.transpose(np.broadcast_to(x, shape), perm))
+    yt = np.ascontiguousarray(np.transpose(np.broadcast_to(y, shape), perm))
+    n = int(np.prod([shape[d] for d in ax])) if ax else 1
+    oshape = tuple(shape[d] for d in keep)
+    rows = int(np.prod(oshape)) if oshape else 1
+    out = np.zeros(rows, dtype=x.dtype)
+    es = x.dtype.itemsize
+    if xt.size:
+        xf, yf = xt.reshape(rows, n), yt.reshape(rows, n)
+        for r in range(rows):
+            rc = lib.numo_mulsum_run(_tcode(xf), 1 if nan else 0, n, C.c_void_p(xf[r].ctypes.data), es,
+                                     C.c_void_p(yf[r].ctypes.data), es, C.c_void_p(out[r:].ctypes.data))
+            if rc:
+                raise ValueError("oracle: mulsum of an unsupported type")
+    res = out.reshape(oshape)
+    if keepdims:
+        res = res.reshape(tuple(1 if d in ax else shape[d] for d in range(len(shape))))
+    return res
 
 
 def _bit_words(nbits):

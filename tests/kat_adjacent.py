@@ -98,6 +98,18 @@ class OracleEngine:
             return OracleArray(self, o.pow_int(np.float64(x), y.a))
         return OracleArray(self, o.binary("pow", float(x), np.ascontiguousarray(y.a), scalar_is_left=True))
 
+    def cum(self, op, x, axis=None, nan=False):
+        return OracleArray(self, self.o.cum(op, x.a, axis=axis, nan=nan))
+
+    def mulsum(self, x, y, axis=None, keepdims=False, nan=False):
+        return OracleArray(self, np.asarray(self.o.mulsum(x.a, y.a, axis=axis, keepdims=keepdims, nan=nan)))
+
+    def mul_sum(self, x, y, axis=None):
+        """(x * y).sum(axis:) as the reference tests write it; exact for the small integers they use"""
+        prod = self.o.binary("mul", np.ascontiguousarray(np.broadcast_to(x.a, np.broadcast_shapes(x.a.shape, y.a.shape))),
+                             np.ascontiguousarray(np.broadcast_to(y.a, np.broadcast_shapes(x.a.shape, y.a.shape))))
+        return OracleArray(self, np.asarray(self.o.reduce("sum", prod, axis=axis)))
+
     def ewcomp(self, op, tname, a, b, nan=False):
         dt = NP[tname]
         ra = a.a.astype(dt) if isinstance(a, OracleArray) else np.array(a, dtype=dt)
@@ -155,6 +167,15 @@ class DeviceEngine:
 
     def ewcomp(self, op, tname, a, b, nan=False):
         return DeviceArray(self, getattr(self.cls(tname), op)(self._u(a), self._u(b), nan=nan))
+
+    def cum(self, op, x, axis=None, nan=False):
+        return DeviceArray(self, getattr(x.a, op)(axis=axis, nan=nan))
+
+    def mulsum(self, x, y, axis=None, keepdims=False, nan=False):
+        return DeviceArray(self, x.a.mulsum(y.a, axis=axis, keepdims=keepdims, nan=nan))
+
+    def mul_sum(self, x, y, axis=None):
+        return DeviceArray(self, (x.a * y.a).sum(axis=axis))
 
 
 # ---------------------------------------------------------------------------
@@ -235,12 +256,109 @@ def case_pow(E, t):
         yield E.pow(deep, E.arr(t, [0.5] * 512).reshape(*([2] * 9))).to_list(), E.pow(deep, 0.5).to_list(), "narray_test.rb:4483"
 
 
+def _running(values, op):
+    out, acc = [], None
+    for v in values:
+        acc = v if acc is None else op(acc, v)
+        out.append(acc)
+    return out
+
+
+def _running_skip_nan(values, op):
+    # narray_test.rb:2876-2888
+    acc = values[0]
+    out = [acc]
+    for y in values[1:]:
+        if acc != acc:
+            acc = y
+        elif y == y:
+            acc = op(acc, y)
+        out.append(acc)
+    return out
+
+
+def case_cum_long_and_views(E, t):
+    # values that keep every partial result exact, so association cannot matter (narray_test.rb:2895-2924)
+    n = 20000
+    adds = [(i % 3) + 1 for i in range(n)]
+    muls = [2 if i % 4 < 2 else 0.5 for i in range(n)]
+    views = [("flat", slice(None)), ("offset 13", slice(13, n)), ("step 2", slice(0, n, 2)), ("reversed", slice(None, None, -1))]
+    a = E.arr(t, adds)
+    for label, sl in views:
+        yield E.cum("cumsum", a.view(sl)).to_list(), _running(adds[sl], lambda x, y: x + y), "narray_test.rb:2913 " + label
+    if t != "int32":
+        b = E.arr(t, muls)
+        for label, sl in views:
+            yield E.cum("cumprod", b.view(sl)).to_list(), _running(muls[sl], lambda x, y: x * y), "narray_test.rb:2921 " + label
+
+
+def case_cum_axis(E, t):
+    rows, cols = 6, 20000
+    adds = [(i % 3) + 1 for i in range(rows * cols)]
+    muls = [2 if i % 4 < 2 else 0.5 for i in range(rows * cols)]
+    a = E.arr(t, adds).reshape(rows, cols)
+    yield E.cum("cumsum", a, axis=1).to_list(), [_running(adds[r * cols:(r + 1) * cols], lambda x, y: x + y) for r in range(rows)], "narray_test.rb:2934"
+    down = [_running([adds[r * cols + c] for r in range(rows)], lambda x, y: x + y) for c in range(cols)]
+    yield E.cum("cumsum", a, axis=0).to_list(), [[down[c][r] for c in range(cols)] for r in range(rows)], "narray_test.rb:2937"
+    b = E.arr(t, muls).reshape(rows, cols)
+    yield E.cum("cumprod", b, axis=1).to_list(), [_running(muls[r * cols:(r + 1) * cols], lambda x, y: x * y) for r in range(rows)], "narray_test.rb:2941"
+
+
+def case_cum_nan(E, t):
+    for n in (64, 20000):
+        for at in (0, 1, n // 2, n - 1):
+            adds = [(i % 3) + 1.0 for i in range(n)]
+            muls = [2.0 if i % 4 < 2 else 0.5 for i in range(n)]
+            adds[at] = NAN
+            muls[at] = NAN
+            lbl = " n=%d at=%d" % (n, at)
+            a, b = E.arr(t, adds), E.arr(t, muls)
+            yield E.cum("cumsum", a).to_list(), _running(adds, lambda x, y: x + y), "narray_test.rb:2956" + lbl
+            yield E.cum("cumsum", a, nan=True).to_list(), _running_skip_nan(adds, lambda x, y: x + y), "narray_test.rb:2957" + lbl
+            yield E.cum("cumprod", b).to_list(), _running(muls, lambda x, y: x * y), "narray_test.rb:2961" + lbl
+            yield E.cum("cumprod", b, nan=True).to_list(), _running_skip_nan(muls, lambda x, y: x * y), "narray_test.rb:2962" + lbl
+
+
+def case_mulsum(E, t):
+    a, b = E.arr(t, [1, 2, 3]), E.arr(t, [2, 3, 4])
+    yield E.mulsum(a, b).to_list(), 1 * 2 + 2 * 3 + 3 * 4, "narray_test.rb:756"
+    if t != "int32":
+        yield E.mulsum(E.arr(t, [NAN, 2, 3]), b, nan=True).to_list(), 0 + 2 * 3 + 3 * 4, "narray_test.rb:764"
+
+    def small(shape):
+        n = 1
+        for v in shape:
+            n *= v
+        return E.arr(t, [i % 4 + 1 for i in range(n)]).reshape(*shape)
+    for shape in ([3], [3, 1], [1, 3], [3, 2], [2, 3], [3, 1, 1], [2, 3, 1], [2, 1, 3], [2, 3, 4]):
+        x = small(shape)
+        for axis in range(-len(shape), len(shape)):
+            yield E.mulsum(x, x, axis=axis).to_list(), E.mul_sum(x, x, axis=axis).to_list(), "narray_test.rb:776 %r axis %d" % (shape, axis)
+    x = small([3, 1])
+    yield E.mulsum(x, x).to_list(), E.mul_sum(x, x).to_list(), "narray_test.rb:782"
+    for shape in ([3, 1], [3, 2], [2, 3], [2, 3, 1], [2, 3, 4]):
+        x = small(shape)
+        two = E.arr(t, [2]).reshape(*([1] * len(shape)))
+        for axis in range(len(shape)):
+            yield E.mulsum(x, two, axis=axis).to_list(), E.mul_sum(x, two, axis=axis).to_list(), "narray_test.rb:790 %r axis %d" % (shape, axis)
+    x = small([6])
+    r = x.view(slice(None, None, -1))
+    yield E.mulsum(r, r, axis=0).to_list(), E.mul_sum(x, x, axis=0).to_list(), "narray_test.rb:797"
+    y = small([3, 2])
+    ry = y.view((slice(None, None, -1), slice(None)))
+    yield E.mulsum(ry, ry, axis=0).to_list(), E.mul_sum(y, y, axis=0).to_list(), "narray_test.rb:799"
+
+
 CASES = [
     ("clip", case_clip, ("sfloat", "dfloat", "int32")),
     ("clip_nan_bounds", case_clip_nan_bounds, ("sfloat", "dfloat")),
     ("clip_raises", case_clip_raises, ("sfloat", "dfloat", "int32")),
     ("ewcomp", case_ewcomp, ("sfloat", "dfloat", "int32")),
     ("pow", case_pow, ("sfloat", "dfloat", "int32")),
+    ("cum_long_and_views", case_cum_long_and_views, ("sfloat", "dfloat", "int32")),
+    ("cum_axis", case_cum_axis, ("dfloat",)),
+    ("cum_nan", case_cum_nan, ("dfloat", "sfloat")),
+    ("mulsum", case_mulsum, ("sfloat", "dfloat", "int32")),
 ]
 
 

@@ -137,3 +137,168 @@ def test_int32_pow_parity_and_type_rules():
     r = x ** y
     assert isinstance(r, cumo_amd.SFloat)
     assert_ulp(r.to_numpy(), oracle.binary("pow", hx.astype(np.float32), np.full((37, 65), 2.0, dtype=np.float32)), 1)
+
+
+def _cum_close(got, want_exact, scale, n, dt, what):
+    """Float scans against the exactly accumulated value: rel 1e-5*log2(n) for SFloat,
+    1e-12*log2(n) for DFloat, of the running sum of magnitudes (the bar the parity
+    contract sets for float reductions)."""
+    tol = (1e-5 if dt == np.float32 else 1e-12) * max(1.0, np.log2(max(n, 2)))
+    err = np.abs(got.astype(np.float64) - want_exact)
+    bad = err > tol * np.maximum(scale, 1e-300)
+    assert not bad.any(), (what, float(err.max()), int(bad.sum()))
+
+
+@pytest.mark.parametrize("tname,dt", ALL)
+def test_cumsum_cumprod_parity(tname, dt):
+    cls = cls_of(tname)
+    rng = np.random.default_rng(51)
+    for shape, axes in [((5,), [None]), ((2049,), [None]), ((70001,), [None]), ((300001,), [None]), ((37, 129), [None, 0, 1, -1]),
+                        ((3, 5, 130), [None, 0, 1, 2, (1, 2), (0, 2), (0, 1)]), ((700, 300), [0, 1]), ((2, 70000), [1])]:
+        if dt == np.int32:
+            h = rng.integers(-5, 6, size=shape).astype(dt)
+        else:
+            h = rng.standard_normal(shape).astype(dt)
+        d = cls.cast(h)
+        for ax in axes:
+            got = d.cumsum(axis=ax).to_numpy()
+            want = oracle.cum("cumsum", h, axis=ax)
+            if dt == np.int32:
+                assert_bits_equal(got, want, (shape, ax))
+            else:
+                axs = tuple(range(h.ndim)) if ax is None else ((ax,) if isinstance(ax, int) else ax)
+                n = int(np.prod([shape[a] for a in axs]))
+                exact = oracle.cum("cumsum", h.astype(np.float64), axis=ax) if dt == np.float32 else None
+                if exact is None:
+                    exact = np.asarray(oracle.cum("cumsum", h.astype(np.longdouble).astype(np.float64), axis=ax))
+                scale = oracle.cum("cumsum", np.abs(h).astype(np.float64), axis=ax)
+                _cum_close(got, exact, scale, n, dt, (shape, ax, "cumsum"))
+                # and the oracle's own sequential answer lies within the same bar of it
+                _cum_close(want, exact, scale, n, dt, (shape, ax, "oracle cumsum"))
+        # views: strided, reversed, transposed
+        if len(shape) == 1 and shape[0] > 100:
+            for sl in (slice(3, None, 2), slice(None, None, -1), slice(7, shape[0] - 5)):
+                got = d[sl].cumsum().to_numpy()
+                hv = np.ascontiguousarray(h[sl])
+                if dt == np.int32:
+                    assert_bits_equal(got, oracle.cum("cumsum", hv), (shape, sl))
+                else:
+                    _cum_close(got, oracle.cum("cumsum", hv.astype(np.float64)), oracle.cum("cumsum", np.abs(hv).astype(np.float64)), hv.size, dt, (shape, sl))
+        if len(shape) == 2:
+            got = d.transpose().cumsum(axis=1).to_numpy()
+            hv = np.ascontiguousarray(h.T)
+            if dt == np.int32:
+                assert_bits_equal(got, oracle.cum("cumsum", hv, axis=1))
+            else:
+                _cum_close(got, oracle.cum("cumsum", hv.astype(np.float64), axis=1), oracle.cum("cumsum", np.abs(hv).astype(np.float64), axis=1),
+                           hv.shape[1], dt, (shape, "T"))
+    # cumprod: powers of two stay exact in every order
+    h = np.where(rng.integers(0, 2, size=(33, 200)) == 0, 2.0, 0.5).astype(dt if dt != np.int32 else np.float32)
+    if dt != np.int32:
+        assert_bits_equal(cls.cast(h).cumprod(axis=1).to_numpy(), oracle.cum("cumprod", h, axis=1))
+        assert_bits_equal(cls.cast(h).cumprod(axis=0).to_numpy(), oracle.cum("cumprod", h, axis=0))
+    else:
+        hi = rng.integers(-3, 4, size=(33, 40)).astype(np.int32)
+        assert_bits_equal(cls.cast(hi).cumprod(axis=1).to_numpy(), oracle.cum("cumprod", hi, axis=1))   # wraps identically
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_cum_nan_forms_on_random_placements(tname, dt):
+    cls = cls_of(tname)
+    rng = np.random.default_rng(52)
+    h = rng.integers(-4, 5, size=(9, 5000)).astype(dt)      # small integers: exact in any order
+    h[rng.integers(0, 9, 300), rng.integers(0, 5000, 300)] = np.nan
+    h[3, :40] = np.nan                                         # a run that starts with NaN
+    h[5, :] = np.nan                                           # and one that is nothing but NaN
+    d = cls.cast(h)
+    for ax in (1, 0, None):
+        assert_bits_equal(d.cumsum(axis=ax, nan=True).to_numpy(), oracle.cum("cumsum", h, axis=ax, nan=True), ("nan", ax))
+        assert_bits_equal(d.cumsum(axis=ax).to_numpy(), oracle.cum("cumsum", h, axis=ax), ("plain", ax))
+
+
+@pytest.mark.parametrize("tname,dt", ALL)
+def test_mulsum_parity(tname, dt):
+    cls = cls_of(tname)
+    rng = np.random.default_rng(53)
+
+    def make(shape):
+        if dt == np.int32:
+            return rng.integers(-1000, 1000, size=shape).astype(dt)
+        return rng.standard_normal(shape).astype(dt)
+
+    def check(got, hx, hy, axis, what, nan=False):
+        want = np.asarray(oracle.mulsum(hx, hy, axis=axis, nan=nan))
+        got = np.asarray(got)
+        assert got.shape == want.shape, (what, got.shape, want.shape)
+        if dt == np.int32:
+            assert_bits_equal(got.astype(np.int32), want.astype(np.int32), what)
+            return
+        bx = np.broadcast_to(hx, np.broadcast_shapes(hx.shape, hy.shape)).astype(np.float64)
+        by = np.broadcast_to(hy, bx.shape).astype(np.float64)
+        if nan:
+            ok = ~(np.isnan(bx) | np.isnan(by))
+            bx, by = np.where(ok, bx, 0), np.where(ok, by, 0)
+        exact = (bx * by).sum(axis=axis)
+        scale = np.abs(bx * by).sum(axis=axis)
+        n = bx.size // max(1, np.asarray(exact).size)
+        tol = (1e-5 if dt == np.float32 else 1e-12) * max(1.0, np.log2(max(n, 2)))
+        assert (np.abs(got.astype(np.float64) - exact) <= tol * np.maximum(scale, 1e-300)).all(), what
+        assert (np.abs(want.astype(np.float64) - exact) <= tol * np.maximum(scale, 1e-300) * 4).all(), (what, "oracle")
+
+    for n in (1, 7, 1000, 4096, 100003, (1 << 22) + 3):
+        hx, hy = make((n,)), make((n,))
+        x, y = cls.cast(hx), cls.cast(hy)
+        check(x.mulsum(y).to_numpy(), hx, hy, None, ("dot", n))
+        if n > 100:
+            check(x[1::2].mulsum(y[:n // 2]).to_numpy(), np.ascontiguousarray(hx[1::2]), np.ascontiguousarray(hy[:n // 2]), None, ("strided dot", n))
+            check(x[::-1].mulsum(y).to_numpy(), np.ascontiguousarray(hx[::-1]), hy, None, ("reversed dot", n))
+    hx, hy = make((37, 65)), make((37, 65))
+    x, y = cls.cast(hx), cls.cast(hy)
+    for ax in (None, 0, 1, -1):
+        check(x.mulsum(y, axis=ax).to_numpy(), hx, hy, ax, ("matrix", ax))
+    check(x.mulsum(y[0], axis=1).to_numpy(), hx, hy[0], 1, "row vector operand")
+    check(x.transpose().mulsum(y.transpose(), axis=0).to_numpy(), np.ascontiguousarray(hx.T), np.ascontiguousarray(hy.T), 0, "transposed")
+    assert x.mulsum(y, axis=1, keepdims=True).to_numpy().shape == (37, 1)
+    # more inner runs than are launched one by one: the products go through the reduction engine
+    hx, hy = make((3000, 40)), make((3000, 40))
+    check(cls.cast(hx).mulsum(cls.cast(hy), axis=1).to_numpy(), hx, hy, 1, "3000 runs")
+    # no reduced dimension left after broadcasting rules: the elementwise form
+    hx, hy = make((5, 1)), make((5, 1))
+    check(cls.cast(hx).mulsum(cls.cast(hy), axis=1).to_numpy(), hx, hy, 1, "runs of one element")
+    if dt != np.int32:
+        hx, hy = make((4, 5000)), make((4, 5000))
+        hx[rng.integers(0, 4, 50), rng.integers(0, 5000, 50)] = np.nan
+        hy[rng.integers(0, 4, 50), rng.integers(0, 5000, 50)] = np.nan
+        check(cls.cast(hx).mulsum(cls.cast(hy), axis=1, nan=True).to_numpy(), hx, hy, 1, "nan: true", nan=True)
+        assert np.isnan(cls.cast(hx).mulsum(cls.cast(hy), axis=1).to_numpy()).all()
+    # mixed types move to the higher one
+    import cumo_amd
+    r = cumo_amd.Int32.cast(np.array([1, 2, 3], dtype=np.int32)).mulsum(cumo_amd.DFloat.cast(np.array([0.5, 0.25, 2.0])))
+    assert isinstance(r, cumo_amd.DFloat) and float(r) == 0.5 + 0.5 + 6.0
+
+
+def test_cum_and_mulsum_launchers_called_directly():
+    """The reference's per-run symbols: narray/gen/tmpl/cum.c:3, accum_binary.c:4-5."""
+    import ctypes as C
+    from cumo_amd import _lib
+    from test_gpu_raw_abi import dev, fetch, free
+    rng = np.random.default_rng(54)
+    n = 50001
+    h = rng.integers(-3, 4, size=2 * n + 5).astype(np.float32)
+    px = dev(h)
+    pz = dev(np.full(n, -7.0, dtype=np.float32))
+    f = _lib.fn("cumo_sfloat_cumsum_kernel_launch", C.c_int, [C.c_void_p, C.c_void_p, C.c_ssize_t, C.c_ssize_t, C.c_uint64])
+    # every other element, starting at element 3, written backwards
+    rc = _lib.call(f, px + 12, pz + 4 * (n - 1), 8, -4, n)
+    assert rc == 0
+    got = fetch(pz, (n,), np.float32)
+    assert_bits_equal(got[::-1], np.cumsum(h[3:3 + 2 * n:2].astype(np.float64)).astype(np.float32))
+    # mulsum adds onto what the result holds
+    py = dev(np.full(n, 2.0, dtype=np.float32))
+    pacc = dev(np.array([100.0], dtype=np.float32))
+    g = _lib.fn("cumo_sfloat_mulsum_reduce_kernel_launch", None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_ssize_t, C.c_ssize_t, C.c_uint64])
+    _lib.call(g, px + 12, py, pacc, 8, 4, n)
+    assert float(fetch(pacc, (1,), np.float32)[0]) == 100.0 + 2.0 * float(h[3:3 + 2 * n:2].astype(np.float64).sum())
+    _lib.call(g, px, py, pacc, 4, 0, 0)                       # an empty run adds nothing
+    assert float(fetch(pacc, (1,), np.float32)[0]) == 100.0 + 2.0 * float(h[3:3 + 2 * n:2].astype(np.float64).sum())
+    free(px, py, pz, pacc)
