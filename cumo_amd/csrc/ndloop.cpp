@@ -1309,6 +1309,13 @@ int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int red
             cumo_hip::report_hip_error((hipError_t)st, "cumsum/cumprod launch");
             rc = CUMO_HIP_ERROR_RUNTIME;
         }
+    } else if (runs.nouter > 0 && s_in != es && runs.ostep_in[runs.nouter - 1] == es && runs.ostep_out[runs.nouter - 1] == es &&
+               runs.oshape[runs.nouter - 1] >= 16) {
+        // the runs lie across memory: lanes along the contiguous dimension
+        const uint64_t cols = runs.oshape[runs.nouter - 1];
+        --runs.nouter;
+        runs.rows /= cols;
+        cumo_hip_scan_cols_kernel_launch(x->type, prod, use_nan ? 1 : 0, &runs, cols);
     } else {
         cumo_hip_scan_rows_kernel_launch(x->type, prod, use_nan ? 1 : 0, &runs);
     }

@@ -241,6 +241,186 @@ __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const char* in, 
     scan_store<T>(out, s_out, first, cnt, v);
 }
 
+// ---- runs that lie across memory (the scan goes down the rows of a matrix) ------
+// Lanes sit along the dimension that is contiguous in memory and each lane walks
+// its VEC columns down the run, so every load is coalesced across the wave. A run
+// is cut into segments to fill the device: phase 0 leaves each segment's total per
+// column, phase 1 turns the totals into running totals, phase 2 scans each segment
+// from the running total before it. With enough columns there is one segment and
+// only phase 2 runs (one read, one write).
+struct ScanColsParams {
+    int nouter;               // dimensions outside the run and the column dimension
+    uint64_t planes, cols, n; // planes = product of those dimensions
+    uint64_t oshape[CUMO_NA_MAX_DIMENSION];
+    int64_t ostep_in[CUMO_NA_MAX_DIMENSION], ostep_out[CUMO_NA_MAX_DIMENSION];
+    int64_t s_in, s_out;      // byte step along the run
+    uint64_t seg_len, n_seg;
+    int tx_bits;              // 2^tx_bits lanes along the columns, the rest of the block along segments
+    const char* in;
+    char* out;
+};
+
+template <class T, int VEC>
+__device__ __forceinline__ void scan_cols_load(const char* p, T (&v)[VEC]) {
+    if constexpr (VEC * sizeof(T) == 16) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        union { u4 q; T t[VEC]; } u;
+        u.q = *reinterpret_cast<const u4*>(p);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = u.t[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = reinterpret_cast<const T*>(p)[j];
+    }
+}
+template <class T, int VEC>
+__device__ __forceinline__ void scan_cols_store(char* p, const T (&v)[VEC]) {
+    if constexpr (VEC * sizeof(T) == 16) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        union { u4 q; T t[VEC]; } u;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) u.t[j] = v[j];
+        *reinterpret_cast<u4*>(p) = u.q;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) reinterpret_cast<T*>(p)[j] = v[j];
+    }
+}
+
+// PHASE 0: totals[(plane * n_seg + seg) * cols + col] = total of the segment.
+// PHASE 2: scan the segment, starting from totals[.. seg - 1 ..] when seg > 0.
+template <class T, class Op, int VEC, int PHASE>
+__global__ __launch_bounds__(kScanBlock) void scan_cols_kernel(ScanColsParams p, T* totals) {
+    constexpr int UNR = 8;
+    const unsigned TX = 1u << p.tx_bits, TY = (unsigned)kScanBlock >> p.tx_bits;
+    const unsigned tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> p.tx_bits;
+    const uint64_t col_groups = p.cols / VEC;
+    const uint64_t strips = (col_groups + TX - 1) / TX;
+    const uint64_t seg_blocks = (p.n_seg + TY - 1) / TY;
+    const uint64_t n_blocks = strips * seg_blocks * p.planes;
+    for (uint64_t b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+        const uint64_t strip = b % strips;
+        const uint64_t sb = (b / strips) % seg_blocks;
+        const uint64_t plane = b / (strips * seg_blocks);
+        const uint64_t cg = strip * TX + tx;
+        const uint64_t seg = sb * TY + ty;
+        if (cg >= col_groups || seg >= p.n_seg) continue;
+        int64_t oi = 0, oo = 0;
+        uint64_t r = plane;
+        for (int d = p.nouter - 1; d >= 0; --d) {
+            const uint64_t m = p.oshape[d];
+            const uint64_t q = r / m;
+            const int64_t k = (int64_t)(r - q * m);
+            r = q;
+            oi += k * p.ostep_in[d];
+            oo += k * p.ostep_out[d];
+        }
+        const uint64_t col = cg * VEC;
+        const uint64_t begin = seg * p.seg_len;
+        uint64_t end = begin + p.seg_len;
+        if (end > p.n) end = p.n;
+        const char* src = p.in + oi + (int64_t)col * (int64_t)sizeof(T);
+        char* dst = p.out + oo + (int64_t)col * (int64_t)sizeof(T);
+        T acc[VEC];
+        bool has = false;
+        if (PHASE == 2 && seg > 0) {
+            scan_cols_load<T, VEC>(reinterpret_cast<const char*>(totals + (plane * p.n_seg + seg - 1) * p.cols + col), acc);
+            has = true;
+        }
+        uint64_t i = begin;
+        for (; i + UNR <= end; i += UNR) {
+            T v[UNR][VEC];
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) scan_cols_load<T, VEC>(src + (int64_t)(i + u) * p.s_in, v[u]);
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = has ? Op::apply(acc[j], v[u][j]) : v[u][j];
+                has = true;
+                if (PHASE == 2) scan_cols_store<T, VEC>(dst + (int64_t)(i + u) * p.s_out, acc);
+            }
+        }
+        for (; i < end; ++i) {
+            T v[VEC];
+            scan_cols_load<T, VEC>(src + (int64_t)i * p.s_in, v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = has ? Op::apply(acc[j], v[j]) : v[j];
+            has = true;
+            if (PHASE == 2) scan_cols_store<T, VEC>(dst + (int64_t)i * p.s_out, acc);
+        }
+        if (PHASE == 0) scan_cols_store<T, VEC>(reinterpret_cast<char*>(totals + (plane * p.n_seg + seg) * p.cols + col), acc);
+    }
+}
+
+// phase 1: per plane and column, the running total over the segments, in place
+template <class T, class Op>
+__global__ __launch_bounds__(kScanBlock) void scan_cols_totals_kernel(T* totals, uint64_t planes, uint64_t n_seg, uint64_t cols) {
+    const uint64_t items = planes * cols;
+    for (uint64_t it = (uint64_t)blockIdx.x * kScanBlock + threadIdx.x; it < items; it += (uint64_t)gridDim.x * kScanBlock) {
+        const uint64_t plane = it / cols, col = it - plane * cols;
+        T* t = totals + plane * n_seg * cols + col;
+        T acc = t[0];
+        for (uint64_t s = 1; s < n_seg; ++s) {
+            acc = Op::apply(acc, t[s * cols]);
+            t[s * cols] = acc;
+        }
+    }
+}
+
+template <class T, class Op, int VEC>
+void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
+    const uint64_t col_groups = p.cols / VEC;
+    int txb = 0;
+    while (txb < 8 && (1ull << txb) < col_groups) ++txb;
+    p.tx_bits = txb;
+    const uint64_t TX = 1ull << txb, TY = (uint64_t)kScanBlock >> txb;
+    // segments: enough threads for eight blocks on every compute unit, at least 16 rows each
+    const uint64_t want_threads = 256ull * 8 * kScanBlock;
+    uint64_t n_seg = (want_threads + col_groups * p.planes - 1) / (col_groups * p.planes);
+    const uint64_t max_seg = (p.n + 15) / 16;
+    if (n_seg > max_seg) n_seg = max_seg;
+    if (n_seg > 1024) n_seg = 1024;
+    if (n_seg < 1) n_seg = 1;
+    p.seg_len = (p.n + n_seg - 1) / n_seg;
+    p.n_seg = (p.n + p.seg_len - 1) / p.seg_len;
+    const uint64_t strips = (col_groups + TX - 1) / TX;
+    uint64_t grid = strips * ((p.n_seg + TY - 1) / TY) * p.planes;
+    if (grid > 0x7fffffffull) grid = 0x7fffffffull;
+    const dim3 g((unsigned)grid), b(kScanBlock);
+    if (p.n_seg == 1) {
+        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2>), g, b, 0, stream, p, (T*)nullptr);
+        return;
+    }
+    T* totals = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * p.planes * p.n_seg * p.cols));
+    if (!totals) return;
+    hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 0>), g, b, 0, stream, p, totals);
+    uint64_t g1 = (p.planes * p.cols + kScanBlock - 1) / kScanBlock;
+    if (g1 > 65536) g1 = 65536;
+    hipLaunchKernelGGL((scan_cols_totals_kernel<T, Op>), dim3((unsigned)g1), b, 0, stream, totals, p.planes, p.n_seg, p.cols);
+    hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2>), g, b, 0, stream, p, totals);
+    cumo_cuda_runtime_free(reinterpret_cast<char*>(totals));
+}
+
+template <class T, class Op>
+void scan_cols_launch(ScanColsParams& p, hipStream_t stream) {
+    constexpr int V = 16 / (int)sizeof(T);
+    bool vec = (p.cols % V) == 0 && ((uintptr_t)p.in % 16) == 0 && ((uintptr_t)p.out % 16) == 0 && (p.s_in % 16) == 0 && (p.s_out % 16) == 0;
+    for (int d = 0; d < p.nouter && vec; ++d) vec = (p.ostep_in[d] % 16) == 0 && (p.ostep_out[d] % 16) == 0;
+    if (vec) scan_cols_launch_vec<T, Op, V>(p, stream);
+    else scan_cols_launch_vec<T, Op, 1>(p, stream);
+}
+
+template <class T>
+void scan_cols_dispatch(int prod, int nan, ScanColsParams& p, hipStream_t stream) {
+    if (prod) {
+        if (nan) scan_cols_launch<T, ScanOp<T, 1, true> >(p, stream);
+        else scan_cols_launch<T, ScanOp<T, 1, false> >(p, stream);
+    } else {
+        if (nan) scan_cols_launch<T, ScanOp<T, 0, true> >(p, stream);
+        else scan_cols_launch<T, ScanOp<T, 0, false> >(p, stream);
+    }
+}
+
 template <class T, class Op>
 void scan_rows_launch(const ScanRowsParams& p, hipStream_t stream) {
     if (p.rows == 0 || p.n == 0) return;
@@ -340,6 +520,33 @@ void cumo_hip_scan_rows_kernel_launch(int type, int prod, int nan, const cumo_hi
         case 0: scan_rows_dispatch<float>(prod, nan, p, stream); break;
         case 1: scan_rows_dispatch<double>(prod, nan, p, stream); break;
         case 2: scan_rows_dispatch<int32_t>(prod, 0, p, stream); break;
+        default: report_error(CUMO_HIP_ERROR_TYPE, 0, "scan: element type is not SFloat, DFloat or Int32"); return;
+    }
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+void cumo_hip_scan_cols_kernel_launch(int type, int prod, int nan, const cumo_hip_scan_rows_t* d, uint64_t cols) {
+    if (!d || d->rows == 0 || d->n == 0 || cols == 0) return;
+    ScanColsParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.nouter = d->nouter;
+    p.planes = d->rows;
+    p.cols = cols;
+    p.n = d->n;
+    for (int k = 0; k < d->nouter && k < CUMO_NA_MAX_DIMENSION; ++k) {
+        p.oshape[k] = d->oshape[k];
+        p.ostep_in[k] = d->ostep_in[k];
+        p.ostep_out[k] = d->ostep_out[k];
+    }
+    p.s_in = d->s_in;
+    p.s_out = d->s_out;
+    p.in = d->in;
+    p.out = d->out;
+    hipStream_t stream = current_stream();
+    switch (type) {
+        case 0: scan_cols_dispatch<float>(prod, nan, p, stream); break;
+        case 1: scan_cols_dispatch<double>(prod, nan, p, stream); break;
+        case 2: scan_cols_dispatch<int32_t>(prod, 0, p, stream); break;
         default: report_error(CUMO_HIP_ERROR_TYPE, 0, "scan: element type is not SFloat, DFloat or Int32"); return;
     }
     cumo_cuda_runtime_check_kernel_launch();

@@ -417,6 +417,10 @@ typedef struct {
     char*    out;
 } cumo_hip_scan_rows_t;
 void cumo_hip_scan_rows_kernel_launch(int type, int prod, int nan, const cumo_hip_scan_rows_t* runs);
+/* The same for runs that lie across memory: `cols` neighbouring runs start one
+ * element apart (the columns of a matrix scanned down its rows); runs->rows counts
+ * the groups of `cols` runs and oshape / ostep_* decompose the group number. */
+void cumo_hip_scan_cols_kernel_launch(int type, int prod, int nan, const cumo_hip_scan_rows_t* runs, uint64_t cols);
 
 /* The stream every launcher and the pool use from this host thread. The
  * reference only ever uses the default stream (cuda/memory_pool.cpp:43-44). */
