@@ -247,6 +247,75 @@ void launch_count(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, ssize_t s1, size_t* i
     cumo_cuda_runtime_check_kernel_launch();
 }
 
+// count_true / count_false along axes, every output in one launch. A work item is
+// one run of bits (the innermost reduced dimension) of one output; a wave takes an
+// item, its lanes share the run (whole masked words when the run is contiguous,
+// single bits otherwise) and the wave's total is added to the output's counter.
+// The counters are integers, so the order of the additions cannot show.
+struct BitCountNd {
+    int out_ndim, red_ndim;
+    uint64_t out_total, red_outer, n_last;
+    uint64_t out_shape[CUMO_NA_MAX_DIMENSION], red_shape[CUMO_NA_MAX_DIMENSION];
+    int64_t in_out_step[CUMO_NA_MAX_DIMENSION], in_red_step[CUMO_NA_MAX_DIMENSION];  // bits
+    int64_t out_step[CUMO_NA_MAX_DIMENSION];                                         // bytes
+    const CUMO_BIT_DIGIT* in;
+    uint64_t pos;
+    char* out;
+};
+
+template <bool COUNT_FALSE>
+__global__ __launch_bounds__(kBlock) void bit_count_nd_kernel(BitCountNd p) {
+    const unsigned lane = threadIdx.x & 63;
+    const uint64_t wave0 = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+    const uint64_t n_waves = ((uint64_t)gridDim.x * kBlock) >> 6;
+    const uint64_t items = p.out_total * p.red_outer;
+    const int64_t s_last = p.red_ndim > 0 ? p.in_red_step[p.red_ndim - 1] : 0;
+    for (uint64_t item = wave0; item < items; item += n_waves) {
+        uint64_t o = item / p.red_outer, r = item - o * p.red_outer;
+        int64_t bit = (int64_t)p.pos, ooff = 0;
+        for (int d = p.out_ndim - 1; d >= 0; --d) {
+            const uint64_t m = p.out_shape[d];
+            const uint64_t q = o / m;
+            const int64_t k = (int64_t)(o - q * m);
+            o = q;
+            bit += k * p.in_out_step[d];
+            ooff += k * p.out_step[d];
+        }
+        for (int d = p.red_ndim - 2; d >= 0; --d) {
+            const uint64_t m = p.red_shape[d];
+            const uint64_t q = r / m;
+            bit += (int64_t)(r - q * m) * p.in_red_step[d];
+            r = q;
+        }
+        uint64_t c = 0;
+        if (s_last == 1) {
+            const uint64_t p1 = (uint64_t)bit, endbit = p1 + p.n_last;
+            const uint64_t w0 = p1 >> 5, w1 = (endbit + 31) >> 5;
+            for (uint64_t w = w0 + lane; w < w1; w += 64) {
+                uint32_t x = p.in[w];
+                if (COUNT_FALSE) x = ~x;
+                const unsigned lo = (w == w0) ? (unsigned)(p1 & 31) : 0u;
+                const unsigned hi = ((w + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (w << 5));
+                x &= low_bits(hi) & ~low_bits(lo);
+                c += (uint64_t)__popc(x);
+            }
+        } else {
+            for (uint64_t i = lane; i < p.n_last; i += 64) {
+                const uint64_t q = (uint64_t)(bit + (int64_t)i * s_last);
+                const uint32_t b = (p.in[q >> 5] >> (q & 31)) & 1u;
+                c += COUNT_FALSE ? (b ^ 1u) : b;
+            }
+        }
+        for (unsigned d = 32; d > 0; d >>= 1) {
+            const uint32_t lo = __shfl_down((uint32_t)c, d);
+            const uint32_t hi = __shfl_down((uint32_t)(c >> 32), d);
+            c += ((uint64_t)hi << 32) | lo;
+        }
+        if (lane == 0 && c) atomicAdd(reinterpret_cast<unsigned long long*>(p.out + ooff), (unsigned long long)c);
+    }
+}
+
+
 }  // namespace
 
 #define CUMO_DEF_BIT_BINARY(name, OP)                                                                                         \
@@ -305,3 +374,43 @@ CUMO_DEF_BIT_COUNT(count_false, true)
 CUMO_DEF_STORE_BIT(sfloat, float)
 CUMO_DEF_STORE_BIT(dfloat, double)
 CUMO_DEF_STORE_BIT(int32, int32_t)
+
+extern "C" void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* d) {
+    if (!d) return;
+    BitCountNd p;
+    std::memset(&p, 0, sizeof(p));
+    p.out_ndim = d->out_ndim;
+    p.red_ndim = d->red_ndim;
+    p.out_total = 1;
+    p.red_outer = 1;
+    for (int k = 0; k < d->out_ndim; ++k) {
+        p.out_shape[k] = d->out_shape[k];
+        p.in_out_step[k] = d->in_out_step[k];
+        p.out_step[k] = d->out_step[k];
+        p.out_total *= d->out_shape[k];
+    }
+    for (int k = 0; k < d->red_ndim; ++k) {
+        p.red_shape[k] = d->red_shape[k];
+        p.in_red_step[k] = d->in_red_step[k];
+        if (k < d->red_ndim - 1) p.red_outer *= d->red_shape[k];
+    }
+    p.n_last = d->red_ndim > 0 ? d->red_shape[d->red_ndim - 1] : 1;
+    if (d->red_ndim == 0) {
+        // nothing is reduced: every element is a run of one bit
+        p.red_ndim = 1;
+        p.red_shape[0] = 1;
+        p.in_red_step[0] = 1;
+    }
+    p.in = d->in;
+    p.pos = d->pos;
+    p.out = d->out;
+    const uint64_t items = p.out_total * p.red_outer;
+    if (items == 0 || p.n_last == 0) return;
+    uint64_t grid = (items * 64 + kBlock - 1) / kBlock;
+    if (grid > 256u * 32u) grid = 256u * 32u;
+    if (d->count_false)
+        hipLaunchKernelGGL((bit_count_nd_kernel<true>), dim3((unsigned)grid), dim3(kBlock), 0, current_stream(), p);
+    else
+        hipLaunchKernelGGL((bit_count_nd_kernel<false>), dim3((unsigned)grid), dim3(kBlock), 0, current_stream(), p);
+    cumo_cuda_runtime_check_kernel_launch();
+}

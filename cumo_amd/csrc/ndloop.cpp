@@ -800,7 +800,34 @@ void count_walk(const LP* lp, int level, size_t pos, char* optr, bool count_fals
     for (size_t i = 0; i < lp->n[level]; i++)
         count_walk(lp, level + 1, pos + (size_t)((ssize_t)i * in.step[level]), optr + (ssize_t)i * out.step[level], count_false);
 }
-void iter_bit_count(LP* lp) { count_walk(lp, 0, lp->args[0].bitpos, lp->args[1].ptr, ((CountOpt*)lp->opt_ptr)->count_false); }
+void iter_bit_count(LP* lp) {
+    const bool count_false = ((CountOpt*)lp->opt_ptr)->count_false;
+    const int nkeep = lp->ndim - lp->reduce_dim;
+    if (nkeep == 0 && lp->reduce_dim == 1) {
+        // one run into one counter: the reference's run launcher, whole device on it
+        count_walk(lp, 0, lp->args[0].bitpos, lp->args[1].ptr, count_false);
+        return;
+    }
+    // every output in one launch instead of the reference's walk over them on the host
+    cumo_hip_bit_count_nd_t d;
+    std::memset(&d, 0, sizeof(d));
+    d.out_ndim = nkeep;
+    d.red_ndim = lp->reduce_dim;
+    for (int k = 0; k < nkeep; ++k) {
+        d.out_shape[k] = lp->n[k];
+        d.in_out_step[k] = lp->args[0].step[k];
+        d.out_step[k] = lp->args[1].step[k];
+    }
+    for (int k = 0; k < lp->reduce_dim; ++k) {
+        d.red_shape[k] = lp->n[nkeep + k];
+        d.in_red_step[k] = lp->args[0].step[nkeep + k];
+    }
+    d.in = (CUMO_BIT_DIGIT*)lp->args[0].ptr;
+    d.pos = lp->args[0].bitpos;
+    d.out = lp->args[1].ptr;
+    d.count_false = count_false ? 1 : 0;
+    cumo_hip_bit_count_nd_kernel_launch(&d);
+}
 
 
 // ---- pow, maximum/minimum, clip (gen/tmpl/pow.c, ewcomp.c, clip.c) ---------------

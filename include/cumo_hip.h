@@ -402,6 +402,23 @@ void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler);
  * NULL, receives a pointer to a thread-local string. */
 int cumo_hip_last_error(const char** message);
 
+/* count_true / count_false along axes in one launch (no counterpart in the
+ * reference, whose ndloop walks every output on the host and launches one run at a
+ * time, narray/ndloop.c:1569-1613 under gen/tmpl_bit/bit_count.c:9-36). The loop is
+ * given as kept dimensions then reduced dimensions; input steps and pos are in bits,
+ * output steps in bytes; the counts are ADDED onto the uint64 results. */
+typedef struct {
+    int      out_ndim, red_ndim;
+    size_t   out_shape[CUMO_NA_MAX_DIMENSION], red_shape[CUMO_NA_MAX_DIMENSION];
+    ssize_t  in_out_step[CUMO_NA_MAX_DIMENSION], in_red_step[CUMO_NA_MAX_DIMENSION];
+    ssize_t  out_step[CUMO_NA_MAX_DIMENSION];
+    CUMO_BIT_DIGIT* in;
+    size_t   pos;
+    char*    out;
+    int      count_false;
+} cumo_hip_bit_count_nd_t;
+void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* counts);
+
 /* Many scan runs in one launch (no counterpart in the reference, which calls the
  * run launcher once per run from a loop on the host, narray/gen/tmpl/cum.c:12-46).
  * Run r starts at in + sum_k i_k * ostep_in[k] where (i_0 .. i_{nouter-1}) is r

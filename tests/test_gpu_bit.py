@@ -96,3 +96,29 @@ def test_compare_then_count_matches_popcount():
     nums = mask._store_into(cumo_amd.Int32)
     assert (nums.to_numpy() == (h > 0.5)).all()
     assert (mask._store_into(cumo_amd.DFloat).to_numpy() == oracle.store_bit(np.float64, (h > 0.5).astype(np.uint8))).all()
+
+
+def test_count_along_axes_in_one_launch_matches_numpy():
+    """Counts along axes go through one launch for all outputs; every layout of the
+    kept and the reduced dimensions against numpy's sums of the same bits."""
+    import cumo_amd
+    rng = np.random.default_rng(77)
+    for shape in [(512, 777), (3, 5, 130), (64, 64), (7, 1, 33), (2, 3, 4, 65)]:
+        h = rng.integers(0, 2, size=shape).astype(np.uint8)
+        b = cumo_amd.Bit.cast(h)
+        nd = len(shape)
+        axes = [None] + list(range(nd)) + [-1] + ([(0, nd - 1)] if nd > 2 else []) + ([(0, 1)] if nd > 2 else [])
+        for ax in axes:
+            want = h.sum(axis=ax, dtype=np.uint64)
+            assert (np.asarray(b.count_true(axis=ax).to_numpy()) == want).all(), (shape, ax)
+            total = np.prod([shape[a] for a in (range(nd) if ax is None else ([ax] if isinstance(ax, int) else ax))])
+            assert (np.asarray(b.count_false(axis=ax).to_numpy()) == total - want).all(), (shape, ax, "false")
+        assert b.count_true(axis=nd - 1, keepdims=True).to_numpy().shape == shape[:-1] + (1,)
+        if nd == 2:
+            # views: rows reversed, every third column, a window that starts inside a word, the transpose
+            for key in ((slice(None, None, -1), slice(None)), (slice(None), slice(1, None, 3)), (slice(5, 50), slice(7, 60)),
+                        (slice(None), slice(None, None, -1))):
+                for ax in (0, 1):
+                    assert (np.asarray(b[key].count_true(axis=ax).to_numpy()) == h[key].sum(axis=ax, dtype=np.uint64)).all(), (shape, key, ax)
+            for ax in (0, 1):
+                assert (np.asarray(b.transpose().count_true(axis=ax).to_numpy()) == h.T.sum(axis=ax, dtype=np.uint64)).all()
