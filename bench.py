@@ -143,6 +143,10 @@ def config_ops(name, cumo, host):
             ("v=var+1e-5", lambda e: e.__setitem__("v", e["var"] + 1e-5), 8 * rx, rx),
             ("sd=NMath.sqrt(v)", lambda e: e.__setitem__("sd", NM.sqrt(e["v"])), 8 * rx, rx),
             ("n=c/sd", lambda e: e.__setitem__("n", e["c"] / e["sd"]), 8 * nx + 4 * rx, nx),
+            # the same two composites as one launch each (library additions beside the chain above):
+            # one read and one write of the array
+            ("Fused.softmax(S)", lambda e: e.__setitem__("pf", cumo.Fused.softmax(e["S"])), 8 * ns, ns),
+            ("Fused.layernorm(X,1e-5)", lambda e: e.__setitem__("nf", cumo.Fused.layernorm(e["X"], 1e-5)), 8 * nx, nx),
         ]
     raise ValueError(name)
 

@@ -1353,6 +1353,92 @@ int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int red
     return rc;
 }
 
+// softmax / layernorm along the last dimension (library additions). One fused launch
+// when the rows are contiguous and fit the row kernels; otherwise the chain of array
+// operations a Cumo program would write (bench/transformer_bench.rb:110-124), whose
+// results the fused launch matches up to the order of the two row sums.
+static int fused_rows(int mode, const cumo_hip_narray_t* x, double eps, cumo_hip_narray_t* z) {
+    int rc = check_view(x, "operand");
+    if (rc) return rc;
+    if (!is_float(x->type)) return fail(CUMO_HIP_ERROR_TYPE, "softmax / layernorm: operand is not SFloat or DFloat");
+    if (x->ndim < 1) return fail(CUMO_HIP_ERROR_DIMENSION, "softmax / layernorm need at least one dimension");
+    const int nd = x->ndim;
+    const size_t n = x->shape[nd - 1];
+    const ssize_t es = kElmsz[x->type];
+    const bool fresh = z->ptr == NULL;
+    if (fresh) {
+        rc = cumo_hip_na_alloc(z, x->type, nd, x->shape);
+        if (rc) return rc;
+    } else {
+        rc = check_view(z, "result");
+        if (rc) return rc;
+        bool same = z->type == x->type && z->ndim == nd;
+        for (int d = 0; same && d < nd; ++d) same = z->shape[d] == x->shape[d];
+        if (!same) return fail(CUMO_HIP_ERROR_SHAPE, "softmax / layernorm: result array has the wrong shape or type");
+    }
+    if (total_of(x) == 0) return CUMO_HIP_OK;
+    // rows as one uniform step: the outer dimensions of both arrays merge into one
+    bool rows_ok = (n == 1 || (x->stride[nd - 1] == es && z->stride[nd - 1] == es));
+    size_t rows = 1;
+    ssize_t xs = 0, zs = 0;
+    {
+        bool first = true;
+        for (int d = nd - 2; d >= 0 && rows_ok; --d) {
+            if (x->shape[d] == 1) continue;
+            if (first) {
+                xs = x->stride[d];
+                zs = z->stride[d];
+                first = false;
+            } else if (x->stride[d] != xs * (ssize_t)rows || z->stride[d] != zs * (ssize_t)rows) {
+                rows_ok = false;
+            }
+            rows *= x->shape[d];
+        }
+    }
+    if (rows_ok) {
+        cumo_hip_fused_rows_t d;
+        d.rows = rows;
+        d.n = n;
+        d.in_row_step = xs;
+        d.out_row_step = zs;
+        d.in = x->ptr + x->offset;
+        d.out = z->ptr + z->offset;
+        d.eps = eps;
+        if (cumo_hip_fused_rows_kernel_launch(x->type, mode, &d)) return CUMO_HIP_OK;
+    }
+    // the chain
+    const unsigned last = 1u << (nd - 1);
+    NA a, b, c, e;
+    a.ptr = b.ptr = c.ptr = e.ptr = NULL;
+    if (mode == 0) {
+        rc = cumo_hip_na_reduce("max", x, last, 1, 0, &a, NULL);
+        if (!rc) rc = cumo_hip_na_binary("sub", x, &a, &b);
+        if (!rc) rc = cumo_hip_na_math("exp", &b, &c);
+        if (!rc) rc = cumo_hip_na_reduce("sum", &c, last, 1, 0, &e, NULL);
+        if (!rc) rc = cumo_hip_na_binary("div", &c, &e, z);
+    } else {
+        NA v2, sd;
+        v2.ptr = sd.ptr = NULL;
+        rc = cumo_hip_na_reduce("mean", x, last, 1, 0, &a, NULL);
+        if (!rc) rc = cumo_hip_na_reduce("var", x, last, 1, 0, &b, NULL);
+        if (!rc) rc = cumo_hip_na_binary("sub", x, &a, &c);
+        if (!rc) rc = cumo_hip_na_binary_s("add", &b, eps, 0, &v2);
+        if (!rc) rc = cumo_hip_na_math("sqrt", &v2, &sd);
+        if (!rc) rc = cumo_hip_na_binary("div", &c, &sd, z);
+        free_tmp(&v2);
+        free_tmp(&sd);
+    }
+    free_tmp(&a);
+    free_tmp(&b);
+    free_tmp(&c);
+    free_tmp(&e);
+    if (rc && fresh) free_tmp(z);
+    return rc;
+}
+
+int cumo_hip_na_softmax(const cumo_hip_narray_t* x, cumo_hip_narray_t* z) { return fused_rows(0, x, 0.0, z); }
+int cumo_hip_na_layernorm(const cumo_hip_narray_t* x, double eps, cumo_hip_narray_t* z) { return fused_rows(1, x, eps, z); }
+
 int cumo_hip_na_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
     int rc = check_arith(x);
     if (rc) return rc;

@@ -703,3 +703,23 @@ class _NMath:
 
 
 NMath = _NMath()
+
+
+class _Fused:
+    """Row-wise composites along the last dimension in one launch (library additions;
+    the reference writes them as chains of array operations,
+    bench/transformer_bench.rb:110-124). Layouts the row kernels do not take fall
+    back to that chain inside the library."""
+
+    @staticmethod
+    def softmax(x):
+        d, z = _NMath._check(x)._desc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_softmax, C.byref(d), C.byref(z), results=(z,))
+
+    @staticmethod
+    def layernorm(x, eps=1e-5):
+        d, z = _NMath._check(x)._desc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_layernorm, C.byref(d), float(eps), C.byref(z), results=(z,))
+
+
+Fused = _Fused()

@@ -419,6 +419,22 @@ typedef struct {
 } cumo_hip_bit_count_nd_t;
 void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* counts);
 
+/* Row-wise softmax and layer normalisation in one pass (no counterpart in the
+ * reference, where they are chains of 5 and 6 array operations,
+ * bench/transformer_bench.rb:110-124). rows runs of n contiguous elements, row r at
+ * in + r * in_row_step; type 0 SFloat, 1 DFloat; mode 0 softmax, 1 layernorm with
+ * eps added to the variance (divisor n - 1, as Cumo's var). Returns 1 when
+ * launched, 0 when the layout is outside what the kernels take (the caller then
+ * composes the chain). */
+typedef struct {
+    uint64_t rows, n;
+    ssize_t  in_row_step, out_row_step;
+    char*    in;
+    char*    out;
+    double   eps;
+} cumo_hip_fused_rows_t;
+int cumo_hip_fused_rows_kernel_launch(int type, int mode, const cumo_hip_fused_rows_t* rows);
+
 /* Many scan runs in one launch (no counterpart in the reference, which calls the
  * run launcher once per run from a loop on the host, narray/gen/tmpl/cum.c:12-46).
  * Run r starts at in + sum_k i_k * ostep_in[k] where (i_0 .. i_{nouter-1}) is r

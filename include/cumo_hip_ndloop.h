@@ -214,6 +214,15 @@ int cumo_hip_na_mulsum(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, u
  * gen/tmpl/cum.c:48-80). nan: NaN elements are skipped (leading ones stay NaN). */
 int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int nan, cumo_hip_narray_t* z);
 
+/* Library additions: softmax and layer normalisation along the LAST dimension,
+ *   softmax:   e = exp(x - max(x)); e / sum(e)
+ *   layernorm: (x - mean(x)) / sqrt(var(x) + eps), var with divisor n - 1 as Cumo's
+ * as one launch when rows are contiguous 128-bit-aligned runs of at most 16384
+ * SFloat / 4096 DFloat elements, else as the chain of array operations. Every
+ * elementwise step is the chain's own; only the order of the two row sums differs. */
+int cumo_hip_na_softmax(const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
+int cumo_hip_na_layernorm(const cumo_hip_narray_t* x, double eps, cumo_hip_narray_t* z);
+
 /* Bit logic: and or xor eq / copy not (reference: gen/tmpl_bit/binary.c, unary.c). */
 int cumo_hip_na_bit_binary(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
 int cumo_hip_na_bit_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
