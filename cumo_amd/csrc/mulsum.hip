@@ -66,7 +66,8 @@ __device__ __forceinline__ T ms_block_sum(T acc) {
 }
 
 // VEC > 1: both runs contiguous and 16-byte aligned at every chunk start
-template <class T, bool NANF, int VEC>
+// NT: non-temporal loads, for runs that do not fit the last-level cache anyway
+template <class T, bool NANF, int VEC, bool NT>
 __global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1, const char* p2, int64_t s1, int64_t s2, uint64_t n,
                                                                   uint64_t chunk, T* partial, T* out) {
     const uint64_t begin = (uint64_t)blockIdx.x * chunk;
@@ -83,8 +84,10 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1
             V a[4], b[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                a[u].q = *reinterpret_cast<const u4*>(p1 + (i + u * stride) * sizeof(T));
-                b[u].q = *reinterpret_cast<const u4*>(p2 + (i + u * stride) * sizeof(T));
+                const u4* pa = reinterpret_cast<const u4*>(p1 + (i + u * stride) * sizeof(T));
+                const u4* pb = reinterpret_cast<const u4*>(p2 + (i + u * stride) * sizeof(T));
+                a[u].q = NT ? __builtin_nontemporal_load(pa) : *pa;
+                b[u].q = NT ? __builtin_nontemporal_load(pb) : *pb;
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u)
@@ -163,11 +166,15 @@ void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, 
         partial = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * grid));
         if (!partial) return;
     }
-    if (vec)
-        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n,
-                           chunk, partial, reinterpret_cast<T*>(p3));
+    const bool nt = 2 * n * sizeof(T) > (320ull << 20);
+    if (vec && nt)
+        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, true>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2,
+                           n, chunk, partial, reinterpret_cast<T*>(p3));
+    else if (vec)
+        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, false>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2,
+                           n, chunk, partial, reinterpret_cast<T*>(p3));
     else
-        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n,
+        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1, false>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n,
                            chunk, partial, reinterpret_cast<T*>(p3));
     if (partial) {
         hipLaunchKernelGGL((mulsum_combine_kernel<T>), dim3(1), dim3(kMsBlock), 0, stream, (const T*)partial, grid, reinterpret_cast<T*>(p3));
