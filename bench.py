@@ -91,7 +91,7 @@ def config_ops(name, cumo, host):
             ("y=t+b", lambda e: e.__setitem__("y", e["t"] + e["b"]), 12 * n, n),
             ("s=y.sum", lambda e: e.__setitem__("s", e["y"].sum()), 4 * n + 4, n),
         ]
-    if name == "c2":
+    if name in ("c2", "c2_large"):
         n = host["A"].shape[0]
         env = {"A": cumo.DFloat.cast(host["A"]), "r": cumo.DFloat.cast(host["r"])}
         full, vec = 8 * n * n, 8 * n
@@ -100,7 +100,7 @@ def config_ops(name, cumo, host):
             ("C.sum(axis:1)", lambda e: e.__setitem__("sum", e["C"].sum(axis=1)), full + vec, n * n),
             ("C.max(axis:1)", lambda e: e.__setitem__("max", e["C"].max(axis=1)), full + vec, n * n),
         ]
-    if name == "c3":
+    if name in ("c3", "c3_large"):
         t = host["T"]
         env = {"T": cumo.SFloat.cast(t)}
         nb, n = t.nbytes, t.size
@@ -153,10 +153,13 @@ def config_ops(name, cumo, host):
 
 HOST_INPUTS = {
     "c1": inputs_c1, "c1_large": lambda: inputs_c1(1 << 26), "c2": inputs_c2, "c3": inputs_c3, "c4": inputs_c4, "c5": inputs_c5,
+    "c2_large": lambda: inputs_c2(8192), "c3_large": lambda: inputs_c3((256, 512, 1024)),
 }
 WORKLOAD_TEXT = {
     "c1": "C1 SFloat axpy + full sum, n=2^20",
     "c1_large": "C1 at n=2^26 (256 MiB per array)",
+    "c2_large": "C2 at 8192 x 8192 (512 MiB per matrix)",
+    "c3_large": "C3 at [256,512,1024] (512 MiB)",
     "c2": "C2 DFloat broadcast add + row reduce: A f64 [4096,4096] + r [1,4096]; C.sum(axis:1); C.max(axis:1)",
     "c3": "C3 SFloat axis reductions on [64,512,1024]",
     "c4": "C4 strided/transposed views on SFloat [8192,8192] + Int32 stride-3 row slice copy",
@@ -257,7 +260,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all-configs", action="store_true", help="measure every op of all five configs with full iteration counts")
-    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c3,c4,c5)")
+    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -358,7 +361,7 @@ def main():
 
     per_config = {}
     if not args.no_per_config:
-        names = [c for c in args.configs.split(",") if c] or ["c1", "c1_large", "c2", "c3", "c4", "c5"]
+        names = [c for c in args.configs.split(",") if c] or ["c1", "c1_large", "c2", "c2_large", "c3", "c3_large", "c4", "c5"]
         iters, warm = (30, 5) if args.all_configs else (7, 2)
         for name in names:
             per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm)}

@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl i
     }
 }
 
-template <class Impl, int VEC, bool PARTIAL>
+template <class Impl, int VEC, bool PARTIAL, bool NT = false>
 __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
     typedef typename Impl::In In;
     typedef typename Impl::Acc Acc;
@@ -312,7 +312,15 @@ __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl i
                     const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
                     roff[u] = off;
                     if constexpr (VEC > 1) {
-                        const RedVec<In, VEC> v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
+                        RedVec<In, VEC> v;
+                        if constexpr (NT && sizeof(RedVec<In, VEC>) == 16) {
+                            typedef uint32_t ntu4 __attribute__((ext_vector_type(4)));
+                            union NTV { ntu4 q; RedVec<In, VEC> r; __device__ NTV() {} } ntv;
+                            ntv.q = __builtin_nontemporal_load(reinterpret_cast<const ntu4*>(base + off));
+                            v = ntv.r;
+                        } else {
+                            v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
+                        }
 #pragma unroll
                         for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
                     } else {
@@ -465,6 +473,12 @@ static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Im
     if (grid > red_grid_cap()) grid = red_grid_cap();
     if (grid == 0) return;
     const dim3 g((unsigned)grid), b(kRedBlock);
+    if constexpr (kMaxVec >= 2) {
+        if (vec == kMaxVec && kp.out_total * kp.red_total * sizeof(typename Impl::In) > kRedNtBytes) {
+            hipLaunchKernelGGL((red_col_kernel<Impl, kMaxVec, PARTIAL, true>), g, b, 0, stream, kp, impl, partial);
+            return;
+        }
+    }
     if constexpr (kMaxVec >= 4) {
         if (vec == 4) { hipLaunchKernelGGL((red_col_kernel<Impl, 4, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
     }
