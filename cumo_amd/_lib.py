@@ -168,6 +168,8 @@ _sig = {
     "cumo_hip_na_pow_s": (C.c_int, [P(NArrayDesc), C.c_double, C.c_int, C.c_int, P(NArrayDesc)]),
     "cumo_hip_na_mulsum": (C.c_int, [P(NArrayDesc), P(NArrayDesc), C.c_uint, C.c_int, C.c_int, P(NArrayDesc)]),
     "cumo_hip_na_cum": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_uint, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_where": (C.c_int, [P(NArrayDesc), C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_mask": (C.c_int, [P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_softmax": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_layernorm": (C.c_int, [P(NArrayDesc), C.c_double, P(NArrayDesc)]),
     "cumo_hip_na_ewcomp": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), C.c_int, P(NArrayDesc)]),

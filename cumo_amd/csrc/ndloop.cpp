@@ -1439,6 +1439,100 @@ static int fused_rows(int mode, const cumo_hip_narray_t* x, double eps, cumo_hip
 int cumo_hip_na_softmax(const cumo_hip_narray_t* x, cumo_hip_narray_t* z) { return fused_rows(0, x, 0.0, z); }
 int cumo_hip_na_layernorm(const cumo_hip_narray_t* x, double eps, cumo_hip_narray_t* z) { return fused_rows(1, x, eps, z); }
 
+// ---- Bit#where, Bit#mask (gen/tmpl_bit/where.c:98-127, mask.c:96-167) --------------
+namespace {
+struct WhereWalk {
+    char* out;
+    size_t elmsz;
+    char* scratch;
+    int invert;
+    uint64_t count;
+};
+void where_walk(const LP* lp, int level, size_t pos, WhereWalk* w) {
+    const cumo_hip_loop_args_t& in = lp->args[0];
+    if (level == lp->ndim - 1) {
+        cumo_bit_where_kernel_launch((CUMO_BIT_DIGIT*)in.ptr, pos, in.step[level], NULL, lp->n[level], w->invert, w->out, w->elmsz, w->count, w->scratch);
+        w->count += lp->n[level];
+        return;
+    }
+    for (size_t i = 0; i < lp->n[level]; i++) where_walk(lp, level + 1, pos + (size_t)((ssize_t)i * in.step[level]), w);
+}
+}  // namespace
+
+// z = positions (row-major, from 0) of the set bits of x, or of the clear ones when
+// invert; Int32, or Int64 for an array of more than 2^32 - 1 elements. The count is
+// read back once to size the result (one stream synchronisation, as where.c:13-28).
+int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t* z) {
+    int rc = check_view(x, "operand");
+    if (rc) return rc;
+    if (x->type != CUMO_HIP_BIT) return no_method("where");
+    if (!z || z->ptr) return fail(CUMO_HIP_ERROR_ARGUMENT, "where: the result is always allocated by the library");
+    NA cnt;
+    cnt.ptr = NULL;
+    rc = cumo_hip_na_bit_count(x, 0, 0, invert, &cnt);
+    if (rc) return rc;
+    uint64_t n_hit = 0;
+    cumo_hip_memcpy_d2h(&n_hit, cnt.ptr + cnt.offset, sizeof(n_hit));
+    free_tmp(&cnt);
+    const size_t total = total_of(x);
+    const int itype = total > 4294967295ull ? CUMO_HIP_INT64 : CUMO_HIP_INT32;
+    size_t shape1[1] = {(size_t)n_hit};
+    rc = cumo_hip_na_alloc(z, itype, 1, shape1);
+    if (rc || n_hit == 0) return rc;
+    cumo_hip_ndfunc_t nf = {NULL, 0, 1, 0, {0, 0}};
+    const NA* in[1] = {x};
+    LP lp;
+    rc = cumo_hip_na_ndloop_prepare(&nf, in, NULL, 0, &lp);
+    if (!rc) {
+        WhereWalk w = {z->ptr, (size_t)kElmsz[itype], cumo_bit_where_scratch_new(), invert ? 1 : 0, 0};
+        if (!w.scratch) {
+            rc = CUMO_HIP_ERROR_OUT_OF_MEMORY;
+        } else {
+            where_walk(&lp, 0, lp.args[0].bitpos, &w);
+            cumo_cuda_runtime_free(w.scratch);
+        }
+    }
+    if (rc) free_tmp(z);
+    return rc;
+}
+
+// z = the elements of x where mask is set, in row-major order (mask.c:96-167 returns
+// a view over an index array; here the elements are gathered into a new array).
+int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
+    int rc = check_view(mask, "mask");
+    if (!rc) rc = check_view(x, "operand");
+    if (rc) return rc;
+    if (mask->type != CUMO_HIP_BIT) return no_method("mask");
+    if (x->type == CUMO_HIP_BIT) return fail(CUMO_HIP_ERROR_TYPE, "mask: a Bit array cannot be the masked array here");
+    bool same = mask->ndim == x->ndim;
+    for (int d = 0; same && d < x->ndim; ++d) same = mask->shape[d] == x->shape[d];
+    if (!same) return fail(CUMO_HIP_ERROR_SHAPE, "mask and masked arrays must have the same shape");
+    if (!z || z->ptr) return fail(CUMO_HIP_ERROR_ARGUMENT, "mask: the result is always allocated by the library");
+    NA pos;
+    pos.ptr = NULL;
+    rc = cumo_hip_na_where(mask, 0, &pos);
+    if (rc) return rc;
+    rc = cumo_hip_na_alloc(z, x->type, 1, pos.shape);
+    if (!rc && pos.shape[0] != 0) {
+        cumo_hip_gather_flat_t g;
+        std::memset(&g, 0, sizeof(g));
+        g.ndim = x->ndim;
+        g.n = pos.shape[0];
+        for (int d = 0; d < x->ndim; ++d) {
+            g.shape[d] = x->shape[d];
+            g.step[d] = x->stride[d];
+        }
+        g.in = x->ptr + x->offset;
+        g.out = z->ptr;
+        g.pos = pos.ptr;
+        g.pos_elmsz = kElmsz[pos.type];
+        g.elmsz = kElmsz[x->type];
+        cumo_hip_gather_flat_kernel_launch(&g);
+    }
+    free_tmp(&pos);
+    return rc;
+}
+
 int cumo_hip_na_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z) {
     int rc = check_arith(x);
     if (rc) return rc;

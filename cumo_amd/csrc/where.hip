@@ -1,0 +1,235 @@
+// Bit#where and Bit#mask: the positions of the set (or clear) bits of a run,
+// compacted in ascending order.
+//
+// Replaces narray/gen/tmpl_bit/where_kernel.cu and mask_kernel.cu of the reference
+// with the same launcher ABI and the same scratch layout (two running cursors, then
+// up to 1024 block counts), so that the host iterators (tmpl_bit/where.c:34-52,
+// mask.c) bind unchanged: a cursor in the scratch carries the output position from
+// one run of a view to the next on the device, and nothing is read back.
+//
+// Three launches per run: every block counts the set bits of its contiguous range
+// of 32-bit chunks; one block turns the counts into output positions (and advances
+// the cursor); every block walks its range again and writes each chunk's positions
+// from where an exclusive scan over the block puts them. Blocks are 256 threads (4
+// wave64): the scan inside a block is a wave scan by shuffles plus four LDS slots.
+// A contiguous run reads whole words (two per chunk when the run starts inside a
+// word); strided and index-array runs gather bit by bit.
+#include "common.h"
+
+#include <cstring>
+
+namespace cumo_hip {
+namespace {
+
+constexpr int kWhBlock = 256;
+constexpr uint64_t kWhMaxBlocks = 1024;  // the scratch holds this many block counts (where_kernel.cu:11)
+
+// the 32 bits [c*32, c*32+32) of the run, bits beyond n cleared
+__device__ __forceinline__ uint32_t wh_chunk(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n, uint64_t c,
+                                             int contiguous, int invert) {
+    const uint64_t first = c * 32;
+    const uint64_t left = n - first;
+    const uint32_t valid = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
+    uint32_t z;
+    if (contiguous) {
+        const uint64_t q = p + first;
+        const uint64_t w = q >> 5;
+        const unsigned sh = (unsigned)(q & 31);
+        z = a[w] >> sh;
+        // the second word only exists when the chunk reaches into it
+        if (sh && (uint64_t)(32 - sh) < left) z |= a[w + 1] << (32 - sh);
+    } else {
+        z = 0;
+        const unsigned m = left >= 32 ? 32u : (unsigned)left;
+        for (unsigned k = 0; k < m; ++k) {
+            const uint64_t q = idx ? (p + idx[first + k]) : (uint64_t)((int64_t)p + (int64_t)(first + k) * s);
+            z |= ((a[q >> 5] >> (q & 31)) & 1u) << k;
+        }
+    }
+    if (invert) z = ~z;
+    return z & valid;
+}
+
+// exclusive scan of one value per thread over the block; *total gets the block's sum
+// in every thread. Two barriers; safe to call again right away.
+__device__ __forceinline__ uint64_t wh_block_exscan(uint64_t v, uint64_t* total) {
+    __shared__ uint64_t wave_sum[kWhBlock / 64];
+    const unsigned lane = threadIdx.x & 63;
+    uint64_t inc = v;
+    for (unsigned d = 1; d < 64; d <<= 1) {
+        const uint32_t lo = __shfl_up((uint32_t)inc, d);
+        const uint32_t hi = __shfl_up((uint32_t)(inc >> 32), d);
+        if (lane >= d) inc += ((uint64_t)hi << 32) | lo;
+    }
+    __syncthreads();  // the slots may still be read from the previous call
+    if (lane == 63) wave_sum[threadIdx.x >> 6] = inc;
+    __syncthreads();
+    uint64_t before = 0, all = 0;
+    for (unsigned w = 0; w < kWhBlock / 64; ++w) {
+        if (w < (threadIdx.x >> 6)) before += wave_sum[w];
+        all += wave_sum[w];
+    }
+    *total = all;
+    return before + inc - v;
+}
+
+__global__ __launch_bounds__(kWhBlock) void where_count_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
+                                                               int contiguous, int invert, uint64_t nchunks, uint64_t cpb, uint64_t* block_sums) {
+    uint64_t start = (uint64_t)blockIdx.x * cpb;
+    if (start > nchunks) start = nchunks;
+    const uint64_t end = (nchunks - start < cpb) ? nchunks : start + cpb;
+    uint64_t cnt = 0;
+    for (uint64_t c = start + threadIdx.x; c < end; c += kWhBlock) cnt += (uint64_t)__popc(wh_chunk(a, p, s, idx, n, c, contiguous, invert));
+    uint64_t total;
+    wh_block_exscan(cnt, &total);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+// block_sums[b] becomes the output position of block b's first hit; *running moves on
+__global__ __launch_bounds__(kWhBlock) void where_scan_kernel(uint64_t* block_sums, uint64_t nblocks, uint64_t* running) {
+    uint64_t acc = *running;
+    for (uint64_t t0 = 0; t0 < nblocks; t0 += kWhBlock) {
+        const uint64_t t = t0 + threadIdx.x;
+        const uint64_t v = t < nblocks ? block_sums[t] : 0;
+        uint64_t total;
+        const uint64_t pre = wh_block_exscan(v, &total);
+        if (t < nblocks) block_sums[t] = acc + pre;
+        acc += total;
+    }
+    __syncthreads();  // every thread has read *running before it is rewritten
+    if (threadIdx.x == 0) *running = acc;
+}
+
+// MASK false: out[o] = count + position in the run, as elmsz-byte integers (where).
+// MASK true:  out[o] = the masked array's element position p2 + j*s2 (or p2 + idx2[j]), as size_t (mask).
+template <bool MASK>
+__global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
+                                                                 int contiguous, int invert, uint64_t nchunks, uint64_t cpb, char* out, size_t elmsz,
+                                                                 uint64_t count, size_t p2, int64_t s2, const size_t* idx2,
+                                                                 const uint64_t* block_sums) {
+    uint64_t start = (uint64_t)blockIdx.x * cpb;
+    if (start > nchunks) start = nchunks;
+    const uint64_t end = (nchunks - start < cpb) ? nchunks : start + cpb;
+    uint64_t off = block_sums[blockIdx.x];
+    for (uint64_t c0 = start; c0 < end; c0 += kWhBlock) {
+        const uint64_t c = c0 + threadIdx.x;
+        uint32_t z = c < end ? wh_chunk(a, p, s, idx, n, c, contiguous, invert) : 0u;
+        uint64_t total;
+        uint64_t o = off + wh_block_exscan((uint64_t)__popc(z), &total);
+        while (z) {
+            const uint64_t j = c * 32 + (uint64_t)(__ffs((int)z) - 1);
+            if (MASK) {
+                reinterpret_cast<size_t*>(out)[o] = idx2 ? (p2 + idx2[j]) : (size_t)((int64_t)p2 + (int64_t)j * s2);
+            } else if (elmsz == 4) {
+                reinterpret_cast<int32_t*>(out)[o] = (int32_t)(count + j);
+            } else {
+                reinterpret_cast<int64_t*>(out)[o] = (int64_t)(count + j);
+            }
+            ++o;
+            z &= z - 1;
+        }
+        off += total;
+    }
+}
+
+template <bool MASK>
+void where_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, int invert, char* out, size_t elmsz, uint64_t count, size_t p2,
+                  ssize_t s2, size_t* idx2, uint64_t* running, uint64_t* block_sums) {
+    if (n == 0) return;  // a grid of no blocks is an invalid launch
+    const uint64_t nchunks = (n + 31) / 32;
+    const int contiguous = (idx == nullptr && s == 1) ? 1 : 0;
+    uint64_t nblocks = (nchunks + kWhBlock - 1) / kWhBlock;
+    if (nblocks > kWhMaxBlocks) nblocks = kWhMaxBlocks;
+    const uint64_t cpb = (nchunks + nblocks - 1) / nblocks;
+    hipStream_t st = current_stream();
+    hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n, contiguous,
+                       invert, nchunks, cpb, block_sums);
+    hipLaunchKernelGGL(where_scan_kernel, dim3(1), dim3(kWhBlock), 0, st, block_sums, nblocks, running);
+    hipLaunchKernelGGL((where_scatter_kernel<MASK>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n,
+                       contiguous, invert, nchunks, cpb, out, elmsz, count, p2, (int64_t)s2, (const size_t*)idx2, (const uint64_t*)block_sums);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+// a tiny fill instead of a memset node, so that a caller may capture the stream
+__global__ void where_zero_kernel(uint64_t* p) {
+    if (threadIdx.x < 2) p[threadIdx.x] = 0;
+}
+
+// z[i] = the element of x at flat (row-major) position pos[i]
+struct GatherParams {
+    int ndim;
+    uint64_t n;
+    uint64_t shape[CUMO_NA_MAX_DIMENSION];
+    int64_t step[CUMO_NA_MAX_DIMENSION];
+    const char* in;
+    char* out;
+    const char* pos;
+    int pos_elmsz, elmsz;
+};
+__global__ __launch_bounds__(256) void gather_flat_kernel(GatherParams g) {
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < g.n; i += (uint64_t)gridDim.x * 256) {
+        uint64_t r = g.pos_elmsz == 4 ? (uint64_t)(uint32_t)reinterpret_cast<const int32_t*>(g.pos)[i] : (uint64_t)reinterpret_cast<const int64_t*>(g.pos)[i];
+        int64_t off = 0;
+        for (int d = g.ndim - 1; d >= 0; --d) {
+            const uint64_t m = g.shape[d];
+            const uint64_t q = r / m;
+            off += (int64_t)(r - q * m) * g.step[d];
+            r = q;
+        }
+        if (g.elmsz == 4) reinterpret_cast<uint32_t*>(g.out)[i] = *reinterpret_cast<const uint32_t*>(g.in + off);
+        else reinterpret_cast<uint64_t*>(g.out)[i] = *reinterpret_cast<const uint64_t*>(g.in + off);
+    }
+}
+
+}  // namespace
+}  // namespace cumo_hip
+
+using namespace cumo_hip;
+
+extern "C" {
+
+// reference: where_kernel.cu:83-89
+char* cumo_bit_where_scratch_new(void) {
+    char* scratch = cumo_cuda_runtime_malloc((2 + kWhMaxBlocks) * sizeof(uint64_t));
+    if (!scratch) return nullptr;
+    hipLaunchKernelGGL(where_zero_kernel, dim3(1), dim3(64), 0, current_stream(), reinterpret_cast<uint64_t*>(scratch));
+    cumo_cuda_runtime_check_kernel_launch();
+    return scratch;
+}
+
+// reference: where_kernel.cu:91-107
+void cumo_bit_where_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, int invert, char* out, size_t elmsz, uint64_t count,
+                                  char* scratch) {
+    uint64_t* running = reinterpret_cast<uint64_t*>(scratch) + (invert ? 1 : 0);
+    where_launch<false>(a, p, s, idx, n, invert, out, elmsz, count, 0, 0, nullptr, running, reinterpret_cast<uint64_t*>(scratch) + 2);
+}
+
+// reference: mask_kernel.cu:36-54
+void cumo_bit_mask_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, size_t* out, size_t p2, ssize_t s2, size_t* idx2,
+                                 char* scratch) {
+    where_launch<true>(a, p, s, idx, n, 0, reinterpret_cast<char*>(out), sizeof(size_t), 0, p2, s2, idx2, reinterpret_cast<uint64_t*>(scratch),
+                       reinterpret_cast<uint64_t*>(scratch) + 2);
+}
+
+void cumo_hip_gather_flat_kernel_launch(const cumo_hip_gather_flat_t* d) {
+    if (!d || d->n == 0) return;
+    GatherParams g;
+    std::memset(&g, 0, sizeof(g));
+    g.ndim = d->ndim;
+    g.n = d->n;
+    for (int k = 0; k < d->ndim && k < CUMO_NA_MAX_DIMENSION; ++k) {
+        g.shape[k] = d->shape[k];
+        g.step[k] = d->step[k];
+    }
+    g.in = d->in;
+    g.out = d->out;
+    g.pos = d->pos;
+    g.pos_elmsz = d->pos_elmsz;
+    g.elmsz = d->elmsz;
+    uint64_t grid = (d->n + 255) / 256;
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(gather_flat_kernel, dim3((unsigned)grid), dim3(256), 0, current_stream(), g);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+}  // extern "C"

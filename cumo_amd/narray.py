@@ -206,6 +206,8 @@ class NArray:
 
     # ---- views (reference: narray/index.c:445-516,602-609, narray/data.c:272-297)
     def __getitem__(self, key):
+        if isinstance(key, NArray) and type(key).__name__ == "Bit":
+            return key.mask(self)  # a[mask]: the elements where the mask is set
         if not isinstance(key, tuple):
             key = (key,)
         if any(k is Ellipsis for k in key):
@@ -640,6 +642,24 @@ class Bit(NArray):
         x, z = self._desc(), NArrayDesc()
         return _run(_L.cumo_hip_na_bit_count, C.byref(x), _reduce_mask(self.ndim, axis), int(bool(keepdims)),
                     1 if count_false else 0, C.byref(z), results=(z,))
+
+    def where(self):
+        """Positions of the set bits (reference: gen/tmpl_bit/where.c:98-127)."""
+        d, z = self._desc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_where, C.byref(d), 0, C.byref(z), results=(z,))
+
+    def where2(self):
+        """[positions of the set bits, positions of the clear bits] (tmpl_bit/where2.c)"""
+        d, z0, z1 = self._desc(), NArrayDesc(), NArrayDesc()
+        return [_run(_L.cumo_hip_na_where, C.byref(d), 0, C.byref(z0), results=(z0,)),
+                _run(_L.cumo_hip_na_where, C.byref(d), 1, C.byref(z1), results=(z1,))]
+
+    def mask(self, array):
+        """The elements of `array` where self is set (reference: gen/tmpl_bit/mask.c:96-167)."""
+        if not isinstance(array, NArray):
+            raise TypeError("mask needs an array")
+        m, x, z = self._desc(), array._desc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_mask, C.byref(m), C.byref(x), C.byref(z), results=(z,))
 
     def count_true(self, axis=None, keepdims=False): return self._count(False, axis, keepdims)
     def count_false(self, axis=None, keepdims=False): return self._count(True, axis, keepdims)

@@ -375,6 +375,16 @@ CUMO_HIP_BIT_UNARY_OPS(CUMO_HIP_DECL_BIT_UNARY)
 CUMO_HIP_DECL_BIT_COUNT(count_true)
 CUMO_HIP_DECL_BIT_COUNT(count_false)
 
+/* Bit#where / Bit#mask compaction: narray/gen/tmpl_bit/where_kernel.cu:83-107 (host
+ * tmpl_bit/where.c:10-11) and tmpl_bit/mask_kernel.cu:36-54. The scratch holds two
+ * running output cursors (ones, zeros) and up to 1024 block counts; the cursor carries
+ * the output position from one run of a view to the next on the device. `out` of where
+ * receives count + position as elmsz-byte (4 or 8) integers, `out` of mask the masked
+ * array's element positions p2 + j*s2 (or p2 + idx2[j]). */
+char *cumo_bit_where_scratch_new(void);
+void cumo_bit_where_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, size_t *idx, uint64_t n, int invert, char *out, size_t elmsz, uint64_t count, char *scratch);
+void cumo_bit_mask_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, size_t *idx, uint64_t n, size_t *out, size_t p2, ssize_t s2, size_t *idx2, char *scratch);
+
 /* ------------------------------------------------------------------------
  * 6. What this library adds (no counterpart symbol in the reference).
  * ---------------------------------------------------------------------- */
@@ -434,6 +444,22 @@ typedef struct {
     double   eps;
 } cumo_hip_fused_rows_t;
 int cumo_hip_fused_rows_kernel_launch(int type, int mode, const cumo_hip_fused_rows_t* rows);
+
+/* out[i] = the element of a strided view at flat row-major position pos[i] (no
+ * counterpart symbol in the reference, where a masked array is a view over an index
+ * array, tmpl_bit/mask.c:141-167, read by the index kernels). Elements of 4 or 8
+ * bytes, positions of 4 or 8 bytes. */
+typedef struct {
+    int      ndim;
+    uint64_t n;
+    size_t   shape[CUMO_NA_MAX_DIMENSION];
+    ssize_t  step[CUMO_NA_MAX_DIMENSION];
+    char*    in;
+    char*    out;
+    char*    pos;
+    int      pos_elmsz, elmsz;
+} cumo_hip_gather_flat_t;
+void cumo_hip_gather_flat_kernel_launch(const cumo_hip_gather_flat_t* gather);
 
 /* Many scan runs in one launch (no counterpart in the reference, which calls the
  * run launcher once per run from a loop on the host, narray/gen/tmpl/cum.c:12-46).

@@ -214,6 +214,14 @@ int cumo_hip_na_mulsum(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, u
  * gen/tmpl/cum.c:48-80). nan: NaN elements are skipped (leading ones stay NaN). */
 int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int nan, cumo_hip_narray_t* z);
 
+/* z = the row-major positions of x's set bits (clear bits when invert), as Int32, or
+ * Int64 for more than 2^32 - 1 elements (reference: gen/tmpl_bit/where.c:98-127). z
+ * must come in with ptr == NULL. */
+int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t* z);
+/* z = the elements of x where mask is set, row-major (reference: gen/tmpl_bit/mask.c:96-167,
+ * which answers a view over an index array; here a new array). Shapes must be equal. */
+int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
+
 /* Library additions: softmax and layer normalisation along the LAST dimension,
  *   softmax:   e = exp(x - max(x)); e / sum(e)
  *   layernorm: (x - mean(x)) / sqrt(var(x) + eps), var with divisor n - 1 as Cumo's

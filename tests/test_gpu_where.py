@@ -1,0 +1,109 @@
+"""Bit#where / where2 / mask: compaction of bit positions on the device against
+numpy's nonzero on the same bits (integer work: bit-exact), over contiguous
+arrays, views that start inside a word, strided and reversed views, and through
+the reference's launcher symbols with a device index array and a cursor carried
+across calls (narray/gen/tmpl_bit/where_kernel.cu:91-107, mask_kernel.cu:36-54)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [1, 31, 32, 33, 1000, 8191, 8192, 100003, (1 << 20) + 5, 1 << 25])
+def test_where_matches_nonzero(n):
+    import cumo_amd
+    rng = np.random.default_rng(900 + n % 1000)
+    density = rng.choice([0.02, 0.5, 0.97])
+    h = (rng.random(n) < density).astype(np.uint8)
+    b = cumo_amd.Bit.cast(h)
+    got = b.where()
+    assert isinstance(got, cumo_amd.Int32)
+    assert (got.to_numpy() == np.flatnonzero(h)).all()
+    t, f = b.where2()
+    assert (t.to_numpy() == np.flatnonzero(h)).all() and (f.to_numpy() == np.flatnonzero(h == 0)).all()
+    if n > 40:
+        for sl in (slice(3, None), slice(5, n - 7), slice(None, None, 2), slice(1, None, 3), slice(None, None, -1)):
+            assert (b[sl].where().to_numpy() == np.flatnonzero(h[sl])).all(), sl
+
+
+def test_where_on_matrices_and_empty_results():
+    import cumo_amd
+    rng = np.random.default_rng(91)
+    h = (rng.random((300, 777)) < 0.3).astype(np.uint8)
+    b = cumo_amd.Bit.cast(h)
+    assert (b.where().to_numpy() == np.flatnonzero(h)).all()
+    # views that do not contract to one run: one launch sequence per row, the cursor carried on the device
+    for key in ((slice(5, 200), slice(7, 600)), (slice(None), slice(None, None, 3)), (slice(None, None, -1), slice(None))):
+        assert (b[key].where().to_numpy() == np.flatnonzero(h[key])).all(), key
+    assert (b.transpose().where().to_numpy() == np.flatnonzero(h.T)).all()
+    z = cumo_amd.Bit.cast(np.zeros(5000, dtype=np.uint8))
+    assert z.where().to_numpy().shape == (0,)
+    assert (z.where2()[1].to_numpy() == np.arange(5000)).all()
+
+
+@pytest.mark.parametrize("tname,dt", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
+def test_mask_gathers_in_row_major_order(tname, dt):
+    import cumo_amd
+    cls = getattr(cumo_amd, tname)
+    rng = np.random.default_rng(92)
+    for shape in [(7,), (100003,), (300, 777), (5, 6, 130)]:
+        hx = rng.integers(-1000, 1000, size=shape).astype(dt)
+        hm = (rng.random(shape) < 0.4)
+        x, m = cls.cast(hx), cumo_amd.Bit.cast(hm.astype(np.uint8))
+        got = m.mask(x)
+        assert isinstance(got, cls) and (got.to_numpy() == hx[hm]).all(), shape
+        assert (x[m].to_numpy() == hx[hm]).all()
+        if len(shape) == 2:
+            # the masked array as a view: transposed, strided; the mask made from a comparison
+            assert (m.transpose().mask(x.transpose()).to_numpy() == hx.T[hm.T]).all()
+            assert (m[::2, 1::3].mask(x[::2, 1::3]).to_numpy() == hx[::2, 1::3][hm[::2, 1::3]]).all()
+            gt = x > 0
+            assert (x[gt].to_numpy() == hx[hx > 0]).all()
+    with pytest.raises(cumo_amd.ShapeError):
+        cumo_amd.Bit.cast(np.ones(4, dtype=np.uint8)).mask(cls.cast(np.zeros(5, dtype=dt)))
+
+
+def test_where_and_mask_launchers_with_index_arrays_and_a_carried_cursor():
+    from cumo_amd import _lib
+    from test_gpu_raw_abi import dev, fetch, free
+    rng = np.random.default_rng(93)
+    nbits = 50000
+    h = (rng.random(nbits) < 0.35).astype(np.uint8)
+    words = np.packbits(h, bitorder="little").view(np.uint32) if nbits % 32 == 0 else np.frombuffer(
+        np.packbits(np.concatenate([h, np.zeros(32 - nbits % 32, np.uint8)]), bitorder="little").tobytes(), dtype=np.uint32)
+    pw = dev(words)
+    new = _lib.fn("cumo_bit_where_scratch_new", C.c_void_p, [])
+    where = _lib.fn("cumo_bit_where_kernel_launch", None,
+                    [C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_void_p, C.c_uint64, C.c_int, C.c_void_p, C.c_size_t, C.c_uint64, C.c_void_p])
+    scratch = _lib.call(new)
+    # two runs, the second through a device index array, both appended to one output
+    n1, p1 = 20000, 13
+    idx = rng.permutation(nbits - 100)[:15000].astype(np.uint64)
+    pidx = dev(idx)
+    want = np.concatenate([np.flatnonzero(h[p1:p1 + n1]), n1 + np.flatnonzero(h[7 + idx.astype(np.int64)])])
+    pout = dev(np.full(want.size + 4, -1, dtype=np.int64))
+    _lib.call(where, pw, p1, 1, None, n1, 0, pout, 8, 0, scratch)
+    _lib.call(where, pw, 7, 0, pidx, idx.size, 0, pout, 8, n1, scratch)
+    got = fetch(pout, (want.size + 4,), np.int64)
+    assert (got[:want.size] == want).all() and (got[want.size:] == -1).all()
+    # the zeros keep their own cursor (scratch word 1): a strided run, every third bit
+    n3 = 9000
+    wantz = np.flatnonzero(h[5:5 + 3 * n3:3] == 0)
+    pz = dev(np.full(wantz.size + 2, -1, dtype=np.int32))
+    _lib.call(where, pw, 5, 3, None, n3, 1, pz, 4, 0, scratch)
+    gz = fetch(pz, (wantz.size + 2,), np.int32)
+    assert (gz[:wantz.size] == wantz).all() and (gz[wantz.size:] == -1).all()
+    # mask: positions of the masked array's elements, base 40 bytes and 8 bytes apart
+    _lib.lib.cumo_cuda_runtime_free(scratch)
+    scratch = _lib.call(new)
+    mask = _lib.fn("cumo_bit_mask_kernel_launch", None,
+                   [C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_void_p, C.c_uint64, C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_void_p, C.c_void_p])
+    wantm = 40 + 8 * np.flatnonzero(h[p1:p1 + n1])
+    pm = dev(np.zeros(wantm.size + 1, dtype=np.uint64))
+    _lib.call(mask, pw, p1, 1, None, n1, pm, 40, 8, None, scratch)
+    gm = fetch(pm, (wantm.size + 1,), np.uint64)
+    assert (gm[:wantm.size] == wantm.astype(np.uint64)).all() and gm[wantm.size] == 0
+    _lib.lib.cumo_cuda_runtime_free(scratch)
+    free(pw, pidx, pout, pz, pm)
