@@ -69,6 +69,12 @@ def inputs_c4(n=8192):
     return {"M": m, "I": i}
 
 
+def inputs_next(shape=(8192, 4096)):
+    rng = np.random.default_rng(5)
+    return {"x": rng.standard_normal(shape, dtype=np.float32), "y": rng.standard_normal(shape, dtype=np.float32),
+            "rows": rng.integers(0, shape[0], shape[0]), "perm": rng.permutation(shape[0])}
+
+
 def inputs_c5(s_shape=(32, 16, 512, 512), x_shape=(8192, 4096)):
     rng = np.random.default_rng(4)
     s = rng.standard_normal(s_shape, dtype=np.float32) * np.float32(2.0)  # N(0,2) read as sigma = 2
@@ -148,18 +154,40 @@ def config_ops(name, cumo, host):
             ("Fused.softmax(S)", lambda e: e.__setitem__("pf", cumo.Fused.softmax(e["S"])), 8 * ns, ns),
             ("Fused.layernorm(X,1e-5)", lambda e: e.__setitem__("nf", cumo.Fused.layernorm(e["X"], 1e-5)), 8 * nx, nx),
         ]
+    if name == "next":
+        x, y = host["x"], host["y"]
+        env = {"x": cumo.SFloat.cast(x), "y": cumo.SFloat.cast(y), "b": cumo.SFloat.cast(y)}
+        env["mask"] = env["x"] > 0.5
+        env["rows"] = host["rows"]
+        env["perm"] = host["perm"]
+        n, nb = x.size, x.nbytes
+        r, c = x.shape
+        cnt = int((x > 0.5).sum())
+        return env, [
+            ("x.mulsum(y,axis:1)", lambda e: e.__setitem__("dot", e["x"].mulsum(e["y"], axis=1)), 2 * nb + 4 * r, n),
+            ("x.clip(-1,1)", lambda e: e.__setitem__("cl", e["x"].clip(-1.0, 1.0)), 2 * nb, n),
+            ("SFloat.maximum(x,y)", lambda e: e.__setitem__("mx", cumo.SFloat.maximum(e["x"], e["y"])), 3 * nb, n),
+            ("x**3", lambda e: e.__setitem__("p3", e["x"] ** 3), 2 * nb, n),
+            ("x.cumsum(axis:1)", lambda e: e.__setitem__("cs", e["x"].cumsum(axis=1)), 2 * nb, n),
+            ("mask.where", lambda e: e.__setitem__("wh", e["mask"].where()), n // 8 + 4 * cnt, n),
+            ("x[mask]", lambda e: e.__setitem__("xm", e["x"][e["mask"]]), n // 8 + 4 * cnt + 4 * cnt, n),
+            # rows drawn with replacement: repeated rows are read from cache
+            ("x[rows,true] (gather)", lambda e: e.__setitem__("g", e["x"][e["rows"]]), 2 * nb + 8 * r, n),
+            ("b[perm,true]=x (scatter)", lambda e: e["b"].__setitem__(e["perm"], e["x"]), 2 * nb + 8 * r, n),
+        ]
     raise ValueError(name)
 
 
 HOST_INPUTS = {
     "c1": inputs_c1, "c1_large": lambda: inputs_c1(1 << 26), "c2": inputs_c2, "c3": inputs_c3, "c4": inputs_c4, "c5": inputs_c5,
-    "c2_large": lambda: inputs_c2(8192), "c3_large": lambda: inputs_c3((256, 512, 1024)),
+    "c2_large": lambda: inputs_c2(8192), "c3_large": lambda: inputs_c3((256, 512, 1024)), "next": inputs_next,
 }
 WORKLOAD_TEXT = {
     "c1": "C1 SFloat axpy + full sum, n=2^20",
     "c1_large": "C1 at n=2^26 (256 MiB per array)",
     "c2_large": "C2 at 8192 x 8192 (512 MiB per matrix)",
     "c3_large": "C3 at [256,512,1024] (512 MiB)",
+    "next": "operations beside the five configs on SFloat [8192,4096]: mulsum, clip, maximum, integer power, cumsum, where, a[mask], row gather and scatter through index arrays",
     "c2": "C2 DFloat broadcast add + row reduce: A f64 [4096,4096] + r [1,4096]; C.sum(axis:1); C.max(axis:1)",
     "c3": "C3 SFloat axis reductions on [64,512,1024]",
     "c4": "C4 strided/transposed views on SFloat [8192,8192] + Int32 stride-3 row slice copy",
@@ -200,9 +228,14 @@ def measure_config(name, cumo, lib, iters, warmup):
         # Python mirror's
         with _lib.record() as calls:
             fn(env)
+        # launches that rewrite an index array in place (positions -> byte offsets) belong to
+        # building the view, not to the copy, and must not run twice on the same array
+        recorded = calls  # holds the temporaries the operation released
+        calls = [c for c in calls if not c[0].__name__.startswith("cumo_na_index_")]
         _lib.replay(calls, warmup)
         ts = [timer.time(lambda: _lib.replay(calls, batch)) / batch for _ in range(iters)]
         ts.sort()
+        del recorded
         med = ts[len(ts) // 2]
         best = ts[0]
         rows.append({
@@ -260,7 +293,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all-configs", action="store_true", help="measure every op of all five configs with full iteration counts")
-    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5)")
+    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -361,7 +394,7 @@ def main():
 
     per_config = {}
     if not args.no_per_config:
-        names = [c for c in args.configs.split(",") if c] or ["c1", "c1_large", "c2", "c2_large", "c3", "c3_large", "c4", "c5"]
+        names = [c for c in args.configs.split(",") if c] or ["c1", "c1_large", "c2", "c2_large", "c3", "c3_large", "c4", "c5", "next"]
         iters, warm = (30, 5) if args.all_configs else (7, 2)
         for name in names:
             per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm)}

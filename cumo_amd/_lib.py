@@ -245,18 +245,26 @@ def call(f, *args):
     return r
 
 
+class _Calls(list):
+    def __init__(self):
+        super().__init__()
+        self.keep = []
+
+
 class record:
     """Collects the library calls (function, arguments) that launch work inside the
     block, so that a caller can issue exactly the same calls again without the
     Python-side work of building them: `with record() as calls: y = a + b`, then
     `replay(calls)`. A recorded host-layer call carries its result descriptor with
     the memory the first call allocated, so a replay writes into the same array;
-    the arrays involved must be kept alive."""
+    the arrays involved must be kept alive. Temporaries the recorded operations
+    themselves release inside the block (index arrays, staging buffers) stay allocated
+    for as long as the returned list lives (its `keep` attribute holds them)."""
 
     def __enter__(self):
         global _recording
         self._prev = _recording
-        _recording = []
+        _recording = _Calls()
         self.calls = _recording
         return self.calls
 

@@ -148,6 +148,93 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_elementwise_kernel(const char
     }
 }
 
+
+// One product sum per row, many rows in one launch: LPR lanes share a row whose two
+// runs are contiguous and 16-byte aligned, four vectors per operand in flight per
+// lane, four accumulators, then a butterfly over the lanes of the row (and the four
+// waves through LDS when a block shares the row). The order is fixed by the layout.
+struct MulsumRows {
+    uint64_t rows, n;
+    int64_t step1, step2, step3;  // bytes from one row to the next
+    const char *p1, *p2;
+    char* out;
+};
+
+template <class T, bool NANF, int LPR, bool NT>
+__global__ __launch_bounds__(kMsBlock) void mulsum_rows_kernel(MulsumRows g) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int RPB = kMsBlock / LPR;
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    union V { u4 q; T t[VEC]; __device__ V() {} };
+    const uint32_t lane = threadIdx.x % LPR;
+    const uint64_t nvec = g.n / VEC;
+    const uint64_t n_blocks = (g.rows + RPB - 1) / RPB;
+    for (uint64_t rb = blockIdx.x; rb < n_blocks; rb += gridDim.x) {
+        const uint64_t row = rb * RPB + threadIdx.x / LPR;
+        const bool ok = row < g.rows;
+        const uint64_t r = ok ? row : 0;  // surplus lanes redo row 0 and store nothing
+        const u4* a4 = reinterpret_cast<const u4*>(g.p1 + (int64_t)r * g.step1);
+        const u4* b4 = reinterpret_cast<const u4*>(g.p2 + (int64_t)r * g.step2);
+        T acc[4] = {T(), T(), T(), T()};
+        uint64_t v = lane;
+        for (; v + 3 * LPR < nvec; v += 4 * LPR) {
+            V a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a[u].q = NT ? __builtin_nontemporal_load(a4 + v + u * LPR) : a4[v + u * LPR];
+                b[u].q = NT ? __builtin_nontemporal_load(b4 + v + u * LPR) : b4[v + u * LPR];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) ms_fold<T, NANF>(a[u].t[j], b[u].t[j], acc[u]);
+        }
+        for (; v < nvec; v += LPR) {
+            V a, b;
+            a.q = a4[v];
+            b.q = b4[v];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) ms_fold<T, NANF>(a.t[j], b.t[j], acc[0]);
+        }
+        T tot = ms_add(ms_add(acc[0], acc[1]), ms_add(acc[2], acc[3]));
+        if constexpr (LPR <= 64) {
+#pragma unroll
+            for (unsigned d = LPR >> 1; d > 0; d >>= 1) tot = ms_add(tot, ms_shfl_down(tot, d));
+        } else {
+            __syncthreads();  // the LDS slots of the previous row have been read
+            tot = ms_block_sum<T>(tot);
+        }
+        if (lane == 0 && ok) {
+            T* z = reinterpret_cast<T*>(g.out + (int64_t)row * g.step3);
+            *z = ms_add(*z, tot);
+        }
+    }
+}
+
+template <class T, bool NANF>
+bool mulsum_rows_launch(const cumo_hip_mulsum_rows_t* d) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (d->n % VEC) return false;
+    if (((uintptr_t)d->p1 | (uintptr_t)d->p2 | (uintptr_t)d->row_step1 | (uintptr_t)d->row_step2) & 15) return false;
+    if (((uintptr_t)d->out | (uintptr_t)d->out_step) % sizeof(T)) return false;
+    MulsumRows g = {d->rows, d->n, (int64_t)d->row_step1, (int64_t)d->row_step2, (int64_t)d->out_step, d->p1, d->p2, d->out};
+    const uint64_t nvec = d->n / VEC;
+    const int lpr = nvec <= 64 ? 16 : (nvec <= 256 ? 64 : 256);
+    const uint64_t rpb = kMsBlock / lpr;
+    uint64_t grid = (d->rows + rpb - 1) / rpb;
+    if (grid > 256u * 64u) grid = 256u * 64u;
+    // both operands streamed once and larger than the last-level cache together
+    const bool nt = d->row_step1 != 0 && d->row_step2 != 0 && 2 * d->rows * d->n * sizeof(T) > (320ull << 20);
+    hipStream_t stream = current_stream();
+#define MS_ROWS(L, N) hipLaunchKernelGGL((mulsum_rows_kernel<T, NANF, L, N>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, g)
+    if (lpr == 16) { if (nt) MS_ROWS(16, true); else MS_ROWS(16, false); }
+    else if (lpr == 64) { if (nt) MS_ROWS(64, true); else MS_ROWS(64, false); }
+    else { if (nt) MS_ROWS(256, true); else MS_ROWS(256, false); }
+#undef MS_ROWS
+    cumo_cuda_runtime_check_kernel_launch();
+    return true;
+}
+
 template <class T, bool NANF>
 void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, uint64_t n) {
     hipStream_t stream = current_stream();
@@ -212,5 +299,18 @@ CUMO_DEF_MULSUM(sfloat, float, mulsum_nan, true)
 CUMO_DEF_MULSUM(dfloat, double, mulsum, false)
 CUMO_DEF_MULSUM(dfloat, double, mulsum_nan, true)
 CUMO_DEF_MULSUM(int32, int32_t, mulsum, false)
+
+// type: 0 SFloat, 1 DFloat, 2 Int32. out[r] += sum over the row of p1 * p2, for every
+// row in one launch. Returns 1 when launched, 0 when the layout is outside what the
+// kernel takes (rows not a whole number of 128-bit vectors, or not 16-byte aligned):
+// the caller then launches the rows one by one.
+int cumo_hip_mulsum_rows_kernel_launch(int type, int nan, const cumo_hip_mulsum_rows_t* d) {
+    if (!d || d->rows == 0 || d->n == 0) return 1;
+    bool ok = false;
+    if (type == 0) ok = nan ? mulsum_rows_launch<float, true>(d) : mulsum_rows_launch<float, false>(d);
+    else if (type == 1) ok = nan ? mulsum_rows_launch<double, true>(d) : mulsum_rows_launch<double, false>(d);
+    else if (type == 2) ok = mulsum_rows_launch<int32_t, false>(d);
+    return ok ? 1 : 0;
+}
 
 }  // extern "C"

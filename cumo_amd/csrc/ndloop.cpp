@@ -1190,7 +1190,20 @@ int cumo_hip_na_mulsum(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, u
             total *= lp.n[d];
             if (d < lp.ndim - 1) launches *= lp.n[d];
         }
-        if (!rc && total_of(z) != 0) {
+        // many short contiguous runs: every row in one launch
+        bool rows_done = false;
+        if (!rc && total_of(z) != 0 && total != 0 && lp.ndim == 2 && lp.args[2].step[1] == 0 && launches >= 2 &&
+            (launches > 1024 || lp.n[1] * (size_t)kElmsz[up] <= (1u << 20)) && lp.args[0].step[1] == (ssize_t)kElmsz[up] &&
+            lp.args[1].step[1] == (ssize_t)kElmsz[up]) {
+            rc = cumo_hip_na_fill(z, 0.0);
+            if (!rc) {
+                cumo_hip_mulsum_rows_t g = {lp.n[0], lp.n[1], lp.args[0].step[0], lp.args[1].step[0], lp.args[2].step[0],
+                                            lp.args[0].ptr, lp.args[1].ptr, lp.args[2].ptr};
+                const int t = up == CUMO_HIP_SFLOAT ? 0 : (up == CUMO_HIP_DFLOAT ? 1 : 2);
+                rows_done = cumo_hip_mulsum_rows_kernel_launch(t, nan != 0 && is_float(up), &g) == 1;
+            }
+        }
+        if (!rc && total_of(z) != 0 && !rows_done) {
             if (launches <= 1024 || total == 0) {
                 rc = cumo_hip_na_fill(z, 0.0);
                 if (!rc && total != 0) {
@@ -1457,6 +1470,19 @@ void where_walk(const LP* lp, int level, size_t pos, WhereWalk* w) {
     }
     for (size_t i = 0; i < lp->n[level]; i++) where_walk(lp, level + 1, pos + (size_t)((ssize_t)i * in.step[level]), w);
 }
+// the 1-D result of where / mask: allocated here, or a caller's array that must be
+// exactly as long as the count turns out to be
+int result_1d(NA* z, int type, size_t n, bool* allocated) {
+    *allocated = false;
+    if (!z->ptr) {
+        size_t shape1[1] = {n};
+        *allocated = true;
+        return cumo_hip_na_alloc(z, type, 1, shape1);
+    }
+    if (z->type != type || z->ndim != 1 || z->shape[0] != n || (n > 1 && z->stride[0] != (ssize_t)kElmsz[type]))
+        return fail(CUMO_HIP_ERROR_SHAPE, "the given result must be a contiguous 1-D array of the result's type and exact length");
+    return 0;
+}
 }  // namespace
 
 // z = positions (row-major, from 0) of the set bits of x, or of the clear ones when
@@ -1466,7 +1492,7 @@ int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t*
     int rc = check_view(x, "operand");
     if (rc) return rc;
     if (x->type != CUMO_HIP_BIT) return no_method("where");
-    if (!z || z->ptr) return fail(CUMO_HIP_ERROR_ARGUMENT, "where: the result is always allocated by the library");
+    if (!z) return fail(CUMO_HIP_ERROR_ARGUMENT, "where: no result descriptor");
     NA cnt;
     cnt.ptr = NULL;
     rc = cumo_hip_na_bit_count(x, 0, 0, invert, &cnt);
@@ -1476,15 +1502,15 @@ int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t*
     free_tmp(&cnt);
     const size_t total = total_of(x);
     const int itype = total > 4294967295ull ? CUMO_HIP_INT64 : CUMO_HIP_INT32;
-    size_t shape1[1] = {(size_t)n_hit};
-    rc = cumo_hip_na_alloc(z, itype, 1, shape1);
+    bool allocated;
+    rc = result_1d(z, itype, (size_t)n_hit, &allocated);
     if (rc || n_hit == 0) return rc;
     cumo_hip_ndfunc_t nf = {NULL, 0, 1, 0, {0, 0}};
     const NA* in[1] = {x};
     LP lp;
     rc = cumo_hip_na_ndloop_prepare(&nf, in, NULL, 0, &lp);
     if (!rc) {
-        WhereWalk w = {z->ptr, (size_t)kElmsz[itype], cumo_bit_where_scratch_new(), invert ? 1 : 0, 0};
+        WhereWalk w = {z->ptr + z->offset, (size_t)kElmsz[itype], cumo_bit_where_scratch_new(), invert ? 1 : 0, 0};
         if (!w.scratch) {
             rc = CUMO_HIP_ERROR_OUT_OF_MEMORY;
         } else {
@@ -1492,7 +1518,7 @@ int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t*
             cumo_cuda_runtime_free(w.scratch);
         }
     }
-    if (rc) free_tmp(z);
+    if (rc && allocated) free_tmp(z);
     return rc;
 }
 
@@ -1507,12 +1533,13 @@ int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, 
     bool same = mask->ndim == x->ndim;
     for (int d = 0; same && d < x->ndim; ++d) same = mask->shape[d] == x->shape[d];
     if (!same) return fail(CUMO_HIP_ERROR_SHAPE, "mask and masked arrays must have the same shape");
-    if (!z || z->ptr) return fail(CUMO_HIP_ERROR_ARGUMENT, "mask: the result is always allocated by the library");
+    if (!z) return fail(CUMO_HIP_ERROR_ARGUMENT, "mask: no result descriptor");
     NA pos;
     pos.ptr = NULL;
     rc = cumo_hip_na_where(mask, 0, &pos);
     if (rc) return rc;
-    rc = cumo_hip_na_alloc(z, x->type, 1, pos.shape);
+    bool allocated;
+    rc = result_1d(z, x->type, pos.shape[0], &allocated);
     if (!rc && pos.shape[0] != 0) {
         cumo_hip_gather_flat_t g;
         std::memset(&g, 0, sizeof(g));
@@ -1523,7 +1550,7 @@ int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, 
             g.step[d] = x->stride[d];
         }
         g.in = x->ptr + x->offset;
-        g.out = z->ptr;
+        g.out = z->ptr + z->offset;
         g.pos = pos.ptr;
         g.pos_elmsz = kElmsz[pos.type];
         g.elmsz = kElmsz[x->type];

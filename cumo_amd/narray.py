@@ -44,6 +44,12 @@ class _Buffer:
 
     def __del__(self):
         try:
+            rec = _lib._recording
+            if self.ptr and rec is not None:
+                # released inside a recording: the recorded calls still name this memory
+                rec.keep.append(_Buffer(self.nbytes, ptr=self.ptr))
+                self.ptr = None
+                return
             if self.ptr:
                 _L.cumo_cuda_runtime_free_no_raise(self.ptr)
                 self.ptr = None
@@ -109,6 +115,60 @@ def _reduce_mask(ndim, axis):
             raise DimensionError("dimension is out of range")
         m |= 1 << a
     return m
+
+
+def _is_index_array(k):
+    if isinstance(k, (list, np.ndarray, range)):
+        return True
+    return isinstance(k, NArray) and type(k).__name__ != "Bit"
+
+
+def _index_positions(k, n):
+    """Positions one index array selects in a dimension of n elements, as the
+    reference parses them on the host (narray/index.c:112-142,201-233): 1-D,
+    negative values count from the end, out of range raises IndexError."""
+    arr = np.asarray(k.to_numpy() if isinstance(k, NArray) else (list(k) if isinstance(k, range) else k))
+    if arr.size == 0:
+        return np.zeros(0, dtype=np.uint64)
+    if arr.ndim != 1:
+        raise IndexError("index array should be 1-dimensional")
+    if arr.dtype.kind not in "iu":
+        if arr.dtype.kind == "f" and np.all(arr == np.floor(arr)):
+            arr = arr.astype(np.int64)
+        else:
+            raise IndexError("index array must hold integers")
+    arr = arr.astype(np.int64)
+    arr = np.where(arr < 0, arr + n, arr)
+    if np.any((arr < 0) | (arr >= n)):
+        raise IndexError("index array value out of range (size %d)" % n)
+    return arr.astype(np.uint64)
+
+
+def _upload_index(pos):
+    buf = _Buffer(8 * max(len(pos), 1))
+    if len(pos):
+        pos = np.ascontiguousarray(pos, dtype=np.uint64)
+        call(_L.cumo_hip_memcpy_h2d, buf.ptr, pos.ctypes.data, pos.nbytes)
+    return buf
+
+
+def _index_launchers():
+    v, sz, ss, u64 = C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_uint64
+    P = C.POINTER
+    return {
+        "aref_nadata_index_stride": _lib.fn("cumo_na_index_aref_nadata_index_stride_kernel_launch", None, [v, ss, u64]),
+        "aref_naview_index_stride": _lib.fn("cumo_na_index_aref_naview_index_stride_kernel_launch", None, [v, ss, u64]),
+        "aref_naview_index_stride_last": _lib.fn("cumo_na_index_aref_naview_index_stride_last_kernel_launch", None, [v, ss, sz, u64]),
+        "at_nadata_index_stride_add": _lib.fn("cumo_na_index_at_nadata_index_stride_add_kernel_launch", None, [v, v, ss, u64]),
+        "at_nadata_index_beg_step_stride": _lib.fn("cumo_na_index_at_nadata_index_beg_step_stride_kernel_launch", None, [v, sz, ss, ss, u64]),
+        "at_nadata_index_beg_step_stride_add": _lib.fn("cumo_na_index_at_nadata_index_beg_step_stride_add_kernel_launch", None, [v, sz, ss, ss, u64]),
+        "copy_bytes": _lib.fn("cumo_iter_copy_bytes_kernel_launch", None, [v, v, ss, ss, v, v, u64, ss]),
+        "copy_to_buffer": _lib.fn("cumo_ndloop_copy_to_buffer_kernel_launch", None, [P(_lib.IArrayStridx), P(_lib.Indexer), v, sz]),
+        "copy_from_buffer": _lib.fn("cumo_ndloop_copy_from_buffer_kernel_launch", None, [P(_lib.IArrayStridx), P(_lib.Indexer), v, sz]),
+    }
+
+
+_IX = _index_launchers()
 
 
 class NArray:
@@ -205,9 +265,7 @@ class NArray:
         return d
 
     # ---- views (reference: narray/index.c:445-516,602-609, narray/data.c:272-297)
-    def __getitem__(self, key):
-        if isinstance(key, NArray) and type(key).__name__ == "Bit":
-            return key.mask(self)  # a[mask]: the elements where the mask is set
+    def _expand_key(self, key):
         if not isinstance(key, tuple):
             key = (key,)
         if any(k is Ellipsis for k in key):
@@ -216,7 +274,14 @@ class NArray:
             key = key[:i] + (slice(None),) * fill + key[i + 1:]
         if len(key) > self.ndim:
             raise IndexError("too many indices")
-        key = key + (slice(None),) * (self.ndim - len(key))
+        return key + (slice(None),) * (self.ndim - len(key))
+
+    def __getitem__(self, key):
+        if isinstance(key, NArray) and type(key).__name__ == "Bit":
+            return key.mask(self)  # a[mask]: the elements where the mask is set
+        key = self._expand_key(key)
+        if any(_is_index_array(k) for k in key):
+            return self._gather(key)
         shape, strides, offset = [], [], self._offset
         for n, st, k in zip(self.shape, self._strides, key):
             if k is True:
@@ -235,8 +300,154 @@ class NArray:
                 shape.append(cnt)
                 strides.append(st * step)
             else:
-                raise TypeError("index arrays are outside this path")
+                raise TypeError("unsupported index %r" % (k,))
         return self._view(shape, strides, offset)
+
+    def __setitem__(self, key, value):
+        """a[key] = value: a store into the view, or a scatter when the key holds
+        index arrays (reference: gen/tmpl/aset.c, narray/ndloop.c:1316)."""
+        if isinstance(key, NArray) and type(key).__name__ == "Bit":
+            raise TypeError("store through a mask is outside this path")
+        key = self._expand_key(key)
+        if any(_is_index_array(k) for k in key):
+            return self._scatter(key, value)
+        self[key].store(value)
+
+    # ---- index arrays (reference: narray/index.c:460-614 builds the view,
+    # narray/ndloop.c:1251-1330 stages it through a contiguous buffer)
+    def _stridx_view(self, key):
+        """The view a key with index arrays selects, as the launcher's descriptor:
+        one device array of byte offsets per indexed dimension, a stride for the rest.
+        Each indexed dimension selects independently (an outer product, not numpy's
+        zipped fancy indexing). Returns (descriptor, indexer, shape, keep-alives)."""
+        if type(self).__name__ == "Bit":
+            raise TypeError("index arrays on Bit are outside this path")
+        a = _lib.IArrayStridx()
+        shape, keep, offset, d = [], [], self._offset, 0
+        for n, st, k in zip(self.shape, self._strides, key):
+            if k is True:
+                k = slice(None)
+            if isinstance(k, numbers.Integral):
+                k = int(k)
+                if k < 0:
+                    k += n
+                if not 0 <= k < n:
+                    raise IndexError("index out of range")
+                offset += k * st
+                continue
+            if isinstance(k, slice):
+                start, stop, step = k.indices(n)
+                shape.append(len(range(start, stop, step)))
+                offset += start * st
+                a.stridx[d] = ((st * step) << 1) | 1
+            else:
+                pos = _index_positions(k, n)
+                buf = _upload_index(pos)
+                keep.append(buf)
+                if len(pos):
+                    if st < 0:
+                        # a reversed dimension counts from its far end (index.c:580-590)
+                        offset += st * (n - 1)
+                        call(_IX["aref_naview_index_stride_last"], buf.ptr, -st, n - 1, len(pos))
+                    else:
+                        call(_IX["aref_naview_index_stride"], buf.ptr, st, len(pos))
+                shape.append(len(pos))
+                a.stridx[d] = buf.ptr or 0
+            d += 1
+        a.ptr = (self._buf.ptr or 0) + offset
+        ix = _lib.Indexer()
+        ix.ndim = len(shape)
+        ix.total_size = _prod(shape)
+        for j, m in enumerate(shape):
+            ix.shape[j] = m
+        return a, ix, shape, keep
+
+    def _gather(self, key):
+        a, ix, shape, keep = self._stridx_view(key)
+        out = type(self)(*shape)
+        if out.size:
+            call(_IX["copy_to_buffer"], C.byref(a), C.byref(ix), out._buf.ptr, self.elmsz)
+        del keep
+        return out
+
+    def _scatter(self, key, value):
+        a, ix, shape, keep = self._stridx_view(key)
+        if (type(value) is type(self) and value.shape == tuple(shape)
+                and value._strides == _contiguous_strides(value.shape, self._unit())):
+            tmp = value  # already the contiguous buffer the scatter reads
+        else:
+            tmp = type(self)(*shape)
+            tmp.store(value)
+        if tmp.size:
+            call(_IX["copy_from_buffer"], C.byref(a), C.byref(ix), tmp._ptr(), self.elmsz)
+        del keep
+
+    def at(self, *keys):
+        """Elements at zipped positions: a.at([0, 1], [2, 3]) answers a[0, 2] and
+        a[1, 3] as a 1-D array (reference: narray/index.c:622-682,842-870). A key is an
+        index array or a range / slice; all must select the same number of positions."""
+        if type(self).__name__ == "Bit":
+            raise TypeError("index arrays on Bit are outside this path")
+        if len(keys) != self.ndim:
+            raise IndexError("the number of arguments must equal the number of dimensions")
+        sel = []
+        for k, n in zip(keys, self.shape):
+            if isinstance(k, range):
+                k = slice(k.start, k.stop, k.step)
+            if isinstance(k, slice):
+                start, stop, step = k.indices(n)
+                sel.append((None, start, step, len(range(start, stop, step))))
+            else:
+                pos = _index_positions(k, n)
+                sel.append((pos, 0, 0, len(pos)))
+        size = sel[-1][3] if sel else 0
+        if size == 0:
+            raise ShapeError("cannot get element of empty array")
+        if any(s[3] != size for s in sel):
+            raise ShapeError("index array sizes mismatch")
+        # the index array accumulates from the last dimension to the first
+        last_pos = sel[-1][0]
+        index = _upload_index(last_pos) if last_pos is not None else _Buffer(8 * size)
+        offset = self._offset
+        for i in range(self.ndim - 1, -1, -1):
+            pos, beg, step, _ = sel[i]
+            st, n = self._strides[i], self.shape[i]
+            first = i == self.ndim - 1
+            if pos is not None:
+                if st < 0 and first:
+                    # a reversed dimension counts from its far end (index.c:745-754)
+                    offset += st * (n - 1)
+                    call(_IX["aref_naview_index_stride_last"], index.ptr, -st, n - 1, size)
+                elif first:
+                    call(_IX["aref_nadata_index_stride"], index.ptr, st, size)
+                else:
+                    other = _upload_index(pos)
+                    call(_IX["at_nadata_index_stride_add"], index.ptr, other.ptr, st, size)
+            else:
+                offset += beg * st
+                name = "at_nadata_index_beg_step_stride" if first else "at_nadata_index_beg_step_stride_add"
+                call(_IX[name], index.ptr, 0, step, st, size)
+        out = type(self)(size)
+        call(_IX["copy_bytes"], (self._buf.ptr or 0) + offset, out._buf.ptr, 0, self.elmsz, index.ptr, None, size, self.elmsz)
+        return out
+
+    def diagonal(self, offset=0, axes=(-2, -1)):
+        """View of a diagonal as the last dimension (reference: narray/data.c:649-820;
+        for views without index arrays it is stride arithmetic only)."""
+        if self.ndim < 2:
+            raise DimensionError("less than 2-d array")
+        ax = [a + self.ndim if a < 0 else a for a in axes]
+        if len(ax) != 2 or ax[0] == ax[1] or not all(0 <= a < self.ndim for a in ax):
+            raise ValueError("invalid axes")
+        k0, k1 = (0, offset) if offset >= 0 else (-offset, 0)
+        n0, n1 = self.shape[ax[0]], self.shape[ax[1]]
+        if k0 >= n0 or k1 >= n1:
+            raise ShapeError("invalid diagonal offset(%d) for the shape" % offset)
+        length = min(n0 - k0, n1 - k1)
+        rest = [d for d in range(self.ndim) if d not in ax]
+        shape = [self.shape[d] for d in rest] + [length]
+        strides = [self._strides[d] for d in rest] + [self._strides[ax[0]] + self._strides[ax[1]]]
+        return self._view(shape, strides, self._offset + k0 * self._strides[ax[0]] + k1 * self._strides[ax[1]])
 
     def transpose(self, *axes):
         if len(axes) == 1 and isinstance(axes[0], (tuple, list)):

@@ -385,6 +385,30 @@ char *cumo_bit_where_scratch_new(void);
 void cumo_bit_where_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, size_t *idx, uint64_t n, int invert, char *out, size_t elmsz, uint64_t count, char *scratch);
 void cumo_bit_mask_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, size_t *idx, uint64_t n, size_t *out, size_t p2, ssize_t s2, size_t *idx2, char *scratch);
 
+/* Index-array views: arithmetic on device index arrays (narray/index_kernel.cu:87-173,
+ * host narray/index.c), the diagonal's index arrays and the 1-D indexed copy
+ * (narray/data_kernel.cu:134-164, host narray/data.c), and the gather / scatter
+ * between a view with index arrays and a contiguous buffer that ndloop stages such
+ * operands through (narray/ndloop_kernel.cu:46-93, host narray/ndloop.c:1251,1316).
+ * Index arrays hold byte offsets (size_t). */
+void cumo_na_index_aref_nadata_index_stride_kernel_launch(size_t *idx, ssize_t s1, uint64_t n);
+void cumo_na_index_aref_naview_index_index_kernel_launch(size_t *idx, size_t *idx1, uint64_t n);
+void cumo_na_index_aref_naview_index_stride_last_kernel_launch(size_t *idx, ssize_t s1, size_t last, uint64_t n);
+void cumo_na_index_aref_naview_index_stride_kernel_launch(size_t *idx, ssize_t s1, uint64_t n);
+void cumo_na_index_aref_naview_index_index_beg_step_kernel_launch(size_t *idx, size_t *idx1, size_t beg, ssize_t step, uint64_t n);
+void cumo_na_index_at_nadata_index_stride_add_kernel_launch(size_t *idx, size_t *idx1, ssize_t s1, uint64_t n);
+void cumo_na_index_at_nadata_index_beg_step_stride_kernel_launch(size_t *idx, size_t beg, ssize_t step, ssize_t s1, uint64_t n);
+void cumo_na_index_at_nadata_index_beg_step_stride_add_kernel_launch(size_t *idx, size_t beg, ssize_t step, ssize_t s1, uint64_t n);
+void cumo_na_index_at_naview_index_index_index_add_kernel_launch(size_t *idx, size_t *idx1, size_t *idx2, uint64_t n);
+void cumo_na_index_at_naview_index_index_beg_step_add_kernel_launch(size_t *idx, size_t *idx1, size_t beg, ssize_t step, uint64_t n);
+void cumo_na_index_at_naview_index_stride_last_add_kernel_launch(size_t *idx, ssize_t s1, size_t last, uint64_t n);
+void cumo_iter_copy_bytes_kernel_launch(char *p1, char *p2, ssize_t s1, ssize_t s2, size_t *idx1, size_t *idx2, uint64_t n, ssize_t elmsz);
+void cumo_na_diagonal_index_index_kernel_launch(size_t *idx, size_t *idx0, size_t *idx1, size_t k0, size_t k1, uint64_t n);
+void cumo_na_diagonal_index_stride_kernel_launch(size_t *idx, size_t *idx0, ssize_t s1, size_t k0, size_t k1, uint64_t n);
+void cumo_na_diagonal_stride_index_kernel_launch(size_t *idx, ssize_t s0, size_t *idx1, size_t k0, size_t k1, uint64_t n);
+void cumo_ndloop_copy_from_buffer_kernel_launch(cumo_na_iarray_stridx_t *a, cumo_na_indexer_t* indexer, char *buf, size_t elmsz);
+void cumo_ndloop_copy_to_buffer_kernel_launch(cumo_na_iarray_stridx_t *a, cumo_na_indexer_t* indexer, char *buf, size_t elmsz);
+
 /* ------------------------------------------------------------------------
  * 6. What this library adds (no counterpart symbol in the reference).
  * ---------------------------------------------------------------------- */
@@ -444,6 +468,22 @@ typedef struct {
     double   eps;
 } cumo_hip_fused_rows_t;
 int cumo_hip_fused_rows_kernel_launch(int type, int mode, const cumo_hip_fused_rows_t* rows);
+
+/* Product sums of many rows in one launch (the reference launches
+ * cumo_<type>_mulsum_reduce_kernel_launch once per row from a host loop,
+ * gen/tmpl/accum_binary.c:20-45): out[r] += sum_i p1[r][i] * p2[r][i] for rows of n
+ * contiguous elements, row r of an operand at p + r * row_step (0 repeats the row).
+ * type 0 SFloat, 1 DFloat, 2 Int32; nan skips NaN factors. Returns 1 when launched,
+ * 0 when the layout is outside what the kernel takes (n not a whole number of
+ * 128-bit vectors, operands or row steps not 16-byte aligned). */
+typedef struct {
+    uint64_t rows, n;
+    ssize_t  row_step1, row_step2, out_step;
+    char*    p1;
+    char*    p2;
+    char*    out;
+} cumo_hip_mulsum_rows_t;
+int cumo_hip_mulsum_rows_kernel_launch(int type, int nan, const cumo_hip_mulsum_rows_t* rows);
 
 /* out[i] = the element of a strided view at flat row-major position pos[i] (no
  * counterpart symbol in the reference, where a masked array is a view over an index

@@ -216,10 +216,12 @@ int cumo_hip_na_cum(const char* op, const cumo_hip_narray_t* x, unsigned int red
 
 /* z = the row-major positions of x's set bits (clear bits when invert), as Int32, or
  * Int64 for more than 2^32 - 1 elements (reference: gen/tmpl_bit/where.c:98-127). z
- * must come in with ptr == NULL. */
+ * normally comes in with ptr == NULL; a given z must be a contiguous 1-D array of that
+ * type and exactly as long as the count, or the call fails with a shape error. */
 int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t* z);
 /* z = the elements of x where mask is set, row-major (reference: gen/tmpl_bit/mask.c:96-167,
- * which answers a view over an index array; here a new array). Shapes must be equal. */
+ * which answers a view over an index array; here a new array). Shapes must be equal.
+ * A given z: as for where, with x's type. */
 int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
 
 /* Library additions: softmax and layer normalisation along the LAST dimension,

@@ -262,6 +262,16 @@ def test_mulsum_parity(tname, dt):
     # more inner runs than are launched one by one: the products go through the reduction engine
     hx, hy = make((3000, 40)), make((3000, 40))
     check(cls.cast(hx).mulsum(cls.cast(hy), axis=1).to_numpy(), hx, hy, 1, "3000 runs")
+    # every row in one launch: 16, 64 and 256 lanes per row, a repeated row operand, rows a step apart
+    for shape in ((5000, 8), (700, 512), (300, 4096), (64, 20000), (3, 1 << 16)):
+        hx, hy = make(shape), make(shape)
+        x, y = cls.cast(hx), cls.cast(hy)
+        check(x.mulsum(y, axis=1).to_numpy(), hx, hy, 1, ("rows", shape))
+        check(x.mulsum(y[0], axis=-1).to_numpy(), hx, hy[0], 1, ("rows, one operand repeated", shape))
+        check(x[::2].mulsum(y[1::2], axis=1).to_numpy(), np.ascontiguousarray(hx[::2]), np.ascontiguousarray(hy[1::2]), 1, ("every other row", shape))
+    hx, hy = make((6, 50, 128)), make((6, 50, 128))
+    check(cls.cast(hx).mulsum(cls.cast(hy), axis=2).to_numpy(), hx, hy, 2, "rows over two outer dimensions")
+    check(cls.cast(hx).mulsum(cls.cast(hy), axis=(1, 2)).to_numpy(), hx, hy, (1, 2), "two reduced dimensions as one run")
     # no reduced dimension left after broadcasting rules: the elementwise form
     hx, hy = make((5, 1)), make((5, 1))
     check(cls.cast(hx).mulsum(cls.cast(hy), axis=1).to_numpy(), hx, hy, 1, "runs of one element")

@@ -32,7 +32,7 @@ def test_exp_equals_the_double_exp_rounded_once_everywhere():
     parts = [
         rng.uniform(-104, 89, size=1 << 22),               # the whole range with finite, non-zero answers
         rng.uniform(-20, 5, size=1 << 22),                 # where softmax inputs live
-        rng.standard_normal(1 << 21) * 1e-3,               # around 1
+        rng.standard_normal(1 << 21) * 1e-3,               # near 1.0
         np.array([0.0, -0.0, 87.0, -87.0, 87.000001, -87.000001, 88.72283, 88.72284, 89.0, -87.33655, -103.97, -103.98,
                   -110.0, 1e-45, -1e-45, np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5, 1e-8]),
     ]

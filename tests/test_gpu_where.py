@@ -107,3 +107,27 @@ def test_where_and_mask_launchers_with_index_arrays_and_a_carried_cursor():
     assert (gm[:wantm.size] == wantm.astype(np.uint64)).all() and gm[wantm.size] == 0
     _lib.lib.cumo_cuda_runtime_free(scratch)
     free(pw, pidx, pout, pz, pm)
+
+
+def test_where_and_mask_into_a_given_result():
+    """A result array of exactly the count's length is written in place; any other length is a shape error."""
+    import ctypes as C
+    import cumo_amd
+    from cumo_amd import _lib
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((50, 70)).astype(np.float32)
+    d = cumo_amd.SFloat.cast(x)
+    m = d > 0.25
+    want_pos = np.flatnonzero(x > np.float32(0.25)).astype(np.int32)
+    pos = cumo_amd.Int32.zeros(len(want_pos))
+    md, zd = m._desc(), pos._desc()
+    _lib.call(_lib.lib.cumo_hip_na_where, C.byref(md), 0, C.byref(zd))
+    assert (pos.to_numpy() == want_pos).all()
+    vals = cumo_amd.SFloat.zeros(len(want_pos))
+    xd, vd = d._desc(), vals._desc()
+    _lib.call(_lib.lib.cumo_hip_na_mask, C.byref(md), C.byref(xd), C.byref(vd))
+    assert (vals.to_numpy() == x.ravel()[want_pos]).all()
+    short = cumo_amd.Int32.zeros(len(want_pos) - 1)
+    sd = short._desc()
+    with pytest.raises(cumo_amd.ShapeError):
+        _lib.call(_lib.lib.cumo_hip_na_where, C.byref(md), 0, C.byref(sd))
