@@ -9,12 +9,17 @@
 //
 // Three launches per run: every block counts the set bits of its contiguous range
 // of 32-bit chunks; one block turns the counts into output positions (and advances
-// the cursor); every block walks its range again and writes each chunk's positions
-// from where an exclusive scan over the block puts them. Blocks are 256 threads (4
-// wave64): the scan inside a block is a wave scan by shuffles plus four LDS slots.
+// the cursor); every block walks its range again, 256 chunks a round: an exclusive
+// scan over the block places each chunk's hits in a list in LDS, and consecutive
+// lanes then write the list out, so the stores of a wave are adjacent. Blocks are 256
+// threads (4 wave64): the scan inside a block is a wave scan by shuffles plus four LDS
+// slots.
 // A contiguous run reads whole words (two per chunk when the run starts inside a
 // word); strided and index-array runs gather bit by bit.
 #include "common.h"
+#include "div31.h"
+
+#include <type_traits>
 
 #include <cstring>
 
@@ -110,23 +115,31 @@ __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_
     uint64_t start = (uint64_t)blockIdx.x * cpb;
     if (start > nchunks) start = nchunks;
     const uint64_t end = (nchunks - start < cpb) ? nchunks : start + cpb;
+    // hits of one round (256 chunks, up to 8192 bits) are listed in LDS by their bit
+    // position within the round, then written out by consecutive lanes
+    __shared__ uint16_t hit[kWhBlock * 32];
     uint64_t off = block_sums[blockIdx.x];
     for (uint64_t c0 = start; c0 < end; c0 += kWhBlock) {
         const uint64_t c = c0 + threadIdx.x;
         uint32_t z = c < end ? wh_chunk(a, p, s, idx, n, c, contiguous, invert) : 0u;
         uint64_t total;
-        uint64_t o = off + wh_block_exscan((uint64_t)__popc(z), &total);
+        // the first barrier inside the scan also ends the previous round's reads of hit[]
+        uint32_t o = (uint32_t)wh_block_exscan((uint64_t)__popc(z), &total);
         while (z) {
-            const uint64_t j = c * 32 + (uint64_t)(__ffs((int)z) - 1);
-            if (MASK) {
-                reinterpret_cast<size_t*>(out)[o] = idx2 ? (p2 + idx2[j]) : (size_t)((int64_t)p2 + (int64_t)j * s2);
-            } else if (elmsz == 4) {
-                reinterpret_cast<int32_t*>(out)[o] = (int32_t)(count + j);
-            } else {
-                reinterpret_cast<int64_t*>(out)[o] = (int64_t)(count + j);
-            }
-            ++o;
+            hit[o++] = (uint16_t)(threadIdx.x * 32 + (unsigned)(__ffs((int)z) - 1));
             z &= z - 1;
+        }
+        __syncthreads();
+        for (uint32_t k = threadIdx.x; k < (uint32_t)total; k += kWhBlock) {
+            const uint64_t j = c0 * 32 + hit[k];
+            const uint64_t w = off + k;
+            if (MASK) {
+                reinterpret_cast<size_t*>(out)[w] = idx2 ? (p2 + idx2[j]) : (size_t)((int64_t)p2 + (int64_t)j * s2);
+            } else if (elmsz == 4) {
+                reinterpret_cast<int32_t*>(out)[w] = (int32_t)(count + j);
+            } else {
+                reinterpret_cast<int64_t*>(out)[w] = (int64_t)(count + j);
+            }
         }
         off += total;
     }
@@ -160,24 +173,40 @@ struct GatherParams {
     int ndim;
     uint64_t n;
     uint64_t shape[CUMO_NA_MAX_DIMENSION];
+    Div31 div[CUMO_NA_MAX_DIMENSION];
     int64_t step[CUMO_NA_MAX_DIMENSION];
     const char* in;
     char* out;
     const char* pos;
-    int pos_elmsz, elmsz;
 };
+// PW, EW: bytes per position and per element (4 or 8). SMALL: the view has fewer than
+// 2^31 elements, so a position splits over the dimensions with 32-bit multiplies.
+template <int PW, int EW, bool SMALL>
 __global__ __launch_bounds__(256) void gather_flat_kernel(GatherParams g) {
+    typedef typename std::conditional<PW == 4, uint32_t, uint64_t>::type P;
+    typedef typename std::conditional<EW == 4, uint32_t, uint64_t>::type E;
     for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < g.n; i += (uint64_t)gridDim.x * 256) {
-        uint64_t r = g.pos_elmsz == 4 ? (uint64_t)(uint32_t)reinterpret_cast<const int32_t*>(g.pos)[i] : (uint64_t)reinterpret_cast<const int64_t*>(g.pos)[i];
+        const uint64_t r0 = (uint64_t)reinterpret_cast<const P*>(g.pos)[i];
         int64_t off = 0;
-        for (int d = g.ndim - 1; d >= 0; --d) {
-            const uint64_t m = g.shape[d];
-            const uint64_t q = r / m;
-            off += (int64_t)(r - q * m) * g.step[d];
-            r = q;
+        if (SMALL) {
+            uint32_t r = (uint32_t)r0;
+            for (int d = g.ndim - 1; d > 0; --d) {
+                const uint32_t q = div31(r, g.div[d]);
+                off += (int64_t)(r - q * (uint32_t)g.shape[d]) * g.step[d];
+                r = q;
+            }
+            off += (int64_t)r * g.step[0];
+        } else {
+            uint64_t r = r0;
+            for (int d = g.ndim - 1; d > 0; --d) {
+                const uint64_t m = g.shape[d];
+                const uint64_t q = r / m;
+                off += (int64_t)(r - q * m) * g.step[d];
+                r = q;
+            }
+            off += (int64_t)r * g.step[0];
         }
-        if (g.elmsz == 4) reinterpret_cast<uint32_t*>(g.out)[i] = *reinterpret_cast<const uint32_t*>(g.in + off);
-        else reinterpret_cast<uint64_t*>(g.out)[i] = *reinterpret_cast<const uint64_t*>(g.in + off);
+        reinterpret_cast<E*>(g.out)[i] = *reinterpret_cast<const E*>(g.in + off);
     }
 }
 
@@ -215,20 +244,47 @@ void cumo_hip_gather_flat_kernel_launch(const cumo_hip_gather_flat_t* d) {
     if (!d || d->n == 0) return;
     GatherParams g;
     std::memset(&g, 0, sizeof(g));
-    g.ndim = d->ndim;
-    g.n = d->n;
+    // dimensions that follow one another in memory count as one; size-1 dimensions drop out
+    uint64_t total = 1;
+    int nd = 0;
     for (int k = 0; k < d->ndim && k < CUMO_NA_MAX_DIMENSION; ++k) {
-        g.shape[k] = d->shape[k];
-        g.step[k] = d->step[k];
+        total *= d->shape[k];
+        if (d->shape[k] == 1) continue;
+        if (nd > 0 && g.step[nd - 1] == (int64_t)d->step[k] * (int64_t)d->shape[k]) {
+            g.shape[nd - 1] *= d->shape[k];
+            g.step[nd - 1] = d->step[k];
+        } else {
+            g.shape[nd] = d->shape[k];
+            g.step[nd] = d->step[k];
+            ++nd;
+        }
     }
+    if (nd == 0) {
+        g.shape[0] = 1;
+        nd = 1;
+    }
+    g.ndim = nd;
+    const bool small = total < (1ull << 31);
+    if (small) {
+        for (int k = 0; k < nd; ++k) g.div[k] = div31_make((uint32_t)g.shape[k]);
+    }
+    g.n = d->n;
     g.in = d->in;
     g.out = d->out;
     g.pos = d->pos;
-    g.pos_elmsz = d->pos_elmsz;
-    g.elmsz = d->elmsz;
     uint64_t grid = (d->n + 255) / 256;
     if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(gather_flat_kernel, dim3((unsigned)grid), dim3(256), 0, current_stream(), g);
+    hipStream_t st = current_stream();
+#define WH_GATHER(PW, EW)                                                                                              \
+    do {                                                                                                               \
+        if (small) hipLaunchKernelGGL((gather_flat_kernel<PW, EW, true>), dim3((unsigned)grid), dim3(256), 0, st, g);  \
+        else hipLaunchKernelGGL((gather_flat_kernel<PW, EW, false>), dim3((unsigned)grid), dim3(256), 0, st, g);       \
+    } while (0)
+    if (d->pos_elmsz == 4 && d->elmsz == 4) WH_GATHER(4, 4);
+    else if (d->pos_elmsz == 4) WH_GATHER(4, 8);
+    else if (d->elmsz == 4) WH_GATHER(8, 4);
+    else WH_GATHER(8, 8);
+#undef WH_GATHER
     cumo_cuda_runtime_check_kernel_launch();
 }
 
