@@ -249,6 +249,35 @@ def measure_config(name, cumo, lib, iters, warmup):
     return rows
 
 
+def measure_host_io(lib, mib=256, reps=5):
+    """Read-back and ingest of one contiguous array between pageable host memory and the
+    device: the library's staged copies beside the runtime's own pageable path (what a
+    plain hipMemcpy gives). PCIe-bound: GB/s here are not comparable with the HBM figures."""
+    from cumo_amd import _lib
+    n = mib << 20
+    h = np.random.default_rng(0).integers(0, 255, n, dtype=np.uint8)
+    back = np.empty_like(h)
+    p = _lib.call(lib.cumo_cuda_runtime_malloc, n)
+    out = {"bytes": n, "unit": "GB/s", "host_memory": "pageable"}
+    for name, f in (("ingest_staged", lambda: lib.cumo_hip_copy_from_host(p, h.ctypes.data, n)),
+                    ("ingest_runtime_memcpy", lambda: lib.cumo_hip_memcpy_h2d(p, h.ctypes.data, n)),
+                    ("readback_staged", lambda: lib.cumo_hip_copy_to_host(back.ctypes.data, p, n)),
+                    ("readback_runtime_memcpy", lambda: lib.cumo_hip_memcpy_d2h(back.ctypes.data, p, n))):
+        f()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            f()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        out[name] = round(n / ts[len(ts) // 2] / 1e9, 2)
+    _lib.check()
+    if not (back == h).all():
+        raise SystemExit("bench: host round trip returned different bytes")
+    lib.cumo_cuda_runtime_free(p)
+    return out
+
+
 def cpu_baseline_c2(budget_s=12.0):
     """Numo-shaped single-thread C loops (the oracle's row loops) on the same C2
     workload, on this machine's host cores. A bounded number of passes."""
@@ -411,6 +440,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline_c2()
     if per_config:
         out["per_config"] = per_config
+        out["host_io"] = measure_host_io(lib)
     print(json.dumps(out))
 
 

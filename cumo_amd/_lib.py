@@ -136,6 +136,8 @@ _sig = {
     "cumo_hip_memcpy_h2d": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_memcpy_d2h": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_memset": (None, [C.c_void_p, C.c_int, C.c_size_t]),
+    "cumo_hip_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "cumo_hip_copy_from_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_pool_malloc": (C.c_int, [C.c_size_t, C.c_void_p, P(C.c_void_p)]),
     "cumo_hip_pool_free": (C.c_int, [C.c_void_p]),
     "cumo_hip_pool_free_all_blocks": (None, []),
@@ -184,6 +186,9 @@ _sig = {
     "cumo_hip_na_store": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_copy": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_fill": (C.c_int, [P(NArrayDesc), C.c_double]),
+    "cumo_hip_na_to_host": (C.c_int, [P(NArrayDesc), C.c_void_p, C.c_size_t]),
+    "cumo_hip_na_from_host": (C.c_int, [P(NArrayDesc), C.c_void_p, C.c_size_t]),
+    "cumo_hip_na_extract": (C.c_int, [P(NArrayDesc), P(C.c_size_t), C.c_void_p]),
     "cumo_hip_na_reduce": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_uint, C.c_int, C.c_int, P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_bit_binary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_bit_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),

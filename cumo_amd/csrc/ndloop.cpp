@@ -1744,6 +1744,80 @@ int cumo_hip_na_copy(const cumo_hip_narray_t* src, cumo_hip_narray_t* dst) {
     return cumo_hip_na_ndloop(&nf, in, out, 0, NULL);
 }
 
+// ---- host read-back and ingest (narray/narray.c:1391-1560 to_binary / from_binary /
+// store_binary, gen/tmpl/extract_cpu.c, gen/tmpl/aref_cpu.c): the reference reads and
+// writes managed memory after a device synchronisation; here the bytes cross by an
+// explicit transfer, staged through a contiguous copy when the view is not contiguous
+namespace {
+// bytes of the view's elements laid out row-major (Bit: whole bytes)
+size_t packed_bytes(const NA* a) {
+    const size_t n = total_of(a);
+    return a->type == CUMO_HIP_BIT ? (n + 7) / 8 : n * (size_t)kElmsz[a->type];
+}
+// a view whose bytes already lie as the transfer wants them
+bool directly_addressable(const NA* a) { return is_contiguous(a) && (a->type != CUMO_HIP_BIT || a->offset % 8 == 0); }
+char* first_byte(const NA* a) { return a->ptr + (a->type == CUMO_HIP_BIT ? a->offset / 8 : a->offset); }
+}  // namespace
+
+// host[0, nbytes) = the first nbytes of x's elements in row-major order
+int cumo_hip_na_to_host(const cumo_hip_narray_t* x, void* host, size_t nbytes) {
+    int rc = check_view(x, "source");
+    if (rc) return rc;
+    if (nbytes > packed_bytes(x)) return fail(CUMO_HIP_ERROR_ARGUMENT, "to_host: more bytes asked for than the array holds");
+    if (nbytes == 0) return CUMO_HIP_OK;
+    if (!host) return fail(CUMO_HIP_ERROR_ARGUMENT, "to_host: no host memory given");
+    if (directly_addressable(x)) return cumo_hip_copy_to_host(host, first_byte(x), nbytes);
+    NA tmp;
+    tmp.ptr = NULL;
+    rc = cumo_hip_na_copy(x, &tmp);  // the dup of narray.c:1543
+    if (!rc) rc = cumo_hip_copy_to_host(host, tmp.ptr, nbytes);
+    free_tmp(&tmp);
+    return rc;
+}
+
+// x's elements in row-major order = host[0, nbytes); nbytes must cover the whole view
+int cumo_hip_na_from_host(cumo_hip_narray_t* x, const void* host, size_t nbytes) {
+    int rc = check_view(x, "destination");
+    if (rc) return rc;
+    const size_t need = packed_bytes(x);
+    if (nbytes < need) return fail(CUMO_HIP_ERROR_ARGUMENT, "string is too short to store");
+    if (need == 0) return CUMO_HIP_OK;
+    if (!host) return fail(CUMO_HIP_ERROR_ARGUMENT, "from_host: no host memory given");
+    if (!x->ptr) return fail(CUMO_HIP_ERROR_ARGUMENT, "from_host: destination has no memory");
+    if (directly_addressable(x) && (x->type != CUMO_HIP_BIT || total_of(x) % 8 == 0)) return cumo_hip_copy_from_host(first_byte(x), host, need);
+    NA tmp;
+    tmp.ptr = NULL;
+    rc = cumo_hip_na_alloc(&tmp, x->type, x->ndim, x->shape);
+    if (!rc) rc = cumo_hip_copy_from_host(tmp.ptr, host, need);
+    if (!rc) rc = cumo_hip_na_store(x, &tmp);
+    free_tmp(&tmp);
+    return rc;
+}
+
+// out = the element at index[0 .. ndim) (NULL: the only element of a one-element
+// array), as the element type; for Bit one unsigned char, 0 or 1
+int cumo_hip_na_extract(const cumo_hip_narray_t* x, const size_t* index, void* out) {
+    int rc = check_view(x, "source");
+    if (rc) return rc;
+    if (!out) return fail(CUMO_HIP_ERROR_ARGUMENT, "extract: no host memory given");
+    ssize_t off = x->offset;
+    if (index) {
+        for (int d = 0; d < x->ndim; ++d) {
+            if (index[d] >= x->shape[d]) return fail(CUMO_HIP_ERROR_ARGUMENT, "index out of range");
+            off += (ssize_t)index[d] * x->stride[d];
+        }
+    } else if (total_of(x) != 1) {
+        return fail(CUMO_HIP_ERROR_SHAPE, "not a single-element array");
+    }
+    if (x->type == CUMO_HIP_BIT) {
+        CUMO_BIT_DIGIT w = 0;
+        rc = cumo_hip_copy_to_host(&w, x->ptr + (off / 32) * 4, sizeof(w));
+        if (!rc) *(unsigned char*)out = (unsigned char)((w >> (off % 32)) & 1u);
+        return rc;
+    }
+    return cumo_hip_copy_to_host(out, x->ptr + off, (size_t)kElmsz[x->type]);
+}
+
 int cumo_hip_na_fill(cumo_hip_narray_t* dst, double value) {
     int rc = check_arith(dst);
     if (rc) return rc;

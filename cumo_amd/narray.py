@@ -224,7 +224,7 @@ class NArray:
         arr = np.ascontiguousarray(np.asarray(data, dtype=cls.np_dtype))
         a = cls(*arr.shape)
         if arr.nbytes:
-            call(_L.cumo_hip_memcpy_h2d, a._buf.ptr, arr.ctypes.data, arr.nbytes)
+            call(_L.cumo_hip_copy_from_host, a._buf.ptr, arr.ctypes.data, arr.nbytes)
         return a
 
     from_numpy = cast
@@ -519,13 +519,78 @@ class NArray:
         _run(_L.cumo_hip_na_fill, C.byref(d), float(value))
         return self
 
-    # ---- host read-back ------------------------------------------------------
+    # ---- host read-back and ingest ------------------------------------------------
     def to_numpy(self):
-        src = self if (self.is_contiguous() and self._strides == _contiguous_strides(self.shape, self._unit())) else self.copy()
         out = np.empty(self.shape, dtype=self.np_dtype)
         if out.nbytes:
-            call(_L.cumo_hip_memcpy_d2h, out.ctypes.data, src._ptr(), out.nbytes)
+            d = self._desc()
+            call(_L.cumo_hip_na_to_host, C.byref(d), out.ctypes.data, out.nbytes)
         return out
+
+    def byte_size(self):
+        return self.size * self.elmsz
+
+    def to_binary(self):
+        """The elements' bytes in row-major order (reference: narray/narray.c:1530-1560)."""
+        out = bytearray(self.byte_size())
+        if out:
+            d = self._desc()
+            call(_L.cumo_hip_na_to_host, C.byref(d), (C.c_char * len(out)).from_buffer(out), len(out))
+        return bytes(out)
+
+    to_string = to_binary
+
+    @classmethod
+    def from_binary(cls, data, shape=None):
+        """reference: narray/narray.c:1391-1461 -- without a shape, as many whole
+        elements as the string holds; with one, the string may be longer, never shorter."""
+        data = bytes(data)
+        unit = cls.elmsz if cls.elmsz else 0.125
+        if shape is None:
+            n = int(len(data) // unit)
+            if n == 0:
+                raise ValueError("string is empty or too short")
+            shape = (n,)
+        elif isinstance(shape, numbers.Integral):
+            shape = (int(shape),)
+        a = cls(*shape)
+        if int(np.ceil(a.size * unit)) > len(data):
+            raise ValueError("specified size is too large")
+        a.store_binary(data)
+        return a
+
+    from_string = from_binary
+
+    def store_binary(self, data, offset=0):
+        """reference: narray/narray.c:1474-1521; answers the number of bytes stored."""
+        data = bytes(data)
+        if len(data) < offset:
+            raise ValueError("offset is larger than string length")
+        need = self.byte_size()
+        if need > len(data) - offset:
+            raise ValueError("string is too short to store")
+        if need:
+            buf = (C.c_char * need).from_buffer_copy(data, offset)
+            d = self._desc()
+            call(_L.cumo_hip_na_from_host, C.byref(d), buf, need)
+        return need
+
+    def aref_cpu(self, *index):
+        """One element read back to the host (reference: gen/tmpl/aref_cpu.c)."""
+        if len(index) != self.ndim:
+            raise IndexError("the number of indices must equal the number of dimensions")
+        idx = (C.c_size_t * max(self.ndim, 1))()
+        for d, (k, n) in enumerate(zip(index, self.shape)):
+            k = int(k)
+            if k < 0:
+                k += n
+            if not 0 <= k < n:
+                raise IndexError("index out of range")
+            idx[d] = k
+        out = np.zeros(1, dtype=self.np_dtype)
+        d = self._desc()
+        call(_L.cumo_hip_na_extract, C.byref(d), idx, out.ctypes.data)
+        return out[0].item()
 
     def to_a(self):
         return self.to_numpy().tolist()
@@ -534,7 +599,10 @@ class NArray:
         """reference: gen/tmpl/extract_cpu.c:17-23 -- a 0-dim array answers its element."""
         if self.size != 1:
             raise ValueError("not a 0-dim / single-element array")
-        return self.to_numpy().reshape(()).item()
+        out = np.zeros(1, dtype=self.np_dtype)
+        d = self._desc()
+        call(_L.cumo_hip_na_extract, C.byref(d), None, out.ctypes.data)
+        return out[0].item()
 
     def __float__(self):
         return float(self.extract_cpu())
@@ -822,11 +890,16 @@ class Bit(NArray):
             call(_L.cumo_hip_memcpy_d2h, words.ctypes.data, self._buf.ptr, nbytes)
         return words
 
+    def byte_size(self):
+        return (self.size + 7) // 8
+
     def to_numpy(self):
-        src = self if (self._offset == 0 and self._strides == _contiguous_strides(self.shape, 1)) else self.copy()
-        words = src._raw_words()
-        bits = np.unpackbits(words.view(np.uint8), bitorder="little")[:self.size]
+        packed = np.frombuffer(self.to_binary(), dtype=np.uint8)
+        bits = np.unpackbits(packed, bitorder="little")[:self.size]
         return bits.reshape(self.shape).astype(np.uint8)
+
+    def aref_cpu(self, *index):
+        return int(NArray.aref_cpu(self, *index))
 
     def fill(self, value):
         raise TypeError("Bit#fill is outside this path")

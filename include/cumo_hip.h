@@ -536,6 +536,16 @@ void  cumo_hip_event_destroy(void* event);
 void  cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n);
 void  cumo_hip_memcpy_d2h(void* dst, const void* src, size_t n);
 void  cumo_hip_memset(void* dst, int byte, size_t n);
+/* The same copies for any size, with CUMO_HIP_OK or an error kind as the result:
+ * pageable host memory moves through a ring of four pinned staging buffers
+ * (CUMO_HIP_STAGE_MIB each, default 8) so that the DMA over PCIe overlaps the host-side
+ * memcpy, which CUMO_HIP_COPY_THREADS threads share (default 4); pinned host memory
+ * goes to the DMA engine directly. Ordered on the current stream after the work
+ * already queued; both return when the bytes have arrived. These stand where the
+ * reference's host code memcpys from / to managed memory after cudaDeviceSynchronize
+ * (narray/narray.c:1455-1460,1514-1518,1551-1557). */
+int   cumo_hip_copy_to_host(void* dst_host, const void* src_device, size_t n);
+int   cumo_hip_copy_from_host(void* dst_device, const void* src_host, size_t n);
 
 /* Memory pool (replaces cumo::internal::MemoryPool, cuda/memory_pool_impl.hpp:160-435).
  * Returns CUMO_HIP_OK or an error kind; never raises. */

@@ -209,6 +209,20 @@ int cumo_hip_na_reduce(const char* op, const cumo_hip_narray_t* x, unsigned int 
  * The result has the higher type of the two (Int32 stays Int32, wrapping). */
 int cumo_hip_na_mulsum(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, unsigned int reduce, int keepdims, int nan,
                        cumo_hip_narray_t* z);
+/* Host read-back and ingest of a view (reference: narray/narray.c:1391-1560
+ * from_binary / store_binary / to_binary, gen/tmpl/extract_cpu.c, aref_cpu.c, which
+ * touch managed memory from the host). The host side is the view's elements in
+ * row-major order, densely packed (Bit: eight to a byte, the first in bit 0). A view
+ * that is not contiguous is staged through a contiguous copy on the device.
+ *   to_host    host[0,nbytes) = the first nbytes of x; nbytes may not exceed x's size
+ *   from_host  x = host[0, x's size); nbytes may be larger, never smaller
+ *              ("string is too short to store", narray.c:1507)
+ *   extract    out = the element at index[0..ndim) (NULL: the single element of a
+ *              one-element array); Bit answers one unsigned char */
+int cumo_hip_na_to_host(const cumo_hip_narray_t* x, void* host, size_t nbytes);
+int cumo_hip_na_from_host(cumo_hip_narray_t* x, const void* host, size_t nbytes);
+int cumo_hip_na_extract(const cumo_hip_narray_t* x, const size_t* index, void* out);
+
 /* op "cumsum" or "cumprod": the running value along the dimensions in `reduce` taken
  * together in row-major order (0 = all); z has x's shape and type (reference:
  * gen/tmpl/cum.c:48-80). nan: NaN elements are skipped (leading ones stay NaN). */
