@@ -18,6 +18,11 @@ void report_hip_error(hipError_t status, const char* what);
 
 hipStream_t current_stream();
 
+// Stream capture (graph.cpp): while a capture is open, released memory stays with the
+// graph being recorded, and the pool hands blocks across streams without events.
+bool capture_defer_free(char* ptr);
+bool capture_active();
+
 static inline bool hip_ok(hipError_t status, const char* what) {
     if (status == hipSuccess) return true;
     report_hip_error(status, what);
