@@ -71,6 +71,28 @@ template <class T> __device__ __forceinline__ T fr_sqrt(T x) { return (T)sqrt((d
 // any-NaN max is NaN on the device: narray_test.rb:2551-2560)
 template <class T> __device__ __forceinline__ T fr_max_nan(T a, T b) { return (a != a) ? a : ((b != b) ? b : (a > b ? a : b)); }
 
+template <class T> __device__ __forceinline__ T fr_fmax(T a, T b);
+template <> __device__ __forceinline__ float fr_fmax<float>(float a, float b) { return __builtin_fmaxf(a, b); }
+template <> __device__ __forceinline__ double fr_fmax<double>(double a, double b) { return __builtin_fmax(a, b); }
+
+// x / s for many x and one s, with the result of the IEEE division in T.
+// float: x / s = float(double(x) * (1.0 / double(s))). The product is within 2^-52 of
+// the quotient, while the quotient of two 24-bit numbers is never closer than 2^-49
+// (relative) to the midpoint of two floats unless it is a float itself, so the one
+// rounding to float lands where the division's does; zero, infinity and NaN behave
+// alike on both routes, and a subnormal quotient is rounded once by the conversion.
+template <class T> struct FrDivisor;
+template <> struct FrDivisor<float> {
+    double r;
+    __device__ __forceinline__ explicit FrDivisor(float s) : r(1.0 / (double)s) {}
+    __device__ __forceinline__ float divide(float x) const { return (float)((double)x * r); }
+};
+template <> struct FrDivisor<double> {
+    double s;
+    __device__ __forceinline__ explicit FrDivisor(double s_) : s(s_) {}
+    __device__ __forceinline__ double divide(double x) const { return x / s; }
+};
+
 struct FusedRowsParams {
     uint64_t rows, n;
     int64_t in_row_step, out_row_step;  // bytes
@@ -107,13 +129,22 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
             x[k].q = NT ? __builtin_nontemporal_load(ld) : *ld;
         }
         if constexpr (MODE == 0) {
-            // lanes without data hold a copy of the row's first vector: harmless in a max
-            T m = x[0].t[0];
+            // Lanes without data hold -inf: neutral in the max, and exp(-inf - m) adds 0 to the sum.
+            // The max keeps the larger non-NaN value per element and notes NaN apart (one maximum and
+            // one compare per element); a NaN anywhere then replaces the row's max, as in the reduction.
+            T m = -INFINITY;
+            bool any_nan = false;
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
 #pragma unroll
-                for (int j = 0; j < V; ++j) m = fr_max_nan(m, x[k].t[j]);
+                for (int j = 0; j < V; ++j) {
+                    const T v = have[k] ? x[k].t[j] : (T)-INFINITY;
+                    x[k].t[j] = v;
+                    any_nan |= (v != v);
+                    m = fr_fmax(m, v);
+                }
             }
+            if (any_nan) m = (T)NAN;
             m = fr_allreduce<T, TPR>(m, [](T a, T b) { return fr_max_nan(a, b); });
             T s = 0;
 #pragma unroll
@@ -122,15 +153,16 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
                 for (int j = 0; j < V; ++j) {
                     const T e = fr_exp<T>(x[k].t[j] - m);
                     x[k].t[j] = e;
-                    if (have[k]) s += e;
+                    s += e;
                 }
             }
             s = fr_allreduce<T, TPR>(s, [](T a, T b) { return a + b; });
+            const FrDivisor<T> by_s(s);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
                 if (have[k]) {
 #pragma unroll
-                    for (int j = 0; j < V; ++j) x[k].t[j] = x[k].t[j] / s;
+                    for (int j = 0; j < V; ++j) x[k].t[j] = by_s.divide(x[k].t[j]);
                     const uint64_t col = ((uint64_t)k * TPR + lane_r) * V;
                     u4* st = reinterpret_cast<u4*>(dst + col * sizeof(T));
                     if (NT) __builtin_nontemporal_store(x[k].q, st);
