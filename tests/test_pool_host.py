@@ -182,3 +182,27 @@ def test_threads():
     n = L.cumo_hip_pool_n_free_blocks()
     L.cumo_hip_pool_free_all_blocks()
     assert L.cumo_hip_pool_total_bytes() == 0, n
+
+
+def test_large_allocations_are_cut_on_two_mebibyte_boundaries(host_pool):
+    """An array of 2 MiB or more taken out of a larger free chunk starts on a 2 MiB
+    boundary; what lies before it stays free and everything merges back."""
+    MIB = 1 << 20
+    rc, block = malloc(9 * MIB + ROUND)   # the host heap gives no particular alignment
+    assert rc == 0
+    L.cumo_hip_pool_free(block)
+    assert L.cumo_hip_pool_n_free_blocks() == 1
+    rc, a = malloc(4 * MIB)
+    assert rc == 0 and a % (2 * MIB) == 0
+    assert block <= a < block + 2 * MIB
+    rc, b = malloc(2 * MIB)
+    assert rc == 0 and b % (2 * MIB) == 0 and b == a + 4 * MIB
+    rc, small = malloc(ROUND)                 # small requests keep taking the best fit as it lies
+    assert rc == 0
+    for q in (a, b, small):
+        assert L.cumo_hip_pool_free(q) == 0
+    assert L.cumo_hip_pool_n_free_blocks() == 1 and L.cumo_hip_pool_used_bytes() == 0
+    assert L.cumo_hip_pool_free_bytes() == 9 * MIB + ROUND
+    rc, again = malloc(9 * MIB + ROUND)       # the whole block again, from its start
+    assert rc == 0 and again == block
+    L.cumo_hip_pool_free(again)
