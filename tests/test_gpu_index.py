@@ -299,3 +299,33 @@ def test_diagonal_views():
     assert d.diagonal().sum(axis=-1).to_a() == np.diagonal(x, 0, -2, -1).sum(axis=-1).tolist()
     with pytest.raises(cumo_amd.ShapeError):
         d.diagonal(7)
+
+
+def test_gather_of_more_than_two_to_the_31_elements():
+    """Past 2^31 elements the flat position no longer fits the 32-bit split: one-byte
+    elements, a repeated first dimension (stride 0) and an index array on the last."""
+    from cumo_amd import _lib
+    rng = np.random.default_rng(12)
+    inner, outer = 1 << 15, (1 << 16) + 1
+    src = rng.integers(0, 256, inner, dtype=np.uint8)
+    perm = rng.permutation(inner)
+    psrc, pidx = dev(src), dev(u64(perm))
+    total = inner * outer
+    assert total > (1 << 31)
+    pbuf = _lib.call(_lib.lib.cumo_cuda_runtime_malloc, total)
+    a = stridx_array(psrc, [0, ("i", pidx)])
+    ix = indexer((outer, inner))
+    to_buf = _lib.fn("cumo_ndloop_copy_to_buffer_kernel_launch", None, [P(_lib.IArrayStridx), P(_lib.Indexer), V, SZ])
+    _lib.call(to_buf, C.byref(a), C.byref(ix), pbuf, 1)
+    want_row = src[perm]
+    # the first rows, the last rows (beyond 2^31) and a few in between
+    for r in (0, 1, 12345, outer - 2, outer - 1):
+        got = np.empty(inner, dtype=np.uint8)
+        _lib.call(_lib.lib.cumo_hip_copy_to_host, got.ctypes.data, pbuf + r * inner, inner)
+        assert (got == want_row).all(), r
+    # and everything, by a checksum of the whole buffer against outer * sum(row)
+    whole = np.empty(total, dtype=np.uint8)
+    _lib.call(_lib.lib.cumo_hip_copy_to_host, whole.ctypes.data, pbuf, total)
+    assert int(whole.sum(dtype=np.uint64)) == outer * int(want_row.sum(dtype=np.uint64))
+    assert (whole.reshape(outer, inner)[::4099] == want_row).all()
+    free(psrc, pidx, pbuf)
