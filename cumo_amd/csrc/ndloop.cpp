@@ -1498,7 +1498,11 @@ int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t*
     rc = cumo_hip_na_bit_count(x, 0, 0, invert, &cnt);
     if (rc) return rc;
     uint64_t n_hit = 0;
-    cumo_hip_memcpy_d2h(&n_hit, cnt.ptr + cnt.offset, sizeof(n_hit));
+    rc = cumo_hip_copy_to_host(&n_hit, cnt.ptr + cnt.offset, sizeof(n_hit));
+    if (rc) {
+        free_tmp(&cnt);
+        return rc;
+    }
     free_tmp(&cnt);
     const size_t total = total_of(x);
     const int itype = total > 4294967295ull ? CUMO_HIP_INT64 : CUMO_HIP_INT32;

@@ -194,6 +194,13 @@ void to_host_locked(Stage* s, hipStream_t st, char* dst, const char* src, size_t
     }
     const size_t sb = s->slot_bytes;
     const size_t chunks = (n + sb - 1) / sb;
+    if (chunks == 1) {
+        // one buffer: wait for the stream itself rather than for an event recorded on it
+        if (err->check(hipMemcpyAsync(s->buf[0], src, n, hipMemcpyDeviceToHost, st), "hipMemcpyAsync(d2h)") &&
+            err->check(hipStreamSynchronize(st), "hipStreamSynchronize"))
+            host_copy(s, dst, s->buf[0], n);
+        return;
+    }
     auto issue = [&](size_t c) -> bool {
         const size_t off = c * sb, len = (n - off < sb) ? n - off : sb;
         const int k = (int)(c % kSlots);

@@ -148,7 +148,7 @@ def _upload_index(pos):
     buf = _Buffer(8 * max(len(pos), 1))
     if len(pos):
         pos = np.ascontiguousarray(pos, dtype=np.uint64)
-        call(_L.cumo_hip_memcpy_h2d, buf.ptr, pos.ctypes.data, pos.nbytes)
+        call(_L.cumo_hip_copy_from_host, buf.ptr, pos.ctypes.data, pos.nbytes)
     return buf
 
 
@@ -877,7 +877,7 @@ class Bit(NArray):
             bits = np.packbits(arr.reshape(-1), bitorder="little")
             words = np.zeros(((n + 31) // 32) * 4, dtype=np.uint8)
             words[:bits.size] = bits
-            call(_L.cumo_hip_memcpy_h2d, a._buf.ptr, words.ctypes.data, words.nbytes)
+            call(_L.cumo_hip_copy_from_host, a._buf.ptr, words.ctypes.data, words.nbytes)
         return a
 
     from_numpy = cast
@@ -887,7 +887,7 @@ class Bit(NArray):
         nbytes = self._buf.nbytes
         words = np.zeros(nbytes // 4, dtype=np.uint32)
         if nbytes:
-            call(_L.cumo_hip_memcpy_d2h, words.ctypes.data, self._buf.ptr, nbytes)
+            call(_L.cumo_hip_copy_to_host, words.ctypes.data, self._buf.ptr, nbytes)
         return words
 
     def byte_size(self):
