@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # counter's reading for --pmc-calibration's plain 256 MiB copy (FETCH_SIZE x 1.9998,
 # WRITE_SIZE x 0.9996): 131137 KiB fetched + 131024 KiB written. The figures and
 # the commands are in profiles/ew_rows2_add_f64_c2_hbm_traffic.txt.
-C2_ADD_TRAFFIC_BYTES = 268452414
+C2_ADD_TRAFFIC_BYTES = 268457021
 METRIC = "achieved HBM GB/s (% of MI355X peak) and GElem/s vs Numo CPU, per config"
 MIB = 1 << 20
 
@@ -359,6 +359,7 @@ def main():
     ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the host transfer and recorded-chain measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch a plain contiguous copy of known size (256 MiB in, 256 MiB out) five times, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command can scale its counters by it")
@@ -474,8 +475,9 @@ def main():
         out["cpu_baseline"] = cpu_baseline_c2()
     if per_config:
         out["per_config"] = per_config
-        out["host_io"] = measure_host_io(lib)
-        out["graph"] = measure_graph(cumo_amd, lib)
+        if not args.no_extras:
+            out["host_io"] = measure_host_io(lib)
+            out["graph"] = measure_graph(cumo_amd, lib)
     print(json.dumps(out))
 
 
