@@ -12,6 +12,8 @@
 #include "plan.h"
 
 #include <cstring>
+#include <mutex>
+#include <unordered_map>
 
 using namespace cumo_hip;
 
@@ -157,6 +159,65 @@ __global__ __launch_bounds__(kBlock) void bit_count_words_kernel(const CUMO_BIT_
     }
     const uint64_t t = block_sum_u64(c);
     if (threadIdx.x == 0 && t) atomicAdd(out, (unsigned long long)t);
+}
+
+// The same count in one launch that needs no zeroed result: every block adds its total
+// and a "one more block done" mark to a ticket word with ONE atomic (count in the low
+// 44 bits, blocks done above them), so the block whose atomic answers "all others were
+// here before me" also holds the grand total, stores it and puts the ticket back to 0.
+// Nothing but that single word is shared between blocks, so no fence is needed.
+// Lanes read 128 bits; the words of the run's first and last vector are masked one by one.
+constexpr int kTicketSlots = 64;
+constexpr int kTicketShift = 44;
+__device__ unsigned long long g_count_ticket[kTicketSlots];
+
+template <bool COUNT_FALSE>
+__global__ __launch_bounds__(kBlock) void bit_count_words_store_kernel(const CUMO_BIT_DIGIT* a, uint64_t p1, uint64_t n, unsigned long long* ticket,
+                                                                       unsigned long long* out) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint64_t endbit = p1 + n;
+    const uint64_t w0 = p1 >> 5, w1 = (endbit + 31) >> 5;  // a is 16-byte aligned
+    const uint64_t v0 = w0 >> 2, v1 = (w1 + 3) >> 2;
+    uint64_t c = 0;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    uint64_t v = v0 + (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    // four interior vectors per lane in flight
+    for (; v > v0 && v + 3 * stride + 1 < v1 - 1; v += 4 * stride) {
+        u4 x[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const u4*>(a + ((v + u * stride) << 2));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (COUNT_FALSE) x[u] = ~x[u];
+            c += (uint64_t)(__popc(x[u].x) + __popc(x[u].y) + __popc(x[u].z) + __popc(x[u].w));
+        }
+    }
+    for (; v < v1; v += stride) {
+        const uint64_t w = v << 2;
+        if (w >= w0 + 1 && w + 4 < w1) {  // four whole words of the run
+            u4 x = *reinterpret_cast<const u4*>(a + w);
+            if (COUNT_FALSE) x = ~x;
+            c += (uint64_t)(__popc(x.x) + __popc(x.y) + __popc(x.z) + __popc(x.w));
+        } else {
+            for (uint64_t k = (w < w0 ? w0 : w); k < w + 4 && k < w1; ++k) {
+                uint32_t x = a[k];
+                if (COUNT_FALSE) x = ~x;
+                const unsigned lo = (k == w0) ? (unsigned)(p1 & 31) : 0u;
+                const unsigned hi = ((k + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (k << 5));
+                x &= low_bits(hi) & ~low_bits(lo);
+                c += (uint64_t)__popc(x);
+            }
+        }
+    }
+    const uint64_t t = block_sum_u64(c);
+    if (threadIdx.x == 0) {
+        const unsigned long long mine = (1ull << kTicketShift) | (unsigned long long)t;
+        const unsigned long long before = atomicAdd(ticket, mine);
+        if ((before >> kTicketShift) == (unsigned long long)gridDim.x - 1) {
+            *out = (before + mine) & ((1ull << kTicketShift) - 1);
+            atomicExch(ticket, 0ull);
+        }
+    }
 }
 
 // any stride or an index array, all into one counter
@@ -374,6 +435,52 @@ CUMO_DEF_BIT_COUNT(count_false, true)
 CUMO_DEF_STORE_BIT(sfloat, float)
 CUMO_DEF_STORE_BIT(dfloat, double)
 CUMO_DEF_STORE_BIT(int32, int32_t)
+
+// *out = the number of set (or clear) bits of the contiguous run [pos, pos + n) of a, in
+// one launch and without a zeroed result. Returns 1 when launched, 0 when it cannot be
+// (more streams in use than there are ticket words, or a run too long for the ticket):
+// the caller then zeroes the result and uses the accumulating launcher.
+extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, int count_false, uint64_t* out) {
+    static std::mutex mu;
+    static std::unordered_map<hipStream_t, int> slot_of;
+    static unsigned long long* tickets = nullptr;
+    if (n == 0 || n >= (1ull << kTicketShift)) return 0;
+    hipStream_t st = current_stream();
+    int slot;
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        if (!tickets) {
+            void* p = nullptr;
+            if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_count_ticket)) != hipSuccess) {
+                (void)hipGetLastError();
+                return 0;
+            }
+            tickets = (unsigned long long*)p;
+        }
+        auto it = slot_of.find(st);
+        if (it == slot_of.end()) {
+            if ((int)slot_of.size() >= kTicketSlots) return 0;
+            it = slot_of.emplace(st, (int)slot_of.size()).first;
+        }
+        slot = it->second;
+    }
+    // whole 128-bit vectors: move the word pointer back to a 16-byte boundary
+    const uintptr_t back = ((uintptr_t)a & 15) / sizeof(CUMO_BIT_DIGIT);
+    a -= back;
+    pos += back * 32;
+    const uint64_t vecs = ((pos + n + 31) / 32 + 3) / 4 - (pos / 32) / 4;
+    uint64_t grid = (vecs + kBlock - 1) / kBlock;
+    if (grid > 128) grid = 128;  // every block ends in one returning atomic on the same word
+    if (grid == 0) grid = 1;
+    if (count_false)
+        hipLaunchKernelGGL((bit_count_words_store_kernel<true>), dim3((unsigned)grid), dim3(kBlock), 0, st, (const CUMO_BIT_DIGIT*)a, (uint64_t)pos, n,
+                           tickets + slot, (unsigned long long*)out);
+    else
+        hipLaunchKernelGGL((bit_count_words_store_kernel<false>), dim3((unsigned)grid), dim3(kBlock), 0, st, (const CUMO_BIT_DIGIT*)a, (uint64_t)pos, n,
+                           tickets + slot, (unsigned long long*)out);
+    cumo_cuda_runtime_check_kernel_launch();
+    return 1;
+}
 
 extern "C" void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* d) {
     if (!d) return;

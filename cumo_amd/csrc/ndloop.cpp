@@ -1918,6 +1918,12 @@ int cumo_hip_na_bit_count(const cumo_hip_narray_t* x, unsigned int reduce, int k
     cumo_hip_loop_t lp;
     rc = cumo_hip_na_ndloop_prepare(&nf, in, out, reduce, &lp);
     if (rc) return rc;
+    // one contiguous run into one counter: a single launch that stores the count
+    if (total_of(x) != 0 && lp.ndim == 1 && lp.reduce_dim == 1 && lp.args[0].step[0] == 1 && total_of(z) == 1) {
+        CUMO_BIT_DIGIT* a = (CUMO_BIT_DIGIT*)lp.args[0].ptr + lp.args[0].bitpos / 32;
+        if (cumo_hip_bit_count_run_store_kernel_launch(a, lp.args[0].bitpos % 32, lp.n[0], count_false != 0, (uint64_t*)lp.args[1].ptr))
+            return CUMO_HIP_OK;
+    }
     // the launchers add onto the result: start from 0 (ndloop.c:853-860)
     size_t zbytes = total_of(z) * 8;
     if (zbytes) cumo_hip_memset(z->ptr + z->offset, 0, zbytes);

@@ -452,6 +452,12 @@ typedef struct {
     int      count_false;
 } cumo_hip_bit_count_nd_t;
 void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* counts);
+/* *out = the count over one contiguous run of bits, in one launch that neither needs
+ * nor reads a zeroed result (the reference zero-fills the result and its launchers add
+ * onto it, ndloop.c:853-860 + tmpl_bit/bit_count.c:9-36: two launches). a + pos/32 words,
+ * bit pos%32 onwards, n bits. Returns 1 when launched, 0 when the caller has to take
+ * the zero-fill + accumulate route. */
+int  cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, int count_false, uint64_t* out);
 
 /* Row-wise softmax and layer normalisation in one pass (no counterpart in the
  * reference, where they are chains of 5 and 6 array operations,
