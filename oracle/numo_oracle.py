@@ -327,6 +327,83 @@ def bit_count(words, pos, step, n, count_false=False):
     return int(lib.numo_bit_count(words.ctypes.data_as(C.c_void_p), pos, step, n, 1 if count_false else 0))
 
 
+def where(bits, invert=False):
+    """Bit#where (narray/gen/tmpl_bit/where.c:34-52,98-127): the row-major positions of
+    the set bits (of the clear ones with invert), ascending, as the index type the
+    reference picks (Int32 unless the array has more than 2^32 - 1 elements)."""
+    flat = np.asarray(bits).reshape(-1) != 0
+    if invert:
+        flat = ~flat
+    pos = [i for i in range(flat.size) if flat[i]] if flat.size <= 4096 else np.flatnonzero(flat)
+    return np.asarray(pos, dtype=np.int64 if flat.size > 4294967295 else np.int32)
+
+
+def mask(bits, x):
+    """Bit#mask (narray/gen/tmpl_bit/mask.c:96-167): the elements of x where the bit of
+    the same position is set, in row-major order; shapes must be equal."""
+    bits, x = np.asarray(bits), np.asarray(x)
+    if bits.shape != x.shape:
+        raise ValueError("mask and masked arrays must have the same shape")
+    return np.ascontiguousarray(x).reshape(-1)[where(bits).astype(np.int64)]
+
+
+def _positions(k, n):
+    """One index of a[...]: an integer, a slice or an index array, as positions in a
+    dimension of n elements (narray/index.c:112-233: negative values count from the end)."""
+    if isinstance(k, (int, np.integer)):
+        k = int(k) + (n if k < 0 else 0)
+        if not 0 <= k < n:
+            raise IndexError("index out of range")
+        return [k], True
+    if isinstance(k, slice):
+        return list(range(*k.indices(n))), False
+    out = []
+    for v in np.asarray(k).reshape(-1).tolist():
+        v = int(v) + (n if v < 0 else 0)
+        if not 0 <= v < n:
+            raise IndexError("index out of range")
+        out.append(v)
+    return out, False
+
+
+def take(x, key):
+    """a[key] with index arrays (narray/index.c:445-614): every dimension selects on its
+    own (an outer product of the selections, not numpy's zipped indexing); an integer
+    drops its dimension."""
+    x = np.asarray(x)
+    key = tuple(key) + (slice(None),) * (x.ndim - len(key))
+    sel = [_positions(k, n) for k, n in zip(key, x.shape)]
+    out = x[np.ix_(*[np.asarray(p, dtype=np.int64) for p, _ in sel])] if x.ndim else x
+    return out.reshape([len(p) for p, drop in sel if not drop])
+
+
+def put(x, key, value):
+    """a[key] = value with index arrays (gen/tmpl/aset.c; the store goes through
+    ndloop's scatter, narray/ndloop.c:1316): x is changed in place, value broadcasts
+    over the selection."""
+    key = tuple(key) + (slice(None),) * (x.ndim - len(key))
+    sel = [_positions(k, n) for k, n in zip(key, x.shape)]
+    shape = [len(p) for p, _ in sel]
+    kept = [len(p) for p, drop in sel if not drop]
+    v = np.broadcast_to(np.asarray(value, dtype=x.dtype), kept).reshape(shape)
+    x[np.ix_(*[np.asarray(p, dtype=np.int64) for p, _ in sel])] = v
+    return x
+
+
+def at(x, *keys):
+    """a.at(i0, i1, ...) (narray/index.c:622-682,842-870): the elements at the zipped
+    positions, as a 1-D array; every key selects the same number of positions."""
+    x = np.asarray(x)
+    if len(keys) != x.ndim:
+        raise IndexError("the number of arguments must equal the number of dimensions")
+    sel = [_positions(slice(k.start, k.stop, k.step) if isinstance(k, range) else k, n)[0] for k, n in zip(keys, x.shape)]
+    if not sel or len(sel[-1]) == 0:
+        raise ValueError("cannot get element of empty array")
+    if any(len(p) != len(sel[-1]) for p in sel):
+        raise ValueError("index array sizes mismatch")
+    return np.array([x[tuple(p[i] for p in sel)] for i in range(len(sel[-1]))], dtype=x.dtype)
+
+
 def store_bit(dst_dtype, bits):
     w = pack(bits)
     shape = bits.shape

@@ -1,5 +1,5 @@
 """Bit#where / where2 / mask: compaction of bit positions on the device against
-numpy's nonzero on the same bits (integer work: bit-exact), over contiguous
+the oracle's where / mask on the same bits (integer work: bit-exact), over contiguous
 arrays, views that start inside a word, strided and reversed views, and through
 the reference's launcher symbols with a device index array and a cursor carried
 across calls (narray/gen/tmpl_bit/where_kernel.cu:91-107, mask_kernel.cu:36-54)."""
@@ -7,6 +7,10 @@ import ctypes as C
 
 import numpy as np
 import pytest
+
+import kat_adjacent as K
+
+oracle = K.OracleEngine().o
 
 pytestmark = pytest.mark.gpu
 
@@ -20,12 +24,12 @@ def test_where_matches_nonzero(n):
     b = cumo_amd.Bit.cast(h)
     got = b.where()
     assert isinstance(got, cumo_amd.Int32)
-    assert (got.to_numpy() == np.flatnonzero(h)).all()
+    assert (got.to_numpy() == oracle.where(h)).all()
     t, f = b.where2()
-    assert (t.to_numpy() == np.flatnonzero(h)).all() and (f.to_numpy() == np.flatnonzero(h == 0)).all()
+    assert (t.to_numpy() == oracle.where(h)).all() and (f.to_numpy() == oracle.where(h, invert=True)).all()
     if n > 40:
         for sl in (slice(3, None), slice(5, n - 7), slice(None, None, 2), slice(1, None, 3), slice(None, None, -1)):
-            assert (b[sl].where().to_numpy() == np.flatnonzero(h[sl])).all(), sl
+            assert (b[sl].where().to_numpy() == oracle.where(h[sl])).all(), sl
 
 
 def test_where_on_matrices_and_empty_results():
@@ -33,11 +37,11 @@ def test_where_on_matrices_and_empty_results():
     rng = np.random.default_rng(91)
     h = (rng.random((300, 777)) < 0.3).astype(np.uint8)
     b = cumo_amd.Bit.cast(h)
-    assert (b.where().to_numpy() == np.flatnonzero(h)).all()
+    assert (b.where().to_numpy() == oracle.where(h)).all()
     # views that do not contract to one run: one launch sequence per row, the cursor carried on the device
     for key in ((slice(5, 200), slice(7, 600)), (slice(None), slice(None, None, 3)), (slice(None, None, -1), slice(None))):
-        assert (b[key].where().to_numpy() == np.flatnonzero(h[key])).all(), key
-    assert (b.transpose().where().to_numpy() == np.flatnonzero(h.T)).all()
+        assert (b[key].where().to_numpy() == oracle.where(h[key])).all(), key
+    assert (b.transpose().where().to_numpy() == oracle.where(h.T)).all()
     z = cumo_amd.Bit.cast(np.zeros(5000, dtype=np.uint8))
     assert z.where().to_numpy().shape == (0,)
     assert (z.where2()[1].to_numpy() == np.arange(5000)).all()
@@ -53,8 +57,8 @@ def test_mask_gathers_in_row_major_order(tname, dt):
         hm = (rng.random(shape) < 0.4)
         x, m = cls.cast(hx), cumo_amd.Bit.cast(hm.astype(np.uint8))
         got = m.mask(x)
-        assert isinstance(got, cls) and (got.to_numpy() == hx[hm]).all(), shape
-        assert (x[m].to_numpy() == hx[hm]).all()
+        assert isinstance(got, cls) and (got.to_numpy() == oracle.mask(hm, hx)).all(), shape
+        assert (x[m].to_numpy() == oracle.mask(hm, hx)).all()
         if len(shape) == 2:
             # the masked array as a view: transposed, strided; the mask made from a comparison
             assert (m.transpose().mask(x.transpose()).to_numpy() == hx.T[hm.T]).all()
@@ -82,7 +86,7 @@ def test_where_and_mask_launchers_with_index_arrays_and_a_carried_cursor():
     n1, p1 = 20000, 13
     idx = rng.permutation(nbits - 100)[:15000].astype(np.uint64)
     pidx = dev(idx)
-    want = np.concatenate([np.flatnonzero(h[p1:p1 + n1]), n1 + np.flatnonzero(h[7 + idx.astype(np.int64)])])
+    want = np.concatenate([oracle.where(h[p1:p1 + n1]), n1 + oracle.where(h[7 + idx.astype(np.int64)])])
     pout = dev(np.full(want.size + 4, -1, dtype=np.int64))
     _lib.call(where, pw, p1, 1, None, n1, 0, pout, 8, 0, scratch)
     _lib.call(where, pw, 7, 0, pidx, idx.size, 0, pout, 8, n1, scratch)
@@ -90,7 +94,7 @@ def test_where_and_mask_launchers_with_index_arrays_and_a_carried_cursor():
     assert (got[:want.size] == want).all() and (got[want.size:] == -1).all()
     # the zeros keep their own cursor (scratch word 1): a strided run, every third bit
     n3 = 9000
-    wantz = np.flatnonzero(h[5:5 + 3 * n3:3] == 0)
+    wantz = oracle.where(h[5:5 + 3 * n3:3] == 0)
     pz = dev(np.full(wantz.size + 2, -1, dtype=np.int32))
     _lib.call(where, pw, 5, 3, None, n3, 1, pz, 4, 0, scratch)
     gz = fetch(pz, (wantz.size + 2,), np.int32)
@@ -100,7 +104,7 @@ def test_where_and_mask_launchers_with_index_arrays_and_a_carried_cursor():
     scratch = _lib.call(new)
     mask = _lib.fn("cumo_bit_mask_kernel_launch", None,
                    [C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_void_p, C.c_uint64, C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_void_p, C.c_void_p])
-    wantm = 40 + 8 * np.flatnonzero(h[p1:p1 + n1])
+    wantm = 40 + 8 * oracle.where(h[p1:p1 + n1])
     pm = dev(np.zeros(wantm.size + 1, dtype=np.uint64))
     _lib.call(mask, pw, p1, 1, None, n1, pm, 40, 8, None, scratch)
     gm = fetch(pm, (wantm.size + 1,), np.uint64)
@@ -118,7 +122,7 @@ def test_where_and_mask_into_a_given_result():
     x = rng.standard_normal((50, 70)).astype(np.float32)
     d = cumo_amd.SFloat.cast(x)
     m = d > 0.25
-    want_pos = np.flatnonzero(x > np.float32(0.25)).astype(np.int32)
+    want_pos = oracle.where(x > np.float32(0.25)).astype(np.int32)
     pos = cumo_amd.Int32.zeros(len(want_pos))
     md, zd = m._desc(), pos._desc()
     _lib.call(_lib.lib.cumo_hip_na_where, C.byref(md), 0, C.byref(zd))

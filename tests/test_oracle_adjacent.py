@@ -81,3 +81,48 @@ def test_clip_by_brute_force_on_random_views():
         got = oracle.clip(np.ascontiguousarray(x[::2, 1::3]), np.ascontiguousarray(lo[::2, 1::3]), np.ascontiguousarray(hi[::2, 1::3]))
         assert (got == np.minimum(np.maximum(x, lo), hi)[::2, 1::3]).all()
         assert (oracle.clip(x, -3, 4) == np.clip(x, -3, 4)).all()
+
+
+def test_where_mask_and_index_arrays_against_the_reference_literals():
+    """test/bit_test.rb:20-37,50-69,161-163 and test/narray_test.rb:124-134,171,294-310,528."""
+    src = [0, 1, 1, 0, 1, 0, 0, 1]
+    for shape in ((8,), (2, 4)):
+        b = np.array(src, dtype=np.uint8).reshape(shape)
+        assert oracle.where(b).tolist() == [1, 2, 4, 7]
+        assert oracle.where(b, invert=True).tolist() == [0, 3, 5, 6]
+        assert oracle.mask(b, np.arange(1.0, 9.0).reshape(shape)).tolist() == [2, 3, 5, 8]
+    assert oracle.where(np.zeros(0, dtype=np.uint8)).tolist() == []
+    assert oracle.mask(np.zeros(0, dtype=np.uint8), np.zeros(0)).tolist() == []
+    with pytest.raises(ValueError):
+        oracle.mask(np.ones(3, dtype=np.uint8), np.ones(4))
+    a = np.array([1, 2, 3, 5, 7, 11], dtype=np.float64)
+    assert oracle.at(a, [3, 4]).tolist() == [5, 7]
+    assert oracle.at(a[2:], [1, 2]).tolist() == [5, 7]
+    assert oracle.at(a, range(3, 5)).tolist() == [5, 7]
+    assert oracle.at(a, [-1]).tolist() == [11]
+    assert oracle.take(a, ([4, 3, 0, 1, 5, 2],)).tolist() == [7, 5, 1, 2, 11, 3]
+    m = np.array([[1, 2, 3], [5, 7, 11]], dtype=np.float64)
+    assert oracle.at(m, [0, 1], [1, 2]).tolist() == [2, 11]
+    assert oracle.at(m, [0, 1], range(0, 3, 2)).tolist() == [1, 11]
+    assert oracle.at(m, range(0, 2), [0, 2]).tolist() == [1, 11]
+    assert oracle.take(m, ([0, 1], [0, 2])).tolist() == [[1, 3], [5, 11]]
+    assert oracle.take(m, (slice(None), [2, 0, 1])).tolist() == [[3, 1, 2], [11, 5, 7]]
+    assert oracle.take(m, (1, [2, 0, 0])).tolist() == [11, 5, 5]
+    c = np.array([[[1, 2], [3, 4]], [[5, 6], [7, 8]]], dtype=np.float64)
+    assert oracle.at(c, [0, 1], [1, 0], [0, 1]).tolist() == [3, 6]
+    with pytest.raises(ValueError):
+        oracle.at(m, [0, 1], [0, 1, 2])
+    with pytest.raises(IndexError):
+        oracle.take(m, ([2], 0))
+    z = m.copy()
+    oracle.put(z, ([1, 0], [0, 2]), 9)
+    assert z.tolist() == [[9, 2, 9], [9, 7, 9]]
+    oracle.put(z, ([0],), np.array([1.0, 2.0, 3.0]))
+    assert z.tolist() == [[1, 2, 3], [9, 7, 9]]
+    # where against a sequential scan on a larger array, mask against where
+    rng = np.random.default_rng(0)
+    bits = (rng.random((37, 41)) < 0.3).astype(np.uint8)
+    seq = [i for i, v in enumerate(bits.reshape(-1).tolist()) if v]
+    assert oracle.where(bits).tolist() == seq
+    vals = rng.standard_normal((37, 41))
+    assert oracle.mask(bits, vals).tolist() == [vals.reshape(-1)[i] for i in seq]
