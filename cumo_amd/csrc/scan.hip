@@ -10,9 +10,10 @@
 // Two kernels:
 //   scan_rows_kernel   one block per run, tile after tile with the running value
 //                      carried along: many runs (an axis of a matrix), or short ones.
-//   three launches     for few long runs: per-tile totals, a scan of the totals by
-//                      one block, then every tile scans itself from its offset.
-//                      Reads the input twice and writes once.
+//   three launches     for few long runs: per-tile totals, a scan of the totals (by this
+//                      same scheme while they are many, else by one block), then every
+//                      tile scans itself from its offset. Reads the input twice and
+//                      writes once.
 // Inside a tile each lane owns 8 consecutive elements: it scans them in registers,
 // the lane totals are scanned across the wave with shuffles and the four wave
 // totals through LDS. Everything is in a fixed order, so results do not change
@@ -211,43 +212,53 @@ __global__ __launch_bounds__(kScanBlock) void scan_rows_kernel(ScanRowsParams p)
     }
 }
 
-// phase 1 of the three-launch form: the total of each tile. A tile of nothing but
-// NaN under a nan operator has the total NaN, which the operator reads as "nothing".
+// phase 1 of the three-launch form: a block takes `per` consecutive tiles and leaves
+// their total. A stretch of nothing but NaN under a nan operator has the total NaN,
+// which the operator reads as "nothing".
 template <class T, class Op>
-__global__ __launch_bounds__(kScanBlock) void scan_tile_totals_kernel(const char* in, int64_t s_in, uint64_t n, T* totals) {
-    const uint64_t first = (uint64_t)blockIdx.x * kScanTile;
-    const uint64_t left = n - first;
-    const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
-    T v[kScanPer];
-    scan_load<T>(in, s_in, first, cnt, v);
+__global__ __launch_bounds__(kScanBlock) void scan_tile_totals_kernel(const char* in, int64_t s_in, uint64_t n, uint64_t per, T* totals) {
     T carry = T();
     bool hc = false;
-    scan_tile<T, Op>(v, cnt, carry, hc);
+    const uint64_t begin = (uint64_t)blockIdx.x * per * kScanTile;
+    for (uint64_t k = 0; k < per; ++k) {
+        const uint64_t first = begin + k * kScanTile;
+        if (first >= n) break;
+        const uint64_t left = n - first;
+        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
+        T v[kScanPer];
+        scan_load<T>(in, s_in, first, cnt, v);
+        scan_tile<T, Op>(v, cnt, carry, hc);
+    }
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-// phase 3: every tile scans itself, starting from the scanned total of the tiles before it
+// phase 3: every block scans its tiles, starting from the scanned total of the blocks before it
 template <class T, class Op>
-__global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const char* in, int64_t s_in, char* out, int64_t s_out, uint64_t n,
+__global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const char* in, int64_t s_in, char* out, int64_t s_out, uint64_t n, uint64_t per,
                                                                 const T* scanned_totals) {
-    const uint64_t first = (uint64_t)blockIdx.x * kScanTile;
-    const uint64_t left = n - first;
-    const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
-    T v[kScanPer];
-    scan_load<T>(in, s_in, first, cnt, v);
     bool hc = blockIdx.x > 0;
     T carry = hc ? scanned_totals[blockIdx.x - 1] : T();
-    scan_tile<T, Op>(v, cnt, carry, hc);
-    scan_store<T>(out, s_out, first, cnt, v);
+    const uint64_t begin = (uint64_t)blockIdx.x * per * kScanTile;
+    for (uint64_t k = 0; k < per; ++k) {
+        const uint64_t first = begin + k * kScanTile;
+        if (first >= n) break;
+        const uint64_t left = n - first;
+        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
+        T v[kScanPer];
+        scan_load<T>(in, s_in, first, cnt, v);
+        scan_tile<T, Op>(v, cnt, carry, hc);
+        scan_store<T>(out, s_out, first, cnt, v);
+    }
 }
 
 // ---- runs that lie across memory (the scan goes down the rows of a matrix) ------
 // Lanes sit along the dimension that is contiguous in memory and each lane walks
 // its VEC columns down the run, so every load is coalesced across the wave. A run
 // is cut into segments to fill the device: phase 0 leaves each segment's total per
-// column, phase 1 turns the totals into running totals, phase 2 scans each segment
-// from the running total before it. With enough columns there is one segment and
-// only phase 2 runs (one read, one write).
+// column and phase 2 scans each segment from what the segments before it add up to:
+// with up to 32 segments it folds their totals itself, with more the totals are first
+// turned into running totals by a column scan of their own (they form a small matrix).
+// With enough columns there is one segment and only phase 2 runs (one read, one write).
 struct ScanColsParams {
     int nouter;               // dimensions outside the run and the column dimension
     uint64_t planes, cols, n; // planes = product of those dimensions
@@ -288,8 +299,11 @@ __device__ __forceinline__ void scan_cols_store(char* p, const T (&v)[VEC]) {
 }
 
 // PHASE 0: totals[(plane * n_seg + seg) * cols + col] = total of the segment.
-// PHASE 2: scan the segment, starting from totals[.. seg - 1 ..] when seg > 0.
-template <class T, class Op, int VEC, int PHASE>
+// PHASE 2: scan the segment, starting from what the segments before it add up to:
+//   LOOKBACK false  totals holds running totals already: one load of totals[.. seg - 1 ..]
+//   LOOKBACK true   totals holds each segment's own total: they are folded here, in
+//                   segment order (few segments: cheaper than a launch that does it)
+template <class T, class Op, int VEC, int PHASE, bool LOOKBACK>
 __global__ __launch_bounds__(kScanBlock) void scan_cols_kernel(ScanColsParams p, T* totals) {
     constexpr int UNR = 8;
     const unsigned TX = 1u << p.tx_bits, TY = (unsigned)kScanBlock >> p.tx_bits;
@@ -324,7 +338,19 @@ __global__ __launch_bounds__(kScanBlock) void scan_cols_kernel(ScanColsParams p,
         T acc[VEC];
         bool has = false;
         if (PHASE == 2 && seg > 0) {
-            scan_cols_load<T, VEC>(reinterpret_cast<const char*>(totals + (plane * p.n_seg + seg - 1) * p.cols + col), acc);
+            if (LOOKBACK) {
+                const T* t = totals + plane * p.n_seg * p.cols + col;
+                scan_cols_load<T, VEC>(reinterpret_cast<const char*>(t), acc);
+#pragma unroll 4
+                for (uint64_t q = 1; q < seg; ++q) {
+                    T v[VEC];
+                    scan_cols_load<T, VEC>(reinterpret_cast<const char*>(t + q * p.cols), v);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[j] = Op::apply(acc[j], v[j]);
+                }
+            } else {
+                scan_cols_load<T, VEC>(reinterpret_cast<const char*>(totals + (plane * p.n_seg + seg - 1) * p.cols + col), acc);
+            }
             has = true;
         }
         uint64_t i = begin;
@@ -352,21 +378,12 @@ __global__ __launch_bounds__(kScanBlock) void scan_cols_kernel(ScanColsParams p,
     }
 }
 
-// phase 1: per plane and column, the running total over the segments, in place
-template <class T, class Op>
-__global__ __launch_bounds__(kScanBlock) void scan_cols_totals_kernel(T* totals, uint64_t planes, uint64_t n_seg, uint64_t cols) {
-    const uint64_t items = planes * cols;
-    for (uint64_t it = (uint64_t)blockIdx.x * kScanBlock + threadIdx.x; it < items; it += (uint64_t)gridDim.x * kScanBlock) {
-        const uint64_t plane = it / cols, col = it - plane * cols;
-        T* t = totals + plane * n_seg * cols + col;
-        T acc = t[0];
-        for (uint64_t s = 1; s < n_seg; ++s) {
-            acc = Op::apply(acc, t[s * cols]);
-            t[s * cols] = acc;
-        }
-    }
-}
+constexpr uint64_t kScanLookbackSegs = 32;
 
+// Two passes over the data with the segment totals between them. With few segments
+// the second pass folds the totals of the segments before its own by itself (two
+// launches); with many, the totals, a [segments x columns] matrix per plane, are
+// scanned in place by this same routine first (a column scan of a much smaller array).
 template <class T, class Op, int VEC>
 void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
     const uint64_t col_groups = p.cols / VEC;
@@ -374,10 +391,13 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
     while (txb < 8 && (1ull << txb) < col_groups) ++txb;
     p.tx_bits = txb;
     const uint64_t TX = 1ull << txb, TY = (uint64_t)kScanBlock >> txb;
-    // segments: enough threads for eight blocks on every compute unit, at least 16 rows each
+    // segments: enough threads for eight blocks on every compute unit, at least 16 rows each;
+    // no more than the second pass folds by itself when those already give every compute unit a block
     const uint64_t want_threads = 256ull * 8 * kScanBlock;
-    uint64_t n_seg = (want_threads + col_groups * p.planes - 1) / (col_groups * p.planes);
+    const uint64_t lanes_per_seg = col_groups * p.planes;
+    uint64_t n_seg = (want_threads + lanes_per_seg - 1) / lanes_per_seg;
     const uint64_t max_seg = (p.n + 15) / 16;
+    if (n_seg > kScanLookbackSegs && lanes_per_seg * kScanLookbackSegs >= 256ull * kScanBlock) n_seg = kScanLookbackSegs;
     if (n_seg > max_seg) n_seg = max_seg;
     if (n_seg > 1024) n_seg = 1024;
     if (n_seg < 1) n_seg = 1;
@@ -388,16 +408,30 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
     if (grid > 0x7fffffffull) grid = 0x7fffffffull;
     const dim3 g((unsigned)grid), b(kScanBlock);
     if (p.n_seg == 1) {
-        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2>), g, b, 0, stream, p, (T*)nullptr);
+        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2, false>), g, b, 0, stream, p, (T*)nullptr);
         return;
     }
     T* totals = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * p.planes * p.n_seg * p.cols));
     if (!totals) return;
-    hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 0>), g, b, 0, stream, p, totals);
-    uint64_t g1 = (p.planes * p.cols + kScanBlock - 1) / kScanBlock;
-    if (g1 > 65536) g1 = 65536;
-    hipLaunchKernelGGL((scan_cols_totals_kernel<T, Op>), dim3((unsigned)g1), b, 0, stream, totals, p.planes, p.n_seg, p.cols);
-    hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2>), g, b, 0, stream, p, totals);
+    hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 0, false>), g, b, 0, stream, p, totals);
+    if (p.n_seg <= kScanLookbackSegs) {
+        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2, true>), g, b, 0, stream, p, totals);
+    } else {
+        ScanColsParams q;
+        std::memset(&q, 0, sizeof(q));
+        q.nouter = 1;
+        q.planes = p.planes;
+        q.oshape[0] = p.planes;
+        q.ostep_in[0] = q.ostep_out[0] = (int64_t)(p.n_seg * p.cols * sizeof(T));
+        q.cols = p.cols;
+        q.n = p.n_seg;
+        q.s_in = q.s_out = (int64_t)(p.cols * sizeof(T));
+        q.in = reinterpret_cast<const char*>(totals);
+        q.out = reinterpret_cast<char*>(totals);
+        scan_cols_launch_vec<T, Op, VEC>(q, stream);  // at most 1024 rows: the next level has at most 64 segments
+        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2, false>), g, b, 0, stream, p, totals);
+    }
+    // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
     cumo_cuda_runtime_free(reinterpret_cast<char*>(totals));
 }
 
@@ -435,7 +469,7 @@ int scan_run_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n
     if (n == 0) return 0;
     hipStream_t stream = current_stream();
     const uint64_t n_tiles = (n + kScanTile - 1) / kScanTile;
-    if (n_tiles <= 8 || n_tiles > 0x7fffffffull) {
+    if (n_tiles <= 8) {
         ScanRowsParams p;
         std::memset(&p, 0, sizeof(p));
         p.rows = 1;
@@ -447,18 +481,22 @@ int scan_run_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n
         scan_rows_launch<T, Op>(p, stream);
         return (int)hipGetLastError();
     }
-    T* totals = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * n_tiles));
+    // One tile per block keeps the most loads in flight (a block that walks a stretch of
+    // tiles waits at two barriers per tile: measured 15 % slower). The totals are scanned
+    // in place by this same routine, so a long run never leaves many tiles to one block.
+    const uint64_t per = 1;
+    const uint64_t n_blocks = n_tiles;
+    if (n_blocks > 0x7fffffffull) return (int)hipErrorInvalidValue;
+    T* totals = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * n_blocks));
     if (!totals) return (int)hipErrorOutOfMemory;
-    hipLaunchKernelGGL((scan_tile_totals_kernel<T, Op>), dim3((unsigned)n_tiles), dim3(kScanBlock), 0, stream, p1, (int64_t)s1, n, totals);
-    ScanRowsParams p;
-    std::memset(&p, 0, sizeof(p));
-    p.rows = 1;
-    p.n = n_tiles;
-    p.s_in = p.s_out = (int64_t)sizeof(T);
-    p.in = reinterpret_cast<const char*>(totals);
-    p.out = reinterpret_cast<char*>(totals);
-    scan_rows_launch<T, Op>(p, stream);
-    hipLaunchKernelGGL((scan_apply_kernel<T, Op>), dim3((unsigned)n_tiles), dim3(kScanBlock), 0, stream, p1, (int64_t)s1, p2, (int64_t)s2, n,
+    hipLaunchKernelGGL((scan_tile_totals_kernel<T, Op>), dim3((unsigned)n_blocks), dim3(kScanBlock), 0, stream, p1, (int64_t)s1, n, per, totals);
+    const int inner = scan_run_launch<T, Op>(reinterpret_cast<const char*>(totals), reinterpret_cast<char*>(totals), (ssize_t)sizeof(T),
+                                             (ssize_t)sizeof(T), n_blocks);
+    if (inner) {
+        cumo_cuda_runtime_free(reinterpret_cast<char*>(totals));
+        return inner;
+    }
+    hipLaunchKernelGGL((scan_apply_kernel<T, Op>), dim3((unsigned)n_blocks), dim3(kScanBlock), 0, stream, p1, (int64_t)s1, p2, (int64_t)s2, n, per,
                        (const T*)totals);
     const int st = (int)hipGetLastError();
     // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream

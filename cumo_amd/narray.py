@@ -956,6 +956,18 @@ class Bit(NArray):
         r = self.count_true()
         return int(r) if not isinstance(r, int) else r
 
+    # all? / any? / none? over the whole array (reference: gen/tmpl_bit/all_p.c, any_p.c,
+    # none_p.c; their per-axis forms, which answer Bit arrays, are outside this path).
+    # One count on the device, one value read back.
+    def all_p(self):
+        return self.size == 0 or int(self.count_false()) == 0
+
+    def any_p(self):
+        return self.size != 0 and int(self.count_true()) != 0
+
+    def none_p(self):
+        return not self.any_p()
+
     def _store_into(self, cls):
         """Bit -> 0/1 numbers (reference: gen/tmpl/store_bit.c)."""
         return self._cast_to(cls)

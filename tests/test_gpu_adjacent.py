@@ -217,6 +217,35 @@ def test_cum_nan_forms_on_random_placements(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", ALL)
+def test_cum_along_columns_of_tall_wide_and_stacked_arrays(tname, dt):
+    """Runs that lie across memory: few segments (the second pass folds their totals
+    itself), many (the totals are scanned first, by the same routine), several planes.
+    Small integers, so float sums are exact in any order and every result is compared
+    bit for bit; products use factors of 1 and -1 and a few 2s."""
+    cls = cls_of(tname)
+    rng = np.random.default_rng(55)
+    for shape, ax in [((70000, 12), 0), ((5000, 2048), 0), ((4, 3000, 64), 1), ((100000, 4), 0), ((3, 40000, 8), 1), ((33000, 1028), 0)]:
+        h = rng.integers(-3, 4, size=shape).astype(dt)
+        d = cls.cast(h)
+        assert_bits_equal(d.cumsum(axis=ax).to_numpy(), oracle.cum("cumsum", h, axis=ax), (shape, "cumsum"))
+        f = rng.choice(np.array([1, -1], dtype=dt), size=shape)
+        f[tuple(rng.integers(0, n, 20) for n in shape)] = 2
+        assert_bits_equal(cls.cast(f).cumprod(axis=ax).to_numpy(), oracle.cum("cumprod", f, axis=ax), (shape, "cumprod"))
+        if dt != np.int32:
+            h[tuple(rng.integers(0, n, 500) for n in shape)] = np.nan
+            if len(shape) == 2:
+                h[:50] = np.nan                                    # every run starts with NaN
+            d = cls.cast(h)
+            assert_bits_equal(d.cumsum(axis=ax, nan=True).to_numpy(), oracle.cum("cumsum", h, axis=ax, nan=True), (shape, "nan: true"))
+            assert_bits_equal(d.cumsum(axis=ax).to_numpy(), oracle.cum("cumsum", h, axis=ax), (shape, "NaN carried"))
+        # a view: every other column, rows reversed
+        if len(shape) == 2 and shape[1] >= 8:
+            hb = h if dt == np.int32 else np.nan_to_num(h)
+            hv = np.ascontiguousarray(hb[::-1, ::2])
+            assert_bits_equal(cls.cast(hb).reverse(0)[:, ::2].cumsum(axis=0).to_numpy(), oracle.cum("cumsum", hv, axis=0), (shape, "view"))
+
+
+@pytest.mark.parametrize("tname,dt", ALL)
 def test_mulsum_parity(tname, dt):
     cls = cls_of(tname)
     rng = np.random.default_rng(53)

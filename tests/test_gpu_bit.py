@@ -29,6 +29,17 @@ def test_bit_test_rb_literals():
     assert m.count_true(axis=0).to_numpy().tolist() == [1, 1, 1, 1]
     assert m.count_true(axis=1).to_numpy().tolist() == [2, 2]
     assert m.count_false(axis=1).to_numpy().tolist() == [2, 2]
+    # test/bit_test.rb:35-40,67-72,161-166: where, where2, mask, all?, any?, none?
+    for v in (a, m):
+        assert v.where().to_a() == [1, 2, 4, 7]
+        assert [w.to_a() for w in v.where2()] == [[1, 2, 4, 7], [0, 3, 5, 6]]
+        assert not v.all_p() and v.any_p() and not v.none_p()
+    assert a.mask(cumo_amd.DFloat.cast([1, 2, 3, 4, 5, 6, 7, 8])).to_a() == [2, 3, 5, 8]
+    assert m.mask(cumo_amd.DFloat.cast([[1, 2, 3, 4], [5, 6, 7, 8]])).to_a() == [2, 3, 5, 8]
+    ones, zeros = cumo_amd.Bit.cast([1] * 70), cumo_amd.Bit.cast([0] * 70)
+    assert ones.all_p() and ones.any_p() and not ones.none_p()
+    assert not zeros.all_p() and not zeros.any_p() and zeros.none_p()
+    assert ones[3:67].all_p() and zeros[::3].none_p()
 
 
 @pytest.mark.parametrize("n", [1, 5, 31, 32, 33, 63, 64, 65, 200, 1000, 100003, 1 << 20])
