@@ -312,6 +312,19 @@ def measure_graph(cumo, lib, iters=200):
     return {"workload": "C1 chain (2.5*x, +b, sum)", "sizes": rows}
 
 
+def measure_host_cost():
+    """Per-operation cost of the C host layer on tiny arrays, from the C driver built next to
+    the library (bench_host_cost.cpp): no interpreter between the calls."""
+    import subprocess
+    tool = os.path.join(ROOT, "cumo_amd", "bench_host_cost")
+    if not os.path.exists(tool):
+        return {"skipped": "cumo_amd/bench_host_cost is not built (python cumo_amd/build.py)"}
+    p = subprocess.run([tool], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    if p.returncode:
+        return {"failed": p.stderr.strip()[-300:]}
+    return json.loads(p.stdout.strip().splitlines()[-1])
+
+
 def cpu_baseline_c2(budget_s=12.0):
     """Numo-shaped single-thread C loops (the oracle's row loops) on the same C2
     workload, on this machine's host cores. A bounded number of passes."""
@@ -478,6 +491,7 @@ def main():
         if not args.no_extras:
             out["host_io"] = measure_host_io(lib)
             out["graph"] = measure_graph(cumo_amd, lib)
+            out["host_cost"] = measure_host_cost()
     print(json.dumps(out))
 
 

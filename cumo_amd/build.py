@@ -18,6 +18,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libcumo_hip.so")
+HOST_COST_TOOL = os.path.join(HERE, "bench_host_cost")
 
 ARCH = "gfx950"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -85,7 +86,21 @@ def build(jobs=None, force=False, verbose=True):
     if p.returncode:
         print(p.stdout)
         raise RuntimeError("link failed")
+    build_host_cost_tool()
     return LIB
+
+
+def build_host_cost_tool():
+    """bench_host_cost.cpp (repository root) -> cumo_amd/bench_host_cost, linked against the library."""
+    src = os.path.join(ROOT, "bench_host_cost.cpp")
+    if not os.path.exists(src):
+        return
+    cmd = ["g++", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"), src, "-o", HOST_COST_TOOL,
+           "-L" + HERE, "-lcumo_hip", "-Wl,-rpath,$ORIGIN"]
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode:
+        print(p.stdout)
+        raise RuntimeError("bench_host_cost: g++ failed")
 
 
 if __name__ == "__main__":
