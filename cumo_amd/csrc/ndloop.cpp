@@ -1538,6 +1538,35 @@ int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, 
     for (int d = 0; same && d < x->ndim; ++d) same = mask->shape[d] == x->shape[d];
     if (!same) return fail(CUMO_HIP_ERROR_SHAPE, "mask and masked arrays must have the same shape");
     if (!z) return fail(CUMO_HIP_ERROR_ARGUMENT, "mask: no result descriptor");
+    // mask and masked array walk as one run each (both contiguous, or sliced alike): the
+    // elements are compacted directly, without the array of positions in between
+    if (total_of(x) != 0) {
+        cumo_hip_ndfunc_t nf = {NULL, 0, 2, 0, {0, 0}};
+        const NA* in[2] = {mask, x};
+        LP lp;
+        if (cumo_hip_na_ndloop_prepare(&nf, in, NULL, 0, &lp) == CUMO_HIP_OK && lp.ndim == 1) {
+            NA cnt;
+            cnt.ptr = NULL;
+            rc = cumo_hip_na_bit_count(mask, 0, 0, 0, &cnt);
+            if (rc) return rc;
+            uint64_t n_hit = 0;
+            rc = cumo_hip_copy_to_host(&n_hit, cnt.ptr + cnt.offset, sizeof(n_hit));
+            free_tmp(&cnt);
+            if (rc) return rc;
+            bool allocated;
+            rc = result_1d(z, x->type, (size_t)n_hit, &allocated);
+            if (rc || n_hit == 0) return rc;
+            char* scratch = cumo_bit_where_scratch_new();
+            if (!scratch) {
+                if (allocated) free_tmp(z);
+                return CUMO_HIP_ERROR_OUT_OF_MEMORY;
+            }
+            cumo_hip_bit_compact_kernel_launch((CUMO_BIT_DIGIT*)lp.args[0].ptr, lp.args[0].bitpos, lp.args[0].step[0], lp.n[0], lp.args[1].ptr,
+                                               lp.args[1].step[0], (size_t)kElmsz[x->type], z->ptr + z->offset, scratch);
+            cumo_cuda_runtime_free(scratch);
+            return CUMO_HIP_OK;
+        }
+    }
     NA pos;
     pos.ptr = NULL;
     rc = cumo_hip_na_where(mask, 0, &pos);

@@ -105,9 +105,11 @@ __global__ __launch_bounds__(kWhBlock) void where_scan_kernel(uint64_t* block_su
     if (threadIdx.x == 0) *running = acc;
 }
 
-// MASK false: out[o] = count + position in the run, as elmsz-byte integers (where).
-// MASK true:  out[o] = the masked array's element position p2 + j*s2 (or p2 + idx2[j]), as size_t (mask).
-template <bool MASK>
+// MODE 0: out[o] = count + position in the run, as elmsz-byte integers (where).
+// MODE 1: out[o] = the masked array's element position p2 + j*s2 (or p2 + idx2[j]), as size_t (mask).
+// MODE 2: out[o] = the masked array's element itself, elmsz (4 or 8) bytes read at p2 + j*s2 where p2 is
+//         its address (the compaction the reference reaches through a view over the positions of mode 1).
+template <int MODE>
 __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
                                                                  int contiguous, int invert, uint64_t nchunks, uint64_t cpb, char* out, size_t elmsz,
                                                                  uint64_t count, size_t p2, int64_t s2, const size_t* idx2,
@@ -133,7 +135,11 @@ __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_
         for (uint32_t k = threadIdx.x; k < (uint32_t)total; k += kWhBlock) {
             const uint64_t j = c0 * 32 + hit[k];
             const uint64_t w = off + k;
-            if (MASK) {
+            if (MODE == 2) {
+                const char* src = reinterpret_cast<const char*>(p2) + (int64_t)j * s2;
+                if (elmsz == 4) reinterpret_cast<uint32_t*>(out)[w] = *reinterpret_cast<const uint32_t*>(src);
+                else reinterpret_cast<uint64_t*>(out)[w] = *reinterpret_cast<const uint64_t*>(src);
+            } else if (MODE == 1) {
                 reinterpret_cast<size_t*>(out)[w] = idx2 ? (p2 + idx2[j]) : (size_t)((int64_t)p2 + (int64_t)j * s2);
             } else if (elmsz == 4) {
                 reinterpret_cast<int32_t*>(out)[w] = (int32_t)(count + j);
@@ -145,7 +151,7 @@ __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_
     }
 }
 
-template <bool MASK>
+template <int MODE>
 void where_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, int invert, char* out, size_t elmsz, uint64_t count, size_t p2,
                   ssize_t s2, size_t* idx2, uint64_t* running, uint64_t* block_sums) {
     if (n == 0) return;  // a grid of no blocks is an invalid launch
@@ -158,7 +164,7 @@ void where_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t 
     hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n, contiguous,
                        invert, nchunks, cpb, block_sums);
     hipLaunchKernelGGL(where_scan_kernel, dim3(1), dim3(kWhBlock), 0, st, block_sums, nblocks, running);
-    hipLaunchKernelGGL((where_scatter_kernel<MASK>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n,
+    hipLaunchKernelGGL((where_scatter_kernel<MODE>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n,
                        contiguous, invert, nchunks, cpb, out, elmsz, count, p2, (int64_t)s2, (const size_t*)idx2, (const uint64_t*)block_sums);
     cumo_cuda_runtime_check_kernel_launch();
 }
@@ -230,14 +236,23 @@ char* cumo_bit_where_scratch_new(void) {
 void cumo_bit_where_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, int invert, char* out, size_t elmsz, uint64_t count,
                                   char* scratch) {
     uint64_t* running = reinterpret_cast<uint64_t*>(scratch) + (invert ? 1 : 0);
-    where_launch<false>(a, p, s, idx, n, invert, out, elmsz, count, 0, 0, nullptr, running, reinterpret_cast<uint64_t*>(scratch) + 2);
+    where_launch<0>(a, p, s, idx, n, invert, out, elmsz, count, 0, 0, nullptr, running, reinterpret_cast<uint64_t*>(scratch) + 2);
 }
 
 // reference: mask_kernel.cu:36-54
 void cumo_bit_mask_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, size_t* out, size_t p2, ssize_t s2, size_t* idx2,
                                  char* scratch) {
-    where_launch<true>(a, p, s, idx, n, 0, reinterpret_cast<char*>(out), sizeof(size_t), 0, p2, s2, idx2, reinterpret_cast<uint64_t*>(scratch),
+    where_launch<1>(a, p, s, idx, n, 0, reinterpret_cast<char*>(out), sizeof(size_t), 0, p2, s2, idx2, reinterpret_cast<uint64_t*>(scratch),
                        reinterpret_cast<uint64_t*>(scratch) + 2);
+}
+
+// out[o] = the o-th element of the run x + j*sx (j = 0 .. n-1) whose bit in the run (a, p, s) is set:
+// the compaction of values in the same three launches as where. elmsz 4 or 8. The scratch is the one of
+// cumo_bit_where_scratch_new; its first cursor carries the output position from one run to the next.
+void cumo_hip_bit_compact_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, uint64_t n, const char* x, ssize_t sx, size_t elmsz, char* out,
+                                        char* scratch) {
+    where_launch<2>(a, p, s, nullptr, n, 0, out, elmsz, 0, (size_t)(uintptr_t)x, sx, nullptr, reinterpret_cast<uint64_t*>(scratch),
+                    reinterpret_cast<uint64_t*>(scratch) + 2);
 }
 
 void cumo_hip_gather_flat_kernel_launch(const cumo_hip_gather_flat_t* d) {

@@ -491,6 +491,14 @@ typedef struct {
 } cumo_hip_mulsum_rows_t;
 int cumo_hip_mulsum_rows_kernel_launch(int type, int nan, const cumo_hip_mulsum_rows_t* rows);
 
+/* out[o] = the o-th element of the run x + j*sx, j = 0 .. n-1, whose bit in the run of
+ * bits (a, p, s) is set: a[mask] for one run in the three launches of where, without
+ * the array of positions the reference goes through (tmpl_bit/mask.c:141-167 makes a
+ * view over them). elmsz 4 or 8; scratch from cumo_bit_where_scratch_new, whose first
+ * cursor carries the output position from one run to the next. */
+void cumo_hip_bit_compact_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, const char *x, ssize_t sx, size_t elmsz,
+                                        char *out, char *scratch);
+
 /* out[i] = the element of a strided view at flat row-major position pos[i] (no
  * counterpart symbol in the reference, where a masked array is a view over an index
  * array, tmpl_bit/mask.c:141-167, read by the index kernels). Elements of 4 or 8

@@ -135,3 +135,28 @@ def test_where_and_mask_into_a_given_result():
     sd = short._desc()
     with pytest.raises(cumo_amd.ShapeError):
         _lib.call(_lib.lib.cumo_hip_na_where, C.byref(md), 0, C.byref(sd))
+
+
+@pytest.mark.parametrize("tname,dt", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
+def test_mask_of_single_runs_with_offsets_steps_and_reversal(tname, dt):
+    """Mask and masked array that each walk as one run (sliced alike) are compacted in place of
+    positions: starts inside a word, steps other than 1, a reversed run, different steps on the two sides."""
+    import cumo_amd
+    cls = getattr(cumo_amd, tname)
+    rng = np.random.default_rng(93)
+    n = 100003
+    hx = rng.integers(-1000, 1000, size=n).astype(dt)
+    hm = rng.random(n) < 0.35
+    x, m = cls.cast(hx), cumo_amd.Bit.cast(hm.astype(np.uint8))
+    for sl in (slice(7, None), slice(33, n - 9), slice(None, None, 2), slice(5, None, 3), slice(None, None, -1), slice(n - 4, 2, -5)):
+        got = m[sl].mask(x[sl]).to_numpy()
+        assert (got == oracle.mask(hm[sl], hx[sl])).all(), sl
+    # the mask contiguous, the masked array every other element of a longer one
+    hy = rng.integers(-1000, 1000, size=2 * n).astype(dt)
+    y = cls.cast(hy)
+    assert (m.mask(y[::2]).to_numpy() == oracle.mask(hm, hy[::2])).all()
+    assert (m[::-1].mask(y[1::2]).to_numpy() == oracle.mask(hm[::-1], hy[1::2])).all()
+    # nothing set, everything set
+    none, every = cumo_amd.Bit.cast(np.zeros(n, dtype=np.uint8)), cumo_amd.Bit.cast(np.ones(n, dtype=np.uint8))
+    assert none.mask(x).to_numpy().shape == (0,)
+    assert (every.mask(x).to_numpy() == hx).all()
