@@ -212,24 +212,51 @@ __global__ __launch_bounds__(kScanBlock) void scan_rows_kernel(ScanRowsParams p)
     }
 }
 
-// phase 1 of the three-launch form: a block takes `per` consecutive tiles and leaves
-// their total. A stretch of nothing but NaN under a nan operator has the total NaN,
-// which the operator reads as "nothing".
-template <class T, class Op>
-__global__ __launch_bounds__(kScanBlock) void scan_tile_totals_kernel(const char* in, int64_t s_in, uint64_t n, uint64_t per, T* totals) {
-    T carry = T();
-    bool hc = false;
-    const uint64_t begin = (uint64_t)blockIdx.x * per * kScanTile;
-    for (uint64_t k = 0; k < per; ++k) {
-        const uint64_t first = begin + k * kScanTile;
-        if (first >= n) break;
-        const uint64_t left = n - first;
-        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
-        T v[kScanPer];
-        scan_load<T>(in, s_in, first, cnt, v);
-        scan_tile<T, Op>(v, cnt, carry, hc);
+template <class T>
+__device__ __forceinline__ T scan_shfl_xor(T v, unsigned m) {
+    if constexpr (sizeof(T) == 8) {
+        union { T t; uint32_t w[2]; } a, b;
+        a.t = v;
+        b.w[0] = __shfl_xor(a.w[0], m);
+        b.w[1] = __shfl_xor(a.w[1], m);
+        return b.t;
+    } else {
+        union { T t; uint32_t w; } a, b;
+        a.t = v;
+        b.w = __shfl_xor(a.w, m);
+        return b.t;
     }
-    if (threadIdx.x == 0) totals[blockIdx.x] = carry;
+}
+
+// phase 1 of the three-launch form: the total of each tile, by a plain fold (the
+// operators are associative and commutative: lane-local fold, wave butterfly, four LDS
+// slots), which is lighter than the scan of the tile. A tile of nothing but NaN under a
+// nan operator has the total NaN, which the operator reads as "nothing". The last tile
+// may be partial; nothing comes after it, so its total is never used and none is formed.
+template <class T, class Op>
+__global__ __launch_bounds__(kScanBlock) void scan_tile_totals_kernel(const char* in, int64_t s_in, uint64_t n, T* totals) {
+    __shared__ T wave_tot[kScanBlock / 64];
+    const uint64_t first = (uint64_t)blockIdx.x * kScanTile;
+    const uint64_t left = n - first;
+    if (left < (uint64_t)kScanTile) {
+        if (threadIdx.x == 0) totals[blockIdx.x] = T();
+        return;
+    }
+    T v[kScanPer];
+    scan_load<T>(in, s_in, first, kScanTile, v);
+    T t = v[0];
+#pragma unroll
+    for (int k = 1; k < kScanPer; ++k) t = Op::apply(t, v[k]);
+#pragma unroll
+    for (unsigned m = 32; m > 0; m >>= 1) t = Op::apply(t, scan_shfl_xor(t, m));
+    if ((threadIdx.x & 63) == 0) wave_tot[threadIdx.x >> 6] = t;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T tot = wave_tot[0];
+#pragma unroll
+        for (int w = 1; w < kScanBlock / 64; ++w) tot = Op::apply(tot, wave_tot[w]);
+        totals[blockIdx.x] = tot;
+    }
 }
 
 // phase 3: every block scans its tiles, starting from the scanned total of the blocks before it
@@ -489,7 +516,7 @@ int scan_run_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n
     if (n_blocks > 0x7fffffffull) return (int)hipErrorInvalidValue;
     T* totals = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * n_blocks));
     if (!totals) return (int)hipErrorOutOfMemory;
-    hipLaunchKernelGGL((scan_tile_totals_kernel<T, Op>), dim3((unsigned)n_blocks), dim3(kScanBlock), 0, stream, p1, (int64_t)s1, n, per, totals);
+    hipLaunchKernelGGL((scan_tile_totals_kernel<T, Op>), dim3((unsigned)n_blocks), dim3(kScanBlock), 0, stream, p1, (int64_t)s1, n, totals);
     const int inner = scan_run_launch<T, Op>(reinterpret_cast<const char*>(totals), reinterpret_cast<char*>(totals), (ssize_t)sizeof(T),
                                              (ssize_t)sizeof(T), n_blocks);
     if (inner) {
