@@ -79,9 +79,6 @@ CUMO_HIP_FUN(OpRint, rint((double)x))
         __device__ __forceinline__ bool operator()(T x, T, T& z) const { z = (T)(EXPR); return true; } };
 CUMO_HIP_FUN(OpSqrt, sqrt((double)x))
 CUMO_HIP_FUN_H(OpCbrt, cbrt((double)x))
-CUMO_HIP_FUN_H(OpLog, log((double)x))
-CUMO_HIP_FUN_H(OpLog2, log2((double)x))
-CUMO_HIP_FUN_H(OpLog10, log10((double)x))
 // SFloat exp: the double-precision exp of the argument, rounded to float once.
 // The argument has 24 significant bits, so k = rint(x / ln 2) times the upper part
 // of ln 2 is exact; exp(r) on |r| <= ln(2)/2 is the Taylor polynomial of degree 13
@@ -117,6 +114,98 @@ __device__ __forceinline__ float exp_float_rounded_once(float xf) {
     const float y = (float)__hiloint2double(hi, __double2loint(p));
     return y + (xc - xc);
 }
+// SFloat log, log2, log10: the double-precision logarithm of the argument, rounded to
+// float once, by the classic reduction x = 2^k (1 + f), sqrt(2)/2 < 1 + f < sqrt(2),
+// s = f / (2 + f), log(1 + f) = f - f^2/2 + s (f^2/2 + R(s^2)) with a degree-7 polynomial R
+// (the public fdlibm scheme and coefficients), every step an IEEE double operation, no
+// branch on the data. BASE 0: k ln2 + log(1 + f) with ln2 in two parts; BASE 2:
+// k + log(1 + f) / ln2 in one fused multiply-add; BASE 10: k log10(2) in two parts plus
+// log(1 + f) / ln10. Run on the CPU against glibc's log, log2 and log10 over every
+// non-negative float bit pattern, the float results differ nowhere. A subnormal float is
+// a normal double, so only 0, negative arguments, infinity and NaN are special.
+template <int BASE>
+__device__ __forceinline__ float log_float_rounded_once(float xf) {
+    const double x = (double)xf;
+    uint32_t hx = (uint32_t)__double2hiint(x);
+    int k = (int)(hx >> 20) - 1023;
+    hx &= 0x000fffffu;
+    const uint32_t i = (hx + 0x95f64u) & 0x100000u;  // mantissa >= sqrt(2): halve it
+    k += (int)(i >> 20);
+    const double m = __hiloint2double((int)(hx | (i ^ 0x3ff00000u)), __double2loint(x));
+    const double f = m - 1.0;
+    const double s = f / (2.0 + f);
+    const double dk = (double)k;
+    const double z = s * s, w = z * z;
+    const double t1 = w * __builtin_fma(w, __builtin_fma(w, 1.531383769920937332e-01, 2.222219843214978396e-01), 3.999999999940941908e-01);
+    const double t2 = z * __builtin_fma(w, __builtin_fma(w, __builtin_fma(w, 1.479819860511658591e-01, 1.818357216161805012e-01),
+                                                         2.857142874366239149e-01), 6.666666666666735130e-01);
+    const double R = t2 + t1;
+    const double hfsq = 0.5 * f * f;
+    double r;
+    if (BASE == 2) {
+        const double lm = f - (hfsq - s * (hfsq + R));
+        r = __builtin_fma(lm, 1.44269504088896338700e+00, dk);
+    } else if (BASE == 10) {
+        const double lm = f - (hfsq - s * (hfsq + R));
+        r = __builtin_fma(dk, 3.69423907715893078616e-13, 4.34294481903251816668e-01 * lm) + dk * 3.01029995663611771306e-01;
+    } else {
+        r = dk * 6.93147180369123816490e-01 - ((hfsq - (s * (hfsq + R) + dk * 1.90821492927058770002e-10)) - f);
+    }
+    // NaN comes back in through xf - xf (which is NaN for an infinity too); then, on the
+    // float and after all the arithmetic: 0 -> -inf, negative -> NaN, +inf -> +inf
+    float y = (float)r + (xf - xf);
+    y = (xf == 0.0f) ? -INFINITY : y;
+    y = (xf < 0.0f) ? NAN : y;
+    y = (xf == INFINITY) ? INFINITY : y;
+    return y;
+}
+#define CUMO_HIP_LOG_OP(NAME, BASE, DEXPR)                                                                                  \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const {                                                    \
+            if constexpr (sizeof(T) == 4) z = (T)log_float_rounded_once<BASE>((float)x);                                    \
+            else z = (T)(DEXPR);                                                                                            \
+            return true; } };
+CUMO_HIP_LOG_OP(OpLog, 0, log((double)x))
+CUMO_HIP_LOG_OP(OpLog2, 2, log2((double)x))
+CUMO_HIP_LOG_OP(OpLog10, 10, log10((double)x))
+
+// SFloat tanh: the double-precision tanh rounded to float once. With e = exp(2|x|) =
+// 2^k (1 + q r) from the same reduction and polynomial as exp above (q = (exp(r) - 1) / r),
+// e - 1 = (2^k - 1) + (2^k q) r comes out of one fused multiply-add without cancellation,
+// and tanh|x| = (e - 1) / ((e - 1) + 2). |x| is clamped at 20, where the answer is 1 in
+// double already. Run on the CPU against glibc's tanh over every float bit pattern, the
+// float results differ nowhere.
+__device__ __forceinline__ float tanh_float_rounded_once(float xf) {
+    float ax = __builtin_fabsf(xf);
+    ax = (ax > 20.0f) ? 20.0f : ax;  // false for NaN, which then travels through the arithmetic
+    const double x2 = 2.0 * (double)ax;
+    const double big = 6755399441055744.0;  // 1.5 * 2^52
+    const double t0 = __builtin_fma(x2, 1.44269504088896338700e+00, big);
+    const double k = t0 - big;
+    const uint32_t ki = (uint32_t)__double2loint(t0);  // 0 .. 58 (anything for a NaN, which r carries on)
+    double r = __builtin_fma(k, -6.93147180369123816490e-01, x2);
+    r = __builtin_fma(k, -1.90821492927058770002e-10, r);
+    const double c[12] = {
+        1.60590438368216133e-10, 2.08767569878681002e-09, 2.50521083854417202e-08, 2.75573192239858883e-07, 2.75573192239858925e-06,
+        2.48015873015873016e-05, 1.98412698412698413e-04, 1.38888888888888894e-03, 8.33333333333333322e-03, 4.16666666666666644e-02,
+        1.66666666666666657e-01, 5.00000000000000000e-01};
+    double q = c[0];
+#pragma unroll
+    for (int i = 1; i < 12; ++i) q = __builtin_fma(q, r, c[i]);
+    q = __builtin_fma(q, r, 1.0);
+    const double qs = __hiloint2double((int)((uint32_t)__double2hiint(q) + (ki << 20)), __double2loint(q));
+    const double p2k = __hiloint2double((int)((1023u + ki) << 20), 0);
+    const double t = __builtin_fma(qs, r, p2k - 1.0);
+    const double y = t / (t + 2.0);
+    const float yf = (float)y;  // |tanh|; a NaN argument has made it NaN
+    return __builtin_copysignf(yf, xf);
+}
+template <class T> struct OpTanh { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
+    __device__ __forceinline__ bool operator()(T x, T, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)tanh_float_rounded_once((float)x);
+        else z = (T)tanh((double)x);
+        return true; } };
+
 template <class T> struct OpExp { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
     __device__ __forceinline__ bool operator()(T x, T, T& z) const {
         if constexpr (sizeof(T) == 4) z = (T)exp_float_rounded_once((float)x);
@@ -132,7 +221,6 @@ CUMO_HIP_FUN_H(OpAcos, acos((double)x))
 CUMO_HIP_FUN_H(OpAtan, atan((double)x))
 CUMO_HIP_FUN_H(OpSinh, sinh((double)x))
 CUMO_HIP_FUN_H(OpCosh, cosh((double)x))
-CUMO_HIP_FUN_H(OpTanh, tanh((double)x))
 CUMO_HIP_FUN_H(OpAsinh, asinh((double)x))
 CUMO_HIP_FUN_H(OpAcosh, acosh((double)x))
 CUMO_HIP_FUN_H(OpAtanh, atanh((double)x))
