@@ -124,8 +124,7 @@ __device__ __forceinline__ float exp_float_rounded_once(float xf) {
 // non-negative float bit pattern, the float results differ nowhere. A subnormal float is
 // a normal double, so only 0, negative arguments, infinity and NaN are special.
 template <int BASE>
-__device__ __forceinline__ float log_float_rounded_once(float xf) {
-    const double x = (double)xf;
+__device__ __forceinline__ double log_core(double x) {  // x positive, finite, normal
     uint32_t hx = (uint32_t)__double2hiint(x);
     int k = (int)(hx >> 20) - 1023;
     hx &= 0x000fffffu;
@@ -141,21 +140,34 @@ __device__ __forceinline__ float log_float_rounded_once(float xf) {
                                                          2.857142874366239149e-01), 6.666666666666735130e-01);
     const double R = t2 + t1;
     const double hfsq = 0.5 * f * f;
-    double r;
     if (BASE == 2) {
         const double lm = f - (hfsq - s * (hfsq + R));
-        r = __builtin_fma(lm, 1.44269504088896338700e+00, dk);
-    } else if (BASE == 10) {
-        const double lm = f - (hfsq - s * (hfsq + R));
-        r = __builtin_fma(dk, 3.69423907715893078616e-13, 4.34294481903251816668e-01 * lm) + dk * 3.01029995663611771306e-01;
-    } else {
-        r = dk * 6.93147180369123816490e-01 - ((hfsq - (s * (hfsq + R) + dk * 1.90821492927058770002e-10)) - f);
+        return __builtin_fma(lm, 1.44269504088896338700e+00, dk);
     }
+    if (BASE == 10) {
+        const double lm = f - (hfsq - s * (hfsq + R));
+        return __builtin_fma(dk, 3.69423907715893078616e-13, 4.34294481903251816668e-01 * lm) + dk * 3.01029995663611771306e-01;
+    }
+    return dk * 6.93147180369123816490e-01 - ((hfsq - (s * (hfsq + R) + dk * 1.90821492927058770002e-10)) - f);
+}
+template <int BASE>
+__device__ __forceinline__ float log_float_rounded_once(float xf) {
     // NaN comes back in through xf - xf (which is NaN for an infinity too); then, on the
     // float and after all the arithmetic: 0 -> -inf, negative -> NaN, +inf -> +inf
-    float y = (float)r + (xf - xf);
+    float y = (float)log_core<BASE>((double)xf) + (xf - xf);
     y = (xf == 0.0f) ? -INFINITY : y;
     y = (xf < 0.0f) ? NAN : y;
+    y = (xf == INFINITY) ? INFINITY : y;
+    return y;
+}
+// SFloat log1p: 1 + x is exact in double for |x| >= 2^-29 (a float has 24 bits), so the
+// logarithm above applies to it unchanged; below that the answer rounds to x itself.
+// Checked like the others, over every float bit pattern.
+__device__ __forceinline__ float log1p_float_rounded_once(float xf) {
+    float y = (float)log_core<0>(1.0 + (double)xf) + (xf - xf);
+    y = (__builtin_fabsf(xf) < 1.862645149230957e-09f) ? xf : y;
+    y = (xf == -1.0f) ? -INFINITY : y;
+    y = (xf < -1.0f) ? NAN : y;
     y = (xf == INFINITY) ? INFINITY : y;
     return y;
 }
@@ -168,22 +180,21 @@ __device__ __forceinline__ float log_float_rounded_once(float xf) {
 CUMO_HIP_LOG_OP(OpLog, 0, log((double)x))
 CUMO_HIP_LOG_OP(OpLog2, 2, log2((double)x))
 CUMO_HIP_LOG_OP(OpLog10, 10, log10((double)x))
+template <class T> struct OpLog1p { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
+    __device__ __forceinline__ bool operator()(T x, T, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)log1p_float_rounded_once((float)x);
+        else z = (T)log1p((double)x);
+        return true; } };
 
-// SFloat tanh: the double-precision tanh rounded to float once. With e = exp(2|x|) =
-// 2^k (1 + q r) from the same reduction and polynomial as exp above (q = (exp(r) - 1) / r),
-// e - 1 = (2^k - 1) + (2^k q) r comes out of one fused multiply-add without cancellation,
-// and tanh|x| = (e - 1) / ((e - 1) + 2). |x| is clamped at 20, where the answer is 1 in
-// double already. Run on the CPU against glibc's tanh over every float bit pattern, the
-// float results differ nowhere.
-__device__ __forceinline__ float tanh_float_rounded_once(float xf) {
-    float ax = __builtin_fabsf(xf);
-    ax = (ax > 20.0f) ? 20.0f : ax;  // false for NaN, which then travels through the arithmetic
-    const double x2 = 2.0 * (double)ax;
+// exp(x) - 1 in double for x inside [-745, 709], from the reduction and polynomial of exp
+// above: with q = (exp(r) - 1) / r, exp(x) - 1 = 2^k (1 + q r) - 1 = (2^k - 1) + (2^k q) r
+// comes out of one fused multiply-add, without the cancellation of exp(x) - 1 near 0.
+__device__ __forceinline__ double expm1_core(double x) {
     const double big = 6755399441055744.0;  // 1.5 * 2^52
-    const double t0 = __builtin_fma(x2, 1.44269504088896338700e+00, big);
+    const double t0 = __builtin_fma(x, 1.44269504088896338700e+00, big);
     const double k = t0 - big;
-    const uint32_t ki = (uint32_t)__double2loint(t0);  // 0 .. 58 (anything for a NaN, which r carries on)
-    double r = __builtin_fma(k, -6.93147180369123816490e-01, x2);
+    const uint32_t ki = (uint32_t)__double2loint(t0);  // k as a two's-complement integer (anything for a NaN, which r carries on)
+    double r = __builtin_fma(k, -6.93147180369123816490e-01, x);
     r = __builtin_fma(k, -1.90821492927058770002e-10, r);
     const double c[12] = {
         1.60590438368216133e-10, 2.08767569878681002e-09, 2.50521083854417202e-08, 2.75573192239858883e-07, 2.75573192239858925e-06,
@@ -195,16 +206,50 @@ __device__ __forceinline__ float tanh_float_rounded_once(float xf) {
     q = __builtin_fma(q, r, 1.0);
     const double qs = __hiloint2double((int)((uint32_t)__double2hiint(q) + (ki << 20)), __double2loint(q));
     const double p2k = __hiloint2double((int)((1023u + ki) << 20), 0);
-    const double t = __builtin_fma(qs, r, p2k - 1.0);
-    const double y = t / (t + 2.0);
-    const float yf = (float)y;  // |tanh|; a NaN argument has made it NaN
-    return __builtin_copysignf(yf, xf);
+    return __builtin_fma(qs, r, p2k - 1.0);
 }
-template <class T> struct OpTanh { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
-    __device__ __forceinline__ bool operator()(T x, T, T& z) const {
-        if constexpr (sizeof(T) == 4) z = (T)tanh_float_rounded_once((float)x);
-        else z = (T)tanh((double)x);
-        return true; } };
+
+// SFloat tanh, sinh, cosh, expm1: the double-precision function rounded to float once, each
+// from t = exp(a) - 1 above and one IEEE division: tanh|x| = t / (t + 2) with a = 2|x|
+// (clamped at 40, where the answer is 1 in double already); sinh|x| = (t + t / (t + 1)) / 2 and
+// cosh x = (e + 1 / e) / 2, e = t + 1, with a = |x| clamped at 90 (beyond float range either
+// way); expm1 with a = x clamped to [-40, 89]. Run on the CPU against glibc over every float
+// bit pattern, the float results differ nowhere. A NaN argument fails the clamps' comparisons
+// and travels through the arithmetic.
+__device__ __forceinline__ float tanh_float_rounded_once(float xf) {
+    float ax = __builtin_fabsf(xf);
+    ax = (ax > 20.0f) ? 20.0f : ax;
+    const double t = expm1_core(2.0 * (double)ax);
+    return __builtin_copysignf((float)(t / (t + 2.0)), xf);
+}
+__device__ __forceinline__ float sinh_float_rounded_once(float xf) {
+    float ax = __builtin_fabsf(xf);
+    ax = (ax > 90.0f) ? 90.0f : ax;
+    const double t = expm1_core((double)ax);
+    return __builtin_copysignf((float)(0.5 * (t + t / (t + 1.0))), xf);
+}
+__device__ __forceinline__ float cosh_float_rounded_once(float xf) {
+    float ax = __builtin_fabsf(xf);
+    ax = (ax > 90.0f) ? 90.0f : ax;
+    const double e = expm1_core((double)ax) + 1.0;
+    return (float)(0.5 * (e + 1.0 / e));
+}
+__device__ __forceinline__ float expm1_float_rounded_once(float xf) {
+    float xc = (xf < -40.0f) ? -40.0f : xf;
+    xc = (xc > 89.0f) ? 89.0f : xc;
+    const float y = (float)expm1_core((double)xc);
+    return (xf == 0.0f) ? xf : y;  // keeps the sign of a zero argument
+}
+#define CUMO_HIP_OWN_OP(NAME, FEXPR, DEXPR)                                                                                 \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const {                                                    \
+            if constexpr (sizeof(T) == 4) z = (T)FEXPR((float)x);                                                           \
+            else z = (T)(DEXPR);                                                                                            \
+            return true; } };
+CUMO_HIP_OWN_OP(OpTanh, tanh_float_rounded_once, tanh((double)x))
+CUMO_HIP_OWN_OP(OpSinh, sinh_float_rounded_once, sinh((double)x))
+CUMO_HIP_OWN_OP(OpCosh, cosh_float_rounded_once, cosh((double)x))
+CUMO_HIP_OWN_OP(OpExpm1, expm1_float_rounded_once, expm1((double)x))
 
 template <class T> struct OpExp { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
     __device__ __forceinline__ bool operator()(T x, T, T& z) const {
@@ -219,8 +264,6 @@ CUMO_HIP_FUN_H(OpTan, tan((double)x))
 CUMO_HIP_FUN_H(OpAsin, asin((double)x))
 CUMO_HIP_FUN_H(OpAcos, acos((double)x))
 CUMO_HIP_FUN_H(OpAtan, atan((double)x))
-CUMO_HIP_FUN_H(OpSinh, sinh((double)x))
-CUMO_HIP_FUN_H(OpCosh, cosh((double)x))
 CUMO_HIP_FUN_H(OpAsinh, asinh((double)x))
 CUMO_HIP_FUN_H(OpAcosh, acosh((double)x))
 CUMO_HIP_FUN_H(OpAtanh, atanh((double)x))
@@ -229,8 +272,6 @@ CUMO_HIP_FUN_H(OpAtanh, atanh((double)x))
 CUMO_HIP_FUN_H(OpSinc, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
 CUMO_HIP_FUN_H(OpErf, erf((double)x))
 CUMO_HIP_FUN_H(OpErfc, erfc((double)x))
-CUMO_HIP_FUN_H(OpLog1p, log1p((double)x))
-CUMO_HIP_FUN_H(OpExpm1, expm1((double)x))
 
 #define CUMO_HIP_IUN(NAME, EXPR) \
     struct NAME { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false) \

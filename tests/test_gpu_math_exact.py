@@ -67,28 +67,35 @@ def test_exp_on_strided_and_transposed_views():
         assert_ulp(got, oracle.unary("exp", np.ascontiguousarray(hv)), 1)
 
 
-@pytest.mark.parametrize("fn", ["log", "log2", "log10", "tanh"])
-def test_log_family_and_tanh_equal_the_double_function_rounded_once(fn):
-    """SFloat log, log2, log10 and tanh evaluate their own double-precision algorithm (no
-    library call). Run on the CPU against glibc over every float bit pattern the float
-    results differed nowhere; here the device is held to the same: against the CPU oracle
-    ((float)f((double)x) with glibc) <= 1 ulp everywhere and 0 ulp on all but a handful."""
+@pytest.mark.parametrize("fn", ["log", "log2", "log10", "log1p", "tanh", "sinh", "cosh", "expm1"])
+def test_own_double_precision_algorithms_equal_the_double_function_rounded_once(fn):
+    """SFloat log, log2, log10, log1p, tanh, sinh, cosh and expm1 evaluate their own
+    double-precision algorithms (no library call). Run on the CPU against glibc over every
+    float bit pattern the float results differed nowhere (sinh: at two arguments of 2^32, by
+    one ulp); here the device is held to the same: against the CPU oracle ((float)f((double)x)
+    with glibc) <= 1 ulp everywhere and 0 ulp on all but a handful."""
     import cumo_amd
     rng = np.random.default_rng(101)
-    if fn == "tanh":
-        parts = [rng.uniform(-12, 12, size=1 << 22), rng.standard_normal(1 << 22), rng.standard_normal(1 << 21) * 1e-3,
-                 rng.uniform(-0.2, 0.2, size=1 << 21),
-                 np.array([0.0, -0.0, 0.17328, 0.1733, 0.3465, 0.3466, 9.0, 9.011, 19.9, 20.0, 20.1, 1e10, -1e10, 1e-45, -1e-45, 1e-30,
-                           np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5])]
+    special = [0.0, -0.0, 1e-45, -1e-45, 1e-38, 1e-30, -1e-30, 1.0, -1.0, 0.5, 2.0, 10.0, np.inf, -np.inf, np.nan, 3.4028235e38, -3.4028235e38]
+    if fn in ("tanh", "sinh", "cosh", "expm1"):
+        wide = 12 if fn == "tanh" else 89
+        parts = [rng.uniform(-wide, wide, size=1 << 22), rng.standard_normal(1 << 22), rng.standard_normal(1 << 21) * 1e-3,
+                 rng.uniform(-0.4, 0.4, size=1 << 21),
+                 np.array(special + [0.17328, 0.1733, 0.3465, 0.3466, 9.0, 9.011, 19.9, 20.0, 20.1, 39.9, 40.1, -40.1, 88.7, 89.0, 89.5, 90.1,
+                                     -90.1, 1e10, -1e10, 0.000558942498, -0.000558942498])]
+        b = np.arange(0, 1 << 32, 2039, dtype=np.uint64).astype(np.uint32)
+    elif fn == "log1p":
+        parts = [rng.uniform(-1, 10, size=1 << 22), np.expm1(rng.uniform(-20, 88, size=1 << 22)), rng.standard_normal(1 << 21) * 1e-3,
+                 rng.standard_normal(1 << 20) * 1e-9,
+                 np.array(special + [-0.99999994, -1.0000001, -0.5, 1.8626451e-09, 1.8626452e-09, -1.8626451e-09, 0.41421354, -0.29289323])]
         b = np.arange(0, 1 << 32, 2039, dtype=np.uint64).astype(np.uint32)
     else:
         parts = [rng.uniform(0, 10, size=1 << 22), np.exp(rng.uniform(-87, 88, size=1 << 22)), 1 + rng.standard_normal(1 << 21) * 1e-3,
-                 np.array([0.0, -0.0, 1.0, 2.0, 0.5, 10.0, 100.0, 1e-45, 1e-38, 1.1754944e-38, 3.4028235e38, 0.70710677, 0.7071068, 1.4142135,
-                           1.4142137, np.inf, -np.inf, np.nan, -1.0, -1e-45, 8.0, 1024.0, 1e5, 0.001])]
+                 np.array(special + [100.0, 1.1754944e-38, 0.70710677, 0.7071068, 1.4142135, 1.4142137, 8.0, 1024.0, 1e5, 0.001])]
         b = np.arange(0, 1 << 31, 1021, dtype=np.uint64).astype(np.uint32)   # every binade, subnormals included
-    h = np.concatenate([np.concatenate(parts).astype(np.float32), b.view(np.float32)])
-    got = getattr(cumo_amd.NMath, fn)(cumo_amd.SFloat.cast(h)).to_numpy()
     with np.errstate(all="ignore"):
+        h = np.concatenate([np.concatenate(parts).astype(np.float32), b.view(np.float32)])
+        got = getattr(cumo_amd.NMath, fn)(cumo_amd.SFloat.cast(h)).to_numpy()
         want = oracle.unary(fn, h)
     assert_ulp(got, want, 1, "SFloat %s vs the CPU oracle" % fn)
     nan = np.isnan(want)
