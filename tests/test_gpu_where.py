@@ -160,3 +160,27 @@ def test_mask_of_single_runs_with_offsets_steps_and_reversal(tname, dt):
     none, every = cumo_amd.Bit.cast(np.zeros(n, dtype=np.uint8)), cumo_amd.Bit.cast(np.ones(n, dtype=np.uint8))
     assert none.mask(x).to_numpy().shape == (0,)
     assert (every.mask(x).to_numpy() == hx).all()
+
+
+def test_where_beyond_two_to_the_32_elements_answers_int64():
+    """More than 2^32 - 1 elements: positions no longer fit Int32 (gen/tmpl_bit/where.c:104-110
+    picks Int64 then). The bits are set on the device buffer word by word; no host array of
+    that length is made."""
+    import ctypes as C
+    import cumo_amd
+    from cumo_amd import _lib
+    n = (1 << 32) + 70
+    b = cumo_amd.Bit.zeros(n)
+    want = [5, (1 << 31) + 3, (1 << 32) - 1, 1 << 32, (1 << 32) + 69]
+    for pos in want:
+        word = np.array([1 << (pos % 32)], dtype=np.uint32)
+        assert _lib.call(_lib.lib.cumo_hip_copy_from_host, b._buf.ptr + (pos // 32) * 4, word.ctypes.data, 4) == 0
+    assert int(b.count_true()) == len(want)
+    got = b.where()
+    assert isinstance(got, cumo_amd.Int64) and got.to_numpy().tolist() == want
+    # a view that starts beyond 2^32 bits
+    tail = b[(1 << 32) - 2:]
+    assert tail.where().to_numpy().tolist() == [1, 2, 71]
+    assert int(tail.count_false()) == 72 - 3
+    del b, tail, got
+    cumo_amd.MemoryPool.free_all_blocks()
