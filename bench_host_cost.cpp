@@ -87,13 +87,20 @@ int main() {
         cumo_hip_na_reduce("sum", &x, 0, 0, 0, &r, NULL);
         cumo_cuda_runtime_free(r.ptr);
     });
+    // the same on a stream of its own instead of the null stream
+    void* st = cumo_hip_stream_create();
+    cumo_hip_set_stream(st);
+    const double empty_own = us_per_call(N, 4, [&] { cumo_hip_launch_empty_kernel(0); });
+    const double add_own = us_per_call(N, 4, [&] { cumo_hip_na_binary("add", &x, &y, &z); });
+    cumo_hip_set_stream(NULL);
+    cumo_hip_stream_destroy(st);
     const char* msg = NULL;
     if (cumo_hip_last_error(&msg)) {
         std::fprintf(stderr, "bench_host_cost: %s\n", msg ? msg : "error");
         return 1;
     }
     std::printf("{\"unit\": \"us per operation\", \"shape\": \"32x32 SFloat\", \"ndloop_prepare\": %.3f, \"empty_launch\": %.2f, \"empty_launch_1k\": %.2f, "
-                "\"launcher_add\": %.2f, \"add_into_result\": %.2f, \"add_issue\": %.2f, \"add_alloc_free\": %.2f, \"sum_alloc_free\": %.2f}\n",
-                prepare, empty, empty_1k, launcher, add_into, add_issue, add_alloc, sum_alloc);
+                "\"launcher_add\": %.2f, \"add_into_result\": %.2f, \"add_issue\": %.2f, \"add_alloc_free\": %.2f, \"sum_alloc_free\": %.2f, \"own_stream_empty_launch\": %.2f, \"own_stream_add_into_result\": %.2f}\n",
+                prepare, empty, empty_1k, launcher, add_into, add_issue, add_alloc, sum_alloc, empty_own, add_own);
     return 0;
 }

@@ -127,6 +127,8 @@ _sig = {
     "cumo_hip_last_error": (C.c_int, [P(C.c_char_p)]),
     "cumo_hip_set_stream": (None, [C.c_void_p]),
     "cumo_hip_get_stream": (C.c_void_p, []),
+    "cumo_hip_stream_create": (C.c_void_p, []),
+    "cumo_hip_stream_destroy": (None, [C.c_void_p]),
     "cumo_hip_device_count": (C.c_int, []),
     "cumo_hip_synchronize": (None, []),
     "cumo_hip_event_create": (C.c_void_p, []),

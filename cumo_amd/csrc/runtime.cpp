@@ -69,6 +69,19 @@ int cumo_hip_last_error(const char** message) {
 void cumo_hip_set_stream(void* hip_stream) { t_stream = (hipStream_t)hip_stream; }
 void* cumo_hip_get_stream(void) { return (void*)t_stream; }
 
+// a stream of the default priority that does not synchronise with the null stream
+void* cumo_hip_stream_create(void) {
+    hipStream_t st = nullptr;
+    if (!hip_ok(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "hipStreamCreate")) return nullptr;
+    return (void*)st;
+}
+
+void cumo_hip_stream_destroy(void* hip_stream) {
+    if (!hip_stream) return;
+    if (t_stream == (hipStream_t)hip_stream) t_stream = nullptr;
+    hip_ok(hipStreamDestroy((hipStream_t)hip_stream), "hipStreamDestroy");
+}
+
 int cumo_hip_device_count(void) {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess) {

@@ -539,6 +539,11 @@ void cumo_hip_scan_cols_kernel_launch(int type, int prod, int nan, const cumo_hi
  * reference only ever uses the default stream (cuda/memory_pool.cpp:43-44). */
 void  cumo_hip_set_stream(void* hip_stream);
 void* cumo_hip_get_stream(void);
+/* a stream of the default priority that does not synchronise with the null stream, for
+ * callers without a HIP binding of their own; destroy resets the current stream to the
+ * null stream if it was this one */
+void* cumo_hip_stream_create(void);
+void  cumo_hip_stream_destroy(void* hip_stream);
 int   cumo_hip_device_count(void);
 void  cumo_hip_synchronize(void);
 /* events on the current stream, for callers that time launches */
