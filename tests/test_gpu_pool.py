@@ -89,3 +89,41 @@ def test_pool_disabled_goes_straight_to_the_device():
         del a
     finally:
         cumo_amd.MemoryPool.enable()
+
+
+def test_two_streams_share_the_pool_without_mixing_results():
+    """Work alternates between the null stream and a stream of the library's own making; arrays
+    released on one stream are taken over by allocations on the other (whole blocks change
+    stream behind an event). Every result must be what the same operations give on one stream."""
+    import cumo_amd
+    from cumo_amd import _lib
+    L = _lib.lib
+    rng = np.random.default_rng(77)
+    n = 1 << 20
+    hx = rng.standard_normal(n).astype(np.float32)
+    x = cumo_amd.SFloat.cast(hx)
+    own = L.cumo_hip_stream_create()
+    assert own
+    try:
+        want = hx
+        got = x
+        for it in range(12):
+            L.cumo_hip_set_stream(own if it % 2 == 0 else None)
+            if it:
+                # what the other stream produced must be complete before this stream reads it
+                L.cumo_hip_set_stream(None if it % 2 == 0 else own)
+                cumo_amd.synchronize()
+                L.cumo_hip_set_stream(own if it % 2 == 0 else None)
+            tmp = got * 1.5            # a temporary that is released at once, on this stream
+            got = tmp + float(it)
+            del tmp
+            want = want * np.float32(1.5) + np.float32(it)
+            cumo_amd.MemoryPool.free_all_blocks() if it == 5 else None
+        cumo_amd.synchronize()
+        L.cumo_hip_set_stream(None)
+        assert (got.to_numpy().view(np.uint32) == want.view(np.uint32)).all()
+    finally:
+        L.cumo_hip_set_stream(None)
+        L.cumo_hip_synchronize()
+        L.cumo_hip_stream_destroy(own)
+    _lib.check()
