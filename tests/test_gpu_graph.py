@@ -71,7 +71,9 @@ def test_mixed_chain_of_every_kernel_family():
     with cumo.Graph() as g:
         got = chain_mixed(cumo, S, X, M, I)
     # intermediates released inside the block stay reserved for the graph
-    assert cumo.MemoryPool.used_bytes() > used_before + sum(r._buf.nbytes for r in got)
+    pooled = cumo.MemoryPool.enabled()   # with CUMO_MEMORY_POOL=OFF the pool's counters stay at 0
+    if pooled:
+        assert cumo.MemoryPool.used_bytes() > used_before + sum(r._buf.nbytes for r in got)
     for k in range(3):
         g.launch()
         for i, (r, w) in enumerate(zip(got, want)):
@@ -83,7 +85,8 @@ def test_mixed_chain_of_every_kernel_family():
         cumo.synchronize()
     held = cumo.MemoryPool.used_bytes()
     g.close()
-    assert cumo.MemoryPool.used_bytes() < held
+    if pooled:
+        assert cumo.MemoryPool.used_bytes() < held
     # the same operations still run one by one afterwards
     again = [r.to_numpy() for r in chain_mixed(cumo, S, X, M, I)]
     for a, w in zip(again, want):
