@@ -67,12 +67,12 @@ def test_exp_on_strided_and_transposed_views():
         assert_ulp(got, oracle.unary("exp", np.ascontiguousarray(hv)), 1)
 
 
-@pytest.mark.parametrize("fn", ["log", "log2", "log10", "log1p", "tanh", "sinh", "cosh", "expm1"])
+@pytest.mark.parametrize("fn", ["log", "log2", "log10", "log1p", "tanh", "sinh", "cosh", "expm1", "asinh", "acosh", "atanh"])
 def test_own_double_precision_algorithms_equal_the_double_function_rounded_once(fn):
-    """SFloat log, log2, log10, log1p, tanh, sinh, cosh and expm1 evaluate their own
-    double-precision algorithms (no library call). Run on the CPU against glibc over every
-    float bit pattern the float results differed nowhere (sinh: at two arguments of 2^32, by
-    one ulp); here the device is held to the same: against the CPU oracle ((float)f((double)x)
+    """SFloat log, log2, log10, log1p, tanh, sinh, cosh, expm1, asinh, acosh and atanh evaluate
+    their own double-precision algorithms (no library call). Run on the CPU against glibc over
+    every float bit pattern the float results differed nowhere (sinh at two arguments of 2^32,
+    asinh at four, acosh at two, each by one ulp); here the device is held to the same: against the CPU oracle ((float)f((double)x)
     with glibc) <= 1 ulp everywhere and 0 ulp on all but a handful."""
     import cumo_amd
     rng = np.random.default_rng(101)
@@ -83,6 +83,19 @@ def test_own_double_precision_algorithms_equal_the_double_function_rounded_once(
                  rng.uniform(-0.4, 0.4, size=1 << 21),
                  np.array(special + [0.17328, 0.1733, 0.3465, 0.3466, 9.0, 9.011, 19.9, 20.0, 20.1, 39.9, 40.1, -40.1, 88.7, 89.0, 89.5, 90.1,
                                      -90.1, 1e10, -1e10, 0.000558942498, -0.000558942498])]
+        b = np.arange(0, 1 << 32, 2039, dtype=np.uint64).astype(np.uint32)
+    elif fn in ("asinh", "acosh", "atanh"):
+        edge = [1.8626451e-09, 1.8626452e-09, -1.8626451e-09, 0.99999994, -0.99999994, 1.0000001, -1.0000001, 4.19005794e18,
+                -4.19005794e18, 2.74915304e28, -2.74915304e28, 1e-20, 1e-5, -1e-5, 0.5, 1e19, 1e20, 3e38]
+        if fn == "atanh":
+            parts = [rng.uniform(-1, 1, size=1 << 22), np.tanh(rng.uniform(-10, 10, size=1 << 22)), rng.standard_normal(1 << 21) * 1e-3,
+                     rng.standard_normal(1 << 20) * 1e-9, rng.uniform(-1.5, 1.5, size=1 << 16), np.array(special + edge)]
+        elif fn == "acosh":
+            parts = [rng.uniform(1, 10, size=1 << 22), np.cosh(rng.uniform(0, 88, size=1 << 22)), 1 + np.abs(rng.standard_normal(1 << 21)) * 1e-4,
+                     rng.uniform(-1, 1, size=1 << 16), np.array(special + edge)]
+        else:
+            parts = [rng.uniform(-10, 10, size=1 << 22), np.sinh(rng.uniform(-88, 88, size=1 << 22)), rng.standard_normal(1 << 21) * 1e-3,
+                     rng.standard_normal(1 << 20) * 1e-9, np.array(special + edge)]
         b = np.arange(0, 1 << 32, 2039, dtype=np.uint64).astype(np.uint32)
     elif fn == "log1p":
         parts = [rng.uniform(-1, 10, size=1 << 22), np.expm1(rng.uniform(-20, 88, size=1 << 22)), rng.standard_normal(1 << 21) * 1e-3,
