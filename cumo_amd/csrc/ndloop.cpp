@@ -1483,6 +1483,30 @@ int result_1d(NA* z, int type, size_t n, bool* allocated) {
         return fail(CUMO_HIP_ERROR_SHAPE, "the given result must be a contiguous 1-D array of the result's type and exact length");
     return 0;
 }
+// A mask that walks as one run: its hits are counted block by block, the counts read back
+// (the one stream synchronisation) and added up here to size the result, and the same
+// counts then place the hits: positions (x == NULL, as itype) or the elements of the run
+// (x, sx) of xtype.
+int where_single_run(const LP& lp, int invert, int rtype, const char* x, ssize_t sx, NA* z) {
+    const cumo_hip_loop_args_t& in = lp.args[0];
+    const uint64_t n = lp.n[0];
+    const size_t nb = cumo_hip_bit_where_blocks(n);
+    uint64_t host_counts[1024];
+    if (nb > sizeof(host_counts) / sizeof(host_counts[0])) return fail(CUMO_HIP_ERROR_ARGUMENT, "where: more block counts than expected");
+    uint64_t* counts = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(nb * sizeof(uint64_t)));
+    if (!counts) return CUMO_HIP_ERROR_OUT_OF_MEMORY;
+    cumo_hip_bit_where_count_kernel_launch((CUMO_BIT_DIGIT*)in.ptr, in.bitpos, in.step[0], n, invert, counts);
+    int rc = cumo_hip_copy_to_host(host_counts, counts, nb * sizeof(uint64_t));
+    uint64_t n_hit = 0;
+    for (size_t b = 0; b < nb; ++b) n_hit += host_counts[b];
+    bool allocated = false;
+    if (!rc) rc = result_1d(z, rtype, (size_t)n_hit, &allocated);
+    if (!rc && n_hit != 0)
+        cumo_hip_bit_where_place_kernel_launch((CUMO_BIT_DIGIT*)in.ptr, in.bitpos, in.step[0], n, invert, counts, x, sx, (size_t)kElmsz[rtype],
+                                               z->ptr + z->offset);
+    cumo_cuda_runtime_free(reinterpret_cast<char*>(counts));
+    return rc;
+}
 }  // namespace
 
 // z = positions (row-major, from 0) of the set bits of x, or of the clear ones when
@@ -1493,6 +1517,13 @@ int cumo_hip_na_where(const cumo_hip_narray_t* x, int invert, cumo_hip_narray_t*
     if (rc) return rc;
     if (x->type != CUMO_HIP_BIT) return no_method("where");
     if (!z) return fail(CUMO_HIP_ERROR_ARGUMENT, "where: no result descriptor");
+    if (total_of(x) != 0) {
+        cumo_hip_ndfunc_t nf1 = {NULL, 0, 1, 0, {0, 0}};
+        const NA* in1[1] = {x};
+        LP lp1;
+        if (cumo_hip_na_ndloop_prepare(&nf1, in1, NULL, 0, &lp1) == CUMO_HIP_OK && lp1.ndim == 1)
+            return where_single_run(lp1, invert ? 1 : 0, total_of(x) > 4294967295ull ? CUMO_HIP_INT64 : CUMO_HIP_INT32, NULL, 0, z);
+    }
     NA cnt;
     cnt.ptr = NULL;
     rc = cumo_hip_na_bit_count(x, 0, 0, invert, &cnt);
@@ -1545,26 +1576,7 @@ int cumo_hip_na_mask(const cumo_hip_narray_t* mask, const cumo_hip_narray_t* x, 
         const NA* in[2] = {mask, x};
         LP lp;
         if (cumo_hip_na_ndloop_prepare(&nf, in, NULL, 0, &lp) == CUMO_HIP_OK && lp.ndim == 1) {
-            NA cnt;
-            cnt.ptr = NULL;
-            rc = cumo_hip_na_bit_count(mask, 0, 0, 0, &cnt);
-            if (rc) return rc;
-            uint64_t n_hit = 0;
-            rc = cumo_hip_copy_to_host(&n_hit, cnt.ptr + cnt.offset, sizeof(n_hit));
-            free_tmp(&cnt);
-            if (rc) return rc;
-            bool allocated;
-            rc = result_1d(z, x->type, (size_t)n_hit, &allocated);
-            if (rc || n_hit == 0) return rc;
-            char* scratch = cumo_bit_where_scratch_new();
-            if (!scratch) {
-                if (allocated) free_tmp(z);
-                return CUMO_HIP_ERROR_OUT_OF_MEMORY;
-            }
-            cumo_hip_bit_compact_kernel_launch((CUMO_BIT_DIGIT*)lp.args[0].ptr, lp.args[0].bitpos, lp.args[0].step[0], lp.n[0], lp.args[1].ptr,
-                                               lp.args[1].step[0], (size_t)kElmsz[x->type], z->ptr + z->offset, scratch);
-            cumo_cuda_runtime_free(scratch);
-            return CUMO_HIP_OK;
+            return where_single_run(lp, 0, x->type, lp.args[1].ptr, lp.args[1].step[0], z);
         }
     }
     NA pos;

@@ -109,7 +109,9 @@ __global__ __launch_bounds__(kWhBlock) void where_scan_kernel(uint64_t* block_su
 // MODE 1: out[o] = the masked array's element position p2 + j*s2 (or p2 + idx2[j]), as size_t (mask).
 // MODE 2: out[o] = the masked array's element itself, elmsz (4 or 8) bytes read at p2 + j*s2 where p2 is
 //         its address (the compaction the reference reaches through a view over the positions of mode 1).
-template <int MODE>
+// COUNTS: block_sums holds the blocks' plain counts (no scan launch ran): the block adds up
+// the counts of the blocks before it.
+template <int MODE, bool COUNTS>
 __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
                                                                  int contiguous, int invert, uint64_t nchunks, uint64_t cpb, char* out, size_t elmsz,
                                                                  uint64_t count, size_t p2, int64_t s2, const size_t* idx2,
@@ -120,10 +122,20 @@ __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_
     // hits of one round (256 chunks, up to 8192 bits) are listed in LDS by their bit
     // position within the round, then written out by consecutive lanes
     __shared__ uint16_t hit[kWhBlock * 32];
-    uint64_t off = block_sums[blockIdx.x];
+    uint64_t off;
+    if (COUNTS) {
+        uint64_t before = 0;
+        for (uint64_t t = threadIdx.x; t < blockIdx.x; t += kWhBlock) before += block_sums[t];
+        wh_block_exscan(before, &off);
+    } else {
+        off = block_sums[blockIdx.x];
+    }
+    // the next round's bits are loaded before this round's are placed
+    uint32_t znext = start + threadIdx.x < end ? wh_chunk(a, p, s, idx, n, start + threadIdx.x, contiguous, invert) : 0u;
     for (uint64_t c0 = start; c0 < end; c0 += kWhBlock) {
-        const uint64_t c = c0 + threadIdx.x;
-        uint32_t z = c < end ? wh_chunk(a, p, s, idx, n, c, contiguous, invert) : 0u;
+        uint32_t z = znext;
+        const uint64_t cn = c0 + kWhBlock + threadIdx.x;
+        znext = cn < end ? wh_chunk(a, p, s, idx, n, cn, contiguous, invert) : 0u;
         uint64_t total;
         // the first barrier inside the scan also ends the previous round's reads of hit[]
         uint32_t o = (uint32_t)wh_block_exscan((uint64_t)__popc(z), &total);
@@ -151,20 +163,31 @@ __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_
     }
 }
 
+// a run of n bits as 32-bit chunks shared out over the blocks, a contiguous range each
+struct WhGeometry {
+    uint64_t nchunks, nblocks, cpb;
+};
+WhGeometry wh_geometry(uint64_t n) {
+    WhGeometry g;
+    g.nchunks = (n + 31) / 32;
+    g.nblocks = (g.nchunks + kWhBlock - 1) / kWhBlock;
+    if (g.nblocks > kWhMaxBlocks) g.nblocks = kWhMaxBlocks;
+    g.cpb = g.nblocks ? (g.nchunks + g.nblocks - 1) / g.nblocks : 0;
+    return g;
+}
+
 template <int MODE>
 void where_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t n, int invert, char* out, size_t elmsz, uint64_t count, size_t p2,
                   ssize_t s2, size_t* idx2, uint64_t* running, uint64_t* block_sums) {
     if (n == 0) return;  // a grid of no blocks is an invalid launch
-    const uint64_t nchunks = (n + 31) / 32;
+    const WhGeometry g = wh_geometry(n);
+    const uint64_t nchunks = g.nchunks, nblocks = g.nblocks, cpb = g.cpb;
     const int contiguous = (idx == nullptr && s == 1) ? 1 : 0;
-    uint64_t nblocks = (nchunks + kWhBlock - 1) / kWhBlock;
-    if (nblocks > kWhMaxBlocks) nblocks = kWhMaxBlocks;
-    const uint64_t cpb = (nchunks + nblocks - 1) / nblocks;
     hipStream_t st = current_stream();
     hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n, contiguous,
                        invert, nchunks, cpb, block_sums);
     hipLaunchKernelGGL(where_scan_kernel, dim3(1), dim3(kWhBlock), 0, st, block_sums, nblocks, running);
-    hipLaunchKernelGGL((where_scatter_kernel<MODE>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n,
+    hipLaunchKernelGGL((where_scatter_kernel<MODE, false>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n,
                        contiguous, invert, nchunks, cpb, out, elmsz, count, p2, (int64_t)s2, (const size_t*)idx2, (const uint64_t*)block_sums);
     cumo_cuda_runtime_check_kernel_launch();
 }
@@ -246,13 +269,37 @@ void cumo_bit_mask_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t*
                        reinterpret_cast<uint64_t*>(scratch) + 2);
 }
 
-// out[o] = the o-th element of the run x + j*sx (j = 0 .. n-1) whose bit in the run (a, p, s) is set:
-// the compaction of values in the same three launches as where. elmsz 4 or 8. The scratch is the one of
-// cumo_bit_where_scratch_new; its first cursor carries the output position from one run to the next.
-void cumo_hip_bit_compact_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, uint64_t n, const char* x, ssize_t sx, size_t elmsz, char* out,
-                                        char* scratch) {
-    where_launch<2>(a, p, s, nullptr, n, 0, out, elmsz, 0, (size_t)(uintptr_t)x, sx, nullptr, reinterpret_cast<uint64_t*>(scratch),
-                    reinterpret_cast<uint64_t*>(scratch) + 2);
+// The same compaction for a caller that sizes the result in between: the blocks' counts of one run
+// (cumo_hip_bit_where_blocks(n) of them, every one written), which the caller reads back and adds
+// up, then the placement, where every block adds up the counts before it. Two launches instead of
+// a count for the size plus the three above.
+size_t cumo_hip_bit_where_blocks(uint64_t n) { return (size_t)wh_geometry(n).nblocks; }
+
+void cumo_hip_bit_where_count_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, uint64_t n, int invert, uint64_t* counts) {
+    if (n == 0) return;
+    const WhGeometry g = wh_geometry(n);
+    hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, current_stream(), a, (uint64_t)p, (int64_t)s,
+                       (const size_t*)nullptr, n, s == 1 ? 1 : 0, invert, g.nchunks, g.cpb, counts);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+// x == NULL: out[o] = the position in the run of the o-th hit, as an elmsz-byte integer (4 or 8);
+// otherwise out[o] = the element (elmsz 4 or 8 bytes) at x + j*sx of the o-th hit j.
+void cumo_hip_bit_where_place_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, uint64_t n, int invert, const uint64_t* counts, const char* x,
+                                            ssize_t sx, size_t elmsz, char* out) {
+    if (n == 0) return;
+    const WhGeometry g = wh_geometry(n);
+    const int contiguous = s == 1 ? 1 : 0;
+    hipStream_t st = current_stream();
+    if (x)
+        hipLaunchKernelGGL((where_scatter_kernel<2, true>), dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s,
+                           (const size_t*)nullptr, n, contiguous, invert, g.nchunks, g.cpb, out, elmsz, (uint64_t)0, (size_t)(uintptr_t)x, (int64_t)sx,
+                           (const size_t*)nullptr, counts);
+    else
+        hipLaunchKernelGGL((where_scatter_kernel<0, true>), dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s,
+                           (const size_t*)nullptr, n, contiguous, invert, g.nchunks, g.cpb, out, elmsz, (uint64_t)0, (size_t)0, (int64_t)0,
+                           (const size_t*)nullptr, counts);
+    cumo_cuda_runtime_check_kernel_launch();
 }
 
 void cumo_hip_gather_flat_kernel_launch(const cumo_hip_gather_flat_t* d) {

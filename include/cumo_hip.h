@@ -491,13 +491,19 @@ typedef struct {
 } cumo_hip_mulsum_rows_t;
 int cumo_hip_mulsum_rows_kernel_launch(int type, int nan, const cumo_hip_mulsum_rows_t* rows);
 
-/* out[o] = the o-th element of the run x + j*sx, j = 0 .. n-1, whose bit in the run of
- * bits (a, p, s) is set: a[mask] for one run in the three launches of where, without
- * the array of positions the reference goes through (tmpl_bit/mask.c:141-167 makes a
- * view over them). elmsz 4 or 8; scratch from cumo_bit_where_scratch_new, whose first
- * cursor carries the output position from one run to the next. */
-void cumo_hip_bit_compact_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, const char *x, ssize_t sx, size_t elmsz,
-                                        char *out, char *scratch);
+/* The compaction of one run for a caller that sizes the result in between (the host
+ * iterator of tmpl_bit/where.c:13-28 counts first, reads the count back and allocates):
+ * count writes the hits of each block's share of the run into counts[0 ..
+ * cumo_hip_bit_where_blocks(n) - 1]; the caller copies them to the host and adds them
+ * up; place puts the o-th hit's position in the run (x == NULL; as elmsz-byte integers,
+ * 4 or 8) or its element x + j*sx (elmsz 4 or 8; a[mask] without the array of positions
+ * that tmpl_bit/mask.c:141-167 makes a view over) at out[o], every block adding up the
+ * counts before it. Two launches where a count for the size plus the three of
+ * cumo_bit_where_kernel_launch were five. invert: the clear bits are the hits. */
+size_t cumo_hip_bit_where_blocks(uint64_t n);
+void cumo_hip_bit_where_count_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, int invert, uint64_t *counts);
+void cumo_hip_bit_where_place_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, int invert, const uint64_t *counts,
+                                            const char *x, ssize_t sx, size_t elmsz, char *out);
 
 /* out[i] = the element of a strided view at flat row-major position pos[i] (no
  * counterpart symbol in the reference, where a masked array is a view over an index

@@ -113,6 +113,54 @@ def test_where_and_mask_launchers_with_index_arrays_and_a_carried_cursor():
     free(pw, pidx, pout, pz, pm)
 
 
+@pytest.mark.parametrize("nbits", [1, 31, 8193, 1 << 20, (1 << 25) + 77])
+def test_count_then_place_launchers(nbits):
+    """The two-launch form for a caller that sizes the result in between: block counts, read back and
+    added up, then the placement of positions (set or clear bits, 4- or 8-byte) or of elements."""
+    from cumo_amd import _lib
+    from test_gpu_raw_abi import dev, fetch, free
+    rng = np.random.default_rng(nbits)
+    lead = 37                                       # the run starts inside a word
+    h = (rng.random(lead + 3 * nbits if nbits < 10000 else lead + nbits) < 0.4).astype(np.uint8)
+    pad = (-h.size) % 32
+    words = np.frombuffer(np.packbits(np.concatenate([h, np.zeros(pad, np.uint8)]), bitorder="little").tobytes(), dtype=np.uint32)
+    pw = dev(words)
+    blocks = _lib.fn("cumo_hip_bit_where_blocks", C.c_size_t, [C.c_uint64])
+    count = _lib.fn("cumo_hip_bit_where_count_kernel_launch", None, [C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_uint64, C.c_int, C.c_void_p])
+    place = _lib.fn("cumo_hip_bit_where_place_kernel_launch", None,
+                    [C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_uint64, C.c_int, C.c_void_p, C.c_void_p, C.c_ssize_t, C.c_size_t, C.c_void_p])
+    nb = blocks(nbits)
+    assert 1 <= nb <= 1024 and blocks(0) == 0
+    x = rng.standard_normal(nbits).astype(np.float32)
+    xd = rng.standard_normal(2 * nbits)             # every second double
+    px, pxd = dev(x), dev(xd)
+    cases = [(1, 0, 8), (1, 1, 4)] + ([(3, 0, 4)] if nbits < 10000 else [])
+    for step, invert, elmsz in cases:
+        run = h[lead:lead + step * nbits:step]
+        hits = np.flatnonzero(run == (0 if invert else 1))
+        pc = dev(np.full(nb + 1, 12345, dtype=np.uint64))
+        _lib.call(count, pw, lead, step, nbits, invert, pc)
+        counts = fetch(pc, (nb + 1,), np.uint64)
+        assert int(counts[:nb].sum()) == hits.size and counts[nb] == 12345
+        it = np.int64 if elmsz == 8 else np.int32
+        po = dev(np.full(hits.size + 3, -1, dtype=it))
+        _lib.call(place, pw, lead, step, nbits, invert, pc, None, 0, elmsz, po)
+        got = fetch(po, (hits.size + 3,), it)
+        assert (got[:hits.size] == hits).all() and (got[hits.size:] == -1).all()
+        if step == 1 and not invert:
+            pv = dev(np.full(hits.size + 1, 7.0, dtype=np.float32))
+            _lib.call(place, pw, lead, 1, nbits, 0, pc, px, 4, 4, pv)
+            gv = fetch(pv, (hits.size + 1,), np.float32)
+            assert (gv[:hits.size] == x[hits]).all() and gv[hits.size] == 7.0
+            pv8 = dev(np.full(hits.size + 1, 7.0, dtype=np.float64))
+            _lib.call(place, pw, lead, 1, nbits, 0, pc, pxd, 16, 8, pv8)
+            gv8 = fetch(pv8, (hits.size + 1,), np.float64)
+            assert (gv8[:hits.size] == xd[::2][hits]).all() and gv8[hits.size] == 7.0
+            free(pv, pv8)
+        free(pc, po)
+    free(pw, px, pxd)
+
+
 def test_where_and_mask_into_a_given_result():
     """A result array of exactly the count's length is written in place; any other length is a shape error."""
     import ctypes as C
