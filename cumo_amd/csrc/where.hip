@@ -12,7 +12,7 @@
 // the cursor); every block walks its range again, 256 chunks a round: an exclusive
 // scan over the block places each chunk's hits in a list in LDS, and consecutive
 // lanes then write the list out, so the stores of a wave are adjacent. Blocks are 256
-// threads (4 wave64): the scan inside a block is a wave scan by shuffles plus four LDS
+// threads (4 wave64): the scan inside a block is a wave scan by DPP steps plus four LDS
 // slots.
 // A contiguous run reads whole words (two per chunk when the run starts inside a
 // word); strided and index-array runs gather bit by bit.
@@ -78,6 +78,42 @@ __device__ __forceinline__ uint64_t wh_block_exscan(uint64_t v, uint64_t* total)
     return before + inc - v;
 }
 
+// A barrier for the LDS traffic only: loads from global memory that were sent ahead stay
+// in flight across it (__syncthreads() waits for them as well).
+__device__ __forceinline__ void wh_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// inclusive scan over the 64 lanes of a wave: four shifts within the rows of 16 lanes,
+// then lane 15 of a row into the next row and lane 31 into the upper half
+__device__ __forceinline__ uint32_t wh_wave_scan(uint32_t v) {
+    int x = (int)v;
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, true);   // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, true);   // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, true);   // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, true);   // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+    return (uint32_t)x;
+}
+
+// exclusive scan of one small value per thread over the block (the sum fits 32 bits); *total
+// gets the block's sum in every thread. Two LDS-only barriers; safe to call again right away.
+__device__ __forceinline__ uint32_t wh_block_exscan32(uint32_t v, uint32_t* total) {
+    __shared__ uint32_t wave_sum32[kWhBlock / 64];
+    const uint32_t inc = wh_wave_scan(v);
+    wh_lds_barrier();  // the slots may still be read from the previous call
+    if ((threadIdx.x & 63) == 63) wave_sum32[threadIdx.x >> 6] = inc;
+    wh_lds_barrier();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (unsigned w = 0; w < kWhBlock / 64; ++w) {
+        const uint32_t ws = wave_sum32[w];
+        before += (w < (threadIdx.x >> 6)) ? ws : 0u;
+        all += ws;
+    }
+    *total = all;
+    return before + inc - v;
+}
+
 __global__ __launch_bounds__(kWhBlock) void where_count_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
                                                                int contiguous, int invert, uint64_t nchunks, uint64_t cpb, uint64_t* block_sums) {
     uint64_t start = (uint64_t)blockIdx.x * cpb;
@@ -105,17 +141,18 @@ __global__ __launch_bounds__(kWhBlock) void where_scan_kernel(uint64_t* block_su
     if (threadIdx.x == 0) *running = acc;
 }
 
-// MODE 0: out[o] = count + position in the run, as elmsz-byte integers (where).
-// MODE 1: out[o] = the masked array's element position p2 + j*s2 (or p2 + idx2[j]), as size_t (mask).
-// MODE 2: out[o] = the masked array's element itself, elmsz (4 or 8) bytes read at p2 + j*s2 where p2 is
+// MODE 0: out[o] = count + position in the run, as ES-byte integers (where).
+// MODE 1: out[o] = the masked array's element position p2 + j*s2 (or p2 + idx2[j]), as size_t (mask; ES 8).
+// MODE 2: out[o] = the masked array's element itself, ES (4 or 8) bytes read at p2 + j*s2 where p2 is
 //         its address (the compaction the reference reaches through a view over the positions of mode 1).
 // COUNTS: block_sums holds the blocks' plain counts (no scan launch ran): the block adds up
 // the counts of the blocks before it.
-template <int MODE, bool COUNTS>
+template <int MODE, int ES, bool COUNTS>
 __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
-                                                                 int contiguous, int invert, uint64_t nchunks, uint64_t cpb, char* out, size_t elmsz,
+                                                                 int contiguous, int invert, uint64_t nchunks, uint64_t cpb, char* out,
                                                                  uint64_t count, size_t p2, int64_t s2, const size_t* idx2,
                                                                  const uint64_t* block_sums) {
+    typedef typename std::conditional<ES == 4, uint32_t, uint64_t>::type E;
     uint64_t start = (uint64_t)blockIdx.x * cpb;
     if (start > nchunks) start = nchunks;
     const uint64_t end = (nchunks - start < cpb) ? nchunks : start + cpb;
@@ -136,27 +173,27 @@ __global__ __launch_bounds__(kWhBlock) void where_scatter_kernel(const CUMO_BIT_
         uint32_t z = znext;
         const uint64_t cn = c0 + kWhBlock + threadIdx.x;
         znext = cn < end ? wh_chunk(a, p, s, idx, n, cn, contiguous, invert) : 0u;
-        uint64_t total;
+        uint32_t total;
         // the first barrier inside the scan also ends the previous round's reads of hit[]
-        uint32_t o = (uint32_t)wh_block_exscan((uint64_t)__popc(z), &total);
+        uint32_t o = wh_block_exscan32((uint32_t)__popc(z), &total);
+        const uint32_t mine = threadIdx.x * 32;
         while (z) {
-            hit[o++] = (uint16_t)(threadIdx.x * 32 + (unsigned)(__ffs((int)z) - 1));
+            hit[o++] = (uint16_t)(mine + (unsigned)__builtin_ctz(z));
             z &= z - 1;
         }
-        __syncthreads();
-        for (uint32_t k = threadIdx.x; k < (uint32_t)total; k += kWhBlock) {
-            const uint64_t j = c0 * 32 + hit[k];
-            const uint64_t w = off + k;
+        wh_lds_barrier();
+        const uint64_t j0 = c0 * 32;             // the round's first bit, and where its hits go
+        E* const dst = reinterpret_cast<E*>(out) + off;
+#pragma unroll 4
+        for (uint32_t k = threadIdx.x; k < total; k += kWhBlock) {
+            const uint32_t h = hit[k];
             if (MODE == 2) {
-                const char* src = reinterpret_cast<const char*>(p2) + (int64_t)j * s2;
-                if (elmsz == 4) reinterpret_cast<uint32_t*>(out)[w] = *reinterpret_cast<const uint32_t*>(src);
-                else reinterpret_cast<uint64_t*>(out)[w] = *reinterpret_cast<const uint64_t*>(src);
+                dst[k] = *reinterpret_cast<const E*>(reinterpret_cast<const char*>(p2) + (int64_t)(j0 + h) * s2);
             } else if (MODE == 1) {
-                reinterpret_cast<size_t*>(out)[w] = idx2 ? (p2 + idx2[j]) : (size_t)((int64_t)p2 + (int64_t)j * s2);
-            } else if (elmsz == 4) {
-                reinterpret_cast<int32_t*>(out)[w] = (int32_t)(count + j);
+                const uint64_t j = j0 + h;
+                dst[k] = (E)(idx2 ? (p2 + idx2[j]) : (size_t)((int64_t)p2 + (int64_t)j * s2));
             } else {
-                reinterpret_cast<int64_t*>(out)[w] = (int64_t)(count + j);
+                dst[k] = (E)(count + j0) + (E)h;
             }
         }
         off += total;
@@ -187,8 +224,16 @@ void where_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t 
     hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n, contiguous,
                        invert, nchunks, cpb, block_sums);
     hipLaunchKernelGGL(where_scan_kernel, dim3(1), dim3(kWhBlock), 0, st, block_sums, nblocks, running);
-    hipLaunchKernelGGL((where_scatter_kernel<MODE, false>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n,
-                       contiguous, invert, nchunks, cpb, out, elmsz, count, p2, (int64_t)s2, (const size_t*)idx2, (const uint64_t*)block_sums);
+#define WH_SCATTER(ES)                                                                                                                      \
+    hipLaunchKernelGGL((where_scatter_kernel<MODE, ES, false>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s,     \
+                       (const size_t*)idx, n, contiguous, invert, nchunks, cpb, out, count, p2, (int64_t)s2, (const size_t*)idx2,               \
+                       (const uint64_t*)block_sums)
+    if (elmsz == 4) {
+        if constexpr (MODE != 1) WH_SCATTER(4);
+    } else {
+        WH_SCATTER(8);
+    }
+#undef WH_SCATTER
     cumo_cuda_runtime_check_kernel_launch();
 }
 
@@ -291,14 +336,18 @@ void cumo_hip_bit_where_place_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t
     const WhGeometry g = wh_geometry(n);
     const int contiguous = s == 1 ? 1 : 0;
     hipStream_t st = current_stream();
-    if (x)
-        hipLaunchKernelGGL((where_scatter_kernel<2, true>), dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s,
-                           (const size_t*)nullptr, n, contiguous, invert, g.nchunks, g.cpb, out, elmsz, (uint64_t)0, (size_t)(uintptr_t)x, (int64_t)sx,
-                           (const size_t*)nullptr, counts);
-    else
-        hipLaunchKernelGGL((where_scatter_kernel<0, true>), dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s,
-                           (const size_t*)nullptr, n, contiguous, invert, g.nchunks, g.cpb, out, elmsz, (uint64_t)0, (size_t)0, (int64_t)0,
-                           (const size_t*)nullptr, counts);
+#define WH_PLACE(MODE, ES, P2, S2)                                                                                                     \
+    hipLaunchKernelGGL((where_scatter_kernel<MODE, ES, true>), dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, \
+                       (const size_t*)nullptr, n, contiguous, invert, g.nchunks, g.cpb, out, (uint64_t)0, (size_t)(P2), (int64_t)(S2),      \
+                       (const size_t*)nullptr, counts)
+    if (x) {
+        if (elmsz == 4) WH_PLACE(2, 4, (uintptr_t)x, sx);
+        else WH_PLACE(2, 8, (uintptr_t)x, sx);
+    } else {
+        if (elmsz == 4) WH_PLACE(0, 4, 0, 0);
+        else WH_PLACE(0, 8, 0, 0);
+    }
+#undef WH_PLACE
     cumo_cuda_runtime_check_kernel_launch();
 }
 
