@@ -32,6 +32,8 @@ CUMO_HIP_FBIN(OpFMod, fmod((double)x, (double)y))
 CUMO_HIP_FBIN(OpCopysign, copysign((double)x, (double)y))
 CUMO_HIP_FBIN(OpAtan2, atan2((double)x, (double)y))
 CUMO_HIP_FBIN(OpHypot, hypot((double)x, (double)y))
+// the second operand arrives in the float type and converts to int (types/float_macro_kernel.h:122)
+CUMO_HIP_FBIN(OpLdexp, ldexp((double)x, (int)y))
 
 // ---- binary, int32 (wrapping arithmetic done in unsigned) -------------------
 #define CUMO_HIP_IBIN(NAME, EXPR) \

@@ -1686,6 +1686,38 @@ int cumo_hip_na_math2_s(const char* op, const cumo_hip_narray_t* x, double sv, i
     return rc;
 }
 
+namespace {
+typedef void (*FrexpFn)(IA*, IA*, IA*, IX*);
+void iter_frexp(LP* lp) {
+    IA a1, a2, a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    cumo_hip_make_iarray(lp, 2, &a3);
+    ((FrexpFn)lp->opt_ptr)(&a1, &a2, &a3, &ix);
+}
+}  // namespace
+
+int cumo_hip_na_frexp(const cumo_hip_narray_t* x, cumo_hip_narray_t* mant, cumo_hip_narray_t* expo) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    if (!mant || !expo) return fail(CUMO_HIP_ERROR_ARGUMENT, "frexp: two result descriptors are needed");
+    const int type = is_float(x->type) ? x->type : CUMO_HIP_DFLOAT;
+    NA tx;
+    const NA* ux;
+    rc = cast_operand(x, type, &tx, &ux);
+    if (!rc) {
+        const FrexpFn f = type == CUMO_HIP_SFLOAT ? cumo_iter_sfloat_math_s_frexp_kernel_launch : cumo_iter_dfloat_math_s_frexp_kernel_launch;
+        cumo_hip_ndfunc_t nf = {iter_frexp, 0, 1, 2, {type, CUMO_HIP_INT32}};
+        const NA* in[1] = {ux};
+        NA* out[2] = {mant, expo};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, (void*)f);
+    }
+    free_tmp(&tx);
+    return rc;
+}
+
 int cumo_hip_na_compare(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {
     int rc = check_arith(x);
     if (!rc) rc = check_arith(y);

@@ -986,7 +986,7 @@ class _NMath:
 
     _ONE = ("sqrt cbrt log log2 log10 exp exp2 exp10 sin cos tan asin acos atan sinh cosh tanh "
             "asinh acosh atanh sinc erf erfc log1p expm1").split()
-    _TWO = ("atan2", "hypot")
+    _TWO = ("atan2", "hypot", "ldexp")
 
     def __getattr__(self, name):
         if name in self._ONE:
@@ -1000,6 +1000,12 @@ class _NMath:
         if not isinstance(x, _Numeric):
             raise TypeError("NMath needs a numeric array")
         return x
+
+    def frexp(self, x):
+        """[mantissa, exponent] with x = mantissa * 2**exponent; the exponent is Int32
+        (reference: gen/tmpl/frexp.c:32-38)."""
+        d, m, e = self._check(x)._desc(), NArrayDesc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_frexp, C.byref(d), C.byref(m), C.byref(e), results=(m, e))
 
     def _call1(self, name, x):
         d, z = self._check(x)._desc(), NArrayDesc()

@@ -155,7 +155,7 @@ size_t* cumo_cuda_runtime_error_item_new(void);
 
 /* NMath two-argument functions: narray/gen/tmpl/binary_s_kernel.cu:7-52, host
  * narray/gen/tmpl/binary_s.c:2-3 */
-#define CUMO_HIP_MATH2_OPS(X, t, c) X(t, c, atan2) X(t, c, hypot)
+#define CUMO_HIP_MATH2_OPS(X, t, c) X(t, c, atan2) X(t, c, hypot) X(t, c, ldexp)
 
 #define CUMO_HIP_DECL_MATH2(t, c, op) \
     void cumo_iter_##t##_math_s_##op##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer); \
@@ -207,6 +207,10 @@ CUMO_HIP_MATH_OPS(CUMO_HIP_DECL_MATH, sfloat, float)
 CUMO_HIP_MATH_OPS(CUMO_HIP_DECL_MATH, dfloat, double)
 CUMO_HIP_MATH2_OPS(CUMO_HIP_DECL_MATH2, sfloat, float)
 CUMO_HIP_MATH2_OPS(CUMO_HIP_DECL_MATH2, dfloat, double)
+/* NMath.frexp: a2 takes the mantissa, a3 the Int32 exponent
+ * (narray/gen/tmpl/frexp_kernel.cu:2-35, host narray/gen/tmpl/frexp.c:1) */
+void cumo_iter_sfloat_math_s_frexp_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
+void cumo_iter_dfloat_math_s_frexp_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
 
 CUMO_HIP_COND_OPS_ALL(CUMO_HIP_DECL_COND, sfloat, float)
 CUMO_HIP_COND_OPS_ALL(CUMO_HIP_DECL_COND, dfloat, double)

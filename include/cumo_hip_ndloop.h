@@ -180,6 +180,9 @@ int cumo_hip_na_clip(const cumo_hip_narray_t* x, int lo_kind, double lo_s, const
 int cumo_hip_na_math(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
 int cumo_hip_na_math2(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
 int cumo_hip_na_math2_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z);
+/* Cumo::NMath.frexp: x = mant * 2**expo, mant of x's float type (DFloat for an Int32 x), expo Int32
+ * (reference: gen/tmpl/frexp.c:32-38). */
+int cumo_hip_na_frexp(const cumo_hip_narray_t* x, cumo_hip_narray_t* mant, cumo_hip_narray_t* expo);
 /* Comparisons and float classification into a Bit result. */
 int cumo_hip_na_compare(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
 int cumo_hip_na_compare_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z);

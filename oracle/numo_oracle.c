@@ -116,6 +116,8 @@ static int T##_binary(const char *op, T x, T y, T *z)                          \
     if (!strcmp(op, "copysign")) { *z = (T)copysign(x, y); return 1; }         \
     if (!strcmp(op, "atan2")) { *z = (T)atan2(x, y); return 1; }               \
     if (!strcmp(op, "hypot")) { *z = (T)hypot(x, y); return 1; }               \
+    if (!strcmp(op, "ldexp")) { /* types/float_macro.h:117; the second    */   \
+        *z = (T)ldexp(x, (int)y); return 1; } /* operand converts to int  */   \
     if (!strcmp(op, "maximum")) { /* types/real_accum.h:444-453 */             \
         *z = (x >= y) ? x : ((y == y) ? y : x); return 1; }                    \
     if (!strcmp(op, "minimum")) { /* types/real_accum.h:466-475 */             \

@@ -121,6 +121,14 @@ def unary(op, x, out=None):
     return res
 
 
+def frexp(x):
+    """(mantissa, Int32 exponent) with x = mantissa * 2**exponent, the C library's frexp
+    element by element (types/float_macro.h:118, gen/tmpl/frexp.c:32-38); numpy calls the
+    same C function."""
+    m, e = np.frexp(x)
+    return m.astype(x.dtype), e.astype(np.int32)
+
+
 def pow_int(x, p):
     """Float array (or one float) ** Int32 array (or one integer): the repeated-product
     form of types/float_macro.h:125-144. Operands are broadcast; x fixes the type."""
