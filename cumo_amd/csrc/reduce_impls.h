@@ -253,16 +253,19 @@ struct KahanImpl {
 // (accum_arg_kernel.cu:15-37). NAN_WINS = true (nan: true): the first NaN wins
 // outright (accum_arg_kernel.cu:40-61). Equal values: lower index.
 // out_mode: 0 store the value (min/max), 4 / 8 store the index as int32 / int64.
-template <class T, bool IS_MAX, bool NAN_WINS>
+// IDX: the type the index is kept in while folding (int32_t halves a 4-byte type's accumulator and
+// the traffic between lanes; the launcher picks it when every index fits).
+template <class T, bool IS_MAX, bool NAN_WINS, class IDX = int64_t>
 struct ArgImpl {
     typedef T In;
-    struct Acc { T value; int64_t index; };
+    struct Acc { T value; IDX index; };
+    static constexpr IDX kNone = sizeof(IDX) == 8 ? (IDX)INT64_MAX : (IDX)INT32_MAX;  // no element seen yet
     static constexpr bool USES_INDEX = true;
     static constexpr int NOUT = 1;
     int out_mode;
     __device__ __forceinline__ Acc identity() const {
-        if (is_float_t<T>::value && !NAN_WINS) return Acc{Lim<T>::skip(), INT64_MAX};
-        return Acc{IS_MAX ? Lim<T>::lowest() : Lim<T>::highest(), INT64_MAX};
+        if (is_float_t<T>::value && !NAN_WINS) return Acc{Lim<T>::skip(), kNone};
+        return Acc{IS_MAX ? Lim<T>::lowest() : Lim<T>::highest(), kNone};
     }
     __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
         if (is_float_t<T>::value) {
@@ -279,7 +282,7 @@ struct ArgImpl {
         const bool better = IS_MAX ? (acc.value < next.value) : (acc.value > next.value);
         if (better || (acc.value == next.value && next.index < acc.index)) acc = next;
     }
-    __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{x, idx}, acc); }
+    __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{x, (IDX)idx}, acc); }
     // N later elements at once. The block's extreme costs one max/min per element;
     // only a block that beats the accumulator is looked at again, to find where its
     // extreme first occurs, and then merged with one combine. An equal value never
@@ -306,7 +309,7 @@ struct ArgImpl {
             }
         } else {
             bool look = IS_MAX ? (m > acc.value) : (m < acc.value);
-            look = look || acc.index == INT64_MAX;
+            look = look || acc.index == kNone;
             if (is_float_t<T>::value) {  // NAN_WINS
                 if (isnan_t(acc.value)) return;  // an earlier NaN already won
                 if (maybe_nan<T, N>(x)) {         // rare: let the exact rule sort it out
@@ -328,7 +331,7 @@ struct ArgImpl {
             first = hit ? k : first;
             v = hit ? x[k] : v;
         }
-        combine(Acc{v, idx0 + first}, acc);
+        combine(Acc{v, (IDX)(idx0 + first)}, acc);
     }
     // U blocks of N at once (all later than what the accumulator holds): when no
     // element of any of them can change the accumulator, one comparison says so.
@@ -344,7 +347,7 @@ struct ArgImpl {
             }
             // false for a NaN on either side, which sends the blocks down the exact path
             if (IS_MAX ? (m <= acc.value) : (m >= acc.value)) {
-                if (is_float_t<T>::value || acc.index != INT64_MAX) return;
+                if (is_float_t<T>::value || acc.index != kNone) return;
             }
         }
 #pragma unroll
@@ -353,7 +356,7 @@ struct ArgImpl {
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
         if (out_mode == 0) *reinterpret_cast<T*>(out) = acc.value;
         else if (out_mode == 4) *reinterpret_cast<int32_t*>(out) = (int32_t)acc.index;
-        else *reinterpret_cast<int64_t*>(out) = acc.index;
+        else *reinterpret_cast<int64_t*>(out) = (int64_t)acc.index;
     }
 };
 
