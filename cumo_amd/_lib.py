@@ -194,6 +194,9 @@ _sig = {
     "cumo_hip_na_store": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_copy": (C.c_int, [P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_fill": (C.c_int, [P(NArrayDesc), C.c_double]),
+    "cumo_hip_na_seq": (C.c_int, [P(NArrayDesc), C.c_double, C.c_double]),
+    "cumo_hip_na_logseq": (C.c_int, [P(NArrayDesc), C.c_double, C.c_double, C.c_double]),
+    "cumo_hip_na_eye": (C.c_int, [P(NArrayDesc), C.c_double, C.c_ssize_t]),
     "cumo_hip_na_to_host": (C.c_int, [P(NArrayDesc), C.c_void_p, C.c_size_t]),
     "cumo_hip_na_from_host": (C.c_int, [P(NArrayDesc), C.c_void_p, C.c_size_t]),
     "cumo_hip_na_extract": (C.c_int, [P(NArrayDesc), P(C.c_size_t), C.c_void_p]),

@@ -1904,6 +1904,97 @@ int cumo_hip_na_fill(cumo_hip_narray_t* dst, double value) {
     return cumo_hip_na_ndloop(&nf, in, NULL, 0, &opt);
 }
 
+namespace {
+struct SeqOpt {
+    double beg, step;
+};
+void iter_seq(LP* lp) {
+    IA a1;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    const SeqOpt* g = (const SeqOpt*)lp->opt_ptr;
+    switch (lp->args[0].type) {
+        case CUMO_HIP_SFLOAT: cumo_iter_sfloat_seq_kernel_launch(&a1, &ix, (float)g->beg, (float)g->step, 0.0); break;
+        case CUMO_HIP_DFLOAT: cumo_iter_dfloat_seq_kernel_launch(&a1, &ix, g->beg, g->step, 0.0); break;
+        default: cumo_iter_int32_seq_kernel_launch(&a1, &ix, g->beg, g->step, 0.0); break;
+    }
+}
+// one run at a time, the count carried from run to run (logseq.c walks the array the same way)
+struct LogseqWalk {
+    int type;
+    double beg, step, base, count;
+};
+void logseq_walk(const LP* lp, int level, char* p, LogseqWalk* w) {
+    const cumo_hip_loop_args_t& a = lp->args[0];
+    if (level == lp->ndim - 1) {
+        const uint64_t n = lp->n[level];
+        if (w->type == CUMO_HIP_SFLOAT)
+            cumo_iter_sfloat_logseq_stride_kernel_launch(p, a.step[level], (float)w->beg, (float)w->step, (float)w->base, w->count, n);
+        else
+            cumo_iter_dfloat_logseq_stride_kernel_launch(p, a.step[level], w->beg, w->step, w->base, w->count, n);
+        w->count += (double)n;
+        return;
+    }
+    for (size_t i = 0; i < lp->n[level]; i++) logseq_walk(lp, level + 1, p + (ssize_t)i * a.step[level], w);
+}
+}  // namespace
+
+int cumo_hip_na_seq(cumo_hip_narray_t* dst, double beg, double step) {
+    int rc = check_arith(dst);
+    if (rc) return rc;
+    SeqOpt opt = {beg, step};
+    cumo_hip_ndfunc_t nf = {iter_seq, 0, 1, 0, {0, 0}};
+    const NA* in[1] = {dst};
+    return cumo_hip_na_ndloop(&nf, in, NULL, 0, &opt);
+}
+
+int cumo_hip_na_logseq(cumo_hip_narray_t* dst, double beg, double step, double base) {
+    int rc = check_arith(dst);
+    if (rc) return rc;
+    if (!is_float(dst->type)) return no_method("logseq");
+    if (total_of(dst) == 0) return CUMO_HIP_OK;
+    cumo_hip_ndfunc_t nf = {NULL, 0, 1, 0, {0, 0}};
+    const NA* in[1] = {dst};
+    LP lp;
+    rc = cumo_hip_na_ndloop_prepare(&nf, in, NULL, 0, &lp);
+    if (rc) return rc;
+    LogseqWalk w = {dst->type, beg, step, base, 0.0};
+    logseq_walk(&lp, 0, lp.args[0].ptr, &w);
+    return CUMO_HIP_OK;
+}
+
+int cumo_hip_na_eye(cumo_hip_narray_t* dst, double element, ssize_t kofs) {
+    int rc = check_arith(dst);
+    if (rc) return rc;
+    const int nd = dst->ndim;
+    if (nd < 2) return fail(CUMO_HIP_ERROR_DIMENSION, "less than 2-d array");
+    if (kofs >= 0 ? (size_t)kofs >= dst->shape[nd - 1] : (size_t)(-kofs) >= dst->shape[nd - 2])
+        return fail(CUMO_HIP_ERROR_ARGUMENT, "invalid diagonal offset for the size of the matrix");
+    if (total_of(dst) == 0) return CUMO_HIP_OK;
+    // the leading dimensions walk on the host, a launch per matrix (eye.c is a user loop over the last two)
+    size_t idx[CUMO_NA_MAX_DIMENSION] = {0};
+    for (;;) {
+        ssize_t off = dst->offset;
+        for (int d = 0; d < nd - 2; ++d) off += (ssize_t)idx[d] * dst->stride[d];
+        char* p = dst->ptr + off;
+        const ssize_t s0 = dst->stride[nd - 2], s1 = dst->stride[nd - 1];
+        const uint64_t n0 = dst->shape[nd - 2], n1 = dst->shape[nd - 1];
+        switch (dst->type) {
+            case CUMO_HIP_SFLOAT: cumo_iter_sfloat_eye_stride_kernel_launch(p, s0, s1, kofs, (float)element, n0, n1); break;
+            case CUMO_HIP_DFLOAT: cumo_iter_dfloat_eye_stride_kernel_launch(p, s0, s1, kofs, element, n0, n1); break;
+            default: cumo_iter_int32_eye_stride_kernel_launch(p, s0, s1, kofs, (int32_t)element, n0, n1); break;
+        }
+        int d = nd - 3;
+        for (; d >= 0; --d) {
+            if (++idx[d] < dst->shape[d]) break;
+            idx[d] = 0;
+        }
+        if (d < 0) break;
+    }
+    return CUMO_HIP_OK;
+}
+
 int cumo_hip_na_reduce(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, int nan,
                        cumo_hip_narray_t* z, cumo_hip_narray_t* z2) {
     int rc = check_arith(x);

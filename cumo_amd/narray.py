@@ -519,6 +519,27 @@ class NArray:
         _run(_L.cumo_hip_na_fill, C.byref(d), float(value))
         return self
 
+    def seq(self, beg=0, step=1):
+        """self's elements in row-major order become beg + step * i (reference: gen/tmpl/seq.c:77-107)."""
+        d = self._desc()
+        _run(_L.cumo_hip_na_seq, C.byref(d), float(beg), float(step))
+        return self
+
+    indgen = seq
+
+    def logseq(self, beg, step, base=10):
+        """base ** (beg + step * i), float types only (reference: gen/tmpl/logseq.c)."""
+        d = self._desc()
+        _run(_L.cumo_hip_na_logseq, C.byref(d), float(beg), float(step), float(base))
+        return self
+
+    def eye(self, element=1, offset=0):
+        """`element` on the diagonal `offset` away from the main one of every matrix of the last
+        two dimensions, zero elsewhere (reference: gen/tmpl/eye.c:52-107)."""
+        d = self._desc()
+        _run(_L.cumo_hip_na_eye, C.byref(d), float(element), int(offset))
+        return self
+
     # ---- host read-back and ingest ------------------------------------------------
     def to_numpy(self):
         out = np.empty(self.shape, dtype=self.np_dtype)

@@ -225,6 +225,22 @@ CUMO_HIP_DECL_FILL(sfloat, float)
 CUMO_HIP_DECL_FILL(dfloat, double)
 CUMO_HIP_DECL_FILL(int32, int32_t)
 
+/* seq: element number i (row-major over the indexer) gets beg + step * (c + i); beg and step come in
+ * the element type, in double for Int32 (narray/gen/tmpl/seq_kernel.cu:14-52, host seq.c:1-21,63-68).
+ * logseq: base ** seq over one run, strided or through an index array, float types only
+ * (logseq_kernel.cu:2-32, host logseq.c). eye: data where row + kofs == column of an n0 x n1 matrix
+ * with byte steps s0, s1, zero elsewhere (eye_kernel.cu:2-18, host eye.c:2,42). */
+void cumo_iter_sfloat_seq_kernel_launch(cumo_na_iarray_t* a1, cumo_na_indexer_t* indexer, float beg, float step, double c);
+void cumo_iter_dfloat_seq_kernel_launch(cumo_na_iarray_t* a1, cumo_na_indexer_t* indexer, double beg, double step, double c);
+void cumo_iter_int32_seq_kernel_launch(cumo_na_iarray_t* a1, cumo_na_indexer_t* indexer, double beg, double step, double c);
+void cumo_iter_sfloat_logseq_stride_kernel_launch(char* p1, ssize_t s1, float beg, float step, float base, double c, uint64_t n);
+void cumo_iter_sfloat_logseq_index_kernel_launch(char* p1, size_t* idx1, float beg, float step, float base, double c, uint64_t n);
+void cumo_iter_dfloat_logseq_stride_kernel_launch(char* p1, ssize_t s1, double beg, double step, double base, double c, uint64_t n);
+void cumo_iter_dfloat_logseq_index_kernel_launch(char* p1, size_t* idx1, double beg, double step, double base, double c, uint64_t n);
+void cumo_iter_sfloat_eye_stride_kernel_launch(char* ptr, ssize_t s0, ssize_t s1, ssize_t kofs, float data, uint64_t n0, uint64_t n1);
+void cumo_iter_dfloat_eye_stride_kernel_launch(char* ptr, ssize_t s0, ssize_t s1, ssize_t kofs, double data, uint64_t n0, uint64_t n1);
+void cumo_iter_int32_eye_stride_kernel_launch(char* ptr, ssize_t s0, ssize_t s1, ssize_t kofs, int32_t data, uint64_t n0, uint64_t n1);
+
 /* pow: narray/gen/tmpl/pow_kernel.cu:6-36,58-113, host narray/gen/tmpl/pow.c:2-6.
  * A numeric exponent or base rides in as sv; an Int32 exponent takes the
  * repeated-product form (types/float_macro_kernel.h:125-149, int_macro_kernel.h:26-42). */

@@ -193,6 +193,14 @@ int cumo_hip_na_store(cumo_hip_narray_t* dst, const cumo_hip_narray_t* src);
 /* dst = contiguous copy of any view of the same type (reference: narray/data.c:84-113). */
 int cumo_hip_na_copy(const cumo_hip_narray_t* src, cumo_hip_narray_t* dst);
 int cumo_hip_na_fill(cumo_hip_narray_t* dst, double value);
+/* dst's elements in row-major order become beg + step * i (reference: gen/tmpl/seq.c:77-107), or
+ * base ** (beg + step * i) for logseq (float types; gen/tmpl/logseq.c). */
+int cumo_hip_na_seq(cumo_hip_narray_t* dst, double beg, double step);
+int cumo_hip_na_logseq(cumo_hip_narray_t* dst, double beg, double step, double base);
+/* Every matrix of the last two dimensions of dst gets `element` on the diagonal offset by kofs (above
+ * the main one for kofs > 0) and zero elsewhere (reference: gen/tmpl/eye.c:52-107: fewer than two
+ * dimensions is a dimension error, an offset beyond the matrix an argument error). */
+int cumo_hip_na_eye(cumo_hip_narray_t* dst, double element, ssize_t kofs);
 
 /* Reductions: sum prod min max ptp mean var stddev rms kahan_sum minmax argmin
  * argmax min_index max_index.

@@ -121,6 +121,39 @@ def unary(op, x, out=None):
     return res
 
 
+def seq(shape, dtype, beg=0, step=1):
+    """A new array whose row-major element i is beg + step * i: the float types take beg and
+    step in their own type, compute in double and round once; Int32 computes in double and
+    converts through a signed 64-bit integer (types/float_macro.h:145-148, xint_macro.h:153-156,
+    gen/tmpl/seq_kernel.cu:14-37)."""
+    dt = np.dtype(dtype)
+    n = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
+    i = np.arange(n, dtype=np.float64)
+    if dt.kind == "f":
+        v = (np.float64(dt.type(beg)) + np.float64(dt.type(step)) * i).astype(dt)
+    else:
+        v = (np.float64(beg) + np.float64(step) * i).astype(np.int64).astype(dt)
+    return v.reshape(shape)
+
+
+def logseq(shape, dtype, beg, step, base=10):
+    """base ** x with x the seq value rounded to the element type first; the power is the C
+    library's double pow, stored once (gen/tmpl/logseq_kernel.cu:5-15, types/float_macro.h:64)."""
+    dt = np.dtype(dtype)
+    x = seq(shape, dt, beg, step)
+    return np.power(np.float64(dt.type(base)), x.astype(np.float64)).astype(dt)
+
+
+def eye(shape, dtype, element=1, offset=0):
+    """`element` where row + offset == column in every matrix of the last two dimensions
+    (gen/tmpl/eye_kernel.cu:2-9)."""
+    out = np.zeros(shape, dtype=dtype)
+    r = np.arange(shape[-2])[:, None]
+    c = np.arange(shape[-1])[None, :]
+    out[..., (r + offset) == c] = np.dtype(dtype).type(element)
+    return out
+
+
 def frexp(x):
     """(mantissa, Int32 exponent) with x = mantissa * 2**exponent, the C library's frexp
     element by element (types/float_macro.h:118, gen/tmpl/frexp.c:32-38); numpy calls the

@@ -54,3 +54,7 @@ def close(expected, actual, rtol=1e-6):
     scale = max(1.0, max(abs(float(v)) for v in expected))
     worst = max(abs(float(e) - float(a)) for e, a in zip(expected, actual))
     return worst < rtol * scale
+
+# seq and logseq (narray_alt_coverage_test.rb:263-272): (arguments, expected)
+SEQ = [((), [0, 1, 2, 3, 4]), ((2,), [2, 3, 4, 5, 6]), ((5, 3), [5, 8, 11, 14, 17])]
+LOGSEQ = [(4, (0, 1), [1, 10, 100, 1000]), (5, (4, -1, 2), [16, 8, 4, 2, 1])]

@@ -83,3 +83,53 @@ def test_ldexp_and_frexp_bit_for_bit_with_the_oracle(cls, dt):
     # an Int32 argument is computed in DFloat
     mi, ei = cumo_amd.NMath.frexp(cumo_amd.Int32.cast(np.array([0, 1, 5, -12], dtype=np.int32)))
     assert isinstance(mi, cumo_amd.DFloat) and (mi.to_numpy() == [0.0, 0.5, 0.625, -0.75]).all() and (ei.to_numpy() == [0, 1, 3, 4]).all()
+
+
+@pytest.mark.parametrize("cls,dt", TYPES + [("Int32", np.int32)])
+def test_seq_logseq_and_eye(cls, dt):
+    """The reference's literal cases (narray_alt_coverage_test.rb:263-272), then the oracle on
+    strided views, many dimensions and the error cases of eye."""
+    import cumo_amd
+    T = getattr(cumo_amd, cls)
+    for args, want in kat_math.SEQ:
+        assert (T.new(5).seq(*args).to_numpy() == np.array(want, dtype=dt)).all()
+    rng = np.random.default_rng(3)
+    for shape in [(1,), (1000003,), (7, 11), (3, 1, 5, 4), (2, 3, 2, 2, 3)]:
+        beg, step = (float(rng.integers(-9, 9)), float(rng.integers(-4, 5))) if dt == np.int32 else (rng.standard_normal(), rng.standard_normal())
+        assert (T.new(*shape).seq(beg, step).to_numpy().view(np.uint8) == oracle.seq(shape, dt, beg, step).view(np.uint8)).all(), shape
+    # through a view: the element number runs over the view in row-major order, the rest stays
+    h = np.full((6, 8), 9, dtype=dt)
+    d = T.cast(h)
+    d[1::2, ::3].seq(1, 2)
+    h[1::2, ::3] = oracle.seq((3, 3), dt, 1, 2)
+    d.transpose()[:2].seq(100)
+    h.T[:2] = oracle.seq((2, 6), dt, 100)
+    assert (d.to_numpy() == h).all()
+    if dt == np.int32:
+        assert (T.new(4).seq(-1.5, 0.75).to_numpy() == [-1, 0, 0, 0]).all()
+        with pytest.raises(Exception):
+            T.new(3).logseq(0, 1)
+    else:
+        for n, args, want in kat_math.LOGSEQ:
+            assert (T.new(n).logseq(*args).to_numpy() == np.array(want, dtype=dt)).all()
+        got = T.new(4, 25).logseq(-3, 0.11, 2.5).to_numpy()
+        want = oracle.logseq((4, 25), dt, -3, 0.11, 2.5)
+        from helpers import assert_ulp
+        assert_ulp(got, want, 1 if dt == np.float32 else 2)
+        v = T.zeros(5, 12)
+        v[:, ::2].logseq(0, 1, 2)
+        assert_ulp(np.ascontiguousarray(v.to_numpy()[:, ::2]), oracle.logseq((5, 6), dt, 0, 1, 2), 0 if dt == np.float32 else 2)
+        assert (v.to_numpy()[:, 1::2] == 0).all()
+    for shape, el, k in [((3, 4), 1, 0), ((4, 4), 2.0, 1), ((2, 3, 5), 7, -2), ((2, 2, 3, 3), 1, 2)]:
+        assert (T.new(*shape).eye(el, k).to_numpy() == oracle.eye(shape, dt, el, k)).all()
+    e = T.cast(np.full((5, 7), 3, dtype=dt))
+    e[1:4, 2:6].eye()
+    want = np.full((5, 7), 3, dtype=dt)
+    want[1:4, 2:6] = np.eye(3, 4)
+    assert (e.to_numpy() == want).all()
+    with pytest.raises(Exception):
+        T.new(5).eye()
+    with pytest.raises(Exception):
+        T.new(3, 3).eye(1, 3)
+    with pytest.raises(Exception):
+        T.new(3, 3).eye(1, -3)

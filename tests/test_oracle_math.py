@@ -30,3 +30,22 @@ def test_two_argument_functions_ldexp_and_frexp(dt):
     m, e = oracle.frexp(np.array(a, dtype=dt))
     assert m.dtype == dt and e.dtype == np.int32
     assert (m == np.array(mant, dtype=dt)).all() and (e == np.array(expo)).all()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32])
+def test_seq_logseq_and_eye(dt):
+    for args, want in kat_math.SEQ:
+        assert (oracle.seq((5,), dt, *args) == np.array(want, dtype=dt)).all()
+    if dt != np.int32:
+        for n, args, want in kat_math.LOGSEQ:
+            assert (oracle.logseq((n,), dt, *args) == np.array(want, dtype=dt)).all()
+        # a step that is not a binary fraction: the float types round beg + step * i once from double
+        got = oracle.seq((7,), dt, 1, -0.2)
+        want = [dt(np.float64(dt(1)) + np.float64(dt(-0.2)) * i) for i in range(7)]
+        assert (got == np.array(want, dtype=dt)).all()
+    else:
+        # Int32 truncates toward zero through a 64-bit integer
+        assert (oracle.seq((4,), dt, -1.5, 0.75) == [-1, 0, 0, 0]).all()
+    assert (oracle.seq((2, 3), dt) == np.arange(6).reshape(2, 3)).all()
+    assert (oracle.eye((3, 4), dt) == np.eye(3, 4)).all()
+    assert (oracle.eye((2, 3, 3), dt, 5, -1) == 5 * np.eye(3, 3, -1)).all()
