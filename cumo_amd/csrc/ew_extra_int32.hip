@@ -4,6 +4,7 @@
 #include "ew_kernels.h"
 #include "ew_ops.h"
 #include "ew_clip3.h"
+#include "ew_ret2.h"
 
 using namespace cumo_hip;
 
@@ -49,6 +50,13 @@ extern "C" void cumo_int32_maximum_kernel_launch(cumo_na_iarray_t* a1, cumo_na_i
 extern "C" void cumo_int32_minimum_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3,
                                                  cumo_na_indexer_t* indexer) {
     ew_launch(OpMinimum<int32_t>{}, a1, a2, a3, nullptr, indexer, (int32_t)0, 0, nullptr);
+}
+
+// ---- divmod (reference: narray/gen/tmpl/binary2.c:2; a zero divisor raises the flag) ---------
+extern "C" void cumo_iter_int32_divmod_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3,
+                                                     cumo_na_iarray_t* a4, cumo_na_indexer_t* indexer, int* divzero) {
+    const cumo_na_iarray_t* arr[4] = {a1, a2, a3, a4};
+    ret2_launch(OpDivmodI{}, arr, indexer, divzero);
 }
 
 // ---- clip ---------------------------------------------------------------------------------

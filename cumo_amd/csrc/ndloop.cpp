@@ -1699,6 +1699,68 @@ void iter_frexp(LP* lp) {
 }
 }  // namespace
 
+namespace {
+struct DivmodOpt {
+    int type;
+    bool flagged;
+};
+void iter_divmod(LP* lp) {
+    IA a1, a2, a3, a4;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &a1);
+    cumo_hip_make_iarray(lp, 1, &a2);
+    cumo_hip_make_iarray(lp, 2, &a3);
+    cumo_hip_make_iarray(lp, 3, &a4);
+    DivmodOpt* o = (DivmodOpt*)lp->opt_ptr;
+    if (o->type == CUMO_HIP_INT32) {
+        int* flag = cumo_cuda_runtime_error_flag_new();
+        cumo_iter_int32_divmod_kernel_launch(&a1, &a2, &a3, &a4, &ix, flag);
+        if (flag && cumo_cuda_runtime_error_flag_get(flag)) o->flagged = true;
+    } else if (o->type == CUMO_HIP_SFLOAT) {
+        cumo_iter_sfloat_divmod_kernel_launch(&a1, &a2, &a3, &a4, &ix, NULL);
+    } else {
+        cumo_iter_dfloat_divmod_kernel_launch(&a1, &a2, &a3, &a4, &ix, NULL);
+    }
+}
+}  // namespace
+
+int cumo_hip_na_divmod(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* quot, cumo_hip_narray_t* rem) {
+    int rc = check_arith(x);
+    if (!rc) rc = check_arith(y);
+    if (rc) return rc;
+    if (!quot || !rem) return fail(CUMO_HIP_ERROR_ARGUMENT, "divmod: two result descriptors are needed");
+    const int up = upcast(x->type, y->type);
+    NA tx, ty;
+    const NA *ux, *uy;
+    rc = cast_operand(x, up, &tx, &ux);
+    if (!rc) rc = cast_operand(y, up, &ty, &uy);
+    else ty.ptr = NULL;
+    DivmodOpt opt = {up, false};
+    if (!rc) {
+        cumo_hip_ndfunc_t nf = {iter_divmod, 0, 2, 2, {up, up}};
+        const NA* in[2] = {ux, uy};
+        NA* out[2] = {quot, rem};
+        rc = cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    }
+    free_tmp(&tx);
+    free_tmp(&ty);
+    if (!rc && opt.flagged) return fail(CUMO_HIP_ERROR_ZERO_DIVISION, "error in NArray operation");
+    return rc;
+}
+
+int cumo_hip_na_modf(const cumo_hip_narray_t* x, cumo_hip_narray_t* frac, cumo_hip_narray_t* whole) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    if (!is_float(x->type)) return no_method("modf");
+    if (!frac || !whole) return fail(CUMO_HIP_ERROR_ARGUMENT, "modf: two result descriptors are needed");
+    const FrexpFn f = x->type == CUMO_HIP_SFLOAT ? cumo_iter_sfloat_modf_kernel_launch : cumo_iter_dfloat_modf_kernel_launch;
+    cumo_hip_ndfunc_t nf = {iter_frexp, 0, 1, 2, {x->type, x->type}};
+    const NA* in[1] = {x};
+    NA* out[2] = {frac, whole};
+    return cumo_hip_na_ndloop(&nf, in, out, 0, (void*)f);
+}
+
 int cumo_hip_na_frexp(const cumo_hip_narray_t* x, cumo_hip_narray_t* mant, cumo_hip_narray_t* expo) {
     int rc = check_arith(x);
     if (rc) return rc;

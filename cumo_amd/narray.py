@@ -660,6 +660,19 @@ class _Numeric(NArray):
         x, y = a._desc(), b._desc()
         return _run(_L.cumo_hip_na_binary, op.encode(), C.byref(x), C.byref(y), C.byref(z), results=(z,))
 
+    def divmod(self, other):
+        """[quotient, remainder] (reference: gen/tmpl/binary2.c; a number is cast to an array
+        first, the template has no scalar form). Int32 by zero raises ZeroDivisionError."""
+        if isinstance(other, numbers.Number):
+            x = self._scalar_operand(other)
+            other = type(x).cast(np.array([other], dtype=x.np_dtype))
+        else:
+            x = self
+        if not isinstance(other, _Numeric):
+            raise TypeError("divmod needs a numeric operand")
+        dx, dy, q, r = x._desc(), other._desc(), NArrayDesc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_divmod, C.byref(dx), C.byref(dy), C.byref(q), C.byref(r), results=(q, r))
+
     def __add__(self, o): return self._binary(o, "add")
     def __radd__(self, o): return self._binary(o, "add", True)
     def __sub__(self, o): return self._binary(o, "sub")
@@ -823,6 +836,11 @@ class _Float(_Numeric):
     def var(self, axis=None, keepdims=False, nan=False): return self._reduce("var", axis, keepdims, nan)
     def stddev(self, axis=None, keepdims=False, nan=False): return self._reduce("stddev", axis, keepdims, nan)
     def rms(self, axis=None, keepdims=False, nan=False): return self._reduce("rms", axis, keepdims, nan)
+
+    def modf(self):
+        """[fraction, integral part], each with the sign of the element (reference: gen/tmpl/unary_ret2.c)."""
+        d, f, w = self._desc(), NArrayDesc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_modf, C.byref(d), C.byref(f), C.byref(w), results=(f, w))
 
     def floor(self): return self._unary("floor")
     def round(self): return self._unary("round")

@@ -225,6 +225,16 @@ CUMO_HIP_DECL_FILL(sfloat, float)
 CUMO_HIP_DECL_FILL(dfloat, double)
 CUMO_HIP_DECL_FILL(int32, int32_t)
 
+/* divmod: a3 = a1 / a2, a4 = a1 mod a2 (fmod for the float types, C remainder for Int32, where a
+ * zero divisor leaves the element unwritten and sets *divzero): narray/gen/tmpl/binary2_kernel.cu:3-42,
+ * host binary2.c:2. modf: a2 the fraction, a3 the integral part, both with the argument's sign:
+ * narray/gen/tmpl/unary_ret2_kernel.cu:2-35, types/float_macro_kernel.h:51. */
+void cumo_iter_sfloat_divmod_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_iarray_t* a4, cumo_na_indexer_t* indexer, int* divzero);
+void cumo_iter_dfloat_divmod_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_iarray_t* a4, cumo_na_indexer_t* indexer, int* divzero);
+void cumo_iter_int32_divmod_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_iarray_t* a4, cumo_na_indexer_t* indexer, int* divzero);
+void cumo_iter_sfloat_modf_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
+void cumo_iter_dfloat_modf_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
+
 /* seq: element number i (row-major over the indexer) gets beg + step * (c + i); beg and step come in
  * the element type, in double for Int32 (narray/gen/tmpl/seq_kernel.cu:14-52, host seq.c:1-21,63-68).
  * logseq: base ** seq over one run, strided or through an index array, float types only

@@ -180,6 +180,11 @@ int cumo_hip_na_clip(const cumo_hip_narray_t* x, int lo_kind, double lo_s, const
 int cumo_hip_na_math(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
 int cumo_hip_na_math2(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
 int cumo_hip_na_math2_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z);
+/* x.divmod(y) -> quotient and remainder with the upcast type of the two (reference: gen/tmpl/binary2.c;
+ * Int32 by zero reports CUMO_HIP_ERROR_ZERO_DIVISION after the launch). x.modf -> fraction and integral
+ * part, float types only (reference: gen/tmpl/unary_ret2.c). */
+int cumo_hip_na_divmod(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* quot, cumo_hip_narray_t* rem);
+int cumo_hip_na_modf(const cumo_hip_narray_t* x, cumo_hip_narray_t* frac, cumo_hip_narray_t* whole);
 /* Cumo::NMath.frexp: x = mant * 2**expo, mant of x's float type (DFloat for an Int32 x), expo Int32
  * (reference: gen/tmpl/frexp.c:32-38). */
 int cumo_hip_na_frexp(const cumo_hip_narray_t* x, cumo_hip_narray_t* mant, cumo_hip_narray_t* expo);

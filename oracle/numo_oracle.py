@@ -154,6 +154,18 @@ def eye(shape, dtype, element=1, offset=0):
     return out
 
 
+def modf(x):
+    """(fraction, integral part), the C library's modf element by element on the promoted
+    argument, each result stored once (types/float_macro.h:48, gen/tmpl/unary_ret2.c)."""
+    f, w = np.modf(x.astype(np.float64))
+    return f.astype(x.dtype), w.astype(x.dtype)
+
+
+def divmod_(x, y):
+    """(x / y, x mod y) by the two operators (types/float_macro.h:32, xint_macro.h:20)."""
+    return binary("div", x, y), binary("mod", x, y)
+
+
 def frexp(x):
     """(mantissa, Int32 exponent) with x = mantissa * 2**exponent, the C library's frexp
     element by element (types/float_macro.h:118, gen/tmpl/frexp.c:32-38); numpy calls the

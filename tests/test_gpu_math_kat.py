@@ -133,3 +133,48 @@ def test_seq_logseq_and_eye(cls, dt):
         T.new(3, 3).eye(1, 3)
     with pytest.raises(Exception):
         T.new(3, 3).eye(1, -3)
+
+
+def test_divmod_and_modf_reference_cases():
+    """narray_test.rb:1413-1420, 2248-2252, 2472-2511 (modf keeps the argument's sign in both parts,
+    zero included; NaN gives NaN twice; an infinity gives a signed zero and itself) and
+    narray_alt_coverage_test.rb:719,741 (Int32 divmod, and by zero)."""
+    import cumo_amd
+    q, r = cumo_amd.Int32.cast(np.array([17, 20, 23], np.int32)).divmod(cumo_amd.Int32.cast(np.array([5, 6, 7], np.int32)))
+    assert (q.to_numpy() == [3, 3, 3]).all() and (r.to_numpy() == [2, 2, 2]).all()
+    q, r = cumo_amd.Int32.cast(np.array([10, 20, 30], np.int32)).divmod(cumo_amd.Int32.cast(np.array([3, 4, 5], np.int32)))
+    assert (q.to_numpy() == [3, 5, 6]).all() and (r.to_numpy() == [1, 0, 0]).all()
+    with pytest.raises(ZeroDivisionError):
+        cumo_amd.Int32.cast(np.array([1, 2, 3], np.int32)).divmod(cumo_amd.Int32.cast(np.array([1, 0, 3], np.int32)))
+    with pytest.raises(ZeroDivisionError):
+        cumo_amd.Int32.cast(np.arange(12, dtype=np.int32).reshape(3, 4))[:, 1:-1].divmod(0)
+    f, w = (cumo_amd.DFloat.new(8).seq(1) / 4).modf()
+    assert (f.to_numpy()[:2] == [0.25, 0.5]).all() and (w.to_numpy()[:2] == [0.0, 0.0]).all()
+    inf = np.inf
+    specials = {0: np.nan, 1: inf, 2: -inf, 3: -0.0}
+    values = np.array([specials.get(i % 9, (i - 100) / 8.0) for i in range(200)])
+    for cls, dt in TYPES:
+        T = getattr(cumo_amd, cls)
+        stored = values.astype(dt)
+        a = T.cast(stored)
+        for view, src in ((a, stored), (a[::3], stored[::3]), (a[::-1], stored[::-1])):
+            f, w = view.modf()
+            wf, ww = oracle.modf(np.ascontiguousarray(src))
+            assert isinstance(f, T) and isinstance(w, T)
+            assert (f.to_numpy().view(np.uint8) == wf.view(np.uint8))[~np.isnan(wf).repeat(wf.itemsize)].all()
+            assert (np.isnan(f.to_numpy()) == np.isnan(wf)).all() and (np.isnan(w.to_numpy()) == np.isnan(ww)).all()
+            assert (w.to_numpy().view(np.uint8) == ww.view(np.uint8))[~np.isnan(ww).repeat(ww.itemsize)].all()
+            m, e = cumo_amd.NMath.frexp(view)
+            wm, we = oracle.frexp(np.ascontiguousarray(src))
+            fin = np.isfinite(src)
+            assert (m.to_numpy()[fin].view(np.uint8) == wm[fin].view(np.uint8)).all() and (e.to_numpy()[fin] == we[fin]).all()
+        # float divmod: the quotient is the plain division, the remainder fmod; broadcast and a number
+        rng = np.random.default_rng(5)
+        x = rng.standard_normal((6, 40)).astype(dt) * 50
+        y = (rng.standard_normal(40).astype(dt) * 7)
+        q, r = T.cast(x).divmod(T.cast(y))
+        wq, wr = oracle.divmod_(x, np.broadcast_to(y, x.shape).copy())
+        assert (q.to_numpy() == wq).all() and (r.to_numpy() == wr).all()
+        q, r = T.cast(x)[::2, 1::2].divmod(4.0)
+        wq, wr = oracle.divmod_(np.ascontiguousarray(x[::2, 1::2]), np.full((3, 20), 4.0, dtype=dt))
+        assert (q.to_numpy() == wq).all() and (r.to_numpy() == wr).all()

@@ -49,3 +49,17 @@ def test_seq_logseq_and_eye(dt):
     assert (oracle.seq((2, 3), dt) == np.arange(6).reshape(2, 3)).all()
     assert (oracle.eye((3, 4), dt) == np.eye(3, 4)).all()
     assert (oracle.eye((2, 3, 3), dt, 5, -1) == 5 * np.eye(3, 3, -1)).all()
+
+
+def test_modf_keeps_the_sign_in_both_parts():
+    """narray_test.rb:2472-2484 (modf_expect) restated case by case."""
+    x = np.array([2.75, -2.75, 0.0, -0.0, np.inf, -np.inf, 3.0, -3.0, 0.25])
+    f, w = oracle.modf(x)
+    assert (f == [0.75, -0.75, 0.0, -0.0, 0.0, -0.0, 0.0, -0.0, 0.25]).all()
+    assert (np.signbit(f) == [False, True, False, True, False, True, False, True, False]).all()
+    assert (w == [2.0, -2.0, 0.0, -0.0, np.inf, -np.inf, 3.0, -3.0, 0.0]).all()
+    assert (np.signbit(w) == [False, True, False, True, False, True, False, True, False]).all()
+    fn, wn = oracle.modf(np.array([np.nan], dtype=np.float32))
+    assert np.isnan(fn[0]) and np.isnan(wn[0]) and fn.dtype == np.float32
+    q, r = oracle.divmod_(np.array([17, 20, 23, -7], np.int32), np.array([5, 6, 7, 3], np.int32))
+    assert (q == [3, 3, 3, -2]).all() and (r == [2, 2, 2, -1]).all()   # C truncation, as xint_macro.h:19-20
