@@ -178,3 +178,23 @@ def test_divmod_and_modf_reference_cases():
         q, r = T.cast(x)[::2, 1::2].divmod(4.0)
         wq, wr = oracle.divmod_(np.ascontiguousarray(x[::2, 1::2]), np.full((3, 20), 4.0, dtype=dt))
         assert (q.to_numpy() == wq).all() and (r.to_numpy() == wr).all()
+
+
+def test_empty_and_single_element_arrays():
+    """total_size == 0 is a no-op without a launch (template_kernel.h:76-81); one element works."""
+    import cumo_amd
+    for cls, dt in TYPES + [("Int32", np.int32)]:
+        T = getattr(cumo_amd, cls)
+        e = T.new(0)
+        assert e.seq().shape == (0,) and T.new(0, 3).eye().shape == (0, 3)
+        q, r = e.divmod(T.new(0))
+        assert q.shape == (0,) and r.shape == (0,)
+        assert (T.new(1).seq(7).to_numpy() == [7]).all()
+        q, r = T.cast(np.array([7], dtype=dt)).divmod(2)
+        assert q.to_numpy()[0] == (3 if dt == np.int32 else 3.5) and r.to_numpy()[0] == 1
+        if dt != np.int32:
+            f, w = e.modf()
+            m, x = cumo_amd.NMath.frexp(e)
+            assert f.shape == w.shape == m.shape == x.shape == (0,)
+            assert e.logseq(0, 1).shape == (0,)
+            assert cumo_amd.NMath.ldexp(e, cumo_amd.Int32.new(0)).shape == (0,)
