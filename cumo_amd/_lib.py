@@ -188,6 +188,7 @@ _sig = {
     "cumo_hip_na_math2": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_math2_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
     "cumo_hip_na_frexp": (C.c_int, [P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
+    "cumo_hip_na_poly": (C.c_int, [P(NArrayDesc), C.c_int, C.POINTER(P(NArrayDesc)), P(NArrayDesc)]),
     "cumo_hip_na_modf": (C.c_int, [P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_divmod": (C.c_int, [P(NArrayDesc), P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_compare": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),

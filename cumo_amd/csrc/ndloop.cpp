@@ -1761,6 +1761,92 @@ int cumo_hip_na_modf(const cumo_hip_narray_t* x, cumo_hip_narray_t* frac, cumo_h
     return cumo_hip_na_ndloop(&nf, in, out, 0, (void*)f);
 }
 
+namespace {
+constexpr int kPolyMaxScalars = 64;
+struct PolyOpt {
+    int ncoef;
+    const NA* const* coef;
+};
+void iter_poly(LP* lp) {
+    IA ax, az, ac[kPolyMaxScalars];
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_iarray(lp, 0, &ax);
+    cumo_hip_make_iarray(lp, 1, &az);
+    const PolyOpt* o = (const PolyOpt*)lp->opt_ptr;
+    for (int k = 0; k < o->ncoef; ++k) {
+        std::memset(&ac[k], 0, sizeof(IA));  // every step 0: the one element repeats
+        ac[k].ptr = o->coef[k]->ptr + o->coef[k]->offset;
+    }
+    switch (lp->args[0].type) {
+        case CUMO_HIP_SFLOAT: cumo_iter_sfloat_poly_kernel_launch(&ax, ac, o->ncoef, &az, &ix); break;
+        case CUMO_HIP_DFLOAT: cumo_iter_dfloat_poly_kernel_launch(&ax, ac, o->ncoef, &az, &ix); break;
+        default: cumo_iter_int32_poly_kernel_launch(&ax, ac, o->ncoef, &az, &ix); break;
+    }
+}
+}  // namespace
+
+int cumo_hip_na_poly(const cumo_hip_narray_t* x, int ncoef, const cumo_hip_narray_t* const* coef, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    if (!z || ncoef < 0 || (ncoef > 0 && !coef)) return fail(CUMO_HIP_ERROR_ARGUMENT, "poly: bad arguments");
+    bool scalars = ncoef <= kPolyMaxScalars;
+    for (int k = 0; k < ncoef; ++k) {
+        rc = check_arith(coef[k]);
+        if (rc) return rc;
+        if (coef[k]->type != x->type) return fail(CUMO_HIP_ERROR_TYPE, "poly: coefficients must have the array's type");
+        if (total_of(coef[k]) != 1) scalars = false;
+    }
+    if (scalars) {
+        PolyOpt opt = {ncoef, coef};
+        cumo_hip_ndfunc_t nf = {iter_poly, 0, 1, 1, {x->type, 0}};
+        const NA* in[1] = {x};
+        NA* out[1] = {z};
+        return cumo_hip_na_ndloop(&nf, in, out, 0, &opt);
+    }
+    if (ncoef == 1) {
+        // the constant term alone, spread over the shape x and it make together
+        const NA* a0 = coef[0];
+        if (!z->ptr) {
+            const int nd = x->ndim > a0->ndim ? x->ndim : a0->ndim;
+            size_t shape[CUMO_NA_MAX_DIMENSION];
+            for (int d = 0; d < nd; ++d) {
+                const int dx = d - (nd - x->ndim), da = d - (nd - a0->ndim);
+                const size_t nx = dx >= 0 ? x->shape[dx] : 1, na = da >= 0 ? a0->shape[da] : 1;
+                if (nx != na && nx != 1 && na != 1) return fail(CUMO_HIP_ERROR_SHAPE, "shape mismatch");
+                shape[d] = nx == 1 ? na : nx;
+            }
+            rc = cumo_hip_na_alloc(z, x->type, nd, shape);
+            if (rc) return rc;
+            rc = cumo_hip_na_store(z, a0);
+            if (rc) free_tmp(z);
+            return rc;
+        }
+        return cumo_hip_na_store(z, a0);
+    }
+    // Horner as array operations: y = a_n; y = x * y + a_k for k = n-1 .. 0
+    NA y, t;
+    y.ptr = t.ptr = NULL;
+    rc = cumo_hip_na_binary("mul", x, coef[ncoef - 1], &y);
+    for (int k = ncoef - 2; k >= 0 && !rc; --k) {
+        const bool last = k == 0;
+        if (k != ncoef - 2) {
+            t.ptr = NULL;
+            rc = cumo_hip_na_binary("mul", x, &y, &t);
+            free_tmp(&y);
+            y = t;
+            if (rc) break;
+        }
+        t.ptr = NULL;
+        rc = cumo_hip_na_binary("add", &y, coef[k], last ? z : &t);
+        free_tmp(&y);
+        if (!last) y = t;
+        else y.ptr = NULL;
+    }
+    if (rc) free_tmp(&y);
+    return rc;
+}
+
 int cumo_hip_na_frexp(const cumo_hip_narray_t* x, cumo_hip_narray_t* mant, cumo_hip_narray_t* expo) {
     int rc = check_arith(x);
     if (rc) return rc;

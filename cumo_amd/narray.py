@@ -673,6 +673,17 @@ class _Numeric(NArray):
         dx, dy, q, r = x._desc(), other._desc(), NArrayDesc(), NArrayDesc()
         return _run(_L.cumo_hip_na_divmod, C.byref(dx), C.byref(dy), C.byref(q), C.byref(r), results=(q, r))
 
+    def poly(self, *coef):
+        """a0 + a1 x + ... + an x**n by Horner's rule in the array's type (reference: gen/tmpl/poly.c:38-78);
+        numbers and arrays are cast to the array's type first."""
+        cls = type(self)
+        arrs = [c if isinstance(c, cls) else (cls.cast(c) if isinstance(c, NArray) else cls.cast(np.array([c], dtype=self.np_dtype)))
+                for c in coef]
+        descs = [a._desc() for a in arrs]
+        ptrs = (C.POINTER(NArrayDesc) * max(1, len(descs)))(*[C.pointer(d) for d in descs])
+        d, z = self._desc(), NArrayDesc()
+        return _run(_L.cumo_hip_na_poly, C.byref(d), len(descs), ptrs, C.byref(z), results=(z,))
+
     def __add__(self, o): return self._binary(o, "add")
     def __radd__(self, o): return self._binary(o, "add", True)
     def __sub__(self, o): return self._binary(o, "sub")

@@ -235,6 +235,13 @@ void cumo_iter_int32_divmod_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t
 void cumo_iter_sfloat_modf_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
 void cumo_iter_dfloat_modf_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer);
 
+/* poly: z = coef[0] + coef[1] x + ... + coef[ncoef-1] x^(ncoef-1) by Horner's rule in the element
+ * type, every coefficient an array descriptor over the same indexer (zero steps for a number);
+ * ncoef == 0 answers x (narray/gen/tmpl/poly_kernel.cu:3-45, host poly.c:2,18). */
+void cumo_iter_sfloat_poly_kernel_launch(cumo_na_iarray_t* x, cumo_na_iarray_t* coef, int ncoef, cumo_na_iarray_t* z, cumo_na_indexer_t* indexer);
+void cumo_iter_dfloat_poly_kernel_launch(cumo_na_iarray_t* x, cumo_na_iarray_t* coef, int ncoef, cumo_na_iarray_t* z, cumo_na_indexer_t* indexer);
+void cumo_iter_int32_poly_kernel_launch(cumo_na_iarray_t* x, cumo_na_iarray_t* coef, int ncoef, cumo_na_iarray_t* z, cumo_na_indexer_t* indexer);
+
 /* seq: element number i (row-major over the indexer) gets beg + step * (c + i); beg and step come in
  * the element type, in double for Int32 (narray/gen/tmpl/seq_kernel.cu:14-52, host seq.c:1-21,63-68).
  * logseq: base ** seq over one run, strided or through an index array, float types only

@@ -185,6 +185,10 @@ int cumo_hip_na_math2_s(const char* op, const cumo_hip_narray_t* x, double sv, i
  * part, float types only (reference: gen/tmpl/unary_ret2.c). */
 int cumo_hip_na_divmod(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* quot, cumo_hip_narray_t* rem);
 int cumo_hip_na_modf(const cumo_hip_narray_t* x, cumo_hip_narray_t* frac, cumo_hip_narray_t* whole);
+/* x.poly(a0, ..., an): the ncoef coefficients are arrays of x's type; one element each (numbers) goes
+ * out as one launch, anything else as the chain y = x * y + a_k of array operations with broadcasting,
+ * which rounds the same way (reference: gen/tmpl/poly.c:38-78). No coefficient answers a copy of x. */
+int cumo_hip_na_poly(const cumo_hip_narray_t* x, int ncoef, const cumo_hip_narray_t* const* coef, cumo_hip_narray_t* z);
 /* Cumo::NMath.frexp: x = mant * 2**expo, mant of x's float type (DFloat for an Int32 x), expo Int32
  * (reference: gen/tmpl/frexp.c:32-38). */
 int cumo_hip_na_frexp(const cumo_hip_narray_t* x, cumo_hip_narray_t* mant, cumo_hip_narray_t* expo);

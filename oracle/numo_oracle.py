@@ -166,6 +166,24 @@ def divmod_(x, y):
     return binary("div", x, y), binary("mod", x, y)
 
 
+def poly(x, *coef):
+    """Horner's rule with the element type's own multiplication and addition, each rounded
+    separately; Int32 wraps (gen/tmpl/poly_kernel.cu:9-17). Coefficients are cast to x's type
+    and broadcast; none answers x."""
+    dt = x.dtype
+    cs = [np.asarray(c).astype(dt) for c in coef]
+    if not cs:
+        return x.copy()
+    shape = np.broadcast_shapes(x.shape, *[c.shape for c in cs])
+    xb = np.broadcast_to(x, shape)
+    y = np.broadcast_to(cs[-1], shape).copy()
+    with np.errstate(all="ignore"):
+        for c in reversed(cs[:-1]):
+            y = (xb * y).astype(dt)
+            y = (y + np.broadcast_to(c, shape)).astype(dt)
+    return y
+
+
 def frexp(x):
     """(mantissa, Int32 exponent) with x = mantissa * 2**exponent, the C library's frexp
     element by element (types/float_macro.h:118, gen/tmpl/frexp.c:32-38); numpy calls the

@@ -198,3 +198,38 @@ def test_empty_and_single_element_arrays():
             assert f.shape == w.shape == m.shape == x.shape == (0,)
             assert e.logseq(0, 1).shape == (0,)
             assert cumo_amd.NMath.ldexp(e, cumo_amd.Int32.new(0)).shape == (0,)
+
+
+@pytest.mark.parametrize("cls,dt", TYPES + [("Int32", np.int32)])
+def test_poly(cls, dt):
+    """The reference's cases (narray_test.rb:1944-1963), then the oracle bit for bit: number
+    coefficients (one launch, more than six coefficients continue from the result), array
+    coefficients with broadcasting (the chain of array operations), views, the constant alone."""
+    import cumo_amd
+    T = getattr(cumo_amd, cls)
+    x = T.new(4).seq(1)
+    assert (x.poly(1, 2).to_numpy() == [3, 5, 7, 9]).all()
+    assert (x.poly(1, 2, 3).to_numpy() == [6, 17, 34, 57]).all()
+    assert (x.poly(3).to_numpy() == [3, 3, 3, 3]).all() and (x.poly().to_numpy() == [1, 2, 3, 4]).all()
+    assert (T.cast(np.array([2], dtype=dt)).poly(1, 2).to_numpy() == [5]).all()
+    assert (x.poly(T.cast(np.ones(4, dtype=dt)), T.cast(np.full(4, 2, dtype=dt))).to_numpy() == [3, 5, 7, 9]).all()
+    rng = np.random.default_rng(11)
+    if dt == np.int32:
+        h = rng.integers(-50000, 50000, size=(37, 53)).astype(dt)
+        coefs = [int(c) for c in rng.integers(-9, 9, size=15)]
+    else:
+        h = rng.standard_normal((37, 53)).astype(dt)
+        coefs = [float(c) for c in rng.standard_normal(15)]
+    d = T.cast(h)
+    for n in (1, 2, 6, 7, 12, 13, 15):
+        got = d.poly(*coefs[:n]).to_numpy()
+        assert (got.view(np.uint8) == oracle.poly(h, *coefs[:n]).view(np.uint8)).all(), n
+    got = d.transpose()[1::2, ::3].poly(*coefs[:8]).to_numpy()
+    assert (got == oracle.poly(np.ascontiguousarray(h.T[1::2, ::3]), *coefs[:8])).all()
+    row = (rng.integers(-5, 5, size=53) if dt == np.int32 else rng.standard_normal(53)).astype(dt)
+    col = (rng.integers(-5, 5, size=(37, 1)) if dt == np.int32 else rng.standard_normal((37, 1))).astype(dt)
+    for cs in ((row,), (row, col), (coefs[0], row, col, coefs[1]), (col, coefs[2], row)):
+        got = d.poly(*[T.cast(c) if isinstance(c, np.ndarray) else c for c in cs]).to_numpy()
+        assert (got.view(np.uint8) == oracle.poly(h, *cs).view(np.uint8)).all()
+    small = T.cast(h[:1])                      # [1, 53] against a column: the constant alone spreads over both
+    assert (small.poly(T.cast(col)).to_numpy() == np.broadcast_to(col, (37, 53))).all()

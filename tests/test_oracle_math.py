@@ -63,3 +63,19 @@ def test_modf_keeps_the_sign_in_both_parts():
     assert np.isnan(fn[0]) and np.isnan(wn[0]) and fn.dtype == np.float32
     q, r = oracle.divmod_(np.array([17, 20, 23, -7], np.int32), np.array([5, 6, 7, 3], np.int32))
     assert (q == [3, 3, 3, -2]).all() and (r == [2, 2, 2, -1]).all()   # C truncation, as xint_macro.h:19-20
+
+
+def test_poly_reference_cases():
+    """narray_test.rb:1944-1963."""
+    x = np.arange(1, 5, dtype=np.float64)
+    assert (oracle.poly(x, 1.0, 2.0) == [3, 5, 7, 9]).all()
+    assert (oracle.poly(x, 1.0, 2.0, 3.0) == [6, 17, 34, 57]).all()
+    assert (oracle.poly(x, 3.0) == [3, 3, 3, 3]).all() and (oracle.poly(x) == x).all()
+    assert (oracle.poly(np.array([2.0]), 1.0, 2.0) == [5.0]).all()
+    assert (oracle.poly(x, np.ones(4), np.full(4, 2.0)) == [3, 5, 7, 9]).all()
+    assert (oracle.poly(x.astype(np.float32), 1.0, 2.0) == [3, 5, 7, 9]).all()
+    assert (oracle.poly(np.arange(1, 5, dtype=np.int32), 1, 2) == [3, 5, 7, 9]).all()
+    # against exact integer arithmetic, wrapping for Int32
+    xi = np.array([3, -7, 100000, 46341], dtype=np.int32)
+    want = [(5 + 4 * int(v) + 3 * int(v) ** 2 + 2 * int(v) ** 3 + 2 ** 31) % 2 ** 32 - 2 ** 31 for v in xi]
+    assert (oracle.poly(xi, 5, 4, 3, 2) == want).all()
