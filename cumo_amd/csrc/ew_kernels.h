@@ -562,10 +562,15 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_kernel(const char* __res
 // vector, or the scalar), and may repeat along rows (a row vector). 32-bit
 // index arithmetic, one 128-bit access per lane, no ragged vectors: the launcher
 // only picks it when inner is a whole number of vectors.
+// Three dimensions (outer x mid x inner, an operand repeating along outer or mid:
+// [B,T,C] with [T,1] or [B,1,C]) use the same tiles over outer * mid rows; a row
+// number then splits once per lane and tile into its two parts.
 // ---------------------------------------------------------------------------
 struct EwR2Params {
     char* ptr[3];        // in1, in2, out
     int64_t rstep[3];    // byte step from one row to the next (0: the operand repeats)
+    int64_t ostep[3];    // three dimensions: byte step along outer (rstep is then the step along mid)
+    uint32_t mid;        // three dimensions: extent of mid; 0 for two dimensions
     int walk[3];         // 1: contiguous along inner, 0: constant along inner
     uint32_t rows;
     uint32_t inner_vecs; // inner / VEC
@@ -597,11 +602,21 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
         const uint32_t row = rt * TY + ty;
         const uint32_t cv = ct * TX + tx;
         if (row >= p.rows || cv >= p.inner_vecs) continue;
+        int64_t roff[3];
+        if (p.mid == 0) {
+#pragma unroll
+            for (int k = 0; k < 3; ++k) roff[k] = (int64_t)row * p.rstep[k];
+        } else {
+            const uint32_t r0 = row / p.mid;
+            const uint32_t r1 = row - r0 * p.mid;
+#pragma unroll
+            for (int k = 0; k < 3; ++k) roff[k] = (int64_t)r0 * p.ostep[k] + (int64_t)r1 * p.rstep[k];
+        }
         A xv[VEC];
         B yv[VEC];
         R zv[VEC];
         if (NIN >= 1) {
-            const char* a = p.ptr[0] + (int64_t)row * p.rstep[0];
+            const char* a = p.ptr[0] + roff[0];
             if (p.walk[0]) {
                 raw_load<A, VEC, NT>(a + (uint64_t)cv * (VEC * sizeof(A)), xv);
             } else {
@@ -611,7 +626,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
             }
         }
         if (two_arrays) {
-            const char* a = p.ptr[1] + (int64_t)row * p.rstep[1];
+            const char* a = p.ptr[1] + roff[1];
             if (p.walk[1]) {
                 raw_load<B, VEC, NT>(a + (uint64_t)cv * (VEC * sizeof(B)), yv);
             } else {
@@ -634,7 +649,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
             if (op(x, y, z)) okmask |= 1u << j;
             zv[j] = z;
         }
-        char* o = p.ptr[2] + (int64_t)row * p.rstep[2] + (uint64_t)cv * (VEC * sizeof(R));
+        char* o = p.ptr[2] + roff[2] + (uint64_t)cv * (VEC * sizeof(R));
         constexpr uint32_t full = (1u << VEC) - 1u;
         if (!Op::CHECKED || okmask == full) {
             raw_store<R, VEC, NT>(o, zv);
@@ -1224,18 +1239,21 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         }
 
         // rows x inner, every operand contiguous or constant along inner
-        bool r2 = n == 2 && (kp.inner % (uint64_t)vec) == 0 && kp.rows < 0xffffffffull && kp.inner / vec < 0xffffffffull;
+        // (or outer x mid x inner, which the planner leaves apart only when an operand repeats along one of the two)
+        bool r2 = (n == 2 || n == 3) && (kp.inner % (uint64_t)vec) == 0 && kp.rows < 0xffffffffull && kp.inner / vec < 0xffffffffull;
         EwR2Params rp;
         std::memset(&rp, 0, sizeof(rp));
+        if (n == 3) rp.mid = (uint32_t)plan.shape[1];
         for (int o = 0; o < nops && r2; ++o) {
             const int sl = slot[o];
             const int64_t es = sl == 0 ? (int64_t)sizeof(A) : (sl == 1 ? (int64_t)sizeof(B) : (int64_t)sizeof(R));
-            const int64_t is = plan.step[o][1];
+            const int64_t is = plan.step[o][n - 1];
             if (is == es) rp.walk[sl] = 1;
             else if (is == 0 && sl != 2) rp.walk[sl] = 0;
             else r2 = false;
             rp.ptr[sl] = const_cast<char*>(ops[o].ptr);
-            rp.rstep[sl] = plan.step[o][0];
+            rp.rstep[sl] = plan.step[o][n - 2];
+            if (n == 3) rp.ostep[sl] = plan.step[o][0];
         }
         if (r2) {
             const uint64_t inner_vecs = kp.inner / vec;

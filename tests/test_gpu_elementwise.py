@@ -86,6 +86,41 @@ def test_broadcast_shapes(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+def test_three_dimensions_with_an_operand_repeating_along_one(tname, dt):
+    """[B,T,C] with [T,1], [B,1,C], [1,T,C], [B,1,1] and a column on both sides: the shapes whose two
+    outer dimensions do not merge; C a whole number of 128-bit vectors and not; outer views."""
+    rng = np.random.default_rng(202)
+    cls = cls_of(tname)
+    for (B, T, Cn) in [(6, 10, 64), (3, 7, 36), (2, 300, 8), (5, 4, 30)]:
+        a = rng.standard_normal((B, T, Cn)).astype(dt)
+        da = cls.cast(a)
+        for shp in [(T, 1), (B, 1, Cn), (1, T, Cn), (B, 1, 1), (1, T, 1), (B, T, 1)]:
+            b = rng.standard_normal(shp).astype(dt)
+            db = cls.cast(b)
+            assert_bits_equal((da + db).to_numpy(), oracle.binary("add", a, b), "%s + %s" % ((B, T, Cn), shp))
+            assert_bits_equal((db / da).to_numpy(), oracle.binary("div", b, a), "%s / %s" % (shp, (B, T, Cn)))
+        # both operands repeat, along different dimensions; a scalar rides along
+        p_ = rng.standard_normal((B, 1, Cn)).astype(dt)
+        q_ = rng.standard_normal((1, T, 1)).astype(dt)
+        assert_bits_equal((cls.cast(p_) * cls.cast(q_)).to_numpy(), oracle.binary("mul", p_, q_))
+        # views: every second outer slice, reversed middle dimension
+        b = rng.standard_normal((T, 1)).astype(dt)
+        assert_bits_equal((da[::2] - cls.cast(b)).to_numpy(), oracle.binary("sub", np.ascontiguousarray(a[::2]), b))
+        assert_bits_equal((da[:, ::-1] - cls.cast(b)).to_numpy(), oracle.binary("sub", np.ascontiguousarray(a[:, ::-1]), b))
+        # into a given result that is itself a view with padded rows
+        out = cls.zeros(B, T, Cn + 4)
+        out[:, :, :Cn].store(da * cls.cast(b))
+        assert_bits_equal(out.to_numpy()[:, :, :Cn], oracle.binary("mul", a, b))
+    import cumo_amd
+    x = rng.integers(-100, 100, size=(4, 5, 8)).astype(np.int32)
+    y = rng.integers(1, 9, size=(5, 1)).astype(np.int32)
+    assert ((cumo_amd.Int32.cast(x) / cumo_amd.Int32.cast(y)).to_numpy() == oracle.binary("div", x, y)).all()
+    y[2, 0] = 0
+    with pytest.raises(ZeroDivisionError):
+        cumo_amd.Int32.cast(x) / cumo_amd.Int32.cast(y)
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 def test_many_dims_and_permuted_views(tname, dt):
     # past the reference's specialised accessors (ndim 5..8: test/narray_test.rb:41-51)
     rng = np.random.default_rng(102)
