@@ -168,6 +168,7 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
     std::memset(plan, 0, sizeof(*plan));
     plan->vec = 1;
     plan->n_split = 1;
+    plan->local_split_bits = 0;
     plan->threads_per_row = 1;
     const int in_ndim = arg->in_indexer.ndim;
     const int out_ndim_in = arg->out_indexer.ndim;
@@ -245,6 +246,12 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
             uint64_t fits = N / 32;
             uint64_t s = want < fits ? want : fits;
             if (s > 1024) s = 1024;
+            // up to 16 ways inside the block (combined through LDS, no second launch); what is still
+            // missing across blocks, with a second launch over that many fewer partial results
+            int bits = 0;
+            while (bits < 4 && (2ull << bits) <= s) ++bits;
+            plan->local_split_bits = bits;
+            s = (s + (1ull << bits) - 1) >> bits;
             if (s >= 2) plan->n_split = (int)s;
         }
         (void)accum_bytes;

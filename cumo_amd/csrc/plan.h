@@ -46,6 +46,7 @@ struct ReducePlan {
     int vec;               // elements per access along the contiguous axis
     int threads_per_row;   // RED_ROW: lanes sharing one output (power of two, <= 256)
     int n_split;           // > 1: the reduce axis is cut into n_split chunks and combined by a second launch
+    int local_split_bits;  // RED_COL: 2^bits lanes of a block share an output's reduce axis and combine through LDS
     int out_ndim, red_ndim;
     uint64_t out_total, red_total;
     uint64_t out_shape[kMaxDim], red_shape[kMaxDim];

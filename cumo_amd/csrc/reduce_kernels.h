@@ -15,6 +15,9 @@
 //                  neighbouring outputs and walks the reduce axis itself, so
 //                  loads are 128-bit and coalesced across lanes and nothing
 //                  is combined across lanes at all.
+//  red_col_local_kernel  the same when the outputs are too few to fill the
+//                  chip: 2..16 lanes of a block share the reduce axis of an
+//                  output group and combine through LDS in axis order.
 //
 // Either kernel can run as the first pass of a split reduction: the reduce
 // axis is cut into n_split chunks, accumulators go to
@@ -54,6 +57,7 @@ struct RedKParams {
     int tpr_bits;        // row kernel: 2^tpr_bits lanes per output
     int index_mode;      // what accumulate() gets as idx: 1 = position along the flattened reduce axes, 2 = element offset from in
     int small;           // totals fit 32 bits
+    int lsplit_bits;     // column kernel: 2^lsplit_bits lanes of a block share an output's reduce axis
     uint64_t out_total, red_total;
     uint64_t n_split, chunk;
     uint64_t out_shape[kMaxDim], red_shape[kMaxDim];
@@ -276,13 +280,92 @@ __global__ __launch_bounds__(kRedBlock) void red_row_kernel(RedKParams p, Impl i
     }
 }
 
+// One lane's VEC neighbouring outputs folded over positions [begin, end) of the reduce axis
+// (base: the first of the outputs at position 0; in_off: its byte offset from the array's start).
+template <class Impl, int VEC, bool NT>
+__device__ __forceinline__ void red_col_walk(const RedKParams& p, const Impl& impl, const char* base, int64_t in_off, uint64_t begin, uint64_t end,
+                                             typename Impl::Acc (&acc)[VEC]) {
+    typedef typename Impl::In In;
+    const int64_t ostep_in = p.in_out_step[p.out_ndim - 1];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = impl.identity();
+
+    for (uint64_t i0 = begin; i0 < end; i0 += kRedUnroll) {
+        In x[kRedUnroll][VEC];
+        int64_t roff[kRedUnroll];
+#pragma unroll
+        for (int u = 0; u < kRedUnroll; ++u) {
+            const uint64_t i = i0 + u;
+            if (i < end) {
+                const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
+                roff[u] = off;
+                if constexpr (VEC > 1) {
+                    RedVec<In, VEC> v;
+                    if constexpr (NT && sizeof(RedVec<In, VEC>) == 16) {
+                        typedef uint32_t ntu4 __attribute__((ext_vector_type(4)));
+                        union NTV { ntu4 q; RedVec<In, VEC> r; __device__ NTV() {} } ntv;
+                        ntv.q = __builtin_nontemporal_load(reinterpret_cast<const ntu4*>(base + off));
+                        v = ntv.r;
+                    } else {
+                        v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
+                    }
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
+                } else {
+                    x[u][0] = *reinterpret_cast<const In*>(base + off);
+                }
+            }
+        }
+        if (i0 + kRedUnroll <= end && p.index_mode != 2) {
+            // a whole block of consecutive positions along the axis for each output
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                In t[kRedUnroll];
+#pragma unroll
+                for (int u = 0; u < kRedUnroll; ++u) t[u] = x[u][j];
+                impl.template accumulate_n<kRedUnroll>(t, (int64_t)i0, acc[j]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kRedUnroll; ++u) {
+                const uint64_t i = i0 + u;
+                if (i < end) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        int64_t idx = 0;
+                        if (Impl::USES_INDEX) {
+                            idx = (p.index_mode == 2) ? ((in_off + roff[u] + (int64_t)j * ostep_in) / (int64_t)sizeof(In)) : (int64_t)i;
+                        }
+                        impl.accumulate(x[u][j], idx, acc[j]);
+                    }
+                }
+            }
+        }
+    }
+    if constexpr (has_exact<Impl>::value) {
+        // this thread walked the axis in order, but its fast fold may still have lost
+        // which of two equal elements came first: walk that output again, exactly
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            if (impl.needs_exact(acc[j])) {
+                typedef typename Impl::Exact Exact;
+                const Exact ex = impl.exact();
+                typename Exact::Acc e = ex.identity();
+                for (uint64_t i = begin; i < end; ++i) {
+                    const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
+                    ex.accumulate(*reinterpret_cast<const In*>(base + off + (int64_t)j * ostep_in), (int64_t)i, e);
+                }
+                acc[j] = impl.from_exact(e);
+            }
+        }
+    }
+}
+
 template <class Impl, int VEC, bool PARTIAL, bool NT = false>
 __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
-    typedef typename Impl::In In;
     typedef typename Impl::Acc Acc;
     const uint64_t groups = p.out_total / VEC;  // planner guarantees divisibility of the innermost out dim
     const uint64_t n_items = groups * p.n_split;
-    const int L = p.out_ndim - 1;
 
     for (uint64_t g = (uint64_t)blockIdx.x * kRedBlock + threadIdx.x; g < n_items; g += (uint64_t)gridDim.x * kRedBlock) {
         uint64_t i_split = 0, cg = g;
@@ -292,85 +375,13 @@ __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl i
         }
         const uint64_t i_out0 = cg * VEC;
         const int64_t in_off = red_decompose(i_out0, p.out_ndim, p.out_shape, p.in_out_step, p.small);
-        const int64_t ostep_in = p.in_out_step[L];
         const char* base = p.in + in_off;
         const uint64_t begin = i_split * p.chunk;
         uint64_t end = begin + p.chunk;
         if (end > p.red_total) end = p.red_total;
 
         Acc acc[VEC];
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] = impl.identity();
-
-        for (uint64_t i0 = begin; i0 < end; i0 += kRedUnroll) {
-            In x[kRedUnroll][VEC];
-            int64_t roff[kRedUnroll];
-#pragma unroll
-            for (int u = 0; u < kRedUnroll; ++u) {
-                const uint64_t i = i0 + u;
-                if (i < end) {
-                    const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
-                    roff[u] = off;
-                    if constexpr (VEC > 1) {
-                        RedVec<In, VEC> v;
-                        if constexpr (NT && sizeof(RedVec<In, VEC>) == 16) {
-                            typedef uint32_t ntu4 __attribute__((ext_vector_type(4)));
-                            union NTV { ntu4 q; RedVec<In, VEC> r; __device__ NTV() {} } ntv;
-                            ntv.q = __builtin_nontemporal_load(reinterpret_cast<const ntu4*>(base + off));
-                            v = ntv.r;
-                        } else {
-                            v = *reinterpret_cast<const RedVec<In, VEC>*>(base + off);
-                        }
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) x[u][j] = v.v[j];
-                    } else {
-                        x[u][0] = *reinterpret_cast<const In*>(base + off);
-                    }
-                }
-            }
-            if (i0 + kRedUnroll <= end && p.index_mode != 2) {
-                // a whole block of consecutive positions along the axis for each output
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    In t[kRedUnroll];
-#pragma unroll
-                    for (int u = 0; u < kRedUnroll; ++u) t[u] = x[u][j];
-                    impl.template accumulate_n<kRedUnroll>(t, (int64_t)i0, acc[j]);
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < kRedUnroll; ++u) {
-                    const uint64_t i = i0 + u;
-                    if (i < end) {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) {
-                            int64_t idx = 0;
-                            if (Impl::USES_INDEX) {
-                                idx = (p.index_mode == 2) ? ((in_off + roff[u] + (int64_t)j * ostep_in) / (int64_t)sizeof(In)) : (int64_t)i;
-                            }
-                            impl.accumulate(x[u][j], idx, acc[j]);
-                        }
-                    }
-                }
-            }
-        }
-        if constexpr (has_exact<Impl>::value) {
-            // this thread walked the axis in order, but its fast fold may still have lost
-            // which of two equal elements came first: walk that output again, exactly
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                if (impl.needs_exact(acc[j])) {
-                    typedef typename Impl::Exact Exact;
-                    const Exact ex = impl.exact();
-                    typename Exact::Acc e = ex.identity();
-                    for (uint64_t i = begin; i < end; ++i) {
-                        const int64_t off = red_decompose(i, p.red_ndim, p.red_shape, p.in_red_step, p.small);
-                        ex.accumulate(*reinterpret_cast<const In*>(base + off + (int64_t)j * ostep_in), (int64_t)i, e);
-                    }
-                    acc[j] = impl.from_exact(e);
-                }
-            }
-        }
+        red_col_walk<Impl, VEC, NT>(p, impl, base, in_off, begin, end, acc);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
             const uint64_t i_out = i_out0 + j;
@@ -382,6 +393,81 @@ __global__ __launch_bounds__(kRedBlock) void red_col_kernel(RedKParams p, Impl i
                 impl.store(acc[j], p.out + o1, (Impl::NOUT > 1) ? (p.out2 + o2) : nullptr);
             }
         }
+    }
+}
+
+// The same with the reduce axis also cut inside the block: 2^lsplit_bits lanes share each group of
+// VEC outputs, each walks its part of the (launch-level) chunk, and the parts are combined through
+// LDS in axis order by the first of them. More blocks for an array with few outputs across memory,
+// without a second launch (or with a much smaller one when the launch-level split is still needed).
+template <class Impl, int VEC, bool PARTIAL, bool NT = false>
+__global__ __launch_bounds__(kRedBlock) void red_col_local_kernel(RedKParams p, Impl impl, typename Impl::Acc* partial) {
+    typedef typename Impl::Acc Acc;
+    __shared__ Acc part[kRedBlock][VEC];
+    const unsigned SB = 1u << p.lsplit_bits;
+    const unsigned cbits = 8u - (unsigned)p.lsplit_bits;  // kRedBlock = 2^8
+    const unsigned CPB = 1u << cbits;
+    const unsigned c = threadIdx.x & (CPB - 1);
+    const unsigned s = threadIdx.x >> cbits;
+    const uint64_t groups = p.out_total / VEC;
+    const uint64_t n_items = groups * p.n_split;
+    const uint64_t n_blocks = (n_items + CPB - 1) / CPB;
+
+    for (uint64_t blk = blockIdx.x; blk < n_blocks; blk += gridDim.x) {
+        const uint64_t g = blk * CPB + c;
+        const bool ok = g < n_items;
+        uint64_t i_split = 0, cg = 0;
+        if (ok) {
+            cg = g;
+            if (p.n_split > 1) {
+                i_split = g / groups;
+                cg = g - i_split * groups;
+            }
+        }
+        const uint64_t i_out0 = cg * VEC;
+        Acc acc[VEC];
+        if (ok) {
+            const int64_t in_off = red_decompose(i_out0, p.out_ndim, p.out_shape, p.in_out_step, p.small);
+            const uint64_t gbegin = i_split * p.chunk;
+            uint64_t gend = gbegin + p.chunk;
+            if (gend > p.red_total) gend = p.red_total;
+            const uint64_t lchunk = (gend - gbegin + SB - 1) / SB;
+            uint64_t begin = gbegin + (uint64_t)s * lchunk;
+            if (begin > gend) begin = gend;
+            uint64_t end = begin + lchunk;
+            if (end > gend) end = gend;
+            red_col_walk<Impl, VEC, NT>(p, impl, p.in + in_off, in_off, begin, end, acc);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = impl.identity();
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = acc[j];
+        __syncthreads();
+        if (ok && s == 0) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if constexpr (has_exact<Impl>::value) {
+                    // the parts are plain values in axis order: fold them with the exact rule
+                    typedef typename Impl::Exact Exact;
+                    const Exact ex = impl.exact();
+                    typename Exact::Acc e = ex.identity();
+                    for (unsigned k = 0; k < SB; ++k) ex.accumulate(part[k * CPB + c][j], (int64_t)k, e);
+                    acc[j] = impl.from_exact(e);
+                } else {
+                    for (unsigned k = 1; k < SB; ++k) impl.combine(part[k * CPB + c][j], acc[j]);
+                }
+                const uint64_t i_out = i_out0 + j;
+                if (PARTIAL) {
+                    partial[i_out * p.n_split + i_split] = acc[j];
+                } else {
+                    const int64_t o1 = red_decompose(i_out, p.out_ndim, p.out_shape, p.out_step, p.small);
+                    const int64_t o2 = (Impl::NOUT > 1) ? red_decompose(i_out, p.out_ndim, p.out_shape, p.out2_step, p.small) : 0;
+                    impl.store(acc[j], p.out + o1, (Impl::NOUT > 1) ? (p.out2 + o2) : nullptr);
+                }
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -469,10 +555,22 @@ template <class Impl, bool PARTIAL>
 static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Impl::Acc* partial, hipStream_t stream) {
     constexpr int kMaxVec = (int)(16 / sizeof(typename Impl::In));
     const uint64_t items = (kp.out_total / vec) * kp.n_split;
-    uint64_t grid = (items + kRedBlock - 1) / kRedBlock;
+    const uint64_t per_block = (uint64_t)kRedBlock >> kp.lsplit_bits;
+    uint64_t grid = (items + per_block - 1) / per_block;
     if (grid > red_grid_cap()) grid = red_grid_cap();
     if (grid == 0) return;
     const dim3 g((unsigned)grid), b(kRedBlock);
+    if (kp.lsplit_bits > 0) {
+        // lanes of a block share the reduce axis of an output (few outputs across memory)
+        if constexpr (kMaxVec >= 4) {
+            if (vec == 4) { hipLaunchKernelGGL((red_col_local_kernel<Impl, 4, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
+        }
+        if constexpr (kMaxVec >= 2) {
+            if (vec == 2) { hipLaunchKernelGGL((red_col_local_kernel<Impl, 2, PARTIAL>), g, b, 0, stream, kp, impl, partial); return; }
+        }
+        hipLaunchKernelGGL((red_col_local_kernel<Impl, 1, PARTIAL>), g, b, 0, stream, kp, impl, partial);
+        return;
+    }
     if constexpr (kMaxVec >= 2) {
         if (vec == kMaxVec && kp.out_total * kp.red_total * sizeof(typename Impl::In) > kRedNtBytes) {
             hipLaunchKernelGGL((red_col_kernel<Impl, kMaxVec, PARTIAL, true>), g, b, 0, stream, kp, impl, partial);
@@ -506,6 +604,7 @@ static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     red_fill_params(&kp, plan, arg, out2, index_mode);
     kp.tpr_bits = 0;
     while ((1 << kp.tpr_bits) < plan.threads_per_row) ++kp.tpr_bits;
+    kp.lsplit_bits = plan.kind == RED_COL ? plan.local_split_bits : 0;
 
     if (plan.n_split <= 1) {
         if (plan.kind == RED_COL) red_launch_col<Impl, false>(kp, plan.vec, impl, nullptr, stream);
@@ -533,6 +632,7 @@ static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
 
     // second pass over partial[out_total][n_split]
     RedKParams k2 = kp;
+    k2.lsplit_bits = 0;
     k2.in = reinterpret_cast<char*>(partial);
     k2.red_ndim = 1;
     k2.red_shape[0] = kp.n_split;
