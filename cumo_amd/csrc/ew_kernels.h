@@ -1164,11 +1164,16 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     int vec = plan.vec;
     // the vector form of a Bit row needs the 32/vec lanes of a word inside one row
     if (Op::BIT_OUT && vec > 1 && kp.inner < 32) vec = 1;
+    bool force_scalar = false;
     {
         static int force1 = -1;
         if (force1 < 0) force1 = std::getenv("CUMO_HIP_FORCE_VEC1") ? 1 : 0;
         if (force1) vec = 1;
+        force_scalar = force1 != 0;
     }
+    // the two lean kernels below also take inputs that only have their element's alignment
+    // (a slice that starts at an odd column): a 128-bit global load works on any 4-byte boundary
+    const int lean_vec = (vec == 1 && plan.vec_loose > 1 && !force_scalar) ? plan.vec_loose : vec;
     const dim3 b(kEwBlock);
 
     // A Bit result over flat inputs, starting on a 128-bit unit: the lean Bit kernel
@@ -1202,7 +1207,8 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     // lane, one 4 KiB tile per block, 32-bit index arithmetic. Measured on 1 GiB
     // arrays against the general kernel below: 83% of peak against 70% (1R+1W),
     // 82% against 61% (2R+1W), 80% against 74% (matrix minus column vector).
-    if (!Op::BIT_OUT && vec > 1) {
+    if (!Op::BIT_OUT && lean_vec > 1) {
+        const int vec = lean_vec;
         // bytes the operation touches: an operand that repeats along a dimension
         // counts once along it
         uint64_t bytes = 0;

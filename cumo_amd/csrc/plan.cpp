@@ -45,6 +45,7 @@ void plan_elementwise(int ndim, const size_t* shape, int nops, const EwOperand* 
     std::memset(plan, 0, sizeof(*plan));
     plan->tr_dim = -1;
     plan->vec = 1;
+    plan->vec_loose = 1;
     uint64_t total = 1;
     for (int d = 0; d < ndim; ++d) total *= shape[d];
     plan->total = total;
@@ -127,6 +128,8 @@ void plan_elementwise(int ndim, const size_t* shape, int nops, const EwOperand* 
     }
     if (min_elmsz == 16) min_elmsz = 4;
     const int L = n - 1;
+    plan->vec_loose = 1;
+    for (int loose = 1; loose >= 0; --loose)
     for (int vec = 16 / min_elmsz; vec > 1; vec >>= 1) {
         bool ok = sh[L] >= (uint64_t)vec;
         for (int o = 0; o < nops && ok; ++o) {
@@ -146,12 +149,17 @@ void plan_elementwise(int ndim, const size_t* shape, int nops, const EwOperand* 
             if (st[o][L] != es) { ok = false; break; }
             int align = vec * es;
             if (align > 16) align = 16;
+            if (loose && o != out && es >= 4) align = es;
             if (((uintptr_t)ops[o].ptr % align) != 0) { ok = false; break; }
             for (int d = 0; d < L; ++d) if (st[o][d] % align) { ok = false; break; }
         }
         // rows that are not a whole number of vectors would leave the next row unaligned
         if (ok && n > 1 && (sh[L] % vec) != 0) ok = false;
-        if (ok) { plan->vec = vec; break; }
+        if (ok) {
+            if (loose) plan->vec_loose = vec;
+            else plan->vec = vec;
+            break;
+        }
     }
 }
 

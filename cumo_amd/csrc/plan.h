@@ -29,6 +29,8 @@ struct EwPlan {
     int kind;
     int ndim;       // collapsed dims; the fast dim is last, for EW_TRANSPOSE the second tile dim is ndim-2
     int vec;        // elements per thread per access (1, 2 or 4)
+    int vec_loose;  // the same when inputs only need their element's alignment (global loads of 128 bits
+                    // work on any 4-byte boundary); the result still starts on a boundary of the access
     int fast_dim;   // which collapsed dim (before the final permutation) became last
     int tr_dim;     // ditto for the transpose partner, -1 otherwise
     uint64_t total;

@@ -120,6 +120,38 @@ def test_three_dimensions_with_an_operand_repeating_along_one(tname, dt):
         cumo_amd.Int32.cast(x) / cumo_amd.Int32.cast(y)
 
 
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_inputs_that_start_off_a_16_byte_boundary(tname, dt):
+    """Slices that begin at an odd column (rows and flat runs whose length is still a whole number of
+    128-bit accesses): the lean kernels read them with 128-bit loads on 4- or 8-byte boundaries."""
+    rng = np.random.default_rng(303)
+    cls = cls_of(tname)
+    mk = (lambda shp: rng.integers(-1000, 1000, size=shp).astype(dt)) if dt == np.int32 else (lambda shp: rng.standard_normal(shp).astype(dt))
+    a, b = mk((37, 1030)), mk((37, 1030))
+    da, db = cls.cast(a), cls.cast(b)
+    for lo in (1, 2, 3, 5):
+        for n in (1000, 1024, 8, 4):
+            va, vb = a[:, lo:lo + n], b[:, lo + 1:lo + 1 + n]
+            assert_bits_equal((da[:, lo:lo + n] * 2).to_numpy(), oracle.binary("mul", np.ascontiguousarray(va), 2), "scalar %d %d" % (lo, n))
+            assert_bits_equal((da[:, lo:lo + n] + db[:, lo + 1:lo + 1 + n]).to_numpy(),
+                              oracle.binary("add", np.ascontiguousarray(va), np.ascontiguousarray(vb)), "two views %d %d" % (lo, n))
+            assert_bits_equal((da[:, lo:lo + n] - db[:, :n]).to_numpy(),
+                              oracle.binary("sub", np.ascontiguousarray(va), np.ascontiguousarray(b[:, :n])), "one view %d %d" % (lo, n))
+    # a flat run, a row vector and a column against it, rows in reverse
+    f = mk(4099 * 3)
+    df = cls.cast(f)
+    for lo in (1, 3):
+        assert_bits_equal((df[lo:lo + 12288] + df[lo + 2:lo + 2 + 12288]).to_numpy(), oracle.binary("add", f[lo:lo + 12288].copy(), f[lo + 2:lo + 2 + 12288].copy()))
+    r, c = mk((1, 1030)), mk((37, 1))
+    assert_bits_equal((da[:, 3:1003] + cls.cast(r)[:, 1:1001]).to_numpy(), oracle.binary("add", a[:, 3:1003].copy(), r[:, 1:1001].copy()))
+    assert_bits_equal((da[:, 3:1003] * cls.cast(c)).to_numpy(), oracle.binary("mul", a[:, 3:1003].copy(), c))
+    assert_bits_equal((da[::-1, 3:1003] - db[:, 2:1002]).to_numpy(), oracle.binary("sub", a[::-1, 3:1003].copy(), b[:, 2:1002].copy()))
+    if dt != np.int32:
+        import cumo_amd
+        got = cumo_amd.NMath.exp(da[:, 1:1001]).to_numpy()
+        assert_ulp(got, oracle.unary("exp", a[:, 1:1001].copy()), 1 if dt == np.float32 else 2)
+
+
 @pytest.mark.parametrize("tname,dt", FLOATS)
 def test_many_dims_and_permuted_views(tname, dt):
     # past the reference's specialised accessors (ndim 5..8: test/narray_test.rb:41-51)
