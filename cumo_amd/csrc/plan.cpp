@@ -239,10 +239,12 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
         const int L = no - 1;
         int vec = 16 / in_elmsz;
         for (; vec > 1; vec >>= 1) {
+            // the input is only read: a 128-bit global load needs no more than the element's alignment
+            const int align = in_elmsz >= 4 ? in_elmsz : vec * in_elmsz;
             bool ok = plan->in_out_step[L] == in_elmsz && (plan->out_shape[L] % vec) == 0 &&
-                      ((uintptr_t)arg->in.ptr % (vec * in_elmsz)) == 0;
-            for (int d = 0; d < L && ok; ++d) ok = (plan->in_out_step[d] % (vec * in_elmsz)) == 0;
-            for (int d = 0; d < nr && ok; ++d) ok = (plan->in_red_step[d] % (vec * in_elmsz)) == 0;
+                      ((uintptr_t)arg->in.ptr % align) == 0;
+            for (int d = 0; d < L && ok; ++d) ok = (plan->in_out_step[d] % align) == 0;
+            for (int d = 0; d < nr && ok; ++d) ok = (plan->in_red_step[d] % align) == 0;
             if (ok) break;
         }
         plan->vec = vec < 1 ? 1 : vec;
@@ -269,10 +271,11 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
     plan->kind = RED_ROW;
     int vec = 16 / in_elmsz;
     for (; vec > 1; vec >>= 1) {
+        const int align = in_elmsz >= 4 ? in_elmsz : vec * in_elmsz;  // read-only: the element's alignment is enough
         bool ok = nr > 0 && plan->in_red_step[nr - 1] == in_elmsz && (plan->red_shape[nr - 1] % vec) == 0 &&
-                  ((uintptr_t)arg->in.ptr % (vec * in_elmsz)) == 0;
-        for (int d = 0; d < nr - 1 && ok; ++d) ok = (plan->in_red_step[d] % (vec * in_elmsz)) == 0;
-        for (int d = 0; d < no && ok; ++d) ok = (plan->in_out_step[d] % (vec * in_elmsz)) == 0;
+                  ((uintptr_t)arg->in.ptr % align) == 0;
+        for (int d = 0; d < nr - 1 && ok; ++d) ok = (plan->in_red_step[d] % align) == 0;
+        for (int d = 0; d < no && ok; ++d) ok = (plan->in_out_step[d] % align) == 0;
         if (ok) break;
     }
     plan->vec = vec < 1 ? 1 : vec;

@@ -283,3 +283,27 @@ def test_few_outputs_across_memory_share_the_axis_inside_a_block(tname, dt, shap
     di = cumo_amd.Int32.cast(hi32)
     for name in ("sum", "min", "max", "argmax", "argmin"):
         assert (getattr(di, name)(axis=axis).to_numpy() == oracle.reduce(name, hi32, axis=axis)).all(), name
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_reductions_of_slices_that_start_off_a_16_byte_boundary(tname, dt):
+    """Inner slices beginning at an odd column, with lengths that are whole 128-bit accesses: the
+    kernels read them with wide loads on element boundaries; along the rows, down the columns, all."""
+    rng = np.random.default_rng(808)
+    cls = cls_of(tname)
+    h = (rng.integers(-64, 64, size=(9, 70, 1040)) / 16.0).astype(dt)
+    d = cls.cast(h)
+    for lo, n in ((1, 1024), (3, 1000), (2, 8), (5, 512)):
+        hv, dv = np.ascontiguousarray(h[:, :, lo:lo + n]), d[:, :, lo:lo + n]
+        for axis in (2, 1, 0, (0, 1), (1, 2), None):
+            for name in ("sum", "min", "max", "argmax", "argmin"):
+                assert_bits_equal(getattr(dv, name)(axis=axis).to_numpy(), oracle.reduce(name, hv, axis=axis), "%s %r %r" % (name, (lo, n), axis))
+            # the moments against the exact value (the sequential float32 loop is itself further from it)
+            exact = hv.astype(np.float64).var(axis=axis, ddof=1)
+            assert np.allclose(dv.var(axis=axis).to_numpy(), exact, rtol=2e-5 if dt == np.float32 else 1e-12, atol=0), ("var", lo, n, axis)
+    i = rng.integers(-1000, 1000, size=(50, 1030)).astype(np.int32)
+    import cumo_amd
+    di = cumo_amd.Int32.cast(i)
+    for axis in (0, 1, None):
+        assert (di[:, 3:1027].sum(axis=axis).to_numpy() == oracle.reduce("sum", np.ascontiguousarray(i[:, 3:1027]), axis=axis)).all()
+        assert (di[:, 3:1027].argmax(axis=axis).to_numpy() == oracle.reduce("argmax", np.ascontiguousarray(i[:, 3:1027]), axis=axis)).all()
