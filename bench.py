@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # counter's reading for --pmc-calibration's plain 256 MiB copy (FETCH_SIZE x 1.9998,
 # WRITE_SIZE x 0.9996): 131137 KiB fetched + 131024 KiB written. The figures and
 # the commands are in profiles/ew_rows2_add_f64_c2_hbm_traffic.txt.
-C2_ADD_TRAFFIC_BYTES = 268466760
+C2_ADD_TRAFFIC_BYTES = 268466618
 METRIC = "achieved HBM GB/s (% of MI355X peak) and GElem/s vs Numo CPU, per config"
 MIB = 1 << 20
 
