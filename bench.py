@@ -10,6 +10,12 @@ C-ABI. `value` is algorithmic bytes per step / seconds per step in GB/s, where
 algorithmic bytes count every distinct input element once and every output element
 once (the reference's own convention, bench/cumo_probe.rb:74-232).
 
+Every GPU figure is taken with ROTATED buffers: consecutive launches (or steps) take
+turns over several distinct sets of operands and results, so that at least 1 GiB of
+other data passes between two uses of a buffer and nothing is served by the 256 MB
+last-level cache -- sustained HBM. The same measurement on one set of buffers, back
+to back, is printed beside it (`value_replay`, `frac_replay`).
+
 `roofline` covers the dominant kernel of the step (the broadcast add, 256 MiB of
 the step's 512 MiB), timed per launch with HIP events on the stream the launchers
 use. `cpu_baseline` times the Numo-shaped single-thread C loops of the oracle on the
@@ -32,12 +38,27 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of the C2 broadcast add, from two rocprofv3 --pmc runs of this
-# file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by the same
-# counter's reading for --pmc-calibration's plain 256 MiB copy (FETCH_SIZE x 1.9998,
-# WRITE_SIZE x 0.9996): 131137 KiB fetched + 131024 KiB written. The figures and
-# the commands are in profiles/ew_rows2_add_f64_c2_hbm_traffic.txt.
-C2_ADD_TRAFFIC_BYTES = 268466618
+ADD_KERNEL = "ew_rows2_kernel<OpAdd<double>, 2, true>"
+# HBM bytes per launch of the C2 broadcast add come from two rocprofv3 --pmc runs of this
+# file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by the same counter's
+# reading for --pmc-calibration's plain 256 MiB copy. The summary of those runs is kept in
+# this file, and the line that starts with TRAFFIC_KEY carries the figure; it is read from
+# there (never typed in here), and reported as null when the summary is absent.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "ew_rows2_add_f64_c2_hbm_traffic.txt")
+TRAFFIC_KEY = "traffic_bytes_per_launch"
+
+
+def read_traffic_bytes():
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith(TRAFFIC_KEY):
+                    return int(line.split("=")[1].split()[0])
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
+
+
 METRIC = "achieved HBM GB/s (% of MI355X peak) and GElem/s vs Numo CPU, per config"
 MIB = 1 << 20
 
@@ -175,12 +196,38 @@ def config_ops(name, cumo, host):
             ("x[rows,true] (gather)", lambda e: e.__setitem__("g", e["x"][e["rows"]]), 2 * nb + 8 * r, n),
             ("b[perm,true]=x (scatter)", lambda e: e["b"].__setitem__(e["perm"], e["x"]), 2 * nb + 8 * r, n),
         ]
+    if name == "nmath":
+        # NMath beyond exp / sqrt, the Float power and the scans on 2^26 elements (256 MiB SFloat,
+        # 512 MiB DFloat per array); arguments positive so that every function is defined
+        x = host["x"]
+        n = x.size
+        env = {"xs": cumo.SFloat.cast(x), "xd": cumo.DFloat.cast(x.astype(np.float64))}
+        env["xs2"] = env["xs"].reshape(8192, n // 8192)
+        ops = []
+        for fname in ("log", "sin", "cos", "tan", "tanh", "erf", "asinh", "atan", "exp", "sqrt"):
+            ops.append(("NMath.%s(SFloat)" % fname, (lambda f: lambda e: e.__setitem__("r", getattr(NM, f)(e["xs"])))(fname), 8 * n, n))
+        for fname in ("log", "sin", "tanh", "erf", "exp", "sqrt"):
+            ops.append(("NMath.%s(DFloat)" % fname, (lambda f: lambda e: e.__setitem__("rd", getattr(NM, f)(e["xd"])))(fname), 16 * n, n))
+        ops += [
+            ("SFloat**2.5", lambda e: e.__setitem__("r", e["xs"] ** 2.5), 8 * n, n),
+            ("DFloat**2.5", lambda e: e.__setitem__("rd", e["xd"] ** 2.5), 16 * n, n),
+            ("SFloat.cumsum (one run of 2^26)", lambda e: e.__setitem__("r", e["xs"].cumsum()), 8 * n, n),
+            ("SFloat[8192,8192].cumsum(axis:0)", lambda e: e.__setitem__("r2", e["xs2"].cumsum(axis=0)), 8 * n, n),
+            ("SFloat[8192,8192].cumsum(axis:1)", lambda e: e.__setitem__("r2", e["xs2"].cumsum(axis=1)), 8 * n, n),
+        ]
+        return env, ops
     raise ValueError(name)
+
+
+def inputs_nmath(n=1 << 26):
+    rng = np.random.default_rng(6)
+    return {"x": rng.uniform(0.05, 3.0, n).astype(np.float32)}
 
 
 HOST_INPUTS = {
     "c1": inputs_c1, "c1_large": lambda: inputs_c1(1 << 26), "c2": inputs_c2, "c3": inputs_c3, "c4": inputs_c4, "c5": inputs_c5,
     "c2_large": lambda: inputs_c2(8192), "c3_large": lambda: inputs_c3((256, 512, 1024)), "next": inputs_next,
+    "nmath": inputs_nmath,
 }
 WORKLOAD_TEXT = {
     "c1": "C1 SFloat axpy + full sum, n=2^20",
@@ -188,6 +235,7 @@ WORKLOAD_TEXT = {
     "c2_large": "C2 at 8192 x 8192 (512 MiB per matrix)",
     "c3_large": "C3 at [256,512,1024] (512 MiB)",
     "next": "operations beside the five configs on SFloat [8192,4096]: mulsum, clip, maximum, integer power, cumsum, where, a[mask], row gather and scatter through index arrays",
+    "nmath": "NMath functions, Float power and cumsum on 2^26 elements (SFloat 256 MiB, DFloat 512 MiB per array), arguments uniform in [0.05, 3)",
     "c2": "C2 DFloat broadcast add + row reduce: A f64 [4096,4096] + r [1,4096]; C.sum(axis:1); C.max(axis:1)",
     "c3": "C3 SFloat axis reductions on [64,512,1024]",
     "c4": "C4 strided/transposed views on SFloat [8192,8192] + Int32 stride-3 row slice copy",
@@ -212,39 +260,83 @@ class Timer:
         self.lib.cumo_hip_event_destroy(self.e1)
 
 
-def measure_config(name, cumo, lib, iters, warmup):
+ROTATE_BYTES = 1 << 30   # memory touched between two uses of one buffer in the rotated figures
+ROTATE_MAX_SETS = 9      # 128 MiB operations: eight other sets (1 GiB) between two uses of a set
+
+
+def rotation_sets(nbytes):
+    """How many distinct operand/result sets an operation of `nbytes` algorithmic bytes
+    is rotated over, so that at least ROTATE_BYTES of other data pass through the caches
+    between two uses of a buffer (the last-level cache holds 256 MB)."""
+    need = -(-ROTATE_BYTES // max(int(nbytes), 1)) + 1
+    return max(2, min(ROTATE_MAX_SETS, need))
+
+
+def measure_config(name, cumo, lib, iters, warmup, replay_too=True):
+    """Every op of a config, timed two ways with HIP events on the launch stream:
+    `rotated` -- consecutive launches take turns over K distinct sets of operands and
+    results (K device copies of the inputs, K results), so a launch finds none of its
+    data in a cache: sustained HBM; and `replay` -- the same call on the same buffers
+    back to back, which at 128-256 MiB is helped by the 256 MB last-level cache.
+    `frac_of_peak`, `gbps`, `gelem_s` are the rotated figures."""
     host = HOST_INPUTS[name]()
-    env, ops = config_ops(name, cumo, host)
+    sets = [config_ops(name, cumo, host)]
+    for _ in range(max(rotation_sets(o[2]) for o in sets[0][1]) - 1):
+        sets.append(config_ops(name, cumo, host))
     del host
     from cumo_amd import _lib
     timer = Timer(lib)
     rows = []
     batch = 10
-    for label, fn, nbytes, nelem in ops:
-        # the op runs once through the host mirror, which records the library calls
-        # it makes; the timed region issues exactly those C-ABI calls again (into the
-        # result the first call allocated), `batch` times back to back between two
-        # events on the launch stream, so the figure is the library's and not the
-        # Python mirror's
-        with _lib.record() as calls:
-            fn(env)
-        # launches that rewrite an index array in place (positions -> byte offsets) belong to
-        # building the view, not to the copy, and must not run twice on the same array
-        recorded = calls  # holds the temporaries the operation released
-        calls = [c for c in calls if not c[0].__name__.startswith("cumo_na_index_")]
-        _lib.replay(calls, warmup)
-        ts = [timer.time(lambda: _lib.replay(calls, batch)) / batch for _ in range(iters)]
-        ts.sort()
-        del recorded
-        med = ts[len(ts) // 2]
-        best = ts[0]
+    n_ops = len(sets[0][1])
+    for i in range(n_ops):
+        label, _, nbytes, nelem = sets[0][1][i]
+        # the op runs once per set through the host mirror, which records the library
+        # calls it makes; the timed region issues exactly those C-ABI calls again (into
+        # the result the first call allocated) between two events on the launch stream,
+        # so the figure is the library's and not the Python mirror's. Every set runs the
+        # op (later ops of the chain need its result), the rotation uses the first K.
+        per_set = []
+        keep = []
+        for env, ops in sets:
+            with _lib.record() as calls:
+                ops[i][1](env)
+            keep.append(calls)  # holds the temporaries the operation released
+            # launches that rewrite an index array in place (positions -> byte offsets) belong to
+            # building the view, not to the copy, and must not run twice on the same array
+            per_set.append([c for c in calls if not c[0].__name__.startswith("cumo_na_index_")])
+        k = rotation_sets(nbytes)
+        rot = per_set[:k]
+        state = [0]
+
+        def rotated(times):
+            j = state[0]
+            for _ in range(times):
+                for f, a in rot[j]:
+                    f(*a)
+                j = j + 1 if j + 1 < k else 0
+            state[0] = j
+            _lib.check()
+
+        rotated(max(warmup, k))
+        ts = sorted(timer.time(lambda: rotated(batch)) / batch for _ in range(iters))
+        del keep
+        med, best = ts[len(ts) // 2], ts[0]
+        row_replay = {}
+        if replay_too:
+            _lib.replay(per_set[0], warmup)
+            tr = sorted(timer.time(lambda: _lib.replay(per_set[0], batch)) / batch for _ in range(iters))
+            med_replay = tr[len(tr) // 2]
+            row_replay = {"ms_median_replay": round(med_replay, 5), "frac_replay": round(nbytes / (med_replay * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
         rows.append({
-            "op": label, "bytes": int(nbytes), "ms_median": round(med, 5), "ms_best": round(best, 5),
+            "op": label, "bytes": int(nbytes), "sets": k, "rotation_bytes": int(nbytes) * k,
+            "ms_median": round(med, 5), "ms_best": round(best, 5),
             "gbps": round(nbytes / (med * 1e-3) / 1e9, 1), "frac_of_peak": round(nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-            "gelem_s": round(nelem / (med * 1e-3) / 1e9, 2),
+            "gelem_s": round(nelem / (med * 1e-3) / 1e9, 2), **row_replay,
         })
     timer.close()
-    env.clear()
+    for env, _ in sets:
+        env.clear()
     # the pool keeps its blocks from one config to the next, as it does in a long-running process
     return rows
 
@@ -369,9 +461,11 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all-configs", action="store_true", help="measure every op of all five configs with full iteration counts")
-    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next)")
+    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next,nmath)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
+    ap.add_argument("--rotated-only", action="store_true",
+                    help="leave out the same-buffer replay legs, so that a kernel trace of this command holds rotated launches only")
     ap.add_argument("--no-extras", action="store_true", help="skip the host transfer and recorded-chain measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch a plain contiguous copy of known size (256 MiB in, 256 MiB out) five times, so that a "
@@ -392,73 +486,125 @@ def main():
     # ---- headline step: C2 -------------------------------------------------------
     host = inputs_c2()
     n = host["A"].shape[0]
-    env, ops = config_ops("c2", cumo_amd, host)
+    K = ROTATE_MAX_SETS
+    sets = [config_ops("c2", cumo_amd, host) for _ in range(K)]
+    env, ops = sets[0]
     step_bytes = sum(o[2] for o in ops)
 
     # The timed step is the chain as the extension's C host side runs it: three
     # calls into the library's host launch layer (broadcast, result allocation
-    # from the pool, descriptors, launch), each result released again once the
-    # chain is done. Only the Ruby VM above it is missing.
+    # from the pool, descriptors, launch). Only the Ruby VM above it is missing.
+    # Consecutive steps take turns over K device copies of the inputs, and a step's
+    # three results are released K steps later, so every buffer a step touches was
+    # last used more than 1 GiB of traffic ago: nothing but the chain's own
+    # producer -> consumer reuse (C is read right after it is written) can come
+    # from a cache.
     NA = _lib.NArrayDesc
-    dA, dr = env["A"]._desc(), env["r"]._desc()
+    descs = [(e["A"]._desc(), e["r"]._desc()) for e, _ in sets]
     na_binary, na_reduce, na_free = lib.cumo_hip_na_binary, lib.cumo_hip_na_reduce, lib.cumo_cuda_runtime_free
     ref = C.byref
+    ring = [None] * K
+    turn = [0]
 
-    def step():
+    def step(rotate=True):
+        j = turn[0] if rotate else 0
+        old = ring[j]
+        if old is not None:
+            na_free(old[1].ptr)
+            na_free(old[2].ptr)
+            na_free(old[0].ptr)
+        dA, dr = descs[j]
         zc, zs, zm = NA(), NA(), NA()
         na_binary(b"add", ref(dA), ref(dr), ref(zc))
         na_reduce(b"sum", ref(zc), 2, 0, 0, ref(zs), None)
         na_reduce(b"max", ref(zc), 2, 0, 0, ref(zm), None)
-        na_free(zs.ptr)
-        na_free(zm.ptr)
-        na_free(zc.ptr)
+        ring[j] = (zc, zs, zm)
+        if rotate:
+            turn[0] = j + 1 if j + 1 < K else 0
 
-    # per-launch timing of the dominant kernel replays the recorded call of the add
-    with _lib.record() as add_calls:
-        ops[0][1](env)
+    def timed_steps(rotate):
+        for _ in range(max(args.warmup, K if rotate else 0)):
+            step(rotate)
+        _lib.check()
+        cumo_amd.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(rotate)
+        cumo_amd.synchronize()
+        dt = time.perf_counter() - t0
+        _lib.check()
+        return dt
 
-    for _ in range(args.warmup):
-        step()
-    _lib.check()
-    cumo_amd.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    cumo_amd.synchronize()
-    wall = time.perf_counter() - t0
-    _lib.check()
+    wall = timed_steps(True)
     ms_per_step = wall / args.steps * 1e3
     value = step_bytes / (wall / args.steps) / 1e9
+    wall_replay = timed_steps(False) if not args.rotated_only else None   # the same step on one set of buffers, back to back
+    for old in ring:
+        if old is not None:
+            for z in old:
+                na_free(z.ptr)
+    ring = None
 
     # the same step driven by the Python host mirror (descriptor building in
     # Python per op), for the record
-    def py_step():
-        for _, fn, _, _ in ops:
-            fn(env)
-    py_step()
+    def py_step(j):
+        e, o = sets[j % K]
+        for _, fn, _, _ in o:
+            fn(e)
+    for j in range(K):
+        py_step(j)
     cumo_amd.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        py_step()
+    for j in range(args.steps):
+        py_step(j)
     cumo_amd.synchronize()
     ms_per_step_python_host = (time.perf_counter() - t0) / args.steps * 1e3
 
     # dominant kernel, per launch: HIP events on the launch stream around batches of
-    # back-to-back launches
+    # launches that take turns over the K sets (rotated: sustained HBM) and around
+    # batches of the same launch on one set (replay: last-level cache helps)
+    add_sets = []
+    for e, o in sets:
+        with _lib.record() as add_calls:
+            o[0][1](e)
+        add_sets.append(add_calls)
     timer = Timer(lib)
     add_bytes = ops[0][2]
     batch = 10
-    ts = sorted(timer.time(lambda: _lib.replay(add_calls, batch)) / batch for _ in range(max(20, args.steps)))
+    pos = [0]
+
+    def rotated(times):
+        j = pos[0]
+        for _ in range(times):
+            for f, a in add_sets[j]:
+                f(*a)
+            j = j + 1 if j + 1 < K else 0
+        pos[0] = j
+
+    rotated(K)
+    ts = sorted(timer.time(lambda: rotated(batch)) / batch for _ in range(max(20, args.steps)))
+    avg_replay_ms = None
+    if not args.rotated_only:
+        _lib.replay(add_sets[0], 3)
+        tr = sorted(timer.time(lambda: _lib.replay(add_sets[0], batch)) / batch for _ in range(max(20, args.steps)))
+        avg_replay_ms = sum(tr) / len(tr)
     timer.close()
     avg_ms = sum(ts) / len(ts)
     achieved = add_bytes / (avg_ms * 1e-3) / 1e9
     roofline = {
-        "bound": "hbm", "kernel": "ew_rows2_kernel<OpAdd<double>, 2, false> (C = A + r, f64 4096x4096 + 1x4096)",
+        "bound": "hbm", "kernel": ADD_KERNEL + " (C = A + r, f64 4096x4096 + 1x4096)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
         "bytes_per_launch": int(add_bytes), "avg_launch_ms": round(avg_ms, 5), "median_launch_ms": round(ts[len(ts) // 2], 5),
-        "traffic": C2_ADD_TRAFFIC_BYTES,
+        "method": "launches take turns over %d operand/result sets (%.2f GiB between two uses of a buffer)" % (K, (K - 1) * add_bytes / 2**30),
+        "traffic": read_traffic_bytes(),
     }
-    env.clear()
+    if avg_replay_ms is not None:
+        roofline["frac_replay"] = round(add_bytes / (avg_replay_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        roofline["avg_launch_ms_replay"] = round(avg_replay_ms, 5)
+    del add_sets
+    for e, _ in sets:
+        e.clear()
+    del sets, env, ops
     cumo_amd.MemoryPool.free_all_blocks()
 
     if args.pmc_calibration:
@@ -471,16 +617,16 @@ def main():
 
     per_config = {}
     if not args.no_per_config:
-        names = [c for c in args.configs.split(",") if c] or ["c1", "c2", "c3", "c4", "c5", "c1_large", "c2_large", "c3_large", "next"]
+        names = [c for c in args.configs.split(",") if c] or ["c1", "c2", "c3", "c4", "c5", "c1_large", "c2_large", "c3_large", "next", "nmath"]
         iters, warm = (30, 5) if args.all_configs else (7, 2)
         for name in names:
-            per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm)}
+            per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm, not args.rotated_only)}
 
     out = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "ms_per_step_python_host": round(ms_per_step_python_host, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 5), "value_replay": round(step_bytes / (wall_replay / args.steps) / 1e9, 1) if wall_replay else None, "ms_per_step_python_host": round(ms_per_step_python_host, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64", "data": "synthetic",
-        "config": {"workload": WORKLOAD_TEXT["c2"], "bytes_per_step": int(step_bytes), "launches_per_step": 3,
+        "config": {"workload": WORKLOAD_TEXT["c2"], "rotation": "steps take turns over %d device copies of the inputs; results are released %d steps later" % (K, K), "bytes_per_step": int(step_bytes), "launches_per_step": 3,
                    "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "gelem_per_s": round(3 * 4096 * 4096 / (wall / args.steps) / 1e9, 2)},
         "roofline": roofline,
     }
