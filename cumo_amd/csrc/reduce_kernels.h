@@ -591,14 +591,23 @@ static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Im
 // pool and goes back right after the second launch is queued: the next owner
 // can only touch it from work queued later on the same stream
 // (reference: include/cumo/reduce_kernel.h:493-496).
+// With `fixed` the partial results of a split reduction go to the caller's device memory
+// instead (fixed->ptr, fixed->bytes): nothing is allocated or released, and a reduction
+// whose partial results do not fit is refused (returns false, nothing launched).
+struct RedScratch {
+    char* ptr;
+    size_t bytes;
+};
+
 template <class Impl>
-static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Impl impl, int index_mode) {
+static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Impl impl, int index_mode,
+                          const RedScratch* fixed = nullptr) {
     typedef typename Impl::In In;
     typedef typename Impl::Acc Acc;
-    if (arg->out_indexer.total_size == 0) return;  // reference: reduce_kernel.h:444-446
+    if (arg->out_indexer.total_size == 0) return true;  // reference: reduce_kernel.h:444-446
     ReducePlan plan;
     plan_reduce(arg, out2, (int)sizeof(In), (int)sizeof(Acc), &plan);
-    if (plan.kind == RED_EMPTY) return;
+    if (plan.kind == RED_EMPTY) return true;
     hipStream_t stream = current_stream();
     RedKParams kp;
     red_fill_params(&kp, plan, arg, out2, index_mode);
@@ -610,7 +619,7 @@ static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
         if (plan.kind == RED_COL) red_launch_col<Impl, false>(kp, plan.vec, impl, nullptr, stream);
         else red_launch_row<Impl, false>(kp, plan.vec, impl, nullptr, stream);
         cumo_cuda_runtime_check_kernel_launch();
-        return;
+        return true;
     }
 
     // first pass
@@ -624,8 +633,14 @@ static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     kp.n_split = (plan.red_total + chunk - 1) / chunk;
     kp.chunk = chunk;
     const uint64_t n_partial = plan.out_total * kp.n_split;
-    Acc* partial = reinterpret_cast<Acc*>(cumo_cuda_runtime_malloc(sizeof(Acc) * n_partial));
-    if (!partial) return;
+    Acc* partial;
+    if (fixed) {
+        if (sizeof(Acc) * n_partial > fixed->bytes) return false;
+        partial = reinterpret_cast<Acc*>(fixed->ptr);
+    } else {
+        partial = reinterpret_cast<Acc*>(cumo_cuda_runtime_malloc(sizeof(Acc) * n_partial));
+        if (!partial) return true;  // the pool has reported it
+    }
     if (plan.kind == RED_COL) red_launch_col<Impl, true>(kp, plan.vec, impl, partial, stream);
     else red_launch_row<Impl, true>(kp, plan.vec, impl, partial, stream);
     cumo_cuda_runtime_check_kernel_launch();
@@ -662,7 +677,8 @@ static void reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
         red_launch_row<CombineImpl<Impl>, false, true>(k2, 1, cimpl, nullptr, stream);
     }
     cumo_cuda_runtime_check_kernel_launch();
-    cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
+    if (!fixed) cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
+    return true;
 }
 
 }  // namespace cumo_hip

@@ -386,6 +386,24 @@ CUMO_HIP_DECL_REDUCE_PAIR(int32, minmax)
 CUMO_HIP_DECL_REDUCE_PAIR(sfloat, minmax_nan)
 CUMO_HIP_DECL_REDUCE_PAIR(dfloat, minmax_nan)
 
+/* The SFloat sum for callers that cannot allocate: code under stream capture, tight
+ * serving loops, harnesses that forbid hipMalloc. It has no counterpart in the
+ * reference, whose split reductions always take their scratch from the memory pool
+ * (include/cumo/reduce_kernel.h:493-496). Same descriptors, planner, kernels and
+ * result bits as cumo_sfloat_sum_kernel_launch, but the partial sums of a split
+ * reduction go to a fixed array of CUMO_HIP_NOALLOC_SCRATCH_BYTES that lives in the
+ * library's device image (each GPU the library runs on holds its own copy until the
+ * process ends); the call makes no hipMalloc / hipFree and does not touch the pool.
+ * Returns CUMO_HIP_OK, or CUMO_HIP_ERROR_ARGUMENT (also latched / handed to the error
+ * handler) without launching anything when the partial sums would not fit: a split
+ * reduction with more than CUMO_HIP_NOALLOC_SCRATCH_BYTES / 4 partial sums, i.e.
+ * outputs x chunks of the reduce axis. Every call on a GPU shares that GPU's array:
+ * calls that can overlap on one GPU (different streams or threads) race and must be
+ * serialised by the caller. Nothing in the array has to start at zero; it keeps the
+ * last call's partial sums. */
+#define CUMO_HIP_NOALLOC_SCRATCH_BYTES (256u << 10)
+int cumo_hip_sfloat_sum_noalloc_kernel_launch(cumo_na_reduction_arg_t* arg);
+
 /* ------------------------------------------------------------------------
  * 5. Bit launchers: narray/gen/tmpl_bit/binary_kernel.cu:1-52 (host
  *    tmpl_bit/binary.c:1-2), tmpl_bit/unary_kernel.cu (host tmpl_bit/unary.c),
