@@ -18,6 +18,17 @@ void report_hip_error(hipError_t status, const char* what);
 
 hipStream_t current_stream();
 
+// A number in [0, kStreamSlots) that belongs to this stream until it is destroyed
+// through cumo_hip_stream_destroy, or -1 when every number is taken. Kernels that
+// keep per-stream words in a fixed device array (tickets) index it with this.
+constexpr int kStreamSlots = 64;
+int stream_slot(hipStream_t stream);
+void stream_slot_release(hipStream_t stream);
+
+// Device address of the reduction ticket words of a stream slot (zero between launches),
+// nullptr after reporting an error. reduce_tickets.hip.
+uint32_t* red_ticket_words(int slot);
+
 // Stream capture (graph.cpp): while a capture is open, released memory stays with the
 // graph being recorded, and the pool hands blocks across streams without events.
 bool capture_defer_free(char* ptr);

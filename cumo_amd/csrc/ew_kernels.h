@@ -581,7 +581,10 @@ struct EwR2Params {
     int* flag;
 };
 
-template <class Op, int VEC, bool NT>
+// NTM: which accesses are non-temporal (bit 0 the first input, bit 1 the second, bit 2 the
+// result). An operand that repeats from row to row is the one thing worth keeping in
+// the caches, so it is read with plain loads while the full-size operands stream past.
+template <class Op, int VEC, int NTM>
 __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op, typename Op::S sv) {
     typedef typename Op::A A;
     typedef typename Op::B B;
@@ -618,7 +621,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
         if (NIN >= 1) {
             const char* a = p.ptr[0] + roff[0];
             if (p.walk[0]) {
-                raw_load<A, VEC, NT>(a + (uint64_t)cv * (VEC * sizeof(A)), xv);
+                raw_load<A, VEC, (NTM & 1) != 0>(a + (uint64_t)cv * (VEC * sizeof(A)), xv);
             } else {
                 const A v = *reinterpret_cast<const A*>(a);
 #pragma unroll
@@ -628,7 +631,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
         if (two_arrays) {
             const char* a = p.ptr[1] + roff[1];
             if (p.walk[1]) {
-                raw_load<B, VEC, NT>(a + (uint64_t)cv * (VEC * sizeof(B)), yv);
+                raw_load<B, VEC, (NTM & 2) != 0>(a + (uint64_t)cv * (VEC * sizeof(B)), yv);
             } else {
                 const B v = *reinterpret_cast<const B*>(a);
 #pragma unroll
@@ -652,7 +655,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
         char* o = p.ptr[2] + roff[2] + (uint64_t)cv * (VEC * sizeof(R));
         constexpr uint32_t full = (1u << VEC) - 1u;
         if (!Op::CHECKED || okmask == full) {
-            raw_store<R, VEC, NT>(o, zv);
+            raw_store<R, VEC, (NTM & 4) != 0>(o, zv);
         } else {
             if (p.flag) *p.flag = 1;
 #pragma unroll
@@ -1007,12 +1010,14 @@ static inline unsigned ew_grid_cap() {
 // Largest x extent of a grid.
 static inline uint64_t ew_grid_max() { return 0x7fffffffull; }
 
-// Non-temporal accesses once the bytes an operation touches exceed what the 256 MB
-// last-level cache can hold (measured: at 384 MiB and above they lift a streaming
-// operation from 74-78% of peak to 82-84%; at 256 MiB and below the default is
-// ahead by up to 8 points, because operands are still found in that cache).
+// Non-temporal accesses once an operation touches more than the caches could keep for
+// the next operation anyway. Measured with every launch on fresh operands (the state a
+// long computation is in): a 1R+1W operation over 2 x 128 MiB runs at 72-73% of the HBM
+// peak with plain accesses and 77-78% with non-temporal ones; no difference at 32 MiB.
+// (Launching the same operation on the same buffers again and again favours plain
+// accesses up to 256 MB, because the last-level cache then still holds the operands.)
 // CUMO_HIP_NT=0 / 1 forces them off / on.
-constexpr uint64_t kEwNtBytes = 320ull << 20;
+constexpr uint64_t kEwNtBytes = 48ull << 20;
 static inline int ew_nt_mode() {
     static int mode = -2;
     if (mode == -2) {
@@ -1282,13 +1287,34 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 if (grid > ew_grid_max()) grid = ew_grid_max();
                 if (heavy && grid > ew_grid_cap()) grid = ew_grid_cap();
                 const dim3 g((unsigned)grid);
-                if (vec == 4) {
-                    if (nt) hipLaunchKernelGGL((ew_rows2_kernel<Op, 4, true>), g, b, 0, stream, rp, op, sv);
-                    else hipLaunchKernelGGL((ew_rows2_kernel<Op, 4, false>), g, b, 0, stream, rp, op, sv);
-                } else {
-                    if (nt) hipLaunchKernelGGL((ew_rows2_kernel<Op, 2, true>), g, b, 0, stream, rp, op, sv);
-                    else hipLaunchKernelGGL((ew_rows2_kernel<Op, 2, false>), g, b, 0, stream, rp, op, sv);
+                // non-temporal for what streams past once; an operand that repeats along the rows stays cached
+                int ntm = 0;
+                if (nt) {
+                    ntm = 4;
+                    if (Op::NIN >= 1 && rp.walk[0] && rp.rstep[0] != 0 && (n == 2 || rp.ostep[0] != 0)) ntm |= 1;
+                    if (Op::NIN >= 2 && use_scalar == 0 && rp.walk[1] && rp.rstep[1] != 0 && (n == 2 || rp.ostep[1] != 0)) ntm |= 2;
                 }
+#define CUMO_R2_LAUNCH(V, M) hipLaunchKernelGGL((ew_rows2_kernel<Op, V, M>), g, b, 0, stream, rp, op, sv)
+#define CUMO_R2_BY_MASK(V)                                            \
+    do {                                                              \
+        bool done = false;                                            \
+        if constexpr (Op::NIN >= 2) {                                 \
+            if (ntm == 7) { CUMO_R2_LAUNCH(V, 7); done = true; }      \
+            else if (ntm == 6) { CUMO_R2_LAUNCH(V, 6); done = true; } \
+        }                                                             \
+        if (!done) {                                                  \
+            if (ntm == 5) CUMO_R2_LAUNCH(V, 5);                       \
+            else if (ntm == 4) CUMO_R2_LAUNCH(V, 4);                  \
+            else CUMO_R2_LAUNCH(V, 0);                                \
+        }                                                             \
+    } while (0);
+                if (vec == 4) {
+                    CUMO_R2_BY_MASK(4)
+                } else {
+                    CUMO_R2_BY_MASK(2)
+                }
+#undef CUMO_R2_BY_MASK
+#undef CUMO_R2_LAUNCH
                 cumo_cuda_runtime_check_kernel_launch();
                 return;
             }

@@ -217,6 +217,44 @@ struct MomentsImpl {
         }
         combine(Acc{(T)N, mb, m2}, acc);
     }
+    // U blocks of N at once: the same two passes over all U * N values, one merge (and one
+    // division) for all of them.
+    static constexpr bool GROUPED = true;
+    template <int U, int N>
+    __device__ __forceinline__ void accumulate_group(const T (&x)[U][N], const int64_t (&idx)[U], Acc& acc) const {
+        constexpr int M = U * N;
+        bool plain = (M & (M - 1)) != 0;
+        if (SKIP_NAN && !plain) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) plain = plain || maybe_nan<T, N>(x[u]);
+        }
+        if (plain) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) accumulate_n<N>(x[u], idx[u], acc);
+            return;
+        }
+        T part[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            part[u] = x[u][0];
+#pragma unroll
+            for (int k = 1; k < N; ++k) part[u] = part[u] + x[u][k];
+        }
+        T s = part[0];
+#pragma unroll
+        for (int u = 1; u < U; ++u) s = s + part[u];
+        const T mb = s * ((T)1 / (T)M);
+        T m2 = (T)0;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                const T d = x[u][k] - mb;
+                m2 = m2 + d * d;
+            }
+        }
+        combine(Acc{(T)M, mb, m2}, acc);
+    }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
         // every element NaN leaves no count; Numo answers +0 there (float_accum_kernel.cu:74-84)
         T v = (SKIP_NAN && acc.n == (T)0) ? (T)0 : acc.m2 / (acc.n - (T)1);

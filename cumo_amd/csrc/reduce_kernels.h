@@ -490,6 +490,12 @@ struct CombineImpl {
     __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const { impl.store(acc, out, out2); }
 };
 
+// Device memory a caller lends for the partial results of a split reduction.
+struct RedScratch {
+    char* ptr;
+    size_t bytes;
+};
+
 static inline unsigned red_grid_cap() {
     static unsigned cap = 0;
     if (cap == 0) {
@@ -524,7 +530,25 @@ static inline void red_fill_params(RedKParams* kp, const ReducePlan& plan, const
     kp->small = (arg->in_indexer.total_size < 0xffffffffull) ? 1 : 0;
 }
 
-constexpr uint64_t kRedNtBytes = 320ull << 20;
+// Inputs beyond this size are read with non-temporal loads: no cache level can hold them
+// until they are needed again, and keeping them out leaves the caches to what can be
+// (measured with every launch on fresh data: 128 MiB of SFloat summed at 76% of the HBM
+// peak with plain loads, 82% with non-temporal ones; no difference at 32 MiB).
+constexpr uint64_t kRedNtBytes = 48ull << 20;
+
+static inline int red_nt_mode() {
+    static int mode = -2;
+    if (mode == -2) {
+        const char* e = std::getenv("CUMO_HIP_NT");
+        mode = e ? (std::atoi(e) != 0 ? 1 : 0) : -1;
+    }
+    return mode;
+}
+
+static inline bool red_use_nt(uint64_t bytes) {
+    const int mode = red_nt_mode();
+    return mode < 0 ? bytes > kRedNtBytes : mode != 0;
+}
 
 template <class Impl, bool PARTIAL, bool SCALAR_ONLY = false>
 static void red_launch_row(const RedKParams& kp, int vec, Impl impl, typename Impl::Acc* partial, hipStream_t stream) {
@@ -537,7 +561,7 @@ static void red_launch_row(const RedKParams& kp, int vec, Impl impl, typename Im
     const dim3 g((unsigned)grid), b(kRedBlock);
     if constexpr (kMaxVec >= 2 && !SCALAR_ONLY) {
         // the widest access of an input too large for the last-level cache: non-temporal
-        if (vec == kMaxVec && kp.out_total * kp.red_total * sizeof(typename Impl::In) > kRedNtBytes) {
+        if (vec == kMaxVec && red_use_nt(kp.out_total * kp.red_total * sizeof(typename Impl::In))) {
             hipLaunchKernelGGL((red_row_kernel<Impl, kMaxVec, PARTIAL, true>), g, b, 0, stream, kp, impl, partial);
             return;
         }
@@ -572,7 +596,7 @@ static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Im
         return;
     }
     if constexpr (kMaxVec >= 2) {
-        if (vec == kMaxVec && kp.out_total * kp.red_total * sizeof(typename Impl::In) > kRedNtBytes) {
+        if (vec == kMaxVec && red_use_nt(kp.out_total * kp.red_total * sizeof(typename Impl::In))) {
             hipLaunchKernelGGL((red_col_kernel<Impl, kMaxVec, PARTIAL, true>), g, b, 0, stream, kp, impl, partial);
             return;
         }
@@ -586,6 +610,150 @@ static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Im
     hipLaunchKernelGGL((red_col_kernel<Impl, 1, PARTIAL>), g, b, 0, stream, kp, impl, partial);
 }
 
+}  // namespace cumo_hip
+
+#include "reduce_stream.h"
+
+namespace cumo_hip {
+
+static inline bool red_stream_enabled() {
+    static int on = -1;
+    if (on < 0) {
+        const char* e = std::getenv("CUMO_HIP_RED_STREAM");
+        on = (e && std::atoi(e) == 0) ? 0 : 1;
+    }
+    return on != 0;
+}
+
+// The lean kernels of reduce_stream.h for the layouts they take. Returns 1 when the
+// reduction has been launched, 0 when the general kernels must take it, -1 when the
+// caller's fixed scratch is too small (nothing launched).
+template <class Impl>
+static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Impl impl,
+                             int index_mode, const RedScratch* fixed, hipStream_t stream) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    constexpr int V = (int)(16 / sizeof(In));
+    if (!red_stream_enabled()) return 0;
+    if (plan.vec != V || plan.red_ndim != 1 || plan.red_total == 0 || plan.out_ndim > 2) return 0;
+    if (plan.out_total >= 0x7fffffffull) return 0;
+    if (plan.kind != RED_ROW && plan.kind != RED_COL) return 0;
+    {
+        static int force1 = -1;
+        if (force1 < 0) force1 = std::getenv("CUMO_HIP_FORCE_VEC1") ? 1 : 0;
+        if (force1) return 0;
+    }
+    RedSParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.in = arg->in.ptr;
+    p.out = arg->out.ptr;
+    p.out2 = out2 ? out2->ptr : nullptr;
+    p.n = plan.red_total;
+    p.red_step = plan.in_red_step[0];
+    p.n_out = (uint32_t)plan.out_total;
+    p.n_split = 1;
+    p.index_mode = index_mode;
+    if (plan.out_ndim == 2) {
+        p.out_inner = (uint32_t)plan.out_shape[1];
+        for (int d = 0; d < 2; ++d) {
+            p.in_step[d] = plan.in_out_step[d];
+            p.out_step[d] = plan.out_step[d];
+            p.out2_step[d] = plan.out2_step[d];
+        }
+    } else {
+        p.out_inner = p.n_out;
+        if (plan.out_ndim == 1) {
+            p.in_step[1] = plan.in_out_step[0];
+            p.out_step[1] = plan.out_step[0];
+            p.out2_step[1] = plan.out2_step[0];
+        }
+    }
+    const bool nt = red_use_nt(plan.out_total * plan.red_total * sizeof(In));
+    const dim3 b(kRedBlock);
+
+    if (plan.kind == RED_COL) {
+        if (plan.n_split > 1) return 0;
+        if (plan.in_out_step[plan.out_ndim - 1] != (int64_t)sizeof(In)) return 0;
+        p.lsplit_bits = (uint32_t)plan.local_split_bits;
+        const uint64_t per_block = (uint64_t)kRedBlock >> p.lsplit_bits;
+        uint64_t grid = (plan.out_total / V + per_block - 1) / per_block;
+        if (grid > red_grid_cap()) grid = red_grid_cap();
+        const dim3 g((unsigned)grid);
+        // four positions of the axis in flight per lane: more of them (or narrower blocks) read
+        // more rows at a time and measured slower
+        if (p.lsplit_bits > 0) {
+            if (nt) hipLaunchKernelGGL((red_scol_kernel<Impl, V, true, true, 4>), g, b, 0, stream, p, impl);
+            else hipLaunchKernelGGL((red_scol_kernel<Impl, V, false, true, 4>), g, b, 0, stream, p, impl);
+        } else {
+            if (nt) hipLaunchKernelGGL((red_scol_kernel<Impl, V, true, false, 4>), g, b, 0, stream, p, impl);
+            else hipLaunchKernelGGL((red_scol_kernel<Impl, V, false, false, 4>), g, b, 0, stream, p, impl);
+        }
+        cumo_cuda_runtime_check_kernel_launch();
+        return 1;
+    }
+
+    if (plan.in_red_step[0] != (int64_t)sizeof(In)) return 0;
+    p.tpr_bits = 0;
+    while ((1 << p.tpr_bits) < plan.threads_per_row) ++p.tpr_bits;
+    {
+        static int force_bits = -2;
+        if (force_bits == -2) {
+            const char* e = std::getenv("CUMO_HIP_RED_TPR_BITS");
+            force_bits = e ? std::atoi(e) : -1;
+        }
+        if (force_bits >= 0 && force_bits <= 8 && plan.n_split <= 1) p.tpr_bits = (uint32_t)force_bits;
+    }
+    if (plan.n_split <= 1) {
+        const uint64_t rpb = (uint64_t)kRedBlock >> p.tpr_bits;
+        uint64_t grid = (plan.out_total + rpb - 1) / rpb;
+        if (grid > red_grid_cap()) grid = red_grid_cap();
+        const dim3 g((unsigned)grid);
+        if (nt) hipLaunchKernelGGL((red_srow_kernel<Impl, V, true>), g, b, 0, stream, p, impl);
+        else hipLaunchKernelGGL((red_srow_kernel<Impl, V, false>), g, b, 0, stream, p, impl);
+        cumo_cuda_runtime_check_kernel_launch();
+        return 1;
+    }
+
+    // the axis cut over several blocks per output, one launch
+    // no more blocks than the axis has tiles (what a block loads in one step)
+    const uint64_t tile = (uint64_t)kRedBlock * V * kRsUnroll;
+    const uint64_t tiles = (plan.red_total + tile - 1) / tile;
+    p.n_split = (uint32_t)((uint64_t)plan.n_split < tiles ? (uint64_t)plan.n_split : tiles);
+    if (p.n_split <= 1) return 0;
+    p.group = p.n_split <= (uint32_t)kRsOneLevel ? p.n_split : (uint32_t)kRsGroup;
+    const uint64_t groups = (p.n_split + p.group - 1) / p.group;
+    {
+        static uint32_t stride = 0;
+        if (stride == 0) {
+            const char* e = std::getenv("CUMO_HIP_RED_TICKET_STRIDE");
+            stride = e ? (uint32_t)std::strtoul(e, nullptr, 10) : 0;
+            if (stride == 0) stride = 64;
+        }
+        p.tstride = stride;
+        while (p.tstride > 1 && plan.out_total * (1 + groups) * p.tstride > kRsTicketWords) p.tstride >>= 1;
+    }
+    if (plan.out_total * (1 + groups) * p.tstride > kRsTicketWords) return 0;
+    const uint64_t n_blocks = plan.out_total * p.n_split;
+    if (n_blocks > 0x7fffffffull) return 0;
+    p.tickets = red_ticket_words(stream_slot(stream));
+    if (p.tickets == nullptr) return 0;
+    const size_t scratch_bytes = sizeof(Acc) * (size_t)n_blocks;
+    if (fixed) {
+        if (scratch_bytes > fixed->bytes) return -1;
+        p.partial = fixed->ptr;
+    } else {
+        p.partial = cumo_cuda_runtime_malloc(scratch_bytes);
+        if (!p.partial) return 1;  // the pool has reported it
+    }
+    const dim3 g((unsigned)n_blocks);
+    if (nt) hipLaunchKernelGGL((red_srow_split_kernel<Impl, V, true>), g, b, 0, stream, p, impl);
+    else hipLaunchKernelGGL((red_srow_split_kernel<Impl, V, false>), g, b, 0, stream, p, impl);
+    cumo_cuda_runtime_check_kernel_launch();
+    // the next owner of the scratch can only touch it from work queued later on this stream
+    if (!fixed) cumo_cuda_runtime_free(p.partial);
+    return 1;
+}
+
 // index_mode: 1 for arg reductions, 2 for *_index reductions, ignored by impls
 // that do not use the index. The scratch of a split reduction comes from the
 // pool and goes back right after the second launch is queued: the next owner
@@ -594,11 +762,6 @@ static void red_launch_col(const RedKParams& kp, int vec, Impl impl, typename Im
 // With `fixed` the partial results of a split reduction go to the caller's device memory
 // instead (fixed->ptr, fixed->bytes): nothing is allocated or released, and a reduction
 // whose partial results do not fit is refused (returns false, nothing launched).
-struct RedScratch {
-    char* ptr;
-    size_t bytes;
-};
-
 template <class Impl>
 static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Impl impl, int index_mode,
                           const RedScratch* fixed = nullptr) {
@@ -609,6 +772,10 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     plan_reduce(arg, out2, (int)sizeof(In), (int)sizeof(Acc), &plan);
     if (plan.kind == RED_EMPTY) return true;
     hipStream_t stream = current_stream();
+    {
+        const int taken = red_stream_launch(plan, arg, out2, impl, index_mode, fixed, stream);
+        if (taken != 0) return taken > 0;
+    }
     RedKParams kp;
     red_fill_params(&kp, plan, arg, out2, index_mode);
     kp.tpr_bits = 0;

@@ -1,0 +1,414 @@
+// Lean reduction kernels for the layouts that carry nearly all the bytes: the
+// reduce axis is ONE run of elements (after merging), the outputs span at most two
+// dimensions, every access is a whole 128-bit vector and all totals fit 32 bits.
+// Included by reduce_kernels.h, which keeps the general kernels for everything else.
+//
+//  red_srow_kernel        the reduce axis runs along memory; 2^k lanes share an output.
+//  red_srow_split_kernel  the same with the axis cut over several blocks per output, in
+//                         ONE launch: every block leaves its accumulator in a scratch
+//                         array and counts in on a ticket; the block that counts in last
+//                         folds the accumulators of its output in index order. The order
+//                         of the fold does not depend on which block that is, so results
+//                         are the same bits on every run, as with a second launch.
+//  red_scol_kernel        the outputs run along memory; a lane owns VEC neighbouring
+//                         outputs and walks the axis; with LOCAL, 2^k lanes of a block
+//                         share the axis and combine through LDS in axis order.
+//
+// What makes them lean: a 136-byte argument block instead of 620 bytes; every load of
+// an unrolled step is unconditional (a position past the end is pulled back inside the
+// run and its value not used), so the four 128-bit loads of a lane are in flight
+// together; no per-element index decomposition at all; non-temporal loads for inputs
+// that no cache level could hold anyway.
+#ifndef CUMO_HIP_REDUCE_STREAM_H
+#define CUMO_HIP_REDUCE_STREAM_H
+
+namespace cumo_hip {
+
+constexpr int kRsUnroll = 4;            // 128-bit loads a lane keeps in flight
+constexpr int kRsGroup = 32;            // blocks that count in on one first-level ticket when an output has more than kRsOneLevel
+constexpr int kRsOneLevel = 128;        // up to this many blocks per output count in on a single ticket
+constexpr uint32_t kRsTicketWords = 16384;  // ticket words per stream slot
+
+struct RedSParams {
+    const char* in;
+    char* out;
+    char* out2;
+    uint64_t n;            // length of the reduce axis in elements
+    int64_t red_step;      // column form: byte step along the reduce axis
+    int64_t in_step[2];    // input byte steps over the (at most two) output dimensions, outer first
+    int64_t out_step[2];
+    int64_t out2_step[2];
+    uint32_t n_out;        // outputs
+    uint32_t out_inner;    // extent of the inner output dimension (= n_out when there is one dimension)
+    uint32_t n_split;      // split form: blocks per output
+    uint32_t group;        // split form: blocks that count in on one first-level ticket
+    uint32_t tstride;      // split form: words between two tickets (tickets in one cache line serialise in one memory channel)
+    uint32_t tpr_bits;     // row form: 2^tpr_bits lanes share an output
+    uint32_t lsplit_bits;  // column form: 2^lsplit_bits lanes of a block share an output group
+    int32_t index_mode;    // what accumulate() gets as idx: 1 = position along the axis, 2 = element offset from `in`
+    char* partial;         // split form: n_out * n_split accumulators
+    uint32_t* tickets;     // split form: n_out + n_out * ceil(n_split / group) words, zero between launches
+};
+
+template <class In, int VEC, bool NT>
+__device__ __forceinline__ void rs_load(const char* p, In (&x)[VEC]) {
+    static_assert(sizeof(In) * VEC == 16, "whole 128-bit vectors");
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    union V {
+        u4 q;
+        In v[VEC];
+        __device__ V() {}
+    } t;
+    if constexpr (NT) t.q = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+    else t.q = *reinterpret_cast<const u4*>(p);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) x[j] = t.v[j];
+}
+
+__device__ __forceinline__ void rs_split_out(const RedSParams& p, uint32_t o, uint32_t& o0, uint32_t& o1) {
+    if (p.out_inner == p.n_out) {
+        o0 = 0;
+        o1 = o;
+    } else {
+        o0 = o / p.out_inner;
+        o1 = o - o0 * p.out_inner;
+    }
+}
+
+// The 2^tpr_bits lanes of a group fold the tiles first, first + every, first + 2 * every, ...
+// of the run [0, end) (base = its element 0); a tile is what the group loads in one step,
+// kRsUnroll vectors per lane. end is a multiple of VEC. Every lane of the group runs the
+// same number of steps.
+template <class Impl, int VEC, bool NT>
+__device__ __forceinline__ typename Impl::Acc rs_row_scan(const Impl& impl, const char* base, uint64_t first, uint64_t every, uint64_t end,
+                                                          unsigned lane_r, unsigned tpr_bits, int64_t idx_base) {
+    typedef typename Impl::In In;
+    typename Impl::Acc acc = impl.identity();
+    const uint64_t stride = (uint64_t)VEC << tpr_bits;
+    const uint64_t per_step = stride * kRsUnroll;
+    const uint64_t tiles = (end + per_step - 1) / per_step;
+    if (first >= tiles) return acc;
+    const uint64_t steps = (tiles - first + every - 1) / every;
+    const uint64_t advance = per_step * every;
+    const uint64_t last = end - VEC;
+    uint64_t i0 = first * per_step + (uint64_t)lane_r * VEC;
+    for (uint64_t s = 0; s < steps; ++s, i0 += advance) {
+        In x[kRsUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kRsUnroll; ++u) {
+            const uint64_t i = i0 + (uint64_t)u * stride;
+            const uint64_t ic = i < end ? i : last;
+            rs_load<In, VEC, NT>(base + ic * sizeof(In), x[u]);
+        }
+        // every load of the step is issued before anything is folded (the scheduler would
+        // otherwise start folding the first vector and hold the later loads back behind it)
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (has_group<Impl>::value) {
+            if (i0 + (uint64_t)(kRsUnroll - 1) * stride < end) {
+                int64_t idx[kRsUnroll];
+#pragma unroll
+                for (int u = 0; u < kRsUnroll; ++u) idx[u] = idx_base + (int64_t)(i0 + (uint64_t)u * stride);
+                impl.template accumulate_group<kRsUnroll, VEC>(x, idx, acc);
+                continue;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRsUnroll; ++u) {
+            const uint64_t i = i0 + (uint64_t)u * stride;
+            if (i < end) impl.template accumulate_n<VEC>(x[u], idx_base + (int64_t)i, acc);
+        }
+    }
+    return acc;
+}
+
+// Lanes of one output combine; the group's first lane (thread 0 when a block shares the
+// output) ends up with everything, later lanes folded into earlier ones in a fixed order.
+template <class Impl>
+__device__ __forceinline__ void rs_group_combine(const Impl& impl, typename Impl::Acc& acc, unsigned tpr_bits,
+                                                 typename Impl::Acc* wave_slots) {
+    typedef typename Impl::Acc Acc;
+    const unsigned TPR = 1u << tpr_bits;
+    const unsigned span = TPR < 64 ? TPR : 64;
+    for (unsigned d = span >> 1; d > 0; d >>= 1) {
+        const Acc other = shfl_down_any(acc, d);
+        impl.combine(other, acc);
+    }
+    if (TPR > 64) {
+        if ((threadIdx.x & 63) == 0) wave_slots[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (unsigned w = 1; w < kRedBlock / 64; ++w) impl.combine(wave_slots[w], acc);
+        }
+        __syncthreads();
+    }
+}
+
+// scan + combine (+ the exact second fold where the impl asks for one)
+template <class Impl, int VEC, bool NT>
+__device__ __forceinline__ typename Impl::Acc rs_row_reduce(const Impl& impl, const char* base, uint64_t first, uint64_t every, uint64_t end,
+                                                            unsigned lane_r, unsigned tpr_bits, int64_t idx_base,
+                                                            typename Impl::Acc* wave_slots, int* s_need) {
+    typedef typename Impl::Acc Acc;
+    Acc acc = rs_row_scan<Impl, VEC, NT>(impl, base, first, every, end, lane_r, tpr_bits, idx_base);
+    rs_group_combine(impl, acc, tpr_bits, wave_slots);
+    if constexpr (has_exact<Impl>::value) {
+        const unsigned TPR = 1u << tpr_bits;
+        bool need;
+        if (TPR > 64) {
+            if (threadIdx.x == 0) *s_need = impl.needs_exact(acc) ? 1 : 0;
+            __syncthreads();
+            need = *s_need != 0;
+            __syncthreads();
+        } else {
+            const int mine = impl.needs_exact(acc) ? 1 : 0;
+            need = __shfl(mine, (int)((threadIdx.x & 63u) & ~(TPR - 1))) != 0;
+        }
+        if (need) {
+            typedef typename Impl::Exact Exact;
+            const Exact ex = impl.exact();
+            // the exact accumulator is wider: its own LDS slots
+            __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
+            typename Exact::Acc e = rs_row_scan<Exact, VEC, false>(ex, base, first, every, end, lane_r, tpr_bits, 0);
+            rs_group_combine(ex, e, tpr_bits, exact_slots);
+            acc = impl.from_exact(e);
+        }
+    }
+    return acc;
+}
+
+template <class Impl, int VEC, bool NT>
+__global__ __launch_bounds__(kRedBlock) void red_srow_kernel(RedSParams p, Impl impl) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    __shared__ Acc wave_slots[kRedBlock / 64];
+    __shared__ int s_need;
+    const unsigned TPR = 1u << p.tpr_bits;
+    const unsigned RPB = (unsigned)kRedBlock >> p.tpr_bits;
+    const unsigned lane_r = threadIdx.x & (TPR - 1);
+    const unsigned row_in_block = threadIdx.x >> p.tpr_bits;
+    const uint32_t n_rb = (p.n_out + RPB - 1) / RPB;
+    for (uint32_t rb = blockIdx.x; rb < n_rb; rb += gridDim.x) {
+        const uint32_t row = rb * RPB + row_in_block;
+        const bool ok = row < p.n_out;
+        uint32_t o0, o1;
+        rs_split_out(p, ok ? row : p.n_out - 1, o0, o1);
+        const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
+        const int64_t idx_base = p.index_mode == 2 ? in_off / (int64_t)sizeof(In) : 0;
+        const Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, 0, 1, p.n, lane_r, p.tpr_bits, idx_base, wave_slots, &s_need);
+        if (ok && lane_r == 0) {
+            const int64_t a = (int64_t)o0 * p.out_step[0] + (int64_t)o1 * p.out_step[1];
+            const int64_t b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)o1 * p.out2_step[1] : 0;
+            impl.store(acc, p.out + a, (Impl::NOUT > 1) ? (p.out2 + b) : nullptr);
+        }
+    }
+}
+
+// accumulators cross between blocks as 32-bit words written through to memory
+template <class Acc>
+__device__ __forceinline__ void rs_publish(char* dst, const Acc& acc) {
+    static_assert(sizeof(Acc) % 4 == 0, "accumulator must be a whole number of 32-bit words");
+    constexpr int W = sizeof(Acc) / 4;
+    union U {
+        Acc a;
+        uint32_t w[W];
+        __device__ U() {}
+    } u;
+    u.a = acc;
+#pragma unroll
+    for (int i = 0; i < W; ++i)
+        __hip_atomic_store(reinterpret_cast<uint32_t*>(dst) + i, u.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// read after the acquire fence of the block that counted in last: plain loads, all in flight together
+template <class Acc>
+__device__ __forceinline__ Acc rs_fetch(const char* src) {
+    return *reinterpret_cast<const Acc*>(src);
+}
+
+// One block per (output, chunk of the axis). blockIdx.x = output * n_split + chunk.
+template <class Impl, int VEC, bool NT>
+__global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p, Impl impl) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    __shared__ Acc wave_slots[kRedBlock / 64];
+    __shared__ int s_need;
+    __shared__ int s_last;
+    const uint32_t vrow = blockIdx.x;
+    const uint32_t i_out = vrow / p.n_split;
+    const uint32_t i_split = vrow - i_out * p.n_split;
+    uint32_t o0, o1;
+    rs_split_out(p, i_out, o0, o1);
+    const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
+    const int64_t idx_base = p.index_mode == 2 ? in_off / (int64_t)sizeof(In) : 0;
+    // the blocks of an output take its 16 KiB tiles in turn, so that together they read one window
+    // of the run at a time (memory sees a few long streams instead of n_split short ones)
+    Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, threadIdx.x, 8, idx_base, wave_slots, &s_need);
+
+    if (threadIdx.x == 0) {
+        // The accumulator is written through to memory and has arrived there before
+        // this block counts in. Blocks count in on their group's ticket; the last of a
+        // group counts in on the output's ticket; the last there finds every
+        // accumulator of the output in memory. Tickets go back to zero on the way.
+        rs_publish<Acc>(p.partial + (size_t)vrow * sizeof(Acc), acc);
+        __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0): the stores are acknowledged
+        const uint32_t groups = (p.n_split + p.group - 1) / p.group;
+        const uint32_t g = i_split / p.group;
+        const uint32_t g_size = (g + 1 == groups) ? p.n_split - g * p.group : p.group;
+        uint32_t* t1 = p.tickets + (size_t)(p.n_out + i_out * groups + g) * p.tstride;
+        uint32_t* t0 = p.tickets + (size_t)i_out * p.tstride;
+        int last = 0;
+        if (__hip_atomic_fetch_add(t1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g_size - 1) {
+            __hip_atomic_store(t1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (groups == 1) {
+                last = 1;  // one group: its last block is the output's last
+            } else if (__hip_atomic_fetch_add(t0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1) {
+                __hip_atomic_store(t0, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = 1;
+            }
+        }
+        s_last = last;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+
+    // fold the output's accumulators in index order: thread t takes chunks t, t + 256, ...
+    const char* mine = p.partial + (size_t)i_out * p.n_split * sizeof(Acc);
+    const int64_t o_a = (int64_t)o0 * p.out_step[0] + (int64_t)o1 * p.out_step[1];
+    const int64_t o_b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)o1 * p.out2_step[1] : 0;
+    if constexpr (has_exact<Impl>::value) {
+        // the accumulators are plain values in axis order: fold them with the exact rule
+        typedef typename Impl::Exact Exact;
+        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
+        const Exact ex = impl.exact();
+        __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
+        typename Exact::Acc e = ex.identity();
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), (int64_t)k, e);
+        rs_group_combine(ex, e, 8, exact_slots);
+        if (threadIdx.x == 0) impl.store(impl.from_exact(e), p.out + o_a, nullptr);
+    } else {
+        Acc total = impl.identity();
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), total);
+        rs_group_combine(impl, total, 8, wave_slots);
+        if (threadIdx.x == 0) impl.store(total, p.out + o_a, (Impl::NOUT > 1) ? (p.out2 + o_b) : nullptr);
+    }
+}
+
+// Column form. n_out is a multiple of VEC and so is out_inner.
+// U: positions of the axis a lane has in flight (more when the outputs alone give too few lanes
+// to keep the memory system busy: a block still reads 4 KiB runs of every row it touches).
+template <class Impl, int VEC, bool NT, bool LOCAL, int U>
+__global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl impl) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    __shared__ Acc part[LOCAL ? kRedBlock : 1][VEC];
+    const unsigned lbits = LOCAL ? p.lsplit_bits : 0u;
+    const unsigned SB = 1u << lbits;
+    const unsigned cbits = 8u - lbits;
+    const unsigned CPB = 1u << cbits;
+    const unsigned c = threadIdx.x & (CPB - 1);
+    const unsigned s = threadIdx.x >> cbits;
+    const uint32_t groups = p.n_out / VEC;
+    const uint32_t n_cb = (groups + CPB - 1) / CPB;
+    const uint64_t lchunk = (p.n + SB - 1) / SB;
+    uint64_t begin = (uint64_t)s * lchunk;
+    if (begin > p.n) begin = p.n;
+    uint64_t end = begin + lchunk;
+    if (end > p.n) end = p.n;
+
+    for (uint32_t cb = blockIdx.x; cb < n_cb; cb += gridDim.x) {
+        const uint32_t g = cb * CPB + c;
+        const bool ok = g < groups;
+        const uint32_t i_out0 = (ok ? g : groups - 1) * VEC;
+        uint32_t o0, o1;
+        rs_split_out(p, i_out0, o0, o1);
+        const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
+        const char* base = p.in + in_off;
+        Acc acc[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = impl.identity();
+        for (uint64_t i0 = begin; i0 < end; i0 += U) {
+            In x[U][VEC];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint64_t i = i0 + u;
+                const uint64_t ic = i < end ? i : end - 1;
+                rs_load<In, VEC, NT>(base + (int64_t)ic * p.red_step, x[u]);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // all loads of the step issued before the first fold
+            if (i0 + U <= end && p.index_mode != 2) {
+                // a whole block of consecutive positions along the axis for each output
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    In t[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) t[u] = x[u][j];
+                    impl.template accumulate_n<U>(t, (int64_t)i0, acc[j]);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint64_t i = i0 + u;
+                    if (i < end) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            int64_t idx = 0;
+                            if (Impl::USES_INDEX)
+                                idx = (p.index_mode == 2) ? ((in_off + (int64_t)i * p.red_step) / (int64_t)sizeof(In) + j) : (int64_t)i;
+                            impl.accumulate(x[u][j], idx, acc[j]);
+                        }
+                    }
+                }
+            }
+        }
+        if constexpr (has_exact<Impl>::value) {
+            // this lane walked its part of the axis in order, but its fast fold may have lost
+            // which of two equal elements came first: walk that output again, exactly
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if (impl.needs_exact(acc[j])) {
+                    typedef typename Impl::Exact Exact;
+                    const Exact ex = impl.exact();
+                    typename Exact::Acc e = ex.identity();
+                    for (uint64_t i = begin; i < end; ++i)
+                        ex.accumulate(*reinterpret_cast<const In*>(base + (int64_t)i * p.red_step + (int64_t)j * (int64_t)sizeof(In)), (int64_t)i, e);
+                    acc[j] = impl.from_exact(e);
+                }
+            }
+        }
+        if constexpr (LOCAL) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = acc[j];
+            __syncthreads();
+            if (s == 0) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    if constexpr (has_exact<Impl>::value) {
+                        // the parts are plain values in axis order: fold them with the exact rule
+                        typedef typename Impl::Exact Exact;
+                        const Exact ex = impl.exact();
+                        typename Exact::Acc e = ex.identity();
+                        for (unsigned k = 0; k < SB; ++k) ex.accumulate(part[k * CPB + c][j], (int64_t)k, e);
+                        acc[j] = impl.from_exact(e);
+                    } else {
+                        for (unsigned k = 1; k < SB; ++k) impl.combine(part[k * CPB + c][j], acc[j]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (ok && s == 0) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                // the VEC outputs of a group are neighbours along the inner output dimension
+                const int64_t a = (int64_t)o0 * p.out_step[0] + (int64_t)(o1 + j) * p.out_step[1];
+                const int64_t b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)(o1 + j) * p.out2_step[1] : 0;
+                impl.store(acc[j], p.out + a, (Impl::NOUT > 1) ? (p.out2 + b) : nullptr);
+            }
+        }
+    }
+}
+
+}  // namespace cumo_hip
+
+#endif

@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstring>
 #include <atomic>
+#include <mutex>
 
 namespace cumo_hip {
 
@@ -45,6 +46,33 @@ void report_hip_error(hipError_t status, const char* what) {
 
 hipStream_t current_stream() { return t_stream; }
 
+// Streams in use get a small number, for kernels that keep per-stream words in a
+// fixed device array (tickets that launches on different streams must not share).
+static std::mutex g_slot_lock;
+static hipStream_t g_slot_stream[kStreamSlots];
+static bool g_slot_used[kStreamSlots];
+
+int stream_slot(hipStream_t stream) {
+    std::lock_guard<std::mutex> hold(g_slot_lock);
+    int free_slot = -1;
+    for (int i = 0; i < kStreamSlots; ++i) {
+        if (g_slot_used[i] && g_slot_stream[i] == stream) return i;
+        if (!g_slot_used[i] && free_slot < 0) free_slot = i;
+    }
+    if (free_slot >= 0) {
+        g_slot_used[free_slot] = true;
+        g_slot_stream[free_slot] = stream;
+    }
+    return free_slot;
+}
+
+void stream_slot_release(hipStream_t stream) {
+    std::lock_guard<std::mutex> hold(g_slot_lock);
+    for (int i = 0; i < kStreamSlots; ++i) {
+        if (g_slot_used[i] && g_slot_stream[i] == stream) g_slot_used[i] = false;
+    }
+}
+
 }  // namespace cumo_hip
 
 using namespace cumo_hip;
@@ -79,6 +107,9 @@ void* cumo_hip_stream_create(void) {
 void cumo_hip_stream_destroy(void* hip_stream) {
     if (!hip_stream) return;
     if (t_stream == (hipStream_t)hip_stream) t_stream = nullptr;
+    // what the stream still has queued may use its slot's words: drain it first
+    hip_ok(hipStreamSynchronize((hipStream_t)hip_stream), "hipStreamSynchronize");
+    stream_slot_release((hipStream_t)hip_stream);
     hip_ok(hipStreamDestroy((hipStream_t)hip_stream), "hipStreamDestroy");
 }
 
