@@ -383,10 +383,29 @@ struct ArgImpl {
 #pragma unroll
                 for (int k = 0; k < N; ++k) m = IS_MAX ? max_skipping_nan<T>(m, x[u][k]) : min_skipping_nan<T>(m, x[u][k]);
             }
-            // false for a NaN on either side, which sends the blocks down the exact path
+            // false for a NaN on either side, which sends the blocks on
             if (IS_MAX ? (m <= acc.value) : (m >= acc.value)) {
                 if (is_float_t<T>::value || acc.index != kNone) return;
             }
+            if (!is_float_t<T>::value || !isnan_t(m)) {
+                // the group's extreme is a number: where it first occurs, without a branch
+                // (positions ascend with u, then k), then one merge. The value is taken from
+                // that position: of +0 and -0 the earlier counts.
+                IDX first = (IDX)idx[0];
+                T v = m;
+#pragma unroll
+                for (int u = U - 1; u >= 0; --u) {
+#pragma unroll
+                    for (int k = N - 1; k >= 0; --k) {
+                        const bool hit = x[u][k] == m;
+                        first = hit ? (IDX)(idx[u] + k) : first;
+                        v = hit ? x[u][k] : v;
+                    }
+                }
+                combine(Acc{v, first}, acc);
+                return;
+            }
+            // every element a NaN, or a signalling NaN poisoned m: the exact rule, block by block
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) accumulate_n<N>(x[u], idx[u], acc);

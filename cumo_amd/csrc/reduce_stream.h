@@ -277,15 +277,24 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
     const int64_t o_a = (int64_t)o0 * p.out_step[0] + (int64_t)o1 * p.out_step[1];
     const int64_t o_b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)o1 * p.out2_step[1] : 0;
     if constexpr (has_exact<Impl>::value) {
-        // the accumulators are plain values in axis order: fold them with the exact rule
+        // the accumulators are plain values in axis order: the fast fold first, and only where
+        // it cannot decide (which of two equal values came first) the exact rule over the same values
         typedef typename Impl::Exact Exact;
         static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
-        const Exact ex = impl.exact();
-        __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
-        typename Exact::Acc e = ex.identity();
-        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), (int64_t)k, e);
-        rs_group_combine(ex, e, 8, exact_slots);
-        if (threadIdx.x == 0) impl.store(impl.from_exact(e), p.out + o_a, nullptr);
+        Acc total = impl.identity();
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), total);
+        rs_group_combine(impl, total, 8, wave_slots);
+        if (threadIdx.x == 0) s_need = impl.needs_exact(total) ? 1 : 0;
+        __syncthreads();
+        if (s_need) {
+            const Exact ex = impl.exact();
+            __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
+            typename Exact::Acc e = ex.identity();
+            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), (int64_t)k, e);
+            rs_group_combine(ex, e, 8, exact_slots);
+            total = impl.from_exact(e);
+        }
+        if (threadIdx.x == 0) impl.store(total, p.out + o_a, nullptr);
     } else {
         Acc total = impl.identity();
         for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), total);
