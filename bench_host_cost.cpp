@@ -10,12 +10,36 @@
 //   add_issue           the host side alone: 1000 such calls queued, timed before the device has drained them
 //   add_alloc_free      the same with the result taken from and returned to the pool
 //   sum_alloc_free      cumo_hip_na_reduce("sum") likewise
+// Compiled with hipcc: the two do-nothing kernels live in this file, not in the library.
+#include <hip/hip_runtime.h>
+
 #include <chrono>
+#include <cstdint>
 #include <cstdio>
 #include <cstring>
 
 #include "cumo_hip.h"
 #include "cumo_hip_ndloop.h"
+
+// Kernels that do nothing, for what one launch costs on the library's current stream
+// (the floor under the per-operation cost of the host layer): one without arguments and
+// one that takes a kilobyte of them by value.
+struct Kilobyte {
+    uint64_t w[128];
+};
+__global__ void empty_kernel() {}
+__global__ void empty_kernel_1k(Kilobyte k, uint64_t* sink) {
+    if (sink) *sink = k.w[threadIdx.x & 127];  // never taken: sink is NULL
+}
+static void launch_empty_kernel(int with_arguments) {
+    hipStream_t st = (hipStream_t)cumo_hip_get_stream();
+    if (with_arguments) {
+        Kilobyte k = {};
+        hipLaunchKernelGGL(empty_kernel_1k, dim3(1), dim3(64), 0, st, k, (uint64_t*)nullptr);
+    } else {
+        hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, st);
+    }
+}
 
 static double now() { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
 
@@ -56,8 +80,8 @@ int main() {
     cumo_hip_narray_t* out[1] = {&z};
     cumo_hip_loop_t lp;
     const double prepare = us_per_call(200000, 3, [&] { cumo_hip_na_ndloop_prepare(&nf, in, out, 0, &lp); });
-    const double empty = us_per_call(N, 4, [&] { cumo_hip_launch_empty_kernel(0); });
-    const double empty_1k = us_per_call(N, 4, [&] { cumo_hip_launch_empty_kernel(1); });
+    const double empty = us_per_call(N, 4, [&] { launch_empty_kernel(0); });
+    const double empty_1k = us_per_call(N, 4, [&] { launch_empty_kernel(1); });
     cumo_na_indexer_t ix;
     cumo_na_iarray_t a1, a2, a3;
     cumo_hip_make_indexer(&lp, &ix);
@@ -90,7 +114,7 @@ int main() {
     // the same on a stream of its own instead of the null stream
     void* st = cumo_hip_stream_create();
     cumo_hip_set_stream(st);
-    const double empty_own = us_per_call(N, 4, [&] { cumo_hip_launch_empty_kernel(0); });
+    const double empty_own = us_per_call(N, 4, [&] { launch_empty_kernel(0); });
     const double add_own = us_per_call(N, 4, [&] { cumo_hip_na_binary("add", &x, &y, &z); });
     cumo_hip_set_stream(NULL);
     cumo_hip_stream_destroy(st);

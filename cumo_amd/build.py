@@ -23,7 +23,7 @@ HOST_COST_TOOL = os.path.join(HERE, "bench_host_cost")
 ARCH = "gfx950"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [
-    "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=default",
+    "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden", "-fvisibility-inlines-hidden",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
     "-Wall", "-Wno-unused-function", "-Wno-deprecated-declarations",
 ]
@@ -81,7 +81,8 @@ def build(jobs=None, force=False, verbose=True):
             objs.append(obj)
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o", LIB] + sorted(objs)
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=" + ARCH, "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"),
+           "-o", LIB] + sorted(objs)
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if p.returncode:
         print(p.stdout)
@@ -95,12 +96,12 @@ def build_host_cost_tool():
     src = os.path.join(ROOT, "bench_host_cost.cpp")
     if not os.path.exists(src):
         return
-    cmd = ["g++", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"), src, "-o", HOST_COST_TOOL,
-           "-L" + HERE, "-lcumo_hip", "-Wl,-rpath,$ORIGIN"]
+    cmd = [HIPCC, "-O2", "-std=c++17", "--offload-arch=" + ARCH, "-x", "hip", "-I" + os.path.join(ROOT, "include"), src,
+           "-o", HOST_COST_TOOL, "-L" + HERE, "-lcumo_hip", "-Wl,-rpath,$ORIGIN"]
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if p.returncode:
         print(p.stdout)
-        raise RuntimeError("bench_host_cost: g++ failed")
+        raise RuntimeError("bench_host_cost: hipcc failed")
 
 
 if __name__ == "__main__":

@@ -23,6 +23,10 @@
 #if defined(__cplusplus)
 extern "C" {
 #endif
+/* The library is built with hidden visibility; what this header declares is what it exports. */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 /* ------------------------------------------------------------------------
  * 1. Launch descriptors (reference: ext/cumo/include/cumo/indexer.h:16-68,
@@ -612,11 +616,6 @@ void* cumo_hip_event_create(void);
 void  cumo_hip_event_record(void* event);
 float cumo_hip_event_elapsed_ms(void* start, void* stop);   /* waits for stop */
 void  cumo_hip_event_destroy(void* event);
-/* launches a kernel that does nothing on the current stream, without arguments or with
- * a kilobyte of them by value (about what an elementwise launch passes): the floor
- * under the per-operation cost that bench_host_cost.cpp measures (no counterpart in
- * the reference) */
-void  cumo_hip_launch_empty_kernel(int with_arguments);
 /* synchronous copies for host read-back/ingest (extract_cpu, to_a, from_binary) */
 void  cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n);
 void  cumo_hip_memcpy_d2h(void* dst, const void* src, size_t n);
@@ -698,6 +697,9 @@ typedef struct {
 } cumo_hip_reduce_plan_t;
 int cumo_hip_plan_reduce(const cumo_na_reduction_arg_t* arg, int in_elmsz, int accum_bytes, cumo_hip_reduce_plan_t* plan);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #if defined(__cplusplus)
 }
 #endif

@@ -31,6 +31,9 @@
 #if defined(__cplusplus)
 extern "C" {
 #endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
 
 /* Element types on the path (reference: the classes of gen/def/{sfloat,dfloat,
  * int32,int64,uint64,bit}.rb). Int64/UInt64 only appear as results (Int32#sum,
@@ -273,6 +276,9 @@ int cumo_hip_na_bit_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_n
 /* count_true / count_false into a UInt64 result (reference: gen/tmpl_bit/bit_count.c:9-110). */
 int cumo_hip_na_bit_count(const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, int count_false, cumo_hip_narray_t* z);
 
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 #if defined(__cplusplus)
 }
 #endif

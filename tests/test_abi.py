@@ -63,6 +63,20 @@ def test_every_declared_symbol_is_exported():
     assert not missing, missing
 
 
+def test_nothing_but_the_declared_interface_is_exported():
+    """The library shares a process with Ruby and the extension: it must export the
+    C-ABI of the two headers and nothing else (no kernel stubs, no C++ internals,
+    no unprefixed helpers that another library's symbols could interpose)."""
+    from cumo_amd import _lib
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], check=True, stdout=subprocess.PIPE, text=True).stdout
+    exported = {line.split()[2] for line in out.splitlines() if len(line.split()) == 3}
+    assert exported, "nm found no exported symbols"
+    stray = sorted(n for n in exported if not n.startswith("cumo_"))
+    assert not stray, stray[:20]
+    undeclared = sorted(exported - set(declared_symbols()))
+    assert not undeclared, undeclared[:20]
+
+
 def test_expected_launcher_names_present():
     names = set(declared_symbols())
     for n in ["cumo_iter_sfloat_add_kernel_launch", "cumo_iter_sfloat_mul_s_kernel_launch", "cumo_iter_dfloat_math_s_exp_kernel_launch",
