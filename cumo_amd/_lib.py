@@ -207,6 +207,7 @@ _sig = {
     "cumo_hip_na_bit_binary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_bit_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_bit_count": (C.c_int, [P(NArrayDesc), C.c_uint, C.c_int, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_bit_reduce": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_uint, C.c_int, P(NArrayDesc)]),
 }
 for _name, (_res, _args) in _sig.items():
     _f = getattr(lib, _name)

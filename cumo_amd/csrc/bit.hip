@@ -8,8 +8,7 @@
 // popcount over whole words, reduced across the wave with shuffles and across
 // the block through LDS, and each block adds its total once. Integer addition
 // commutes, so the answer does not depend on the order the blocks arrive in.
-#include "common.h"
-#include "plan.h"
+#include "bit_common.h"
 
 #include <cstring>
 #include <mutex>
@@ -19,24 +18,9 @@ using namespace cumo_hip;
 
 namespace {
 
-constexpr int kBlock = 256;
-constexpr unsigned kGridCap = kNumCU * 8;
 // counting ends in one atomic add per block on a single word, so fewer, longer
 // blocks: one per compute unit
 constexpr unsigned kCountGridCap = kNumCU;
-
-__device__ __forceinline__ uint32_t low_bits(unsigned n) { return n >= 32 ? 0xffffffffu : ((1u << n) - 1u); }
-
-// 32 bits of `a` starting at absolute bit position q (q may be negative at the
-// front edge or run past the end; bits outside [0, 32*nw) read as 0)
-__device__ __forceinline__ uint32_t bits_at(const CUMO_BIT_DIGIT* a, int64_t q, uint64_t nw) {
-    const int64_t w = q >> 5;  // floor
-    const unsigned sh = (unsigned)(q & 31);
-    uint32_t lo = (w >= 0 && (uint64_t)w < nw) ? a[w] : 0u;
-    if (sh == 0) return lo;
-    uint32_t hi = (w + 1 >= 0 && (uint64_t)(w + 1) < nw) ? a[w + 1] : 0u;
-    return (lo >> sh) | (hi << (32 - sh));
-}
 
 enum { B_AND, B_OR, B_XOR, B_EQ, B_COPY, B_NOT };
 
@@ -71,40 +55,6 @@ __global__ __launch_bounds__(kBlock) void bit_contiguous_kernel(const CUMO_BIT_D
         if (mask == 0xffffffffu) a3[w] = z;
         else a3[w] = (z & mask) | (a3[w] & ~mask);
     }
-}
-
-struct BitNd {
-    int ndim;
-    uint64_t total;
-    uint64_t shape[kMaxDim];
-};
-
-// bit position / byte offset of flat element i of an operand that is strided or
-// indexed per dimension
-__device__ __forceinline__ int64_t stridx_offset(const cumo_stridx_t* sdx, const BitNd& nd, uint64_t i) {
-    int64_t off = 0;
-    for (int d = nd.ndim - 1; d >= 0; --d) {
-        uint64_t k;
-        if (d == 0) {
-            k = i;
-        } else {
-            const uint64_t q = i / nd.shape[d];
-            k = i - q * nd.shape[d];
-            i = q;
-        }
-        const cumo_stridx_t s = sdx[d];
-        if (s.stride & 1) off += (s.stride >> 1) * (int64_t)k;
-        else off += (int64_t)s.index[k];
-    }
-    return off;
-}
-
-__device__ __forceinline__ uint32_t load_bit(const CUMO_BIT_DIGIT* a, uint64_t pos) { return (a[pos >> 5] >> (pos & 31)) & 1u; }
-
-__device__ __forceinline__ void store_bit_atomic(CUMO_BIT_DIGIT* a, uint64_t pos, uint32_t v) {
-    const uint32_t bit = 1u << (pos & 31);
-    if (v) atomicOr(&a[pos >> 5], bit);
-    else atomicAnd(&a[pos >> 5], ~bit);
 }
 
 template <int OP, bool BINARY>
@@ -243,22 +193,6 @@ __global__ __launch_bounds__(kBlock) void bit_count_scatter_kernel(const CUMO_BI
         const uint32_t x = load_bit(a, pos);
         if (COUNT_FALSE ? (x == 0) : (x != 0)) *reinterpret_cast<uint64_t*>(p2 + (int64_t)i * s2) += 1;
     }
-}
-
-unsigned grid_for(uint64_t items, unsigned cap = kGridCap) {
-    uint64_t g = (items + kBlock - 1) / kBlock;
-    if (g > cap) g = cap;
-    if (g == 0) g = 1;
-    return (unsigned)g;
-}
-
-BitNd make_nd(const cumo_na_indexer_t* indexer) {
-    BitNd nd;
-    std::memset(&nd, 0, sizeof(nd));
-    nd.ndim = indexer->ndim;
-    nd.total = indexer->total_size;
-    for (int d = 0; d < indexer->ndim; ++d) nd.shape[d] = indexer->shape[d];
-    return nd;
 }
 
 template <int OP, bool BINARY>
@@ -442,11 +376,11 @@ CUMO_DEF_STORE_BIT(int32, int32_t)
 // the caller then zeroes the result and uses the accumulating launcher.
 extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, int count_false, uint64_t* out) {
     static std::mutex mu;
-    static std::unordered_map<hipStream_t, int> slot_of;
     static unsigned long long* tickets = nullptr;
     if (n == 0 || n >= (1ull << kTicketShift)) return 0;
     hipStream_t st = current_stream();
-    int slot;
+    const int slot = stream_slot(st);  // the stream's own ticket word; given back when the stream is destroyed
+    if (slot < 0 || slot >= kTicketSlots) return 0;
     {
         std::lock_guard<std::mutex> lk(mu);
         if (!tickets) {
@@ -457,12 +391,6 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
             }
             tickets = (unsigned long long*)p;
         }
-        auto it = slot_of.find(st);
-        if (it == slot_of.end()) {
-            if ((int)slot_of.size() >= kTicketSlots) return 0;
-            it = slot_of.emplace(st, (int)slot_of.size()).first;
-        }
-        slot = it->second;
     }
     // whole 128-bit vectors: move the word pointer back to a 16-byte boundary
     const uintptr_t back = ((uintptr_t)a & 15) / sizeof(CUMO_BIT_DIGIT);

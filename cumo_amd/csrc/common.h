@@ -25,6 +25,9 @@ constexpr int kStreamSlots = 64;
 int stream_slot(hipStream_t stream);
 void stream_slot_release(hipStream_t stream);
 
+// pool.cpp: files everything the pool holds for a drained stream under the null stream.
+void pool_retire_stream(hipStream_t stream);
+
 // Device address of the reduction ticket words of a stream slot (zero between launches),
 // nullptr after reporting an error. reduce_tickets.hip.
 uint32_t* red_ticket_words(int slot);

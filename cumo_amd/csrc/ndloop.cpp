@@ -428,6 +428,12 @@ typedef void (*StoreBitFn)(cumo_na_iarray_stridx_t*, cumo_na_bit_iarray_stridx_t
 const StoreBitFn kStoreBit[3] = {cumo_iter_sfloat_store_bit_kernel_launch, cumo_iter_dfloat_store_bit_kernel_launch,
                                  cumo_iter_int32_store_bit_kernel_launch};
 
+// number -> Bit, by source type code (sfloat dfloat int32 int64 uint64)
+typedef void (*BitStoreFromFn)(cumo_na_bit_iarray_stridx_t*, cumo_na_iarray_stridx_t*, IX*);
+const BitStoreFromFn kBitStoreFrom[5] = {cumo_iter_bit_store_sfloat_kernel_launch, cumo_iter_bit_store_dfloat_kernel_launch,
+                                         cumo_iter_bit_store_int32_kernel_launch, cumo_iter_bit_store_int64_kernel_launch,
+                                         cumo_iter_bit_store_uint64_kernel_launch};
+
 typedef void (*ReduceFn)(cumo_na_reduction_arg_t*);
 typedef void (*ReducePairFn)(cumo_na_reduction_arg_t*, IA*);
 struct ReduceRow {
@@ -685,6 +691,25 @@ void iter_store_bit(LP* lp) {  // args: dst (number), src (Bit)  (gen/tmpl/store
     cumo_hip_make_iarray_stridx(lp, 0, &a1);
     cumo_hip_make_bit_iarray_stridx(lp, 1, &a2);
     ((StoreBitFn)lp->opt_ptr)(&a1, &a2, &ix);
+}
+
+void iter_bit_store_from(LP* lp) {  // args: dst (Bit), src (number)  (gen/tmpl_bit/store_from.c:56-62)
+    BSX a1;
+    cumo_na_iarray_stridx_t a2;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_bit_iarray_stridx(lp, 0, &a1);
+    cumo_hip_make_iarray_stridx(lp, 1, &a2);
+    ((BitStoreFromFn)lp->opt_ptr)(&a1, &a2, &ix);
+}
+
+void iter_bit_fill(LP* lp) {  // args: dst (Bit); opt: the bit  (gen/tmpl_bit/fill.c:11-40)
+    BSX a3;
+    IX ix;
+    cumo_hip_make_indexer(lp, &ix);
+    cumo_hip_make_bit_iarray_stridx(lp, 0, &a3);
+    // the launcher itself takes the word-wise form for one run of step 1
+    cumo_iter_bit_fill_kernel_launch(&a3, *(const CUMO_BIT_DIGIT*)lp->opt_ptr, &ix);
 }
 
 void iter_copy_bytes(LP* lp) {  // args: src, dst  (narray/data.c:84-92)
@@ -1921,8 +1946,11 @@ int cumo_hip_na_store(cumo_hip_narray_t* dst, const cumo_hip_narray_t* src) {
     cumo_hip_ndfunc_t nf = {NULL, 0, 2, 0, {0, 0}};
     void* opt = NULL;
     StoreOpt sopt;
-    if (dst->type == CUMO_HIP_BIT) {
-        if (src->type != CUMO_HIP_BIT) return fail(CUMO_HIP_ERROR_TYPE, "store: only Bit can be stored into Bit on this path");
+    if (dst->type == CUMO_HIP_BIT && src->type != CUMO_HIP_BIT) {
+        if (src->type < 0 || src->type > CUMO_HIP_UINT64) return fail(CUMO_HIP_ERROR_TYPE, "store: unsupported source type");
+        nf.func = iter_bit_store_from;  // nonzero is 1 (types/bit_kernel.h:13-19)
+        opt = (void*)kBitStoreFrom[src->type];
+    } else if (dst->type == CUMO_HIP_BIT) {
         const BitUnaryRow* row = find_row(kBitUnary, "copy");
         nf.func = iter_bit_unary;  // args: src, dst
         opt = (void*)row;
@@ -2044,6 +2072,16 @@ int cumo_hip_na_extract(const cumo_hip_narray_t* x, const size_t* index, void* o
 }
 
 int cumo_hip_na_fill(cumo_hip_narray_t* dst, double value) {
+    if (dst && dst->type == CUMO_HIP_BIT) {
+        int rcb = check_view(dst, "destination");
+        if (rcb) return rcb;
+        // reference: gen/tmpl_bit/fill.c:27-36
+        if (value != 0.0 && value != 1.0) return fail(CUMO_HIP_ERROR_ARGUMENT, "invalid value for Bit");
+        CUMO_BIT_DIGIT y = value != 0.0 ? ~(CUMO_BIT_DIGIT)0 : 0;
+        cumo_hip_ndfunc_t nfb = {iter_bit_fill, 0, 1, 0, {0, 0}};
+        const NA* inb[1] = {dst};
+        return cumo_hip_na_ndloop(&nfb, inb, NULL, 0, &y);
+    }
     int rc = check_arith(dst);
     if (rc) return rc;
     FillOpt opt = {value};
@@ -2244,6 +2282,71 @@ int cumo_hip_na_bit_count(const cumo_hip_narray_t* x, unsigned int reduce, int k
     lp.opt_ptr = &opt;
     iter_bit_count(&lp);
     return lp.status;
+}
+
+// all? / any? along axes into a Bit result (reference: gen/tmpl_bit/bit_reduce.c:5-146). The
+// result starts out as the init bit (1 for all?, 0 for any?) and the launchers flip it. The
+// reference walks every dimension but the innermost on the host and launches once per run;
+// so does this for up to 32 runs. With more runs it takes the counts along the same axes
+// instead (one launch, whatever the shape): any? = (count_true != 0), all? = !(count_false != 0).
+int cumo_hip_na_bit_reduce(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, cumo_hip_narray_t* z) {
+    int rc = check_view(x, "operand");
+    if (rc) return rc;
+    if (!op || (std::strcmp(op, "all_p") != 0 && std::strcmp(op, "any_p") != 0)) return no_method(op ? op : "(null)");
+    const bool all = op[1] == 'l';
+    if (x->type != CUMO_HIP_BIT) return no_method(all ? "all?" : "any?");
+    if (x->ndim < 32 && (reduce >> x->ndim)) return fail(CUMO_HIP_ERROR_DIMENSION, "dimension is out of range");
+    if (!reduce) reduce = all_dims(x);
+    const unsigned flag = CUMO_HIP_NDF_FLAT_REDUCE | (keepdims ? CUMO_HIP_NDF_KEEP_DIM : 0u);
+    cumo_hip_ndfunc_t nf = {NULL, flag, 1, 1, {CUMO_HIP_BIT, 0}};
+    const NA* in[1] = {x};
+    NA* out[1] = {z};
+    cumo_hip_loop_t lp;
+    rc = cumo_hip_na_ndloop_prepare(&nf, in, out, reduce, &lp);
+    if (rc) return rc;
+    if (total_of(z) == 0) return CUMO_HIP_OK;
+    rc = cumo_hip_na_fill(z, all ? 1.0 : 0.0);
+    if (rc || total_of(x) == 0) return rc;
+
+    size_t runs = 1;
+    for (int d = 0; d + 1 < lp.ndim; d++) runs *= lp.n[d];
+    if (lp.ndim == 0 || runs > 32) {
+        NA counts;
+        std::memset(&counts, 0, sizeof(counts));
+        rc = cumo_hip_na_bit_count(x, reduce, keepdims, all ? 1 : 0, &counts);
+        if (!rc) rc = cumo_hip_na_store(z, &counts);  // nonzero -> 1
+        free_tmp(&counts);
+        if (!rc && all) rc = cumo_hip_na_bit_unary("not", z, z);
+        return rc;
+    }
+    CUMO_BIT_DIGIT* a1 = (CUMO_BIT_DIGIT*)lp.args[0].ptr;
+    CUMO_BIT_DIGIT* a2 = (CUMO_BIT_DIGIT*)lp.args[1].ptr;
+    const int last = lp.ndim - 1;
+    const ssize_t s1 = lp.args[0].step[last], s2 = lp.args[1].step[last];
+    const uint64_t n = lp.n[last];
+    size_t idx[CUMO_NA_MAX_DIMENSION] = {0};
+    for (size_t r = 0; r < runs; r++) {
+        ssize_t p1 = (ssize_t)lp.args[0].bitpos, p2 = (ssize_t)lp.args[1].bitpos;
+        for (int d = 0; d < last; d++) {
+            p1 += (ssize_t)idx[d] * lp.args[0].step[d];
+            p2 += (ssize_t)idx[d] * lp.args[1].step[d];
+        }
+        if (s2 != 0) {
+            if (all) cumo_iter_bit_all_p_elementwise_kernel_launch(a1, (size_t)p1, s1, NULL, a2, (size_t)p2, s2, NULL, n);
+            else cumo_iter_bit_any_p_elementwise_kernel_launch(a1, (size_t)p1, s1, NULL, a2, (size_t)p2, s2, NULL, n);
+        } else if (s1 == 1) {
+            if (all) cumo_iter_bit_all_p_contiguous_reduce_kernel_launch(a1, (size_t)p1, a2, (size_t)p2, n);
+            else cumo_iter_bit_any_p_contiguous_reduce_kernel_launch(a1, (size_t)p1, a2, (size_t)p2, n);
+        } else {
+            if (all) cumo_iter_bit_all_p_reduce_kernel_launch(a1, (size_t)p1, s1, NULL, a2, (size_t)p2, n);
+            else cumo_iter_bit_any_p_reduce_kernel_launch(a1, (size_t)p1, s1, NULL, a2, (size_t)p2, n);
+        }
+        for (int d = last - 1; d >= 0; d--) {
+            if (++idx[d] < lp.n[d]) break;
+            idx[d] = 0;
+        }
+    }
+    return CUMO_HIP_OK;
 }
 
 }  // extern "C"

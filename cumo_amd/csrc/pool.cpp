@@ -243,6 +243,29 @@ void read_env() {
 }
 
 }  // namespace
+
+// A stream that is about to be destroyed (and has been drained): every chunk filed under
+// it, free or in use, moves to the null stream's arena, so that nothing stays keyed by a
+// dead handle (its free chunks could never be reused or ordered against otherwise).
+void pool_retire_stream(hipStream_t stream) {
+    if (stream == nullptr) return;
+    Pool& p = g_pool;
+    std::unique_lock<std::mutex> lock(p.mu);
+    std::vector<Chunk*> moved;
+    auto a = p.arenas.find(stream);
+    if (a != p.arenas.end()) {
+        for (auto& e : a->second) moved.push_back(e.second);
+    }
+    for (Chunk* c : moved) {
+        p.arena_erase(c);
+        c->stream = nullptr;
+        p.arena_insert(c);
+    }
+    for (auto& kv : p.in_use) {
+        if (kv.second->stream == stream) kv.second->stream = nullptr;
+    }
+}
+
 }  // namespace cumo_hip
 
 using namespace cumo_hip;
@@ -266,7 +289,7 @@ int cumo_hip_pool_malloc(size_t size, void* hip_stream, void** out) {
         if (c && !p.host_backend && !capture_active()) {
             // everything queued so far on the giving stream must finish before
             // work queued from now on the taking stream touches the chunk
-            hipEvent_t ev;
+            hipEvent_t ev = nullptr;
             bool ok = hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess;
             ok = ok && hipEventRecord(ev, from) == hipSuccess;
             ok = ok && hipStreamWaitEvent(stream, ev, 0) == hipSuccess;

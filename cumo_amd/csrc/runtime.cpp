@@ -110,6 +110,7 @@ void cumo_hip_stream_destroy(void* hip_stream) {
     // what the stream still has queued may use its slot's words: drain it first
     hip_ok(hipStreamSynchronize((hipStream_t)hip_stream), "hipStreamSynchronize");
     stream_slot_release((hipStream_t)hip_stream);
+    pool_retire_stream((hipStream_t)hip_stream);
     hip_ok(hipStreamDestroy((hipStream_t)hip_stream), "hipStreamDestroy");
 }
 

@@ -920,6 +920,15 @@ class Bit(NArray):
 
     @classmethod
     def cast(cls, data):
+        """Bit.cast(array): nonzero is 1. An array on the device is stored by the number -> Bit
+        launcher (reference: gen/tmpl_bit/store_from.c); host data is packed into a staging
+        buffer, bit 0 first, and placed by the store_array launcher, as the reference does for
+        a Ruby Array (gen/tmpl_bit/store_array.c:60-113)."""
+        if isinstance(data, NArray):
+            a = cls(*data.shape)
+            if data.size:
+                a.store(data)
+            return a
         arr = np.ascontiguousarray(np.asarray(data) != 0)
         a = cls(*arr.shape)
         n = arr.size
@@ -927,7 +936,14 @@ class Bit(NArray):
             bits = np.packbits(arr.reshape(-1), bitorder="little")
             words = np.zeros(((n + 31) // 32) * 4, dtype=np.uint8)
             words[:bits.size] = bits
-            call(_L.cumo_hip_copy_from_host, a._buf.ptr, words.ctypes.data, words.nbytes)
+            stage = call(_L.cumo_cuda_runtime_malloc, words.nbytes)
+            try:
+                call(_L.cumo_hip_copy_from_host, stage, words.ctypes.data, words.nbytes)
+                f = _lib.fn("cumo_iter_bit_store_array_contiguous_kernel_launch", None,
+                            [C.c_void_p, C.c_size_t, C.c_void_p, C.c_uint64])
+                call(f, a._buf.ptr, a._offset, stage, n)
+            finally:
+                _L.cumo_cuda_runtime_free(stage)   # stream ordered: the launch above is already queued
         return a
 
     from_numpy = cast
@@ -952,7 +968,14 @@ class Bit(NArray):
         return int(NArray.aref_cpu(self, *index))
 
     def fill(self, value):
-        raise TypeError("Bit#fill is outside this path")
+        """reference: gen/tmpl_bit/fill.c:11-58 -- 0 / 1 / false / true, anything else is an ArgumentError."""
+        if value is True or value is False:
+            value = int(value)
+        if not isinstance(value, numbers.Number) or value not in (0, 1):
+            raise ValueError("invalid value for Bit")
+        d = self._desc()
+        _run(_L.cumo_hip_na_fill, C.byref(d), float(value))
+        return self
 
     def _bit_op2(self, other, op):
         if not isinstance(other, Bit):
@@ -1006,17 +1029,27 @@ class Bit(NArray):
         r = self.count_true()
         return int(r) if not isinstance(r, int) else r
 
-    # all? / any? / none? over the whole array (reference: gen/tmpl_bit/all_p.c, any_p.c,
-    # none_p.c; their per-axis forms, which answer Bit arrays, are outside this path).
-    # One count on the device, one value read back.
-    def all_p(self):
-        return self.size == 0 or int(self.count_false()) == 0
+    # all? / any? / none? (reference: gen/tmpl_bit/bit_reduce.c:106-146, none_p.c; spec.rb:185-186).
+    # Without axis the answer is true / false, read back from a one-bit result; with axis it is
+    # a Bit array. An empty array answers false (bit_reduce.c:132-134).
+    def _bit_reduce(self, op, axis, keepdims):
+        if self.size == 0:
+            return False
+        x, z = self._desc(), NArrayDesc()
+        r = _run(_L.cumo_hip_na_bit_reduce, op, C.byref(x), _reduce_mask(self.ndim, axis), int(bool(keepdims)), C.byref(z), results=(z,))
+        if axis is None and not keepdims:
+            return bool(r.extract_cpu())
+        return r
 
-    def any_p(self):
-        return self.size != 0 and int(self.count_true()) != 0
+    def all_p(self, axis=None, keepdims=False):
+        return self._bit_reduce(b"all_p", axis, keepdims)
 
-    def none_p(self):
-        return not self.any_p()
+    def any_p(self, axis=None, keepdims=False):
+        return self._bit_reduce(b"any_p", axis, keepdims)
+
+    def none_p(self, axis=None, keepdims=False):
+        r = self.any_p(axis, keepdims)
+        return (not r) if isinstance(r, bool) else ~r
 
     def _store_into(self, cls):
         """Bit -> 0/1 numbers (reference: gen/tmpl/store_bit.c)."""

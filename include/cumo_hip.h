@@ -345,6 +345,20 @@ CUMO_HIP_DECL_MULSUM(int32, mulsum)
     void cumo_iter_##dst##_store_##src##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer);
 CUMO_HIP_STORE_PAIRS(CUMO_HIP_DECL_STORE)
 
+/* The same-type store between views that may carry index arrays
+ * (narray/gen/tmpl/store_from_kernel.cu:19-35, host store_from.c:5,82), and the ingest of a
+ * host Array staged in device memory (narray/gen/tmpl/store_array_kernel.cu:2-60, host
+ * store_array.c:2-5): element i of the run goes to p1 + idx1[i] or p1 + i*s1 (bytes). */
+#define CUMO_HIP_DECL_STORE_STRIDX(t, c) \
+    void cumo_iter_##t##_store_##t##_stridx_kernel_launch(cumo_na_iarray_stridx_t* a1, cumo_na_iarray_stridx_t* a2, cumo_na_indexer_t* indexer); \
+    void cumo_iter_##t##_store_array_index_kernel_launch(char *p1, size_t *idx1, c* z, uint64_t n); \
+    void cumo_iter_##t##_store_array_stride_kernel_launch(char *p1, ssize_t s1, c* z, uint64_t n); \
+    void cumo_iter_##t##_store_array_index_scalar_kernel_launch(char *p1, size_t *idx1, c z, uint64_t n); \
+    void cumo_iter_##t##_store_array_stride_scalar_kernel_launch(char *p1, ssize_t s1, c z, uint64_t n);
+CUMO_HIP_DECL_STORE_STRIDX(sfloat, float)
+CUMO_HIP_DECL_STORE_STRIDX(dfloat, double)
+CUMO_HIP_DECL_STORE_STRIDX(int32, int32_t)
+
 /* copy of any view, a1 = source, a2 = destination:
  * narray/data_kernel.cu:47-132, host narray/data.c:56,84-92 */
 void cumo_iter_copy_bytes_indexer_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2, cumo_na_indexer_t* indexer, ssize_t elmsz);
@@ -433,6 +447,42 @@ CUMO_HIP_BIT_BINARY_OPS(CUMO_HIP_DECL_BIT_BINARY)
 CUMO_HIP_BIT_UNARY_OPS(CUMO_HIP_DECL_BIT_UNARY)
 CUMO_HIP_DECL_BIT_COUNT(count_true)
 CUMO_HIP_DECL_BIT_COUNT(count_false)
+
+/* all? / any? (narray/gen/tmpl_bit/bit_reduce_kernel.cu:5-77, host tmpl_bit/bit_reduce.c:1-3;
+ * spec.rb:185-186). The result bits start out as 1 (all?) or 0 (any?) -- ndloop fills them
+ * with the init value -- and an element that differs flips its result bit; nothing flips it
+ * back. elementwise: element i answers result bit p2 + i*s2 (or p2 + idx2[i]); reduce: every
+ * element of a strided or indexed run answers the one bit p2; contiguous_reduce: the same for
+ * a run of step 1, compared a word at a time. */
+#define CUMO_HIP_DECL_BIT_REDUCE(name) \
+    void cumo_iter_bit_##name##_elementwise_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, ssize_t s1, size_t *idx1, CUMO_BIT_DIGIT *a2, size_t p2, ssize_t s2, size_t *idx2, uint64_t n); \
+    void cumo_iter_bit_##name##_reduce_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, ssize_t s1, size_t *idx1, CUMO_BIT_DIGIT *a2, size_t p2, uint64_t n); \
+    void cumo_iter_bit_##name##_contiguous_reduce_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, CUMO_BIT_DIGIT *a2, size_t p2, uint64_t n);
+CUMO_HIP_DECL_BIT_REDUCE(all_p)
+CUMO_HIP_DECL_BIT_REDUCE(any_p)
+
+/* Bit#fill (narray/gen/tmpl_bit/fill_kernel.cu:2-46, host tmpl_bit/fill.c:1-2): y is 0 or all
+ * ones for the contiguous form (a3 = first word of the run, p3 = bit offset in it), its lowest
+ * bit for the general form. */
+void cumo_iter_bit_fill_kernel_launch(cumo_na_bit_iarray_stridx_t* a3, CUMO_BIT_DIGIT y, cumo_na_indexer_t* indexer);
+void cumo_iter_bit_fill_contiguous_kernel_launch(CUMO_BIT_DIGIT *a3, size_t p3, uint64_t n, CUMO_BIT_DIGIT y);
+
+/* number -> Bit, nonzero is 1 (narray/gen/tmpl_bit/store_from_kernel.cu:3-29, host
+ * tmpl_bit/store_from.c:2; element rule include/cumo/types/bit_kernel.h:13-19). a1 is the
+ * destination. */
+#define CUMO_HIP_BIT_STORE_SOURCES(X) X(sfloat) X(dfloat) X(int32) X(int64) X(uint64)
+#define CUMO_HIP_DECL_BIT_STORE_FROM(t) \
+    void cumo_iter_bit_store_##t##_kernel_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_iarray_stridx_t* a2, cumo_na_indexer_t* indexer);
+CUMO_HIP_BIT_STORE_SOURCES(CUMO_HIP_DECL_BIT_STORE_FROM)
+
+/* Ingest of a host Array staged in device memory, Bit destination
+ * (narray/gen/tmpl_bit/store_array_kernel.cu:2-95, host tmpl_bit/store_array.c:1-5): z is a
+ * packed buffer whose bit 0 is the run's first element, or one value for the scalar forms. */
+void cumo_iter_bit_store_array_index_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, size_t *idx1, CUMO_BIT_DIGIT* z, uint64_t n);
+void cumo_iter_bit_store_array_stride_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, ssize_t s1, CUMO_BIT_DIGIT* z, uint64_t n);
+void cumo_iter_bit_store_array_contiguous_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, CUMO_BIT_DIGIT* z, uint64_t n);
+void cumo_iter_bit_store_array_index_scalar_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, size_t *idx1, CUMO_BIT_DIGIT z, uint64_t n);
+void cumo_iter_bit_store_array_stride_scalar_kernel_launch(CUMO_BIT_DIGIT *a1, size_t p1, ssize_t s1, CUMO_BIT_DIGIT z, uint64_t n);
 
 /* Bit#where / Bit#mask compaction: narray/gen/tmpl_bit/where_kernel.cu:83-107 (host
  * tmpl_bit/where.c:10-11) and tmpl_bit/mask_kernel.cu:36-54. The scratch holds two

@@ -275,6 +275,10 @@ int cumo_hip_na_bit_binary(const char* op, const cumo_hip_narray_t* x, const cum
 int cumo_hip_na_bit_unary(const char* op, const cumo_hip_narray_t* x, cumo_hip_narray_t* z);
 /* count_true / count_false into a UInt64 result (reference: gen/tmpl_bit/bit_count.c:9-110). */
 int cumo_hip_na_bit_count(const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, int count_false, cumo_hip_narray_t* z);
+/* all? / any? along axes into a Bit result; op is "all_p" or "any_p" (reference:
+ * gen/tmpl_bit/bit_reduce.c:106-146, spec.rb:185-186). An empty operand leaves the init value
+ * (the reference's method answers false for it before the loop, bit_reduce.c:132-134). */
+int cumo_hip_na_bit_reduce(const char* op, const cumo_hip_narray_t* x, unsigned int reduce, int keepdims, cumo_hip_narray_t* z);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop
