@@ -10,11 +10,25 @@
 #ifndef CUMO_HIP_EW_OPS_H
 #define CUMO_HIP_EW_OPS_H
 
+// CUMO_HIP_HOST_CHECK: a CPU build of the element functions, for tests that run the
+// float algorithms below on the host against reference values. The including file then
+// supplies __device__, __forceinline__ and the bit-cast intrinsics.
+#ifndef CUMO_HIP_HOST_CHECK
 #include <hip/hip_runtime.h>
+#endif
 #include <stdint.h>
 #include <float.h>
 
 namespace cumo_hip {
+
+// 1 / x to about one ulp (v_rcp_f32); only used where that is more than enough
+__device__ __forceinline__ float rcp_approx(float x) {
+#ifdef CUMO_HIP_HOST_CHECK
+    return 1.0f / x;
+#else
+    return __builtin_amdgcn_rcpf(x);
+#endif
+}
 
 #define CUMO_HIP_OP_COMMON(TA, TB, TR, NIN_, BIT_, CHK_) \
     typedef TA A; typedef TB B; typedef TR R; typedef TA S; \
@@ -269,7 +283,7 @@ __device__ __forceinline__ float expm1_float_rounded_once(float xf) {
 __device__ __forceinline__ double log1p_core(double u) {
     const double w = 1.0 + u;
     const double c = u - (w - 1.0);
-    return __builtin_fma(c, (double)__builtin_amdgcn_rcpf((float)w), log_core<0>(w));
+    return __builtin_fma(c, (double)rcp_approx((float)w), log_core<0>(w));
 }
 __device__ __forceinline__ float asinh_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);

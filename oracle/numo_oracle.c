@@ -20,17 +20,19 @@
  *   - addressing / broadcast                   : brute force vs numpy
  *     as_strided.
  *   - sum/mean/var/stddev/rms                  : closed forms, exact rational
- *     arithmetic and literals held by the reference tests; the float f_*
- *     loops are also checked against the reference's own real_accum.h
- *     compiled as oracle/_ref.
+ *     arithmetic and literals held by the reference tests.
  *   - min/max/argmin/argmax (NaN, ties, +-0)   : enumerated cases from the
- *     reference tests plus oracle/_ref.
+ *     reference tests, brute force on small inputs.
  *   - Bit packing / count_true                 : popcount closed form, brute
  *     force.
- *   - SFloat/DFloat transcendental last ulp    : PARITY UNPINNED. Restated as
- *     (float)f((double)x) per types/float_macro.h:84-118, which is what the
- *     host macros compile to; the libm version Numo would link on another
- *     machine is not observable here.
+ *   - SFloat/DFloat NMath functions and pow    : restated as (float)f((double)x)
+ *     / f(x) per types/float_macro.h:84-118, which is what the host macros
+ *     compile to, with this machine's glibc for f. Pinned against correctly
+ *     rounded vectors (tests/golden/nmath_vectors.npz, mpmath at 400 bits):
+ *     every SFloat function and most DFloat ones are within 1 ulp of them;
+ *     glibc's DFloat cbrt (3 ulp), exp10, tanh and erfc (2 ulp) are not, and
+ *     the tests say so where they use them. Which libm Numo links on another
+ *     machine is not observable; the vectors are the fixed point instead.
  */
 #define _GNU_SOURCE
 #include <math.h>
@@ -639,8 +641,7 @@ static int32_t i32_f_max(size_t n, const int32_t *p) { int32_t y = p[0]; for (si
 static size_t i32_f_min_index(size_t n, const int32_t *p) { size_t j = 0; int32_t y = p[0]; for (size_t i = 1; i < n; ++i) if (p[i] < y) { y = p[i]; j = i; } return j; }
 static size_t i32_f_max_index(size_t n, const int32_t *p) { size_t j = 0; int32_t y = p[0]; for (size_t i = 1; i < n; ++i) if (p[i] > y) { y = p[i]; j = i; } return j; }
 
-/* 1-d entry points so the f_* loops can be pinned directly against
- * oracle/_ref (the reference's own real_accum.h) and timed by the benchmark. */
+/* 1-d entry points of the f_* loops (tests, and the benchmark's CPU leg). */
 float numo_sfloat_f(const char *op, size_t n, const float *p);
 double numo_dfloat_f(const char *op, size_t n, const double *p);
 

@@ -13,7 +13,6 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libnumo_oracle.so")
-REF_LIB = os.path.join(HERE, "_ref", "libref_accum.so")
 
 T_SFLOAT, T_DFLOAT, T_INT32, T_INT64, T_UINT64 = 0, 1, 2, 3, 4
 _TCODE = {np.dtype(np.float32): T_SFLOAT, np.dtype(np.float64): T_DFLOAT, np.dtype(np.int32): T_INT32,
@@ -21,7 +20,7 @@ _TCODE = {np.dtype(np.float32): T_SFLOAT, np.dtype(np.float64): T_DFLOAT, np.dty
 
 
 def build():
-    """Compiles the oracle (and oracle/_ref where the reference tree exists)."""
+    """Compiles the oracle."""
     subprocess.run(["make", "-C", HERE], check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
 
 
@@ -531,35 +530,3 @@ def f1d(op, x):
         return int(f(op.encode(), x.size, x.ctypes.data_as(C.c_void_p)))
     f = lib.numo_sfloat_f if x.dtype == np.float32 else lib.numo_dfloat_f
     return f(op.encode(), x.size, x.ctypes.data_as(C.c_void_p))
-
-
-# ---- oracle/_ref: the reference's own real_accum.h ---------------------------------
-def ref_available():
-    return os.path.exists(REF_LIB)
-
-
-_ref = None
-
-
-def _ref_lib():
-    global _ref
-    if _ref is None:
-        _ref = C.CDLL(REF_LIB)
-        for t in ("sfloat", "dfloat"):
-            f = getattr(_ref, t + "_ref_f")
-            f.restype = C.c_double
-            f.argtypes = [C.c_char_p, SZ, C.c_void_p, SSZ]
-            g = getattr(_ref, t + "_ref_index_f")
-            g.restype = C.c_int64
-            g.argtypes = [C.c_char_p, SZ, C.c_void_p, SSZ]
-    return _ref
-
-
-def ref_f1d(op, x):
-    """f_<op> of the reference's real_accum.h on a 1-d array (any stride)."""
-    r = _ref_lib()
-    t = "sfloat" if x.dtype == np.float32 else "dfloat"
-    p = C.c_void_p(x.__array_interface__["data"][0])
-    if op.endswith("_index") or op.endswith("_index_nan"):
-        return int(getattr(r, t + "_ref_index_f")(op.encode(), x.size, p, x.strides[0]))
-    return getattr(r, t + "_ref_f")(op.encode(), x.size, p, x.strides[0])

@@ -1,0 +1,105 @@
+// CPU build of the SFloat / DFloat function cores of cumo_amd/csrc/ew_ops.h, for
+// tests/test_nmath_vectors.py. Every step of those algorithms is an IEEE operation
+// (fused multiply-adds included), so this program computes what the device computes.
+//
+//   float_cores_check vectors <file>   reads "name type n" blocks of arguments (hex bit
+//                                      patterns), prints the results as hex bit patterns
+//   float_cores_check sweep <stride>   every stride-th float bit pattern through each SFloat
+//                                      core against (float)glibc((double)x); prints, per
+//                                      function, patterns tried, mismatches and the largest
+//                                      difference in ulps
+#define CUMO_HIP_HOST_CHECK 1
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+#define __device__
+#define __host__
+#define __forceinline__ inline __attribute__((always_inline))
+static inline int __double2hiint(double d) { uint64_t u; std::memcpy(&u, &d, 8); return (int)(uint32_t)(u >> 32); }
+static inline int __double2loint(double d) { uint64_t u; std::memcpy(&u, &d, 8); return (int)(uint32_t)u; }
+static inline double __hiloint2double(int hi, int lo) { uint64_t u = ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo; double d; std::memcpy(&d, &u, 8); return d; }
+static inline long long __double_as_longlong(double d) { long long u; std::memcpy(&u, &d, 8); return u; }
+static inline double __longlong_as_double(long long u) { double d; std::memcpy(&d, &u, 8); return d; }
+static inline int __float_as_int(float f) { int u; std::memcpy(&u, &f, 4); return u; }
+static inline float __int_as_float(int u) { float f; std::memcpy(&f, &u, 4); return f; }
+static inline unsigned __float_as_uint(float f) { unsigned u; std::memcpy(&u, &f, 4); return u; }
+static inline float __uint_as_float(unsigned u) { float f; std::memcpy(&f, &u, 4); return f; }
+
+#include "../cumo_amd/csrc/ew_ops.h"
+
+using namespace cumo_hip;
+
+typedef float (*F32)(float);
+typedef double (*F64)(double);
+struct Core32 { const char* name; F32 f; F64 ref; };
+static const Core32 kCores32[] = {
+    {"exp", exp_float_rounded_once, exp},     {"log", log_float_rounded_once<0>, log},   {"log2", log_float_rounded_once<2>, log2},
+    {"log10", log_float_rounded_once<10>, log10}, {"log1p", log1p_float_rounded_once, log1p}, {"tanh", tanh_float_rounded_once, tanh},
+    {"sinh", sinh_float_rounded_once, sinh},  {"cosh", cosh_float_rounded_once, cosh},   {"expm1", expm1_float_rounded_once, expm1},
+    {"asinh", asinh_float_rounded_once, asinh}, {"acosh", acosh_float_rounded_once, acosh}, {"atanh", atanh_float_rounded_once, atanh},
+};
+struct Core64 { const char* name; F64 f; };
+static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>}};
+
+static int64_t ordered(float f) { int32_t i; std::memcpy(&i, &f, 4); return i < 0 ? (int64_t)INT32_MIN - i : i; }
+
+int main(int argc, char** argv) {
+    if (argc >= 3 && std::strcmp(argv[1], "sweep") == 0) {
+        const uint32_t stride = (uint32_t)std::strtoul(argv[2], nullptr, 10);
+        for (const Core32& c : kCores32) {
+            uint64_t tried = 0, bad = 0;
+            int64_t worst = 0;
+            for (uint64_t b = 0; b < (1ull << 32); b += stride) {
+                uint32_t u = (uint32_t)b;
+                float x; std::memcpy(&x, &u, 4);
+                const float got = c.f(x), want = (float)c.ref((double)x);
+                ++tried;
+                if (got != got && want != want) continue;
+                uint32_t gu, wu; std::memcpy(&gu, &got, 4); std::memcpy(&wu, &want, 4);
+                if (gu == wu) continue;
+                if (got != got || want != want) { ++bad; worst = 1 << 30; continue; }
+                if (got == want) { ++bad; if (worst < 1) worst = 1; continue; }  // +0 against -0
+                int64_t d = ordered(got) - ordered(want);
+                if (d < 0) d = -d;
+                ++bad;
+                if (d > worst) worst = d;
+            }
+            std::printf("%s %llu %llu %lld\n", c.name, (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
+        }
+        return 0;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "vectors") == 0) {
+        FILE* f = std::fopen(argv[2], "r");
+        if (!f) return 2;
+        char name[32], type[8];
+        unsigned long n;
+        while (std::fscanf(f, "%31s %7s %lu", name, type, &n) == 3) {
+            std::printf("%s %s %lu\n", name, type, n);
+            const bool is32 = std::strcmp(type, "f32") == 0;
+            F32 f32 = nullptr; F64 f64 = nullptr;
+            if (is32) { for (const Core32& c : kCores32) if (std::strcmp(c.name, name) == 0) f32 = c.f; }
+            else { for (const Core64& c : kCores64) if (std::strcmp(c.name, name) == 0) f64 = c.f; }
+            for (unsigned long i = 0; i < n; ++i) {
+                unsigned long long bits;
+                if (std::fscanf(f, "%llx", &bits) != 1) return 3;
+                if (is32) {
+                    uint32_t u = (uint32_t)bits; float x; std::memcpy(&x, &u, 4);
+                    float y = f32 ? f32(x) : NAN; std::memcpy(&u, &y, 4);
+                    std::printf("%x\n", u);
+                } else {
+                    uint64_t u = bits; double x; std::memcpy(&x, &u, 8);
+                    double y = f64 ? f64(x) : NAN; std::memcpy(&u, &y, 8);
+                    std::printf("%llx\n", (unsigned long long)u);
+                }
+            }
+        }
+        std::fclose(f);
+        return 0;
+    }
+    std::fprintf(stderr, "usage: float_cores_check sweep <stride> | vectors <file>\n");
+    return 1;
+}
