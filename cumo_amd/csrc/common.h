@@ -37,6 +37,11 @@ uint32_t* red_ticket_words(int slot);
 bool capture_defer_free(char* ptr);
 bool capture_active();
 
+// CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
+// general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)
+// stand aside. For tests: the wide paths otherwise only run on arrays beyond 2^32 elements.
+bool force_wide_indices();
+
 static inline bool hip_ok(hipError_t status, const char* what) {
     if (status == hipSuccess) return true;
     report_hip_error(status, what);

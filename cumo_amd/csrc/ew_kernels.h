@@ -1179,7 +1179,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     kp.nouter = n - 1;
     kp.use_scalar = use_scalar;
     kp.flag = flag;
-    kp.small_rows = kp.rows < 0xffffffffull ? 1 : 0;
+    kp.small_rows = (kp.rows < 0xffffffffull && !force_wide_indices()) ? 1 : 0;
     for (int d = 0; d < n - 1; ++d) kp.oshape[d] = plan.shape[d];
     for (int o = 0; o < nops; ++o) {
         const int s = slot[o];
@@ -1201,7 +1201,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     }
     // the two lean kernels below also take inputs that only have their element's alignment
     // (a slice that starts at an odd column): a 128-bit global load works on any 4-byte boundary
-    const int lean_vec = (vec == 1 && plan.vec_loose > 1 && !force_scalar) ? plan.vec_loose : vec;
+    const int lean_vec = force_wide_indices() ? 1 : ((vec == 1 && plan.vec_loose > 1 && !force_scalar) ? plan.vec_loose : vec);
     const dim3 b(kEwBlock);
 
     // A Bit result over flat inputs, starting on a 128-bit unit: the lean Bit kernel
@@ -1357,7 +1357,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     kp.col_tiles = (span + tile_cols - 1) / tile_cols;
     const uint64_t row_tiles = (kp.rows + TY - 1) / TY;
     kp.n_tiles = kp.col_tiles * row_tiles;
-    kp.small_tiles = kp.n_tiles < 0xffffffffull ? 1 : 0;
+    kp.small_tiles = (kp.n_tiles < 0xffffffffull && !force_wide_indices()) ? 1 : 0;
     uint64_t grid = kp.n_tiles;
     if (grid > ew_grid_cap()) grid = ew_grid_cap();
     const dim3 g((unsigned)grid);

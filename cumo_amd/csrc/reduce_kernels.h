@@ -527,7 +527,7 @@ static inline void red_fill_params(RedKParams* kp, const ReducePlan& plan, const
     kp->in = arg->in.ptr;
     kp->out = arg->out.ptr;
     kp->out2 = out2 ? out2->ptr : nullptr;
-    kp->small = (arg->in_indexer.total_size < 0xffffffffull) ? 1 : 0;
+    kp->small = (arg->in_indexer.total_size < 0xffffffffull && !force_wide_indices()) ? 1 : 0;
 }
 
 // Inputs beyond this size are read with non-temporal loads: no cache level can hold them
@@ -634,7 +634,7 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     typedef typename Impl::In In;
     typedef typename Impl::Acc Acc;
     constexpr int V = (int)(16 / sizeof(In));
-    if (!red_stream_enabled()) return 0;
+    if (!red_stream_enabled() || force_wide_indices()) return 0;
     if (plan.vec != V || plan.red_ndim != 1 || plan.red_total == 0 || plan.out_ndim > 2) return 0;
     if (plan.out_total >= 0x7fffffffull) return 0;
     if (plan.kind != RED_ROW && plan.kind != RED_COL) return 0;
@@ -827,7 +827,7 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
         k2.in_out_step[d] = s;
         s *= (int64_t)plan.out_shape[d];
     }
-    k2.small = (n_partial < 0xffffffffull && plan.out_total < 0xffffffffull) ? 1 : 0;
+    k2.small = (n_partial < 0xffffffffull && plan.out_total < 0xffffffffull && !force_wide_indices()) ? 1 : 0;
     int tpr = 1;
     while (tpr < 64 && (uint64_t)tpr * 4 < kp.n_split) tpr <<= 1;
     if (kp.n_split > 1024) tpr = 256;

@@ -8,6 +8,7 @@
 #include "common.h"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <atomic>
 #include <mutex>
@@ -45,6 +46,14 @@ void report_hip_error(hipError_t status, const char* what) {
 }
 
 hipStream_t current_stream() { return t_stream; }
+
+bool force_wide_indices() {
+    static const bool on = [] {
+        const char* e = std::getenv("CUMO_HIP_FORCE_WIDE");
+        return e != nullptr && e[0] != 0 && e[0] != '0';
+    }();
+    return on;
+}
 
 // Streams in use get a small number, for kernels that keep per-stream words in a
 // fixed device array (tickets that launches on different streams must not share).
