@@ -397,6 +397,8 @@ int cumo_hip_pool_enable(int on) {
     return prev;
 }
 
+void cumo_hip_pool_retire_stream(void* hip_stream) { pool_retire_stream((hipStream_t)hip_stream); }
+
 void cumo_hip_pool_set_limit(size_t bytes) { std::unique_lock<std::mutex> l(g_pool.mu); g_pool.limit = bytes; }
 
 // Test hook: back the pool with the host heap (1) or the device (0). Only

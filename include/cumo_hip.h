@@ -704,6 +704,9 @@ int    cumo_hip_pool_malloc(size_t size, void* hip_stream, void** ptr);
 int    cumo_hip_pool_free(void* ptr);                       /* CUMO_HIP_ERROR_ARGUMENT if the pool does not own ptr */
 void   cumo_hip_pool_free_all_blocks(void);
 void   cumo_hip_pool_free_all_blocks_stream(void* hip_stream);
+/* files everything the pool holds for a stream (free or in use) under the null stream; the
+ * stream must have finished its work. cumo_hip_stream_destroy calls it. */
+void   cumo_hip_pool_retire_stream(void* hip_stream);
 size_t cumo_hip_pool_n_free_blocks(void);
 size_t cumo_hip_pool_used_bytes(void);
 size_t cumo_hip_pool_free_bytes(void);
