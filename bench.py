@@ -370,40 +370,6 @@ def measure_host_io(lib, mib=256, reps=5):
     return out
 
 
-def measure_graph(cumo, lib, iters=200):
-    """The C1 chain 2.5*x, +b, sum at sizes where every operation costs its launch,
-    launched one operation at a time through the C host layer, beside one submission of
-    the same chain recorded as a graph. Microseconds per chain."""
-    from cumo_amd import _lib
-    timer = Timer(lib)
-    rows = []
-    for n in (1 << 12, 1 << 20):
-        h = inputs_c1(n)
-        x, b = cumo.SFloat.cast(h["x"]), cumo.SFloat.cast(h["b"])
-
-        def chain():
-            t = 2.5 * x
-            y = t + b
-            return t, y, y.sum()
-
-        with _lib.record() as calls:
-            eager = chain()
-        _lib.replay(calls, 20)
-        t_eager = min(timer.time(lambda: _lib.replay(calls, iters)) / iters for _ in range(5))
-        with cumo.Graph() as g:
-            rec = chain()
-        g.launch(20)
-        t_graph = min(timer.time(lambda: g.launch(iters)) / iters for _ in range(5))
-        cumo.synchronize()
-        same = all((a.to_numpy().view(np.uint32) == r.to_numpy().view(np.uint32)).all() for a, r in zip(eager, rec))
-        if not same:
-            raise SystemExit("bench: the recorded chain and the eager chain disagree")
-        rows.append({"n": n, "launches": g.nodes, "us_per_chain_eager": round(t_eager * 1e3, 2), "us_per_chain_graph": round(t_graph * 1e3, 2)})
-        g.close()
-    timer.close()
-    return {"workload": "C1 chain (2.5*x, +b, sum)", "sizes": rows}
-
-
 def measure_host_cost():
     """Per-operation cost of the C host layer on tiny arrays, from the C driver built next to
     the library (bench_host_cost.cpp): no interpreter between the calls."""
@@ -466,7 +432,7 @@ def main():
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--rotated-only", action="store_true",
                     help="leave out the same-buffer replay legs, so that a kernel trace of this command holds rotated launches only")
-    ap.add_argument("--no-extras", action="store_true", help="skip the host transfer and recorded-chain measurements")
+    ap.add_argument("--no-extras", action="store_true", help="skip the host transfer and host-cost measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch a plain contiguous copy of known size (256 MiB in, 256 MiB out) five times, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command can scale its counters by it")
@@ -636,7 +602,6 @@ def main():
         out["per_config"] = per_config
         if not args.no_extras:
             out["host_io"] = measure_host_io(lib)
-            out["graph"] = measure_graph(cumo_amd, lib)
             out["host_cost"] = measure_host_cost()
     print(json.dumps(out))
 

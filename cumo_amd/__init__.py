@@ -8,7 +8,6 @@ CPU fallback.
 """
 from . import _lib
 from ._lib import OutOfMemoryError, RuntimeError_ as RuntimeError, ShapeError
-from .graph import Graph
 from .narray import Bit, DFloat, Fused, Int32, Int64, NArray, NMath, SFloat, UInt64
 
 
@@ -48,5 +47,5 @@ def device_count():
     return _lib.lib.cumo_hip_device_count()
 
 
-__all__ = ["SFloat", "DFloat", "Int32", "Int64", "UInt64", "Bit", "NArray", "NMath", "Fused", "Graph", "MemoryPool", "ShapeError",
+__all__ = ["SFloat", "DFloat", "Int32", "Int64", "UInt64", "Bit", "NArray", "NMath", "Fused", "MemoryPool", "ShapeError",
            "OutOfMemoryError", "RuntimeError", "synchronize", "device_count"]

@@ -138,11 +138,6 @@ _sig = {
     "cumo_hip_memcpy_h2d": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_memcpy_d2h": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_memset": (None, [C.c_void_p, C.c_int, C.c_size_t]),
-    "cumo_hip_graph_begin": (C.c_int, []),
-    "cumo_hip_graph_end": (C.c_void_p, []),
-    "cumo_hip_graph_launch": (C.c_int, [C.c_void_p]),
-    "cumo_hip_graph_node_count": (C.c_size_t, [C.c_void_p]),
-    "cumo_hip_graph_destroy": (None, [C.c_void_p]),
     "cumo_hip_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_copy_from_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "cumo_hip_pool_malloc": (C.c_int, [C.c_size_t, C.c_void_p, P(C.c_void_p)]),

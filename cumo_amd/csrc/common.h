@@ -32,11 +32,6 @@ void pool_retire_stream(hipStream_t stream);
 // nullptr after reporting an error. reduce_tickets.hip.
 uint32_t* red_ticket_words(int slot);
 
-// Stream capture (graph.cpp): while a capture is open, released memory stays with the
-// graph being recorded, and the pool hands blocks across streams without events.
-bool capture_defer_free(char* ptr);
-bool capture_active();
-
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)
 // stand aside. For tests: the wide paths otherwise only run on arrays beyond 2^32 elements.

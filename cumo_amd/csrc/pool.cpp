@@ -286,7 +286,7 @@ int cumo_hip_pool_malloc(size_t size, void* hip_stream, void** out) {
     if (!c) {
         hipStream_t from = nullptr;
         c = p.steal(stream, size, &from);
-        if (c && !p.host_backend && !capture_active()) {
+        if (c && !p.host_backend) {
             // everything queued so far on the giving stream must finish before
             // work queued from now on the taking stream touches the chunk
             hipEvent_t ev = nullptr;
@@ -442,7 +442,6 @@ char* cumo_cuda_runtime_malloc(size_t size) {
 
 static int runtime_free(char* ptr) {
     if (!ptr) return 0;
-    if (capture_defer_free(ptr)) return 0;  // every replay of the graph being recorded uses it again
     // offer the pointer to the pool first whatever the enabled flag says now
     // (reference: cuda/memory_pool.cpp:98-117)
     if (cumo_hip_pool_free(ptr) == CUMO_HIP_OK) return 0;

@@ -681,23 +681,6 @@ void  cumo_hip_memset(void* dst, int byte, size_t n);
 int   cumo_hip_copy_to_host(void* dst_host, const void* src_device, size_t n);
 int   cumo_hip_copy_from_host(void* dst_device, const void* src_host, size_t n);
 
-/* A recorded chain of operations replayed with one submission (no counterpart in the
- * reference, which launches every operation separately; for callers that repeat the
- * same chain on the same arrays while each launch costs more than its kernel).
- * Between begin and end the library's launches are captured on a stream of its own
- * instead of running; end answers a handle (NULL on failure) and the chain has not run
- * yet; launch queues one run of the whole chain on the current stream. Arrays
- * allocated inside the capture belong to the caller and are rewritten by every
- * replay; memory released inside it stays reserved until destroy. Operations that
- * need the host in the middle (Int32 division / abs error flags, Bit#where / mask,
- * read-back) cannot be captured: end then fails with a runtime error. One capture
- * at a time per process. destroy waits for the device first. */
-int    cumo_hip_graph_begin(void);
-void*  cumo_hip_graph_end(void);
-int    cumo_hip_graph_launch(void* graph);
-size_t cumo_hip_graph_node_count(void* graph);
-void   cumo_hip_graph_destroy(void* graph);
-
 /* Memory pool (replaces cumo::internal::MemoryPool, cuda/memory_pool_impl.hpp:160-435).
  * Returns CUMO_HIP_OK or an error kind; never raises. */
 int    cumo_hip_pool_malloc(size_t size, void* hip_stream, void** ptr);
