@@ -37,6 +37,13 @@ uint32_t* red_ticket_words(int slot);
 // stand aside. For tests: the wide paths otherwise only run on arrays beyond 2^32 elements.
 bool force_wide_indices();
 
+// Whether a launch that moves `bytes` through memory once should use non-temporal
+// accesses: from 48 MiB upward the data neither comes from nor is wanted in the caches,
+// and keeping it out of them is measurably faster on operands that were not just
+// touched. CUMO_HIP_NT=0 / 1 (read once) forces the answer.
+constexpr uint64_t kStreamNtBytes = 48ull << 20;
+bool stream_past_caches(uint64_t bytes);
+
 static inline bool hip_ok(hipError_t status, const char* what) {
     if (status == hipSuccess) return true;
     report_hip_error(status, what);

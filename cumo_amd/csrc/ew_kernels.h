@@ -1019,16 +1019,7 @@ static inline uint64_t ew_grid_max() { return 0x7fffffffull; }
 // peak with plain accesses and 77-78% with non-temporal ones; no difference at 32 MiB.
 // (Launching the same operation on the same buffers again and again favours plain
 // accesses up to 256 MB, because the last-level cache then still holds the operands.)
-// CUMO_HIP_NT=0 / 1 forces them off / on.
-constexpr uint64_t kEwNtBytes = 48ull << 20;
-static inline int ew_nt_mode() {
-    static int mode = -2;
-    if (mode == -2) {
-        const char* e = std::getenv("CUMO_HIP_NT");
-        mode = e ? (std::atoi(e) != 0 ? 1 : 0) : -1;
-    }
-    return mode;
-}
+// The decision is stream_past_caches(bytes), shared by every kernel family.
 
 // in1/in2 may be NULL (NIN < 2 or the scalar form). out_bit is non-NULL for a
 // Bit result, in which case out is ignored.
@@ -1073,8 +1064,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 if (plan.step[o][d] != 0) nb *= plan.shape[d];
             tr_bytes += nb;
         }
-        const int nt_mode = ew_nt_mode();
-        const bool tr_nt = nt_mode < 0 ? tr_bytes > kEwNtBytes : nt_mode != 0;
+        const bool tr_nt = stream_past_caches(tr_bytes);
         {
             static int order = -2;
             if (order == -2) {
@@ -1219,8 +1209,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             const uint64_t groups = (kp.inner + 127) / 128;
             const uint64_t blocks = (groups * (32 / VB) + kEwBlock - 1) / kEwBlock;
             if (flat && blocks <= ew_grid_max()) {
-                const int mode = ew_nt_mode();
-                const bool nt = mode < 0 ? kp.inner * sizeof(A) * (uint64_t)(nops - 1) > kEwNtBytes : mode != 0;
+                const bool nt = stream_past_caches(kp.inner * sizeof(A) * (uint64_t)(nops - 1));
                 CUMO_BIT_DIGIT* dst = reinterpret_cast<CUMO_BIT_DIGIT*>(const_cast<char*>(ops[nops - 1].ptr)) + out_bit->pos / 32;
                 const dim3 g((unsigned)blocks);
                 if (nt) hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], dst, kp.inner, use_scalar, op, sv);
@@ -1247,8 +1236,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 if (plan.step[o][d] != 0) nb *= plan.shape[d];
             bytes += nb;
         }
-        const int mode = ew_nt_mode();
-        const bool nt = mode < 0 ? bytes > kEwNtBytes : mode != 0;
+        const bool nt = stream_past_caches(bytes);
 
         // every operand one contiguous run
         bool flat = n == 1;

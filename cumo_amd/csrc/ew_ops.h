@@ -29,6 +29,31 @@ __device__ __forceinline__ float rcp_approx(float x) {
     return __builtin_amdgcn_rcpf(x);
 #endif
 }
+// 1 / b for a finite, normal, non-zero double to about 2^-44: the hardware's estimate (good to
+// some 2^-23) and one Newton step, 6 instructions where the IEEE division takes about 25. For
+// results that are rounded to float afterwards.
+__device__ __forceinline__ double rcp_refined(double b) {
+#ifdef CUMO_HIP_HOST_CHECK
+    return 1.0 / b;
+#else
+    const double r = __builtin_amdgcn_rcp(b);
+    return __builtin_fma(__builtin_fma(-b, r, 1.0), r, r);
+#endif
+}
+// sqrt(a) for a positive, finite, normal double to about 2^-44, the same way
+__device__ __forceinline__ double sqrt_refined(double a) {
+#ifdef CUMO_HIP_HOST_CHECK
+    return sqrt(a);
+#else
+    const double y = __builtin_amdgcn_rsq(a);
+    const double s = a * y;
+    return __builtin_fma(__builtin_fma(-s, s, a) * 0.5, y, s);
+#endif
+}
+// (double)k without the quarter-rate conversion: 2^52 + 2^31 + k sits in the mantissa
+__device__ __forceinline__ double int_to_double(int k) {
+    return __hiloint2double(0x43300000, (int)((uint32_t)k ^ 0x80000000u)) - 4503601774854144.0;
+}
 
 #define CUMO_HIP_OP_COMMON(TA, TB, TR, NIN_, BIT_, CHK_) \
     typedef TA A; typedef TB B; typedef TR R; typedef TA S; \
@@ -166,15 +191,57 @@ __device__ __forceinline__ double log_core(double x, int kadj = 0) {  // x posit
     }
     return dk * 6.93147180369123816490e-01 - ((hfsq - (s * (hfsq + R) + dk * 1.90821492927058770002e-10)) - f);
 }
+// The same logarithm for a result that is rounded to float: log(1 + f) = 2 s + s z R(z), z = s^2,
+// with a degree-4 fit of R (2^-43 relative on 0 <= z <= 0.0295), the division by the refined
+// reciprocal and k converted through the mantissa trick: about half the instructions of the
+// form above. x positive, finite and normal.
+template <int BASE, bool EXTRA = false>
+__device__ __forceinline__ double log_core_for_float(double x) {
+    uint32_t hx = (uint32_t)__double2hiint(x);
+    int k = (int)(hx >> 20) - 1023;
+    hx &= 0x000fffffu;
+    const uint32_t i = (hx + 0x95f64u) & 0x100000u;
+    k += (int)(i >> 20);
+    const double m = __hiloint2double((int)(hx | (i ^ 0x3ff00000u)), __double2loint(x));
+    const double f = m - 1.0;
+    const double d = 2.0 + f;
+    double rd = rcp_refined(d);
+    double R;
+    if (EXTRA) {  // 2^-50: a second Newton step and one more term (for pow, whose exponent multiplies the error)
+        rd = __builtin_fma(__builtin_fma(-d, rd, 1.0), rd, rd);
+        R = 0.16625981808365656;
+    }
+    const double s = f * rd;
+    const double z = s * s;
+    if (EXTRA) {
+        R = __builtin_fma(R, z, 0.181399072797897);
+        R = __builtin_fma(R, z, 0.22222869146289312);
+        R = __builtin_fma(R, z, 0.28571424071527063);
+        R = __builtin_fma(R, z, 0.4000000001143263);
+        R = __builtin_fma(R, z, 0.6666666666666199);
+    } else {
+        R = 0.19366868181730357;
+        R = __builtin_fma(R, z, 0.22191171841584165);
+        R = __builtin_fma(R, z, 0.2857175839580272);
+        R = __builtin_fma(R, z, 0.3999999877669915);
+        R = __builtin_fma(R, z, 0.6666666666739216);
+    }
+    const double lm = __builtin_fma(s * z, R, s + s);
+    const double dk = int_to_double(k);
+    if (BASE == 2) return __builtin_fma(lm, 1.44269504088896338700e+00, dk);
+    if (BASE == 10) return __builtin_fma(dk, 3.01029995663981198017e-01, 4.34294481903251816668e-01 * lm);
+    if (EXTRA) return __builtin_fma(dk, 6.93147180369123816490e-01, __builtin_fma(dk, 1.90821492927058770002e-10, lm));
+    return __builtin_fma(dk, 6.93147180559945286227e-01, lm);
+}
 template <int BASE>
 __device__ __forceinline__ float log_float_rounded_once(float xf) {
-    // NaN comes back in through xf - xf (which is NaN for an infinity too); then, on the
-    // float and after all the arithmetic: 0 -> -inf, negative -> NaN, +inf -> +inf
-    float y = (float)log_core<BASE>((double)xf) + (xf - xf);
-    y = (xf == 0.0f) ? -INFINITY : y;
-    y = (xf < 0.0f) ? NAN : y;
-    y = (xf == INFINITY) ? INFINITY : y;
-    return y;
+    // a subnormal float is a normal double; zero, negative arguments, infinity and NaN take the branch
+    if (__float_as_uint(xf) - 1u >= 0x7f7fffffu) {
+        if (xf == 0.0f) return -INFINITY;
+        if (xf < 0.0f) return NAN;
+        return xf + xf;
+    }
+    return (float)log_core_for_float<BASE>((double)xf);
 }
 // DFloat log, log2, log10: the same algorithm on a double argument (a subnormal one is
 // scaled by 2^54 first). Against glibc on 2 * 10^8 random doubles per function (all
@@ -193,7 +260,7 @@ __device__ __forceinline__ double log_double(double x) {
 // logarithm above applies to it unchanged; below that the answer rounds to x itself.
 // Checked like the others, over every float bit pattern.
 __device__ __forceinline__ float log1p_float_rounded_once(float xf) {
-    float y = (float)log_core<0>(1.0 + (double)xf) + (xf - xf);
+    float y = (float)log_core_for_float<0>(1.0 + (double)xf) + (xf - xf);
     y = (__builtin_fabsf(xf) < 1.862645149230957e-09f) ? xf : y;
     y = (xf == -1.0f) ? -INFINITY : y;
     y = (xf < -1.0f) ? NAN : y;
@@ -212,56 +279,64 @@ CUMO_HIP_LOG_OP(OpLog10, 10)
 template <class T> struct OpLog1p { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
     __device__ __forceinline__ bool operator()(T x, T, T& z) const {
         if constexpr (sizeof(T) == 4) z = (T)log1p_float_rounded_once((float)x);
-        else z = (T)log1p((double)x);
+        else z = (x == 0) ? x : (T)log1p((double)x);  // the library answers +0 for -0
         return true; } };
 
-// exp(x) - 1 in double for x inside [-745, 709], from the reduction and polynomial of exp
-// above: with q = (exp(r) - 1) / r, exp(x) - 1 = 2^k (1 + q r) - 1 = (2^k - 1) + (2^k q) r
-// comes out of one fused multiply-add, without the cancellation of exp(x) - 1 near 0.
-__device__ __forceinline__ double expm1_core(double x) {
+// exp(x) - 1 for x inside [-745, 709] and a result that is rounded to float, from the reduction
+// of exp above: with q = (exp(r) - 1) / r (a degree-8 fit, 2^-44 relative on |r| <= ln(2)/2),
+// exp(x) - 1 = 2^k (1 + q r) - 1 = (2^k - 1) + (2^k q) r comes out of one fused multiply-add,
+// without the cancellation of exp(x) - 1 near 0.
+// EXPM1 false: exp(x) itself, 2^k (1 + q r), for x inside [-700, 700].
+template <bool EXPM1>
+__device__ __forceinline__ double exp_core_for_float(double x) {
     const double big = 6755399441055744.0;  // 1.5 * 2^52
     const double t0 = __builtin_fma(x, 1.44269504088896338700e+00, big);
     const double k = t0 - big;
     const uint32_t ki = (uint32_t)__double2loint(t0);  // k as a two's-complement integer (anything for a NaN, which r carries on)
     double r = __builtin_fma(k, -6.93147180369123816490e-01, x);
     r = __builtin_fma(k, -1.90821492927058770002e-10, r);
-    const double c[12] = {
-        1.60590438368216133e-10, 2.08767569878681002e-09, 2.50521083854417202e-08, 2.75573192239858883e-07, 2.75573192239858925e-06,
-        2.48015873015873016e-05, 1.98412698412698413e-04, 1.38888888888888894e-03, 8.33333333333333322e-03, 4.16666666666666644e-02,
-        1.66666666666666657e-01, 5.00000000000000000e-01};
-    double q = c[0];
-#pragma unroll
-    for (int i = 1; i < 12; ++i) q = __builtin_fma(q, r, c[i]);
+    double q = 2.7632704798457074e-06;
+    q = __builtin_fma(q, r, 2.486788542787532e-05);
+    q = __builtin_fma(q, r, 0.0001984119277622577);
+    q = __builtin_fma(q, r, 0.0013888839087169604);
+    q = __builtin_fma(q, r, 0.008333333363318172);
+    q = __builtin_fma(q, r, 0.04166666678635317);
+    q = __builtin_fma(q, r, 0.16666666666633861);
+    q = __builtin_fma(q, r, 0.4999999999995511);
     q = __builtin_fma(q, r, 1.0);
+    if (!EXPM1) {
+        const double e = __builtin_fma(q, r, 1.0);
+        return __hiloint2double((int)((uint32_t)__double2hiint(e) + (ki << 20)), __double2loint(e));
+    }
     const double qs = __hiloint2double((int)((uint32_t)__double2hiint(q) + (ki << 20)), __double2loint(q));
     const double p2k = __hiloint2double((int)((1023u + ki) << 20), 0);
     return __builtin_fma(qs, r, p2k - 1.0);
 }
+__device__ __forceinline__ double expm1_core(double x) { return exp_core_for_float<true>(x); }
 
-// SFloat tanh, sinh, cosh, expm1: the double-precision function rounded to float once, each
-// from t = exp(a) - 1 above and one IEEE division: tanh|x| = t / (t + 2) with a = 2|x|
-// (clamped at 40, where the answer is 1 in double already); sinh|x| = (t + t / (t + 1)) / 2 and
-// cosh x = (e + 1 / e) / 2, e = t + 1, with a = |x| clamped at 90 (beyond float range either
-// way); expm1 with a = x clamped to [-40, 89]. Run on the CPU against glibc over every float
-// bit pattern, the float results differ nowhere. A NaN argument fails the clamps' comparisons
-// and travels through the arithmetic.
+// SFloat tanh, sinh, cosh, expm1: the function evaluated in double (to 2^-43 or better) and
+// rounded to float once, each from t = exp(a) - 1 above and one refined reciprocal:
+// tanh|x| = t / (t + 2) with a = 2|x| (clamped at 40, where the answer is 1 in double already);
+// sinh|x| = (t + t / (t + 1)) / 2 and cosh x = (e + 1 / e) / 2, e = t + 1, with a = |x| clamped
+// at 90 (beyond float range either way); expm1 with a = x clamped to [-40, 89]. A NaN argument
+// fails the clamps' comparisons and travels through the arithmetic.
 __device__ __forceinline__ float tanh_float_rounded_once(float xf) {
     float ax = __builtin_fabsf(xf);
     ax = (ax > 20.0f) ? 20.0f : ax;
     const double t = expm1_core(2.0 * (double)ax);
-    return __builtin_copysignf((float)(t / (t + 2.0)), xf);
+    return __builtin_copysignf((float)(t * rcp_refined(t + 2.0)), xf);
 }
 __device__ __forceinline__ float sinh_float_rounded_once(float xf) {
     float ax = __builtin_fabsf(xf);
     ax = (ax > 90.0f) ? 90.0f : ax;
     const double t = expm1_core((double)ax);
-    return __builtin_copysignf((float)(0.5 * (t + t / (t + 1.0))), xf);
+    return __builtin_copysignf((float)(0.5 * __builtin_fma(t, rcp_refined(t + 1.0), t)), xf);
 }
 __device__ __forceinline__ float cosh_float_rounded_once(float xf) {
     float ax = __builtin_fabsf(xf);
     ax = (ax > 90.0f) ? 90.0f : ax;
     const double e = expm1_core((double)ax) + 1.0;
-    return (float)(0.5 * (e + 1.0 / e));
+    return (float)(0.5 * (e + rcp_refined(e)));
 }
 __device__ __forceinline__ float expm1_float_rounded_once(float xf) {
     float xc = (xf < -40.0f) ? -40.0f : xf;
@@ -269,27 +344,24 @@ __device__ __forceinline__ float expm1_float_rounded_once(float xf) {
     const float y = (float)expm1_core((double)xc);
     return (xf == 0.0f) ? xf : y;  // keeps the sign of a zero argument
 }
-// SFloat asinh, acosh, atanh: the double-precision function rounded to float once, on the
-// logarithm above. log(1 + u) for a double u >= 0 whose sum 1 + u is not exact: the part c
+// SFloat asinh, acosh, atanh: the function evaluated in double and rounded to float once, on the
+// logarithm above (the form for float results, refined reciprocal and square root). log(1 + u) for a double u >= 0 whose sum 1 + u is not exact: the part c
 // of u that the sum w loses comes back as c / w (c is below one ulp of w, so a float
 // reciprocal is more than enough). asinh|x| = log1p(a + a^2 / (1 + sqrt(1 + a^2))) and
 // acosh x = log1p(t + sqrt(t^2 + 2 t)), t = x - 1 (exact), hold over the whole float range
 // (a^2 and t^2 are exact in double and stay far below its overflow); atanh|x| =
 // log1p(2a / (1 - a)) / 2 with 1 - a exact, so that the quotient's half ulp is all the
-// argument's error. Below 2^-29 asinh and atanh round to the argument. Run on the CPU
-// against glibc over every float bit pattern, the float results of atanh differ nowhere,
-// those of asinh at four arguments (+-4.19005794e18, +-2.74915304e28) and those of acosh
-// at the positive two of them, by one ulp.
+// argument's error. Below 2^-29 asinh and atanh round to the argument.
 __device__ __forceinline__ double log1p_core(double u) {
     const double w = 1.0 + u;
     const double c = u - (w - 1.0);
-    return __builtin_fma(c, (double)rcp_approx((float)w), log_core<0>(w));
+    return __builtin_fma(c, (double)rcp_approx((float)w), log_core_for_float<0>(w));
 }
 __device__ __forceinline__ float asinh_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);
     const double a = (double)af;
     const double a2 = a * a;
-    const double u = a + a2 / (1.0 + sqrt(1.0 + a2));
+    const double u = __builtin_fma(a2, rcp_refined(1.0 + sqrt_refined(1.0 + a2)), a);
     float y = (float)log1p_core(u);       // NaN travels through; an infinity gives NaN here and is put right below
     y = (af < 1.862645149230957e-09f) ? af : y;
     y = (af == INFINITY) ? INFINITY : y;
@@ -298,7 +370,8 @@ __device__ __forceinline__ float asinh_float_rounded_once(float xf) {
 __device__ __forceinline__ float acosh_float_rounded_once(float xf) {
     const float xc = (xf < 1.0f) ? 1.0f : xf;  // keeps the square root's argument in range; a NaN stays
     const double t = (double)xc - 1.0;
-    const double u = t + sqrt(__builtin_fma(t, t, 2.0 * t));
+    const double q = __builtin_fma(t, t, 2.0 * t);
+    const double u = t + ((q > 0.0) ? sqrt_refined(q) : 0.0);   // a NaN gives 0 here and comes back through t
     float y = (float)log1p_core(u);
     y = (xf < 1.0f) ? NAN : y;
     y = (xf == INFINITY) ? INFINITY : y;
@@ -308,11 +381,112 @@ __device__ __forceinline__ float atanh_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);
     const float ac = (af < 1.0f) ? af : 0.5f;   // a stand-in for |x| >= 1, settled below
     const double a = (double)ac;
-    float y = (float)(0.5 * log1p_core((a + a) / (1.0 - a)));
+    float y = (float)(0.5 * log1p_core((a + a) * rcp_refined(1.0 - a)));
     y = (af < 1.862645149230957e-09f) ? af : y;
     y = (af == 1.0f) ? INFINITY : y;
     y = (af > 1.0f) ? NAN : y;
     y = (xf != xf) ? xf : y;
+    return __builtin_copysignf(y, xf);
+}
+// SFloat sin, cos, tan: evaluated in double and rounded to float once. Below 10^6 in magnitude:
+// k = rint(x 2/pi) by the 1.5 * 2^52 trick, r = x - k pi/2 with pi/2 in two parts (the upper 33
+// bits, so that k times it is exact), then sin r = r + r z S(z) and cos r = 1 - z/2 + z^2 C(z),
+// z = r^2, from degree-4 and degree-3 fits (2^-35 and 2^-40 relative on |r| <= pi/4), both
+// evaluated, the quadrant choosing between them and the sign. Beyond that the device library's
+// double function (its argument reduction is a branch of its own). WHICH: 0 sin, 1 cos, 2 tan.
+template <int WHICH>
+__device__ __forceinline__ float trig_float_rounded_once(float xf) {
+    if (!(__builtin_fabsf(xf) < 1.0e6f)) {   // large, infinite or NaN
+        if (WHICH == 0) return (float)sin((double)xf);
+        if (WHICH == 1) return (float)cos((double)xf);
+        return (float)tan((double)xf);
+    }
+    const double x = (double)xf;
+    const double big = 6755399441055744.0;  // 1.5 * 2^52
+    const double t = __builtin_fma(x, 6.36619772367581382433e-01, big);
+    const double k = t - big;
+    const uint32_t ki = (uint32_t)__double2loint(t);
+    double r = __builtin_fma(k, -1.57079632673412561417e+00, x);  // pi/2, upper 33 bits
+    r = __builtin_fma(k, -6.07710050650619224932e-11, r);         // pi/2, the rest
+    const double z = r * r;
+    double ps = -2.4805649861027395e-08;
+    ps = __builtin_fma(ps, z, 2.7555991132757367e-06);
+    ps = __builtin_fma(ps, z, -0.0001984126691790408);
+    ps = __builtin_fma(ps, z, 0.008333333331080512);
+    ps = __builtin_fma(ps, z, -0.16666666666663896);
+    const double sn = __builtin_fma(r * z, ps, r);
+    double pc = -2.7300987836458486e-07;
+    pc = __builtin_fma(pc, z, 2.480060068144107e-05);
+    pc = __builtin_fma(pc, z, -0.0013888887672811724);
+    pc = __builtin_fma(pc, z, 0.04166666666432424);
+    const double cs = __builtin_fma(z * z, pc, __builtin_fma(z, -0.5, 1.0));
+    if (WHICH == 2) {
+        const bool odd = (ki & 1u) != 0;
+        const float y = (float)((odd ? -cs : sn) * rcp_refined(odd ? sn : cs));
+        return (xf == 0.0f) ? xf : y;
+    }
+    // sin: quadrant 0 s, 1 c, 2 -s, 3 -c; cos is sin a quadrant further on
+    const uint32_t q = WHICH == 0 ? ki : ki + 1u;
+    const double v = (q & 1u) ? cs : sn;
+    const float y = (float)__hiloint2double(__double2hiint(v) ^ (int)((q & 2u) << 30), __double2loint(v));
+    return (WHICH == 0 && xf == 0.0f) ? xf : y;
+}
+// SFloat atan, the same way: one refined reciprocal brings the argument below tan(pi/8)
+// (t = a there, (a - 1)/(a + 1) plus pi/4 up to tan(3 pi/8), -1/a plus pi/2 above), then
+// atan t = t + t z A(z), z = t^2, with a degree-7 fit of A (2^-43 relative).
+__device__ __forceinline__ float atan_float_rounded_once(float xf) {
+    const float af = __builtin_fabsf(xf);
+    const double a = (double)((af > 1.0e30f) ? 1.0e30f : af);  // the answer is pi/2 in float from 2^25 on; a NaN passes
+    const bool mid = af > 0.41421356f, top = af > 2.41421356f;
+    const double num = top ? -1.0 : (mid ? a - 1.0 : a);
+    const double den = top ? a : (mid ? a + 1.0 : 1.0);
+    const double off = top ? 1.57079632679489655800e+00 : (mid ? 7.85398163397448278999e-01 : 0.0);
+    const double t = num * rcp_refined(den);
+    const double z = t * t;
+    double p = 0.033038827515269494;
+    p = __builtin_fma(p, z, -0.06032248119994454);
+    p = __builtin_fma(p, z, 0.07605969344616582);
+    p = __builtin_fma(p, z, -0.09084239163280672);
+    p = __builtin_fma(p, z, 0.11110827992295265);
+    p = __builtin_fma(p, z, -0.1428570834807845);
+    p = __builtin_fma(p, z, 0.19999999952417688);
+    p = __builtin_fma(p, z, -0.33333333333270726);
+    return __builtin_copysignf((float)(off + __builtin_fma(t * z, p, t)), xf);
+}
+// SFloat erf, the same way: below 1, erf a = a P(a^2) with a degree-8 fit (2^-40 relative);
+// from 1 on, erf a = 1 - exp(-a S(a)) with a degree-10 fit of S = -log(erfc a)/a on [1, 4]
+// (2^-41 absolute in erf) and exp(.) - 1 from the core above. In float, erf is 1 from 3.92 on.
+__device__ __forceinline__ float erf_float_rounded_once(float xf) {
+    const float af = __builtin_fabsf(xf);
+    const double a = (double)af;
+    float y;
+    if (af < 1.0f) {
+        const double z = a * a;
+        double p = 1.0601184931822625e-06;
+        p = __builtin_fma(p, z, -1.3914064883994308e-05);
+        p = __builtin_fma(p, z, 0.00011957330950188644);
+        p = __builtin_fma(p, z, -0.0008542703072832773);
+        p = __builtin_fma(p, z, 0.00522378653090469);
+        p = __builtin_fma(p, z, -0.026866134013422204);
+        p = __builtin_fma(p, z, 0.11283791318349341);
+        p = __builtin_fma(p, z, -0.3761263889010029);
+        p = __builtin_fma(p, z, 1.128379167094713);
+        y = (float)(a * p);
+    } else {
+        const double ac = (af > 4.0f) ? 4.0 : a;  // a NaN passes
+        double sp = -1.0762777310949488e-07;
+        sp = __builtin_fma(sp, ac, 2.5858233440202685e-06);
+        sp = __builtin_fma(sp, ac, -2.8055149962875097e-05);
+        sp = __builtin_fma(sp, ac, 0.00017968025342242425);
+        sp = __builtin_fma(sp, ac, -0.0007285698386718862);
+        sp = __builtin_fma(sp, ac, 0.0016962354086159648);
+        sp = __builtin_fma(sp, ac, -2.9800151096382062e-05);
+        sp = __builtin_fma(sp, ac, -0.019378056134721402);
+        sp = __builtin_fma(sp, ac, 0.10294844019086533);
+        sp = __builtin_fma(sp, ac, 0.636553217738299);
+        sp = __builtin_fma(sp, ac, 1.1283899394236938);
+        y = (float)(-expm1_core(-ac * sp));
+    }
     return __builtin_copysignf(y, xf);
 }
 #define CUMO_HIP_OWN_OP(NAME, FEXPR, DEXPR)                                                                                 \
@@ -324,7 +498,7 @@ __device__ __forceinline__ float atanh_float_rounded_once(float xf) {
 CUMO_HIP_OWN_OP(OpTanh, tanh_float_rounded_once, tanh((double)x))
 CUMO_HIP_OWN_OP(OpSinh, sinh_float_rounded_once, sinh((double)x))
 CUMO_HIP_OWN_OP(OpCosh, cosh_float_rounded_once, cosh((double)x))
-CUMO_HIP_OWN_OP(OpExpm1, expm1_float_rounded_once, expm1((double)x))
+CUMO_HIP_OWN_OP(OpExpm1, expm1_float_rounded_once, (x == 0) ? (double)x : expm1((double)x))  // the library answers +0 for -0
 
 template <class T> struct OpExp { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
     __device__ __forceinline__ bool operator()(T x, T, T& z) const {
@@ -333,19 +507,19 @@ template <class T> struct OpExp { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) s
         return true; } };
 CUMO_HIP_FUN_H(OpExp2, exp2((double)x))
 CUMO_HIP_FUN_H(OpExp10, exp10((double)x))
-CUMO_HIP_FUN_H(OpSin, sin((double)x))
-CUMO_HIP_FUN_H(OpCos, cos((double)x))
-CUMO_HIP_FUN_H(OpTan, tan((double)x))
+CUMO_HIP_OWN_OP(OpSin, trig_float_rounded_once<0>, sin((double)x))
+CUMO_HIP_OWN_OP(OpCos, trig_float_rounded_once<1>, cos((double)x))
+CUMO_HIP_OWN_OP(OpTan, trig_float_rounded_once<2>, tan((double)x))
 CUMO_HIP_FUN_H(OpAsin, asin((double)x))
 CUMO_HIP_FUN_H(OpAcos, acos((double)x))
-CUMO_HIP_FUN_H(OpAtan, atan((double)x))
+CUMO_HIP_OWN_OP(OpAtan, atan_float_rounded_once, atan((double)x))
 CUMO_HIP_OWN_OP(OpAsinh, asinh_float_rounded_once, asinh((double)x))
 CUMO_HIP_OWN_OP(OpAcosh, acosh_float_rounded_once, acosh((double)x))
 CUMO_HIP_OWN_OP(OpAtanh, atanh_float_rounded_once, atanh((double)x))
 // the host macro guards x == 0 (types/float_macro.h:113); the reference's device
 // macro does not and answers NaN there, which Numo does not
 CUMO_HIP_FUN_H(OpSinc, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
-CUMO_HIP_FUN_H(OpErf, erf((double)x))
+CUMO_HIP_OWN_OP(OpErf, erf_float_rounded_once, erf((double)x))
 CUMO_HIP_FUN_H(OpErfc, erfc((double)x))
 
 #define CUMO_HIP_IUN(NAME, EXPR) \
@@ -371,8 +545,25 @@ struct OpIAbs { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, true)
 // ---- pow, maximum/minimum, clip ----------------------------------------------
 // Float ** float: the host macro's pow in double, rounded once
 // (reference: types/float_macro.h m_pow; device types/float_macro_kernel.h:36).
+// SFloat: for a positive finite base and a finite exponent, exp(y log x) in double with the
+// logarithm good to 2^-50 (|y log x| stays below 110 wherever the float answer is neither 0 nor
+// infinite, so the exponent's error stays below 2^-42) and the exp of the core above; everything
+// else (zero, negative, infinite or NaN base, infinite or NaN exponent: the sign, domain and
+// limit rules) is the device library's pow.
+__device__ __forceinline__ float pow_float_rounded_once(float xf, float yf) {
+    if (__float_as_uint(xf) - 1u < 0x7f7fffffu && __builtin_fabsf(yf) < INFINITY) {
+        double p = (double)yf * log_core_for_float<0, true>((double)xf);
+        p = (p < -110.0) ? -110.0 : p;
+        p = (p > 90.0) ? 90.0 : p;
+        return (float)exp_core_for_float<false>(p);
+    }
+    return (float)pow((double)xf, (double)yf);
+}
 template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) static constexpr bool HEAVY = true;
-    __device__ __forceinline__ bool operator()(T x, T y, T& z) const { z = (T)pow((double)x, (double)y); return true; } };
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)pow_float_rounded_once((float)x, (float)y);
+        else z = (T)pow((double)x, (double)y);
+        return true; } };
 
 // Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
 // element type for small exponents, pow() beyond 64, the reciprocal for negative ones.

@@ -215,7 +215,7 @@ void fr_launch_one(const FusedRowsParams& p, hipStream_t stream) {
     uint64_t grid = (p.rows + RPB - 1) / RPB;
     if (grid > 256u * 64u) grid = 256u * 64u;
     // one read and one write of the array: beyond the 256 MB last-level cache, stream past it
-    const bool nt = 2 * p.rows * p.n * sizeof(T) > (320ull << 20);
+    const bool nt = stream_past_caches(2 * p.rows * p.n * sizeof(T));
     if (nt) hipLaunchKernelGGL((fused_rows_kernel<T, MODE, TPR, NV, true>), dim3((unsigned)grid), dim3(kFrBlock), 0, stream, p);
     else hipLaunchKernelGGL((fused_rows_kernel<T, MODE, TPR, NV, false>), dim3((unsigned)grid), dim3(kFrBlock), 0, stream, p);
 }

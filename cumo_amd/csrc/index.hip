@@ -172,9 +172,9 @@ __global__ __launch_bounds__(kIxBlock) void stridx_buffer_kernel(StridxView v, c
 // The last dimension is contiguous in the view: rows of row_bytes move whole, as
 // 128-bit vectors where the row's address in the view allows. A row is cut into
 // segments of at most seg_vecs vectors; LPR lanes share one segment, four vectors each
-// per step. v.ndim counts the outer dimensions only. NT: non-temporal accesses on the
-// buffer side (touched exactly once; rows of the view may repeat), for copies larger
-// than the last-level cache.
+// per step. v.ndim counts the outer dimensions only. NT, for copies that stream past the
+// caches: non-temporal stores, and non-temporal loads from the buffer (touched exactly
+// once; rows read from the view may repeat, so those loads stay cached).
 struct StridxRows {
     uint32_t units;      // rows * segs_per_row  (< 2^31)
     uint32_t segs_per_row;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(kIxBlock) void stridx_rows_kernel(StridxView v, Str
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     if (b + k * LPR + lane < nv) {
-                        if (NT && TO_BUFFER) __builtin_nontemporal_store(x[k], d4 + (b + k * LPR + lane));
+                        if (NT) __builtin_nontemporal_store(x[k], d4 + (b + k * LPR + lane));
                         else d4[b + k * LPR + lane] = x[k];
                     }
                 }
@@ -270,7 +270,7 @@ void stridx_buffer_launch(const cumo_na_iarray_stridx_t* a, const cumo_na_indexe
                 uint64_t grid = (units + upb - 1) / upb;
                 if (grid > 256u * 64u) grid = 256u * 64u;
                 // one read and one write of every byte: past the 256 MB last-level cache, stream by it
-                const bool nt = 2 * rows * row_bytes > (320ull << 20);
+                const bool nt = stream_past_caches(2 * rows * row_bytes);
 #define IX_ROWS(L, N) hipLaunchKernelGGL((stridx_rows_kernel<TO_BUFFER, L, N>), dim3((unsigned)grid), dim3(kIxBlock), 0, stream, v, g, buf)
                 if (lpr == 16) { if (nt) IX_ROWS(16, true); else IX_ROWS(16, false); }
                 else if (lpr == 64) { if (nt) IX_ROWS(64, true); else IX_ROWS(64, false); }

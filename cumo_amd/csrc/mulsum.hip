@@ -224,7 +224,7 @@ bool mulsum_rows_launch(const cumo_hip_mulsum_rows_t* d) {
     uint64_t grid = (d->rows + rpb - 1) / rpb;
     if (grid > 256u * 64u) grid = 256u * 64u;
     // both operands streamed once and larger than the last-level cache together
-    const bool nt = d->row_step1 != 0 && d->row_step2 != 0 && 2 * d->rows * d->n * sizeof(T) > (320ull << 20);
+    const bool nt = d->row_step1 != 0 && d->row_step2 != 0 && stream_past_caches(2 * d->rows * d->n * sizeof(T));
     hipStream_t stream = current_stream();
 #define MS_ROWS(L, N) hipLaunchKernelGGL((mulsum_rows_kernel<T, NANF, L, N>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, g)
     if (lpr == 16) { if (nt) MS_ROWS(16, true); else MS_ROWS(16, false); }
@@ -253,7 +253,7 @@ void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, 
         partial = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * grid));
         if (!partial) return;
     }
-    const bool nt = 2 * n * sizeof(T) > (320ull << 20);
+    const bool nt = stream_past_caches(2 * n * sizeof(T));
     if (vec && nt)
         hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, true>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2,
                            n, chunk, partial, reinterpret_cast<T*>(p3));

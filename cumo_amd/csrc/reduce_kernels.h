@@ -534,21 +534,7 @@ static inline void red_fill_params(RedKParams* kp, const ReducePlan& plan, const
 // until they are needed again, and keeping them out leaves the caches to what can be
 // (measured with every launch on fresh data: 128 MiB of SFloat summed at 76% of the HBM
 // peak with plain loads, 82% with non-temporal ones; no difference at 32 MiB).
-constexpr uint64_t kRedNtBytes = 48ull << 20;
-
-static inline int red_nt_mode() {
-    static int mode = -2;
-    if (mode == -2) {
-        const char* e = std::getenv("CUMO_HIP_NT");
-        mode = e ? (std::atoi(e) != 0 ? 1 : 0) : -1;
-    }
-    return mode;
-}
-
-static inline bool red_use_nt(uint64_t bytes) {
-    const int mode = red_nt_mode();
-    return mode < 0 ? bytes > kRedNtBytes : mode != 0;
-}
+static inline bool red_use_nt(uint64_t bytes) { return stream_past_caches(bytes); }
 
 template <class Impl, bool PARTIAL, bool SCALAR_ONLY = false>
 static void red_launch_row(const RedKParams& kp, int vec, Impl impl, typename Impl::Acc* partial, hipStream_t stream) {

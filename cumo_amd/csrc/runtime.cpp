@@ -55,6 +55,14 @@ bool force_wide_indices() {
     return on;
 }
 
+bool stream_past_caches(uint64_t bytes) {
+    static const int mode = [] {
+        const char* e = std::getenv("CUMO_HIP_NT");
+        return e ? (std::atoi(e) != 0 ? 1 : 0) : -1;
+    }();
+    return mode < 0 ? bytes > kStreamNtBytes : mode != 0;
+}
+
 // Streams in use get a small number, for kernels that keep per-stream words in a
 // fixed device array (tickets that launches on different streams must not share).
 static std::mutex g_slot_lock;

@@ -1,6 +1,8 @@
 // CPU build of the SFloat / DFloat function cores of cumo_amd/csrc/ew_ops.h, for
-// tests/test_nmath_vectors.py. Every step of those algorithms is an IEEE operation
-// (fused multiply-adds included), so this program computes what the device computes.
+// tests/test_nmath_vectors.py. Every step of those algorithms is an IEEE operation (fused
+// multiply-adds included) except the device's reciprocal and reciprocal square root estimates,
+// which the algorithms refine by a Newton step to 2^-44 and for which the exact quotient and
+// root stand in here: this program computes what the device computes up to that.
 //
 //   float_cores_check vectors <file>   reads "name type n" blocks of arguments (hex bit
 //                                      patterns), prints the results as hex bit patterns
@@ -41,6 +43,8 @@ static const Core32 kCores32[] = {
     {"log10", log_float_rounded_once<10>, log10}, {"log1p", log1p_float_rounded_once, log1p}, {"tanh", tanh_float_rounded_once, tanh},
     {"sinh", sinh_float_rounded_once, sinh},  {"cosh", cosh_float_rounded_once, cosh},   {"expm1", expm1_float_rounded_once, expm1},
     {"asinh", asinh_float_rounded_once, asinh}, {"acosh", acosh_float_rounded_once, acosh}, {"atanh", atanh_float_rounded_once, atanh},
+    {"sin", trig_float_rounded_once<0>, sin}, {"cos", trig_float_rounded_once<1>, cos}, {"tan", trig_float_rounded_once<2>, tan},
+    {"atan", atan_float_rounded_once, atan},  {"erf", erf_float_rounded_once, erf},
 };
 struct Core64 { const char* name; F64 f; };
 static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>}};
