@@ -413,6 +413,9 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
 // for a plain copy the single vector is ahead, 164 us against 175 us).
 template <class O, class = void> struct op_is_heavy { static constexpr bool value = false; };
 template <class O> struct op_is_heavy<O, decltype((void)O::HEAVY)> { static constexpr bool value = O::HEAVY; };
+// Ops that declare HAS_RARE offer fast / rare / slow beside operator() (see ew_ops.h).
+template <class O, class = void> struct op_has_rare { static constexpr bool value = false; };
+template <class O> struct op_has_rare<O, decltype((void)O::HAS_RARE)> { static constexpr bool value = O::HAS_RARE; };
 
 template <class Op, int VEC, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restrict__ px, const char* __restrict__ py,
@@ -433,17 +436,64 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
     for (int u = 0; u < UNR; ++u) {
         const uint64_t i = i0 + (uint64_t)u * (kEwBlock * VEC);
         whole[u] = i + VEC <= n;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) { xv[u][j] = A(); yv[u][j] = B(); }
         if (whole[u]) {
             if (NIN >= 1) raw_load<A, VEC, NT>(px + i * sizeof(A), xv[u]);
             if (two_arrays) raw_load<B, VEC, NT>(py + i * sizeof(B), yv[u]);
         }
     }
+    // Every vector is evaluated, loaded or not (an absent one holds zeros and is not stored):
+    // with no branch around the arithmetic the compiler interleaves the elements of all the
+    // lane's vectors, which the long dependent chains of the NMath functions need.
+    R zv[UNR][VEC];
+    bool ok[UNR];
+    if constexpr (op_has_rare<Op>::value) {
+        // the arithmetic for every element first, then one loop (not unrolled: the out-of-line
+        // answer is called from one place, after the arithmetic has let go of its registers)
+        // over the lane's elements if any of them is of the rare kind
+        A xe[UNR * VEC];
+        B ye[UNR * VEC];
+        bool any = false;
 #pragma unroll
-    for (int u = 0; u < UNR; ++u) {
-        const uint64_t i = i0 + (uint64_t)u * (kEwBlock * VEC);
-        if (whole[u]) {
-            R zv[VEC];
-            bool ok = true;
+        for (int u = 0; u < UNR; ++u) {
+            ok[u] = true;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                A x = xv[u][j];
+                B y = B();
+                if (TWO) {
+                    if (use_scalar == 0) y = yv[u][j];
+                    else if (use_scalar == 1) y = (B)sv;
+                    else { y = (B)x; x = (A)sv; }
+                }
+                xe[u * VEC + j] = x;
+                ye[u * VEC + j] = y;
+                op.fast(x, y, zv[u][j]);
+                any = any || op.rare(x, y);
+            }
+        }
+        if (any) {
+#pragma clang loop unroll(disable)
+            for (int e = 0; e < UNR * VEC; ++e) {
+                A x = xe[0];
+                B y = ye[0];
+#pragma unroll
+                for (int q = 1; q < UNR * VEC; ++q) {
+                    x = (e == q) ? xe[q] : x;
+                    y = (e == q) ? ye[q] : y;
+                }
+                if (op.rare(x, y)) {
+                    const R r = op.slow(x, y);
+#pragma unroll
+                    for (int q = 0; q < UNR * VEC; ++q) zv[q / VEC][q % VEC] = (e == q) ? r : zv[q / VEC][q % VEC];
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            ok[u] = true;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 A x = (NIN >= 1) ? xv[u][j] : A();
@@ -453,13 +503,17 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
                     else if (use_scalar == 1) y = (B)sv;
                     else { y = (B)x; x = (A)sv; }
                 }
-                zv[j] = R();
-                ok = op(x, y, zv[j]) && ok;
+                zv[u][j] = R();
+                ok[u] = op(x, y, zv[u][j]) && ok[u];
             }
-            if (!Op::CHECKED || ok) {
-                raw_store<R, VEC, NT>(pz + i * sizeof(R), zv);
-                continue;
-            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const uint64_t i = i0 + (uint64_t)u * (kEwBlock * VEC);
+        if (whole[u] && (!Op::CHECKED || ok[u])) {
+            raw_store<R, VEC, NT>(pz + i * sizeof(R), zv[u]);
+            continue;
         }
         if (i >= n) continue;
         // the last, ragged vector of the run, or a vector with a rejected element: one by one

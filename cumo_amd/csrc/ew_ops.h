@@ -235,13 +235,14 @@ __device__ __forceinline__ double log_core_for_float(double x) {
 }
 template <int BASE>
 __device__ __forceinline__ float log_float_rounded_once(float xf) {
-    // a subnormal float is a normal double; zero, negative arguments, infinity and NaN take the branch
-    if (__float_as_uint(xf) - 1u >= 0x7f7fffffu) {
-        if (xf == 0.0f) return -INFINITY;
-        if (xf < 0.0f) return NAN;
-        return xf + xf;
-    }
-    return (float)log_core_for_float<BASE>((double)xf);
+    // No branch on the data, so that the elements of a vector are evaluated side by side. A
+    // subnormal float is a normal double. NaN comes back in through xf - xf (which is NaN for an
+    // infinity too); then, on the float: 0 -> -inf, negative -> NaN, +inf -> +inf
+    float y = (float)log_core_for_float<BASE>((double)xf) + (xf - xf);
+    y = (xf == 0.0f) ? -INFINITY : y;
+    y = (xf < 0.0f) ? NAN : y;
+    y = (xf == INFINITY) ? INFINITY : y;
+    return y;
 }
 // DFloat log, log2, log10: the same algorithm on a double argument (a subnormal one is
 // scaled by 2^54 first). Against glibc on 2 * 10^8 random doubles per function (all
@@ -345,17 +346,19 @@ __device__ __forceinline__ float expm1_float_rounded_once(float xf) {
     return (xf == 0.0f) ? xf : y;  // keeps the sign of a zero argument
 }
 // SFloat asinh, acosh, atanh: the function evaluated in double and rounded to float once, on the
-// logarithm above (the form for float results, refined reciprocal and square root). log(1 + u) for a double u >= 0 whose sum 1 + u is not exact: the part c
-// of u that the sum w loses comes back as c / w (c is below one ulp of w, so a float
-// reciprocal is more than enough). asinh|x| = log1p(a + a^2 / (1 + sqrt(1 + a^2))) and
-// acosh x = log1p(t + sqrt(t^2 + 2 t)), t = x - 1 (exact), hold over the whole float range
-// (a^2 and t^2 are exact in double and stay far below its overflow); atanh|x| =
-// log1p(2a / (1 - a)) / 2 with 1 - a exact, so that the quotient's half ulp is all the
-// argument's error. Below 2^-29 asinh and atanh round to the argument.
+// logarithm above (the form for float results, refined reciprocal and square root). log(1 + u)
+// for a double u >= 0 whose sum 1 + u is not exact: the part c of u that the sum w loses comes
+// back as c / w. asinh|x| = log1p(a + a^2 / (1 + sqrt(1 + a^2))) and acosh x =
+// log1p(t + sqrt(t^2 + 2 t)), t = x - 1 (exact), hold over the whole float range (a^2 and t^2
+// are exact in double and stay far below its overflow); atanh|x| = log1p(2a / (1 - a)) / 2 with
+// 1 - a exact. Below 2^-29 asinh and atanh round to the argument.
 __device__ __forceinline__ double log1p_core(double u) {
     const double w = 1.0 + u;
     const double c = u - (w - 1.0);
-    return __builtin_fma(c, (double)rcp_approx((float)w), log_core_for_float<0>(w));
+    // c / w: c is below 2^-53 w, so the term only counts where u is small, and there 1 / w = 1 - u
+    // will do (past u = 2^-10 it is below 2^-43 of the answer, past 1 it is left out)
+    const double um = (u < 1.0) ? u : 1.0;
+    return __builtin_fma(c, 1.0 - um, log_core_for_float<0>(w));
 }
 __device__ __forceinline__ float asinh_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);
@@ -394,13 +397,16 @@ __device__ __forceinline__ float atanh_float_rounded_once(float xf) {
 // z = r^2, from degree-4 and degree-3 fits (2^-35 and 2^-40 relative on |r| <= pi/4), both
 // evaluated, the quadrant choosing between them and the sign. Beyond that the device library's
 // double function (its argument reduction is a branch of its own). WHICH: 0 sin, 1 cos, 2 tan.
+// (out of line for the same reason as the library's pow further down)
 template <int WHICH>
-__device__ __forceinline__ float trig_float_rounded_once(float xf) {
-    if (!(__builtin_fabsf(xf) < 1.0e6f)) {   // large, infinite or NaN
-        if (WHICH == 0) return (float)sin((double)xf);
-        if (WHICH == 1) return (float)cos((double)xf);
-        return (float)tan((double)xf);
-    }
+__device__ __attribute__((noinline)) float trig_by_the_library(float xf) {
+    if (WHICH == 0) return (float)sin((double)xf);
+    if (WHICH == 1) return (float)cos((double)xf);
+    return (float)tan((double)xf);
+}
+// the arithmetic alone: right below 10^6 in magnitude, some finite number or NaN beyond
+template <int WHICH>
+__device__ __forceinline__ float trig_fast(float xf) {
     const double x = (double)xf;
     const double big = 6755399441055744.0;  // 1.5 * 2^52
     const double t = __builtin_fma(x, 6.36619772367581382433e-01, big);
@@ -420,16 +426,26 @@ __device__ __forceinline__ float trig_float_rounded_once(float xf) {
     pc = __builtin_fma(pc, z, -0.0013888887672811724);
     pc = __builtin_fma(pc, z, 0.04166666666432424);
     const double cs = __builtin_fma(z * z, pc, __builtin_fma(z, -0.5, 1.0));
+    float y;
     if (WHICH == 2) {
         const bool odd = (ki & 1u) != 0;
-        const float y = (float)((odd ? -cs : sn) * rcp_refined(odd ? sn : cs));
-        return (xf == 0.0f) ? xf : y;
+        y = (float)((odd ? -cs : sn) * rcp_refined(odd ? sn : cs));
+    } else {
+        // sin: quadrant 0 s, 1 c, 2 -s, 3 -c; cos is sin a quadrant further on
+        const uint32_t q = WHICH == 0 ? ki : ki + 1u;
+        const double v = (q & 1u) ? cs : sn;
+        y = (float)__hiloint2double(__double2hiint(v) ^ (int)((q & 2u) << 30), __double2loint(v));
     }
-    // sin: quadrant 0 s, 1 c, 2 -s, 3 -c; cos is sin a quadrant further on
-    const uint32_t q = WHICH == 0 ? ki : ki + 1u;
-    const double v = (q & 1u) ? cs : sn;
-    const float y = (float)__hiloint2double(__double2hiint(v) ^ (int)((q & 2u) << 30), __double2loint(v));
-    return (WHICH == 0 && xf == 0.0f) ? xf : y;
+    if (WHICH != 1) y = (xf == 0.0f) ? xf : y;  // keeps the sign of a zero argument
+    return y;
+}
+__device__ __forceinline__ bool trig_is_rare(float xf) { return !(__builtin_fabsf(xf) < 1.0e6f); }  // large, infinite or NaN
+template <int WHICH>
+__device__ __forceinline__ float trig_float_rounded_once(float xf) {
+    // the rare argument after the arithmetic, so that the elements of a vector are evaluated side by side
+    float y = trig_fast<WHICH>(xf);
+    if (trig_is_rare(xf)) y = trig_by_the_library<WHICH>(xf);
+    return y;
 }
 // SFloat atan, the same way: one refined reciprocal brings the argument below tan(pi/8)
 // (t = a there, (a - 1)/(a + 1) plus pi/4 up to tan(3 pi/8), -1/a plus pi/2 above), then
@@ -453,41 +469,29 @@ __device__ __forceinline__ float atan_float_rounded_once(float xf) {
     p = __builtin_fma(p, z, -0.33333333333270726);
     return __builtin_copysignf((float)(off + __builtin_fma(t * z, p, t)), xf);
 }
-// SFloat erf, the same way: below 1, erf a = a P(a^2) with a degree-8 fit (2^-40 relative);
-// from 1 on, erf a = 1 - exp(-a S(a)) with a degree-10 fit of S = -log(erfc a)/a on [1, 4]
-// (2^-41 absolute in erf) and exp(.) - 1 from the core above. In float, erf is 1 from 3.92 on.
+// SFloat erf, the same way, in one form over the whole range: erf a = 1 - exp(-a S(a)) with a
+// degree-14 fit of S = -log(erfc a) / a on [0, 4] (2^-41 relative in erf, near 0 included:
+// S(0) = 2/sqrt(pi)) and exp(.) - 1 from the core above, which keeps the small results whole.
+// In float, erf is 1 from 3.92 on.
 __device__ __forceinline__ float erf_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);
-    const double a = (double)af;
-    float y;
-    if (af < 1.0f) {
-        const double z = a * a;
-        double p = 1.0601184931822625e-06;
-        p = __builtin_fma(p, z, -1.3914064883994308e-05);
-        p = __builtin_fma(p, z, 0.00011957330950188644);
-        p = __builtin_fma(p, z, -0.0008542703072832773);
-        p = __builtin_fma(p, z, 0.00522378653090469);
-        p = __builtin_fma(p, z, -0.026866134013422204);
-        p = __builtin_fma(p, z, 0.11283791318349341);
-        p = __builtin_fma(p, z, -0.3761263889010029);
-        p = __builtin_fma(p, z, 1.128379167094713);
-        y = (float)(a * p);
-    } else {
-        const double ac = (af > 4.0f) ? 4.0 : a;  // a NaN passes
-        double sp = -1.0762777310949488e-07;
-        sp = __builtin_fma(sp, ac, 2.5858233440202685e-06);
-        sp = __builtin_fma(sp, ac, -2.8055149962875097e-05);
-        sp = __builtin_fma(sp, ac, 0.00017968025342242425);
-        sp = __builtin_fma(sp, ac, -0.0007285698386718862);
-        sp = __builtin_fma(sp, ac, 0.0016962354086159648);
-        sp = __builtin_fma(sp, ac, -2.9800151096382062e-05);
-        sp = __builtin_fma(sp, ac, -0.019378056134721402);
-        sp = __builtin_fma(sp, ac, 0.10294844019086533);
-        sp = __builtin_fma(sp, ac, 0.636553217738299);
-        sp = __builtin_fma(sp, ac, 1.1283899394236938);
-        y = (float)(-expm1_core(-ac * sp));
-    }
-    return __builtin_copysignf(y, xf);
+    const double a = (double)((af > 4.0f) ? 4.0f : af);  // a NaN passes
+    double sp = 1.2454485957275264e-09;
+    sp = __builtin_fma(sp, a, -3.292031665613006e-08);
+    sp = __builtin_fma(sp, a, 3.959960484006724e-07);
+    sp = __builtin_fma(sp, a, -2.8566560041378794e-06);
+    sp = __builtin_fma(sp, a, 1.3576807482500019e-05);
+    sp = __builtin_fma(sp, a, -4.281130444734605e-05);
+    sp = __builtin_fma(sp, a, 7.680414177713242e-05);
+    sp = __builtin_fma(sp, a, 1.7468095488586178e-05);
+    sp = __builtin_fma(sp, a, -0.0005860400176985031);
+    sp = __builtin_fma(sp, a, 0.0016948435469004315);
+    sp = __builtin_fma(sp, a, -0.00020889888424513057);
+    sp = __builtin_fma(sp, a, -0.019128485397176796);
+    sp = __builtin_fma(sp, a, 0.10277260588324502);
+    sp = __builtin_fma(sp, a, 0.6366197723000346);
+    sp = __builtin_fma(sp, a, 1.1283791670957979);
+    return __builtin_copysignf((float)(-expm1_core(-a * sp)), xf);
 }
 #define CUMO_HIP_OWN_OP(NAME, FEXPR, DEXPR)                                                                                 \
     template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
@@ -507,9 +511,22 @@ template <class T> struct OpExp { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) s
         return true; } };
 CUMO_HIP_FUN_H(OpExp2, exp2((double)x))
 CUMO_HIP_FUN_H(OpExp10, exp10((double)x))
-CUMO_HIP_OWN_OP(OpSin, trig_float_rounded_once<0>, sin((double)x))
-CUMO_HIP_OWN_OP(OpCos, trig_float_rounded_once<1>, cos((double)x))
-CUMO_HIP_OWN_OP(OpTan, trig_float_rounded_once<2>, tan((double)x))
+// SFloat ops whose arithmetic covers all but a rare kind of argument also offer the three parts
+// apart (fast: the arithmetic; rare: whether the argument is of that kind; slow: the out-of-line
+// answer for it), for kernels that evaluate a lane's elements first and mend the rare ones after.
+#define CUMO_HIP_TRIG_OP(NAME, WHICH, DEXPR)                                                                                \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
+        static constexpr bool HAS_RARE = sizeof(T) == 4;                                                                    \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const {                                                    \
+            if constexpr (sizeof(T) == 4) z = (T)trig_float_rounded_once<WHICH>((float)x);                                  \
+            else z = (T)(DEXPR);                                                                                            \
+            return true; }                                                                                                  \
+        __device__ __forceinline__ void fast(T x, T, T& z) const { z = (T)trig_fast<WHICH>((float)x); }                    \
+        __device__ __forceinline__ bool rare(T x, T) const { return trig_is_rare((float)x); }                              \
+        __device__ __forceinline__ T slow(T x, T) const { return (T)trig_by_the_library<WHICH>((float)x); } };
+CUMO_HIP_TRIG_OP(OpSin, 0, sin((double)x))
+CUMO_HIP_TRIG_OP(OpCos, 1, cos((double)x))
+CUMO_HIP_TRIG_OP(OpTan, 2, tan((double)x))
 CUMO_HIP_FUN_H(OpAsin, asin((double)x))
 CUMO_HIP_FUN_H(OpAcos, acos((double)x))
 CUMO_HIP_OWN_OP(OpAtan, atan_float_rounded_once, atan((double)x))
@@ -550,20 +567,30 @@ struct OpIAbs { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, true)
 // infinite, so the exponent's error stays below 2^-42) and the exp of the core above; everything
 // else (zero, negative, infinite or NaN base, infinite or NaN exponent: the sign, domain and
 // limit rules) is the device library's pow.
+// kept out of line: inlined next to every element it would spread the few instructions
+// that run over many times their size of instructions that almost never do
+__device__ __attribute__((noinline)) float pow_by_the_library(float xf, float yf) { return (float)pow((double)xf, (double)yf); }
+__device__ __forceinline__ float pow_fast(float xf, float yf) {
+    double p = (double)yf * log_core_for_float<0, true>((double)xf);
+    p = __builtin_fmin(__builtin_fmax(p, -110.0), 90.0);  // (a NaN only comes from a rare argument)
+    return (float)exp_core_for_float<false>(p);
+}
+__device__ __forceinline__ bool pow_is_rare(float xf, float yf) { return !(__float_as_uint(xf) - 1u < 0x7f7fffffu && __builtin_fabsf(yf) < INFINITY); }
 __device__ __forceinline__ float pow_float_rounded_once(float xf, float yf) {
-    if (__float_as_uint(xf) - 1u < 0x7f7fffffu && __builtin_fabsf(yf) < INFINITY) {
-        double p = (double)yf * log_core_for_float<0, true>((double)xf);
-        p = (p < -110.0) ? -110.0 : p;
-        p = (p > 90.0) ? 90.0 : p;
-        return (float)exp_core_for_float<false>(p);
-    }
-    return (float)pow((double)xf, (double)yf);
+    // the rare other case after the arithmetic, so that the elements of a vector are evaluated side by side
+    float z = pow_fast(xf, yf);
+    if (pow_is_rare(xf, yf)) z = pow_by_the_library(xf, yf);
+    return z;
 }
 template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) static constexpr bool HEAVY = true;
+    static constexpr bool HAS_RARE = sizeof(T) == 4;
     __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
         if constexpr (sizeof(T) == 4) z = (T)pow_float_rounded_once((float)x, (float)y);
         else z = (T)pow((double)x, (double)y);
-        return true; } };
+        return true; }
+    __device__ __forceinline__ void fast(T x, T y, T& z) const { z = (T)pow_fast((float)x, (float)y); }
+    __device__ __forceinline__ bool rare(T x, T y) const { return pow_is_rare((float)x, (float)y); }
+    __device__ __forceinline__ T slow(T x, T y) const { return (T)pow_by_the_library((float)x, (float)y); } };
 
 // Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
 // element type for small exponents, pow() beyond 64, the reciprocal for negative ones.
