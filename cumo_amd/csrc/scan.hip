@@ -20,6 +20,7 @@
 // from launch to launch.
 #include "common.h"
 
+#include <cstdlib>
 #include <cstring>
 
 namespace cumo_hip {
@@ -138,7 +139,7 @@ __device__ __forceinline__ void scan_tile(T (&v)[kScanPer], int cnt, T& carry, b
     has_carry = run_has;
 }
 
-template <class T>
+template <class T, bool NT = false>
 __device__ __forceinline__ void scan_load(const char* p, int64_t s, uint64_t first, int cnt, T (&v)[kScanPer]) {
     const int base = threadIdx.x * kScanPer;
     if (s == (int64_t)sizeof(T) && base + kScanPer <= cnt && ((reinterpret_cast<uintptr_t>(p) + (first + base) * sizeof(T)) & 15) == 0) {
@@ -147,7 +148,7 @@ __device__ __forceinline__ void scan_load(const char* p, int64_t s, uint64_t fir
         union { T t[kScanPer]; u4 q[NV]; } u;
         const u4* src = reinterpret_cast<const u4*>(p + (first + base) * sizeof(T));
 #pragma unroll
-        for (int i = 0; i < NV; ++i) u.q[i] = src[i];
+        for (int i = 0; i < NV; ++i) u.q[i] = NT ? __builtin_nontemporal_load(src + i) : src[i];
 #pragma unroll
         for (int k = 0; k < kScanPer; ++k) v[k] = u.t[k];
         return;
@@ -157,7 +158,7 @@ __device__ __forceinline__ void scan_load(const char* p, int64_t s, uint64_t fir
         if (base + k < cnt) v[k] = *reinterpret_cast<const T*>(p + (int64_t)(first + base + k) * s);
 }
 
-template <class T>
+template <class T, bool NT = false>
 __device__ __forceinline__ void scan_store(char* p, int64_t s, uint64_t first, int cnt, const T (&v)[kScanPer]) {
     const int base = threadIdx.x * kScanPer;
     if (s == (int64_t)sizeof(T) && base + kScanPer <= cnt && ((reinterpret_cast<uintptr_t>(p) + (first + base) * sizeof(T)) & 15) == 0) {
@@ -168,7 +169,10 @@ __device__ __forceinline__ void scan_store(char* p, int64_t s, uint64_t first, i
         for (int k = 0; k < kScanPer; ++k) u.t[k] = v[k];
         u4* dst = reinterpret_cast<u4*>(p + (first + base) * sizeof(T));
 #pragma unroll
-        for (int i = 0; i < NV; ++i) dst[i] = u.q[i];
+        for (int i = 0; i < NV; ++i) {
+            if (NT) __builtin_nontemporal_store(u.q[i], dst + i);
+            else dst[i] = u.q[i];
+        }
         return;
     }
 #pragma unroll
@@ -276,6 +280,429 @@ __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const char* in, 
         scan_tile<T, Op>(v, cnt, carry, hc);
         scan_store<T>(out, s_out, first, cnt, v);
     }
+}
+
+// ---- one long run in one pass ----------------------------------------------------
+// Every block takes the next tile from a ticket (so a tile only ever waits for tiles whose
+// blocks are already running), scans it in registers, publishes the tile's total and then
+// needs the total of everything before it. That comes in a fixed shape, so that results
+// do not change from launch to launch: tiles form groups of 64 and groups form supergroups
+// of 64; the last tile of a group also publishes the group's total and the last tile of a
+// supergroup the supergroup's. A tile folds, each with one wave-wide butterfly, the totals
+// of the earlier tiles of its group, of the earlier groups of its supergroup and of the
+// earlier supergroups. Reads the input once and writes the output once.
+// A published value travels as 64-bit words {1, 32 bits of the value}, stored and loaded
+// with agent-scope atomics: a word is there when its upper half is 1, no fence needed.
+// The words must be zero before the launch. A wait gives up after kChainSpinLimit polls
+// (it cannot be reached while every tile before this one has a running block); the count
+// of such give-ups is kept in g_scan_chain_gave_up.
+constexpr uint32_t kChainSpinLimit = 1u << 22;
+constexpr uint64_t kChainMaxTiles = 64ull * 64ull * 64ull;
+__device__ uint32_t g_scan_chain_gave_up;
+
+template <class T>
+struct ScanChain {
+    static constexpr int W = (int)(sizeof(T) / 4);
+    static constexpr int SUB = 64 / (int)sizeof(T) / 2;        // sub-tiles of the block-wide scan per tile: 64 KiB of elements
+    static constexpr int TILE = kScanTile * SUB;
+    uint32_t* ticket;
+    uint64_t* tile;    // [n_tiles * W]
+    uint64_t* group;   // [n_groups * W]
+    uint64_t* super;   // [n_supers * W]
+};
+
+template <class T>
+__device__ __forceinline__ void chain_publish(uint64_t* slot, T value) {
+    constexpr int W = ScanChain<T>::W;
+    union { T t; uint32_t w[W]; } u;
+    u.t = value;
+#pragma unroll
+    for (int i = 0; i < W; ++i)
+        __hip_atomic_store(slot + i, (1ull << 32) | u.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// one look at a published value: true when all of it is there
+template <class T>
+__device__ __forceinline__ bool chain_peek(const uint64_t* slot, T& value) {
+    constexpr int W = ScanChain<T>::W;
+    union { T t; uint32_t w[W]; } u;
+    uint64_t x[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) x[i] = __hip_atomic_load(slot + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool all = true;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+        all = all && (x[i] >> 32) != 0;
+        u.w[i] = (uint32_t)x[i];
+    }
+    value = u.t;
+    return all;
+}
+
+// (x, has) of the 64 lanes folded in a fixed shape; every lane ends with the result
+template <class T, class Op>
+__device__ __forceinline__ void chain_wave_fold(T& x, bool& has) {
+    const unsigned lane = threadIdx.x & 63u;
+#pragma unroll
+    for (unsigned m = 1; m < 64; m <<= 1) {
+        const T o = scan_shfl_xor(x, m);
+        const bool oh = __shfl_xor((int)has, (int)m) != 0;
+        if (oh) {
+            if (!has) x = o;
+            else x = (lane & m) ? Op::apply(o, x) : Op::apply(x, o);
+            has = true;
+        }
+    }
+}
+
+template <class T, class Op>
+__device__ __forceinline__ void chain_join(T& a, bool& a_has, T b, bool b_has) {  // a = a (+) b, a the earlier
+    if (b_has) {
+        a = a_has ? Op::apply(a, b) : b;
+        a_has = true;
+    }
+}
+
+template <class T>
+__device__ __forceinline__ T scan_shfl_idx(T v, int src) {
+    if constexpr (sizeof(T) == 8) {
+        union { T t; uint32_t w[2]; } a, b;
+        a.t = v;
+        b.w[0] = __shfl(a.w[0], src);
+        b.w[1] = __shfl(a.w[1], src);
+        return b.t;
+    } else {
+        union { T t; uint32_t w; } a, b;
+        a.t = v;
+        b.w = __shfl(a.w, src);
+        return b.t;
+    }
+}
+
+// What a tile needs from the tiles before it, through the published totals (wave 0 of the
+// block; every lane returns the same). Lane l wants the l-th earlier tile of this group, the
+// l-th earlier group of this supergroup and the l-th supergroup. Whatever this tile waits
+// for, the tile just before it publishes last, so one lane first polls that one word, with
+// pauses (64 lanes of every running block polling would flood the memory system); then every
+// lane looks at its own words, all in flight together, until they are there.
+template <class T, class Op>
+__device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t t, T total, bool total_has, T& prefix, bool& prefix_has) {
+    constexpr int W = ScanChain<T>::W;
+    const unsigned lane = threadIdx.x & 63u;
+    const uint32_t pos = t & 63u, g = t >> 6, gpos = g & 63u, sg = g >> 6;
+    if (lane == 0) chain_publish<T>(c.tile + (size_t)t * W, total);
+    T x = T(), y = T(), z = T();
+    const bool has_x = lane < pos, has_y = lane < gpos, has_z = lane < sg;
+    bool need_x = has_x, need_y = has_y, need_z = has_z;
+    const uint64_t* px = c.tile + (size_t)(g * 64u + lane) * W;
+    const uint64_t* py = c.group + (size_t)(sg * 64u + lane) * W;
+    const uint64_t* pz = c.super + (size_t)lane * W;
+    uint32_t polls = 0;
+    if (t > 0) {
+        // the last word that the tile before this one publishes
+        const uint64_t* latest = pos > 0 ? c.tile + (size_t)(t - 1) * W + (W - 1)
+                                         : (gpos > 0 ? c.group + (size_t)(g - 1) * W + (W - 1) : c.super + (size_t)(sg - 1) * W + (W - 1));
+        if (lane == 0) {
+            while ((__hip_atomic_load(latest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == 0) {
+                if (++polls > kChainSpinLimit) break;
+                __builtin_amdgcn_s_sleep(16);
+            }
+        }
+    }
+    // A tile that closes its group publishes the group's total as soon as the group's tiles
+    // are in, before it has everything it needs itself (and likewise the supergroup's):
+    // otherwise every group would wait for the group before it, one memory round trip each.
+    const bool closes_group = pos == 63u, closes_super = closes_group && gpos == 63u;
+    bool group_out = !closes_group, super_out = !closes_super;
+    bool xh = has_x, yh = has_y, zh = has_z;
+    bool x_folded = false, y_folded = false;
+    T gt = T();
+    bool gt_has = false;
+    for (;;) {
+        if (need_x) need_x = !chain_peek<T>(px, x);
+        if (need_y) need_y = !chain_peek<T>(py, y);
+        if (need_z) need_z = !chain_peek<T>(pz, z);
+        if (!x_folded && __ballot(need_x) == 0) {
+            chain_wave_fold<T, Op>(x, xh);
+            x_folded = true;
+            if (!group_out) {
+                gt = x;
+                gt_has = xh;
+                chain_join<T, Op>(gt, gt_has, total, total_has);
+                if (lane == 0) chain_publish<T>(c.group + (size_t)g * W, gt);
+                group_out = true;
+            }
+        }
+        if (!y_folded && x_folded && __ballot(need_y) == 0) {
+            chain_wave_fold<T, Op>(y, yh);
+            y_folded = true;
+            if (!super_out) {
+                T st = y;
+                bool st_has = yh;
+                chain_join<T, Op>(st, st_has, gt, gt_has);
+                if (lane == 0) chain_publish<T>(c.super + (size_t)sg * W, st);
+                super_out = true;
+            }
+        }
+        if (__ballot(need_x || need_y || need_z) == 0) break;
+        if (++polls > kChainSpinLimit) {
+            if (lane == 0) __hip_atomic_fetch_add(&g_scan_chain_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(16);
+    }
+    if (!x_folded) chain_wave_fold<T, Op>(x, xh);  // (only after giving up)
+    if (!y_folded) chain_wave_fold<T, Op>(y, yh);
+    chain_wave_fold<T, Op>(z, zh);
+    chain_join<T, Op>(z, zh, y, yh);
+    chain_join<T, Op>(z, zh, x, xh);
+    prefix = z;
+    prefix_has = zh;
+}
+
+// Both sides are contiguous and 16-byte aligned. A whole tile goes wave by wave: a wave owns a
+// quarter of the tile as R rows of 64 vectors, lane l holding vector l of every row (each load
+// and store covers 1 KiB without gaps); the rows are scanned side by side with shuffles, the
+// four waves meet once, in LDS, and what is left to add after the look-back is one value per
+// wave, so only the tile's elements stay in registers while the block waits. The ragged last
+// tile of a run goes sub-tile by sub-tile through the block-wide scan, reading its input twice.
+// Measured on 2^26 SFloat (fresh operands): 116 us with 64 KiB tiles, against 139 us with
+// 32 KiB tiles (twice the tickets and look-backs, each a trip through memory with nothing else
+// for the block to do), 155 us for the three launches, and 92 us for the same kernel with
+// neither ticket nor look-back. Blocks that keep a second tile's loads in flight while they
+// wait were slower still (170 us): the registers that takes cost more blocks than it wins.
+template <class T>
+struct ChainVec {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    static constexpr int V = 16 / (int)sizeof(T);
+    union { u4 q; T e[V]; };
+};
+
+struct ChainShared {
+    uint32_t tile;
+    int prefix_has;
+};
+
+template <class T, bool NT, int R>
+__device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first, ChainVec<T> (&v)[R]) {
+    typedef typename ChainVec<T>::u4 u4;
+    constexpr int V = ChainVec<T>::V;
+    const unsigned lane = threadIdx.x & 63u;
+    const int w = threadIdx.x >> 6;
+    const u4* src = reinterpret_cast<const u4*>(in + (first + (uint64_t)w * (R * 64 * V)) * sizeof(T)) + lane;
+#pragma unroll
+    for (int r = 0; r < R; ++r) v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
+}
+
+// The tile in v (already loaded) scanned by itself: afterwards every element holds the running
+// value from the start of its wave's quarter, `total` is the tile's total and `wave_pre` the
+// total of the waves before this one (for wave 0: nothing). One barrier, met by every thread.
+template <class T, class Op, int R>
+__device__ __forceinline__ void chain_scan_tile(ChainVec<T> (&v)[R], T* s_wave_tot, T& total, T& wave_pre) {
+    constexpr int V = ChainVec<T>::V;
+    const unsigned lane = threadIdx.x & 63u;
+    const int w = threadIdx.x >> 6;
+    T inc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int e = 1; e < V; ++e) v[r].e[e] = Op::apply(v[r].e[e - 1], v[r].e[e]);
+        inc[r] = v[r].e[V - 1];
+    }
+    // the lane totals of each row, scanned across the wave (the rows are independent)
+#pragma unroll
+    for (unsigned d = 1; d < 64; d <<= 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const T o = scan_shfl_up(inc[r], d);
+            if (lane >= d) inc[r] = Op::apply(o, inc[r]);
+        }
+    }
+    // every element takes on what precedes its vector inside the wave's quarter
+    T run = T();  // the rows so far
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const T ex = scan_shfl_up(inc[r], 1);       // the lanes before, in this row
+        const T row = scan_shfl_idx(inc[r], 63);    // the whole row
+        T before = ex;
+        if (r > 0) before = lane > 0 ? Op::apply(run, ex) : run;
+        if (r > 0 || lane > 0) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[r].e[e] = Op::apply(before, v[r].e[e]);
+        }
+        run = r == 0 ? row : Op::apply(run, row);
+    }
+    if (lane == 0) s_wave_tot[w] = run;
+    __syncthreads();
+    total = s_wave_tot[0];
+    wave_pre = T();
+#pragma unroll
+    for (int j = 1; j < kScanBlock / 64; ++j) {
+        if (j == w) wave_pre = total;
+        total = Op::apply(total, s_wave_tot[j]);
+    }
+}
+
+// adds what precedes the tile (if anything) and the earlier waves' total, and stores
+template <class T, class Op, bool NT, int R>
+__device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, ChainVec<T> (&v)[R], T head, bool head_has, T wave_pre) {
+    typedef typename ChainVec<T>::u4 u4;
+    constexpr int V = ChainVec<T>::V;
+    const unsigned lane = threadIdx.x & 63u;
+    const int w = threadIdx.x >> 6;
+    if (w > 0) {
+        head = head_has ? Op::apply(head, wave_pre) : wave_pre;
+        head_has = true;
+    }
+    u4* dst = reinterpret_cast<u4*>(out + (first + (uint64_t)w * (R * 64 * V)) * sizeof(T)) + lane;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (head_has) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[r].e[e] = Op::apply(head, v[r].e[e]);
+        }
+        if (NT) __builtin_nontemporal_store(v[r].q, dst + r * 64);
+        else dst[r * 64] = v[r].q;
+    }
+}
+
+// scans the tile in v (already loaded), looks back, stores; the barriers inside are met by every thread
+template <class T, class Op, bool NT, int R>
+__device__ __forceinline__ void chain_finish_tile(char* out, uint64_t first, uint32_t t, ChainVec<T> (&v)[R], const ScanChain<T>& c,
+                                                  T* s_wave_tot, T* s_prefix, ChainShared* sh) {
+    T total, wave_pre;
+    chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
+    if (threadIdx.x < 64) {
+        T pre;
+        bool pre_has;
+        chain_look_back<T, Op>(c, t, total, true, pre, pre_has);
+        if (threadIdx.x == 0) {
+            *s_prefix = pre;
+            sh->prefix_has = pre_has ? 1 : 0;
+        }
+    }
+    __syncthreads();
+    chain_store_tile<T, Op, NT, R>(out, first, v, *s_prefix, sh->prefix_has != 0, wave_pre);
+}
+
+// Many runs, each contiguous on both sides, 16-byte aligned and a whole number of chunks of
+// R * 256 vectors long: one block per run, chunk after chunk in the same wave-by-wave form,
+// the running value handed on in a register.
+template <class T, class Op, bool NT, int R>
+__global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsParams p) {
+    constexpr int V = ChainVec<T>::V;
+    constexpr uint64_t CHUNK = (uint64_t)R * kScanBlock * V;
+    __shared__ T s_wave_tot[kScanBlock / 64];
+    for (uint64_t row = blockIdx.x; row < p.rows; row += gridDim.x) {
+        int64_t oi = 0, oo = 0;
+        uint64_t q = row;
+        for (int d = p.nouter - 1; d >= 0; --d) {
+            const uint64_t m = p.oshape[d];
+            const uint64_t qq = q / m;
+            const int64_t k = (int64_t)(q - qq * m);
+            q = qq;
+            oi += k * p.ostep_in[d];
+            oo += k * p.ostep_out[d];
+        }
+        T carry = T();
+        bool has_carry = false;
+        for (uint64_t first = 0; first < p.n; first += CHUNK) {
+            ChainVec<T> v[R];
+            chain_issue_loads<T, NT, R>(p.in + oi, first, v);
+            T total, wave_pre;
+            chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
+            chain_store_tile<T, Op, NT, R>(p.out + oo, first, v, carry, has_carry, wave_pre);
+            carry = has_carry ? Op::apply(carry, total) : total;
+            has_carry = true;
+            __syncthreads();  // s_wave_tot is written again by the next chunk
+        }
+    }
+}
+
+template <class T, class Op, bool NT>
+__global__ __launch_bounds__(kScanBlock) void scan_chain_kernel(const char* in, char* out, uint64_t n, ScanChain<T> c) {
+    constexpr int TILE = ScanChain<T>::TILE;
+    constexpr int V = ChainVec<T>::V;
+    constexpr int R = TILE / (kScanBlock * V);
+    __shared__ ChainShared sh;
+    __shared__ T s_prefix;
+    __shared__ T s_wave_tot[kScanBlock / 64];
+    if (threadIdx.x == 0) sh.tile = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint32_t t = sh.tile;
+    const uint64_t first = (uint64_t)t * TILE;
+    if (first >= n) return;  // (the grid is exactly the tiles; a stray ticket does nothing)
+    if (n - first >= (uint64_t)TILE) {
+        ChainVec<T> v[R];
+        chain_issue_loads<T, NT, R>(in, first, v);
+        chain_finish_tile<T, Op, NT, R>(out, first, t, v, c, s_wave_tot, &s_prefix, &sh);
+        return;
+    }
+    // the ragged last tile: its total first, then the scan from what the look-back gives
+    T total = T();
+    bool total_has = false;
+#pragma clang loop unroll(disable)
+    for (uint64_t f = first; f < n; f += kScanTile) {
+        const uint64_t left = n - f;
+        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
+        T v[kScanPer];
+        scan_load<T>(in, (int64_t)sizeof(T), f, cnt, v);
+        scan_tile<T, Op>(v, cnt, total, total_has);
+    }
+    if (threadIdx.x < 64) {
+        T pre;
+        bool pre_has;
+        chain_look_back<T, Op>(c, t, total, total_has, pre, pre_has);
+        if (threadIdx.x == 0) {
+            s_prefix = pre;
+            sh.prefix_has = pre_has ? 1 : 0;
+        }
+    }
+    __syncthreads();
+    T carry = s_prefix;
+    bool has_carry = sh.prefix_has != 0;
+#pragma clang loop unroll(disable)
+    for (uint64_t f = first; f < n; f += kScanTile) {
+        const uint64_t left = n - f;
+        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
+        T v[kScanPer];
+        scan_load<T>(in, (int64_t)sizeof(T), f, cnt, v);
+        scan_tile<T, Op>(v, cnt, carry, has_carry);
+        scan_store<T>(out, (int64_t)sizeof(T), f, cnt, v);
+    }
+}
+
+__global__ __launch_bounds__(256) void scan_chain_clear_kernel(uint64_t* words, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) words[i] = 0;
+}
+
+// returns hipSuccess, or an error; -1 when the run does not suit this form
+template <class T, class Op>
+int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n, hipStream_t stream) {
+    constexpr int W = ScanChain<T>::W;
+    const uint64_t n_tiles = (n + ScanChain<T>::TILE - 1) / ScanChain<T>::TILE;
+    if (n_tiles < 64 || n_tiles > kChainMaxTiles) return -1;
+    if (s1 != (ssize_t)sizeof(T) || s2 != (ssize_t)sizeof(T) || (((uintptr_t)p1 | (uintptr_t)p2) & 15) != 0) return -1;
+    const uint64_t n_groups = (n_tiles + 63) / 64, n_supers = (n_groups + 63) / 64;
+    const uint64_t words = 1 + (n_tiles + n_groups + n_supers) * W;
+    uint64_t* ws = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(words * sizeof(uint64_t)));
+    if (!ws) return (int)hipErrorOutOfMemory;
+    uint64_t clear_grid = (words + 255) / 256;
+    if (clear_grid > 1024) clear_grid = 1024;
+    hipLaunchKernelGGL(scan_chain_clear_kernel, dim3((unsigned)clear_grid), dim3(256), 0, stream, ws, words);
+    ScanChain<T> c;
+    c.ticket = reinterpret_cast<uint32_t*>(ws);
+    c.tile = ws + 1;
+    c.group = c.tile + n_tiles * W;
+    c.super = c.group + n_groups * W;
+    const bool nt = stream_past_caches(2 * n * sizeof(T));
+    const uint64_t grid = n_tiles;
+    if (nt) hipLaunchKernelGGL((scan_chain_kernel<T, Op, true>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
+    else hipLaunchKernelGGL((scan_chain_kernel<T, Op, false>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
+    const int st = (int)hipGetLastError();
+    // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
+    cumo_cuda_runtime_free(reinterpret_cast<char*>(ws));
+    return st;
 }
 
 // ---- runs that lie across memory (the scan goes down the rows of a matrix) ------
@@ -487,10 +914,37 @@ void scan_rows_launch(const ScanRowsParams& p, hipStream_t stream) {
     if (p.rows == 0 || p.n == 0) return;
     uint64_t grid = p.rows;
     if (grid > 65536) grid = 65536;
+    constexpr uint64_t V = 16 / sizeof(T);
+    bool whole = p.s_in == (int64_t)sizeof(T) && p.s_out == (int64_t)sizeof(T) && p.n % (kScanBlock * V) == 0 &&
+                 (((uintptr_t)p.in | (uintptr_t)p.out) & 15) == 0;
+    for (int d = 0; d < p.nouter && whole; ++d) whole = (p.ostep_in[d] % 16) == 0 && (p.ostep_out[d] % 16) == 0;
+    if (whole) {
+        const uint64_t vec_rows = p.n / (kScanBlock * V);  // rows of 256 vectors in a run
+        const bool nt = stream_past_caches(2 * p.rows * p.n * sizeof(T));
+        const dim3 g((unsigned)grid), b(kScanBlock);
+#define CUMO_SCAN_WHOLE(R_) do { if (nt) hipLaunchKernelGGL((scan_rows_whole_kernel<T, Op, true, R_>), g, b, 0, stream, p); \
+                                 else hipLaunchKernelGGL((scan_rows_whole_kernel<T, Op, false, R_>), g, b, 0, stream, p); } while (0)
+        if (vec_rows % 8 == 0) CUMO_SCAN_WHOLE(8);
+        else if (vec_rows % 4 == 0) CUMO_SCAN_WHOLE(4);
+        else if (vec_rows % 2 == 0) CUMO_SCAN_WHOLE(2);
+        else CUMO_SCAN_WHOLE(1);
+#undef CUMO_SCAN_WHOLE
+        return;
+    }
     hipLaunchKernelGGL((scan_rows_kernel<T, Op>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p);
 }
 
-// One run of n elements. Short runs take one block; long ones the three launches.
+// CUMO_HIP_SCAN_CHAIN=0 (read once): long runs take the three launches instead of the one pass
+static bool scan_chain_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("CUMO_HIP_SCAN_CHAIN");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+// One run of n elements. Short runs take one block; from 64 tiles of 64 KiB on, contiguous and aligned, the one pass;
+// the three launches are what is left (runs beyond 2^30 elements, or the knob above).
 template <class T, class Op>
 int scan_run_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n) {
     if (n == 0) return 0;
@@ -507,6 +961,10 @@ int scan_run_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n
         p.out = p2;
         scan_rows_launch<T, Op>(p, stream);
         return (int)hipGetLastError();
+    }
+    if (scan_chain_enabled()) {
+        const int st = scan_chain_launch<T, Op>(p1, p2, s1, s2, n, stream);
+        if (st >= 0) return st;
     }
     // One tile per block keeps the most loads in flight (a block that walks a stretch of
     // tiles waits at two barriers per tile: measured 15 % slower). The totals are scanned

@@ -220,6 +220,79 @@ def test_cum_nan_forms_on_random_placements(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", ALL)
+def test_cum_along_contiguous_runs_of_whole_chunks(tname, dt):
+    """Many contiguous runs whose length is a whole number of 256 vectors take a kernel that
+    scans a run chunk by chunk in registers: one, two, four and eight rows of vectors per
+    chunk, one and several chunks per run, outer dimensions with padding between the runs.
+    Small integers (float sums exact in any order): bit for bit against the sequential scan."""
+    cls = cls_of(tname)
+    rng = np.random.default_rng(59)
+    per = 256 * (16 // np.dtype(dt).itemsize)
+    for shape in [(33, per), (7, 3 * per), (5, 2 * per), (6, 4 * per), (5, 8 * per), (3, 16 * per), (4, 6, 2 * per), (3, 24 * per)]:
+        h = rng.integers(-3, 4, size=shape).astype(dt)
+        if dt != np.int32:
+            h[..., ::3] = 0
+        d = cls.cast(h)
+        assert_bits_equal(d.cumsum(axis=-1).to_numpy(), oracle.cum("cumsum", h, axis=len(shape) - 1), (shape, "cumsum"))
+        f = rng.choice(np.array([1, -1], dtype=dt), size=shape)
+        f.reshape(-1)[rng.integers(0, f.size, 12)] = 2
+        assert_bits_equal(cls.cast(f).cumprod(axis=-1).to_numpy(), oracle.cum("cumprod", f, axis=len(shape) - 1), (shape, "cumprod"))
+        if dt != np.int32:
+            g = h.copy()
+            g.reshape(-1)[rng.integers(0, g.size, 200)] = np.nan
+            g[0, ..., :700] = np.nan
+            d = cls.cast(g)
+            assert_bits_equal(d.cumsum(axis=-1, nan=True).to_numpy(), oracle.cum("cumsum", g, axis=len(shape) - 1, nan=True), (shape, "nan: true"))
+            assert_bits_equal(d.cumsum(axis=-1).to_numpy(), oracle.cum("cumsum", g, axis=len(shape) - 1), (shape, "NaN carried"))
+        if len(shape) == 2:
+            # every other run of a wider array: the runs stay contiguous, the step between them doubles
+            wide = rng.integers(-3, 4, size=(2 * shape[0], shape[1])).astype(dt)
+            hv = np.ascontiguousarray(wide[::2])
+            assert_bits_equal(cls.cast(wide)[::2].cumsum(axis=1).to_numpy(), oracle.cum("cumsum", hv, axis=1), (shape, "every other run"))
+
+
+@pytest.mark.parametrize("tname,dt", ALL)
+def test_one_long_run_in_one_pass(tname, dt):
+    """Runs from 64 tiles of 64 KiB on are scanned in one pass, tiles handing their
+    totals on through groups of 64 and supergroups of 64 groups: sizes that end exactly on a
+    group, one element past it, inside the second supergroup; small integers (float sums
+    exact in any order), so every result is compared bit for bit with the sequential scan.
+    Then what only the order-free comparison can hold: products of +-1 and 2, NaN skipped
+    (the run starts with a tile of nothing but NaN) and carried, a strided view on each side,
+    and the same call twice giving the same bits on random floats."""
+    cls = cls_of(tname)
+    rng = np.random.default_rng(57)
+    tile = 65536 // np.dtype(dt).itemsize
+    for n in (64 * tile, 64 * tile + 1, 65 * tile + 3001, 64 * 64 * tile + 70001):
+        h = rng.integers(-3, 4, size=n).astype(dt)
+        if dt != np.int32:
+            h[::3] = 0   # keeps the running float sums far below 2^24
+        d = cls.cast(h)
+        assert_bits_equal(d.cumsum().to_numpy(), oracle.cum("cumsum", h), (n, "cumsum"))
+    n = 64 * tile * 3 + 17
+    f = rng.choice(np.array([1, -1], dtype=dt), size=n)
+    f[rng.integers(0, n, 25)] = 2
+    assert_bits_equal(cls.cast(f).cumprod().to_numpy(), oracle.cum("cumprod", f), "cumprod")
+    h = rng.integers(-3, 4, size=2 * n).astype(dt)
+    hv = np.ascontiguousarray(h[::2])
+    assert_bits_equal(cls.cast(h)[::2].cumsum().to_numpy(), oracle.cum("cumsum", hv), "strided input")
+    if dt != np.int32:
+        g = rng.integers(-3, 4, size=n).astype(dt)
+        g[rng.integers(0, n, 3000)] = np.nan
+        g[:5000] = np.nan
+        d = cls.cast(g)
+        assert_bits_equal(d.cumsum(nan=True).to_numpy(), oracle.cum("cumsum", g, nan=True), "nan: true")
+        assert_bits_equal(d.cumsum().to_numpy(), oracle.cum("cumsum", g), "NaN carried")
+        r = rng.standard_normal(n).astype(dt)
+        d = cls.cast(r)
+        first = d.cumsum().to_numpy()
+        for _ in range(3):
+            assert_bits_equal(d.cumsum().to_numpy(), first, "same bits from launch to launch")
+        exact = np.cumsum(r.astype(np.float64)) if dt == np.float32 else np.asarray(np.cumsum(r.astype(np.longdouble))).astype(np.float64)
+        _cum_close(first, exact, np.cumsum(np.abs(r).astype(np.float64)), n, dt, "random floats")
+
+
+@pytest.mark.parametrize("tname,dt", ALL)
 def test_cum_along_columns_of_tall_wide_and_stacked_arrays(tname, dt):
     """Runs that lie across memory: few segments (the second pass folds their totals
     itself), many (the totals are scanned first, by the same routine), several planes.
