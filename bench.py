@@ -204,7 +204,7 @@ def config_ops(name, cumo, host):
         env = {"xs": cumo.SFloat.cast(x), "xd": cumo.DFloat.cast(x.astype(np.float64))}
         env["xs2"] = env["xs"].reshape(8192, n // 8192)
         ops = []
-        for fname in ("log", "sin", "cos", "tan", "tanh", "erf", "asinh", "atan", "exp", "sqrt"):
+        for fname in ("log", "sin", "cos", "tan", "tanh", "erf", "asinh", "atan", "exp", "sqrt", "log1p", "sinh", "erfc", "cbrt"):
             ops.append(("NMath.%s(SFloat)" % fname, (lambda f: lambda e: e.__setitem__("r", getattr(NM, f)(e["xs"])))(fname), 8 * n, n))
         for fname in ("log", "sin", "tanh", "erf", "exp", "sqrt"):
             ops.append(("NMath.%s(DFloat)" % fname, (lambda f: lambda e: e.__setitem__("rd", getattr(NM, f)(e["xd"])))(fname), 16 * n, n))

@@ -122,8 +122,8 @@ CUMO_HIP_FUN(OpSqrt, sqrt((double)x))
 CUMO_HIP_FUN_H(OpCbrt, cbrt((double)x))
 // SFloat exp: the double-precision exp of the argument, rounded to float once.
 // The argument has 24 significant bits, so k = rint(x / ln 2) times the upper part
-// of ln 2 is exact; exp(r) on |r| <= ln(2)/2 is the Taylor polynomial of degree 13
-// (truncation below 2^-57), scaled by 2^k. Only full-rate instructions besides the
+// of ln 2 is exact; exp(r) on |r| <= ln(2)/2 is a degree-10 polynomial (2^-50; four
+// multiply-adds fewer than the Taylor polynomial of the same accuracy), scaled by 2^k. Only full-rate instructions besides the
 // two conversions: k is rounded by adding 1.5 * 2^52 (its integer value is then
 // the low word of the sum), and 2^k is applied by adding k to the exponent field,
 // which is safe because the clamp keeps the result a normal double. Outside
@@ -141,14 +141,16 @@ __device__ __forceinline__ float exp_float_rounded_once(float xf) {
     const int ki = (int)(uint32_t)__double_as_longlong(t);
     double r = __builtin_fma(k, -6.93147180369123816490e-01, x);  // ln 2, upper 32 bits
     r = __builtin_fma(k, -1.90821492927058770002e-10, r);         // ln 2, the rest
-    const double c[12] = {
-        1.60590438368216133e-10 /* 1/13! */, 2.08767569878681002e-09 /* 1/12! */, 2.50521083854417202e-08 /* 1/11! */,
-        2.75573192239858883e-07 /* 1/10! */, 2.75573192239858925e-06 /* 1/9! */,  2.48015873015873016e-05 /* 1/8! */,
-        1.98412698412698413e-04 /* 1/7! */,  1.38888888888888894e-03 /* 1/6! */,  8.33333333333333322e-03 /* 1/5! */,
-        4.16666666666666644e-02 /* 1/4! */,  1.66666666666666657e-01 /* 1/3! */,  5.00000000000000000e-01 /* 1/2! */};
-    double p = c[0];
-#pragma unroll
-    for (int i = 1; i < 12; ++i) p = __builtin_fma(p, r, c[i]);
+    // exp(r) = 1 + r (1 + r E(r)) with a degree-8 fit of E = (exp(r) - 1 - r) / r^2 (2^-50 relative on |r| <= ln(2)/2)
+    double p = 2.762343374154865e-07;
+    p = __builtin_fma(p, r, 2.7625077174598027e-06);
+    p = __builtin_fma(p, r, 2.480151290638607e-05);
+    p = __builtin_fma(p, r, 0.00019841208813878425);
+    p = __builtin_fma(p, r, 0.00138888889238219);
+    p = __builtin_fma(p, r, 0.008333333353676958);
+    p = __builtin_fma(p, r, 0.04166666666660734);
+    p = __builtin_fma(p, r, 0.16666666666648428);
+    p = __builtin_fma(p, r, 0.5000000000000002);
     p = __builtin_fma(p, r, 1.0);
     p = __builtin_fma(p, r, 1.0);
     const int hi = __double2hiint(p) + (ki << 20);
@@ -404,9 +406,10 @@ __device__ __attribute__((noinline)) float trig_by_the_library(float xf) {
     if (WHICH == 1) return (float)cos((double)xf);
     return (float)tan((double)xf);
 }
-// the arithmetic alone: right below 10^6 in magnitude, some finite number or NaN beyond
+// the arithmetic alone, before the rounding to float: right below 10^6 in magnitude, some
+// finite number or NaN beyond
 template <int WHICH>
-__device__ __forceinline__ float trig_fast(float xf) {
+__device__ __forceinline__ double trig_core(float xf) {
     const double x = (double)xf;
     const double big = 6755399441055744.0;  // 1.5 * 2^52
     const double t = __builtin_fma(x, 6.36619772367581382433e-01, big);
@@ -426,18 +429,19 @@ __device__ __forceinline__ float trig_fast(float xf) {
     pc = __builtin_fma(pc, z, -0.0013888887672811724);
     pc = __builtin_fma(pc, z, 0.04166666666432424);
     const double cs = __builtin_fma(z * z, pc, __builtin_fma(z, -0.5, 1.0));
-    float y;
     if (WHICH == 2) {
         const bool odd = (ki & 1u) != 0;
-        y = (float)((odd ? -cs : sn) * rcp_refined(odd ? sn : cs));
-    } else {
-        // sin: quadrant 0 s, 1 c, 2 -s, 3 -c; cos is sin a quadrant further on
-        const uint32_t q = WHICH == 0 ? ki : ki + 1u;
-        const double v = (q & 1u) ? cs : sn;
-        y = (float)__hiloint2double(__double2hiint(v) ^ (int)((q & 2u) << 30), __double2loint(v));
+        return (odd ? -cs : sn) * rcp_refined(odd ? sn : cs);
     }
-    if (WHICH != 1) y = (xf == 0.0f) ? xf : y;  // keeps the sign of a zero argument
-    return y;
+    // sin: quadrant 0 s, 1 c, 2 -s, 3 -c; cos is sin a quadrant further on
+    const uint32_t q = WHICH == 0 ? ki : ki + 1u;
+    const double v = (q & 1u) ? cs : sn;
+    return __hiloint2double(__double2hiint(v) ^ (int)((q & 2u) << 30), __double2loint(v));
+}
+template <int WHICH>
+__device__ __forceinline__ float trig_fast(float xf) {
+    const float y = (float)trig_core<WHICH>(xf);
+    return (WHICH != 1 && xf == 0.0f) ? xf : y;  // keeps the sign of a zero argument
 }
 __device__ __forceinline__ bool trig_is_rare(float xf) { return !(__builtin_fabsf(xf) < 1.0e6f); }  // large, infinite or NaN
 template <int WHICH>
@@ -469,6 +473,40 @@ __device__ __forceinline__ float atan_float_rounded_once(float xf) {
     p = __builtin_fma(p, z, -0.33333333333270726);
     return __builtin_copysignf((float)(off + __builtin_fma(t * z, p, t)), xf);
 }
+// SFloat asin, acos, the same way: up to 1/2, asin a = a + a z P(z), z = a^2, with a degree-8 fit
+// of P (2^-42 relative on z <= 1/4); beyond, the same series at s = sqrt((1 - a) / 2) (1 - a is
+// exact, the square root refined) gives asin a = pi/2 - 2 asin s. acos x is 2 asin s above 1/2,
+// pi - 2 asin s below -1/2 and pi/2 - asin x between.
+template <bool ACOS>
+__device__ __forceinline__ float asin_acos_float_rounded_once(float xf) {
+    const float af = __builtin_fabsf(xf);
+    const double a = (double)af;
+    const bool outer = af > 0.5f;
+    const double z = outer ? 0.5 * (1.0 - a) : a * a;
+    const bool z_pos = z > 0.0;
+    double s = sqrt_refined((outer && z_pos) ? z : 1.0);
+    s = outer ? (z_pos ? s : 0.0) : a;     // (|x| = 1: s = 0; |x| > 1 is settled below; a NaN passes through a)
+    double p = 0.02857943531987056;
+    p = __builtin_fma(p, z, 0.0008360525284043926);
+    p = __builtin_fma(p, z, 0.01695759046734276);
+    p = __builtin_fma(p, z, 0.016883023346408812);
+    p = __builtin_fma(p, z, 0.022414706851110307);
+    p = __builtin_fma(p, z, 0.030379800562048823);
+    p = __builtin_fma(p, z, 0.04464291095965551);
+    p = __builtin_fma(p, z, 0.0749999994813725);
+    p = __builtin_fma(p, z, 0.16666666666748844);
+    const double as = __builtin_fma(s * z, p, s);   // asin s
+    const double pio2 = 1.57079632679489655800e+00, pi = 3.14159265358979311600e+00;
+    float y;
+    if (ACOS) {
+        const double neg = (xf < 0.0f) ? -as : as;
+        const double r = outer ? ((xf < 0.0f) ? pi - 2.0 * as : 2.0 * as) : pio2 - neg;
+        y = (float)r;
+    } else {
+        y = __builtin_copysignf((float)(outer ? pio2 - 2.0 * as : as), xf);
+    }
+    return (af > 1.0f) ? NAN : y;
+}
 // SFloat erf, the same way, in one form over the whole range: erf a = 1 - exp(-a S(a)) with a
 // degree-14 fit of S = -log(erfc a) / a on [0, 4] (2^-41 relative in erf, near 0 included:
 // S(0) = 2/sqrt(pi)) and exp(.) - 1 from the core above, which keeps the small results whole.
@@ -492,6 +530,34 @@ __device__ __forceinline__ float erf_float_rounded_once(float xf) {
     sp = __builtin_fma(sp, a, 0.6366197723000346);
     sp = __builtin_fma(sp, a, 1.1283791670957979);
     return __builtin_copysignf((float)(-expm1_core(-a * sp)), xf);
+}
+// SFloat erfc, the same way: erfc a = t exp(-a^2 + P(t)), t = 2 / (2 + a), with a degree-16 fit
+// of P on 0 <= a <= 10.2 (2^-39 relative in erfc; a^2 is exact in double, and beyond 10.06 the
+// float answer is 0); erfc(-a) = 2 - erfc a.
+__device__ __forceinline__ float erfc_float_rounded_once(float xf) {
+    const float af = __builtin_fabsf(xf);
+    const double a = (double)((af > 10.2f) ? 10.2f : af);  // a NaN passes
+    const double t = 2.0 * rcp_refined(2.0 + a);
+    double p = 0.08559139243524283;
+    p = __builtin_fma(p, t, -0.6542044248194727);
+    p = __builtin_fma(p, t, 1.9990352510531308);
+    p = __builtin_fma(p, t, -2.5941568730621682);
+    p = __builtin_fma(p, t, -0.8737363806023866);
+    p = __builtin_fma(p, t, 8.652953555628644);
+    p = __builtin_fma(p, t, -14.909187280785874);
+    p = __builtin_fma(p, t, 14.312468419074285);
+    p = __builtin_fma(p, t, -9.029793572490398);
+    p = __builtin_fma(p, t, 4.291175130459545);
+    p = __builtin_fma(p, t, -1.5542215474097043);
+    p = __builtin_fma(p, t, 0.22800239714528087);
+    p = __builtin_fma(p, t, -0.1551378787683726);
+    p = __builtin_fma(p, t, 0.09249811135208773);
+    p = __builtin_fma(p, t, 0.3741830048987767);
+    p = __builtin_fma(p, t, 1.000043891501855);
+    p = __builtin_fma(p, t, -1.2655131956093486);
+    const double e = t * exp_core_for_float<false>(__builtin_fma(-a, a, p));
+    const float y = (float)((xf < 0.0f) ? 2.0 - e : e);
+    return (xf != xf) ? xf : y;
 }
 #define CUMO_HIP_OWN_OP(NAME, FEXPR, DEXPR)                                                                                 \
     template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
@@ -527,17 +593,23 @@ CUMO_HIP_FUN_H(OpExp10, exp10((double)x))
 CUMO_HIP_TRIG_OP(OpSin, 0, sin((double)x))
 CUMO_HIP_TRIG_OP(OpCos, 1, cos((double)x))
 CUMO_HIP_TRIG_OP(OpTan, 2, tan((double)x))
-CUMO_HIP_FUN_H(OpAsin, asin((double)x))
-CUMO_HIP_FUN_H(OpAcos, acos((double)x))
+CUMO_HIP_OWN_OP(OpAsin, asin_acos_float_rounded_once<false>, asin((double)x))
+CUMO_HIP_OWN_OP(OpAcos, asin_acos_float_rounded_once<true>, acos((double)x))
 CUMO_HIP_OWN_OP(OpAtan, atan_float_rounded_once, atan((double)x))
 CUMO_HIP_OWN_OP(OpAsinh, asinh_float_rounded_once, asinh((double)x))
 CUMO_HIP_OWN_OP(OpAcosh, acosh_float_rounded_once, acosh((double)x))
 CUMO_HIP_OWN_OP(OpAtanh, atanh_float_rounded_once, atanh((double)x))
 // the host macro guards x == 0 (types/float_macro.h:113); the reference's device
 // macro does not and answers NaN there, which Numo does not
-CUMO_HIP_FUN_H(OpSinc, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
+__device__ __attribute__((noinline)) float sinc_by_the_library(float xf) { return (float)(sin((double)xf) / (double)xf); }
+__device__ __forceinline__ float sinc_float_rounded_once(float xf) {
+    float y = (float)(trig_core<0>(xf) * rcp_refined((double)xf));
+    if (trig_is_rare(xf)) y = sinc_by_the_library(xf);
+    return (xf == 0.0f) ? 1.0f : y;
+}
+CUMO_HIP_OWN_OP(OpSinc, sinc_float_rounded_once, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
 CUMO_HIP_OWN_OP(OpErf, erf_float_rounded_once, erf((double)x))
-CUMO_HIP_FUN_H(OpErfc, erfc((double)x))
+CUMO_HIP_OWN_OP(OpErfc, erfc_float_rounded_once, erfc((double)x))
 
 #define CUMO_HIP_IUN(NAME, EXPR) \
     struct NAME { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false) \

@@ -35,6 +35,7 @@ static inline float __uint_as_float(unsigned u) { float f; std::memcpy(&f, &u, 4
 
 using namespace cumo_hip;
 
+static double sinc_ref(double x) { return x == 0 ? 1.0 : std::sin(x) / x; }
 typedef float (*F32)(float);
 typedef double (*F64)(double);
 struct Core32 { const char* name; F32 f; F64 ref; };
@@ -45,6 +46,8 @@ static const Core32 kCores32[] = {
     {"asinh", asinh_float_rounded_once, asinh}, {"acosh", acosh_float_rounded_once, acosh}, {"atanh", atanh_float_rounded_once, atanh},
     {"sin", trig_float_rounded_once<0>, sin}, {"cos", trig_float_rounded_once<1>, cos}, {"tan", trig_float_rounded_once<2>, tan},
     {"atan", atan_float_rounded_once, atan},  {"erf", erf_float_rounded_once, erf},
+    {"asin", asin_acos_float_rounded_once<false>, asin}, {"acos", asin_acos_float_rounded_once<true>, acos},
+    {"erfc", erfc_float_rounded_once, erfc},  {"sinc", sinc_float_rounded_once, sinc_ref},
 };
 struct Core64 { const char* name; F64 f; };
 static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>}};
