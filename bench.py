@@ -38,7 +38,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-ADD_KERNEL = "ew_rows2_kernel<OpAdd<double>, 2, 5>"
+ADD_KERNEL = "ew_rows2_lean_kernel<OpAdd<double>, 2, 5>"
 # HBM bytes per launch of the C2 broadcast add come from two rocprofv3 --pmc runs of this
 # file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by the same counter's
 # reading for --pmc-calibration's plain 256 MiB copy. The summary of those runs is kept in
