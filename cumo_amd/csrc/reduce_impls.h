@@ -189,7 +189,8 @@ struct MomentsImpl {
         if (acc.n == (T)0) { acc = next; return; }
         const T n = acc.n + next.n;
         const T delta = next.mean - acc.mean;
-        const T w = next.n / n;
+        // equal counts (every step of the combine across lanes that hold equal shares): no division
+        const T w = (next.n == acc.n) ? (T)0.5 : next.n / n;
         acc.mean = acc.mean + delta * w;
         acc.m2 += next.m2 + delta * delta * acc.n * w;
         acc.n = n;
@@ -244,15 +245,19 @@ struct MomentsImpl {
 #pragma unroll
         for (int u = 1; u < U; ++u) s = s + part[u];
         const T mb = s * ((T)1 / (T)M);
-        T m2 = (T)0;
+        T q[U];   // one chain of additions per vector, so that they run side by side
 #pragma unroll
         for (int u = 0; u < U; ++u) {
+            q[u] = (T)0;
 #pragma unroll
             for (int k = 0; k < N; ++k) {
                 const T d = x[u][k] - mb;
-                m2 = m2 + d * d;
+                q[u] = q[u] + d * d;
             }
         }
+        T m2 = q[0];
+#pragma unroll
+        for (int u = 1; u < U; ++u) m2 = m2 + q[u];
         combine(Acc{(T)M, mb, m2}, acc);
     }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
