@@ -44,7 +44,7 @@ ADD_KERNEL = "ew_rows2_lean_kernel<OpAdd<double>, 2, 5>"
 # reading for --pmc-calibration's plain 256 MiB copy. The summary of those runs is kept in
 # this file, and the line that starts with TRAFFIC_KEY carries the figure; it is read from
 # there (never typed in here), and reported as null when the summary is absent.
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "ew_rows2_add_f64_c2_hbm_traffic.txt")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "ew_rows2_lean_add_f64_c2_hbm_traffic.txt")
 TRAFFIC_KEY = "traffic_bytes_per_launch"
 
 
