@@ -31,6 +31,8 @@ void pool_retire_stream(hipStream_t stream);
 // Device address of the reduction ticket words of a stream slot (zero between launches),
 // nullptr after reporting an error. reduce_tickets.hip.
 uint32_t* red_ticket_words(int slot);
+// the slot's hand-over words for one launch of a full reduction, and that launch's number (never 0)
+uint64_t* red_handover_words(int slot, uint32_t* launch_number);
 
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)

@@ -611,6 +611,15 @@ static inline bool red_stream_enabled() {
     return on != 0;
 }
 
+// CUMO_HIP_RED_POLL=0 (read once): full reductions take the ticket form
+static bool red_poll_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("CUMO_HIP_RED_POLL");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 // The lean kernels of reduce_stream.h for the layouts they take. Returns 1 when the
 // reduction has been launched, 0 when the general kernels must take it, -1 when the
 // caller's fixed scratch is too small (nothing launched).
@@ -706,6 +715,18 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     const uint64_t tiles = (plan.red_total + tile - 1) / tile;
     p.n_split = (uint32_t)((uint64_t)plan.n_split < tiles ? (uint64_t)plan.n_split : tiles);
     if (p.n_split <= 1) return 0;
+    // one output (a full reduction): the form without tickets, when the accumulators fit the hand-over words
+    if (plan.out_total == 1 && !fixed && red_poll_enabled() && (uint64_t)p.n_split * (sizeof(Acc) / 4) <= kRsHandoverWords) {
+        uint32_t launch = 0;
+        uint64_t* words = red_handover_words(stream_slot(stream), &launch);
+        if (words != nullptr) {
+            const dim3 g((unsigned)p.n_split + 1u);
+            if (nt) hipLaunchKernelGGL((red_srow_poll_kernel<Impl, V, true>), g, b, 0, stream, p, impl, words, launch);
+            else hipLaunchKernelGGL((red_srow_poll_kernel<Impl, V, false>), g, b, 0, stream, p, impl, words, launch);
+            cumo_cuda_runtime_check_kernel_launch();
+            return 1;
+        }
+    }
     p.group = p.n_split <= (uint32_t)kRsOneLevel ? p.n_split : (uint32_t)kRsGroup;
     const uint64_t groups = (p.n_split + p.group - 1) / p.group;
     {

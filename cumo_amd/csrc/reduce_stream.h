@@ -303,6 +303,100 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
     }
 }
 
+// One output, the axis cut over n_split blocks, one launch, no tickets: block 0 reads nothing of
+// the input; it waits for the other blocks' accumulators, which arrive as 64-bit words {launch
+// number, 32 bits of the accumulator} written with agent-scope atomic stores, and folds them in
+// index order as the split form above does. The chain after the last block has finished its
+// part is then one store becoming visible and one look at it, instead of store, acknowledgement,
+// two tickets in turn, fence and loads (C3 T.sum(): 25.5 -> see the measurements). A streaming
+// block never waits for anything, so block 0 (which the dispatcher starts first) cannot hold
+// the others up; its wait gives up after kRsPollLimit looks (the count of that is kept).
+constexpr uint32_t kRsHandoverWords = 8192;
+constexpr uint32_t kRsPollLimit = 1u << 24;
+__device__ uint32_t g_red_poll_gave_up;
+
+template <class Acc>
+__device__ __forceinline__ Acc rs_await(const uint64_t* slot, uint32_t launch) {
+    constexpr int W = sizeof(Acc) / 4;
+    union U {
+        Acc a;
+        uint32_t w[W];
+        __device__ U() {}
+    } u;
+    uint64_t x[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) x[i] = __hip_atomic_load(slot + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t looks = 0;
+    for (;;) {
+        bool all = true;
+#pragma unroll
+        for (int i = 0; i < W; ++i) all = all && (uint32_t)(x[i] >> 32) == launch;
+        if (all) break;
+        if (++looks > kRsPollLimit) {
+            __hip_atomic_fetch_add(&g_red_poll_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+#pragma unroll
+        for (int i = 0; i < W; ++i)
+            if ((uint32_t)(x[i] >> 32) != launch) x[i] = __hip_atomic_load(slot + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int i = 0; i < W; ++i) u.w[i] = (uint32_t)x[i];
+    return u.a;
+}
+
+template <class Impl, int VEC, bool NT>
+__global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, Impl impl, uint64_t* words, uint32_t launch) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    constexpr int W = sizeof(Acc) / 4;
+    static_assert(sizeof(Acc) % 4 == 0, "accumulator must be a whole number of 32-bit words");
+    __shared__ Acc wave_slots[kRedBlock / 64];
+    __shared__ int s_need;
+    if (blockIdx.x != 0) {
+        const uint32_t i_split = blockIdx.x - 1;
+        const int64_t idx_base = 0;  // one output: the run starts at the array's first element
+        Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in, i_split, p.n_split, p.n, threadIdx.x, 8, idx_base, wave_slots, &s_need);
+        if (threadIdx.x == 0) {
+            union U {
+                Acc a;
+                uint32_t w[W];
+                __device__ U() {}
+            } u;
+            u.a = acc;
+#pragma unroll
+            for (int i = 0; i < W; ++i)
+                __hip_atomic_store(words + (size_t)i_split * W + i, ((uint64_t)launch << 32) | u.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+    // fold the accumulators in index order: thread t takes chunks t, t + 256, ...
+    if constexpr (has_exact<Impl>::value) {
+        typedef typename Impl::Exact Exact;
+        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
+        Acc total = impl.identity();
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(words + (size_t)k * W, launch), total);
+        rs_group_combine(impl, total, 8, wave_slots);
+        if (threadIdx.x == 0) s_need = impl.needs_exact(total) ? 1 : 0;
+        __syncthreads();
+        if (s_need) {
+            const Exact ex = impl.exact();
+            __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
+            typename Exact::Acc e = ex.identity();
+            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_await<Acc>(words + (size_t)k * W, launch), (int64_t)k, e);
+            rs_group_combine(ex, e, 8, exact_slots);
+            total = impl.from_exact(e);
+        }
+        if (threadIdx.x == 0) impl.store(total, p.out, nullptr);
+    } else {
+        Acc total = impl.identity();
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(words + (size_t)k * W, launch), total);
+        rs_group_combine(impl, total, 8, wave_slots);
+        if (threadIdx.x == 0) impl.store(total, p.out, (Impl::NOUT > 1) ? p.out2 : nullptr);
+    }
+}
+
 // Column form. n_out is a multiple of VEC and so is out_inner.
 // U: positions of the axis a lane has in flight (more when the outputs alone give too few lanes
 // to keep the memory system busy: a block still reads 4 KiB runs of every row it touches).
