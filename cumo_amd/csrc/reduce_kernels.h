@@ -715,12 +715,13 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     const uint64_t tiles = (plan.red_total + tile - 1) / tile;
     p.n_split = (uint32_t)((uint64_t)plan.n_split < tiles ? (uint64_t)plan.n_split : tiles);
     if (p.n_split <= 1) return 0;
-    // one output (a full reduction): the form without tickets, when the accumulators fit the hand-over words
-    if (plan.out_total == 1 && !fixed && red_poll_enabled() && (uint64_t)p.n_split * (sizeof(Acc) / 4) <= kRsHandoverWords) {
+    // few outputs: the form without tickets, when the accumulators fit the hand-over words
+    if (!fixed && red_poll_enabled() && plan.out_total <= 256 &&
+        plan.out_total * (uint64_t)p.n_split * (sizeof(Acc) / 4) <= kRsHandoverWords) {
         uint32_t launch = 0;
         uint64_t* words = red_handover_words(stream_slot(stream), &launch);
         if (words != nullptr) {
-            const dim3 g((unsigned)p.n_split + 1u);
+            const dim3 g((unsigned)(plan.out_total * p.n_split + plan.out_total));
             if (nt) hipLaunchKernelGGL((red_srow_poll_kernel<Impl, V, true>), g, b, 0, stream, p, impl, words, launch);
             else hipLaunchKernelGGL((red_srow_poll_kernel<Impl, V, false>), g, b, 0, stream, p, impl, words, launch);
             cumo_cuda_runtime_check_kernel_launch();

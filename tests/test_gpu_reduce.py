@@ -99,7 +99,7 @@ def test_float_reductions_every_axis(tname, dt, view):
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((1000003,), None), ((7, 100000), 1), ((100000, 7), 0), ((3, 40000, 5), 1),
                                         ((64, 64, 64), (0, 2)), ((2, 3), None), ((1,), None), ((70000, 3), 1),
-                                        ((5, 8192), 1), ((4096, 33), 0), ((33, 4096), 0)])
+                                        ((5, 8192), 1), ((4096, 33), 0), ((33, 4096), 0), ((3, 2000003), 1), ((130, 40000), 1), ((260, 30000), 1)])
 def test_random_float_sums(tname, dt, shape, axis):
     rng = np.random.default_rng(201)
     cls = cls_of(tname)
