@@ -715,8 +715,15 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     const uint64_t tiles = (plan.red_total + tile - 1) / tile;
     p.n_split = (uint32_t)((uint64_t)plan.n_split < tiles ? (uint64_t)plan.n_split : tiles);
     if (p.n_split <= 1) return 0;
-    // few outputs: the form without tickets, when the accumulators fit the hand-over words
-    if (!fixed && red_poll_enabled() && plan.out_total <= 256 &&
+    // few outputs: the form without tickets, when the accumulators fit the hand-over words. Not while
+    // the stream is being captured: a replayed launch would carry the same launch number again and
+    // find the last replay's words (the ticket form leaves its words at zero and replays safely).
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusActive;
+    }
+    if (!fixed && red_poll_enabled() && capturing == hipStreamCaptureStatusNone && plan.out_total <= 256 &&
         plan.out_total * (uint64_t)p.n_split * (sizeof(Acc) / 4) <= kRsHandoverWords) {
         uint32_t launch = 0;
         uint64_t* words = red_handover_words(stream_slot(stream), &launch);
