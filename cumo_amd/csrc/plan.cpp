@@ -289,9 +289,13 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
     if (N >= 8192) tpr = 256;
     else if (tpr > 64) tpr = 64;
     if (tpr < 1) tpr = 1;
-    // rows of 16 KiB and more that would leave fewer than eight blocks per compute unit with a
-    // wave each: a whole block per row (every lane still has four 128-bit loads to overlap)
-    if (tpr == 64 && N * (uint64_t)in_elmsz >= 16384 && out_total * 64 / 256 < (uint64_t)kNumCU * 8) tpr = 256;
+    // rows of 16 KiB and more: a whole block per row (every lane still has four 128-bit loads to
+    // overlap, and a block reads one long run instead of four rows at once). Measured on SFloat
+    // [8192,4096] (fresh operands): mean 22.9 -> 21.3 us, var 24.1 -> 22.2 us.
+    // (An accumulator wider than an element makes the fold across the block dear: then only
+    // from 16 elements per lane on. DFloat [8192,2048] var: 25.6 us with a wave per row, 35.4 us
+    // with a block.)
+    if (tpr == 64 && N * (uint64_t)in_elmsz >= 16384 && (accum_bytes <= in_elmsz || N >= 4096)) tpr = 256;
     plan->threads_per_row = tpr;
 
     uint64_t blocks = (out_total * (uint64_t)tpr + 255) / 256;
