@@ -725,12 +725,12 @@ struct ScanColsParams {
     char* out;
 };
 
-template <class T, int VEC>
+template <class T, int VEC, bool NT = false>
 __device__ __forceinline__ void scan_cols_load(const char* p, T (&v)[VEC]) {
     if constexpr (VEC * sizeof(T) == 16) {
         typedef uint32_t u4 __attribute__((ext_vector_type(4)));
         union { u4 q; T t[VEC]; } u;
-        u.q = *reinterpret_cast<const u4*>(p);
+        u.q = NT ? __builtin_nontemporal_load(reinterpret_cast<const u4*>(p)) : *reinterpret_cast<const u4*>(p);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = u.t[j];
     } else {
@@ -738,14 +738,15 @@ __device__ __forceinline__ void scan_cols_load(const char* p, T (&v)[VEC]) {
         for (int j = 0; j < VEC; ++j) v[j] = reinterpret_cast<const T*>(p)[j];
     }
 }
-template <class T, int VEC>
+template <class T, int VEC, bool NT = false>
 __device__ __forceinline__ void scan_cols_store(char* p, const T (&v)[VEC]) {
     if constexpr (VEC * sizeof(T) == 16) {
         typedef uint32_t u4 __attribute__((ext_vector_type(4)));
         union { u4 q; T t[VEC]; } u;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) u.t[j] = v[j];
-        *reinterpret_cast<u4*>(p) = u.q;
+        if (NT) __builtin_nontemporal_store(u.q, reinterpret_cast<u4*>(p));
+        else *reinterpret_cast<u4*>(p) = u.q;
     } else {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) reinterpret_cast<T*>(p)[j] = v[j];
@@ -757,9 +758,9 @@ __device__ __forceinline__ void scan_cols_store(char* p, const T (&v)[VEC]) {
 //   LOOKBACK false  totals holds running totals already: one load of totals[.. seg - 1 ..]
 //   LOOKBACK true   totals holds each segment's own total: they are folded here, in
 //                   segment order (few segments: cheaper than a launch that does it)
-template <class T, class Op, int VEC, int PHASE, bool LOOKBACK>
+template <class T, class Op, int VEC, int PHASE, bool LOOKBACK, bool NT>
 __global__ __launch_bounds__(kScanBlock) void scan_cols_kernel(ScanColsParams p, T* totals) {
-    constexpr int UNR = 8;
+    constexpr int UNR = 4;  // four rows in flight per lane (more open more rows at once in memory and measured slower)
     const unsigned TX = 1u << p.tx_bits, TY = (unsigned)kScanBlock >> p.tx_bits;
     const unsigned tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> p.tx_bits;
     const uint64_t col_groups = p.cols / VEC;
@@ -811,22 +812,23 @@ __global__ __launch_bounds__(kScanBlock) void scan_cols_kernel(ScanColsParams p,
         for (; i + UNR <= end; i += UNR) {
             T v[UNR][VEC];
 #pragma unroll
-            for (int u = 0; u < UNR; ++u) scan_cols_load<T, VEC>(src + (int64_t)(i + u) * p.s_in, v[u]);
+            for (int u = 0; u < UNR; ++u) scan_cols_load<T, VEC, NT>(src + (int64_t)(i + u) * p.s_in, v[u]);
+            __builtin_amdgcn_sched_barrier(0);  // the step's loads go out before anything is folded
 #pragma unroll
             for (int u = 0; u < UNR; ++u) {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) acc[j] = has ? Op::apply(acc[j], v[u][j]) : v[u][j];
                 has = true;
-                if (PHASE == 2) scan_cols_store<T, VEC>(dst + (int64_t)(i + u) * p.s_out, acc);
+                if (PHASE == 2) scan_cols_store<T, VEC, NT>(dst + (int64_t)(i + u) * p.s_out, acc);
             }
         }
         for (; i < end; ++i) {
             T v[VEC];
-            scan_cols_load<T, VEC>(src + (int64_t)i * p.s_in, v);
+            scan_cols_load<T, VEC, NT>(src + (int64_t)i * p.s_in, v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[j] = has ? Op::apply(acc[j], v[j]) : v[j];
             has = true;
-            if (PHASE == 2) scan_cols_store<T, VEC>(dst + (int64_t)i * p.s_out, acc);
+            if (PHASE == 2) scan_cols_store<T, VEC, NT>(dst + (int64_t)i * p.s_out, acc);
         }
         if (PHASE == 0) scan_cols_store<T, VEC>(reinterpret_cast<char*>(totals + (plane * p.n_seg + seg) * p.cols + col), acc);
     }
@@ -846,12 +848,13 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
     p.tx_bits = txb;
     const uint64_t TX = 1ull << txb, TY = (uint64_t)kScanBlock >> txb;
     // segments: enough threads for eight blocks on every compute unit, at least 16 rows each;
-    // no more than the second pass folds by itself when those already give every compute unit a block
+    // no more than the second pass folds by itself when those already give every compute unit four
+    // blocks (with one block each, SFloat [8192,8192] ran its first pass at half the bandwidth)
     const uint64_t want_threads = 256ull * 8 * kScanBlock;
     const uint64_t lanes_per_seg = col_groups * p.planes;
     uint64_t n_seg = (want_threads + lanes_per_seg - 1) / lanes_per_seg;
     const uint64_t max_seg = (p.n + 15) / 16;
-    if (n_seg > kScanLookbackSegs && lanes_per_seg * kScanLookbackSegs >= 256ull * kScanBlock) n_seg = kScanLookbackSegs;
+    if (n_seg > kScanLookbackSegs && lanes_per_seg * kScanLookbackSegs >= 1024ull * kScanBlock) n_seg = kScanLookbackSegs;
     if (n_seg > max_seg) n_seg = max_seg;
     if (n_seg > 1024) n_seg = 1024;
     if (n_seg < 1) n_seg = 1;
@@ -861,15 +864,21 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
     uint64_t grid = strips * ((p.n_seg + TY - 1) / TY) * p.planes;
     if (grid > 0x7fffffffull) grid = 0x7fffffffull;
     const dim3 g((unsigned)grid), b(kScanBlock);
+    const bool nt = stream_past_caches(2 * p.planes * p.n * p.cols * sizeof(T));
+#define CUMO_SCAN_COLS(PHASE_, LB_, TOTALS_)                                                                                  \
+    do {                                                                                                                      \
+        if (nt) hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, PHASE_, LB_, true>), g, b, 0, stream, p, TOTALS_);           \
+        else hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, PHASE_, LB_, false>), g, b, 0, stream, p, TOTALS_);             \
+    } while (0)
     if (p.n_seg == 1) {
-        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2, false>), g, b, 0, stream, p, (T*)nullptr);
+        CUMO_SCAN_COLS(2, false, (T*)nullptr);
         return;
     }
     T* totals = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * p.planes * p.n_seg * p.cols));
     if (!totals) return;
-    hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 0, false>), g, b, 0, stream, p, totals);
+    CUMO_SCAN_COLS(0, false, totals);
     if (p.n_seg <= kScanLookbackSegs) {
-        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2, true>), g, b, 0, stream, p, totals);
+        CUMO_SCAN_COLS(2, true, totals);
     } else {
         ScanColsParams q;
         std::memset(&q, 0, sizeof(q));
@@ -883,8 +892,9 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
         q.in = reinterpret_cast<const char*>(totals);
         q.out = reinterpret_cast<char*>(totals);
         scan_cols_launch_vec<T, Op, VEC>(q, stream);  // at most 1024 rows: the next level has at most 64 segments
-        hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC, 2, false>), g, b, 0, stream, p, totals);
+        CUMO_SCAN_COLS(2, false, totals);
     }
+#undef CUMO_SCAN_COLS
     // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
     cumo_cuda_runtime_free(reinterpret_cast<char*>(totals));
 }
