@@ -451,6 +451,16 @@ struct ValueExtremeImpl {
 #pragma unroll
         for (int k = 0; k < N; ++k) acc = pick(acc, x[k]);
     }
+    // a whole step at once (no test per vector between the loads' arrivals)
+    static constexpr bool GROUPED = true;
+    template <int U, int N>
+    __device__ __forceinline__ void accumulate_group(const T (&x)[U][N], const int64_t (&)[U], Acc& acc) const {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) acc = pick(acc, x[u][k]);
+        }
+    }
     __device__ __forceinline__ bool needs_exact(const Acc& acc) const { return acc == (T)0; }
     __host__ __device__ __forceinline__ Exact exact() const { return Exact{0}; }
     __device__ __forceinline__ Acc from_exact(const typename Exact::Acc& e) const { return e.value; }
