@@ -303,6 +303,38 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
     }
 }
 
+// The exact second fold by ONE wave over the tiles that a whole block (tpr_bits 8) folded: the
+// tiles first, first + every, ... of kRedBlock * VEC * kRsUnroll elements each, every vector of
+// them taken by one of the 64 lanes. For the streaming blocks of the kernel below, where only
+// the first wave learns (by a shuffle, no barrier, no LDS) that the block's result needs it:
+// it is rare (a minimum or maximum that is a zero), and asking the whole block cost every
+// launch 0.7 us. Lane 0 returns the result.
+template <class Impl, int VEC>
+__device__ __attribute__((noinline)) typename Impl::Acc rs_exact_refold_wave(const Impl& impl, const char* base, uint64_t first, uint64_t every,
+                                                                              uint64_t end) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Exact Exact;
+    const Exact ex = impl.exact();
+    typename Exact::Acc e = ex.identity();
+    const uint64_t per_tile = (uint64_t)kRedBlock * VEC * kRsUnroll;
+    const uint64_t tiles = (end + per_tile - 1) / per_tile;
+    const unsigned lane = threadIdx.x & 63u;
+    for (uint64_t t = first; t < tiles; t += every) {
+        const uint64_t t0 = t * per_tile;
+        const uint64_t t1 = t0 + per_tile < end ? t0 + per_tile : end;
+        for (uint64_t i = t0 + (uint64_t)lane * VEC; i < t1; i += 64u * VEC) {
+            In x[VEC];
+            rs_load<In, VEC, false>(base + i * sizeof(In), x);
+            ex.template accumulate_n<VEC>(x, (int64_t)i, e);
+        }
+    }
+    for (unsigned d = 32; d > 0; d >>= 1) {
+        const typename Exact::Acc other = shfl_down_any(e, d);
+        ex.combine(other, e);
+    }
+    return impl.from_exact(e);
+}
+
 // Few outputs, the axis of each cut over n_split blocks, one launch, no tickets: the first n_out
 // blocks read nothing of the input; each waits for the accumulators of its output's other blocks,
 // which arrive as 64-bit words {launch number, 32 bits of the accumulator} written with agent-scope
@@ -363,7 +395,14 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
         rs_split_out(p, i_out, o0, o1);
         const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
         const int64_t idx_base = p.index_mode == 2 ? in_off / (int64_t)sizeof(In) : 0;
-        Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, threadIdx.x, 8, idx_base, wave_slots, &s_need);
+        Acc acc = rs_row_scan<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, threadIdx.x, 8, idx_base);
+        rs_group_combine(impl, acc, 8, wave_slots);
+        if constexpr (has_exact<Impl>::value) {
+            // thread 0 holds the block's result; its wave alone repeats the fold where that is needed
+            if (threadIdx.x >= 64) return;
+            const int mine = impl.needs_exact(acc) ? 1 : 0;
+            if (__shfl(mine, 0) != 0) acc = rs_exact_refold_wave<Impl, VEC>(impl, p.in + in_off, i_split, p.n_split, p.n);
+        }
         if (threadIdx.x == 0) {
             union U {
                 Acc a;
