@@ -69,8 +69,38 @@ __device__ __forceinline__ T ms_block_sum(T acc) {
 // NT: non-temporal loads, for runs that do not fit the last-level cache anyway
 template <class T, bool NANF, int VEC, bool NT>
 __global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1, const char* p2, int64_t s1, int64_t s2, uint64_t n,
-                                                                  uint64_t chunk, T* partial, T* out) {
-    const uint64_t begin = (uint64_t)blockIdx.x * chunk;
+                                                                  uint64_t chunk, T* partial, T* out, uint64_t* words, uint32_t launch) {
+    constexpr int W = (int)(sizeof(T) / 4);
+    uint32_t block = blockIdx.x;
+    if (words) {
+        // One launch for the whole sum: block 0 reads nothing of the operands; it waits for the other
+        // blocks' totals, which arrive as 64-bit words {launch number, 32 bits of the total} written
+        // with agent-scope atomic stores, folds them in index order and adds onto the result.
+        if (block == 0) {
+            const uint32_t n_parts = gridDim.x - 1;
+            T acc = T();
+            for (uint32_t i = threadIdx.x; i < n_parts; i += kMsBlock) {
+                union { T t; uint32_t w[W]; } u;
+#pragma unroll
+                for (int k = 0; k < W; ++k) {
+                    const uint64_t* slot = words + (size_t)i * W + k;
+                    uint64_t x = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    uint32_t looks = 0;
+                    while ((uint32_t)(x >> 32) != launch && ++looks < (1u << 24)) {
+                        __builtin_amdgcn_s_sleep(4);
+                        x = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    u.w[k] = (uint32_t)x;
+                }
+                acc = ms_add(acc, u.t);
+            }
+            acc = ms_block_sum<T>(acc);
+            if (threadIdx.x == 0) *out = ms_add(*out, acc);
+            return;
+        }
+        block -= 1;
+    }
+    const uint64_t begin = (uint64_t)block * chunk;
     uint64_t end = begin + chunk;
     if (end > n) end = n;
     T acc[4] = {T(), T(), T(), T()};
@@ -124,8 +154,17 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1
     T tot = ms_add(ms_add(acc[0], acc[1]), ms_add(acc[2], acc[3]));
     tot = ms_block_sum<T>(tot);
     if (threadIdx.x == 0) {
-        if (partial) partial[blockIdx.x] = tot;
-        else *out = ms_add(*out, tot);
+        if (words) {
+            union { T t; uint32_t w[W]; } u;
+            u.t = tot;
+#pragma unroll
+            for (int k = 0; k < W; ++k)
+                __hip_atomic_store(words + (size_t)block * W + k, ((uint64_t)launch << 32) | u.w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (partial) {
+            partial[block] = tot;
+        } else {
+            *out = ms_add(*out, tot);
+        }
     }
 }
 
@@ -248,23 +287,32 @@ void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, 
     chunk = ((chunk + round - 1) / round) * round;
     grid = n ? (n + chunk - 1) / chunk : 1;
     const bool vec = s1 == (ssize_t)sizeof(T) && s2 == (ssize_t)sizeof(T) && ((uintptr_t)p1 % 16) == 0 && ((uintptr_t)p2 % 16) == 0;
+    // several blocks: their totals go to the stream's hand-over words and block 0 of the same launch
+    // folds them (not while the stream is being captured: a replayed launch would carry the same
+    // launch number again), else to scratch from the pool and a second launch
     T* partial = nullptr;
+    uint64_t* words = nullptr;
+    uint32_t launch = 0;
     if (grid > 1) {
-        partial = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * grid));
-        if (!partial) return;
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+            (void)hipGetLastError();
+            capturing = hipStreamCaptureStatusActive;
+        }
+        if (capturing == hipStreamCaptureStatusNone && grid * (sizeof(T) / 4) <= 8192) words = red_handover_words(stream_slot(stream), &launch);
+        if (!words) {
+            partial = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * grid));
+            if (!partial) return;
+        }
     }
     const bool nt = stream_past_caches(2 * n * sizeof(T));
-    if (vec && nt)
-        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, true>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2,
-                           n, chunk, partial, reinterpret_cast<T*>(p3));
-    else if (vec)
-        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, false>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2,
-                           n, chunk, partial, reinterpret_cast<T*>(p3));
-    else
-        hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1, false>), dim3((unsigned)grid), dim3(kMsBlock), 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n,
-                           chunk, partial, reinterpret_cast<T*>(p3));
+    const dim3 g((unsigned)(words ? grid + 1 : grid)), b(kMsBlock);
+    T* out = reinterpret_cast<T*>(p3);
+    if (vec && nt) hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, true>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch);
+    else if (vec) hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, false>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch);
+    else hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1, false>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch);
     if (partial) {
-        hipLaunchKernelGGL((mulsum_combine_kernel<T>), dim3(1), dim3(kMsBlock), 0, stream, (const T*)partial, grid, reinterpret_cast<T*>(p3));
+        hipLaunchKernelGGL((mulsum_combine_kernel<T>), dim3(1), dim3(kMsBlock), 0, stream, (const T*)partial, grid, out);
         cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
     }
     cumo_cuda_runtime_check_kernel_launch();
