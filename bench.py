@@ -416,7 +416,7 @@ def cpu_baseline_c2(budget_s=12.0):
     one_pass()
     t0 = time.perf_counter()
     passes = 0
-    while passes < 2 or (time.perf_counter() - t0 < budget_s and passes < 200):
+    while passes < 2 or (time.perf_counter() - t0 < budget_s and passes < 600):
         one_pass()
         passes += 1
     dt = (time.perf_counter() - t0) / passes
