@@ -192,8 +192,10 @@ def config_ops(name, cumo, host):
             ("x.cumsum(axis:1)", lambda e: e.__setitem__("cs", e["x"].cumsum(axis=1)), 2 * nb, n),
             ("mask.where", lambda e: e.__setitem__("wh", e["mask"].where()), n // 8 + 4 * cnt, n),
             ("x[mask]", lambda e: e.__setitem__("xm", e["x"][e["mask"]]), n // 8 + 4 * cnt + 4 * cnt, n),
-            # rows drawn with replacement: repeated rows are read from cache
+            # rows drawn with replacement: repeated rows are read from cache, and some 37% of the rows are never
+            # read; the permutation beside it reads every row once, as the scatter writes every row once
             ("x[rows,true] (gather)", lambda e: e.__setitem__("g", e["x"][e["rows"]]), 2 * nb + 8 * r, n),
+            ("x[perm,true] (gather, every row once)", lambda e: e.__setitem__("g", e["x"][e["perm"]]), 2 * nb + 8 * r, n),
             ("b[perm,true]=x (scatter)", lambda e: e["b"].__setitem__(e["perm"], e["x"]), 2 * nb + 8 * r, n),
         ]
     if name == "nmath":
