@@ -899,11 +899,273 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
     cumo_cuda_runtime_free(reinterpret_cast<char*>(totals));
 }
 
+// ---- long runs across memory in one pass ---------------------------------------
+// The matrix is cut into tiles of NW * 16 rows by 64 vectors (1 KiB of a row): wave w of
+// a block holds 16 rows of the tile, lane l their vector l, all in registers. A tile adds
+// up its columns (in the lane, then across the waves through LDS), publishes the column
+// totals, gathers what the tiles above it published, and scans its rows from there: the
+// data is read once and written once. The published words are {1, 32 bits of the value};
+// they must be zero before the launch. Tiles take their places by ticket, level by level
+// (all strips of one band of rows, then the next band), so whatever a tile waits for
+// belongs to a block that is already running, and no tile waits before it has published
+// its own totals. What a tile gathers has a fixed shape, so results do not change from
+// launch to launch: tiles come in groups of 8 and groups in supergroups of 8; a tile folds
+// the supergroups before its own, then the groups before its own, then the tiles before it
+// in its group, each in order. The tile that closes a group publishes the group's total,
+// the one that closes a supergroup the supergroup's.
+constexpr int kColsChainRows = 16;
+constexpr uint32_t kColsChainFan = 8;
+
+template <class T>
+struct ScanColsChain {
+    static constexpr int W = (int)(sizeof(T) / 4);
+    uint32_t* ticket;
+    uint64_t* tile;    // [strip][level][column][W]
+    uint64_t* group;   // [strip][group][column][W]
+    uint64_t* super;   // [strip][supergroup][column][W]
+    uint32_t depth, n_groups, n_supers;  // per strip
+    uint32_t strips;                     // per plane
+    uint32_t all_strips;                 // planes * strips
+};
+
+// Up to seven published values, `stride` words apart, the earliest first: all are asked for at
+// once (eight-byte types: four, then three; seven would not fit the registers beside the tile),
+// asked for again until they are there, then folded in order. False when count is 0.
+template <class T, class Op>
+__device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t stride, uint32_t count, T& out) {
+    constexpr int W = ScanColsChain<T>::W;
+    constexpr uint32_t N = kColsChainFan - 1, C = sizeof(T) == 8 ? 4 : N;
+    uint32_t polls = 0;
+    bool has = false;
+#pragma unroll
+    for (uint32_t c0 = 0; c0 < N; c0 += C) {
+        uint64_t x[C][W];
+#pragma unroll
+        for (uint32_t i = 0; i < C; ++i)
+#pragma unroll
+            for (int h = 0; h < W; ++h)
+                x[i][h] = c0 + i < count ? __hip_atomic_load(base + (c0 + i) * stride + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (1ull << 32);
+        for (;;) {
+            uint64_t all = ~0ull;
+#pragma unroll
+            for (uint32_t i = 0; i < C; ++i)
+#pragma unroll
+                for (int h = 0; h < W; ++h) all &= x[i][h];
+            if ((all >> 32) & 1u) break;
+            if (++polls > kChainSpinLimit) {
+                __hip_atomic_fetch_add(&g_scan_chain_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+#pragma unroll
+            for (uint32_t i = 0; i < C; ++i)
+#pragma unroll
+                for (int h = 0; h < W; ++h)
+                    if (((x[i][h] >> 32) & 1u) == 0) x[i][h] = __hip_atomic_load(base + (c0 + i) * stride + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < C; ++i) {
+            if (c0 + i < count) {
+                union { T t; uint32_t w[W]; } u;
+#pragma unroll
+                for (int h = 0; h < W; ++h) u.w[h] = (uint32_t)x[i][h];
+                out = has ? Op::apply(out, u.t) : u.t;
+                has = true;
+            }
+        }
+    }
+    return has;
+}
+
+template <class T, class Op, bool NT, int NW>
+__global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams p, ScanColsChain<T> c) {
+    constexpr int V = 16 / (int)sizeof(T), R = kColsChainRows, SW = 64 * V, W = ScanColsChain<T>::W;
+    __shared__ T part[NW][SW];
+    __shared__ T s_groups[SW], s_supers[SW];
+    __shared__ uint32_t s_ticket;
+    static_assert(NW * 64 >= 3 * SW, "three roles of SW threads each");
+    const unsigned w = threadIdx.x >> 6, l = threadIdx.x & 63u;
+    if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint32_t id = s_ticket;
+    const uint32_t k = id / c.all_strips, ps = id - k * c.all_strips;
+    const uint32_t plane = ps / c.strips, strip = ps - plane * c.strips;
+    int64_t oi = 0, oo = 0;
+    if (p.nouter > 0) {
+        uint64_t r = plane;
+#pragma unroll 1
+        for (int d = p.nouter - 1; d >= 0; --d) {
+            const uint64_t m = p.oshape[d];
+            const uint64_t q = r / m;
+            const int64_t i = (int64_t)(r - q * m);
+            r = q;
+            oi += i * p.ostep_in[d];
+            oo += i * p.ostep_out[d];
+        }
+    }
+    const int64_t row0 = (int64_t)k * (NW * R) + (int64_t)w * R;
+    const int64_t colb = ((int64_t)strip * SW + (int64_t)l * V) * (int64_t)sizeof(T);
+    const char* src = p.in + oi + row0 * p.s_in + colb;
+    char* dst = p.out + oo + row0 * p.s_out + colb;
+    T raw[R][V];
+#pragma unroll
+    for (int r = 0; r < R; ++r) scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
+    {
+        T tot[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) tot[j] = raw[0][j];
+#pragma unroll
+        for (int r = 1; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < V; ++j) tot[j] = Op::apply(tot[j], raw[r][j]);
+#pragma unroll
+        for (int j = 0; j < V; ++j) part[w][l * V + j] = tot[j];
+    }
+    __syncthreads();
+    // Threads 0 .. SW-1 see to the tile's own totals and to the tiles before it in its group,
+    // the next SW threads to the groups before its group, the SW after those to the supergroups:
+    // the three waits run side by side in different waves, each with seven loads in flight.
+    const unsigned col = threadIdx.x % SW, role = threadIdx.x / SW;
+    const uint32_t pos = k % kColsChainFan, g = k / kColsChainFan, gpos = g % kColsChainFan, sg = g / kColsChainFan;
+    const size_t cw = (size_t)SW * W;  // words from one tile's (group's) totals to the next one's
+    T gt = T();
+    if (role == 0) {
+        // part[ww][col] becomes what the waves above ww add up to; gt, the tile's total
+        gt = part[0][col];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) {
+            const T e = gt;
+            gt = Op::apply(gt, part[ww][col]);
+            part[ww][col] = e;
+        }
+        chain_publish<T>(c.tile + (((size_t)ps * c.depth + k) * SW + col) * W, gt);
+    }
+    const uint64_t* from = c.tile + (((size_t)ps * c.depth + (size_t)g * kColsChainFan) * SW + col) * W;
+    uint32_t count = pos;
+    if (role == 1) {
+        from = c.group + (((size_t)ps * c.n_groups + (size_t)sg * kColsChainFan) * SW + col) * W;
+        count = gpos;
+    } else if (role == 2) {
+        from = c.super + ((size_t)ps * c.n_supers * SW + col) * W;
+        count = sg;
+    } else if (role > 2) {
+        count = 0;
+    }
+    T xs = T();
+    const bool xh = cols_chain_gather<T, Op>(from, cw, count, xs);
+    if (role == 0) {
+        if (xh) gt = Op::apply(xs, gt);  // the group's total so far
+        if (pos == kColsChainFan - 1) chain_publish<T>(c.group + (((size_t)ps * c.n_groups + g) * SW + col) * W, gt);
+    } else if (role == 1) {
+        s_groups[col] = xs;
+    } else if (role == 2) {
+        s_supers[col] = xs;
+    }
+    __syncthreads();
+    if (role == 0 && k > 0) {
+        const bool yh = gpos > 0;
+        T ys = T();
+        if (yh) ys = s_groups[col];
+        if (pos == kColsChainFan - 1 && gpos == kColsChainFan - 1) {
+            const T st = yh ? Op::apply(ys, gt) : gt;
+            chain_publish<T>(c.super + (((size_t)ps * c.n_supers + sg) * SW + col) * W, st);
+        }
+        bool ph = sg > 0;
+        T pre = T();
+        if (ph) pre = s_supers[col];
+        if (yh) { pre = ph ? Op::apply(pre, ys) : ys; ph = true; }
+        if (xh) { pre = ph ? Op::apply(pre, xs) : xs; ph = true; }
+        // k > 0: something lies above, so ph holds
+        part[0][col] = pre;
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) part[ww][col] = Op::apply(pre, part[ww][col]);
+    }
+    __syncthreads();
+    // The topmost wave of the topmost tile has nothing above it; it goes the same way as the others
+    // from a first row the compiler cannot see through (it would otherwise find this wave's running
+    // values equal to the column totals' and keep all sixteen of them in registers from there to here,
+    // beside the tile: there is no room for both).
+    T acc[V];
+    const bool topmost = k == 0 && w == 0;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const T above = topmost ? raw[0][j] : part[w][l * V + j];
+        acc[j] = topmost ? above : Op::apply(above, raw[0][j]);
+        if constexpr (sizeof(T) == 8) {
+            union { T t; uint64_t u; } o;
+            o.t = acc[j];
+            asm volatile("" : "+v"(o.u));
+            acc[j] = o.t;
+        } else {
+            union { T t; uint32_t u; } o;
+            o.t = acc[j];
+            asm volatile("" : "+v"(o.u));
+            acc[j] = o.t;
+        }
+    }
+    scan_cols_store<T, V, NT>(dst, acc);
+#pragma unroll
+    for (int r = 1; r < R; ++r) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = Op::apply(acc[j], raw[r][j]);
+        scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
+    }
+}
+
+static bool scan_cols_chain_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("CUMO_HIP_SCAN_COLS_CHAIN");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+// true when the launch was made (or failed: the error is left for the caller's check)
+template <class T, class Op>
+bool scan_cols_chain_launch(ScanColsParams& p, hipStream_t stream) {
+    constexpr int V = 16 / (int)sizeof(T), W = ScanColsChain<T>::W, NW = 16;
+    constexpr uint64_t SW = 64 * V, TR = (uint64_t)NW * kColsChainRows;
+    if (!scan_cols_chain_enabled()) return false;
+    if (p.cols % SW != 0 || p.n % TR != 0) return false;
+    const uint64_t depth = p.n / TR, strips = p.cols / SW;
+    constexpr uint64_t F = kColsChainFan;
+    if (depth < 2 || depth > F * F * F) return false;
+    const uint64_t all_strips = strips * p.planes;
+    const uint64_t n_tiles = all_strips * depth;
+    if (n_tiles < 512 || n_tiles > 0x7fffffffull) return false;
+    const uint64_t n_groups = (depth + F - 1) / F, n_supers = (n_groups + F - 1) / F;
+    const uint64_t head = 32;  // the ticket, and the totals on a line of their own
+    const uint64_t words = head + all_strips * (depth + n_groups + n_supers) * SW * W;
+    uint64_t* ws = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(words * sizeof(uint64_t)));
+    if (!ws) return true;
+    uint64_t clear_grid = (words + 255) / 256;
+    if (clear_grid > 2048) clear_grid = 2048;
+    hipLaunchKernelGGL(scan_chain_clear_kernel, dim3((unsigned)clear_grid), dim3(256), 0, stream, ws, words);
+    ScanColsChain<T> c;
+    c.ticket = reinterpret_cast<uint32_t*>(ws);
+    c.tile = ws + head;
+    c.group = c.tile + all_strips * depth * SW * W;
+    c.super = c.group + all_strips * n_groups * SW * W;
+    c.depth = (uint32_t)depth;
+    c.n_groups = (uint32_t)n_groups;
+    c.n_supers = (uint32_t)n_supers;
+    c.strips = (uint32_t)strips;
+    c.all_strips = (uint32_t)all_strips;
+    const bool nt = stream_past_caches(2 * p.planes * p.n * p.cols * sizeof(T));
+    const dim3 g((unsigned)n_tiles), b(NW * 64);
+    if (nt) hipLaunchKernelGGL((scan_cols_chain_kernel<T, Op, true, NW>), g, b, 0, stream, p, c);
+    else hipLaunchKernelGGL((scan_cols_chain_kernel<T, Op, false, NW>), g, b, 0, stream, p, c);
+    // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
+    cumo_cuda_runtime_free(reinterpret_cast<char*>(ws));
+    return true;
+}
+
 template <class T, class Op>
 void scan_cols_launch(ScanColsParams& p, hipStream_t stream) {
     constexpr int V = 16 / (int)sizeof(T);
     bool vec = (p.cols % V) == 0 && ((uintptr_t)p.in % 16) == 0 && ((uintptr_t)p.out % 16) == 0 && (p.s_in % 16) == 0 && (p.s_out % 16) == 0;
     for (int d = 0; d < p.nouter && vec; ++d) vec = (p.ostep_in[d] % 16) == 0 && (p.ostep_out[d] % 16) == 0;
+    if (vec && scan_cols_chain_launch<T, Op>(p, stream)) return;
     if (vec) scan_cols_launch_vec<T, Op, V>(p, stream);
     else scan_cols_launch_vec<T, Op, 1>(p, stream);
 }

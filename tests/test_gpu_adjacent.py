@@ -322,6 +322,52 @@ def test_cum_along_columns_of_tall_wide_and_stacked_arrays(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", ALL)
+def test_long_columns_in_one_pass(tname, dt):
+    """Runs across memory whose matrix cuts into at least 512 tiles of 256 rows by 64 vectors are
+    scanned in one pass: tiles publish their column totals and gather what lies above them through
+    groups of 8 tiles and supergroups of 8 groups. Depths of 70 tiles (two supergroups), 35 tiles
+    in four planes and 8 tiles (one group, closed by the last tile). Small integers (float sums
+    exact in any order): bit for bit against the sequential scan; products of +-1 and a few 2s;
+    NaN skipped (every run starts with more than a tile of NaN) and carried; every other row of a
+    taller array; random floats give the same bits from launch to launch and stay close."""
+    cls = cls_of(tname)
+    rng = np.random.default_rng(61)
+    sw = 64 * (16 // np.dtype(dt).itemsize)
+    for shape, ax in [((256 * 70, 8 * sw), 0), ((4, 256 * 35, 4 * sw), 1), ((256 * 8, 64 * sw), 0)]:
+        h = rng.integers(-3, 4, size=shape).astype(dt)
+        if dt != np.int32:
+            h[..., ::3] = 0
+        d = cls.cast(h)
+        assert_bits_equal(d.cumsum(axis=ax).to_numpy(), oracle.cum("cumsum", h, axis=ax), (shape, "cumsum"))
+        f = rng.choice(np.array([1, -1], dtype=dt), size=shape)
+        f[tuple(rng.integers(0, n, 40) for n in shape)] = 2
+        assert_bits_equal(cls.cast(f).cumprod(axis=ax).to_numpy(), oracle.cum("cumprod", f, axis=ax), (shape, "cumprod"))
+        if dt != np.int32:
+            g = h.copy()
+            g[tuple(rng.integers(0, n, 3000) for n in shape)] = np.nan
+            if len(shape) == 2:
+                g[:300] = np.nan
+            else:
+                g[:, :300] = np.nan
+            d = cls.cast(g)
+            assert_bits_equal(d.cumsum(axis=ax, nan=True).to_numpy(), oracle.cum("cumsum", g, axis=ax, nan=True), (shape, "nan: true"))
+            assert_bits_equal(d.cumsum(axis=ax).to_numpy(), oracle.cum("cumsum", g, axis=ax), (shape, "NaN carried"))
+        del d
+    shape = (256 * 16, 32 * sw)
+    wide = rng.integers(-3, 4, size=(2 * shape[0], shape[1])).astype(dt)
+    hv = np.ascontiguousarray(wide[::2])
+    assert_bits_equal(cls.cast(wide)[::2].cumsum(axis=0).to_numpy(), oracle.cum("cumsum", hv, axis=0), "every other row")
+    if dt != np.int32:
+        r = rng.standard_normal(shape).astype(dt)
+        d = cls.cast(r)
+        first = d.cumsum(axis=0).to_numpy()
+        for _ in range(3):
+            assert_bits_equal(d.cumsum(axis=0).to_numpy(), first, "same bits from launch to launch")
+        exact = np.cumsum(r.astype(np.float64), axis=0) if dt == np.float32 else np.asarray(np.cumsum(r.astype(np.longdouble), axis=0)).astype(np.float64)
+        _cum_close(first, exact, np.cumsum(np.abs(r).astype(np.float64), axis=0), shape[0], dt, "random floats")
+
+
+@pytest.mark.parametrize("tname,dt", ALL)
 def test_mulsum_parity(tname, dt):
     cls = cls_of(tname)
     rng = np.random.default_rng(53)
