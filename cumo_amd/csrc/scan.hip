@@ -22,6 +22,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 namespace cumo_hip {
 namespace {
@@ -291,9 +292,12 @@ __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const char* in, 
 // supergroup the supergroup's. A tile folds, each with one wave-wide butterfly, the totals
 // of the earlier tiles of its group, of the earlier groups of its supergroup and of the
 // earlier supergroups. Reads the input once and writes the output once.
-// A published value travels as 64-bit words {1, 32 bits of the value}, stored and loaded
-// with agent-scope atomics: a word is there when its upper half is 1, no fence needed.
-// The words must be zero before the launch. A wait gives up after kChainSpinLimit polls
+// A published value travels as 64-bit words {the launch's number, 32 bits of the value},
+// stored and loaded with agent-scope atomics: a word is there when its upper half is the
+// launch's number, no fence needed. The words live in a region that the stream keeps from
+// launch to launch (chain_words_acquire below), so nothing is cleared: what an earlier launch
+// left carries another number, and the ticket word just counts on (a launch takes exactly one
+// ticket per block; the host knows where it stood). A wait gives up after kChainSpinLimit polls
 // (it cannot be reached while every tile before this one has a running block); the count
 // of such give-ups is kept in g_scan_chain_gave_up.
 constexpr uint32_t kChainSpinLimit = 1u << 22;
@@ -309,21 +313,23 @@ struct ScanChain {
     uint64_t* tile;    // [n_tiles * W]
     uint64_t* group;   // [n_groups * W]
     uint64_t* super;   // [n_supers * W]
+    uint32_t flag;         // the upper half of a word of this launch
+    uint32_t ticket_base;  // what the ticket word held before this launch
 };
 
 template <class T>
-__device__ __forceinline__ void chain_publish(uint64_t* slot, T value) {
+__device__ __forceinline__ void chain_publish(uint64_t* slot, T value, uint32_t flag) {
     constexpr int W = ScanChain<T>::W;
     union { T t; uint32_t w[W]; } u;
     u.t = value;
 #pragma unroll
     for (int i = 0; i < W; ++i)
-        __hip_atomic_store(slot + i, (1ull << 32) | u.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(slot + i, ((uint64_t)flag << 32) | u.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // one look at a published value: true when all of it is there
 template <class T>
-__device__ __forceinline__ bool chain_peek(const uint64_t* slot, T& value) {
+__device__ __forceinline__ bool chain_peek(const uint64_t* slot, T& value, uint32_t flag) {
     constexpr int W = ScanChain<T>::W;
     union { T t; uint32_t w[W]; } u;
     uint64_t x[W];
@@ -332,7 +338,7 @@ __device__ __forceinline__ bool chain_peek(const uint64_t* slot, T& value) {
     bool all = true;
 #pragma unroll
     for (int i = 0; i < W; ++i) {
-        all = all && (x[i] >> 32) != 0;
+        all = all && (uint32_t)(x[i] >> 32) == flag;
         u.w[i] = (uint32_t)x[i];
     }
     value = u.t;
@@ -390,7 +396,7 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
     constexpr int W = ScanChain<T>::W;
     const unsigned lane = threadIdx.x & 63u;
     const uint32_t pos = t & 63u, g = t >> 6, gpos = g & 63u, sg = g >> 6;
-    if (lane == 0) chain_publish<T>(c.tile + (size_t)t * W, total);
+    if (lane == 0) chain_publish<T>(c.tile + (size_t)t * W, total, c.flag);
     T x = T(), y = T(), z = T();
     const bool has_x = lane < pos, has_y = lane < gpos, has_z = lane < sg;
     bool need_x = has_x, need_y = has_y, need_z = has_z;
@@ -403,7 +409,7 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
         const uint64_t* latest = pos > 0 ? c.tile + (size_t)(t - 1) * W + (W - 1)
                                          : (gpos > 0 ? c.group + (size_t)(g - 1) * W + (W - 1) : c.super + (size_t)(sg - 1) * W + (W - 1));
         if (lane == 0) {
-            while ((__hip_atomic_load(latest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == 0) {
+            while ((uint32_t)(__hip_atomic_load(latest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != c.flag) {
                 if (++polls > kChainSpinLimit) break;
                 __builtin_amdgcn_s_sleep(16);
             }
@@ -419,9 +425,9 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
     T gt = T();
     bool gt_has = false;
     for (;;) {
-        if (need_x) need_x = !chain_peek<T>(px, x);
-        if (need_y) need_y = !chain_peek<T>(py, y);
-        if (need_z) need_z = !chain_peek<T>(pz, z);
+        if (need_x) need_x = !chain_peek<T>(px, x, c.flag);
+        if (need_y) need_y = !chain_peek<T>(py, y, c.flag);
+        if (need_z) need_z = !chain_peek<T>(pz, z, c.flag);
         if (!x_folded && __ballot(need_x) == 0) {
             chain_wave_fold<T, Op>(x, xh);
             x_folded = true;
@@ -429,7 +435,7 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
                 gt = x;
                 gt_has = xh;
                 chain_join<T, Op>(gt, gt_has, total, total_has);
-                if (lane == 0) chain_publish<T>(c.group + (size_t)g * W, gt);
+                if (lane == 0) chain_publish<T>(c.group + (size_t)g * W, gt, c.flag);
                 group_out = true;
             }
         }
@@ -440,7 +446,7 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
                 T st = y;
                 bool st_has = yh;
                 chain_join<T, Op>(st, st_has, gt, gt_has);
-                if (lane == 0) chain_publish<T>(c.super + (size_t)sg * W, st);
+                if (lane == 0) chain_publish<T>(c.super + (size_t)sg * W, st, c.flag);
                 super_out = true;
             }
         }
@@ -620,14 +626,14 @@ __global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsPar
 }
 
 template <class T, class Op, bool NT>
-__global__ __launch_bounds__(kScanBlock) void scan_chain_kernel(const char* in, char* out, uint64_t n, ScanChain<T> c) {
+__global__ __launch_bounds__(kScanBlock, sizeof(T) == 8 ? 3 : 4) void scan_chain_kernel(const char* in, char* out, uint64_t n, ScanChain<T> c) {
     constexpr int TILE = ScanChain<T>::TILE;
     constexpr int V = ChainVec<T>::V;
     constexpr int R = TILE / (kScanBlock * V);
     __shared__ ChainShared sh;
     __shared__ T s_prefix;
     __shared__ T s_wave_tot[kScanBlock / 64];
-    if (threadIdx.x == 0) sh.tile = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) sh.tile = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - c.ticket_base;
     __syncthreads();
     const uint32_t t = sh.tile;
     const uint64_t first = (uint64_t)t * TILE;
@@ -676,6 +682,118 @@ __global__ __launch_bounds__(256) void scan_chain_clear_kernel(uint64_t* words, 
     for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) words[i] = 0;
 }
 
+// The words of one launch: the ticket word first, the published totals from word kChainHead on.
+// A stream that is not being captured keeps a region of its own (per device and stream slot,
+// allocated from the driver at first use, grown when a launch needs more, never cleared after
+// that): launches on it are numbered, and a launch's words carry its number. Under capture (a
+// replay would repeat the number), without a slot, or beyond kChainKeptWords the words come from
+// the pool and a small kernel clears them first; the number is 1 then.
+constexpr uint64_t kChainHead = 32;
+constexpr uint64_t kChainKeptWords = 8ull << 20;  // 64 MiB
+constexpr int kChainDevices = 16;
+struct ChainRegion {
+    uint64_t* ptr;
+    uint64_t cap;
+    uint32_t launch, ticket;
+};
+ChainRegion g_chain_region[kChainDevices][kStreamSlots];
+std::mutex g_chain_lock;
+
+struct ChainWords {
+    uint64_t* ws;
+    uint32_t flag, ticket_base;
+    bool pooled;
+};
+
+// CUMO_HIP_SCAN_KEEP_WORDS=0 (read once): always the pool and the clearing kernel
+static bool chain_keep_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("CUMO_HIP_SCAN_KEEP_WORDS");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+// words counts the head; tickets = blocks of the launch. False: no memory (the error is set).
+static bool chain_words_acquire(hipStream_t stream, uint64_t words, uint32_t tickets, ChainWords* w) {
+    w->flag = 1;
+    w->ticket_base = 0;
+    w->pooled = true;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusActive;
+    }
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        dev = -1;
+    }
+    const int slot = stream_slot(stream);
+    if (chain_keep_enabled() && capturing == hipStreamCaptureStatusNone && slot >= 0 && dev >= 0 && dev < kChainDevices && words <= kChainKeptWords) {
+        // held until chain_words_release, that is across the launch itself: launches that share a
+        // stream must reach it in the order of their numbers and tickets
+        g_chain_lock.lock();
+        ChainRegion& r = g_chain_region[dev][slot];
+        bool ok = true;
+        if (r.cap < words) {
+            if (r.ptr) {
+                // only this stream's launches use the region
+                ok = hipStreamSynchronize(stream) == hipSuccess && hipFree(r.ptr) == hipSuccess;
+                r.ptr = nullptr;
+                r.cap = 0;
+            }
+            uint64_t cap = 1ull << 16;
+            while (cap < words) cap <<= 1;
+            void* p = nullptr;
+            if (ok && hipMalloc(&p, cap * sizeof(uint64_t)) == hipSuccess) {
+                if (hipMemsetAsync(p, 0, cap * sizeof(uint64_t), stream) == hipSuccess) {
+                    r.ptr = static_cast<uint64_t*>(p);
+                    r.cap = cap;
+                    r.launch = 0;
+                    r.ticket = 0;
+                } else {
+                    (void)hipFree(p);
+                    ok = false;
+                }
+            } else {
+                ok = false;
+            }
+            if (!ok) (void)hipGetLastError();
+        }
+        if (ok && r.launch == 0xffffffffu) {
+            // every number has been used once: start over from cleared words
+            ok = hipMemsetAsync(r.ptr, 0, r.cap * sizeof(uint64_t), stream) == hipSuccess;
+            r.launch = 0;
+            r.ticket = 0;
+            if (!ok) (void)hipGetLastError();
+        }
+        if (ok) {
+            r.launch += 1;
+            w->ws = r.ptr;
+            w->flag = r.launch;
+            w->ticket_base = r.ticket;
+            r.ticket += tickets;
+            w->pooled = false;
+            return true;
+        }
+        g_chain_lock.unlock();
+    }
+    w->ws = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(words * sizeof(uint64_t)));
+    if (!w->ws) return false;
+    uint64_t clear_grid = (words + 255) / 256;
+    if (clear_grid > 2048) clear_grid = 2048;
+    hipLaunchKernelGGL(scan_chain_clear_kernel, dim3((unsigned)clear_grid), dim3(256), 0, stream, w->ws, words);
+    return true;
+}
+
+// after the launch that uses the words has been issued
+static void chain_words_release(const ChainWords& w) {
+    // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
+    if (w.pooled) cumo_cuda_runtime_free(reinterpret_cast<char*>(w.ws));
+    else g_chain_lock.unlock();
+}
+
 // returns hipSuccess, or an error; -1 when the run does not suit this form
 template <class T, class Op>
 int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n, hipStream_t stream) {
@@ -684,24 +802,22 @@ int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t
     if (n_tiles < 64 || n_tiles > kChainMaxTiles) return -1;
     if (s1 != (ssize_t)sizeof(T) || s2 != (ssize_t)sizeof(T) || (((uintptr_t)p1 | (uintptr_t)p2) & 15) != 0) return -1;
     const uint64_t n_groups = (n_tiles + 63) / 64, n_supers = (n_groups + 63) / 64;
-    const uint64_t words = 1 + (n_tiles + n_groups + n_supers) * W;
-    uint64_t* ws = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(words * sizeof(uint64_t)));
-    if (!ws) return (int)hipErrorOutOfMemory;
-    uint64_t clear_grid = (words + 255) / 256;
-    if (clear_grid > 1024) clear_grid = 1024;
-    hipLaunchKernelGGL(scan_chain_clear_kernel, dim3((unsigned)clear_grid), dim3(256), 0, stream, ws, words);
+    const uint64_t words = kChainHead + (n_tiles + n_groups + n_supers) * W;
+    ChainWords cw;
+    if (!chain_words_acquire(stream, words, (uint32_t)n_tiles, &cw)) return (int)hipErrorOutOfMemory;
     ScanChain<T> c;
-    c.ticket = reinterpret_cast<uint32_t*>(ws);
-    c.tile = ws + 1;
+    c.ticket = reinterpret_cast<uint32_t*>(cw.ws);
+    c.tile = cw.ws + kChainHead;
     c.group = c.tile + n_tiles * W;
     c.super = c.group + n_groups * W;
+    c.flag = cw.flag;
+    c.ticket_base = cw.ticket_base;
     const bool nt = stream_past_caches(2 * n * sizeof(T));
     const uint64_t grid = n_tiles;
     if (nt) hipLaunchKernelGGL((scan_chain_kernel<T, Op, true>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
     else hipLaunchKernelGGL((scan_chain_kernel<T, Op, false>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
     const int st = (int)hipGetLastError();
-    // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
-    cumo_cuda_runtime_free(reinterpret_cast<char*>(ws));
+    chain_words_release(cw);
     return st;
 }
 
@@ -904,8 +1020,8 @@ void scan_cols_launch_vec(ScanColsParams& p, hipStream_t stream) {
 // a block holds 16 rows of the tile, lane l their vector l, all in registers. A tile adds
 // up its columns (in the lane, then across the waves through LDS), publishes the column
 // totals, gathers what the tiles above it published, and scans its rows from there: the
-// data is read once and written once. The published words are {1, 32 bits of the value};
-// they must be zero before the launch. Tiles take their places by ticket, level by level
+// data is read once and written once. The published words are {the launch's number, 32 bits of
+// the value}, in the region the stream keeps (see above). Tiles take their places by ticket, level by level
 // (all strips of one band of rows, then the next band), so whatever a tile waits for
 // belongs to a block that is already running, and no tile waits before it has published
 // its own totals. What a tile gathers has a fixed shape, so results do not change from
@@ -926,13 +1042,15 @@ struct ScanColsChain {
     uint32_t depth, n_groups, n_supers;  // per strip
     uint32_t strips;                     // per plane
     uint32_t all_strips;                 // planes * strips
+    uint32_t flag;                       // the upper half of a word of this launch
+    uint32_t ticket_base;                // what the ticket word held before this launch
 };
 
 // Up to seven published values, `stride` words apart, the earliest first: all are asked for at
 // once (eight-byte types: four, then three; seven would not fit the registers beside the tile),
 // asked for again until they are there, then folded in order. False when count is 0.
 template <class T, class Op>
-__device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t stride, uint32_t count, T& out) {
+__device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t stride, uint32_t count, uint32_t flag, T& out) {
     constexpr int W = ScanColsChain<T>::W;
     constexpr uint32_t N = kColsChainFan - 1, C = sizeof(T) == 8 ? 4 : N;
     uint32_t polls = 0;
@@ -944,14 +1062,14 @@ __device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t s
         for (uint32_t i = 0; i < C; ++i)
 #pragma unroll
             for (int h = 0; h < W; ++h)
-                x[i][h] = c0 + i < count ? __hip_atomic_load(base + (c0 + i) * stride + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (1ull << 32);
+                x[i][h] = c0 + i < count ? __hip_atomic_load(base + (c0 + i) * stride + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : ((uint64_t)flag << 32);
         for (;;) {
-            uint64_t all = ~0ull;
+            bool all = true;
 #pragma unroll
             for (uint32_t i = 0; i < C; ++i)
 #pragma unroll
-                for (int h = 0; h < W; ++h) all &= x[i][h];
-            if ((all >> 32) & 1u) break;
+                for (int h = 0; h < W; ++h) all = all && (uint32_t)(x[i][h] >> 32) == flag;
+            if (all) break;
             if (++polls > kChainSpinLimit) {
                 __hip_atomic_fetch_add(&g_scan_chain_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 break;
@@ -961,7 +1079,7 @@ __device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t s
             for (uint32_t i = 0; i < C; ++i)
 #pragma unroll
                 for (int h = 0; h < W; ++h)
-                    if (((x[i][h] >> 32) & 1u) == 0) x[i][h] = __hip_atomic_load(base + (c0 + i) * stride + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if ((uint32_t)(x[i][h] >> 32) != flag) x[i][h] = __hip_atomic_load(base + (c0 + i) * stride + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
 #pragma unroll
         for (uint32_t i = 0; i < C; ++i) {
@@ -985,7 +1103,7 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
     __shared__ uint32_t s_ticket;
     static_assert(NW * 64 >= 3 * SW, "three roles of SW threads each");
     const unsigned w = threadIdx.x >> 6, l = threadIdx.x & 63u;
-    if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - c.ticket_base;
     __syncthreads();
     const uint32_t id = s_ticket;
     const uint32_t k = id / c.all_strips, ps = id - k * c.all_strips;
@@ -1038,7 +1156,7 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
             gt = Op::apply(gt, part[ww][col]);
             part[ww][col] = e;
         }
-        chain_publish<T>(c.tile + (((size_t)ps * c.depth + k) * SW + col) * W, gt);
+        chain_publish<T>(c.tile + (((size_t)ps * c.depth + k) * SW + col) * W, gt, c.flag);
     }
     const uint64_t* from = c.tile + (((size_t)ps * c.depth + (size_t)g * kColsChainFan) * SW + col) * W;
     uint32_t count = pos;
@@ -1052,10 +1170,10 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
         count = 0;
     }
     T xs = T();
-    const bool xh = cols_chain_gather<T, Op>(from, cw, count, xs);
+    const bool xh = cols_chain_gather<T, Op>(from, cw, count, c.flag, xs);
     if (role == 0) {
         if (xh) gt = Op::apply(xs, gt);  // the group's total so far
-        if (pos == kColsChainFan - 1) chain_publish<T>(c.group + (((size_t)ps * c.n_groups + g) * SW + col) * W, gt);
+        if (pos == kColsChainFan - 1) chain_publish<T>(c.group + (((size_t)ps * c.n_groups + g) * SW + col) * W, gt, c.flag);
     } else if (role == 1) {
         s_groups[col] = xs;
     } else if (role == 2) {
@@ -1068,7 +1186,7 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
         if (yh) ys = s_groups[col];
         if (pos == kColsChainFan - 1 && gpos == kColsChainFan - 1) {
             const T st = yh ? Op::apply(ys, gt) : gt;
-            chain_publish<T>(c.super + (((size_t)ps * c.n_supers + sg) * SW + col) * W, st);
+            chain_publish<T>(c.super + (((size_t)ps * c.n_supers + sg) * SW + col) * W, st, c.flag);
         }
         bool ph = sg > 0;
         T pre = T();
@@ -1132,18 +1250,16 @@ bool scan_cols_chain_launch(ScanColsParams& p, hipStream_t stream) {
     if (depth < 2 || depth > F * F * F) return false;
     const uint64_t all_strips = strips * p.planes;
     const uint64_t n_tiles = all_strips * depth;
-    if (n_tiles < 512 || n_tiles > 0x7fffffffull) return false;
+    if (n_tiles < 256 || n_tiles > 0x7fffffffull) return false;  // a tile for every compute unit at least
     const uint64_t n_groups = (depth + F - 1) / F, n_supers = (n_groups + F - 1) / F;
-    const uint64_t head = 32;  // the ticket, and the totals on a line of their own
-    const uint64_t words = head + all_strips * (depth + n_groups + n_supers) * SW * W;
-    uint64_t* ws = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(words * sizeof(uint64_t)));
-    if (!ws) return true;
-    uint64_t clear_grid = (words + 255) / 256;
-    if (clear_grid > 2048) clear_grid = 2048;
-    hipLaunchKernelGGL(scan_chain_clear_kernel, dim3((unsigned)clear_grid), dim3(256), 0, stream, ws, words);
+    const uint64_t words = kChainHead + all_strips * (depth + n_groups + n_supers) * SW * W;
+    ChainWords cw;
+    if (!chain_words_acquire(stream, words, (uint32_t)n_tiles, &cw)) return true;
     ScanColsChain<T> c;
-    c.ticket = reinterpret_cast<uint32_t*>(ws);
-    c.tile = ws + head;
+    c.ticket = reinterpret_cast<uint32_t*>(cw.ws);
+    c.tile = cw.ws + kChainHead;
+    c.flag = cw.flag;
+    c.ticket_base = cw.ticket_base;
     c.group = c.tile + all_strips * depth * SW * W;
     c.super = c.group + all_strips * n_groups * SW * W;
     c.depth = (uint32_t)depth;
@@ -1155,8 +1271,7 @@ bool scan_cols_chain_launch(ScanColsParams& p, hipStream_t stream) {
     const dim3 g((unsigned)n_tiles), b(NW * 64);
     if (nt) hipLaunchKernelGGL((scan_cols_chain_kernel<T, Op, true, NW>), g, b, 0, stream, p, c);
     else hipLaunchKernelGGL((scan_cols_chain_kernel<T, Op, false, NW>), g, b, 0, stream, p, c);
-    // stream-ordered reuse: whoever gets the block next can only touch it from later work on this stream
-    cumo_cuda_runtime_free(reinterpret_cast<char*>(ws));
+    chain_words_release(cw);
     return true;
 }
 

@@ -323,7 +323,7 @@ def test_cum_along_columns_of_tall_wide_and_stacked_arrays(tname, dt):
 
 @pytest.mark.parametrize("tname,dt", ALL)
 def test_long_columns_in_one_pass(tname, dt):
-    """Runs across memory whose matrix cuts into at least 512 tiles of 256 rows by 64 vectors are
+    """Runs across memory whose matrix cuts into at least 256 tiles of 256 rows by 64 vectors are
     scanned in one pass: tiles publish their column totals and gather what lies above them through
     groups of 8 tiles and supergroups of 8 groups. Depths of 70 tiles (two supergroups), 35 tiles
     in four planes and 8 tiles (one group, closed by the last tile). Small integers (float sums
@@ -333,7 +333,7 @@ def test_long_columns_in_one_pass(tname, dt):
     cls = cls_of(tname)
     rng = np.random.default_rng(61)
     sw = 64 * (16 // np.dtype(dt).itemsize)
-    for shape, ax in [((256 * 70, 8 * sw), 0), ((4, 256 * 35, 4 * sw), 1), ((256 * 8, 64 * sw), 0)]:
+    for shape, ax in [((256 * 70, 4 * sw), 0), ((4, 256 * 35, 2 * sw), 1), ((256 * 8, 32 * sw), 0)]:
         h = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
             h[..., ::3] = 0
@@ -353,7 +353,7 @@ def test_long_columns_in_one_pass(tname, dt):
             assert_bits_equal(d.cumsum(axis=ax, nan=True).to_numpy(), oracle.cum("cumsum", g, axis=ax, nan=True), (shape, "nan: true"))
             assert_bits_equal(d.cumsum(axis=ax).to_numpy(), oracle.cum("cumsum", g, axis=ax), (shape, "NaN carried"))
         del d
-    shape = (256 * 16, 32 * sw)
+    shape = (256 * 16, 16 * sw)
     wide = rng.integers(-3, 4, size=(2 * shape[0], shape[1])).astype(dt)
     hv = np.ascontiguousarray(wide[::2])
     assert_bits_equal(cls.cast(wide)[::2].cumsum(axis=0).to_numpy(), oracle.cum("cumsum", hv, axis=0), "every other row")

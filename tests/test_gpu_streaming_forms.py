@@ -6,6 +6,8 @@ run on the ordinary suites' small inputs in child processes:
   CUMO_HIP_RED_POLL=0      split reductions with tickets instead of the hand-over words;
   CUMO_HIP_SCAN_CHAIN=0    long runs scanned by the three launches instead of the one pass;
   CUMO_HIP_SCAN_COLS_CHAIN=0  long runs across memory scanned in two passes over segments;
+  CUMO_HIP_SCAN_KEEP_WORDS=0  the one-pass scans with their words from the pool, cleared by a kernel
+                           before each launch (what a stream under capture gets);
   CUMO_HIP_EW_LEAN_ROWS=0  (with CUMO_HIP_NT=1) the general row kernel in its non-temporal forms.
 Each child runs the same parity tests against the oracle as the main suite does."""
 import os
@@ -30,7 +32,7 @@ REDUCE = ["tests/test_gpu_reduce.py::test_float_reductions_every_axis", "tests/t
           "tests/test_gpu_reduce.py::test_min_max_keep_the_zero_that_came_first"]
 ADJACENT = ["tests/test_gpu_adjacent.py::test_clip_parity_over_views", "tests/test_gpu_adjacent.py::test_float_pow_parity",
             "tests/test_gpu_adjacent.py::test_cumsum_cumprod_parity", "tests/test_gpu_adjacent.py::test_cum_along_contiguous_runs_of_whole_chunks",
-            "tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass", "tests/test_gpu_adjacent.py::test_long_columns_in_one_pass",
+            "tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass",
             "tests/test_gpu_adjacent.py::test_cum_along_columns_of_tall_wide_and_stacked_arrays", "tests/test_gpu_adjacent.py::test_mulsum_parity"]
 OTHERS = ["tests/test_gpu_index.py::test_gather_and_scatter_between_view_and_buffer", "tests/test_gpu_index.py::test_getitem_with_index_arrays",
           "tests/test_gpu_index.py::test_setitem_with_index_arrays_and_slices", "tests/test_gpu_fused.py", "tests/test_gpu_configs.py"]
@@ -59,5 +61,10 @@ def test_reductions_with_tickets():
 
 def test_long_runs_scanned_by_three_launches():
     run_child({"CUMO_HIP_SCAN_CHAIN": "0", "CUMO_HIP_SCAN_COLS_CHAIN": "0"},
-              ["tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass", "tests/test_gpu_adjacent.py::test_long_columns_in_one_pass",
-               "tests/test_gpu_adjacent.py::test_cumsum_cumprod_parity"])
+              ["tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass", "tests/test_gpu_adjacent.py::test_cumsum_cumprod_parity",
+               "tests/test_gpu_adjacent.py::test_long_columns_in_one_pass"])
+
+
+def test_one_pass_scans_with_cleared_words_from_the_pool():
+    run_child({"CUMO_HIP_SCAN_KEEP_WORDS": "0"},
+              ["tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass", "tests/test_gpu_adjacent.py::test_long_columns_in_one_pass"])
