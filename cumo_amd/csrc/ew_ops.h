@@ -668,6 +668,10 @@ template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) s
 
 // Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
 // element type for small exponents, pow() beyond 64, the reciprocal for negative ones.
+// (out of line: inlined at every element, the library's pow took 66 registers of a kernel that needs 10)
+template <class T>
+__device__ __attribute__((noinline)) T pow_float_int_by_the_library(T x, uint32_t q) { return (T)pow((double)x, (double)q); }
+
 template <class T>
 __device__ __forceinline__ T pow_float_int(T x, int32_t p) {
     const bool neg = p < 0;
@@ -681,7 +685,7 @@ __device__ __forceinline__ T pow_float_int(T x, int32_t p) {
         case 4: x = x * x; r = x * x; break;
         default:
             if (q > 64) {
-                r = (T)pow((double)x, (double)q);
+                r = pow_float_int_by_the_library<T>(x, q);
             } else {
                 while (q) {
                     if (q & 1u) r *= x;
