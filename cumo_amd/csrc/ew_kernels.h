@@ -928,14 +928,13 @@ __device__ __forceinline__ void ew_tile_at(const EwTParams& p, uint64_t tile, ui
 // NT: the transposed reads and the stores are non-temporal (operations too large for
 // the caches; measured on an 8192 x 4096 SFloat transposed copy with every launch on
 // fresh operands: 58 us with plain accesses, 50 us with non-temporal ones).
-template <class Op, int TG, bool PREFETCH, int TRMODE, bool NT>
+template <class Op, int TF, int TG, bool PREFETCH, int TRMODE, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p, Op op, typename Op::S sv) {
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;
     constexpr int NIN = Op::NIN;
     constexpr bool TWO = (NIN == 2);
-    constexpr int TF = 64;
     constexpr int V = 16 / (int)sizeof(A);
     constexpr unsigned GV = TG / V;          // 128-bit slots along G
     constexpr unsigned FP = kEwBlock / GV;   // F positions per pass of the read
@@ -1314,11 +1313,18 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 // an op with many instructions per element: 256-byte tiles, eight blocks per compute
                 // unit, each with its next tile in flight. Otherwise tiles of 512 bytes along the
                 // transposed inputs' fast dimension, one per block (measured on a transposed
-                // 8192 x 4096 SFloat copy: 39.4 us against 45.3 us with 256 bytes).
+                // 8192 x 4096 SFloat copy that finds its operands in the caches: 39.4 us against 45.3 us
+                // with 256 bytes).
+                // Operations that stream past the caches take tiles of 128 x 256 bytes instead: the stores
+                // then fill 512 bytes of a result row at a time (bare transposed copy of the 8192 x 4096
+                // SFloat view on fresh operands: 49.1 -> 47.6 us).
                 constexpr bool PF = op_is_heavy<Op>::value;
-                constexpr int TGV = (PF ? 256 : 512) / (int)sizeof(A);
+                constexpr int TGC = (PF ? 256 : 512) / (int)sizeof(A), TFC = 64;   // operands in the caches
+                constexpr int TGS = 256 / (int)sizeof(A), TFS = PF ? 64 : 128;      // streaming
+                const int TGV = tr_nt ? TGS : TGC, TFV = tr_nt ? TFS : TFC;
+                tp.f_tiles = (tp.nf + TFV - 1) / TFV;
                 tp.g_tiles = (tp.ng + TGV - 1) / TGV;
-                if (tp.order == 2 && (tp.g_tiles & 7)) tp.order = 0;
+                if (tp.order == 2 && ((tp.f_tiles & 7) || (tp.g_tiles & 7))) tp.order = 0;
                 tp.n_tiles = tp.f_tiles * tp.g_tiles * outer;
                 grid = tp.n_tiles < vgrid ? tp.n_tiles : vgrid;
                 if (PF) {
@@ -1330,12 +1336,19 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                     }
                     if (grid > pgrid) grid = pgrid;
                 }
-                const size_t lds = sizeof(A) * TGV * 65 + (b_through_lds ? sizeof(B) * TGV * 65 : 0);
+                const size_t lds = sizeof(A) * TGV * (TFV + 1) + (b_through_lds ? sizeof(B) * TGV * (TFV + 1) : 0);
                 const dim3 g((unsigned)grid), b(kEwBlock);
 #define CUMO_TR_LAUNCH(MODE)                                                                                                       \
     do {                                                                                                                            \
-        if (tr_nt) hipLaunchKernelGGL((ew_transpose_vec_kernel<Op, TGV, PF, MODE, true>), g, b, lds, stream, tp, op, sv);          \
-        else hipLaunchKernelGGL((ew_transpose_vec_kernel<Op, TGV, PF, MODE, false>), g, b, lds, stream, tp, op, sv);               \
+        if (tr_nt) {                                                                                                                \
+            auto kernel = ew_transpose_vec_kernel<Op, TFS, TGS, PF, MODE, true>;                                                    \
+            if (lds > 65536) (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
+            hipLaunchKernelGGL(kernel, g, b, lds, stream, tp, op, sv);                                                              \
+        } else {                                                                                                                    \
+            auto kernel = ew_transpose_vec_kernel<Op, TFC, TGC, PF, MODE, false>;                                                   \
+            if (lds > 65536) (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
+            hipLaunchKernelGGL(kernel, g, b, lds, stream, tp, op, sv);                                                              \
+        }                                                                                                                           \
     } while (0)
                 if constexpr (Op::NIN >= 2) {
                     if (a_through_lds && b_through_lds) CUMO_TR_LAUNCH(3);
