@@ -75,10 +75,10 @@ __device__ __forceinline__ T scan_shfl_up(T v, unsigned d) {
 // `carry` is the running value before the tile and has_carry says whether there is
 // one. Returns the running value after the tile in every lane (has_carry becomes true
 // when the tile is not empty).
-template <class T, class Op>
+template <class T, class Op, int NWAVES = kScanBlock / 64>
 __device__ __forceinline__ void scan_tile(T (&v)[kScanPer], int cnt, T& carry, bool& has_carry) {
-    __shared__ T wave_tot[kScanBlock / 64];
-    __shared__ int wave_has[kScanBlock / 64];
+    __shared__ T wave_tot[NWAVES];
+    __shared__ int wave_has[NWAVES];
     const int t = threadIdx.x;
     const int base = t * kScanPer;
     int mine = cnt - base;  // how many of this lane's elements exist
@@ -118,7 +118,7 @@ __device__ __forceinline__ void scan_tile(T (&v)[kScanPer], int cnt, T& carry, b
     T run = carry;          // the running value after the whole tile, for every lane
     bool run_has = has_carry;
 #pragma unroll
-    for (int j = 0; j < kScanBlock / 64; ++j) {
+    for (int j = 0; j < NWAVES; ++j) {
         if (wave_has[j]) {
             run = run_has ? Op::apply(run, wave_tot[j]) : wave_tot[j];
             run_has = true;
@@ -503,7 +503,7 @@ __device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first
 // The tile in v (already loaded) scanned by itself: afterwards every element holds the running
 // value from the start of its wave's quarter, `total` is the tile's total and `wave_pre` the
 // total of the waves before this one (for wave 0: nothing). One barrier, met by every thread.
-template <class T, class Op, int R>
+template <class T, class Op, int R, int NW = kScanBlock / 64>
 __device__ __forceinline__ void chain_scan_tile(ChainVec<T> (&v)[R], T* s_wave_tot, T& total, T& wave_pre) {
     constexpr int V = ChainVec<T>::V;
     const unsigned lane = threadIdx.x & 63u;
@@ -543,7 +543,7 @@ __device__ __forceinline__ void chain_scan_tile(ChainVec<T> (&v)[R], T* s_wave_t
     total = s_wave_tot[0];
     wave_pre = T();
 #pragma unroll
-    for (int j = 1; j < kScanBlock / 64; ++j) {
+    for (int j = 1; j < NW; ++j) {
         if (j == w) wave_pre = total;
         total = Op::apply(total, s_wave_tot[j]);
     }
@@ -573,11 +573,11 @@ __device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, Chai
 }
 
 // scans the tile in v (already loaded), looks back, stores; the barriers inside are met by every thread
-template <class T, class Op, bool NT, int R>
+template <class T, class Op, bool NT, int R, int NW>
 __device__ __forceinline__ void chain_finish_tile(char* out, uint64_t first, uint32_t t, ChainVec<T> (&v)[R], const ScanChain<T>& c,
                                                   T* s_wave_tot, T* s_prefix, ChainShared* sh) {
     T total, wave_pre;
-    chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
+    chain_scan_tile<T, Op, R, NW>(v, s_wave_tot, total, wave_pre);
     if (threadIdx.x < 64) {
         T pre;
         bool pre_has;
@@ -625,14 +625,15 @@ __global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsPar
     }
 }
 
-template <class T, class Op, bool NT>
-__global__ __launch_bounds__(kScanBlock, sizeof(T) == 8 ? 3 : 4) void scan_chain_kernel(const char* in, char* out, uint64_t n, ScanChain<T> c) {
-    constexpr int TILE = ScanChain<T>::TILE;
+template <class T, class Op, bool NT, int NW>
+__global__ __launch_bounds__(NW * 64, sizeof(T) == 8 ? 3 : 4) void scan_chain_kernel(const char* in, char* out, uint64_t n, ScanChain<T> c) {
     constexpr int V = ChainVec<T>::V;
-    constexpr int R = TILE / (kScanBlock * V);
+    constexpr int R = ScanChain<T>::TILE / (kScanBlock * V);   // rows of 64 vectors per wave
+    constexpr int TILE = NW * R * 64 * V;
+    constexpr int PIECE = NW * 64 * kScanPer;                  // what the block-wide scan takes at a time
     __shared__ ChainShared sh;
     __shared__ T s_prefix;
-    __shared__ T s_wave_tot[kScanBlock / 64];
+    __shared__ T s_wave_tot[NW];
     if (threadIdx.x == 0) sh.tile = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - c.ticket_base;
     __syncthreads();
     const uint32_t t = sh.tile;
@@ -641,19 +642,19 @@ __global__ __launch_bounds__(kScanBlock, sizeof(T) == 8 ? 3 : 4) void scan_chain
     if (n - first >= (uint64_t)TILE) {
         ChainVec<T> v[R];
         chain_issue_loads<T, NT, R>(in, first, v);
-        chain_finish_tile<T, Op, NT, R>(out, first, t, v, c, s_wave_tot, &s_prefix, &sh);
+        chain_finish_tile<T, Op, NT, R, NW>(out, first, t, v, c, s_wave_tot, &s_prefix, &sh);
         return;
     }
     // the ragged last tile: its total first, then the scan from what the look-back gives
     T total = T();
     bool total_has = false;
 #pragma clang loop unroll(disable)
-    for (uint64_t f = first; f < n; f += kScanTile) {
+    for (uint64_t f = first; f < n; f += PIECE) {
         const uint64_t left = n - f;
-        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
+        const int cnt = left < (uint64_t)PIECE ? (int)left : PIECE;
         T v[kScanPer];
         scan_load<T>(in, (int64_t)sizeof(T), f, cnt, v);
-        scan_tile<T, Op>(v, cnt, total, total_has);
+        scan_tile<T, Op, NW>(v, cnt, total, total_has);
     }
     if (threadIdx.x < 64) {
         T pre;
@@ -668,12 +669,12 @@ __global__ __launch_bounds__(kScanBlock, sizeof(T) == 8 ? 3 : 4) void scan_chain
     T carry = s_prefix;
     bool has_carry = sh.prefix_has != 0;
 #pragma clang loop unroll(disable)
-    for (uint64_t f = first; f < n; f += kScanTile) {
+    for (uint64_t f = first; f < n; f += PIECE) {
         const uint64_t left = n - f;
-        const int cnt = left < (uint64_t)kScanTile ? (int)left : kScanTile;
+        const int cnt = left < (uint64_t)PIECE ? (int)left : PIECE;
         T v[kScanPer];
         scan_load<T>(in, (int64_t)sizeof(T), f, cnt, v);
-        scan_tile<T, Op>(v, cnt, carry, has_carry);
+        scan_tile<T, Op, NW>(v, cnt, carry, has_carry);
         scan_store<T>(out, (int64_t)sizeof(T), f, cnt, v);
     }
 }
@@ -798,7 +799,16 @@ static void chain_words_release(const ChainWords& w) {
 template <class T, class Op>
 int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n, hipStream_t stream) {
     constexpr int W = ScanChain<T>::W;
-    const uint64_t n_tiles = (n + ScanChain<T>::TILE - 1) / ScanChain<T>::TILE;
+    // blocks of four waves and 64 KiB tiles; from 512 tiles of 128 KiB on, blocks of eight waves (half the
+    // tickets and look-backs; CUMO_HIP_SCAN_CHAIN_WAVES=4 or 8, read once, fixes the choice)
+    static const int forced_waves = [] {
+        const char* e = std::getenv("CUMO_HIP_SCAN_CHAIN_WAVES");
+        return e ? std::atoi(e) : 0;
+    }();
+    const uint64_t wide_tile = 2ull * ScanChain<T>::TILE;
+    const bool wide = forced_waves == 8 || (forced_waves != 4 && n / wide_tile >= 512);
+    const uint64_t tile = wide ? wide_tile : (uint64_t)ScanChain<T>::TILE;
+    const uint64_t n_tiles = (n + tile - 1) / tile;
     if (n_tiles < 64 || n_tiles > kChainMaxTiles) return -1;
     if (s1 != (ssize_t)sizeof(T) || s2 != (ssize_t)sizeof(T) || (((uintptr_t)p1 | (uintptr_t)p2) & 15) != 0) return -1;
     const uint64_t n_groups = (n_tiles + 63) / 64, n_supers = (n_groups + 63) / 64;
@@ -814,8 +824,13 @@ int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t
     c.ticket_base = cw.ticket_base;
     const bool nt = stream_past_caches(2 * n * sizeof(T));
     const uint64_t grid = n_tiles;
-    if (nt) hipLaunchKernelGGL((scan_chain_kernel<T, Op, true>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
-    else hipLaunchKernelGGL((scan_chain_kernel<T, Op, false>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
+    if (wide) {
+        if (nt) hipLaunchKernelGGL((scan_chain_kernel<T, Op, true, 8>), dim3((unsigned)grid), dim3(8 * 64), 0, stream, p1, p2, n, c);
+        else hipLaunchKernelGGL((scan_chain_kernel<T, Op, false, 8>), dim3((unsigned)grid), dim3(8 * 64), 0, stream, p1, p2, n, c);
+    } else {
+        if (nt) hipLaunchKernelGGL((scan_chain_kernel<T, Op, true, 4>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
+        else hipLaunchKernelGGL((scan_chain_kernel<T, Op, false, 4>), dim3((unsigned)grid), dim3(kScanBlock), 0, stream, p1, p2, n, c);
+    }
     const int st = (int)hipGetLastError();
     chain_words_release(cw);
     return st;

@@ -5,6 +5,8 @@ run on the ordinary suites' small inputs in child processes:
                            non-temporal gather / scatter, mulsum, scans and fused rows;
   CUMO_HIP_RED_POLL=0      split reductions with tickets instead of the hand-over words;
   CUMO_HIP_SCAN_CHAIN=0    long runs scanned by the three launches instead of the one pass;
+  CUMO_HIP_SCAN_CHAIN_WAVES=4 the one pass over one long run by blocks of four waves at every size (4097 tiles: the
+                           second supergroup);
   CUMO_HIP_SCAN_COLS_CHAIN=0  long runs across memory scanned in two passes over segments;
   CUMO_HIP_SCAN_KEEP_WORDS=0  the one-pass scans with their words from the pool, cleared by a kernel
                            before each launch (what a stream under capture gets);
@@ -68,3 +70,7 @@ def test_long_runs_scanned_by_three_launches():
 def test_one_pass_scans_with_cleared_words_from_the_pool():
     run_child({"CUMO_HIP_SCAN_KEEP_WORDS": "0"},
               ["tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass", "tests/test_gpu_adjacent.py::test_long_columns_in_one_pass"])
+
+
+def test_one_long_run_by_blocks_of_four_waves():
+    run_child({"CUMO_HIP_SCAN_CHAIN_WAVES": "4"}, ["tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass"])
