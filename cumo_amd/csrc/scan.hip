@@ -799,14 +799,17 @@ static void chain_words_release(const ChainWords& w) {
 template <class T, class Op>
 int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t n, hipStream_t stream) {
     constexpr int W = ScanChain<T>::W;
-    // blocks of four waves and 64 KiB tiles; from 512 tiles of 128 KiB on, blocks of eight waves (half the
-    // tickets and look-backs; CUMO_HIP_SCAN_CHAIN_WAVES=4 or 8, read once, fixes the choice)
+    // Blocks of eight waves and 128 KiB tiles for four-byte elements wherever that leaves 64 tiles (half the
+    // tickets and look-backs per byte: 2^26 SFloat 115 -> 111 us, 2^24 39 -> 33 us), else blocks of four waves
+    // and 64 KiB tiles; eight-byte elements always those (their kernel needs 168 registers, and one block of
+    // eight waves would have a compute unit to itself: 2^26 DFloat 224 us against 260 us).
+    // CUMO_HIP_SCAN_CHAIN_WAVES=4 or 8, read once, fixes the choice.
     static const int forced_waves = [] {
         const char* e = std::getenv("CUMO_HIP_SCAN_CHAIN_WAVES");
         return e ? std::atoi(e) : 0;
     }();
     const uint64_t wide_tile = 2ull * ScanChain<T>::TILE;
-    const bool wide = forced_waves == 8 || (forced_waves != 4 && n / wide_tile >= 512);
+    const bool wide = forced_waves == 8 || (forced_waves != 4 && sizeof(T) == 4 && (n + wide_tile - 1) / wide_tile >= 64);
     const uint64_t tile = wide ? wide_tile : (uint64_t)ScanChain<T>::TILE;
     const uint64_t n_tiles = (n + tile - 1) / tile;
     if (n_tiles < 64 || n_tiles > kChainMaxTiles) return -1;

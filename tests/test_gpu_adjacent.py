@@ -253,10 +253,10 @@ def test_cum_along_contiguous_runs_of_whole_chunks(tname, dt):
 
 @pytest.mark.parametrize("tname,dt", ALL)
 def test_one_long_run_in_one_pass(tname, dt):
-    """Runs from 64 tiles of 64 KiB on are scanned in one pass (from 512 tiles of 128 KiB on, by
-    blocks of eight waves with those tiles), tiles handing their totals on through groups of 64
-    and supergroups of 64 groups: sizes that end exactly on a group, one element past it, exactly
-    where the larger tiles begin and one element past that, and 4096 small (2048 large) tiles with
+    """Runs from 64 tiles of 64 KiB on are scanned in one pass (four-byte elements: by blocks of
+    eight waves with tiles of 128 KiB once there are 64 of those), tiles handing their totals on
+    through groups of 64 and supergroups of 64 groups: sizes that end exactly on a group, one
+    element past it, the same for the larger tiles, and 4096 small (2048 large) tiles with
     a ragged tail; small integers (float sums
     exact in any order), so every result is compared bit for bit with the sequential scan.
     Then what only the order-free comparison can hold: products of +-1 and 2, NaN skipped
@@ -265,7 +265,7 @@ def test_one_long_run_in_one_pass(tname, dt):
     cls = cls_of(tname)
     rng = np.random.default_rng(57)
     tile = 65536 // np.dtype(dt).itemsize
-    for n in (64 * tile, 64 * tile + 1, 65 * tile + 3001, 1024 * tile, 1024 * tile + 1, 64 * 64 * tile + 70001):
+    for n in (64 * tile, 64 * tile + 1, 65 * tile + 3001, 128 * tile, 128 * tile + 1, 131 * tile + 77, 64 * 64 * tile + 70001):
         h = rng.integers(-3, 4, size=n).astype(dt)
         if dt != np.int32:
             h[::3] = 0   # keeps the running float sums far below 2^24
