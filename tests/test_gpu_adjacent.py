@@ -325,7 +325,7 @@ def test_cum_along_columns_of_tall_wide_and_stacked_arrays(tname, dt):
 
 @pytest.mark.parametrize("tname,dt", ALL)
 def test_long_columns_in_one_pass(tname, dt):
-    """Runs across memory whose matrix cuts into at least 256 tiles of 256 rows by 64 vectors are
+    """Runs across memory whose matrix cuts into at least 16 tiles of 256 rows by 64 vectors are
     scanned in one pass: tiles publish their column totals and gather what lies above them through
     groups of 8 tiles and supergroups of 8 groups. Depths of 70 tiles (two supergroups), 35 tiles
     in four planes and 8 tiles (one group, closed by the last tile). Small integers (float sums
@@ -335,7 +335,7 @@ def test_long_columns_in_one_pass(tname, dt):
     cls = cls_of(tname)
     rng = np.random.default_rng(61)
     sw = 64 * (16 // np.dtype(dt).itemsize)
-    for shape, ax in [((256 * 70, 4 * sw), 0), ((4, 256 * 35, 2 * sw), 1), ((256 * 8, 32 * sw), 0)]:
+    for shape, ax in [((256 * 70, 4 * sw), 0), ((4, 256 * 35, 2 * sw), 1), ((256 * 8, 32 * sw), 0), ((256 * 9, 2 * sw), 0), ((512, 8 * sw), 0)]:
         h = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
             h[..., ::3] = 0
