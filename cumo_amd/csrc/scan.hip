@@ -1143,9 +1143,24 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
     const int64_t colb = ((int64_t)strip * SW + (int64_t)l * V) * (int64_t)sizeof(T);
     const char* src = p.in + oi + row0 * p.s_in + colb;
     char* dst = p.out + oo + row0 * p.s_out + colb;
+    // A tile at the lower edge has fewer rows and one at the right edge fewer columns: this wave's first
+    // `rows` rows exist, and this lane's columns do or do not. What such a tile reads as missing is zeros;
+    // the totals they enter are only ever used by rows or columns that do not exist either.
+    const int64_t rows_left = (int64_t)p.n - row0;
+    const int rows = rows_left >= R ? R : (rows_left > 0 ? (int)rows_left : 0);
+    const bool cols_here = (uint64_t)strip * SW + (uint64_t)l * V < p.cols;
     T raw[R][V];
+    if (rows == R && __builtin_amdgcn_ballot_w64(!cols_here) == 0) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
+        for (int r = 0; r < R; ++r) scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) raw[r][j] = T();
+            if (r < rows && cols_here) scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
+        }
+    }
     {
         T tot[V];
 #pragma unroll
@@ -1239,12 +1254,22 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
             acc[j] = o.t;
         }
     }
-    scan_cols_store<T, V, NT>(dst, acc);
+    if (rows == R && __builtin_amdgcn_ballot_w64(!cols_here) == 0) {
+        scan_cols_store<T, V, NT>(dst, acc);
 #pragma unroll
-    for (int r = 1; r < R; ++r) {
+        for (int r = 1; r < R; ++r) {
 #pragma unroll
-        for (int j = 0; j < V; ++j) acc[j] = Op::apply(acc[j], raw[r][j]);
-        scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
+            for (int j = 0; j < V; ++j) acc[j] = Op::apply(acc[j], raw[r][j]);
+            scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
+        }
+    } else if (cols_here) {
+        if (rows > 0) scan_cols_store<T, V, NT>(dst, acc);
+#pragma unroll
+        for (int r = 1; r < R; ++r) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] = Op::apply(acc[j], raw[r][j]);
+            if (r < rows) scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
+        }
     }
 }
 
@@ -1262,8 +1287,8 @@ bool scan_cols_chain_launch(ScanColsParams& p, hipStream_t stream) {
     constexpr int V = 16 / (int)sizeof(T), W = ScanColsChain<T>::W, NW = 16;
     constexpr uint64_t SW = 64 * V, TR = (uint64_t)NW * kColsChainRows;
     if (!scan_cols_chain_enabled()) return false;
-    if (p.cols % SW != 0 || p.n % TR != 0) return false;
-    const uint64_t depth = p.n / TR, strips = p.cols / SW;
+    if (p.cols < SW) return false;  // (a strip of 64 vectors is the unit: narrower arrays would leave most lanes idle)
+    const uint64_t depth = (p.n + TR - 1) / TR, strips = (p.cols + SW - 1) / SW;
     constexpr uint64_t F = kColsChainFan;
     if (depth < 2 || depth > F * F * F) return false;
     const uint64_t all_strips = strips * p.planes;

@@ -328,14 +328,18 @@ def test_long_columns_in_one_pass(tname, dt):
     """Runs across memory whose matrix cuts into at least 16 tiles of 256 rows by 64 vectors are
     scanned in one pass: tiles publish their column totals and gather what lies above them through
     groups of 8 tiles and supergroups of 8 groups. Depths of 70 tiles (two supergroups), 35 tiles
-    in four planes and 8 tiles (one group, closed by the last tile). Small integers (float sums
+    in four planes and 8 tiles (one group, closed by the last tile); tiles at the lower and right
+    edges that are only partly there (845 rows by two strips and three vectors; three planes of
+    1000 rows by a strip and a vector). Small integers (float sums
     exact in any order): bit for bit against the sequential scan; products of +-1 and a few 2s;
     NaN skipped (every run starts with more than a tile of NaN) and carried; every other row of a
     taller array; random floats give the same bits from launch to launch and stay close."""
     cls = cls_of(tname)
     rng = np.random.default_rng(61)
     sw = 64 * (16 // np.dtype(dt).itemsize)
-    for shape, ax in [((256 * 70, 4 * sw), 0), ((4, 256 * 35, 2 * sw), 1), ((256 * 8, 32 * sw), 0), ((256 * 9, 2 * sw), 0), ((512, 8 * sw), 0)]:
+    vec = 16 // np.dtype(dt).itemsize
+    for shape, ax in [((256 * 70, 4 * sw), 0), ((4, 256 * 35, 2 * sw), 1), ((256 * 8, 32 * sw), 0), ((256 * 9, 2 * sw), 0), ((512, 8 * sw), 0),
+                      ((256 * 3 + 77, 6 * sw + 3 * vec), 0), ((3, 1000, 2 * sw + vec), 1), ((257, 16 * sw), 0)]:
         h = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
             h[..., ::3] = 0
