@@ -7,13 +7,19 @@
 // treat NaN as "nothing yet", which makes them associative like the plain ones.
 // Like a sum, a parallel float scan does not add strictly left to right.
 //
-// Two kernels:
-//   scan_rows_kernel   one block per run, tile after tile with the running value
-//                      carried along: many runs (an axis of a matrix), or short ones.
-//   three launches     for few long runs: per-tile totals, a scan of the totals (by this
-//                      same scheme while they are many, else by one block), then every
-//                      tile scans itself from its offset. Reads the input twice and
-//                      writes once.
+// The forms, by layout:
+//   scan_rows_kernel        one block per run, tile after tile with the running value
+//                           carried along: many runs (an axis of a matrix), or short ones;
+//   scan_rows_whole_kernel  the same for contiguous runs of whole 256-vector chunks, held
+//                           in registers wave by wave;
+//   scan_chain_kernel       one long contiguous run in one pass: tiles hand their totals on
+//                           through words in memory (read once, written once);
+//   three launches          one long run that is strided or unaligned: per-tile totals, a
+//                           scan of the totals, then every tile scans itself from its
+//                           offset (reads the input twice);
+//   scan_cols_chain_kernel  long runs that lie across memory (down the rows of a matrix) in
+//                           one pass, tiles of 256 rows handing on their column totals;
+//   scan_cols_kernel        other runs across memory, in segments and two passes.
 // Inside a tile each lane owns 8 consecutive elements: it scans them in registers,
 // the lane totals are scanned across the wave with shuffles and the four wave
 // totals through LDS. Everything is in a fixed order, so results do not change
