@@ -495,15 +495,25 @@ struct ChainShared {
     int prefix_has;
 };
 
-template <class T, bool NT, int R>
-__device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first, ChainVec<T> (&v)[R]) {
+// RAGGED: only the first nvec vectors from `first` on exist; the others read as zeros (they lie
+// after everything that exists, so what they add to never reaches an element that is stored)
+template <class T, bool NT, int R, bool RAGGED = false>
+__device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first, ChainVec<T> (&v)[R], uint32_t nvec = 0) {
     typedef typename ChainVec<T>::u4 u4;
     constexpr int V = ChainVec<T>::V;
     const unsigned lane = threadIdx.x & 63u;
     const int w = threadIdx.x >> 6;
     const u4* src = reinterpret_cast<const u4*>(in + (first + (uint64_t)w * (R * 64 * V)) * sizeof(T)) + lane;
 #pragma unroll
-    for (int r = 0; r < R; ++r) v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
+    for (int r = 0; r < R; ++r) {
+        if (RAGGED) {
+            const u4 zero = {0u, 0u, 0u, 0u};
+            v[r].q = zero;
+            if ((uint32_t)(w * R * 64 + r * 64) + lane < nvec) v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
+        } else {
+            v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
+        }
+    }
 }
 
 // The tile in v (already loaded) scanned by itself: afterwards every element holds the running
@@ -556,8 +566,8 @@ __device__ __forceinline__ void chain_scan_tile(ChainVec<T> (&v)[R], T* s_wave_t
 }
 
 // adds what precedes the tile (if anything) and the earlier waves' total, and stores
-template <class T, class Op, bool NT, int R>
-__device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, ChainVec<T> (&v)[R], T head, bool head_has, T wave_pre) {
+template <class T, class Op, bool NT, int R, bool RAGGED = false>
+__device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, ChainVec<T> (&v)[R], T head, bool head_has, T wave_pre, uint32_t nvec = 0) {
     typedef typename ChainVec<T>::u4 u4;
     constexpr int V = ChainVec<T>::V;
     const unsigned lane = threadIdx.x & 63u;
@@ -573,6 +583,7 @@ __device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, Chai
 #pragma unroll
             for (int e = 0; e < V; ++e) v[r].e[e] = Op::apply(head, v[r].e[e]);
         }
+        if (RAGGED && !((uint32_t)(w * R * 64 + r * 64) + lane < nvec)) continue;
         if (NT) __builtin_nontemporal_store(v[r].q, dst + r * 64);
         else dst[r * 64] = v[r].q;
     }
@@ -597,9 +608,9 @@ __device__ __forceinline__ void chain_finish_tile(char* out, uint64_t first, uin
     chain_store_tile<T, Op, NT, R>(out, first, v, *s_prefix, sh->prefix_has != 0, wave_pre);
 }
 
-// Many runs, each contiguous on both sides, 16-byte aligned and a whole number of chunks of
-// R * 256 vectors long: one block per run, chunk after chunk in the same wave-by-wave form,
-// the running value handed on in a register.
+// Many runs, each contiguous on both sides, 16-byte aligned and a whole number of vectors
+// long: one block per run, chunk after chunk of R * 256 vectors in the same wave-by-wave form,
+// the running value handed on in a register; the last chunk may be partly there.
 template <class T, class Op, bool NT, int R>
 __global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsParams p) {
     constexpr int V = ChainVec<T>::V;
@@ -620,10 +631,18 @@ __global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsPar
         bool has_carry = false;
         for (uint64_t first = 0; first < p.n; first += CHUNK) {
             ChainVec<T> v[R];
-            chain_issue_loads<T, NT, R>(p.in + oi, first, v);
             T total, wave_pre;
-            chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
-            chain_store_tile<T, Op, NT, R>(p.out + oo, first, v, carry, has_carry, wave_pre);
+            if (p.n - first >= CHUNK) {
+                chain_issue_loads<T, NT, R>(p.in + oi, first, v);
+                chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
+                chain_store_tile<T, Op, NT, R>(p.out + oo, first, v, carry, has_carry, wave_pre);
+            } else {
+                // the run's last chunk, partly there (the run is a whole number of vectors)
+                const uint32_t nvec = (uint32_t)((p.n - first) / V);
+                chain_issue_loads<T, NT, R, true>(p.in + oi, first, v, nvec);
+                chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
+                chain_store_tile<T, Op, NT, R, true>(p.out + oo, first, v, carry, has_carry, wave_pre, nvec);
+            }
             carry = has_carry ? Op::apply(carry, total) : total;
             has_carry = true;
             __syncthreads();  // s_wave_tot is written again by the next chunk
@@ -1353,18 +1372,19 @@ void scan_rows_launch(const ScanRowsParams& p, hipStream_t stream) {
     uint64_t grid = p.rows;
     if (grid > 65536) grid = 65536;
     constexpr uint64_t V = 16 / sizeof(T);
-    bool whole = p.s_in == (int64_t)sizeof(T) && p.s_out == (int64_t)sizeof(T) && p.n % (kScanBlock * V) == 0 &&
+    bool whole = p.s_in == (int64_t)sizeof(T) && p.s_out == (int64_t)sizeof(T) && p.n % V == 0 && p.n >= 64 * V &&
                  (((uintptr_t)p.in | (uintptr_t)p.out) & 15) == 0;
     for (int d = 0; d < p.nouter && whole; ++d) whole = (p.ostep_in[d] % 16) == 0 && (p.ostep_out[d] % 16) == 0;
     if (whole) {
-        const uint64_t vec_rows = p.n / (kScanBlock * V);  // rows of 256 vectors in a run
+        const uint64_t vec_rows = (p.n + kScanBlock * V - 1) / (kScanBlock * V);  // rows of 256 vectors in a run, the last one maybe partly there
         const bool nt = stream_past_caches(2 * p.rows * p.n * sizeof(T));
         const dim3 g((unsigned)grid), b(kScanBlock);
 #define CUMO_SCAN_WHOLE(R_) do { if (nt) hipLaunchKernelGGL((scan_rows_whole_kernel<T, Op, true, R_>), g, b, 0, stream, p); \
                                  else hipLaunchKernelGGL((scan_rows_whole_kernel<T, Op, false, R_>), g, b, 0, stream, p); } while (0)
-        if (vec_rows % 8 == 0) CUMO_SCAN_WHOLE(8);
-        else if (vec_rows % 4 == 0) CUMO_SCAN_WHOLE(4);
-        else if (vec_rows % 2 == 0) CUMO_SCAN_WHOLE(2);
+        // chunks of 8, 4, 2 or 1 such rows: the largest that the run fills at least once, or that holds all of it
+        if (vec_rows > 4) CUMO_SCAN_WHOLE(8);
+        else if (vec_rows > 2) CUMO_SCAN_WHOLE(4);
+        else if (vec_rows > 1) CUMO_SCAN_WHOLE(2);
         else CUMO_SCAN_WHOLE(1);
 #undef CUMO_SCAN_WHOLE
         return;

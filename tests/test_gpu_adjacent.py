@@ -221,14 +221,18 @@ def test_cum_nan_forms_on_random_placements(tname, dt):
 
 @pytest.mark.parametrize("tname,dt", ALL)
 def test_cum_along_contiguous_runs_of_whole_chunks(tname, dt):
-    """Many contiguous runs whose length is a whole number of 256 vectors take a kernel that
-    scans a run chunk by chunk in registers: one, two, four and eight rows of vectors per
-    chunk, one and several chunks per run, outer dimensions with padding between the runs.
+    """Many contiguous runs whose length is a whole number of vectors (64 at least) take a kernel
+    that scans a run chunk by chunk in registers: one, two, four and eight rows of 256 vectors per
+    chunk, one and several chunks per run, the last chunk full or partly there (down to one vector
+    past a chunk, and a run of 65 vectors), outer dimensions with padding between the runs.
     Small integers (float sums exact in any order): bit for bit against the sequential scan."""
     cls = cls_of(tname)
     rng = np.random.default_rng(59)
     per = 256 * (16 // np.dtype(dt).itemsize)
-    for shape in [(33, per), (7, 3 * per), (5, 2 * per), (6, 4 * per), (5, 8 * per), (3, 16 * per), (4, 6, 2 * per), (3, 24 * per)]:
+    vec = 16 // np.dtype(dt).itemsize
+    for shape in [(33, per), (7, 3 * per), (5, 2 * per), (6, 4 * per), (5, 8 * per), (3, 16 * per), (4, 6, 2 * per), (3, 24 * per),
+                  (33, per - vec), (7, 3 * per + 5 * vec), (5, 8 * per + vec), (9, 65 * vec), (4, 6, 2 * per - 3 * vec), (3, 13 * per + 77 * vec),
+                  (40, 250 * vec), (11, 5 * per - vec)]:
         h = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
             h[..., ::3] = 0
