@@ -256,10 +256,18 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
             uint64_t fits = N / 32;
             uint64_t s = want < fits ? want : fits;
             if (s > 1024) s = 1024;
-            // up to 16 ways inside the block (combined through LDS, no second launch); what is still
-            // missing across blocks, with a second launch over that many fewer partial results
+            // Up to 16 ways inside the block (combined through LDS, no second launch). Beyond that a
+            // second launch over the partial results is needed anyway, and then the block stays wider
+            // (four ways inside, 64 vectors of every row it reads) and the rest is cut across blocks:
+            // 16 ways inside leave a block 16 vectors of a row, 256 bytes at a time (column sums of
+            // a 4096 x 4096 DFloat: 30.4 us that way, 27.2 us this way; of a 4096 x 4095 one, which
+            // the general kernels take: 41 -> 29 us).
             int bits = 0;
-            while (bits < 4 && (2ull << bits) <= s) ++bits;
+            if (s > 16) {
+                bits = 2;
+            } else {
+                while (bits < 4 && (2ull << bits) <= s) ++bits;
+            }
             plan->local_split_bits = bits;
             s = (s + (1ull << bits) - 1) >> bits;
             if (s >= 2) plan->n_split = (int)s;

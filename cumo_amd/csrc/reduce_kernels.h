@@ -620,6 +620,46 @@ static bool red_poll_enabled() {
     return on;
 }
 
+// Second pass of a reduction whose axis was cut across blocks: folds partial[out_total][n_split]
+// (accumulators in axis order) into the results. kp: the first pass's parameters.
+template <class Impl>
+static void red_fold_partials(const ReducePlan& plan, const RedKParams& kp, typename Impl::Acc* partial, Impl impl, hipStream_t stream) {
+    typedef typename Impl::In In;
+    typedef typename Impl::Acc Acc;
+    const uint64_t n_partial = plan.out_total * kp.n_split;
+    RedKParams k2 = kp;
+    k2.lsplit_bits = 0;
+    k2.in = reinterpret_cast<char*>(partial);
+    k2.red_ndim = 1;
+    k2.red_shape[0] = kp.n_split;
+    k2.in_red_step[0] = (int64_t)sizeof(Acc);
+    k2.red_total = kp.n_split;
+    k2.n_split = 1;
+    k2.chunk = kp.n_split;
+    int64_t s = (int64_t)sizeof(Acc) * (int64_t)kp.n_split;
+    for (int d = plan.out_ndim - 1; d >= 0; --d) {
+        k2.in_out_step[d] = s;
+        s *= (int64_t)plan.out_shape[d];
+    }
+    k2.small = (n_partial < 0xffffffffull && plan.out_total < 0xffffffffull && !force_wide_indices()) ? 1 : 0;
+    int tpr = 1;
+    while (tpr < 64 && (uint64_t)tpr * 4 < kp.n_split) tpr <<= 1;
+    if (kp.n_split > 1024) tpr = 256;
+    k2.tpr_bits = 0;
+    while ((1 << k2.tpr_bits) < tpr) ++k2.tpr_bits;
+    if constexpr (has_exact<Impl>::value) {
+        // the partials are plain values in axis order: fold them with the exact rule
+        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
+        k2.index_mode = 1;
+        red_launch_row<typename Impl::Exact, false, true>(k2, 1, impl.exact(), nullptr, stream);
+    } else {
+        CombineImpl<Impl> cimpl;
+        cimpl.impl = impl;
+        red_launch_row<CombineImpl<Impl>, false, true>(k2, 1, cimpl, nullptr, stream);
+    }
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
 // The lean kernels of reduce_stream.h for the layouts they take. Returns 1 when the
 // reduction has been launched, 0 when the general kernels must take it, -1 when the
 // caller's fixed scratch is too small (nothing launched).
@@ -667,11 +707,39 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     const dim3 b(kRedBlock);
 
     if (plan.kind == RED_COL) {
-        if (plan.n_split > 1) return 0;
         if (plan.in_out_step[plan.out_ndim - 1] != (int64_t)sizeof(In)) return 0;
         p.lsplit_bits = (uint32_t)plan.local_split_bits;
         const uint64_t per_block = (uint64_t)kRedBlock >> p.lsplit_bits;
         uint64_t grid = (plan.out_total / V + per_block - 1) / per_block;
+        if (plan.n_split > 1) {
+            // The axis is cut across blocks as well: accumulators to scratch, a second launch folds them.
+            if (p.lsplit_bits == 0 || grid > 65535) return 0;
+            const uint64_t bchunk = (plan.red_total + (uint64_t)plan.n_split - 1) / (uint64_t)plan.n_split;
+            const uint64_t n_split = (plan.red_total + bchunk - 1) / bchunk;  // no part is empty
+            if (n_split < 2 || n_split > 65535) return 0;
+            p.n_split = (uint32_t)n_split;
+            const uint64_t scratch_bytes = sizeof(Acc) * plan.out_total * n_split;
+            if (fixed) {
+                if (scratch_bytes > fixed->bytes) return -1;
+                p.partial = fixed->ptr;
+            } else {
+                p.partial = cumo_cuda_runtime_malloc(scratch_bytes);
+                if (!p.partial) return 1;  // the pool has reported it
+            }
+            const dim3 g2((unsigned)grid, (unsigned)n_split);
+            if (nt) hipLaunchKernelGGL((red_scol_kernel<Impl, V, true, true, 4, true>), g2, b, 0, stream, p, impl);
+            else hipLaunchKernelGGL((red_scol_kernel<Impl, V, false, true, 4, true>), g2, b, 0, stream, p, impl);
+            cumo_cuda_runtime_check_kernel_launch();
+            RedKParams kp;
+            red_fill_params(&kp, plan, arg, out2, index_mode);
+            kp.tpr_bits = 0;
+            kp.lsplit_bits = 0;
+            kp.n_split = n_split;
+            kp.chunk = bchunk;
+            red_fold_partials<Impl>(plan, kp, reinterpret_cast<Acc*>(p.partial), impl, stream);
+            if (!fixed) cumo_cuda_runtime_free(p.partial);
+            return 1;
+        }
         if (grid > red_grid_cap()) grid = red_grid_cap();
         const dim3 g((unsigned)grid);
         // four positions of the axis in flight per lane: more of them (or narrower blocks) read
@@ -827,38 +895,7 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     else red_launch_row<Impl, true>(kp, plan.vec, impl, partial, stream);
     cumo_cuda_runtime_check_kernel_launch();
 
-    // second pass over partial[out_total][n_split]
-    RedKParams k2 = kp;
-    k2.lsplit_bits = 0;
-    k2.in = reinterpret_cast<char*>(partial);
-    k2.red_ndim = 1;
-    k2.red_shape[0] = kp.n_split;
-    k2.in_red_step[0] = (int64_t)sizeof(Acc);
-    k2.red_total = kp.n_split;
-    k2.n_split = 1;
-    k2.chunk = kp.n_split;
-    int64_t s = (int64_t)sizeof(Acc) * (int64_t)kp.n_split;
-    for (int d = plan.out_ndim - 1; d >= 0; --d) {
-        k2.in_out_step[d] = s;
-        s *= (int64_t)plan.out_shape[d];
-    }
-    k2.small = (n_partial < 0xffffffffull && plan.out_total < 0xffffffffull && !force_wide_indices()) ? 1 : 0;
-    int tpr = 1;
-    while (tpr < 64 && (uint64_t)tpr * 4 < kp.n_split) tpr <<= 1;
-    if (kp.n_split > 1024) tpr = 256;
-    k2.tpr_bits = 0;
-    while ((1 << k2.tpr_bits) < tpr) ++k2.tpr_bits;
-    if constexpr (has_exact<Impl>::value) {
-        // the partials are plain values in axis order: fold them with the exact rule
-        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
-        k2.index_mode = 1;
-        red_launch_row<typename Impl::Exact, false, true>(k2, 1, impl.exact(), nullptr, stream);
-    } else {
-        CombineImpl<Impl> cimpl;
-        cimpl.impl = impl;
-        red_launch_row<CombineImpl<Impl>, false, true>(k2, 1, cimpl, nullptr, stream);
-    }
-    cumo_cuda_runtime_check_kernel_launch();
+    red_fold_partials<Impl>(plan, kp, partial, impl, stream);
     if (!fixed) cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));
     return true;
 }

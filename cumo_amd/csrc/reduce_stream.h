@@ -451,7 +451,10 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
 // Column form. n_out is a multiple of VEC and so is out_inner.
 // U: positions of the axis a lane has in flight (more when the outputs alone give too few lanes
 // to keep the memory system busy: a block still reads 4 KiB runs of every row it touches).
-template <class Impl, int VEC, bool NT, bool LOCAL, int U>
+// PARTIAL: the axis is also cut across blocks, p.n_split ways (blockIdx.y says which part this
+// block has); a block leaves its accumulators in p.partial[output * n_split + part] and a second
+// launch folds them. Blocks stay 128 or 256 vectors wide that way however few the outputs are.
+template <class Impl, int VEC, bool NT, bool LOCAL, int U, bool PARTIAL = false>
 __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl impl) {
     typedef typename Impl::In In;
     typedef typename Impl::Acc Acc;
@@ -464,11 +467,20 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
     const unsigned s = threadIdx.x >> cbits;
     const uint32_t groups = p.n_out / VEC;
     const uint32_t n_cb = (groups + CPB - 1) / CPB;
-    const uint64_t lchunk = (p.n + SB - 1) / SB;
-    uint64_t begin = (uint64_t)s * lchunk;
-    if (begin > p.n) begin = p.n;
+    // this block's stretch of the axis, then this lane's part of it
+    uint64_t b0 = 0, b1 = p.n;
+    if (PARTIAL) {
+        const uint64_t bchunk = (p.n + p.n_split - 1) / p.n_split;
+        b0 = (uint64_t)blockIdx.y * bchunk;
+        if (b0 > p.n) b0 = p.n;
+        b1 = b0 + bchunk;
+        if (b1 > p.n) b1 = p.n;
+    }
+    const uint64_t lchunk = (b1 - b0 + SB - 1) / SB;
+    uint64_t begin = b0 + (uint64_t)s * lchunk;
+    if (begin > b1) begin = b1;
     uint64_t end = begin + lchunk;
-    if (end > p.n) end = p.n;
+    if (end > b1) end = b1;
 
     for (uint32_t cb = blockIdx.x; cb < n_cb; cb += gridDim.x) {
         const uint32_t g = cb * CPB + c;
@@ -550,6 +562,14 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
                 }
             }
             __syncthreads();
+        }
+        if (PARTIAL) {
+            if (ok && s == 0) {
+                Acc* partial = reinterpret_cast<Acc*>(p.partial);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) partial[(size_t)(i_out0 + j) * p.n_split + blockIdx.y] = acc[j];
+            }
+            continue;
         }
         if (ok && s == 0) {
 #pragma unroll
