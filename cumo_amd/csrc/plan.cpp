@@ -172,7 +172,7 @@ static int ceil_pow2(uint64_t x) {
 }
 
 void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, int in_elmsz, int accum_bytes,
-                 ReducePlan* plan) {
+                 ReducePlan* plan, bool allow_tail) {
     std::memset(plan, 0, sizeof(*plan));
     plan->vec = 1;
     plan->n_split = 1;
@@ -280,13 +280,16 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
     int vec = 16 / in_elmsz;
     for (; vec > 1; vec >>= 1) {
         const int align = in_elmsz >= 4 ? in_elmsz : vec * in_elmsz;  // read-only: the element's alignment is enough
-        bool ok = nr > 0 && plan->in_red_step[nr - 1] == in_elmsz && (plan->red_shape[nr - 1] % vec) == 0 &&
-                  ((uintptr_t)arg->in.ptr % align) == 0;
+        // (a single long axis may end in part of a vector where the caller folds that part by itself)
+        const bool whole = nr > 0 && ((plan->red_shape[nr - 1] % vec) == 0 ||
+                                      (allow_tail && nr == 1 && plan->red_shape[0] >= (uint64_t)vec * 256));
+        bool ok = nr > 0 && plan->in_red_step[nr - 1] == in_elmsz && whole && ((uintptr_t)arg->in.ptr % align) == 0;
         for (int d = 0; d < nr - 1 && ok; ++d) ok = (plan->in_red_step[d] % align) == 0;
         for (int d = 0; d < no && ok; ++d) ok = (plan->in_out_step[d] % align) == 0;
         if (ok) break;
     }
     plan->vec = vec < 1 ? 1 : vec;
+    plan->red_tail = (plan->vec > 1 && nr == 1) ? (int)(plan->red_shape[0] % (uint64_t)plan->vec) : 0;
 
     // lanes per output: enough that each lane still has a few accesses to overlap
     uint64_t per_lane = (uint64_t)plan->vec * 4;

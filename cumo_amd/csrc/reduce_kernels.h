@@ -756,6 +756,8 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     }
 
     if (plan.in_red_step[0] != (int64_t)sizeof(In)) return 0;
+    p.tail = (uint32_t)plan.red_tail;
+    p.n = plan.red_total - p.tail;
     p.tpr_bits = 0;
     while ((1 << p.tpr_bits) < plan.threads_per_row) ++p.tpr_bits;
     {
@@ -852,13 +854,16 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     typedef typename Impl::Acc Acc;
     if (arg->out_indexer.total_size == 0) return true;  // reference: reduce_kernel.h:444-446
     ReducePlan plan;
-    plan_reduce(arg, out2, (int)sizeof(In), (int)sizeof(Acc), &plan);
+    // the lean row kernels fold what a run has past its last whole vector by themselves
+    plan_reduce(arg, out2, (int)sizeof(In), (int)sizeof(Acc), &plan, true);
     if (plan.kind == RED_EMPTY) return true;
     hipStream_t stream = current_stream();
     {
         const int taken = red_stream_launch(plan, arg, out2, impl, index_mode, fixed, stream);
         if (taken != 0) return taken > 0;
     }
+    // the general kernels want whole vectors
+    if (plan.red_tail != 0) plan_reduce(arg, out2, (int)sizeof(In), (int)sizeof(Acc), &plan, false);
     RedKParams kp;
     red_fill_params(&kp, plan, arg, out2, index_mode);
     kp.tpr_bits = 0;

@@ -33,7 +33,8 @@ struct RedSParams {
     const char* in;
     char* out;
     char* out2;
-    uint64_t n;            // length of the reduce axis in elements
+    uint64_t n;            // length of the reduce axis in elements (row form: of its whole vectors)
+    uint32_t tail;         // row form: elements of the axis past its last whole vector (fewer than a vector)
     int64_t red_step;      // column form: byte step along the reduce axis
     int64_t in_step[2];    // input byte steps over the (at most two) output dimensions, outer first
     int64_t out_step[2];
@@ -78,10 +79,11 @@ __device__ __forceinline__ void rs_split_out(const RedSParams& p, uint32_t o, ui
 // The 2^tpr_bits lanes of a group fold the tiles first, first + every, first + 2 * every, ...
 // of the run [0, end) (base = its element 0); a tile is what the group loads in one step,
 // kRsUnroll vectors per lane. end is a multiple of VEC. Every lane of the group runs the
-// same number of steps.
+// same number of steps. The run may go on for `tail` more elements, fewer than a vector: the
+// group's first lane folds those one by one when the group has the run's first tile (first == 0).
 template <class Impl, int VEC, bool NT>
 __device__ __forceinline__ typename Impl::Acc rs_row_scan(const Impl& impl, const char* base, uint64_t first, uint64_t every, uint64_t end,
-                                                          unsigned lane_r, unsigned tpr_bits, int64_t idx_base) {
+                                                          uint32_t tail, unsigned lane_r, unsigned tpr_bits, int64_t idx_base) {
     typedef typename Impl::In In;
     typename Impl::Acc acc = impl.identity();
     const uint64_t stride = (uint64_t)VEC << tpr_bits;
@@ -118,6 +120,11 @@ __device__ __forceinline__ typename Impl::Acc rs_row_scan(const Impl& impl, cons
             if (i < end) impl.template accumulate_n<VEC>(x[u], idx_base + (int64_t)i, acc);
         }
     }
+    // (after the lane's other elements: a lane folds in the order of the axis, which an impl may rely on)
+    if (tail != 0 && first == 0 && lane_r == 0) {
+        const In* rest = reinterpret_cast<const In*>(base) + end;
+        for (uint32_t e = 0; e < tail; ++e) impl.accumulate(rest[e], idx_base + (int64_t)(end + e), acc);
+    }
     return acc;
 }
 
@@ -146,10 +153,10 @@ __device__ __forceinline__ void rs_group_combine(const Impl& impl, typename Impl
 // scan + combine (+ the exact second fold where the impl asks for one)
 template <class Impl, int VEC, bool NT>
 __device__ __forceinline__ typename Impl::Acc rs_row_reduce(const Impl& impl, const char* base, uint64_t first, uint64_t every, uint64_t end,
-                                                            unsigned lane_r, unsigned tpr_bits, int64_t idx_base,
+                                                            uint32_t tail, unsigned lane_r, unsigned tpr_bits, int64_t idx_base,
                                                             typename Impl::Acc* wave_slots, int* s_need) {
     typedef typename Impl::Acc Acc;
-    Acc acc = rs_row_scan<Impl, VEC, NT>(impl, base, first, every, end, lane_r, tpr_bits, idx_base);
+    Acc acc = rs_row_scan<Impl, VEC, NT>(impl, base, first, every, end, tail, lane_r, tpr_bits, idx_base);
     rs_group_combine(impl, acc, tpr_bits, wave_slots);
     if constexpr (has_exact<Impl>::value) {
         const unsigned TPR = 1u << tpr_bits;
@@ -168,7 +175,7 @@ __device__ __forceinline__ typename Impl::Acc rs_row_reduce(const Impl& impl, co
             const Exact ex = impl.exact();
             // the exact accumulator is wider: its own LDS slots
             __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
-            typename Exact::Acc e = rs_row_scan<Exact, VEC, false>(ex, base, first, every, end, lane_r, tpr_bits, 0);
+            typename Exact::Acc e = rs_row_scan<Exact, VEC, false>(ex, base, first, every, end, tail, lane_r, tpr_bits, 0);
             rs_group_combine(ex, e, tpr_bits, exact_slots);
             acc = impl.from_exact(e);
         }
@@ -194,7 +201,7 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_kernel(RedSParams p, Impl 
         rs_split_out(p, ok ? row : p.n_out - 1, o0, o1);
         const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
         const int64_t idx_base = p.index_mode == 2 ? in_off / (int64_t)sizeof(In) : 0;
-        const Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, 0, 1, p.n, lane_r, p.tpr_bits, idx_base, wave_slots, &s_need);
+        const Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, 0, 1, p.n, p.tail, lane_r, p.tpr_bits, idx_base, wave_slots, &s_need);
         if (ok && lane_r == 0) {
             const int64_t a = (int64_t)o0 * p.out_step[0] + (int64_t)o1 * p.out_step[1];
             const int64_t b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)o1 * p.out2_step[1] : 0;
@@ -242,7 +249,7 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
     const int64_t idx_base = p.index_mode == 2 ? in_off / (int64_t)sizeof(In) : 0;
     // the blocks of an output take its 16 KiB tiles in turn, so that together they read one window
     // of the run at a time (memory sees a few long streams instead of n_split short ones)
-    Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, threadIdx.x, 8, idx_base, wave_slots, &s_need);
+    Acc acc = rs_row_reduce<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, p.tail, threadIdx.x, 8, idx_base, wave_slots, &s_need);
 
     if (threadIdx.x == 0) {
         // The accumulator is written through to memory and has arrived there before
@@ -311,7 +318,7 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
 // launch 0.7 us. Lane 0 returns the result.
 template <class Impl, int VEC>
 __device__ __attribute__((noinline)) typename Impl::Acc rs_exact_refold_wave(const Impl& impl, const char* base, uint64_t first, uint64_t every,
-                                                                              uint64_t end) {
+                                                                              uint64_t end, uint32_t tail) {
     typedef typename Impl::In In;
     typedef typename Impl::Exact Exact;
     const Exact ex = impl.exact();
@@ -327,6 +334,10 @@ __device__ __attribute__((noinline)) typename Impl::Acc rs_exact_refold_wave(con
             rs_load<In, VEC, false>(base + i * sizeof(In), x);
             ex.template accumulate_n<VEC>(x, (int64_t)i, e);
         }
+    }
+    if (tail != 0 && first == 0 && lane == 0) {
+        const In* rest = reinterpret_cast<const In*>(base) + end;
+        for (uint32_t k = 0; k < tail; ++k) ex.accumulate(rest[k], (int64_t)(end + k), e);
     }
     for (unsigned d = 32; d > 0; d >>= 1) {
         const typename Exact::Acc other = shfl_down_any(e, d);
@@ -395,13 +406,13 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
         rs_split_out(p, i_out, o0, o1);
         const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
         const int64_t idx_base = p.index_mode == 2 ? in_off / (int64_t)sizeof(In) : 0;
-        Acc acc = rs_row_scan<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, threadIdx.x, 8, idx_base);
+        Acc acc = rs_row_scan<Impl, VEC, NT>(impl, p.in + in_off, i_split, p.n_split, p.n, p.tail, threadIdx.x, 8, idx_base);
         rs_group_combine(impl, acc, 8, wave_slots);
         if constexpr (has_exact<Impl>::value) {
             // thread 0 holds the block's result; its wave alone repeats the fold where that is needed
             if (threadIdx.x >= 64) return;
             const int mine = impl.needs_exact(acc) ? 1 : 0;
-            if (__shfl(mine, 0) != 0) acc = rs_exact_refold_wave<Impl, VEC>(impl, p.in + in_off, i_split, p.n_split, p.n);
+            if (__shfl(mine, 0) != 0) acc = rs_exact_refold_wave<Impl, VEC>(impl, p.in + in_off, i_split, p.n_split, p.n, p.tail);
         }
         if (threadIdx.x == 0) {
             union U {

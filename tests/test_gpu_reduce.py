@@ -287,6 +287,61 @@ def test_few_outputs_across_memory_share_the_axis_inside_a_block(tname, dt, shap
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("shape,axis", [((7, 1027), 1), ((1, 4099), 1), ((2051,), None), ((3, 5, 1030), 2), ((300001,), None), ((40, 20011), 1)])
+def test_runs_that_end_in_part_of_a_vector(tname, dt, shape, axis):
+    """A contiguous reduce axis of 256 vectors or more that is not a whole number of vectors: the
+    lean row kernels take its whole vectors and one lane folds the last one to three elements.
+    What decides the answer is put into those last elements: the extreme, a tie with an earlier
+    element (the earlier index wins), the zero of the other sign (the one that came first wins),
+    a NaN (skipped, or winning with nan: true), a large addend; the ordinary case beside them."""
+    import cumo_amd
+    rng = np.random.default_rng(91)
+    cls = cls_of(tname)
+    n = shape[-1]
+    base = (rng.integers(-8, 8, size=shape) / 4.0).astype(dt)
+    cases = {"plain": base}
+    h = base.copy(); h[..., -1] = 50.0; h[..., -2] = -50.0
+    cases["extremes at the end"] = h
+    h = base.copy(); h[..., 5] = 9.0; h[..., -1] = 9.0; h[..., 7] = -9.0; h[..., -1 - (n % 2)] = -9.0 if n % 2 else h[..., -1]
+    cases["ties with the end"] = h
+    h = np.abs(base) + 1.0; h[..., 3] = -0.0; h[..., -1] = 0.0
+    cases["zeros: minus first, plus in the last element"] = h
+    h = -np.abs(base) - 1.0; h[..., -1] = -0.0; h[..., 11] = 0.0
+    cases["zeros: plus first, minus in the last element"] = h
+    h = base.copy(); h[..., -1] = np.nan
+    cases["NaN in the last element"] = h
+    h = base.copy(); h[..., -1] = 2.0 ** 20
+    cases["a large last addend"] = h
+    for what, h in cases.items():
+        d = cls.cast(h)
+        has_nan = bool(np.isnan(h).any())
+        for name in ("min", "max", "argmin", "argmax", "sum", "ptp"):
+            for nan in ((False, True) if has_nan and name != "ptp" else (False,)):
+                kw = {"nan": True} if nan else {}
+                got = getattr(d, name)(axis=axis, **kw).to_numpy()
+                want = oracle.reduce(name, h, axis=axis, **kw)
+                assert_bits_equal(got, want, "%s: %s nan=%s" % (what, name, nan))
+        lo, hi = d.minmax(axis=axis)
+        assert_bits_equal(lo.to_numpy(), oracle.reduce("min", h, axis=axis), what)
+        assert_bits_equal(hi.to_numpy(), oracle.reduce("max", h, axis=axis), what)
+        if not has_nan:
+            # against the value in extended precision (a float32 oracle that adds 300001 squares in turn is
+            # itself further from it than the bar)
+            for name in ("mean", "var", "stddev", "rms"):
+                want = exact_reduce(name, h, axis)
+                scale = abs_sum(h, axis) / n if name == "mean" else np.abs(want) + 1e-30
+                assert_reduction_close(getattr(d, name)(axis=axis).to_numpy(), want.astype(dt), n, scale, "%s: %s" % (what, name))
+            hp = np.where(rng.random(shape) < 0.01, 2.0, 1.0).astype(dt) * np.where(rng.random(shape) < 0.5, 1.0, -1.0).astype(dt)
+            hp[..., -1] = -2.0
+            assert_bits_equal(cls.cast(hp).prod(axis=axis).to_numpy(), np.asarray(oracle.reduce("prod", hp, axis=axis)), what + ": prod")
+    hi32 = rng.integers(-1000, 1000, size=shape).astype(np.int32)
+    hi32[..., -1] = 5000
+    di = cumo_amd.Int32.cast(hi32)
+    for name in ("sum", "min", "max", "argmax", "argmin"):
+        assert (getattr(di, name)(axis=axis).to_numpy() == oracle.reduce(name, hi32, axis=axis)).all(), name
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 def test_reductions_of_slices_that_start_off_a_16_byte_boundary(tname, dt):
     """Inner slices beginning at an odd column, with lengths that are whole 128-bit accesses: the
     kernels read them with wide loads on element boundaries; along the rows, down the columns, all."""
