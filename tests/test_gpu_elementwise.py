@@ -86,6 +86,43 @@ def test_broadcast_shapes(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+def test_matrices_with_rows_of_an_odd_length_and_a_second_operand(tname, dt):
+    """A contiguous matrix whose rows are not a whole number of 128-bit vectors (op) a row vector, a
+    column vector or a strided view of its own shape, on either side: the matrix and the result go
+    as one run each, the other operand is addressed by row and column. Totals that end in part of
+    a vector; a row shorter than two vectors from the end (vectors that straddle two rows)."""
+    import cumo_amd
+    rng = np.random.default_rng(303)
+    cls = cls_of(tname)
+    for (R, Cn) in [(37, 65), (130, 4095), (5, 1001), (64, 67), (3, 70001), (1025, 129)]:
+        a = rng.standard_normal((R, Cn)).astype(dt)
+        da = cls.cast(a)
+        wide = rng.standard_normal((R, 2 * Cn)).astype(dt)
+        for what, b, db in [("row", None, None), ("column", None, None), ("view", None, None)]:
+            if what == "row":
+                b = rng.standard_normal((1, Cn)).astype(dt); db = cls.cast(b)
+            elif what == "column":
+                b = rng.standard_normal((R, 1)).astype(dt); db = cls.cast(b)
+            else:
+                b = np.ascontiguousarray(wide[:, ::2]); db = cls.cast(wide)[:, ::2]
+            for name, f in (("add", lambda x, y: x + y), ("sub", lambda x, y: x - y), ("mul", lambda x, y: x * y), ("div", lambda x, y: x / y)):
+                assert_bits_equal(f(da, db).to_numpy(), oracle.binary(name, a, b), "%s: matrix %s %s" % ((R, Cn), name, what))
+                assert_bits_equal(f(db, da).to_numpy(), oracle.binary(name, b, a), "%s: %s %s matrix" % ((R, Cn), what, name))
+    # Int32: wrapping arithmetic, and a division that meets a zero raises as everywhere else
+    hi = rng.integers(-2 ** 31, 2 ** 31 - 1, size=(33, 131)).astype(np.int32)
+    hr = rng.integers(-1000, 1000, size=(1, 131)).astype(np.int32)
+    di, dr = cumo_amd.Int32.cast(hi), cumo_amd.Int32.cast(hr)
+    assert ((di + dr).to_numpy() == oracle.binary("add", hi, hr)).all()
+    assert ((dr * di).to_numpy() == oracle.binary("mul", hr, hi)).all()
+    hz = hr.copy()
+    hz[hz == 0] = 7
+    assert ((di / cumo_amd.Int32.cast(hz)).to_numpy() == oracle.binary("div", hi, hz)).all()
+    hz[0, 100] = 0
+    with pytest.raises(ZeroDivisionError):
+        (di / cumo_amd.Int32.cast(hz)).to_numpy()
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 def test_three_dimensions_with_an_operand_repeating_along_one(tname, dt):
     """[B,T,C] with [T,1], [B,1,C], [1,T,C], [B,1,1] and a column on both sides: the shapes whose two
     outer dimensions do not merge; C a whole number of 128-bit vectors and not; outer views."""
