@@ -102,7 +102,7 @@ struct FusedRowsParams {
 };
 
 // MODE 0 softmax, 1 layernorm. TPR lanes share a row, each holding NV vectors of V
-// elements (TPR * NV * V >= n). Rows and vectors beyond the data are masked.
+// elements (TPR * NV * V >= n). Rows, vectors and the elements of a row's last vector beyond the data are masked.
 // NT: non-temporal accesses, for arrays larger than the last-level cache.
 template <class T, int MODE, int TPR, int NV, bool NT>
 __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p) {
@@ -119,15 +119,38 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
         const char* src = p.in + (int64_t)(row_ok ? row : 0) * p.in_row_step;
         char* dst = p.out + (int64_t)(row_ok ? row : 0) * p.out_row_step;
         Vec x[NV];
-        bool have[NV];
+        int cnt[NV];  // how many elements of the vector exist: V, none, or (the row's last vector) fewer
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint64_t col = ((uint64_t)k * TPR + lane_r) * V;
-            have[k] = row_ok && col < p.n;  // n is a whole number of vectors
-            // a lane without data re-reads the row's first vector: no branch between the loads
-            const u4* ld = reinterpret_cast<const u4*>(src + (have[k] ? col : 0) * sizeof(T));
+            const int64_t left = (int64_t)p.n - (int64_t)col;
+            cnt[k] = row_ok ? (left >= V ? V : (left > 0 ? (int)left : 0)) : 0;
+            // a lane without a whole vector re-reads the row's first one: no branch between the loads
+            const u4* ld = reinterpret_cast<const u4*>(src + (cnt[k] == V ? col : 0) * sizeof(T));
             x[k].q = NT ? __builtin_nontemporal_load(ld) : *ld;
         }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            if (cnt[k] > 0 && cnt[k] < V) {
+                // part of a vector at the row's end: element by element, nothing read past the row
+                const uint64_t col = ((uint64_t)k * TPR + lane_r) * V;
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    if (j < cnt[k]) x[k].t[j] = reinterpret_cast<const T*>(src)[col + j];
+            }
+        }
+        auto put = [&](int k) {
+            const uint64_t col = ((uint64_t)k * TPR + lane_r) * V;
+            if (cnt[k] == V) {
+                u4* st = reinterpret_cast<u4*>(dst + col * sizeof(T));
+                if (NT) __builtin_nontemporal_store(x[k].q, st);
+                else *st = x[k].q;
+            } else {
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    if (j < cnt[k]) reinterpret_cast<T*>(dst)[col + j] = x[k].t[j];
+            }
+        };
         if constexpr (MODE == 0) {
             // Lanes without data hold -inf: neutral in the max, and exp(-inf - m) adds 0 to the sum.
             // The max keeps the larger non-NaN value per element and notes NaN apart (one maximum and
@@ -138,7 +161,7 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
             for (int k = 0; k < NV; ++k) {
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
-                    const T v = have[k] ? x[k].t[j] : (T)-INFINITY;
+                    const T v = j < cnt[k] ? x[k].t[j] : (T)-INFINITY;
                     x[k].t[j] = v;
                     any_nan |= (v != v);
                     m = fr_fmax(m, v);
@@ -160,13 +183,10 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
             const FrDivisor<T> by_s(s);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                if (have[k]) {
+                if (cnt[k] > 0) {
 #pragma unroll
                     for (int j = 0; j < V; ++j) x[k].t[j] = by_s.divide(x[k].t[j]);
-                    const uint64_t col = ((uint64_t)k * TPR + lane_r) * V;
-                    u4* st = reinterpret_cast<u4*>(dst + col * sizeof(T));
-                    if (NT) __builtin_nontemporal_store(x[k].q, st);
-                    else *st = x[k].q;
+                    put(k);
                 }
             }
         } else {
@@ -174,10 +194,9 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
             T s = 0;
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                if (have[k]) {
 #pragma unroll
-                    for (int j = 0; j < V; ++j) s += x[k].t[j];
-                }
+                for (int j = 0; j < V; ++j)
+                    if (j < cnt[k]) s += x[k].t[j];
             }
             s = fr_allreduce<T, TPR>(s, [](T a, T b) { return a + b; });
             const T mean = s / (T)p.n;
@@ -188,7 +207,7 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
                 for (int j = 0; j < V; ++j) {
                     const T c = x[k].t[j] - mean;
                     x[k].t[j] = c;
-                    if (have[k]) q += c * c;
+                    if (j < cnt[k]) q += c * c;
                 }
             }
             q = fr_allreduce<T, TPR>(q, [](T a, T b) { return a + b; });
@@ -196,13 +215,10 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
             const T sd = fr_sqrt<T>(var + (T)p.eps);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                if (have[k]) {
+                if (cnt[k] > 0) {
 #pragma unroll
                     for (int j = 0; j < V; ++j) x[k].t[j] = x[k].t[j] / sd;
-                    const uint64_t col = ((uint64_t)k * TPR + lane_r) * V;
-                    u4* st = reinterpret_cast<u4*>(dst + col * sizeof(T));
-                    if (NT) __builtin_nontemporal_store(x[k].q, st);
-                    else *st = x[k].q;
+                    put(k);
                 }
             }
         }
@@ -226,7 +242,7 @@ void fr_launch_one(const FusedRowsParams& p, hipStream_t stream) {
 template <class T, int MODE>
 bool fr_launch(const FusedRowsParams& p, hipStream_t stream) {
     constexpr int V = 16 / (int)sizeof(T);
-    const uint64_t nv = p.n / V;  // vectors per row
+    const uint64_t nv = (p.n + V - 1) / V;  // vectors per row, the last one maybe partly there
     if (nv <= 8) fr_launch_one<T, MODE, 8, 1>(p, stream);
     else if (nv <= 16) fr_launch_one<T, MODE, 8, 2>(p, stream);
     else if (nv <= 32) fr_launch_one<T, MODE, 8, 4>(p, stream);
@@ -247,16 +263,18 @@ bool fr_launch(const FusedRowsParams& p, hipStream_t stream) {
 using namespace cumo_hip;
 
 // type: 0 SFloat, 1 DFloat. mode: 0 softmax, 1 layernorm. Returns 1 when the launch
-// was made, 0 when the shape is outside what the kernels take (rows that are not a
-// whole number of 128-bit vectors, not 16-byte aligned, or too long): the caller
+// was made, 0 when the shape is outside what the kernels take (rows shorter than one
+// 128-bit vector, not aligned as their elements are, or too long): the caller
 // composes the operations instead.
 extern "C" int cumo_hip_fused_rows_kernel_launch(int type, int mode, const cumo_hip_fused_rows_t* d) {
     if (!d || d->rows == 0 || d->n == 0) return 1;
     const int es = type == 0 ? 4 : 8;
     const uint64_t v = 16 / es;
     if (type < 0 || type > 1 || mode < 0 || mode > 1) return 0;
-    if (d->n % v) return 0;
-    if (((uintptr_t)d->in % 16) || ((uintptr_t)d->out % 16) || (d->in_row_step % 16) || (d->out_row_step % 16)) return 0;
+    // rows need their element's alignment only (128-bit accesses work on any 4-byte boundary) and may end in
+    // part of a vector, which goes element by element
+    if (d->n < v) return 0;
+    if (((uintptr_t)d->in % es) || ((uintptr_t)d->out % es) || (d->in_row_step % es) || (d->out_row_step % es)) return 0;
     FusedRowsParams p;
     p.rows = d->rows;
     p.n = d->n;

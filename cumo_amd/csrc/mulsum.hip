@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_elementwise_kernel(const char
 
 
 // One product sum per row, many rows in one launch: LPR lanes share a row whose two
-// runs are contiguous and 16-byte aligned, four vectors per operand in flight per
+// runs are contiguous (aligned as their elements are), four vectors per operand in flight per
 // lane, four accumulators, then a butterfly over the lanes of the row (and the four
 // waves through LDS when a block shares the row). The order is fixed by the layout.
 struct MulsumRows {
@@ -235,6 +235,12 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_rows_kernel(MulsumRows g) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) ms_fold<T, NANF>(a.t[j], b.t[j], acc[0]);
         }
+        // what the row has past its last whole vector (fewer than VEC elements)
+        if (lane == 0) {
+            const T* a1 = reinterpret_cast<const T*>(a4);
+            const T* b1 = reinterpret_cast<const T*>(b4);
+            for (uint64_t e = nvec * VEC; e < g.n; ++e) ms_fold<T, NANF>(a1[e], b1[e], acc[1]);
+        }
         T tot = ms_add(ms_add(acc[0], acc[1]), ms_add(acc[2], acc[3]));
         if constexpr (LPR <= 64) {
 #pragma unroll
@@ -253,8 +259,10 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_rows_kernel(MulsumRows g) {
 template <class T, bool NANF>
 bool mulsum_rows_launch(const cumo_hip_mulsum_rows_t* d) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    if (d->n % VEC) return false;
-    if (((uintptr_t)d->p1 | (uintptr_t)d->p2 | (uintptr_t)d->row_step1 | (uintptr_t)d->row_step2) & 15) return false;
+    // rows need their element's alignment only (a 128-bit load works on any 4-byte boundary) and may end in
+    // part of a vector, which the row's first lane folds element by element
+    if (d->n < (uint64_t)VEC * 16) return false;
+    if (((uintptr_t)d->p1 | (uintptr_t)d->p2 | (uintptr_t)d->row_step1 | (uintptr_t)d->row_step2) % sizeof(T)) return false;
     if (((uintptr_t)d->out | (uintptr_t)d->out_step) % sizeof(T)) return false;
     MulsumRows g = {d->rows, d->n, (int64_t)d->row_step1, (int64_t)d->row_step2, (int64_t)d->out_step, d->p1, d->p2, d->out};
     const uint64_t nvec = d->n / VEC;

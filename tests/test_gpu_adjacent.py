@@ -424,7 +424,8 @@ def test_mulsum_parity(tname, dt):
     hx, hy = make((3000, 40)), make((3000, 40))
     check(cls.cast(hx).mulsum(cls.cast(hy), axis=1).to_numpy(), hx, hy, 1, "3000 runs")
     # every row in one launch: 16, 64 and 256 lanes per row, a repeated row operand, rows a step apart
-    for shape in ((5000, 8), (700, 512), (300, 4096), (64, 20000), (3, 1 << 16)):
+    # (and rows that end in part of a 128-bit vector, which also start off a 16-byte boundary)
+    for shape in ((5000, 8), (700, 512), (300, 4096), (64, 20000), (3, 1 << 16), (300, 4095), (700, 131), (64, 20001), (50, 67), (10, 4094)):
         hx, hy = make(shape), make(shape)
         x, y = cls.cast(hx), cls.cast(hy)
         check(x.mulsum(y, axis=1).to_numpy(), hx, hy, 1, ("rows", shape))

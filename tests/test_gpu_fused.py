@@ -45,7 +45,9 @@ def test_softmax_matches_the_chain(dt):
     import cumo_amd as m
     cls = m.SFloat if dt == np.float32 else m.DFloat
     rng = np.random.default_rng(61)
-    for shape in [(1, 4), (5, 8), (33, 64), (100, 512), (7, 1000), (3, 4, 2048), (9, 4096), (2, 16384), (4, 20000), (6, 7), (2, 3, 5, 128)]:
+    # (rows that end in part of a 128-bit vector, and so start off a 16-byte boundary: 1001, 4095, 13, 131, 7)
+    for shape in [(1, 4), (5, 8), (33, 64), (100, 512), (7, 1000), (3, 4, 2048), (9, 4096), (2, 16384), (4, 20000), (6, 7), (2, 3, 5, 128),
+                  (7, 1001), (37, 4095), (50, 13), (19, 131), (3, 16383), (5, 4094)]:
         h = (rng.standard_normal(shape) * 2).astype(dt)
         x = cls.cast(h)
         got = m.Fused.softmax(x).to_numpy()
@@ -79,7 +81,8 @@ def test_layernorm_matches_the_chain(dt):
     import cumo_amd as m
     cls = m.SFloat if dt == np.float32 else m.DFloat
     rng = np.random.default_rng(62)
-    for shape in [(3, 4), (5, 8), (33, 64), (100, 512), (7, 1000), (64, 4096), (3, 16384), (4, 20000), (6, 7), (2, 3, 128)]:
+    for shape in [(3, 4), (5, 8), (33, 64), (100, 512), (7, 1000), (64, 4096), (3, 16384), (4, 20000), (6, 7), (2, 3, 128),
+                  (7, 1001), (37, 4095), (50, 13), (19, 131), (3, 16383), (5, 4094)]:
         h = (rng.standard_normal(shape) * 3 + 1).astype(dt)
         x = cls.cast(h)
         got = m.Fused.layernorm(x, 1e-5).to_numpy()
