@@ -495,10 +495,11 @@ struct ChainShared {
     int prefix_has;
 };
 
-// RAGGED: only the first nvec vectors from `first` on exist; the others read as zeros (they lie
-// after everything that exists, so what they add to never reaches an element that is stored)
+// RAGGED: only the first nelem elements from `first` on exist; the others read as zeros (they lie
+// after everything that exists, so what they add to never reaches an element that is stored).
+// The one vector that is partly there goes element by element: nothing is read past the run.
 template <class T, bool NT, int R, bool RAGGED = false>
-__device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first, ChainVec<T> (&v)[R], uint32_t nvec = 0) {
+__device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first, ChainVec<T> (&v)[R], uint32_t nelem = 0) {
     typedef typename ChainVec<T>::u4 u4;
     constexpr int V = ChainVec<T>::V;
     const unsigned lane = threadIdx.x & 63u;
@@ -509,7 +510,15 @@ __device__ __forceinline__ void chain_issue_loads(const char* in, uint64_t first
         if (RAGGED) {
             const u4 zero = {0u, 0u, 0u, 0u};
             v[r].q = zero;
-            if ((uint32_t)(w * R * 64 + r * 64) + lane < nvec) v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
+            const uint32_t e0 = ((uint32_t)(w * R * 64 + r * 64) + lane) * V;
+            if (e0 + V <= nelem) {
+                v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
+            } else if (e0 < nelem) {
+                const T* s1 = reinterpret_cast<const T*>(src + r * 64);
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                    if (e0 + e < nelem) v[r].e[e] = s1[e];
+            }
         } else {
             v[r].q = NT ? __builtin_nontemporal_load(src + r * 64) : src[r * 64];
         }
@@ -567,7 +576,7 @@ __device__ __forceinline__ void chain_scan_tile(ChainVec<T> (&v)[R], T* s_wave_t
 
 // adds what precedes the tile (if anything) and the earlier waves' total, and stores
 template <class T, class Op, bool NT, int R, bool RAGGED = false>
-__device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, ChainVec<T> (&v)[R], T head, bool head_has, T wave_pre, uint32_t nvec = 0) {
+__device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, ChainVec<T> (&v)[R], T head, bool head_has, T wave_pre, uint32_t nelem = 0) {
     typedef typename ChainVec<T>::u4 u4;
     constexpr int V = ChainVec<T>::V;
     const unsigned lane = threadIdx.x & 63u;
@@ -583,7 +592,17 @@ __device__ __forceinline__ void chain_store_tile(char* out, uint64_t first, Chai
 #pragma unroll
             for (int e = 0; e < V; ++e) v[r].e[e] = Op::apply(head, v[r].e[e]);
         }
-        if (RAGGED && !((uint32_t)(w * R * 64 + r * 64) + lane < nvec)) continue;
+        if (RAGGED) {
+            const uint32_t e0 = ((uint32_t)(w * R * 64 + r * 64) + lane) * V;
+            if (e0 >= nelem) continue;
+            if (e0 + V > nelem) {
+                T* d1 = reinterpret_cast<T*>(dst + r * 64);
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                    if (e0 + e < nelem) d1[e] = v[r].e[e];
+                continue;
+            }
+        }
         if (NT) __builtin_nontemporal_store(v[r].q, dst + r * 64);
         else dst[r * 64] = v[r].q;
     }
@@ -608,8 +627,8 @@ __device__ __forceinline__ void chain_finish_tile(char* out, uint64_t first, uin
     chain_store_tile<T, Op, NT, R>(out, first, v, *s_prefix, sh->prefix_has != 0, wave_pre);
 }
 
-// Many runs, each contiguous on both sides, 16-byte aligned and a whole number of vectors
-// long: one block per run, chunk after chunk of R * 256 vectors in the same wave-by-wave form,
+// Many runs, each contiguous on both sides (64 vectors at least, aligned as their elements are):
+// one block per run, chunk after chunk of R * 256 vectors in the same wave-by-wave form,
 // the running value handed on in a register; the last chunk may be partly there.
 template <class T, class Op, bool NT, int R>
 __global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsParams p) {
@@ -637,11 +656,11 @@ __global__ __launch_bounds__(kScanBlock) void scan_rows_whole_kernel(ScanRowsPar
                 chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
                 chain_store_tile<T, Op, NT, R>(p.out + oo, first, v, carry, has_carry, wave_pre);
             } else {
-                // the run's last chunk, partly there (the run is a whole number of vectors)
-                const uint32_t nvec = (uint32_t)((p.n - first) / V);
-                chain_issue_loads<T, NT, R, true>(p.in + oi, first, v, nvec);
+                // the run's last chunk, partly there
+                const uint32_t nelem = (uint32_t)(p.n - first);
+                chain_issue_loads<T, NT, R, true>(p.in + oi, first, v, nelem);
                 chain_scan_tile<T, Op, R>(v, s_wave_tot, total, wave_pre);
-                chain_store_tile<T, Op, NT, R, true>(p.out + oo, first, v, carry, has_carry, wave_pre, nvec);
+                chain_store_tile<T, Op, NT, R, true>(p.out + oo, first, v, carry, has_carry, wave_pre, nelem);
             }
             carry = has_carry ? Op::apply(carry, total) : total;
             has_carry = true;
@@ -1169,13 +1188,15 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
     const char* src = p.in + oi + row0 * p.s_in + colb;
     char* dst = p.out + oo + row0 * p.s_out + colb;
     // A tile at the lower edge has fewer rows and one at the right edge fewer columns: this wave's first
-    // `rows` rows exist, and this lane's columns do or do not. What such a tile reads as missing is zeros;
+    // `rows` rows exist, and of this lane's columns the first ncol. What such a tile reads as missing is zeros;
     // the totals they enter are only ever used by rows or columns that do not exist either.
     const int64_t rows_left = (int64_t)p.n - row0;
     const int rows = rows_left >= R ? R : (rows_left > 0 ? (int)rows_left : 0);
-    const bool cols_here = (uint64_t)strip * SW + (uint64_t)l * V < p.cols;
+    const int64_t cols_left = (int64_t)p.cols - (int64_t)((uint64_t)strip * SW + (uint64_t)l * V);
+    const int ncol = cols_left >= V ? V : (cols_left > 0 ? (int)cols_left : 0);  // this lane's columns that exist
+    const bool all_there = rows == R && __builtin_amdgcn_ballot_w64(ncol != V) == 0;
     T raw[R][V];
-    if (rows == R && __builtin_amdgcn_ballot_w64(!cols_here) == 0) {
+    if (all_there) {
 #pragma unroll
         for (int r = 0; r < R; ++r) scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
     } else {
@@ -1183,7 +1204,16 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
         for (int r = 0; r < R; ++r) {
 #pragma unroll
             for (int j = 0; j < V; ++j) raw[r][j] = T();
-            if (r < rows && cols_here) scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
+            if (r < rows) {
+                if (ncol == V) {
+                    scan_cols_load<T, V, NT>(src + (int64_t)r * p.s_in, raw[r]);
+                } else {
+                    // the row's last vector, partly there: element by element, nothing read past the row
+#pragma unroll
+                    for (int j = 0; j < V; ++j)
+                        if (j < ncol) raw[r][j] = reinterpret_cast<const T*>(src + (int64_t)r * p.s_in)[j];
+                }
+            }
         }
     }
     {
@@ -1279,7 +1309,7 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
             acc[j] = o.t;
         }
     }
-    if (rows == R && __builtin_amdgcn_ballot_w64(!cols_here) == 0) {
+    if (all_there) {
         scan_cols_store<T, V, NT>(dst, acc);
 #pragma unroll
         for (int r = 1; r < R; ++r) {
@@ -1287,13 +1317,22 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
             for (int j = 0; j < V; ++j) acc[j] = Op::apply(acc[j], raw[r][j]);
             scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
         }
-    } else if (cols_here) {
-        if (rows > 0) scan_cols_store<T, V, NT>(dst, acc);
+    } else if (ncol > 0) {
+        auto put = [&](int r) {
+            if (ncol == V) {
+                scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
+            } else {
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    if (j < ncol) reinterpret_cast<T*>(dst + (int64_t)r * p.s_out)[j] = acc[j];
+            }
+        };
+        if (rows > 0) put(0);
 #pragma unroll
         for (int r = 1; r < R; ++r) {
 #pragma unroll
             for (int j = 0; j < V; ++j) acc[j] = Op::apply(acc[j], raw[r][j]);
-            if (r < rows) scan_cols_store<T, V, NT>(dst + (int64_t)r * p.s_out, acc);
+            if (r < rows) put(r);
         }
     }
 }
@@ -1350,7 +1389,12 @@ void scan_cols_launch(ScanColsParams& p, hipStream_t stream) {
     constexpr int V = 16 / (int)sizeof(T);
     bool vec = (p.cols % V) == 0 && ((uintptr_t)p.in % 16) == 0 && ((uintptr_t)p.out % 16) == 0 && (p.s_in % 16) == 0 && (p.s_out % 16) == 0;
     for (int d = 0; d < p.nouter && vec; ++d) vec = (p.ostep_in[d] % 16) == 0 && (p.ostep_out[d] % 16) == 0;
-    if (vec && scan_cols_chain_launch<T, Op>(p, stream)) return;
+    // the one-pass form needs the elements' alignment only (128-bit accesses work on any 4-byte boundary)
+    // and takes a last vector of a row that is partly there
+    bool elem = ((uintptr_t)p.in % sizeof(T)) == 0 && ((uintptr_t)p.out % sizeof(T)) == 0 && (p.s_in % (int64_t)sizeof(T)) == 0 &&
+                (p.s_out % (int64_t)sizeof(T)) == 0;
+    for (int d = 0; d < p.nouter && elem; ++d) elem = (p.ostep_in[d] % (int64_t)sizeof(T)) == 0 && (p.ostep_out[d] % (int64_t)sizeof(T)) == 0;
+    if (elem && scan_cols_chain_launch<T, Op>(p, stream)) return;
     if (vec) scan_cols_launch_vec<T, Op, V>(p, stream);
     else scan_cols_launch_vec<T, Op, 1>(p, stream);
 }
@@ -1372,9 +1416,10 @@ void scan_rows_launch(const ScanRowsParams& p, hipStream_t stream) {
     uint64_t grid = p.rows;
     if (grid > 65536) grid = 65536;
     constexpr uint64_t V = 16 / sizeof(T);
-    bool whole = p.s_in == (int64_t)sizeof(T) && p.s_out == (int64_t)sizeof(T) && p.n % V == 0 && p.n >= 64 * V &&
-                 (((uintptr_t)p.in | (uintptr_t)p.out) & 15) == 0;
-    for (int d = 0; d < p.nouter && whole; ++d) whole = (p.ostep_in[d] % 16) == 0 && (p.ostep_out[d] % 16) == 0;
+    // (runs need their element's alignment only: 128-bit accesses work on any 4-byte boundary)
+    bool whole = p.s_in == (int64_t)sizeof(T) && p.s_out == (int64_t)sizeof(T) && p.n >= 64 * V &&
+                 (((uintptr_t)p.in | (uintptr_t)p.out) % sizeof(T)) == 0;
+    for (int d = 0; d < p.nouter && whole; ++d) whole = (p.ostep_in[d] % (int64_t)sizeof(T)) == 0 && (p.ostep_out[d] % (int64_t)sizeof(T)) == 0;
     if (whole) {
         const uint64_t vec_rows = (p.n + kScanBlock * V - 1) / (kScanBlock * V);  // rows of 256 vectors in a run, the last one maybe partly there
         const bool nt = stream_past_caches(2 * p.rows * p.n * sizeof(T));

@@ -232,7 +232,8 @@ def test_cum_along_contiguous_runs_of_whole_chunks(tname, dt):
     vec = 16 // np.dtype(dt).itemsize
     for shape in [(33, per), (7, 3 * per), (5, 2 * per), (6, 4 * per), (5, 8 * per), (3, 16 * per), (4, 6, 2 * per), (3, 24 * per),
                   (33, per - vec), (7, 3 * per + 5 * vec), (5, 8 * per + vec), (9, 65 * vec), (4, 6, 2 * per - 3 * vec), (3, 13 * per + 77 * vec),
-                  (40, 250 * vec), (11, 5 * per - vec)]:
+                  (40, 250 * vec), (11, 5 * per - vec), (33, per + 1), (7, 3 * per - 1), (5, 8 * per + vec + 1), (9, 65 * vec + 2 % vec + 1),
+                  (4, 6, 2 * per - 3), (20, 4095), (6, 1001)]:
         h = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
             h[..., ::3] = 0
@@ -343,7 +344,8 @@ def test_long_columns_in_one_pass(tname, dt):
     sw = 64 * (16 // np.dtype(dt).itemsize)
     vec = 16 // np.dtype(dt).itemsize
     for shape, ax in [((256 * 70, 4 * sw), 0), ((4, 256 * 35, 2 * sw), 1), ((256 * 8, 32 * sw), 0), ((256 * 9, 2 * sw), 0), ((512, 8 * sw), 0),
-                      ((256 * 3 + 77, 6 * sw + 3 * vec), 0), ((3, 1000, 2 * sw + vec), 1), ((257, 16 * sw), 0)]:
+                      ((256 * 3 + 77, 6 * sw + 3 * vec), 0), ((3, 1000, 2 * sw + vec), 1), ((257, 16 * sw), 0),
+                      ((256 * 3 + 5, 6 * sw + 1), 0), ((1000, 4095), 0), ((3, 700, 2 * sw + vec + 1), 1)]:
         h = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
             h[..., ::3] = 0
