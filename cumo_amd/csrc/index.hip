@@ -169,8 +169,9 @@ __global__ __launch_bounds__(kIxBlock) void stridx_buffer_kernel(StridxView v, c
     }
 }
 
-// The last dimension is contiguous in the view: rows of row_bytes move whole, as
-// 128-bit vectors where the row's address in the view allows. A row is cut into
+// The last dimension is contiguous in the view: rows of row_bytes (a whole number of 4-byte
+// words) move whole, as 128-bit vectors and up to three words after them where the row's
+// address in the view is a 4-byte boundary, byte by byte otherwise. A row is cut into
 // segments of at most seg_vecs vectors; LPR lanes share one segment, four vectors each
 // per step. v.ndim counts the outer dimensions only. NT, for copies that stream past the
 // caches: non-temporal stores, and non-temporal loads from the buffer (touched exactly
@@ -179,8 +180,10 @@ struct StridxRows {
     uint32_t units;      // rows * segs_per_row  (< 2^31)
     uint32_t segs_per_row;
     Div31 seg_div;
-    uint32_t row_vecs;   // row_bytes / 16
+    uint32_t row_vecs;   // whole 16-byte vectors of a row
     uint32_t seg_vecs;
+    uint32_t tail_words; // 4-byte words of a row after its whole vectors (0..3)
+    uint64_t row_bytes;
 };
 
 typedef uint32_t ix_u4 __attribute__((ext_vector_type(4)));
@@ -202,10 +205,16 @@ __global__ __launch_bounds__(kIxBlock) void stridx_rows_kernel(StridxView v, Str
         const uint32_t first = seg * g.seg_vecs;
         const uint32_t nv = min(g.seg_vecs, g.row_vecs - first);
         char* in_view = v.ptr + off + (uint64_t)first * 16;
-        char* in_buf = buf + ((uint64_t)row * g.row_vecs + first) * 16;
+        char* in_buf = buf + (uint64_t)row * g.row_bytes + (uint64_t)first * 16;
         const char* src = TO_BUFFER ? in_view : in_buf;
         char* dst = TO_BUFFER ? in_buf : in_view;
-        if (((uintptr_t)in_view & 15) == 0) {
+        // (a 128-bit access works on any 4-byte boundary)
+        if (((uintptr_t)in_view & 3) == 0) {
+            if (seg + 1 == g.segs_per_row && lane < g.tail_words) {
+                // the words of the row after its last whole vector
+                const uint64_t at = (uint64_t)(g.row_vecs - first) * 16 + (uint64_t)lane * 4;
+                *reinterpret_cast<uint32_t*>(dst + at) = *reinterpret_cast<const uint32_t*>(src + at);
+            }
             const ix_u4* s4 = reinterpret_cast<const ix_u4*>(src);
             ix_u4* d4 = reinterpret_cast<ix_u4*>(dst);
             for (uint32_t b = 0; b < nv; b += 4 * LPR) {
@@ -223,12 +232,9 @@ __global__ __launch_bounds__(kIxBlock) void stridx_rows_kernel(StridxView v, Str
                     }
                 }
             }
-        } else if (((uintptr_t)in_view & 3) == 0) {
-            const uint32_t* s1 = reinterpret_cast<const uint32_t*>(src);
-            uint32_t* d1 = reinterpret_cast<uint32_t*>(dst);
-            for (uint32_t b = lane; b < nv * 4; b += LPR) d1[b] = s1[b];
         } else {
-            for (uint32_t b = lane; b < nv * 16; b += LPR) dst[b] = src[b];
+            const uint32_t nb = nv * 16 + ((seg + 1 == g.segs_per_row) ? g.tail_words * 4 : 0);
+            for (uint32_t b = lane; b < nb; b += LPR) dst[b] = src[b];
         }
     }
 }
@@ -251,11 +257,13 @@ void stridx_buffer_launch(const cumo_na_iarray_stridx_t* a, const cumo_na_indexe
     hipStream_t stream = current_stream();
     // whole rows: the last dimension runs contiguously in the view
     const int last = v.ndim - 1;
-    if (small && v.ndim >= 1 && !v.index[last] && v.stride[last] == (int64_t)elmsz && ((uintptr_t)buf & 15) == 0) {
+    if (small && v.ndim >= 1 && !v.index[last] && v.stride[last] == (int64_t)elmsz && ((uintptr_t)buf & 3) == 0) {
         const uint64_t row_bytes = v.shape[last] * elmsz;
-        if (row_bytes % 16 == 0 && row_bytes >= 256) {
+        if (row_bytes % 4 == 0 && row_bytes >= 256) {
             StridxRows g;
             g.row_vecs = (uint32_t)(row_bytes / 16);
+            g.tail_words = (uint32_t)((row_bytes % 16) / 4);
+            g.row_bytes = row_bytes;
             g.seg_vecs = 1024;
             g.segs_per_row = (g.row_vecs + g.seg_vecs - 1) / g.seg_vecs;
             const uint64_t rows = v.total / v.shape[last];

@@ -221,6 +221,38 @@ def test_getitem_with_index_arrays(cls_name, dtype):
 
 
 @pytest.mark.parametrize("cls_name,dtype", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
+def test_whole_rows_through_an_index_array(cls_name, dtype):
+    """Rows of 256 bytes and more move as 128-bit vectors plus up to three 4-byte words, from any 4-byte
+    boundary: row lengths that are and are not whole vectors, a view whose rows start one element in,
+    rows picked twice when reading, a permutation when writing, two outer dimensions."""
+    import cumo_amd
+    cls = getattr(cumo_amd, cls_name)
+    rng = np.random.default_rng(12)
+    for shape in [(50, 64), (50, 67), (30, 131), (9, 4095), (12, 1000), (7, 1029), (40, 65)]:
+        x = rng.integers(-1000, 1000, shape).astype(dtype)
+        d = cls.cast(x)
+        rows = rng.integers(0, shape[0], 2 * shape[0])
+        perm = rng.permutation(shape[0])
+        assert_bits_equal(d[rows].to_numpy(), x[rows], (shape, "rows with repeats"))
+        assert_bits_equal(d[perm, True].to_numpy(), x[perm], (shape, "permutation"))
+        assert_bits_equal(d[:, 1:][perm].to_numpy(), x[:, 1:][perm], (shape, "rows that start one element in"))
+        b = cls.cast(np.zeros(shape, dtype=dtype))
+        b[perm] = d
+        want = np.zeros(shape, dtype=dtype)
+        want[perm] = x
+        assert_bits_equal(b.to_numpy(), want, (shape, "scatter"))
+        c = cls.cast(np.zeros(shape, dtype=dtype))
+        c[:, 1:][perm] = d[:, 1:]
+        want = np.zeros(shape, dtype=dtype)
+        want[:, 1:][perm] = x[:, 1:]
+        assert_bits_equal(c.to_numpy(), want, (shape, "scatter into rows that start one element in"))
+    x = rng.integers(-1000, 1000, (6, 5, 67)).astype(dtype)
+    d = cls.cast(x)
+    assert_bits_equal(d[[4, 0, 4], True, True].to_numpy(), x[[4, 0, 4]], "two outer dimensions")
+    assert_bits_equal(d[True, [3, 1], True].to_numpy(), x[:, [3, 1]], "index array in the middle")
+
+
+@pytest.mark.parametrize("cls_name,dtype", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
 def test_setitem_with_index_arrays_and_slices(cls_name, dtype):
     import cumo_amd
     cls = getattr(cumo_amd, cls_name)
