@@ -691,6 +691,83 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_kernel(const char* __res
     }
 }
 
+// The same over a contiguous matrix (op) a second two-dimensional operand that is addressed by row
+// and column (a row vector, a column vector, a view): the matrix and the bits are each one run, so
+// this takes `matrix > row` for any row length (it went through the general row kernel: SFloat
+// [8192,4096] > [1,4096] 30.6 us, [8192,4095] 100 us). Both inputs of one type; n < 2^31.
+template <class Op, int VEC, bool NT>
+__global__ __launch_bounds__(kEwBlock) void ew_flat_bit_period_kernel(const char* __restrict__ pfull, const char* __restrict__ pper,
+                                                                      CUMO_BIT_DIGIT* __restrict__ pz, uint32_t n, EwPeriod pr, Op op) {
+    typedef typename Op::A A;
+    static_assert(Op::NIN == 2, "two inputs");
+    constexpr int UNR = 4;
+    constexpr unsigned G = 32 / VEC;
+    const uint32_t lane = blockIdx.x * (uint32_t)kEwBlock + threadIdx.x;
+    const uint32_t group = lane / G;
+    const unsigned k = lane % G;
+    const uint64_t first64 = (uint64_t)group * (32 * UNR);  // the group's first element
+    if (first64 >= n) return;
+    const uint32_t first = (uint32_t)first64;
+    const uint32_t e0 = first + k * VEC;
+    auto addressed = [&](uint32_t e, int j) -> A {
+        const uint32_t q = div31(e + j, pr.div);
+        const uint32_t r = e + j - q * pr.period;
+        return *reinterpret_cast<const A*>(pper + (int64_t)q * pr.s_outer + (int64_t)r * pr.s_inner);
+    };
+    if (first64 + 32 * UNR <= n) {
+        A fv[UNR][VEC], pv[UNR][VEC];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) raw_load<A, VEC, NT>(pfull + (uint64_t)(e0 + 32 * u) * sizeof(A), fv[u]);
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const uint32_t e = e0 + 32 * u;
+            const uint32_t q = div31(e, pr.div);
+            const uint32_t r = e - q * pr.period;
+            const char* prow = pper + (int64_t)q * pr.s_outer;
+            if (r + VEC <= pr.period && pr.s_inner == (int64_t)sizeof(A)) {
+                raw_load<A, VEC, false>(prow + (int64_t)r * (int64_t)sizeof(A), pv[u]);
+            } else if (r + VEC <= pr.period && pr.s_inner == 0) {
+                const A v = *reinterpret_cast<const A*>(prow);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) pv[u][j] = v;
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) pv[u][j] = addressed(e, j);
+            }
+        }
+        uint32_t words[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            uint32_t bits = 0;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const A x = pr.first ? pv[u][j] : fv[u][j];
+                const A y = pr.first ? fv[u][j] : pv[u][j];
+                uint32_t z = 0;
+                op(x, y, z);
+                bits |= (z ? 1u : 0u) << j;
+            }
+            words[u] = ew_gather_word<VEC>(bits);
+        }
+        if (k == 0) *reinterpret_cast<u32x4*>(pz + (size_t)group * UNR) = u32x4{words[0], words[1], words[2], words[3]};
+        return;
+    }
+    // the ragged end: at most 32 * UNR - 1 elements in the whole launch
+    for (int u = 0; u < UNR; ++u) {
+        for (int j = 0; j < VEC; ++j) {
+            const uint64_t e = (uint64_t)e0 + 32 * u + j;
+            if (e >= n) continue;
+            const A f = reinterpret_cast<const A*>(pfull)[e];
+            const A a = addressed((uint32_t)e, 0);
+            uint32_t z = 0;
+            op(pr.first ? a : f, pr.first ? f : a, z);
+            const uint32_t bit = 1u << (e & 31);
+            if (z) atomicOr(&pz[e >> 5], bit);
+            else atomicAnd(&pz[e >> 5], ~bit);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Two-dimensional kernel for typed results: rows x inner, every operand either
 // walks the inner dimension contiguously or is constant along it (a column
@@ -1502,6 +1579,36 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 else hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], dst, kp.inner, use_scalar, op, sv);
                 cumo_cuda_runtime_check_kernel_launch();
                 return;
+            }
+            // a contiguous matrix (op) a second two-dimensional operand, the bits one run as well
+            if constexpr (Op::NIN == 2 && std::is_same<A, B>::value) {
+                if (n == 2 && nops == 3 && use_scalar == 0 && !force_scalar && !force_wide_indices() && plan.total < 0x7fffffffull && kp.inner >= 64 &&
+                    plan.step[2][1] == 1 && plan.step[2][0] == (int64_t)kp.inner && (out_bit->pos % 128) == 0 && ((uintptr_t)out_bit->ptr % 16) == 0) {
+                    const int64_t es = (int64_t)sizeof(A);
+                    auto one_run = [&](int sl) { return kp.istep[sl] == es && kp.ostep[sl][0] == es * (int64_t)kp.inner && ((uintptr_t)kp.ptr[sl] % 16) == 0; };
+                    const int full = one_run(0) ? 0 : (one_run(1) ? 1 : -1);
+                    if (full >= 0) {
+                        const int per = 1 - full;
+                        EwPeriod pr;
+                        pr.period = (uint32_t)kp.inner;
+                        pr.div = div31_make(pr.period);
+                        pr.s_outer = kp.ostep[per][0];
+                        pr.s_inner = kp.istep[per];
+                        pr.first = per == 0 ? 1 : 0;
+                        const uint32_t total = (uint32_t)plan.total;
+                        const uint64_t pgroups = ((uint64_t)total + 127) / 128;
+                        const uint64_t pblocks = (pgroups * (32 / VB) + kEwBlock - 1) / kEwBlock;
+                        if (pblocks <= ew_grid_max()) {
+                            const bool nt = stream_past_caches((uint64_t)total * sizeof(A));
+                            CUMO_BIT_DIGIT* dst = reinterpret_cast<CUMO_BIT_DIGIT*>(const_cast<char*>(ops[nops - 1].ptr)) + out_bit->pos / 32;
+                            const dim3 g((unsigned)pblocks);
+                            if (nt) hipLaunchKernelGGL((ew_flat_bit_period_kernel<Op, VB, true>), g, b, 0, stream, kp.ptr[full], kp.ptr[per], dst, total, pr, op);
+                            else hipLaunchKernelGGL((ew_flat_bit_period_kernel<Op, VB, false>), g, b, 0, stream, kp.ptr[full], kp.ptr[per], dst, total, pr, op);
+                            cumo_cuda_runtime_check_kernel_launch();
+                            return;
+                        }
+                    }
+                }
             }
         }
     }

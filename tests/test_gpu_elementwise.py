@@ -386,7 +386,11 @@ def test_fill_and_store_into_views():
 def test_compare_into_bit(tname, dt, op):
     rng = np.random.default_rng(109)
     cls = cls_of(tname)
-    for shape in [(1,), (31,), (32,), (33,), (64,), (1000,), (5, 67), (7, 64), (3, 5, 96), (129, 33)]:
+    # (from 64 columns on, matrix (op) row / column / view goes flat over the matrix and the bits, the other
+    # operand addressed by row and column: row lengths that are and are not whole vectors, totals that end
+    # inside a group of 128 bits)
+    for shape in [(1,), (31,), (32,), (33,), (64,), (1000,), (5, 67), (7, 64), (3, 5, 96), (129, 33), (37, 65), (130, 4095), (64, 128),
+                  (9, 1001), (33, 256)]:
         hx = rng.integers(-3, 4, size=shape).astype(dt)
         hy = rng.integers(-3, 4, size=shape).astype(dt)
         if dt != np.int32:
@@ -398,6 +402,12 @@ def test_compare_into_bit(tname, dt, op):
             assert (getattr(dx.transpose(), op)(dy.transpose()).to_numpy() == oracle.compare(op, hx.T, hy.T)).all(), (shape, op, "T")
             assert (getattr(dx[:, ::2], op)(0).to_numpy() == oracle.compare(op, hx[:, ::2], 0)).all()
             assert (getattr(dx, op)(dy[0]).to_numpy() == oracle.compare(op, hx, hy[0])).all(), (shape, op, "bcast")
+            assert (getattr(dy[0], op)(dx).to_numpy() == oracle.compare(op, hy[0], hx)).all(), (shape, op, "row on the left")
+            col, hcol = dy[:, :1], hy[:, :1]
+            assert (getattr(dx, op)(col).to_numpy() == oracle.compare(op, hx, hcol)).all(), (shape, op, "column")
+            assert (getattr(col, op)(dx).to_numpy() == oracle.compare(op, hcol, hx)).all(), (shape, op, "column on the left")
+            wide = cls.cast(np.repeat(hy, 2, axis=1))
+            assert (getattr(dx, op)(wide[:, ::2]).to_numpy() == oracle.compare(op, hx, hy)).all(), (shape, op, "view")
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
