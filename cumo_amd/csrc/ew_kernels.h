@@ -1070,9 +1070,10 @@ __device__ __forceinline__ void ew_tile_at(const EwTParams& p, uint64_t tile, ui
     g0 = gt * TG;
 }
 
-// The 128-bit form: every operand tolerates 128-bit accesses along its own fast
-// dimension (the launcher checks alignment and divisibility), so both the reads
-// along G and the writes along F move 16 bytes per lane.
+// The 128-bit form: every operand is contiguous along its own fast dimension, so both
+// the reads along G and the writes along F move 16 bytes per lane (from any 4-byte
+// boundary; the one vector on either side that lies partly inside the array goes
+// element by element).
 // PREFETCH: a block walks several tiles and keeps the transposed inputs of its
 // next tile in flight, in registers, while it computes and stores the current
 // one. That pays for an op with many instructions per element, whose blocks
@@ -1115,11 +1116,14 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p,
     uint64_t f0 = 0, g0 = 0;
     int64_t off[3] = {0, 0, 0};
 
-    // Loads of a tile's edge are not skipped but pulled back inside the array (G and F
-    // extents are whole vectors here): with no branch between them the loads of a
-    // lane go out back to back. What the pulled-back lanes put into LDS is never read.
+    // Loads of a tile's edge are not skipped but pulled back inside the array: with no
+    // branch between them the loads of a lane go out back to back. What the pulled-back
+    // lanes put into LDS is never read. The one vector along G that is partly inside the
+    // array (G need not be a whole number of vectors) is read element by element, in place.
     auto fetch = [&](uint64_t tf0, uint64_t tg0, const int64_t (&toff)[3]) {
-        uint64_t g = tg0 + (uint64_t)gv * V;
+        const uint64_t g_own = tg0 + (uint64_t)gv * V;
+        const bool partial = g_own < p.ng && g_own + V > p.ng;
+        uint64_t g = g_own;
         if (g > p.ng - V) g = p.ng - V;
         if (tr_a) {
             const char* src = p.ptr[0] + toff[0] + (int64_t)g * (int64_t)sizeof(A);
@@ -1128,6 +1132,17 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p,
                 uint64_t f = tf0 + lf0 + k * FP;
                 if (f > p.nf - 1) f = p.nf - 1;
                 raw_load<A, V, NT>(src + (int64_t)f * p.fstep[0], va[k]);
+            }
+            if (partial) {
+                const char* own = p.ptr[0] + toff[0] + (int64_t)g_own * (int64_t)sizeof(A);
+#pragma unroll
+                for (unsigned k = 0; k < NP; ++k) {
+                    uint64_t f = tf0 + lf0 + k * FP;
+                    if (f > p.nf - 1) f = p.nf - 1;
+#pragma unroll
+                    for (int q = 0; q < V; ++q)
+                        if (g_own + q < p.ng) va[k][q] = reinterpret_cast<const A*>(own + (int64_t)f * p.fstep[0])[q];
+                }
             }
         }
         if constexpr (TWO) {
@@ -1138,6 +1153,17 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p,
                     uint64_t f = tf0 + lf0 + k * FP;
                     if (f > p.nf - 1) f = p.nf - 1;
                     raw_load<B, V, NT>(src + (int64_t)f * p.fstep[1], vb[k]);
+                }
+                if (partial) {
+                    const char* own = p.ptr[1] + toff[1] + (int64_t)g_own * (int64_t)sizeof(B);
+#pragma unroll
+                    for (unsigned k = 0; k < NP; ++k) {
+                        uint64_t f = tf0 + lf0 + k * FP;
+                        if (f > p.nf - 1) f = p.nf - 1;
+#pragma unroll
+                        for (int q = 0; q < V; ++q)
+                            if (g_own + q < p.ng) vb[k][q] = reinterpret_cast<const B*>(own + (int64_t)f * p.fstep[1])[q];
+                    }
                 }
             }
         }
@@ -1179,7 +1205,31 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p,
         }
         // lanes along F: pick the tile up transposed, compute, store
         const uint64_t f = f0 + (uint64_t)fv * V;
-        if (f < p.nf) {
+        if (f < p.nf && f + V > p.nf) {
+            // the one vector along F that is partly inside the array (F need not be a whole number
+            // of vectors): its elements one by one, nothing read or written past the row
+            for (unsigned k = 0; k < NQ; ++k) {
+                const unsigned lg = lg0 + k * GP;
+                const uint64_t g = g0 + lg;
+                if (g >= p.ng) continue;
+                for (int q = 0; q < V; ++q) {
+                    if (f + q >= p.nf) break;
+                    A xa = A();
+                    B yb = B();
+                    if (NIN >= 1) xa = tr_a ? tile_a[lg][fv * V + q]
+                                            : *reinterpret_cast<const A*>(p.ptr[0] + off[0] + (int64_t)g * p.gstep[0] + (int64_t)(f + q) * p.fstep[0]);
+                    if (TWO) {
+                        if (p.use_scalar == 0) yb = tr_b ? tile_b[lg][fv * V + q]
+                                                         : *reinterpret_cast<const B*>(p.ptr[1] + off[1] + (int64_t)g * p.gstep[1] + (int64_t)(f + q) * p.fstep[1]);
+                        else if (p.use_scalar == 1) yb = (B)sv;
+                        else { yb = (B)xa; xa = (A)sv; }
+                    }
+                    R zz = R();
+                    if (op(xa, yb, zz)) *reinterpret_cast<R*>(p.ptr[2] + off[2] + (int64_t)g * p.gstep[2] + (int64_t)(f + q) * (int64_t)sizeof(R)) = zz;
+                    else if (p.flag) *p.flag = 1;
+                }
+            }
+        } else if (f < p.nf) {
             // an op with many instructions per element is not unrolled over the rows:
             // its V elements side by side already fill the registers eight waves can have
             constexpr int UNROLL_ROWS = op_is_heavy<Op>::value ? 1 : (int)NQ;
@@ -1450,8 +1500,11 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         // 128-bit form: same element size everywhere, whole vectors in both tile
         // directions, every operand aligned along the dimension it is walked in
         constexpr int V = 16 / (int)sizeof(A);
+        // (neither extent need be a whole number of vectors, and the operands need their element's alignment
+        // only: a 128-bit access works on any 4-byte boundary, and the one vector that is partly inside the
+        // array on either side goes element by element)
         bool vt = sizeof(A) == sizeof(R) && (Op::NIN < 2 || sizeof(B) == sizeof(A)) && (16 % sizeof(A)) == 0 && sizeof(A) >= 4 &&
-                  (tp.ng % V) == 0 && (tp.nf % V) == 0;
+                  tp.ng >= (uint64_t)V && tp.nf >= (uint64_t)V;
         for (int o = 0; o < nops && vt; ++o) {
             const int sl = slot[o];
             const int64_t es = (int64_t)sizeof(A);
@@ -1459,8 +1512,8 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             const int64_t along = through_lds ? tp.gstep[sl] : tp.fstep[sl];
             const int64_t across = through_lds ? tp.fstep[sl] : tp.gstep[sl];
             if (sl < 2 && !through_lds && along == 0) continue;  // broadcast along F: scalar loads
-            vt = along == es && (across % 16) == 0 && ((uintptr_t)tp.ptr[sl] % 16) == 0;
-            for (int d = 0; d < n - 2 && vt; ++d) vt = (tp.ostep[sl][d] % 16) == 0;
+            vt = along == es && (across % es) == 0 && ((uintptr_t)tp.ptr[sl] % es) == 0;
+            for (int d = 0; d < n - 2 && vt; ++d) vt = (tp.ostep[sl][d] % es) == 0;
         }
         if constexpr (sizeof(A) == sizeof(R) && (Op::NIN < 2 || sizeof(B) == sizeof(A)) && (16 % sizeof(A)) == 0 && sizeof(A) >= 4) {
             if (vt) {

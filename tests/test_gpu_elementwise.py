@@ -123,6 +123,39 @@ def test_matrices_with_rows_of_an_odd_length_and_a_second_operand(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+def test_transposed_operands_whose_extents_are_not_whole_vectors(tname, dt):
+    """Transposed views go through LDS tiles with 128-bit accesses on both sides; neither extent need be
+    a whole number of vectors, and rows need their element's alignment only: extents of 4k + 1, 2, 3,
+    one and both inputs transposed, a transposed input beside a plain one and beside a scalar, a heavy
+    function, stacked matrices, and Int32 with a division that meets a zero at the ragged edge."""
+    import cumo_amd
+    rng = np.random.default_rng(404)
+    cls = cls_of(tname)
+    for (R, Cn) in [(67, 131), (130, 4095), (4095, 130), (33, 65), (258, 1027), (5, 70), (1001, 9)]:
+        a = rng.standard_normal((R, Cn)).astype(dt)
+        b = rng.standard_normal((Cn, R)).astype(dt)
+        c = rng.standard_normal((R, Cn)).astype(dt)
+        da, db, dc = cls.cast(a), cls.cast(b), cls.cast(c)
+        at = np.ascontiguousarray(a.T)
+        assert_bits_equal((da.transpose() + 1.5).to_numpy(), oracle.binary("add", at, 1.5), ((R, Cn), "transposed + scalar"))
+        assert_bits_equal((da.transpose() * db).to_numpy(), oracle.binary("mul", at, b), ((R, Cn), "transposed * plain"))
+        assert_bits_equal((db - da.transpose()).to_numpy(), oracle.binary("sub", b, at), ((R, Cn), "plain - transposed"))
+        assert_bits_equal((da.transpose() / dc.transpose()).to_numpy(), oracle.binary("div", at, np.ascontiguousarray(c.T)), ((R, Cn), "both transposed"))
+        assert_bits_equal((-da.transpose()).to_numpy(), oracle.unary("minus", at), ((R, Cn), "unary"))
+        assert_ulp(cumo_amd.NMath.exp(da.transpose()).to_numpy(), oracle.unary("exp", at), 1)
+        assert_ulp((da.transpose().abs() ** 2.5).to_numpy(), oracle.binary("pow", np.abs(at), 2.5), 1 if dt == np.float32 else 2)
+    s = rng.standard_normal((3, 37, 66)).astype(dt)
+    assert_bits_equal((cls.cast(s).transpose(0, 2, 1) + 0.25).to_numpy(), oracle.binary("add", np.ascontiguousarray(s.transpose(0, 2, 1)), 0.25), "stacked")
+    hi = rng.integers(-1000, 1000, size=(67, 131)).astype(np.int32)
+    hz = rng.integers(1, 50, size=(131, 67)).astype(np.int32)
+    di, dz = cumo_amd.Int32.cast(hi), cumo_amd.Int32.cast(hz)
+    assert ((di.transpose() / dz).to_numpy() == oracle.binary("div", np.ascontiguousarray(hi.T), hz)).all()
+    hz[130, 66] = 0
+    with pytest.raises(ZeroDivisionError):
+        di.transpose() / cumo_amd.Int32.cast(hz)
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 def test_three_dimensions_with_an_operand_repeating_along_one(tname, dt):
     """[B,T,C] with [T,1], [B,1,C], [1,T,C], [B,1,1] and a column on both sides: the shapes whose two
     outer dimensions do not merge; C a whole number of 128-bit vectors and not; outer views."""
