@@ -241,15 +241,17 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
         for (; vec > 1; vec >>= 1) {
             // the input is only read: a 128-bit global load needs no more than the element's alignment
             const int align = in_elmsz >= 4 ? in_elmsz : vec * in_elmsz;
-            bool ok = plan->in_out_step[L] == in_elmsz && (plan->out_shape[L] % vec) == 0 &&
-                      ((uintptr_t)arg->in.ptr % align) == 0;
+            // (outputs along one dimension may end in part of a vector where the caller's kernel sees to it)
+            const bool whole = (plan->out_shape[L] % vec) == 0 || (allow_tail && no == 1 && plan->out_shape[L] >= (uint64_t)vec * 64);
+            bool ok = plan->in_out_step[L] == in_elmsz && whole && ((uintptr_t)arg->in.ptr % align) == 0;
             for (int d = 0; d < L && ok; ++d) ok = (plan->in_out_step[d] % align) == 0;
             for (int d = 0; d < nr && ok; ++d) ok = (plan->in_red_step[d] % align) == 0;
             if (ok) break;
         }
         plan->vec = vec < 1 ? 1 : vec;
+        plan->red_tail = plan->vec > 1 ? (int)(plan->out_shape[L] % (uint64_t)plan->vec) : 0;
         // few outputs and a long axis: cut the axis across blocks
-        uint64_t threads = out_total / plan->vec;
+        uint64_t threads = (out_total + plan->vec - 1) / plan->vec;
         uint64_t blocks = (threads + 255) / 256;
         if (blocks < (uint64_t)kNumCU * 2 && N >= 128) {
             uint64_t want = ((uint64_t)kNumCU * 4 + blocks - 1) / blocks;

@@ -49,7 +49,8 @@ struct ReducePlan {
     int threads_per_row;   // RED_ROW: lanes sharing one output (power of two, <= 256)
     int n_split;           // > 1: the reduce axis is cut into n_split chunks and combined by a second launch
     int local_split_bits;  // RED_COL: 2^bits lanes of a block share an output's reduce axis and combine through LDS
-    int red_tail;          // RED_ROW, only when the caller allowed it: elements of the axis past its last whole vector
+    int red_tail;          // only when the caller allowed it: RED_ROW, elements of the axis past its last whole vector;
+                           // RED_COL, outputs past the last whole vector of outputs
     int out_ndim, red_ndim;
     uint64_t out_total, red_total;
     uint64_t out_shape[kMaxDim], red_shape[kMaxDim];
@@ -61,8 +62,8 @@ struct ReducePlan {
 
 // in_elmsz: bytes per input element. accum_bytes: sizeof the accumulator, which
 // sizes the scratch of a split reduction. out2 may be NULL.
-// allow_tail: a contiguous reduce axis need not be a whole number of vectors (red_tail says what is left over);
-// for callers whose kernels fold those elements separately.
+// allow_tail: a contiguous reduce axis (or, with the outputs along memory, their one dimension) need not be a
+// whole number of vectors (red_tail says what is left over); for callers whose kernels see to the rest.
 void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, int in_elmsz, int accum_bytes,
                  ReducePlan* plan, bool allow_tail = false);
 

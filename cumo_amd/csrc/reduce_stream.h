@@ -459,7 +459,7 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
     }
 }
 
-// Column form. n_out is a multiple of VEC and so is out_inner.
+// Column form. out_inner is a multiple of VEC, or the outputs span one dimension (n_out >= VEC).
 // U: positions of the axis a lane has in flight (more when the outputs alone give too few lanes
 // to keep the memory system busy: a block still reads 4 KiB runs of every row it touches).
 // PARTIAL: the axis is also cut across blocks, p.n_split ways (blockIdx.y says which part this
@@ -476,7 +476,9 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
     const unsigned CPB = 1u << cbits;
     const unsigned c = threadIdx.x & (CPB - 1);
     const unsigned s = threadIdx.x >> cbits;
-    const uint32_t groups = p.n_out / VEC;
+    // (the outputs need not be a whole number of vectors when they span one dimension: the last group
+    // is pulled back to the last VEC outputs and stores only those the group before it does not)
+    const uint32_t groups = (p.n_out + VEC - 1) / VEC;
     const uint32_t n_cb = (groups + CPB - 1) / CPB;
     // this block's stretch of the axis, then this lane's part of it
     uint64_t b0 = 0, b1 = p.n;
@@ -496,7 +498,8 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
     for (uint32_t cb = blockIdx.x; cb < n_cb; cb += gridDim.x) {
         const uint32_t g = cb * CPB + c;
         const bool ok = g < groups;
-        const uint32_t i_out0 = (ok ? g : groups - 1) * VEC;
+        const uint32_t own0 = (ok ? g : groups - 1) * VEC;           // the group's first output
+        const uint32_t i_out0 = own0 + VEC <= p.n_out ? own0 : p.n_out - VEC;  // where its vector starts
         uint32_t o0, o1;
         rs_split_out(p, i_out0, o0, o1);
         const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
@@ -578,13 +581,15 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
             if (ok && s == 0) {
                 Acc* partial = reinterpret_cast<Acc*>(p.partial);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) partial[(size_t)(i_out0 + j) * p.n_split + blockIdx.y] = acc[j];
+                for (int j = 0; j < VEC; ++j)
+                    if (i_out0 + j >= own0) partial[(size_t)(i_out0 + j) * p.n_split + blockIdx.y] = acc[j];
             }
             continue;
         }
         if (ok && s == 0) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
+                if (i_out0 + j < own0) continue;  // (the pulled-back last group: the group before it has these)
                 // the VEC outputs of a group are neighbours along the inner output dimension
                 const int64_t a = (int64_t)o0 * p.out_step[0] + (int64_t)(o1 + j) * p.out_step[1];
                 const int64_t b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)(o1 + j) * p.out2_step[1] : 0;

@@ -247,7 +247,8 @@ def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((700, 24), 0), ((3, 700, 24), 1), ((40000, 8), 0), ((2, 5000, 3), 1), ((130, 1024), 0),
-                                        ((3000, 1000), 0), ((4096, 520), 0), ((2, 2100, 516), 1)])
+                                        ((3000, 1000), 0), ((4096, 520), 0), ((2, 2100, 516), 1), ((3000, 1001), 0), ((700, 4095), 0),
+                                        ((40, 70001), 0), ((5000, 259), 0)])
 def test_few_outputs_across_memory_share_the_axis_inside_a_block(tname, dt, shape, axis):
     """The column kernel with the reduce axis cut inside the block (and, for the long ones, across
     blocks as well): ties resolve to the lowest index across the parts, NaN rules, both results of
