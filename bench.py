@@ -198,6 +198,29 @@ def config_ops(name, cumo, host):
             ("x[perm,true] (gather, every row once)", lambda e: e.__setitem__("g", e["x"][e["perm"]]), 2 * nb + 8 * r, n),
             ("b[perm,true]=x (scatter)", lambda e: e["b"].__setitem__(e["perm"], e["x"]), 2 * nb + 8 * r, n),
         ]
+    if name == "odd":
+        # the hot-path operations on a matrix whose rows are not a whole number of 128-bit vectors (4095 SFloat:
+        # every row after the first starts off a 16-byte boundary)
+        x, y, r = host["x"], host["y"], host["r"]
+        env = {"x": cumo.SFloat.cast(x), "y": cumo.SFloat.cast(y), "r": cumo.SFloat.cast(r), "perm": host["perm"]}
+        n, nb = x.size, x.nbytes
+        rows, cols = x.shape
+        return env, [
+            ("A+r (row vector)", lambda e: e.__setitem__("c", e["x"] + e["r"]), 2 * nb + 4 * cols, n),
+            ("A+B", lambda e: e.__setitem__("c", e["x"] + e["y"]), 3 * nb, n),
+            ("A>r into Bit", lambda e: e.__setitem__("m", e["x"] > e["r"]), nb + n // 8, n),
+            ("A.transpose + 1", lambda e: e.__setitem__("t", e["x"].transpose() + 1.0), 2 * nb, n),
+            ("A.sum(axis:1)", lambda e: e.__setitem__("s", e["x"].sum(axis=1)), nb + 4 * rows, n),
+            ("A.max(axis:1)", lambda e: e.__setitem__("s", e["x"].max(axis=1)), nb + 4 * rows, n),
+            ("A.sum(axis:0)", lambda e: e.__setitem__("s0", e["x"].sum(axis=0)), nb + 4 * cols, n),
+            ("A.sum", lambda e: e.__setitem__("s1", e["x"].sum()), nb, n),
+            ("A.mulsum(B,axis:1)", lambda e: e.__setitem__("d", e["x"].mulsum(e["y"], axis=1)), 2 * nb + 4 * rows, n),
+            ("Fused.softmax(A)", lambda e: e.__setitem__("p", cumo.Fused.softmax(e["x"])), 2 * nb, n),
+            ("Fused.layernorm(A)", lambda e: e.__setitem__("l", cumo.Fused.layernorm(e["x"], 1e-5)), 2 * nb, n),
+            ("A[perm,true]", lambda e: e.__setitem__("g", e["x"][e["perm"]]), 2 * nb + 8 * rows, n),
+            ("A.cumsum(axis:1)", lambda e: e.__setitem__("c1", e["x"].cumsum(axis=1)), 2 * nb, n),
+            ("A.cumsum(axis:0)", lambda e: e.__setitem__("c0", e["x"].cumsum(axis=0)), 2 * nb, n),
+        ]
     if name == "nmath":
         # NMath beyond exp / sqrt, the Float power and the scans on 2^26 elements (256 MiB SFloat,
         # 512 MiB DFloat per array); arguments positive so that every function is defined
@@ -221,6 +244,12 @@ def config_ops(name, cumo, host):
     raise ValueError(name)
 
 
+def inputs_odd(shape=(8192, 4095)):
+    rng = np.random.default_rng(7)
+    return {"x": rng.standard_normal(shape, dtype=np.float32), "y": rng.standard_normal(shape, dtype=np.float32),
+            "r": rng.standard_normal((1, shape[1]), dtype=np.float32), "perm": rng.permutation(shape[0])}
+
+
 def inputs_nmath(n=1 << 26):
     rng = np.random.default_rng(6)
     return {"x": rng.uniform(0.05, 3.0, n).astype(np.float32)}
@@ -229,7 +258,7 @@ def inputs_nmath(n=1 << 26):
 HOST_INPUTS = {
     "c1": inputs_c1, "c1_large": lambda: inputs_c1(1 << 26), "c2": inputs_c2, "c3": inputs_c3, "c4": inputs_c4, "c5": inputs_c5,
     "c2_large": lambda: inputs_c2(8192), "c3_large": lambda: inputs_c3((256, 512, 1024)), "next": inputs_next,
-    "nmath": inputs_nmath,
+    "nmath": inputs_nmath, "odd": inputs_odd,
 }
 WORKLOAD_TEXT = {
     "c1": "C1 SFloat axpy + full sum, n=2^20",
@@ -237,6 +266,7 @@ WORKLOAD_TEXT = {
     "c2_large": "C2 at 8192 x 8192 (512 MiB per matrix)",
     "c3_large": "C3 at [256,512,1024] (512 MiB)",
     "next": "operations beside the five configs on SFloat [8192,4096]: mulsum, clip, maximum, integer power, cumsum, where, a[mask], row gather and scatter through index arrays",
+    "odd": "the hot-path operations on SFloat [8192,4095]: rows that are not a whole number of 128-bit vectors and start off 16-byte boundaries",
     "nmath": "NMath functions, Float power and cumsum on 2^26 elements (SFloat 256 MiB, DFloat 512 MiB per array), arguments uniform in [0.05, 3)",
     "c2": "C2 DFloat broadcast add + row reduce: A f64 [4096,4096] + r [1,4096]; C.sum(axis:1); C.max(axis:1)",
     "c3": "C3 SFloat axis reductions on [64,512,1024]",
@@ -437,7 +467,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all-configs", action="store_true", help="measure every op of all five configs with full iteration counts")
-    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next,nmath)")
+    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next,nmath,odd)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--rotated-only", action="store_true",
@@ -593,7 +623,7 @@ def main():
 
     per_config = {}
     if not args.no_per_config:
-        names = [c for c in args.configs.split(",") if c] or ["c1", "c2", "c3", "c4", "c5", "c1_large", "c2_large", "c3_large", "next", "nmath"]
+        names = [c for c in args.configs.split(",") if c] or ["c1", "c2", "c3", "c4", "c5", "c1_large", "c2_large", "c3_large", "next", "nmath", "odd"]
         iters, warm = (30, 5) if args.all_configs else (7, 2)
         for name in names:
             per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm, not args.rotated_only)}
