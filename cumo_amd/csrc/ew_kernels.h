@@ -431,7 +431,19 @@ struct EwPeriod {
     Div31 div;
     int64_t s_outer, s_inner;  // the addressed operand's byte steps per row and per column
     int first;            // 1: the addressed operand is the op's first input
+    // three dimensions (outer x mid x inner): rows are numbered outer * mid + mid position, and the
+    // addressed operand steps s_outer per mid position and s_outermost per outer position; mid 0 = two dimensions
+    uint32_t mid;
+    Div31 div_mid;
+    int64_t s_outermost;
 };
+
+// byte offset of row q of the addressed operand
+__device__ __forceinline__ int64_t ew_period_row(const EwPeriod& pr, uint32_t q) {
+    if (pr.mid == 0) return (int64_t)q * pr.s_outer;
+    const uint32_t o = div31(q, pr.div_mid);
+    return (int64_t)o * pr.s_outermost + (int64_t)(q - o * pr.mid) * pr.s_outer;
+}
 
 template <class Op, int VEC, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_flat_period_kernel(const char* __restrict__ pfull, const char* __restrict__ pper,
@@ -456,7 +468,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_period_kernel(const char* __
     }
     // the vector lies inside one row nearly always: then the addressed operand gives one (unaligned)
     // 128-bit load where it is contiguous along the row, one element where it is constant along it
-    const char* prow = pper + (int64_t)q * pr.s_outer;
+    const char* prow = pper + ew_period_row(pr, q);
     if (cnt == VEC && r + VEC <= pr.period && pr.s_inner == (int64_t)sizeof(A)) {
         raw_load<A, VEC, false>(prow + (int64_t)r * (int64_t)sizeof(A), pv);
     } else if (cnt == VEC && r + VEC <= pr.period && pr.s_inner == 0) {
@@ -468,7 +480,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_period_kernel(const char* __
         for (int j = 0; j < VEC; ++j) {
             uint32_t rr = r + j, qq = q;
             if (rr >= pr.period) { rr -= pr.period; ++qq; }
-            if ((uint32_t)j < cnt) pv[j] = *reinterpret_cast<const A*>(pper + (int64_t)qq * pr.s_outer + (int64_t)rr * pr.s_inner);
+            if ((uint32_t)j < cnt) pv[j] = *reinterpret_cast<const A*>(pper + ew_period_row(pr, qq) + (int64_t)rr * pr.s_inner);
         }
     }
     R zv[VEC];
@@ -712,7 +724,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_period_kernel(const char
     auto addressed = [&](uint32_t e, int j) -> A {
         const uint32_t q = div31(e + j, pr.div);
         const uint32_t r = e + j - q * pr.period;
-        return *reinterpret_cast<const A*>(pper + (int64_t)q * pr.s_outer + (int64_t)r * pr.s_inner);
+        return *reinterpret_cast<const A*>(pper + ew_period_row(pr, q) + (int64_t)r * pr.s_inner);
     };
     if (first64 + 32 * UNR <= n) {
         A fv[UNR][VEC], pv[UNR][VEC];
@@ -723,7 +735,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_period_kernel(const char
             const uint32_t e = e0 + 32 * u;
             const uint32_t q = div31(e, pr.div);
             const uint32_t r = e - q * pr.period;
-            const char* prow = pper + (int64_t)q * pr.s_outer;
+            const char* prow = pper + ew_period_row(pr, q);
             if (r + VEC <= pr.period && pr.s_inner == (int64_t)sizeof(A)) {
                 raw_load<A, VEC, false>(prow + (int64_t)r * (int64_t)sizeof(A), pv[u]);
             } else if (r + VEC <= pr.period && pr.s_inner == 0) {
@@ -1635,19 +1647,28 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             }
             // a contiguous matrix (op) a second two-dimensional operand, the bits one run as well
             if constexpr (Op::NIN == 2 && std::is_same<A, B>::value) {
-                if (n == 2 && nops == 3 && use_scalar == 0 && !force_scalar && !force_wide_indices() && plan.total < 0x7fffffffull && kp.inner >= 64 &&
-                    plan.step[2][1] == 1 && plan.step[2][0] == (int64_t)kp.inner && (out_bit->pos % 128) == 0 && ((uintptr_t)out_bit->ptr % 16) == 0) {
+                bool bits_one_run = (n == 2 || n == 3) && plan.step[2][n - 1] == 1 && plan.step[2][n - 2] == (int64_t)kp.inner;
+                if (n == 3) bits_one_run = bits_one_run && plan.step[2][0] == (int64_t)kp.inner * (int64_t)plan.shape[1];
+                if (bits_one_run && nops == 3 && use_scalar == 0 && !force_scalar && !force_wide_indices() && plan.total < 0x7fffffffull && kp.inner >= 64 &&
+                    (out_bit->pos % 128) == 0 && ((uintptr_t)out_bit->ptr % 16) == 0) {
                     const int64_t es = (int64_t)sizeof(A);
-                    auto one_run = [&](int sl) { return kp.istep[sl] == es && kp.ostep[sl][0] == es * (int64_t)kp.inner && ((uintptr_t)kp.ptr[sl] % 16) == 0; };
+                    auto one_run = [&](int sl) {
+                        bool run = kp.istep[sl] == es && kp.ostep[sl][n - 2] == es * (int64_t)kp.inner && ((uintptr_t)kp.ptr[sl] % 16) == 0;
+                        if (n == 3) run = run && kp.ostep[sl][0] == es * (int64_t)kp.inner * (int64_t)plan.shape[1];
+                        return run;
+                    };
                     const int full = one_run(0) ? 0 : (one_run(1) ? 1 : -1);
                     if (full >= 0) {
                         const int per = 1 - full;
                         EwPeriod pr;
                         pr.period = (uint32_t)kp.inner;
                         pr.div = div31_make(pr.period);
-                        pr.s_outer = kp.ostep[per][0];
+                        pr.s_outer = kp.ostep[per][n - 2];
                         pr.s_inner = kp.istep[per];
                         pr.first = per == 0 ? 1 : 0;
+                        pr.mid = n == 3 ? (uint32_t)plan.shape[1] : 0u;
+                        pr.div_mid = div31_make(n == 3 ? (uint32_t)plan.shape[1] : 1u);
+                        pr.s_outermost = n == 3 ? kp.ostep[per][0] : 0;
                         const uint32_t total = (uint32_t)plan.total;
                         const uint64_t pgroups = ((uint64_t)total + 127) / 128;
                         const uint64_t pblocks = (pgroups * (32 / VB) + kEwBlock - 1) / kEwBlock;
@@ -1671,10 +1692,14 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     if constexpr (!Op::BIT_OUT && Op::NIN == 2 && std::is_same<A, B>::value && sizeof(A) == sizeof(R) && (sizeof(A) == 4 || sizeof(A) == 8) &&
                   !op_is_heavy<Op>::value && !op_has_rare<Op>::value) {
         constexpr int V = 16 / (int)sizeof(A);
-        if (n == 2 && nops == 3 && use_scalar == 0 && !heavy && !force_scalar && !force_wide_indices() && (kp.inner % V) != 0 && kp.inner >= 64 &&
+        if ((n == 2 || n == 3) && nops == 3 && use_scalar == 0 && !heavy && !force_scalar && !force_wide_indices() && (kp.inner % V) != 0 && kp.inner >= 64 &&
             plan.total < 0x7fffffffull) {
             const int64_t es = (int64_t)sizeof(A);
-            auto one_run = [&](int sl) { return kp.istep[sl] == es && kp.ostep[sl][0] == es * (int64_t)kp.inner && ((uintptr_t)kp.ptr[sl] % 16) == 0; };
+            auto one_run = [&](int sl) {
+                bool run = kp.istep[sl] == es && kp.ostep[sl][n - 2] == es * (int64_t)kp.inner && ((uintptr_t)kp.ptr[sl] % 16) == 0;
+                if (n == 3) run = run && kp.ostep[sl][0] == es * (int64_t)kp.inner * (int64_t)plan.shape[1];
+                return run;
+            };
             int full = -1;
             if (one_run(2)) {
                 if (one_run(0)) full = 0;
@@ -1685,9 +1710,12 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 EwPeriod pr;
                 pr.period = (uint32_t)kp.inner;
                 pr.div = div31_make(pr.period);
-                pr.s_outer = kp.ostep[per][0];
+                pr.s_outer = kp.ostep[per][n - 2];
                 pr.s_inner = kp.istep[per];
                 pr.first = per == 0 ? 1 : 0;
+                pr.mid = n == 3 ? (uint32_t)plan.shape[1] : 0u;
+                pr.div_mid = div31_make(n == 3 ? (uint32_t)plan.shape[1] : 1u);
+                pr.s_outermost = n == 3 ? kp.ostep[per][0] : 0;
                 const uint32_t total = (uint32_t)plan.total;
                 const uint64_t blocks = ((uint64_t)total + (uint64_t)kEwBlock * V - 1) / ((uint64_t)kEwBlock * V);
                 if (blocks <= ew_grid_max()) {

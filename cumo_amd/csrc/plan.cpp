@@ -242,7 +242,7 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
             // the input is only read: a 128-bit global load needs no more than the element's alignment
             const int align = in_elmsz >= 4 ? in_elmsz : vec * in_elmsz;
             // (outputs along one dimension may end in part of a vector where the caller's kernel sees to it)
-            const bool whole = (plan->out_shape[L] % vec) == 0 || (allow_tail && no == 1 && plan->out_shape[L] >= (uint64_t)vec * 64);
+            const bool whole = (plan->out_shape[L] % vec) == 0 || (allow_tail && no <= 2 && plan->out_shape[L] >= (uint64_t)vec * 16);
             bool ok = plan->in_out_step[L] == in_elmsz && whole && ((uintptr_t)arg->in.ptr % align) == 0;
             for (int d = 0; d < L && ok; ++d) ok = (plan->in_out_step[d] % align) == 0;
             for (int d = 0; d < nr && ok; ++d) ok = (plan->in_red_step[d] % align) == 0;
@@ -251,7 +251,7 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
         plan->vec = vec < 1 ? 1 : vec;
         plan->red_tail = plan->vec > 1 ? (int)(plan->out_shape[L] % (uint64_t)plan->vec) : 0;
         // few outputs and a long axis: cut the axis across blocks
-        uint64_t threads = (out_total + plan->vec - 1) / plan->vec;
+        uint64_t threads = (out_total / plan->out_shape[L]) * ((plan->out_shape[L] + plan->vec - 1) / plan->vec);
         uint64_t blocks = (threads + 255) / 256;
         if (blocks < (uint64_t)kNumCU * 2 && N >= 128) {
             uint64_t want = ((uint64_t)kNumCU * 4 + blocks - 1) / blocks;
@@ -284,7 +284,7 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
         const int align = in_elmsz >= 4 ? in_elmsz : vec * in_elmsz;  // read-only: the element's alignment is enough
         // (a single long axis may end in part of a vector where the caller folds that part by itself)
         const bool whole = nr > 0 && ((plan->red_shape[nr - 1] % vec) == 0 ||
-                                      (allow_tail && nr == 1 && plan->red_shape[0] >= (uint64_t)vec * 256));
+                                      (allow_tail && nr == 1 && plan->red_shape[0] >= (uint64_t)vec * 16));
         bool ok = nr > 0 && plan->in_red_step[nr - 1] == in_elmsz && whole && ((uintptr_t)arg->in.ptr % align) == 0;
         for (int d = 0; d < nr - 1 && ok; ++d) ok = (plan->in_red_step[d] % align) == 0;
         for (int d = 0; d < no && ok; ++d) ok = (plan->in_out_step[d] % align) == 0;

@@ -710,7 +710,8 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
         if (plan.in_out_step[plan.out_ndim - 1] != (int64_t)sizeof(In)) return 0;
         p.lsplit_bits = (uint32_t)plan.local_split_bits;
         const uint64_t per_block = (uint64_t)kRedBlock >> p.lsplit_bits;
-        uint64_t grid = ((plan.out_total + V - 1) / V + per_block - 1) / per_block;
+        const uint64_t groups = (uint64_t)(p.n_out / p.out_inner) * (((uint64_t)p.out_inner + V - 1) / V);
+        uint64_t grid = (groups + per_block - 1) / per_block;
         if (plan.n_split > 1) {
             // The axis is cut across blocks as well: accumulators to scratch, a second launch folds them.
             if (p.lsplit_bits == 0 || grid > 65535) return 0;

@@ -476,9 +476,10 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
     const unsigned CPB = 1u << cbits;
     const unsigned c = threadIdx.x & (CPB - 1);
     const unsigned s = threadIdx.x >> cbits;
-    // (the outputs need not be a whole number of vectors when they span one dimension: the last group
-    // is pulled back to the last VEC outputs and stores only those the group before it does not)
-    const uint32_t groups = (p.n_out + VEC - 1) / VEC;
+    // (the inner output dimension need not be a whole number of vectors: its last group is pulled
+    // back to its last VEC outputs and stores only those the group before it does not)
+    const uint32_t gpo = (p.out_inner + VEC - 1) / VEC;            // groups per position of the outer output dimension
+    const uint32_t groups = (p.n_out / p.out_inner) * gpo;
     const uint32_t n_cb = (groups + CPB - 1) / CPB;
     // this block's stretch of the axis, then this lane's part of it
     uint64_t b0 = 0, b1 = p.n;
@@ -498,10 +499,12 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
     for (uint32_t cb = blockIdx.x; cb < n_cb; cb += gridDim.x) {
         const uint32_t g = cb * CPB + c;
         const bool ok = g < groups;
-        const uint32_t own0 = (ok ? g : groups - 1) * VEC;           // the group's first output
-        const uint32_t i_out0 = own0 + VEC <= p.n_out ? own0 : p.n_out - VEC;  // where its vector starts
-        uint32_t o0, o1;
-        rs_split_out(p, i_out0, o0, o1);
+        const uint32_t gg = ok ? g : groups - 1;
+        const uint32_t o0 = p.out_inner == p.n_out ? 0u : gg / gpo;
+        const uint32_t own1 = (gg - o0 * gpo) * VEC;
+        const uint32_t o1 = own1 + VEC <= p.out_inner ? own1 : p.out_inner - VEC;  // where the group's vector starts
+        const uint32_t own0 = o0 * p.out_inner + own1;                // the group's first output
+        const uint32_t i_out0 = o0 * p.out_inner + o1;
         const int64_t in_off = (int64_t)o0 * p.in_step[0] + (int64_t)o1 * p.in_step[1];
         const char* base = p.in + in_off;
         Acc acc[VEC];

@@ -123,6 +123,27 @@ def test_matrices_with_rows_of_an_odd_length_and_a_second_operand(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+def test_stacked_matrices_with_rows_of_an_odd_length_and_a_second_operand(tname, dt):
+    """Three dimensions, the innermost not a whole number of vectors: a contiguous array (op) an operand
+    that repeats along the first or the second dimension (or both), on either side, into a typed
+    result and, for comparisons, into Bit."""
+    import cumo_amd
+    rng = np.random.default_rng(505)
+    cls = cls_of(tname)
+    for (O, M, Cn) in [(3, 37, 65), (7, 5, 1023), (2, 130, 259), (5, 3, 70001), (64, 2, 67)]:
+        a = (rng.integers(-8, 8, size=(O, M, Cn)) / 4.0).astype(dt)
+        da = cls.cast(a)
+        for bshape in [(M, 1), (O, 1, Cn), (1, M, Cn), (O, 1, 1), (1, 1, Cn), (O, M, 1)]:
+            b = (rng.integers(-8, 8, size=bshape) / 4.0).astype(dt)
+            db = cls.cast(b)
+            for name, f in (("add", lambda x, y: x + y), ("sub", lambda x, y: x - y)):
+                assert_bits_equal(f(da, db).to_numpy(), oracle.binary(name, a, b), "%s %s %s" % ((O, M, Cn), name, bshape))
+                assert_bits_equal(f(db, da).to_numpy(), oracle.binary(name, b, a), "%s %s %s (swapped)" % ((O, M, Cn), name, bshape))
+            assert ((da > db).to_numpy() == (a > b)).all(), ((O, M, Cn), bshape)
+            assert ((db >= da).to_numpy() == (b >= a)).all(), ((O, M, Cn), bshape)
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 def test_transposed_operands_whose_extents_are_not_whole_vectors(tname, dt):
     """Transposed views go through LDS tiles with 128-bit accesses on both sides; neither extent need be
     a whole number of vectors, and rows need their element's alignment only: extents of 4k + 1, 2, 3,

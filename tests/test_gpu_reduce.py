@@ -248,7 +248,9 @@ def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((700, 24), 0), ((3, 700, 24), 1), ((40000, 8), 0), ((2, 5000, 3), 1), ((130, 1024), 0),
                                         ((3000, 1000), 0), ((4096, 520), 0), ((2, 2100, 516), 1), ((3000, 1001), 0), ((700, 4095), 0),
-                                        ((40, 70001), 0), ((5000, 259), 0)])
+                                        ((40, 70001), 0), ((5000, 259), 0),
+                                        ((3, 700, 67), 1), ((5, 64, 1023), 1), ((2, 2100, 517), 1), ((9, 130, 259), 1), ((64, 40, 131), 1),
+                                        ((300, 20, 33), 1)])
 def test_few_outputs_across_memory_share_the_axis_inside_a_block(tname, dt, shape, axis):
     """The column kernel with the reduce axis cut inside the block (and, for the long ones, across
     blocks as well): ties resolve to the lowest index across the parts, NaN rules, both results of
@@ -288,9 +290,10 @@ def test_few_outputs_across_memory_share_the_axis_inside_a_block(tname, dt, shap
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
-@pytest.mark.parametrize("shape,axis", [((7, 1027), 1), ((1, 4099), 1), ((2051,), None), ((3, 5, 1030), 2), ((300001,), None), ((40, 20011), 1)])
+@pytest.mark.parametrize("shape,axis", [((7, 1027), 1), ((1, 4099), 1), ((2051,), None), ((3, 5, 1030), 2), ((300001,), None), ((40, 20011), 1),
+                                        ((64, 1023), 1), ((9, 5, 131), 2), ((33, 67), 1), ((5, 33), 1)])
 def test_runs_that_end_in_part_of_a_vector(tname, dt, shape, axis):
-    """A contiguous reduce axis of 256 vectors or more that is not a whole number of vectors: the
+    """A contiguous reduce axis of 16 vectors or more that is not a whole number of vectors: the
     lean row kernels take its whole vectors and one lane folds the last one to three elements.
     What decides the answer is put into those last elements: the extreme, a tie with an earlier
     element (the earlier index wins), the zero of the other sign (the one that came first wins),
