@@ -57,6 +57,61 @@ __global__ __launch_bounds__(kBlock) void bit_contiguous_kernel(const CUMO_BIT_D
     }
 }
 
+// 128 bits of `a` from bit position q on (q >= 0): one 128-bit load from a 4-byte boundary, and the
+// word after it when q is not at the start of a word. The caller has checked that all of it is there.
+template <bool NT>
+__device__ __forceinline__ uint4 bits128_at(const CUMO_BIT_DIGIT* a, uint64_t q) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint64_t w = q >> 5;
+    const unsigned sh = (unsigned)(q & 31);
+    const u4 x = NT ? __builtin_nontemporal_load(reinterpret_cast<const u4*>(a + w)) : *reinterpret_cast<const u4*>(a + w);
+    if (sh == 0) return make_uint4(x.x, x.y, x.z, x.w);
+    const uint32_t e = a[w + 4];
+    const unsigned up = 32 - sh;
+    return make_uint4((x.x >> sh) | (x.y << up), (x.y >> sh) | (x.z << up), (x.z >> sh) | (x.w << up), (x.w >> sh) | (e << up));
+}
+
+// The same, four output words per lane. The output vectors are the 16-byte aligned ones (`lead` = words
+// between the boundary before a3 and a3); a vector whose words all lie inside the run away from its
+// first and last word goes as a whole, the words of the others one by one as above.
+template <int OP, bool BINARY, bool NT>
+__global__ __launch_bounds__(kBlock) void bit_contiguous_vec_kernel(const CUMO_BIT_DIGIT* a1, uint64_t p1, const CUMO_BIT_DIGIT* a2, uint64_t p2,
+                                                                    CUMO_BIT_DIGIT* a3, uint64_t p3, uint64_t n, unsigned lead) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint64_t nw1 = (p1 + n + 31) >> 5, nw2 = (p2 + n + 31) >> 5, nw3 = (p3 + n + 31) >> 5;
+    const uint64_t nvec = (nw3 + lead + 3) >> 2;
+    const uint64_t endbit = p3 + n;
+    for (uint64_t v = (uint64_t)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += (uint64_t)gridDim.x * kBlock) {
+        const int64_t w0 = (int64_t)(v << 2) - (int64_t)lead;
+        if (w0 >= 1 && (uint64_t)w0 + 4 <= nw3 - 1) {
+            const uint64_t e0 = ((uint64_t)w0 << 5) - p3;
+            const uint4 x = bits128_at<NT>(a1, e0 + p1);
+            uint4 y = make_uint4(0u, 0u, 0u, 0u);
+            if (BINARY) y = bits128_at<NT>(a2, e0 + p2);
+            u4 z;
+            z.x = bit_apply<OP>(x.x, y.x);
+            z.y = bit_apply<OP>(x.y, y.y);
+            z.z = bit_apply<OP>(x.z, y.z);
+            z.w = bit_apply<OP>(x.w, y.w);
+            if (NT) __builtin_nontemporal_store(z, reinterpret_cast<u4*>(a3 + w0));
+            else *reinterpret_cast<u4*>(a3 + w0) = z;
+            continue;
+        }
+        for (int64_t ww = w0 < 0 ? 0 : w0; ww < w0 + 4 && (uint64_t)ww < nw3; ++ww) {
+            const uint64_t w = (uint64_t)ww;
+            const int64_t e0 = (int64_t)(w << 5) - (int64_t)p3;
+            const uint32_t x = bits_at(a1, e0 + (int64_t)p1, nw1);
+            const uint32_t y = BINARY ? bits_at(a2, e0 + (int64_t)p2, nw2) : 0u;
+            const uint32_t z = bit_apply<OP>(x, y);
+            const unsigned lo = (w == 0) ? (unsigned)p3 : 0u;
+            const unsigned hi = ((w + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (w << 5));
+            const uint32_t mask = low_bits(hi) & ~low_bits(lo);
+            if (mask == 0xffffffffu) a3[w] = z;
+            else a3[w] = (z & mask) | (a3[w] & ~mask);
+        }
+    }
+}
+
 template <int OP, bool BINARY>
 __global__ __launch_bounds__(kBlock) void bit_generic_kernel(cumo_na_bit_iarray_stridx_t a1, cumo_na_bit_iarray_stridx_t a2,
                                                              cumo_na_bit_iarray_stridx_t a3, BitNd nd) {
@@ -67,12 +122,205 @@ __global__ __launch_bounds__(kBlock) void bit_generic_kernel(cumo_na_bit_iarray_
     }
 }
 
+// Views whose innermost dimension runs along the bits (step 1) in every operand and that use no index
+// array: a lane takes one word of one result row. nw1 / nw2: words of a1 / a2 up to the last bit the
+// view reaches (nothing past them is read). A row's first and last word may be shared with its
+// neighbours in memory, so those two are changed with atomics; the words between them belong to the
+// row alone.
+struct BitRowsOp {
+    int ndim;
+    uint64_t items, chunks, inner;   // chunks: result words a row can span
+    uint64_t shape[kMaxDim];
+    int64_t s1[kMaxDim], s2[kMaxDim], s3[kMaxDim];  // bit steps of the outer dimensions
+    uint64_t nw1, nw2;
+};
+
+template <int OP, bool BINARY>
+__global__ __launch_bounds__(kBlock) void bit_rows_kernel(const CUMO_BIT_DIGIT* a1, uint64_t p1, const CUMO_BIT_DIGIT* a2, uint64_t p2,
+                                                          CUMO_BIT_DIGIT* a3, uint64_t p3, BitRowsOp nd) {
+    for (uint64_t item = (uint64_t)blockIdx.x * kBlock + threadIdx.x; item < nd.items; item += (uint64_t)gridDim.x * kBlock) {
+        uint64_t q = item / nd.chunks;
+        const uint64_t k = item - q * nd.chunks;
+        int64_t q1 = (int64_t)p1, q2 = (int64_t)p2, q3 = (int64_t)p3;
+        for (int d = nd.ndim - 2; d >= 0; --d) {
+            uint64_t i = q;
+            if (d > 0) {
+                const uint64_t up = q / nd.shape[d];
+                i = q - up * nd.shape[d];
+                q = up;
+            }
+            q1 += (int64_t)i * nd.s1[d];
+            q2 += (int64_t)i * nd.s2[d];
+            q3 += (int64_t)i * nd.s3[d];
+        }
+        const uint64_t w_first = (uint64_t)q3 >> 5, w_last = ((uint64_t)q3 + nd.inner - 1) >> 5;
+        const uint64_t w = w_first + k;
+        if (w > w_last) continue;
+        const int64_t e0 = (int64_t)(w << 5) - q3;  // the row's element at bit 0 of this word (negative in its first word)
+        const uint32_t x = bits_at(a1, q1 + e0, nd.nw1);
+        const uint32_t y = BINARY ? bits_at(a2, q2 + e0, nd.nw2) : 0u;
+        const uint32_t z = bit_apply<OP>(x, y);
+        const unsigned lo = (w == w_first) ? (unsigned)((uint64_t)q3 & 31) : 0u;
+        const unsigned hi = (w == w_last) ? (unsigned)(((uint64_t)q3 + nd.inner - 1) & 31) + 1u : 32u;
+        const uint32_t mask = low_bits(hi) & ~low_bits(lo);
+        if (w != w_first && w != w_last) {
+            a3[w] = z;
+        } else {
+            atomicAnd(&a3[w], ~mask);
+            atomicOr(&a3[w], z & mask);
+        }
+    }
+}
+
+// launches the row form when the operands allow it; false: the caller uses the bit-by-bit kernel
+template <int OP, bool BINARY>
+bool bit_rows_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_bit_iarray_stridx_t* a3, cumo_na_indexer_t* indexer) {
+    const int n = indexer->ndim;
+    if (n < 2 || n > kMaxDim || force_wide_indices() || indexer->shape[n - 1] < 32) return false;
+    cumo_na_bit_iarray_stridx_t* ops[3] = {a1, BINARY ? a2 : a1, a3};
+    BitRowsOp nd;
+    std::memset(&nd, 0, sizeof(nd));
+    uint64_t reach[3];
+    for (int j = 0; j < 3; ++j) {
+        int64_t lowest = (int64_t)ops[j]->pos, highest = (int64_t)ops[j]->pos;
+        for (int d = 0; d < n; ++d) {
+            if (!CUMO_SDX_IS_STRIDE(ops[j]->stridx[d])) return false;
+            const int64_t st = (int64_t)CUMO_SDX_GET_STRIDE(ops[j]->stridx[d]);
+            if (d == n - 1 && st != 1) return false;
+            const int64_t span = st * (int64_t)(indexer->shape[d] - 1);
+            if (span < 0) lowest += span;
+            else highest += span;
+        }
+        if (lowest < 0) return false;  // (bit positions are computed unsigned)
+        // a result row that lies across another's words in memory (a repeated or reversed-overlapping view) is not taken
+        if (j == 2) {
+            for (int d = 0; d < n - 1; ++d) {
+                const int64_t st = (int64_t)CUMO_SDX_GET_STRIDE(a3->stridx[d]);
+                if ((st < 0 ? -st : st) < (int64_t)indexer->shape[n - 1]) return false;
+            }
+        }
+        reach[j] = ((uint64_t)highest + 32) >> 5;
+    }
+    nd.ndim = n;
+    nd.inner = indexer->shape[n - 1];
+    nd.chunks = (nd.inner + 31) / 32 + 1;
+    nd.items = nd.chunks;
+    for (int d = 0; d < n; ++d) {
+        nd.shape[d] = indexer->shape[d];
+        if (d < n - 1) {
+            nd.items *= indexer->shape[d];
+            nd.s1[d] = (int64_t)CUMO_SDX_GET_STRIDE(ops[0]->stridx[d]);
+            nd.s2[d] = (int64_t)CUMO_SDX_GET_STRIDE(ops[1]->stridx[d]);
+            nd.s3[d] = (int64_t)CUMO_SDX_GET_STRIDE(ops[2]->stridx[d]);
+        }
+    }
+    nd.nw1 = reach[0];
+    nd.nw2 = reach[1];
+    hipLaunchKernelGGL((bit_rows_kernel<OP, BINARY>), dim3(grid_for(nd.items, kNumCU * 32)), dim3(kBlock), 0, current_stream(),
+                       (const CUMO_BIT_DIGIT*)ops[0]->ptr, (uint64_t)ops[0]->pos, (const CUMO_BIT_DIGIT*)ops[1]->ptr, (uint64_t)ops[1]->pos, a3->ptr,
+                       (uint64_t)a3->pos, nd);
+    cumo_cuda_runtime_check_kernel_launch();
+    return true;
+}
+
 template <class T>
 __global__ __launch_bounds__(kBlock) void store_bit_kernel(cumo_na_iarray_stridx_t dst, cumo_na_bit_iarray_stridx_t src, BitNd nd) {
     for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < nd.total; i += (uint64_t)gridDim.x * kBlock) {
         const uint32_t x = load_bit(src.ptr, src.pos + (uint64_t)stridx_offset(src.stridx, nd, i));
         *reinterpret_cast<T*>(dst.ptr + stridx_offset(dst.stridx, nd, i)) = (T)x;
     }
+}
+
+// Bit -> number where both run along the innermost dimension (bit step 1, element step sizeof(T)) and
+// no dimension goes through an index array: a lane takes four neighbouring elements of a row, reads the
+// one or two words that hold their bits and stores them as 128-bit vectors (which need the element's
+// alignment only). s_src (bits) and s_dst (bytes) are the steps of the outer dimensions.
+struct BitRowsNd {
+    int ndim;
+    uint64_t items, chunks;          // work items; chunks of four elements in a row
+    uint64_t shape[kMaxDim];
+    int64_t s_src[kMaxDim], s_dst[kMaxDim];
+};
+
+template <class T, bool NT>
+__global__ __launch_bounds__(kBlock) void store_bit_rows_kernel(char* dst, const CUMO_BIT_DIGIT* src, uint64_t pos, BitRowsNd nd) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint64_t inner = nd.shape[nd.ndim - 1];
+    for (uint64_t item = (uint64_t)blockIdx.x * kBlock + threadIdx.x; item < nd.items; item += (uint64_t)gridDim.x * kBlock) {
+        uint64_t c = item;
+        int64_t bit = (int64_t)pos, off = 0;
+        if (nd.ndim > 1) {
+            uint64_t q = item / nd.chunks;
+            c = item - q * nd.chunks;
+            for (int d = nd.ndim - 2; d >= 0; --d) {
+                uint64_t k = q;
+                if (d > 0) {
+                    const uint64_t q2 = q / nd.shape[d];
+                    k = q - q2 * nd.shape[d];
+                    q = q2;
+                }
+                bit += (int64_t)k * nd.s_src[d];
+                off += (int64_t)k * nd.s_dst[d];
+            }
+        }
+        const uint64_t e0 = c * 4;
+        const unsigned cnt = inner - e0 >= 4 ? 4u : (unsigned)(inner - e0);
+        const uint64_t b0 = (uint64_t)bit + e0;
+        const unsigned sh = (unsigned)(b0 & 31);
+        uint32_t x = src[b0 >> 5] >> sh;
+        if (sh + cnt > 32) x |= src[(b0 >> 5) + 1] << (32 - sh);
+        T* out = reinterpret_cast<T*>(dst + off) + e0;
+        if (cnt == 4) {
+            union V {
+                u4 q[sizeof(T) / 4];
+                T v[4];
+                __device__ V() {}
+            } t;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) t.v[j] = (T)((x >> j) & 1u);
+#pragma unroll
+            for (int k = 0; k < (int)(sizeof(T) / 4); ++k) {
+                if (NT) __builtin_nontemporal_store(t.q[k], reinterpret_cast<u4*>(out) + k);
+                else reinterpret_cast<u4*>(out)[k] = t.q[k];
+            }
+        } else {
+            for (unsigned j = 0; j < cnt; ++j) out[j] = (T)((x >> j) & 1u);
+        }
+    }
+}
+
+// launches the row form when the operands allow it; false: the caller uses the element-wise kernel
+template <class T>
+bool store_bit_rows_launch(cumo_na_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_indexer_t* indexer) {
+    const int n = indexer->ndim;
+    if (n < 1 || n > kMaxDim || force_wide_indices()) return false;
+    for (int d = 0; d < n; ++d)
+        if (!CUMO_SDX_IS_STRIDE(a1->stridx[d]) || !CUMO_SDX_IS_STRIDE(a2->stridx[d])) return false;
+    if (CUMO_SDX_GET_STRIDE(a1->stridx[n - 1]) != (ssize_t)sizeof(T) || CUMO_SDX_GET_STRIDE(a2->stridx[n - 1]) != 1) return false;
+    if (((uintptr_t)a1->ptr % alignof(T)) != 0 || indexer->shape[n - 1] < 16) return false;
+    BitRowsNd nd;
+    std::memset(&nd, 0, sizeof(nd));
+    nd.ndim = n;
+    nd.chunks = (indexer->shape[n - 1] + 3) / 4;
+    nd.items = nd.chunks;
+    int64_t lowest = 0;
+    for (int d = 0; d < n; ++d) {
+        nd.shape[d] = indexer->shape[d];
+        if (d < n - 1) {
+            nd.items *= indexer->shape[d];
+            nd.s_src[d] = (int64_t)CUMO_SDX_GET_STRIDE(a2->stridx[d]);
+            nd.s_dst[d] = (int64_t)CUMO_SDX_GET_STRIDE(a1->stridx[d]);
+            if ((nd.s_dst[d] % (int64_t)alignof(T)) != 0) return false;
+            if (nd.s_src[d] < 0) lowest += nd.s_src[d] * (int64_t)(indexer->shape[d] - 1);
+        }
+    }
+    if ((int64_t)a2->pos + lowest < 0) return false;  // (bit positions are computed unsigned)
+    const bool nt = stream_past_caches((uint64_t)indexer->total_size * sizeof(T));
+    const dim3 g(grid_for(nd.items, kNumCU * 32)), b(kBlock);
+    if (nt) hipLaunchKernelGGL((store_bit_rows_kernel<T, true>), g, b, 0, current_stream(), a1->ptr, (const CUMO_BIT_DIGIT*)a2->ptr, (uint64_t)a2->pos, nd);
+    else hipLaunchKernelGGL((store_bit_rows_kernel<T, false>), g, b, 0, current_stream(), a1->ptr, (const CUMO_BIT_DIGIT*)a2->ptr, (uint64_t)a2->pos, nd);
+    cumo_cuda_runtime_check_kernel_launch();
+    return true;
 }
 
 // ---- counting -------------------------------------------------------------------
@@ -199,6 +447,18 @@ template <int OP, bool BINARY>
 void launch_contiguous(CUMO_BIT_DIGIT* a1, size_t p1, CUMO_BIT_DIGIT* a2, size_t p2, CUMO_BIT_DIGIT* a3, size_t p3, uint64_t n) {
     if (n == 0) return;
     const uint64_t nw3 = (p3 + n + 31) >> 5;
+    if (nw3 >= 64 && p1 < 32 && p2 < 32 && p3 < 32) {
+        const unsigned lead = (unsigned)(((uintptr_t)a3 % 16) / sizeof(CUMO_BIT_DIGIT));
+        const dim3 g(grid_for((nw3 + lead + 3) / 4, kNumCU * 16)), b(kBlock);
+        if (stream_past_caches(nw3 * 4 * (BINARY ? 3 : 2)))
+            hipLaunchKernelGGL((bit_contiguous_vec_kernel<OP, BINARY, true>), g, b, 0, current_stream(), a1, (uint64_t)p1, a2, (uint64_t)p2, a3,
+                               (uint64_t)p3, n, lead);
+        else
+            hipLaunchKernelGGL((bit_contiguous_vec_kernel<OP, BINARY, false>), g, b, 0, current_stream(), a1, (uint64_t)p1, a2, (uint64_t)p2, a3,
+                               (uint64_t)p3, n, lead);
+        cumo_cuda_runtime_check_kernel_launch();
+        return;
+    }
     hipLaunchKernelGGL((bit_contiguous_kernel<OP, BINARY>), dim3(grid_for(nw3)), dim3(kBlock), 0, current_stream(), a1, (uint64_t)p1, a2,
                        (uint64_t)p2, a3, (uint64_t)p3, n);
     cumo_cuda_runtime_check_kernel_launch();
@@ -219,6 +479,7 @@ void launch_generic(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t
                                       BINARY ? a2->pos % 32 : 0, a3->ptr + a3->pos / 32, a3->pos % 32, indexer->total_size);
         return;
     }
+    if (bit_rows_launch<OP, BINARY>(a1, a2, a3, indexer)) return;
     BitNd nd = make_nd(indexer);
     hipLaunchKernelGGL((bit_generic_kernel<OP, BINARY>), dim3(grid_for(nd.total)), dim3(kBlock), 0, current_stream(), *a1,
                        BINARY ? *a2 : *a1, *a3, nd);
@@ -286,13 +547,42 @@ __global__ __launch_bounds__(kBlock) void bit_count_nd_kernel(BitCountNd p) {
         if (s_last == 1) {
             const uint64_t p1 = (uint64_t)bit, endbit = p1 + p.n_last;
             const uint64_t w0 = p1 >> 5, w1 = (endbit + 31) >> 5;
-            for (uint64_t w = w0 + lane; w < w1; w += 64) {
-                uint32_t x = p.in[w];
-                if (COUNT_FALSE) x = ~x;
-                const unsigned lo = (w == w0) ? (unsigned)(p1 & 31) : 0u;
-                const unsigned hi = ((w + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (w << 5));
-                x &= low_bits(hi) & ~low_bits(lo);
-                c += (uint64_t)__popc(x);
+            // four words per lane (a 128-bit load from a 4-byte boundary), two such loads in flight
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            for (uint64_t wa = w0 + 4 * lane; wa < w1; wa += 512) {
+                u4 t[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint64_t w = wa + 256 * u;
+                    if (w + 4 <= w1) {
+                        t[u] = *reinterpret_cast<const u4*>(p.in + w);
+                    } else {
+                        t[u].x = w < w1 ? p.in[w] : 0u;
+                        t[u].y = w + 1 < w1 ? p.in[w + 1] : 0u;
+                        t[u].z = w + 2 < w1 ? p.in[w + 2] : 0u;
+                        t[u].w = 0u;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint64_t w = wa + 256 * u;
+                    const uint32_t xs[4] = {t[u].x, t[u].y, t[u].z, t[u].w};
+                    if (w > w0 && w + 4 < w1) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) c += (uint64_t)__popc(COUNT_FALSE ? ~xs[j] : xs[j]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const uint64_t k = w + j;
+                            if (k >= w1) continue;
+                            uint32_t x = COUNT_FALSE ? ~xs[j] : xs[j];
+                            const unsigned lo = (k == w0) ? (unsigned)(p1 & 31) : 0u;
+                            const unsigned hi = ((k + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (k << 5));
+                            x &= low_bits(hi) & ~low_bits(lo);
+                            c += (uint64_t)__popc(x);
+                        }
+                    }
+                }
             }
         } else {
             for (uint64_t i = lane; i < p.n_last; i += 64) {
@@ -310,6 +600,125 @@ __global__ __launch_bounds__(kBlock) void bit_count_nd_kernel(BitCountNd p) {
     }
 }
 
+// Counts down columns: the kept dimension that runs along the bits (step 1) has `cols` outputs, the one
+// reduced dimension steps `s_red` bits, and an optional outer kept dimension steps s_outer bits /
+// o_outer bytes. A block of 16 waves has 64 x 32 neighbouring columns of one outer position and a
+// stretch of the rows, a sixteenth of it per wave; a lane owns 32 columns: it reads their word row by
+// row (two words where the row does not start on a word) and counts every column in byte-wide counters,
+// four to a register (column j of the 32 sits in counter j / 8 of register j % 8), moved to 32-bit
+// counters before a byte could overflow. The waves add their totals up in LDS, and the block adds the
+// sums onto the 64-bit results, one atomic per column that has any.
+constexpr int kCountColsBlock = 1024;
+
+struct BitCountCols {
+    const CUMO_BIT_DIGIT* in;
+    char* out;
+    uint64_t pos;
+    uint32_t cols, chunks, chunk_blocks, rows, rows_per_wave, row_parts, n_outer;
+    int64_t s_red, s_outer, o_outer, o_col;
+};
+
+template <bool COUNT_FALSE>
+__global__ __launch_bounds__(kCountColsBlock) void bit_count_cols_kernel(BitCountCols p) {
+    __shared__ uint32_t sums[32][64];
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t cb = blockIdx.x % p.chunk_blocks;
+    const uint32_t b2 = blockIdx.x / p.chunk_blocks;
+    const uint32_t part = b2 % p.row_parts;
+    const uint32_t o = b2 / p.row_parts;
+    for (unsigned i = threadIdx.x; i < 32 * 64; i += kCountColsBlock) (&sums[0][0])[i] = 0u;
+    __syncthreads();
+    const uint32_t c = cb * 64u + lane;
+    if (c < p.chunks) {
+        const uint64_t first_row = ((uint64_t)part * 16 + wave) * p.rows_per_wave;
+        const uint32_t r0 = first_row < p.rows ? (uint32_t)first_row : p.rows;
+        const uint32_t r1 = r0 + p.rows_per_wave < p.rows ? r0 + p.rows_per_wave : p.rows;
+        const unsigned cnt = p.cols - c * 32u >= 32u ? 32u : p.cols - c * 32u;
+        const uint32_t keep = low_bits(cnt);
+        const int64_t first = (int64_t)p.pos + (int64_t)o * p.s_outer + (int64_t)c * 32;
+        uint32_t total[32];
+#pragma unroll
+        for (int j = 0; j < 32; ++j) total[j] = 0u;
+        for (uint32_t ra = r0; ra < r1; ra += 252) {
+            const uint32_t rb = ra + 252 < r1 ? ra + 252 : r1;
+            uint32_t bytes[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) bytes[k] = 0u;
+            for (uint32_t r = ra; r < rb; r += 4) {
+                uint32_t x[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t rr = r + u < rb ? r + u : rb - 1;
+                    const uint64_t q = (uint64_t)(first + (int64_t)rr * p.s_red);
+                    const unsigned sh = (unsigned)(q & 31);
+                    uint32_t w = p.in[q >> 5] >> sh;
+                    if (sh + cnt > 32) w |= p.in[(q >> 5) + 1] << (32 - sh);
+                    if (COUNT_FALSE) w = ~w;
+                    x[u] = (r + u < rb) ? (w & keep) : 0u;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) bytes[k] += (x[u] >> k) & 0x01010101u;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 32; ++j) total[j] += (bytes[j & 7] >> (8 * (j >> 3))) & 0xffu;
+        }
+        if (r0 < r1) {
+#pragma unroll
+            for (int j = 0; j < 32; ++j)
+                if (total[j] != 0u) atomicAdd(&sums[j][lane], total[j]);
+        }
+    }
+    __syncthreads();
+    for (unsigned i = threadIdx.x; i < 32 * 64; i += kCountColsBlock) {
+        // consecutive threads, consecutive columns
+        const unsigned l = i >> 5, j = i & 31;
+        const uint32_t col = (cb * 64u + l) * 32u + j;
+        const uint32_t v = sums[j][l];
+        if (col < p.cols && v != 0u)
+            atomicAdd(reinterpret_cast<unsigned long long*>(p.out + (int64_t)o * p.o_outer + (int64_t)col * p.o_col), (unsigned long long)v);
+    }
+}
+
+// launches the column form when the loop allows it; false: the caller uses the general kernel
+bool bit_count_cols_launch(const cumo_hip_bit_count_nd_t* d) {
+    if (d->red_ndim != 1 || d->out_ndim < 1 || d->out_ndim > 2 || force_wide_indices()) return false;
+    const int L = d->out_ndim - 1;
+    if (d->in_out_step[L] != 1 || d->in_red_step[0] <= 0 || d->out_shape[L] < 64 || d->red_shape[0] < 2) return false;
+    if (d->out_shape[L] >= 0x7fffffffull || d->red_shape[0] >= 0x7fffffffull) return false;
+    if (L == 1 && (d->in_out_step[0] < 0 || d->out_shape[0] >= 0x10000ull)) return false;
+    BitCountCols p;
+    std::memset(&p, 0, sizeof(p));
+    p.in = d->in;
+    p.out = d->out;
+    p.pos = d->pos;
+    p.cols = (uint32_t)d->out_shape[L];
+    p.chunks = (p.cols + 31u) / 32u;
+    p.chunk_blocks = (p.chunks + 63u) / 64u;
+    p.rows = (uint32_t)d->red_shape[0];
+    p.n_outer = L == 1 ? (uint32_t)d->out_shape[0] : 1u;
+    p.s_red = d->in_red_step[0];
+    p.s_outer = L == 1 ? d->in_out_step[0] : 0;
+    p.o_outer = L == 1 ? d->out_step[0] : 0;
+    p.o_col = d->out_step[L];
+    // two blocks for every compute unit where the rows allow it, stretches of 32 rows or more per wave
+    const uint64_t across = (uint64_t)p.chunk_blocks * p.n_outer;
+    uint64_t parts = ((uint64_t)kNumCU * 2 + across - 1) / across;
+    const uint64_t most = ((uint64_t)p.rows + 32 * 16 - 1) / (32 * 16);
+    if (parts > most) parts = most;
+    if (parts < 1) parts = 1;
+    p.rows_per_wave = (uint32_t)(((uint64_t)p.rows + parts * 16 - 1) / (parts * 16));
+    p.row_parts = (uint32_t)(((uint64_t)p.rows + (uint64_t)p.rows_per_wave * 16 - 1) / ((uint64_t)p.rows_per_wave * 16));
+    const uint64_t blocks = across * p.row_parts;
+    if (blocks > 0x7fffffffull) return false;
+    const dim3 g((unsigned)blocks), b(kCountColsBlock);
+    if (d->count_false) hipLaunchKernelGGL((bit_count_cols_kernel<true>), g, b, 0, current_stream(), p);
+    else hipLaunchKernelGGL((bit_count_cols_kernel<false>), g, b, 0, current_stream(), p);
+    cumo_cuda_runtime_check_kernel_launch();
+    return true;
+}
 
 }  // namespace
 
@@ -362,6 +771,7 @@ CUMO_DEF_BIT_COUNT(count_false, true)
     extern "C" void cumo_iter_##t##_store_bit_kernel_launch(cumo_na_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2,     \
                                                             cumo_na_indexer_t* indexer) {                                     \
         if (indexer->total_size == 0) return;                                                                                 \
+        if (store_bit_rows_launch<c>(a1, a2, indexer)) return;                                                                \
         BitNd nd = make_nd(indexer);                                                                                          \
         hipLaunchKernelGGL((store_bit_kernel<c>), dim3(grid_for(nd.total)), dim3(kBlock), 0, current_stream(), *a1, *a2, nd); \
         cumo_cuda_runtime_check_kernel_launch();                                                                              \
@@ -398,7 +808,7 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
     pos += back * 32;
     const uint64_t vecs = ((pos + n + 31) / 32 + 3) / 4 - (pos / 32) / 4;
     uint64_t grid = (vecs + kBlock - 1) / kBlock;
-    if (grid > 128) grid = 128;  // every block ends in one returning atomic on the same word
+    if (grid > 512) grid = 512;  // every block ends in one returning atomic on the same word
     if (grid == 0) grid = 1;
     if (count_false)
         hipLaunchKernelGGL((bit_count_words_store_kernel<true>), dim3((unsigned)grid), dim3(kBlock), 0, st, (const CUMO_BIT_DIGIT*)a, (uint64_t)pos, n,
@@ -412,6 +822,7 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
 
 extern "C" void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* d) {
     if (!d) return;
+    if (bit_count_cols_launch(d)) return;
     BitCountNd p;
     std::memset(&p, 0, sizeof(p));
     p.out_ndim = d->out_ndim;

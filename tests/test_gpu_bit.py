@@ -133,3 +133,111 @@ def test_count_along_axes_in_one_launch_matches_numpy():
                     assert (np.asarray(b[key].count_true(axis=ax).to_numpy()) == h[key].sum(axis=ax, dtype=np.uint64)).all(), (shape, key, ax)
             for ax in (0, 1):
                 assert (np.asarray(b.transpose().count_true(axis=ax).to_numpy()) == h.T.sum(axis=ax, dtype=np.uint64)).all()
+
+
+def test_rows_of_bits_in_views_word_by_word():
+    """Logical operations and copies on views whose rows run along the bits but do not form one run
+    (windows that start inside a word, rows that share their first and last word with neighbours,
+    skipped and reversed rows, three dimensions): a lane takes a word of a result row. Storing into
+    such a view leaves every bit around it as it was."""
+    import cumo_amd
+    rng = np.random.default_rng(611)
+    for shape in [(70, 131), (5, 4099), (300, 33), (9, 7, 67), (64, 64), (33, 1000)]:
+        ha = rng.integers(0, 2, size=shape).astype(np.uint8)
+        hb = rng.integers(0, 2, size=shape).astype(np.uint8)
+        a, b = cumo_amd.Bit.cast(ha), cumo_amd.Bit.cast(hb)
+        keys = [(Ellipsis, slice(1, None)), (Ellipsis, slice(None, -1)), (slice(None, None, 2), Ellipsis, slice(3, -5)),
+                (slice(None, None, -1), Ellipsis, slice(2, None)), (slice(1, None), Ellipsis, slice(0, 40))]
+        for ka in keys:
+            for kb in keys:
+                va, vb = ha[ka], hb[kb]
+                if va.shape != vb.shape:
+                    continue
+                da, db = a[ka], b[kb]
+                assert ((da & db).to_numpy() == oracle.bit_binary("and", va, vb)).all(), (shape, ka, kb)
+                assert ((da ^ db).to_numpy() == oracle.bit_binary("xor", va, vb)).all(), (shape, ka, kb)
+                assert (da.eq(db).to_numpy() == oracle.bit_binary("eq", va, vb)).all(), (shape, ka, kb)
+            assert ((~a[ka]).to_numpy() == oracle.bit_binary("not", ha[ka])).all(), (shape, ka)
+            assert (a[ka].copy().to_numpy() == ha[ka]).all(), (shape, ka)
+        # into a window of an existing array
+        for key, src_key in (((Ellipsis, slice(1, None)), (Ellipsis, slice(None, -1))), ((slice(1, None), Ellipsis, slice(3, 33)), (slice(None, -1), Ellipsis, slice(0, 30)))):
+            hz = rng.integers(0, 2, size=shape).astype(np.uint8)
+            z = cumo_amd.Bit.cast(hz)
+            z[key] = a[src_key]
+            hz[key] = ha[src_key]
+            assert (z.to_numpy() == hz).all(), (shape, key)
+
+
+@pytest.mark.parametrize("n", [2048, 2049, 5000, 100003, (1 << 22) + 77])
+def test_long_runs_of_bits_by_whole_vectors(n):
+    """One run (op) one run into one run, each starting at any bit of a word and any word of a 16-byte
+    vector: four result words per lane, the run's first and last words one by one."""
+    import cumo_amd
+    rng = np.random.default_rng(612 + n % 1000)
+    ha = rng.integers(0, 2, size=n + 200).astype(np.uint8)
+    hb = rng.integers(0, 2, size=n + 200).astype(np.uint8)
+    a, b = cumo_amd.Bit.cast(ha), cumo_amd.Bit.cast(hb)
+    for (oa, ob) in [(0, 0), (1, 0), (0, 31), (5, 37), (64, 3), (33, 33), (96, 127), (130, 65)]:
+        va, vb = ha[oa:oa + n], hb[ob:ob + n]
+        da, db = a[oa:oa + n], b[ob:ob + n]
+        assert ((da & db).to_numpy() == oracle.bit_binary("and", va, vb)).all(), (oa, ob)
+        assert ((da | db).to_numpy() == oracle.bit_binary("or", va, vb)).all(), (oa, ob)
+        assert (da.eq(db).to_numpy() == oracle.bit_binary("eq", va, vb)).all(), (oa, ob)
+        assert ((~da).to_numpy() == oracle.bit_binary("not", va)).all(), (oa, ob)
+        hz = rng.integers(0, 2, size=n + 200).astype(np.uint8)
+        z = cumo_amd.Bit.cast(hz)
+        z[ob:ob + n] = da                      # into a run that starts elsewhere: the bits around it stay
+        hz[ob:ob + n] = va
+        assert (z.to_numpy() == hz).all(), (oa, ob)
+        assert int(da.count_true()) == int(va.sum()) and int(db.count_false()) == int(n - vb.sum())
+
+
+def test_counts_down_columns_and_along_long_rows():
+    """count_true / count_false (and with them all? / any? along an axis) where the kept dimension runs
+    along the bits: 32 columns per lane in byte-wide counters, rows cut over lanes (more than 252 rows
+    per lane: the counters are emptied in between); and along rows of many words (128-bit loads from
+    any word). Shapes whose rows do not start on words, views, three dimensions."""
+    import cumo_amd
+    rng = np.random.default_rng(613)
+    for shape in [(300, 70), (1000, 4097), (5, 64), (40000, 65), (3, 500, 130), (2, 70000, 96), (700, 1000), (33, 32767), (70, 5000)]:
+        h = (rng.random(shape) < 0.7).astype(np.uint8)
+        h[..., 1] = 1                          # a column that is all set, one that is all clear
+        h[..., 2] = 0
+        b = cumo_amd.Bit.cast(h)
+        nd = len(shape)
+        for ax in (nd - 2, nd - 1):
+            want = h.sum(axis=ax, dtype=np.uint64)
+            assert (np.asarray(b.count_true(axis=ax).to_numpy()) == want).all(), (shape, ax)
+            assert (np.asarray(b.count_false(axis=ax).to_numpy()) == shape[ax] - want).all(), (shape, ax)
+            assert (b.all_p(axis=ax).to_numpy() == h.all(axis=ax)).all(), (shape, ax)
+            assert (b.any_p(axis=ax).to_numpy() == h.any(axis=ax)).all(), (shape, ax)
+            assert (b.none_p(axis=ax).to_numpy() == ~h.any(axis=ax)).all(), (shape, ax)
+        for key in ((Ellipsis, slice(3, None)), (Ellipsis, slice(None, None, -1), slice(1, -1)), (Ellipsis, slice(None, None, 2), slice(5, 69))):
+            v, dv = h[key], b[key]
+            for ax in (nd - 2, nd - 1):
+                assert (np.asarray(dv.count_true(axis=ax).to_numpy()) == v.sum(axis=ax, dtype=np.uint64)).all(), (shape, key, ax)
+        assert int(b.count_true()) == int(h.sum())
+
+
+@pytest.mark.parametrize("tname,dt", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
+def test_bits_to_numbers_by_rows(tname, dt):
+    """Bit -> number where both run along the innermost dimension: four elements per lane, stored as
+    128-bit vectors from any element boundary; rows that end in part of a vector, windows that start
+    inside a word, skipped rows, a destination that is a window of a larger array."""
+    import cumo_amd
+    rng = np.random.default_rng(614)
+    cls = getattr(cumo_amd, tname)
+    for shape in [(70, 131), (5, 4099), (300, 33), (9, 7, 67), (64, 64), (1, 100003), (100003,)]:
+        h = rng.integers(0, 2, size=shape).astype(np.uint8)
+        b = cumo_amd.Bit.cast(h)
+        assert (b._store_into(cls).to_numpy() == oracle.store_bit(dt, h)).all(), shape
+        for key in ((Ellipsis, slice(1, None)), (Ellipsis, slice(3, -5)), (slice(None, None, 2),), (slice(None, None, -1), Ellipsis, slice(2, None))):
+            if len(shape) == 1 and len([k for k in key if k is not Ellipsis]) > 1:
+                continue
+            assert (b[key]._store_into(cls).to_numpy() == oracle.store_bit(dt, h[key])).all(), (shape, key)
+        if len(shape) > 1:
+            hz = rng.standard_normal(shape).astype(dt)
+            z = cls.cast(hz)
+            z[..., 1:] = b[..., :-1]
+            hz[..., 1:] = h[..., :-1]
+            assert (z.to_numpy() == hz).all(), shape
