@@ -1946,10 +1946,18 @@ int cumo_hip_na_store(cumo_hip_narray_t* dst, const cumo_hip_narray_t* src) {
     cumo_hip_ndfunc_t nf = {NULL, 0, 2, 0, {0, 0}};
     void* opt = NULL;
     StoreOpt sopt;
+    CondOpt copt;
     if (dst->type == CUMO_HIP_BIT && src->type != CUMO_HIP_BIT) {
         if (src->type < 0 || src->type > CUMO_HIP_UINT64) return fail(CUMO_HIP_ERROR_TYPE, "store: unsupported source type");
         nf.func = iter_bit_store_from;  // nonzero is 1 (types/bit_kernel.h:13-19)
         opt = (void*)kBitStoreFrom[src->type];
+        // into a whole contiguous Bit array this is the comparison "x != 0", which has the vector kernels
+        const CondRow* ne = is_arith(src->type) ? find_row(kCond, "ne") : NULL;
+        if (ne && cond_has(ne, src->type) && dst->offset == 0 && is_contiguous(dst)) {
+            copt = {ne, src->type, true, 0.0, 0};
+            nf.func = iter_cond;  // args: src, dst
+            opt = &copt;
+        }
     } else if (dst->type == CUMO_HIP_BIT) {
         const BitUnaryRow* row = find_row(kBitUnary, "copy");
         nf.func = iter_bit_unary;  // args: src, dst
@@ -1969,7 +1977,7 @@ int cumo_hip_na_store(cumo_hip_narray_t* dst, const cumo_hip_narray_t* src) {
     // the loop must have the destination's shape: the source may repeat, the destination may not
     cumo_hip_loop_t lp;
     const NA* in[2] = {dst, src};
-    if (nf.func == iter_bit_unary) {
+    if (nf.func == iter_bit_unary || nf.func == iter_cond) {
         in[0] = src;
         in[1] = dst;
     }

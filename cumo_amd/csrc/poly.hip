@@ -8,6 +8,7 @@
 // multiplication and addition, rounded separately (types/float_macro_kernel.h m_mul, m_add),
 // Int32 wrapping.
 #include "common.h"
+#include "plan.h"
 
 #include <type_traits>
 
@@ -75,6 +76,80 @@ __global__ __launch_bounds__(256) void poly_kernel(PolyParams p) {
     }
 }
 
+// x and z one contiguous run each and every coefficient a single number: a 128-bit vector per lane
+// (from any element boundary), the coefficients read once per lane.
+struct PolyFlat {
+    int nc, from_z;
+    const char* c[kPolyChunk];
+};
+
+template <class T, bool NT>
+__global__ __launch_bounds__(256) void poly_flat_kernel(const T* x, T* z, uint64_t n, PolyFlat p) {
+    constexpr int V = 16 / sizeof(T);
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    union Vec {
+        u4 q;
+        T v[V];
+        __device__ Vec() {}
+    };
+    T a[kPolyChunk];
+#pragma unroll
+    for (int k = 0; k < kPolyChunk; ++k) a[k] = k < p.nc ? *reinterpret_cast<const T*>(p.c[k]) : (T)0;
+    const uint64_t nv = (n + V - 1) / V;
+    for (uint64_t v = (uint64_t)blockIdx.x * 256 + threadIdx.x; v < nv; v += (uint64_t)gridDim.x * 256) {
+        const uint64_t e = v * V;
+        const bool whole = e + V <= n;
+        Vec xs, ys;
+        if (whole) {
+            xs.q = NT ? __builtin_nontemporal_load(reinterpret_cast<const u4*>(x + e)) : *reinterpret_cast<const u4*>(x + e);
+            if (p.from_z) ys.q = *reinterpret_cast<const u4*>(z + e);
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                xs.v[j] = e + j < n ? x[e + j] : (T)0;
+                ys.v[j] = (p.from_z && e + j < n) ? z[e + j] : (T)0;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            T y;
+            int k = 0;
+            if (p.from_z) {
+                y = ys.v[j];
+            } else if (p.nc > 0) {
+                y = a[0];
+                k = 1;
+            } else {
+                y = xs.v[j];
+            }
+#pragma unroll
+            for (int q = 0; q < kPolyChunk; ++q) {
+                if (q >= k && q < p.nc) y = poly_step<T>(xs.v[j], y, a[q]);
+            }
+            ys.v[j] = y;
+        }
+        if (whole) {
+            if (NT) __builtin_nontemporal_store(ys.q, reinterpret_cast<u4*>(z + e));
+            else *reinterpret_cast<u4*>(z + e) = ys.q;
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+                if (e + j < n) z[e + j] = ys.v[j];
+        }
+    }
+}
+
+// whether the operand's elements lie one after another in row-major order
+inline bool poly_one_run(const cumo_na_iarray_t* a, const cumo_na_indexer_t* indexer, size_t elmsz) {
+    int64_t want = (int64_t)elmsz;
+    for (int d = indexer->ndim - 1; d >= 0; --d) {
+        if (indexer->shape[d] == 1) continue;
+        if ((int64_t)a->step[d] != want) return false;
+        want *= (int64_t)indexer->shape[d];
+    }
+    return ((uintptr_t)a->ptr % alignof(uint32_t)) == 0 && ((uintptr_t)a->ptr % elmsz) == 0;
+}
+
 template <class T>
 void poly_launch(const cumo_na_iarray_t* x, const cumo_na_iarray_t* coef, int ncoef, const cumo_na_iarray_t* z, const cumo_na_indexer_t* indexer) {
     if (indexer->total_size == 0) return;
@@ -94,6 +169,33 @@ void poly_launch(const cumo_na_iarray_t* x, const cumo_na_iarray_t* coef, int nc
     // coefficients from the highest power down, kPolyChunk a launch
     int next = ncoef - 1;
     bool first = true;
+    bool flat = !force_wide_indices() && p.total >= 1024 && poly_one_run(x, indexer, sizeof(T)) && poly_one_run(z, indexer, sizeof(T));
+    for (int k = 0; k < ncoef && flat; ++k)
+        for (int d = 0; d < indexer->ndim; ++d)
+            if (indexer->shape[d] != 1 && coef[k].step[d] != 0) flat = false;
+    if (flat) {
+        const bool nt = stream_past_caches(p.total * sizeof(T) * 2);
+        constexpr uint64_t V = 16 / sizeof(T);
+        uint64_t g = ((p.total + V - 1) / V + 255) / 256;
+        if (g > (uint64_t)kNumCU * 32) g = (uint64_t)kNumCU * 32;
+        do {
+            PolyFlat f;
+            f.from_z = first ? 0 : 1;
+            f.nc = 0;
+            for (int k = 0; k < kPolyChunk; ++k) {
+                f.c[k] = next >= 0 ? coef[next].ptr : nullptr;
+                if (next >= 0) {
+                    ++f.nc;
+                    --next;
+                }
+            }
+            if (nt) hipLaunchKernelGGL((poly_flat_kernel<T, true>), dim3((unsigned)g), dim3(256), 0, st, (const T*)x->ptr, (T*)z->ptr, p.total, f);
+            else hipLaunchKernelGGL((poly_flat_kernel<T, false>), dim3((unsigned)g), dim3(256), 0, st, (const T*)x->ptr, (T*)z->ptr, p.total, f);
+            first = false;
+        } while (next >= 0);
+        cumo_cuda_runtime_check_kernel_launch();
+        return;
+    }
     do {
         p.from_z = first ? 0 : 1;
         p.nc = 0;

@@ -241,3 +241,33 @@ def test_bits_to_numbers_by_rows(tname, dt):
             z[..., 1:] = b[..., :-1]
             hz[..., 1:] = h[..., :-1]
             assert (z.to_numpy() == hz).all(), shape
+
+
+@pytest.mark.parametrize("tname,dt", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
+def test_numbers_to_bits_of_a_whole_array_and_of_windows(tname, dt):
+    """number -> Bit (nonzero is 1, NaN included, the zero of either sign is 0): into a whole array
+    (the comparison kernels take it), into the front part of a longer one (the bits after it stay),
+    into windows, from a source that repeats."""
+    import cumo_amd
+    rng = np.random.default_rng(615)
+    cls = getattr(cumo_amd, tname)
+    for shape in [(70, 131), (5, 4099), (100003,), (8, 4096), (64, 64), (3, 5, 67)]:
+        h = (rng.integers(-2, 3, size=shape)).astype(dt)
+        if dt != np.int32:
+            h.reshape(-1)[::7] = np.nan
+            h.reshape(-1)[3::11] = -0.0
+        want = (h != 0).astype(np.uint8)
+        d = cls.cast(h)
+        assert (cumo_amd.Bit.cast(np.zeros(shape, dtype=np.uint8)).store(d).to_numpy() == want).all(), shape
+        hz = rng.integers(0, 2, size=(2,) + shape).astype(np.uint8)
+        z = cumo_amd.Bit.cast(hz)
+        z[0] = d                               # the front part of a longer array
+        hz[0] = want
+        assert (z.to_numpy() == hz).all(), shape
+        z[1, ..., 1:] = d[..., :-1]            # a window that starts inside a word
+        hz[1, ..., 1:] = want[..., :-1]
+        assert (z.to_numpy() == hz).all(), shape
+        if len(shape) == 2:
+            z2 = cumo_amd.Bit.cast(np.zeros(shape, dtype=np.uint8))
+            z2.store(d[:1])                    # one row repeated down the array
+            assert (z2.to_numpy() == np.broadcast_to(want[:1], shape)).all(), shape

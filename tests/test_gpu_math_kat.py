@@ -227,6 +227,11 @@ def test_poly(cls, dt):
         assert (got.view(np.uint8) == oracle.poly(h, *coefs[:n]).view(np.uint8)).all(), n
     got = d.transpose()[1::2, ::3].poly(*coefs[:8]).to_numpy()
     assert (got == oracle.poly(np.ascontiguousarray(h.T[1::2, ::3]), *coefs[:8])).all()
+    # one run that starts off a 16-byte boundary and ends in part of a vector
+    flat = T.cast(h.reshape(-1))
+    for lo, hi in ((5, None), (1, -2), (3, 1030)):
+        got = flat[lo:hi].poly(*coefs[:9]).to_numpy()
+        assert (got.view(np.uint8) == oracle.poly(np.ascontiguousarray(h.reshape(-1)[lo:hi]), *coefs[:9]).view(np.uint8)).all(), (lo, hi)
     row = (rng.integers(-5, 5, size=53) if dt == np.int32 else rng.standard_normal(53)).astype(dt)
     col = (rng.integers(-5, 5, size=(37, 1)) if dt == np.int32 else rng.standard_normal((37, 1))).astype(dt)
     for cs in ((row,), (row, col), (coefs[0], row, col, coefs[1]), (col, coefs[2], row)):
