@@ -52,11 +52,108 @@ __global__ __launch_bounds__(256) void ret2_kernel(Ret2Params p, Op op) {
     }
 }
 
+// Every operand one contiguous run: a lane takes the elements of one 128-bit vector of the input type
+// (vectors need the element's alignment only); an element that the op refuses is left unwritten, so a
+// vector with one of those is stored element by element.
+template <class X, int V, bool NT>
+__device__ __forceinline__ void ret2_load(const X* p, X (&v)[V]) {
+    typedef X XV __attribute__((ext_vector_type(V)));
+    const XV t = NT ? __builtin_nontemporal_load(reinterpret_cast<const XV*>(p)) : *reinterpret_cast<const XV*>(p);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v[j] = t[j];
+}
+template <class X, int V, bool NT>
+__device__ __forceinline__ void ret2_store(X* p, const X (&v)[V]) {
+    typedef X XV __attribute__((ext_vector_type(V)));
+    XV t;
+#pragma unroll
+    for (int j = 0; j < V; ++j) t[j] = v[j];
+    if (NT) __builtin_nontemporal_store(t, reinterpret_cast<XV*>(p));
+    else *reinterpret_cast<XV*>(p) = t;
+}
+
+template <class Op, bool NT>
+__global__ __launch_bounds__(256) void ret2_flat_kernel(const typename Op::In* px, const typename Op::In* py, typename Op::Out1* pa,
+                                                        typename Op::Out2* pb, uint64_t n, int* flag, Op op) {
+    typedef typename Op::In In;
+    constexpr int V = 16 / sizeof(In);
+    const uint64_t nv = (n + V - 1) / V;
+    for (uint64_t v = (uint64_t)blockIdx.x * 256 + threadIdx.x; v < nv; v += (uint64_t)gridDim.x * 256) {
+        const uint64_t e = v * V;
+        const bool whole = e + V <= n;
+        In x[V], y[V];
+        if (whole) {
+            ret2_load<In, V, NT>(px + e, x);
+            if (Op::NIN == 2) ret2_load<In, V, NT>(py + e, y);
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                x[j] = e + j < n ? px[e + j] : In();
+                if (Op::NIN == 2) y[j] = e + j < n ? py[e + j] : In();
+            }
+        }
+        typename Op::Out1 a[V];
+        typename Op::Out2 b[V];
+        bool ok[V], all = true;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            ok[j] = op(x[j], Op::NIN == 2 ? y[j] : In(), a[j], b[j]);
+            if (whole || e + j < n) all = all && ok[j];
+        }
+        if (whole && all) {
+            ret2_store<typename Op::Out1, V, NT>(pa + e, a);
+            ret2_store<typename Op::Out2, V, NT>(pb + e, b);
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                if (e + j < n && ok[j]) {
+                    pa[e + j] = a[j];
+                    pb[e + j] = b[j];
+                }
+            }
+            if (!all && flag) *flag = 1;
+        }
+    }
+}
+
+template <class X>
+static bool ret2_one_run(const cumo_na_iarray_t* a, const cumo_na_indexer_t* indexer) {
+    int64_t want = (int64_t)sizeof(X);
+    for (int d = indexer->ndim - 1; d >= 0; --d) {
+        if (indexer->shape[d] == 1) continue;
+        if ((int64_t)a->step[d] != want) return false;
+        want *= (int64_t)indexer->shape[d];
+    }
+    return ((uintptr_t)a->ptr % sizeof(X)) == 0;
+}
+
 // arr: the NIN inputs, then the two results
 template <class Op>
 static void ret2_launch(Op op, const cumo_na_iarray_t* const* arr, const cumo_na_indexer_t* indexer, int* flag) {
     if (indexer->total_size == 0) return;
     constexpr int NA = Op::NIN + 2;
+    {
+        typedef typename Op::In In;
+        bool flat = !force_wide_indices() && indexer->total_size >= 1024 && ret2_one_run<In>(arr[0], indexer);
+        if (Op::NIN == 2) flat = flat && ret2_one_run<In>(arr[1], indexer);
+        flat = flat && ret2_one_run<typename Op::Out1>(arr[Op::NIN], indexer) && ret2_one_run<typename Op::Out2>(arr[Op::NIN + 1], indexer);
+        if (flat) {
+            constexpr uint64_t V = 16 / sizeof(In);
+            const uint64_t n = indexer->total_size;
+            uint64_t g = ((n + V - 1) / V + 255) / 256;
+            if (g > 256u * 32u) g = 256u * 32u;
+            const In* px = reinterpret_cast<const In*>(arr[0]->ptr);
+            const In* py = Op::NIN == 2 ? reinterpret_cast<const In*>(arr[1]->ptr) : nullptr;
+            typename Op::Out1* pa = reinterpret_cast<typename Op::Out1*>(arr[Op::NIN]->ptr);
+            typename Op::Out2* pb = reinterpret_cast<typename Op::Out2*>(arr[Op::NIN + 1]->ptr);
+            if (stream_past_caches(n * sizeof(In) * 2))
+                hipLaunchKernelGGL((ret2_flat_kernel<Op, true>), dim3((unsigned)g), dim3(256), 0, current_stream(), px, py, pa, pb, n, flag, op);
+            else
+                hipLaunchKernelGGL((ret2_flat_kernel<Op, false>), dim3((unsigned)g), dim3(256), 0, current_stream(), px, py, pa, pb, n, flag, op);
+            cumo_cuda_runtime_check_kernel_launch();
+            return;
+        }
+    }
     Ret2Params p;
     p.ndim = indexer->ndim;
     p.total = indexer->total_size;

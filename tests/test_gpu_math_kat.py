@@ -239,3 +239,45 @@ def test_poly(cls, dt):
         assert (got.view(np.uint8) == oracle.poly(h, *cs).view(np.uint8)).all()
     small = T.cast(h[:1])                      # [1, 53] against a column: the constant alone spreads over both
     assert (small.poly(T.cast(col)).to_numpy() == np.broadcast_to(col, (37, 53))).all()
+
+
+def test_two_result_operations_over_whole_runs():
+    """modf, frexp and divmod where every operand is one contiguous run (128-bit vectors per lane, from
+    any element boundary, lengths that end in part of a vector) against the oracle bit for bit; an
+    Int32 division that meets a zero somewhere inside raises."""
+    import cumo_amd
+    rng = np.random.default_rng(77)
+    for cls, dt in TYPES:
+        T = getattr(cumo_amd, cls)
+        for shape in [(37, 53), (5000,), (3, 7, 101)]:
+            x = (rng.standard_normal(shape) * 50).astype(dt)
+            y = (rng.standard_normal(shape) * 7).astype(dt)
+            x.reshape(-1)[::97] = np.inf
+            x.reshape(-1)[5::89] = -0.0
+            f, w = T.cast(x).modf()
+            wf, ww = oracle.modf(x)
+            assert (f.to_numpy().view(np.uint8) == wf.view(np.uint8)).all() and (w.to_numpy().view(np.uint8) == ww.view(np.uint8)).all(), shape
+            fin = np.isfinite(x)
+            m, e = cumo_amd.NMath.frexp(T.cast(x))
+            wm, we = oracle.frexp(x)
+            assert (m.to_numpy()[fin].view(np.uint8) == wm[fin].view(np.uint8)).all() and (e.to_numpy()[fin] == we[fin]).all(), shape
+            xf = np.where(fin, x, 1.0).astype(dt)
+            q, r = T.cast(xf).divmod(T.cast(y))
+            wq, wr = oracle.divmod_(xf, y)
+            assert (q.to_numpy().view(np.uint8) == wq.view(np.uint8)).all() and (r.to_numpy().view(np.uint8) == wr.view(np.uint8)).all(), shape
+        flat = (rng.standard_normal(3000) * 9).astype(dt)
+        d = T.cast(flat)
+        for lo, hi in ((1, None), (3, -2), (5, 1500)):
+            f, w = d[lo:hi].modf()
+            wf, ww = oracle.modf(np.ascontiguousarray(flat[lo:hi]))
+            assert (f.to_numpy().view(np.uint8) == wf.view(np.uint8)).all() and (w.to_numpy().view(np.uint8) == ww.view(np.uint8)).all(), (lo, hi)
+    a = rng.integers(-10 ** 6, 10 ** 6, size=(41, 67)).astype(np.int32)
+    b = rng.integers(1, 500, size=(41, 67)).astype(np.int32) * rng.choice([-1, 1], size=(41, 67)).astype(np.int32)
+    a[3, 5] = -2 ** 31
+    b[3, 5] = -1
+    q, r = cumo_amd.Int32.cast(a).divmod(cumo_amd.Int32.cast(b))
+    wq, wr = oracle.divmod_(a, b)
+    assert (q.to_numpy() == wq).all() and (r.to_numpy() == wr).all()
+    b[20, 33] = 0
+    with pytest.raises(ZeroDivisionError):
+        cumo_amd.Int32.cast(a).divmod(cumo_amd.Int32.cast(b))
