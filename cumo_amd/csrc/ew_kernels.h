@@ -1755,11 +1755,15 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             const int64_t es = sl == 0 ? (int64_t)sizeof(A) : (sl == 1 ? (int64_t)sizeof(B) : (int64_t)sizeof(R));
             flat = plan.step[o][0] == es;
         }
-        const uint64_t per_block = (uint64_t)kEwBlock * vec * (op_is_heavy<Op>::value ? 2 : 1);
+        // A result wider than the input (SFloat or Int32 -> DFloat): two elements per lane, so that a lane
+        // stores one 128-bit vector and a wave one contiguous KiB, rather than two vectors 32 bytes apart
+        // (SFloat [8192,4096] -> DFloat: 89.7 -> 62.4 us).
+        const int fvec = (sizeof(R) > sizeof(A) && vec == 4) ? 2 : vec;
+        const uint64_t per_block = (uint64_t)kEwBlock * fvec * (op_is_heavy<Op>::value ? 2 : 1);
         const uint64_t blocks = (kp.inner + per_block - 1) / per_block;
         if (flat && blocks <= ew_grid_max()) {
             const dim3 g((unsigned)blocks);
-            if (vec == 4) {
+            if (fvec == 4) {
                 if (nt) hipLaunchKernelGGL((ew_flat_kernel<Op, 4, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
                 else hipLaunchKernelGGL((ew_flat_kernel<Op, 4, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
             } else {
