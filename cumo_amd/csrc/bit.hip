@@ -808,7 +808,12 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
     pos += back * 32;
     const uint64_t vecs = ((pos + n + 31) / 32 + 3) / 4 - (pos / 32) / 4;
     uint64_t grid = (vecs + kBlock - 1) / kBlock;
-    if (grid > 512) grid = 512;  // every block ends in one returning atomic on the same word
+    // every block ends in one returning atomic on the same word, which serialise: 128 blocks, and more
+    // (up to 512) only where every lane still has sixteen vectors to read
+    uint64_t most = vecs / ((uint64_t)kBlock * 16);
+    if (most < 128) most = 128;
+    if (most > 512) most = 512;
+    if (grid > most) grid = most;
     if (grid == 0) grid = 1;
     if (count_false)
         hipLaunchKernelGGL((bit_count_words_store_kernel<true>), dim3((unsigned)grid), dim3(kBlock), 0, st, (const CUMO_BIT_DIGIT*)a, (uint64_t)pos, n,
