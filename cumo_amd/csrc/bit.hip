@@ -788,6 +788,8 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
     static std::mutex mu;
     static unsigned long long* tickets = nullptr;
     if (n == 0 || n >= (1ull << kTicketShift)) return 0;
+    // a long run goes through the reduction kernels (2^29 bits: 21 us with the ticket kernel on 512 blocks)
+    if (bit_count_run_reduce(a, pos, n, count_false, out)) return 1;
     hipStream_t st = current_stream();
     const int slot = stream_slot(st);  // the stream's own ticket word; given back when the stream is destroyed
     if (slot < 0 || slot >= kTicketSlots) return 0;
@@ -828,6 +830,7 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
 extern "C" void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* d) {
     if (!d) return;
     if (bit_count_cols_launch(d)) return;
+    if (bit_count_rows_reduce(d)) return;
     BitCountNd p;
     std::memset(&p, 0, sizeof(p));
     p.out_ndim = d->out_ndim;

@@ -199,7 +199,8 @@ def test_counts_down_columns_and_along_long_rows():
     any word). Shapes whose rows do not start on words, views, three dimensions."""
     import cumo_amd
     rng = np.random.default_rng(613)
-    for shape in [(300, 70), (1000, 4097), (5, 64), (40000, 65), (3, 500, 130), (2, 70000, 96), (700, 1000), (33, 32767), (70, 5000)]:
+    for shape in [(300, 70), (1000, 4097), (5, 64), (40000, 65), (3, 500, 130), (2, 70000, 96), (700, 1000), (33, 32767), (70, 5000),
+                  (70, 4096), (300, 2048), (9, 5, 2112), (3, 100000 * 32)]:
         h = (rng.random(shape) < 0.7).astype(np.uint8)
         h[..., 1] = 1                          # a column that is all set, one that is all clear
         h[..., 2] = 0
@@ -271,3 +272,21 @@ def test_numbers_to_bits_of_a_whole_array_and_of_windows(tname, dt):
             z2 = cumo_amd.Bit.cast(np.zeros(shape, dtype=np.uint8))
             z2.store(d[:1])                    # one row repeated down the array
             assert (z2.to_numpy() == np.broadcast_to(want[:1], shape)).all(), shape
+
+
+@pytest.mark.parametrize("n", [1 << 24, (1 << 24) + 77, (1 << 25) + 31])
+def test_counts_of_very_long_runs(n):
+    """A run of 2^24 bits or more is counted by the reduction kernels over its words, the first and
+    the last word masked: runs that start at any bit, that end in part of a word, set and clear bits."""
+    import cumo_amd
+    rng = np.random.default_rng(616)
+    h = (rng.random(n + 100) < 0.3).astype(np.uint8)
+    b = cumo_amd.Bit.cast(h)
+    for lo in (0, 1, 31, 32, 45):
+        for cut in (0, 1, 33):
+            v = h[lo:n + 100 - cut]
+            d = b[lo:n + 100 - cut]
+            assert int(d.count_true()) == int(v.sum()), (lo, cut)
+            assert int(d.count_false()) == int(v.size - v.sum()), (lo, cut)
+    ones = cumo_amd.Bit.cast(np.ones(n, dtype=np.uint8))
+    assert int(ones.count_true()) == n and int(ones.count_false()) == 0 and ones.all_p() and not ones.none_p()
