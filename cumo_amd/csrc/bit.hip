@@ -123,13 +123,13 @@ __global__ __launch_bounds__(kBlock) void bit_generic_kernel(cumo_na_bit_iarray_
 }
 
 // Views whose innermost dimension runs along the bits (step 1) in every operand and that use no index
-// array: a lane takes one word of one result row. nw1 / nw2: words of a1 / a2 up to the last bit the
-// view reaches (nothing past them is read). A row's first and last word may be shared with its
-// neighbours in memory, so those two are changed with atomics; the words between them belong to the
-// row alone.
+// array: a lane takes four words of one result row, as a vector where the row has all four to itself.
+// nw1 / nw2: words of a1 / a2 up to the last bit the view reaches (nothing past them is read). A
+// row's first and last word may be shared with its neighbours in memory, so those two are changed
+// with atomics; the words between them belong to the row alone.
 struct BitRowsOp {
     int ndim;
-    uint64_t items, chunks, inner;   // chunks: result words a row can span
+    uint64_t items, chunks, inner;   // chunks: lanes per row, each with four of the result words the row can span
     uint64_t shape[kMaxDim];
     int64_t s1[kMaxDim], s2[kMaxDim], s3[kMaxDim];  // bit steps of the outer dimensions
     uint64_t nw1, nw2;
@@ -138,9 +138,10 @@ struct BitRowsOp {
 template <int OP, bool BINARY>
 __global__ __launch_bounds__(kBlock) void bit_rows_kernel(const CUMO_BIT_DIGIT* a1, uint64_t p1, const CUMO_BIT_DIGIT* a2, uint64_t p2,
                                                           CUMO_BIT_DIGIT* a3, uint64_t p3, BitRowsOp nd) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
     for (uint64_t item = (uint64_t)blockIdx.x * kBlock + threadIdx.x; item < nd.items; item += (uint64_t)gridDim.x * kBlock) {
         uint64_t q = item / nd.chunks;
-        const uint64_t k = item - q * nd.chunks;
+        const uint64_t k = (item - q * nd.chunks) * 4;  // a lane takes four words of the row
         int64_t q1 = (int64_t)p1, q2 = (int64_t)p2, q3 = (int64_t)p3;
         for (int d = nd.ndim - 2; d >= 0; --d) {
             uint64_t i = q;
@@ -154,20 +155,37 @@ __global__ __launch_bounds__(kBlock) void bit_rows_kernel(const CUMO_BIT_DIGIT* 
             q3 += (int64_t)i * nd.s3[d];
         }
         const uint64_t w_first = (uint64_t)q3 >> 5, w_last = ((uint64_t)q3 + nd.inner - 1) >> 5;
-        const uint64_t w = w_first + k;
-        if (w > w_last) continue;
-        const int64_t e0 = (int64_t)(w << 5) - q3;  // the row's element at bit 0 of this word (negative in its first word)
-        const uint32_t x = bits_at(a1, q1 + e0, nd.nw1);
-        const uint32_t y = BINARY ? bits_at(a2, q2 + e0, nd.nw2) : 0u;
-        const uint32_t z = bit_apply<OP>(x, y);
-        const unsigned lo = (w == w_first) ? (unsigned)((uint64_t)q3 & 31) : 0u;
-        const unsigned hi = (w == w_last) ? (unsigned)(((uint64_t)q3 + nd.inner - 1) & 31) + 1u : 32u;
-        const uint32_t mask = low_bits(hi) & ~low_bits(lo);
-        if (w != w_first && w != w_last) {
-            a3[w] = z;
-        } else {
-            atomicAnd(&a3[w], ~mask);
-            atomicOr(&a3[w], z & mask);
+        const uint64_t w0 = w_first + k;
+        if (w0 > w_last) continue;
+        const int64_t e00 = (int64_t)(w0 << 5) - q3;  // the row's element at bit 0 of the lane's first word (negative in the row's first word)
+        // four words that the row has to itself, whose inputs (five words each when they start inside a word) are all there
+        if (w0 > w_first && w0 + 3 < w_last && (((uint64_t)(q1 + e00)) >> 5) + 5 <= nd.nw1 &&
+            (!BINARY || (((uint64_t)(q2 + e00)) >> 5) + 5 <= nd.nw2)) {
+            const uint4 x = bits128_at<false>(a1, (uint64_t)(q1 + e00));
+            uint4 y = make_uint4(0u, 0u, 0u, 0u);
+            if (BINARY) y = bits128_at<false>(a2, (uint64_t)(q2 + e00));
+            u4 z;
+            z.x = bit_apply<OP>(x.x, y.x);
+            z.y = bit_apply<OP>(x.y, y.y);
+            z.z = bit_apply<OP>(x.z, y.z);
+            z.w = bit_apply<OP>(x.w, y.w);
+            *reinterpret_cast<u4*>(a3 + w0) = z;
+            continue;
+        }
+        for (uint64_t w = w0; w < w0 + 4 && w <= w_last; ++w) {
+            const int64_t e0 = (int64_t)(w << 5) - q3;
+            const uint32_t x = bits_at(a1, q1 + e0, nd.nw1);
+            const uint32_t y = BINARY ? bits_at(a2, q2 + e0, nd.nw2) : 0u;
+            const uint32_t z = bit_apply<OP>(x, y);
+            const unsigned lo = (w == w_first) ? (unsigned)((uint64_t)q3 & 31) : 0u;
+            const unsigned hi = (w == w_last) ? (unsigned)(((uint64_t)q3 + nd.inner - 1) & 31) + 1u : 32u;
+            const uint32_t mask = low_bits(hi) & ~low_bits(lo);
+            if (w != w_first && w != w_last) {
+                a3[w] = z;
+            } else {
+                atomicAnd(&a3[w], ~mask);
+                atomicOr(&a3[w], z & mask);
+            }
         }
     }
 }
@@ -203,7 +221,7 @@ bool bit_rows_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_
     }
     nd.ndim = n;
     nd.inner = indexer->shape[n - 1];
-    nd.chunks = (nd.inner + 31) / 32 + 1;
+    nd.chunks = ((nd.inner + 31) / 32 + 1 + 3) / 4;  // lanes a row can need: four of its words each
     nd.items = nd.chunks;
     for (int d = 0; d < n; ++d) {
         nd.shape[d] = indexer->shape[d];
