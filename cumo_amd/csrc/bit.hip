@@ -285,8 +285,11 @@ __global__ __launch_bounds__(kBlock) void store_bit_rows_kernel(char* dst, const
         const unsigned cnt = inner - e0 >= 4 ? 4u : (unsigned)(inner - e0);
         const uint64_t b0 = (uint64_t)bit + e0;
         const unsigned sh = (unsigned)(b0 & 31);
-        uint32_t x = src[b0 >> 5] >> sh;
-        if (sh + cnt > 32) x |= src[(b0 >> 5) + 1] << (32 - sh);
+        // (both words loaded with no branch between them: the second from the first's address when it is not needed)
+        const uint32_t lo = src[b0 >> 5];
+        const uint32_t hi = src[(b0 >> 5) + (sh + cnt > 32 ? 1 : 0)];
+        uint32_t x = lo >> sh;
+        if (sh != 0) x |= hi << (32 - sh);
         T* out = reinterpret_cast<T*>(dst + off) + e0;
         if (cnt == 4) {
             union V {
@@ -620,13 +623,15 @@ __global__ __launch_bounds__(kBlock) void bit_count_nd_kernel(BitCountNd p) {
 
 // Counts down columns: the kept dimension that runs along the bits (step 1) has `cols` outputs, the one
 // reduced dimension steps `s_red` bits, and an optional outer kept dimension steps s_outer bits /
-// o_outer bytes. A block of 16 waves has 64 x 32 neighbouring columns of one outer position and a
-// stretch of the rows, a sixteenth of it per wave; a lane owns 32 columns: it reads their word row by
-// row (two words where the row does not start on a word) and counts every column in byte-wide counters,
-// four to a register (column j of the 32 sits in counter j / 8 of register j % 8), moved to 32-bit
-// counters before a byte could overflow. The waves add their totals up in LDS, and the block adds the
-// sums onto the 64-bit results, one atomic per column that has any.
+// o_outer bytes. A block of 1024 lanes has 32 x 32 neighbouring columns of one outer position and a
+// stretch of the rows, a thirty-second of it per group of 32 lanes; a lane owns 32 columns: it reads
+// their word row by row (two words where the row does not start on a word; eight rows' loads go out
+// before the first is waited for, with no branch between them) and counts every column in byte-wide
+// counters, four to a register (column j of the 32 sits in counter j / 8 of register j % 8), moved to
+// 32-bit counters before a byte could overflow. The groups add their totals up in LDS, and the block
+// adds the sums onto the 64-bit results, one atomic per column that has any.
 constexpr int kCountColsBlock = 1024;
+constexpr int kCountColsRows = 8;   // rows a lane has in flight
 
 struct BitCountCols {
     const CUMO_BIT_DIGIT* in;
@@ -638,17 +643,18 @@ struct BitCountCols {
 
 template <bool COUNT_FALSE>
 __global__ __launch_bounds__(kCountColsBlock) void bit_count_cols_kernel(BitCountCols p) {
-    __shared__ uint32_t sums[32][64];
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ uint32_t sums[32][32];
+    // half a wave has 32 neighbouring chunks of columns (128 bytes of a row), the other half the same chunks of another stretch of rows
+    const unsigned lane = threadIdx.x & 31, group = threadIdx.x >> 5;
     const uint32_t cb = blockIdx.x % p.chunk_blocks;
     const uint32_t b2 = blockIdx.x / p.chunk_blocks;
     const uint32_t part = b2 % p.row_parts;
     const uint32_t o = b2 / p.row_parts;
-    for (unsigned i = threadIdx.x; i < 32 * 64; i += kCountColsBlock) (&sums[0][0])[i] = 0u;
+    for (unsigned i = threadIdx.x; i < 32 * 32; i += kCountColsBlock) (&sums[0][0])[i] = 0u;
     __syncthreads();
-    const uint32_t c = cb * 64u + lane;
+    const uint32_t c = cb * 32u + lane;
     if (c < p.chunks) {
-        const uint64_t first_row = ((uint64_t)part * 16 + wave) * p.rows_per_wave;
+        const uint64_t first_row = ((uint64_t)part * 32 + group) * p.rows_per_wave;
         const uint32_t r0 = first_row < p.rows ? (uint32_t)first_row : p.rows;
         const uint32_t r1 = r0 + p.rows_per_wave < p.rows ? r0 + p.rows_per_wave : p.rows;
         const unsigned cnt = p.cols - c * 32u >= 32u ? 32u : p.cols - c * 32u;
@@ -657,25 +663,35 @@ __global__ __launch_bounds__(kCountColsBlock) void bit_count_cols_kernel(BitCoun
         uint32_t total[32];
 #pragma unroll
         for (int j = 0; j < 32; ++j) total[j] = 0u;
-        for (uint32_t ra = r0; ra < r1; ra += 252) {
-            const uint32_t rb = ra + 252 < r1 ? ra + 252 : r1;
+        for (uint32_t ra = r0; ra < r1; ra += 240) {
+            const uint32_t rb = ra + 240 < r1 ? ra + 240 : r1;
             uint32_t bytes[8];
 #pragma unroll
             for (int k = 0; k < 8; ++k) bytes[k] = 0u;
-            for (uint32_t r = ra; r < rb; r += 4) {
-                uint32_t x[4];
+            for (uint32_t r = ra; r < rb; r += kCountColsRows) {
+                // every load of the step goes out before anything waits for one: no branch between them (the
+                // word after a row's word is loaded whether needed or not, from the same address when not)
+                uint32_t x[kCountColsRows], lo[kCountColsRows], hi[kCountColsRows];
+                unsigned shs[kCountColsRows];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < kCountColsRows; ++u) {
                     const uint32_t rr = r + u < rb ? r + u : rb - 1;
                     const uint64_t q = (uint64_t)(first + (int64_t)rr * p.s_red);
-                    const unsigned sh = (unsigned)(q & 31);
-                    uint32_t w = p.in[q >> 5] >> sh;
-                    if (sh + cnt > 32) w |= p.in[(q >> 5) + 1] << (32 - sh);
+                    shs[u] = (unsigned)(q & 31);
+                    const uint64_t w = q >> 5;
+                    lo[u] = p.in[w];
+                    hi[u] = p.in[w + (shs[u] + cnt > 32 ? 1 : 0)];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < kCountColsRows; ++u) {
+                    uint32_t w = lo[u] >> shs[u];
+                    if (shs[u] != 0) w |= hi[u] << (32 - shs[u]);
                     if (COUNT_FALSE) w = ~w;
                     x[u] = (r + u < rb) ? (w & keep) : 0u;
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < kCountColsRows; ++u) {
 #pragma unroll
                     for (int k = 0; k < 8; ++k) bytes[k] += (x[u] >> k) & 0x01010101u;
                 }
@@ -690,10 +706,10 @@ __global__ __launch_bounds__(kCountColsBlock) void bit_count_cols_kernel(BitCoun
         }
     }
     __syncthreads();
-    for (unsigned i = threadIdx.x; i < 32 * 64; i += kCountColsBlock) {
+    for (unsigned i = threadIdx.x; i < 32 * 32; i += kCountColsBlock) {
         // consecutive threads, consecutive columns
         const unsigned l = i >> 5, j = i & 31;
-        const uint32_t col = (cb * 64u + l) * 32u + j;
+        const uint32_t col = (cb * 32u + l) * 32u + j;
         const uint32_t v = sums[j][l];
         if (col < p.cols && v != 0u)
             atomicAdd(reinterpret_cast<unsigned long long*>(p.out + (int64_t)o * p.o_outer + (int64_t)col * p.o_col), (unsigned long long)v);
@@ -714,21 +730,22 @@ bool bit_count_cols_launch(const cumo_hip_bit_count_nd_t* d) {
     p.pos = d->pos;
     p.cols = (uint32_t)d->out_shape[L];
     p.chunks = (p.cols + 31u) / 32u;
-    p.chunk_blocks = (p.chunks + 63u) / 64u;
+    p.chunk_blocks = (p.chunks + 31u) / 32u;
     p.rows = (uint32_t)d->red_shape[0];
     p.n_outer = L == 1 ? (uint32_t)d->out_shape[0] : 1u;
     p.s_red = d->in_red_step[0];
     p.s_outer = L == 1 ? d->in_out_step[0] : 0;
     p.o_outer = L == 1 ? d->out_step[0] : 0;
     p.o_col = d->out_step[L];
-    // two blocks for every compute unit where the rows allow it, stretches of 32 rows or more per wave
+    // a block for every compute unit where the rows allow it (with two, the atomics at the end double and
+    // [16384,32768] takes 28 us instead of 25), stretches of 32 rows or more per lane
     const uint64_t across = (uint64_t)p.chunk_blocks * p.n_outer;
-    uint64_t parts = ((uint64_t)kNumCU * 2 + across - 1) / across;
-    const uint64_t most = ((uint64_t)p.rows + 32 * 16 - 1) / (32 * 16);
+    uint64_t parts = ((uint64_t)kNumCU + across - 1) / across;
+    const uint64_t most = ((uint64_t)p.rows + 32 * 32 - 1) / (32 * 32);
     if (parts > most) parts = most;
     if (parts < 1) parts = 1;
-    p.rows_per_wave = (uint32_t)(((uint64_t)p.rows + parts * 16 - 1) / (parts * 16));
-    p.row_parts = (uint32_t)(((uint64_t)p.rows + (uint64_t)p.rows_per_wave * 16 - 1) / ((uint64_t)p.rows_per_wave * 16));
+    p.rows_per_wave = (uint32_t)(((uint64_t)p.rows + parts * 32 - 1) / (parts * 32));
+    p.row_parts = (uint32_t)(((uint64_t)p.rows + (uint64_t)p.rows_per_wave * 32 - 1) / ((uint64_t)p.rows_per_wave * 32));
     const uint64_t blocks = across * p.row_parts;
     if (blocks > 0x7fffffffull) return false;
     const dim3 g((unsigned)blocks), b(kCountColsBlock);
