@@ -159,6 +159,11 @@ def test_rows_of_bits_in_views_word_by_word():
                 assert (da.eq(db).to_numpy() == oracle.bit_binary("eq", va, vb)).all(), (shape, ka, kb)
             assert ((~a[ka]).to_numpy() == oracle.bit_binary("not", ha[ka])).all(), (shape, ka)
             assert (a[ka].copy().to_numpy() == ha[ka]).all(), (shape, ka)
+        # an operand that repeats down the rows, on either side
+        first = (0,) * (len(shape) - 1)
+        assert ((a & b[first]).to_numpy() == (ha & hb[first])).all(), shape
+        assert ((b[first] ^ a[..., :]).to_numpy() == (hb[first] ^ ha)).all(), shape
+        assert ((a[..., 1:] | b[first][1:]).to_numpy() == (ha[..., 1:] | hb[first][1:])).all(), shape
         # into a window of an existing array
         for key, src_key in (((Ellipsis, slice(1, None)), (Ellipsis, slice(None, -1))), ((slice(1, None), Ellipsis, slice(3, 33)), (slice(None, -1), Ellipsis, slice(0, 30)))):
             hz = rng.integers(0, 2, size=shape).astype(np.uint8)
@@ -214,7 +219,8 @@ def test_counts_down_columns_and_along_long_rows():
             assert (b.any_p(axis=ax).to_numpy() == h.any(axis=ax)).all(), (shape, ax)
             assert (b.none_p(axis=ax).to_numpy() == ~h.any(axis=ax)).all(), (shape, ax)
         for key in ((Ellipsis, slice(3, None)), (Ellipsis, slice(None, None, -1), slice(1, -1)), (Ellipsis, slice(None, None, 2), slice(5, 69)),
-                    (Ellipsis, slice(128, None)), (Ellipsis, slice(None, None, 3), slice(64, 64 + 128))):
+                    (Ellipsis, slice(128, None)), (Ellipsis, slice(None, None, 3), slice(64, 64 + 128)),
+                    (Ellipsis, slice(None, None, -1), slice(None)), (Ellipsis, slice(None, None, -2), slice(32, None))):
             v, dv = h[key], b[key]
             if v.size == 0:
                 continue
