@@ -504,6 +504,18 @@ struct MinMaxImpl {
         b.template accumulate_n<N>(x, idx0, h);
         acc.hi = One{h.value, h.index};
     }
+    // a whole step at once: each end runs its own group rule (one comparison when nothing in the
+    // step can change that end)
+    static constexpr bool GROUPED = true;
+    template <int U, int N>
+    __device__ __forceinline__ void accumulate_group(const T (&x)[U][N], const int64_t (&idx)[U], Acc& acc) const {
+        ArgImpl<T, false, NAN_WINS> a{0};
+        ArgImpl<T, true, NAN_WINS> b{0};
+        a.template accumulate_group<U, N>(x, idx, acc.lo);
+        typename ArgImpl<T, true, NAN_WINS>::Acc h{acc.hi.value, acc.hi.index};
+        b.template accumulate_group<U, N>(x, idx, h);
+        acc.hi = One{h.value, h.index};
+    }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const {
         if (out_mode == 0) {
             *reinterpret_cast<T*>(out) = acc.lo.value;

@@ -277,6 +277,10 @@ def test_numbers_to_bits_of_a_whole_array_and_of_windows(tname, dt):
         z[1, ..., 1:] = d[..., :-1]            # a window that starts inside a word
         hz[1, ..., 1:] = want[..., :-1]
         assert (z.to_numpy() == hz).all(), shape
+        for one in (3, 0):                     # a single number spread over the array
+            z1 = cumo_amd.Bit.cast(rng.integers(0, 2, size=shape).astype(np.uint8))
+            z1.store(cls.cast(np.array([one], dtype=dt)))
+            assert (z1.to_numpy() == (1 if one else 0)).all(), (shape, one)
         if len(shape) == 2:
             z2 = cumo_amd.Bit.cast(np.zeros(shape, dtype=np.uint8))
             z2.store(d[:1])                    # one row repeated down the array
