@@ -864,8 +864,16 @@ extern "C" int cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, siz
 
 extern "C" void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* d) {
     if (!d) return;
+    // (counts of whole-word rows can be stored; every other kernel adds, onto results that hold zero)
+    const int L = d->out_ndim - 1;
+    const bool down_columns = d->red_ndim == 1 && d->out_ndim >= 1 && d->in_out_step[L] == 1;
+    if (!down_columns && bit_count_rows_reduce(d)) return;
+    if (d->overwrite) {
+        size_t outs = 1;
+        for (int k = 0; k < d->out_ndim; ++k) outs *= d->out_shape[k];
+        if (outs) cumo_hip_memset(d->out, 0, outs * 8);
+    }
     if (bit_count_cols_launch(d)) return;
-    if (bit_count_rows_reduce(d)) return;
     BitCountNd p;
     std::memset(&p, 0, sizeof(p));
     p.out_ndim = d->out_ndim;

@@ -65,7 +65,7 @@ int cumo_hip::bit_count_run_reduce(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, in
     return launch<false>(&arg, first_mask, last_mask, (int64_t)nw - 1, count_false != 0) ? 1 : 0;
 }
 
-// Counts along the innermost dimension, added onto the results, where every run is whole words: the
+// Counts along the innermost dimension, added onto the results (or stored, with `overwrite`), where every run is whole words: the
 // runs start on words (pos and the kept dimensions' steps are multiples of 32), run along the bits and
 // are a multiple of 32 long. Returns 1 when launched, 0 when the loop is not of that kind.
 int cumo_hip::bit_count_rows_reduce(const cumo_hip_bit_count_nd_t* d) {
@@ -92,5 +92,6 @@ int cumo_hip::bit_count_rows_reduce(const cumo_hip_bit_count_nd_t* d) {
     arg.out_indexer.ndim = (unsigned char)d->out_ndim;
     arg.out_indexer.total_size = outs;
     if (outs == 0 || nw == 0) return 0;
+    if (d->overwrite) return launch<false>(&arg, 0xffffffffu, 0xffffffffu, (int64_t)nw - 1, d->count_false != 0) ? 1 : 0;
     return launch<true>(&arg, 0xffffffffu, 0xffffffffu, (int64_t)nw - 1, d->count_false != 0) ? 1 : 0;
 }

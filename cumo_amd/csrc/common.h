@@ -37,7 +37,7 @@ uint64_t* red_handover_words(int slot, uint32_t* launch_number);
 // Bit counts through the reduction kernels (bit_count_reduce.hip): 1 when launched, 0 when the run or
 // the loop is not one they take (the caller then uses the Bit kernels' own forms).
 int bit_count_run_reduce(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, int count_false, uint64_t* out);
-int bit_count_rows_reduce(const cumo_hip_bit_count_nd_t* counts);
+int bit_count_rows_reduce(const cumo_hip_bit_count_nd_t* counts);  // (stores the counts when counts->overwrite, adds them otherwise)
 
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)

@@ -800,6 +800,7 @@ void iter_bit_unary(LP* lp) {  // gen/tmpl_bit/unary.c
 // host-walked loop of ndloop.c:1569-1613).
 struct CountOpt {
     bool count_false;
+    bool overwrite;  // the results need not hold zero: the launcher sees to it (only the launch for every output at once takes this)
 };
 void count_walk(const LP* lp, int level, size_t pos, char* optr, bool count_false) {
     const cumo_hip_loop_args_t& in = lp->args[0];
@@ -851,6 +852,7 @@ void iter_bit_count(LP* lp) {
     d.pos = lp->args[0].bitpos;
     d.out = lp->args[1].ptr;
     d.count_false = count_false ? 1 : 0;
+    d.overwrite = ((CountOpt*)lp->opt_ptr)->overwrite ? 1 : 0;
     cumo_hip_bit_count_nd_kernel_launch(&d);
 }
 
@@ -2282,11 +2284,13 @@ int cumo_hip_na_bit_count(const cumo_hip_narray_t* x, unsigned int reduce, int k
         if (cumo_hip_bit_count_run_store_kernel_launch(a, lp.args[0].bitpos % 32, lp.n[0], count_false != 0, (uint64_t*)lp.args[1].ptr))
             return CUMO_HIP_OK;
     }
-    // the launchers add onto the result: start from 0 (ndloop.c:853-860)
+    // the launchers add onto the result: start from 0 (ndloop.c:853-860). The launch that takes every
+    // output at once zeroes the results itself where its kernel adds, and not where it stores.
+    const bool at_once = total_of(x) != 0 && !(lp.ndim - lp.reduce_dim == 0 && lp.reduce_dim == 1);
     size_t zbytes = total_of(z) * 8;
-    if (zbytes) cumo_hip_memset(z->ptr + z->offset, 0, zbytes);
+    if (zbytes && !at_once) cumo_hip_memset(z->ptr + z->offset, 0, zbytes);
     if (total_of(x) == 0) return CUMO_HIP_OK;
-    CountOpt opt = {count_false != 0};
+    CountOpt opt = {count_false != 0, at_once};
     lp.opt_ptr = &opt;
     iter_bit_count(&lp);
     return lp.status;

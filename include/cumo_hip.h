@@ -549,7 +549,10 @@ int cumo_hip_last_error(const char** message);
  * reference, whose ndloop walks every output on the host and launches one run at a
  * time, narray/ndloop.c:1569-1613 under gen/tmpl_bit/bit_count.c:9-36). The loop is
  * given as kept dimensions then reduced dimensions; input steps and pos are in bits,
- * output steps in bytes; the counts are ADDED onto the uint64 results. */
+ * output steps in bytes; the counts are ADDED onto the uint64 results, or, with
+ * `overwrite` set, REPLACE them: the results (out_total contiguous uint64 from `out`,
+ * out_step that of a contiguous array) then need not hold zero, and the launcher
+ * zeroes them itself where its kernel adds. */
 typedef struct {
     int      out_ndim, red_ndim;
     size_t   out_shape[CUMO_NA_MAX_DIMENSION], red_shape[CUMO_NA_MAX_DIMENSION];
@@ -559,6 +562,7 @@ typedef struct {
     size_t   pos;
     char*    out;
     int      count_false;
+    int      overwrite;
 } cumo_hip_bit_count_nd_t;
 void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* counts);
 /* *out = the count over one contiguous run of bits, in one launch that neither needs
