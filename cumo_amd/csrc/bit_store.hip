@@ -123,6 +123,24 @@ void launch_reduce_gather(CUMO_BIT_DIGIT* a1, size_t p1, ssize_t s1, size_t* idx
     cumo_cuda_runtime_check_kernel_launch();
 }
 
+// ---- counts -> bits -----------------------------------------------------------------
+// bit i of the run that starts at bit `pos` of dst = (counts[i] != 0), or (counts[i] == 0) with
+// zero_is_one: what all? / any? along axes make of the counts of clear / set bits. A lane packs one
+// word of the run; the bits of the run's first and last word that lie outside it stay.
+__global__ __launch_bounds__(kBlock) void bit_from_counts_kernel(const uint64_t* counts, uint64_t n, int zero_is_one, CUMO_BIT_DIGIT* dst, uint64_t pos) {
+    const uint64_t nw = (pos + n + 31) >> 5;
+    for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < nw; w += (uint64_t)gridDim.x * kBlock) {
+        uint32_t word = 0u;
+        for (unsigned j = 0; j < 32; ++j) {
+            const uint64_t q = (w << 5) + j;  // bit position in dst
+            if (q < pos || q >= pos + n) continue;
+            const bool zero = counts[q - pos] == 0;
+            if (zero == (zero_is_one != 0)) word |= 1u << j;
+        }
+        store_word_masked(dst, w, word, run_mask(pos, n, w));
+    }
+}
+
 // ---- fill --------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void bit_fill_words_kernel(CUMO_BIT_DIGIT* a3, uint64_t p3, uint64_t n, uint32_t word) {
     const uint64_t w0 = p3 >> 5, w1 = (p3 + n + 31) >> 5;
@@ -283,4 +301,13 @@ extern "C" void cumo_iter_bit_store_array_index_scalar_kernel_launch(CUMO_BIT_DI
 }
 extern "C" void cumo_iter_bit_store_array_stride_scalar_kernel_launch(CUMO_BIT_DIGIT* a1, size_t p1, ssize_t s1, CUMO_BIT_DIGIT z, uint64_t n) {
     launch_store_array_scatter(a1, p1, s1, nullptr, nullptr, z, 1, n);
+}
+
+extern "C" void cumo_hip_bit_from_counts_kernel_launch(const uint64_t* counts, uint64_t n, int zero_is_one, CUMO_BIT_DIGIT* dst, size_t pos) {
+    if (n == 0) return;
+    dst += pos / 32;
+    pos %= 32;
+    hipLaunchKernelGGL(bit_from_counts_kernel, dim3(grid_for((pos + n + 31) / 32)), dim3(kBlock), 0, current_stream(), counts, n, zero_is_one, dst,
+                       (uint64_t)pos);
+    cumo_cuda_runtime_check_kernel_launch();
 }

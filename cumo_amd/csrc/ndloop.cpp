@@ -2317,15 +2317,24 @@ int cumo_hip_na_bit_reduce(const char* op, const cumo_hip_narray_t* x, unsigned 
     rc = cumo_hip_na_ndloop_prepare(&nf, in, out, reduce, &lp);
     if (rc) return rc;
     if (total_of(z) == 0) return CUMO_HIP_OK;
-    rc = cumo_hip_na_fill(z, all ? 1.0 : 0.0);
-    if (rc || total_of(x) == 0) return rc;
-
     size_t runs = 1;
     for (int d = 0; d + 1 < lp.ndim; d++) runs *= lp.n[d];
-    if (lp.ndim == 0 || runs > 32) {
+    const bool by_counts = total_of(x) != 0 && (lp.ndim == 0 || runs > 32);  // (every bit of the result gets written then)
+    if (!by_counts) {
+        rc = cumo_hip_na_fill(z, all ? 1.0 : 0.0);
+        if (rc || total_of(x) == 0) return rc;
+    }
+    if (by_counts) {
         NA counts;
         std::memset(&counts, 0, sizeof(counts));
         rc = cumo_hip_na_bit_count(x, reduce, keepdims, all ? 1 : 0, &counts);
+        if (!rc && is_contiguous(z) && is_contiguous(&counts) && z->offset >= 0 && total_of(&counts) == total_of(z)) {
+            // any? = some bit set, all? = no bit clear: packed from the counts in one launch
+            cumo_hip_bit_from_counts_kernel_launch((const uint64_t*)(counts.ptr + counts.offset), total_of(z), all ? 1 : 0, (CUMO_BIT_DIGIT*)z->ptr,
+                                                   (size_t)z->offset);
+            free_tmp(&counts);
+            return CUMO_HIP_OK;
+        }
         if (!rc) rc = cumo_hip_na_store(z, &counts);  // nonzero -> 1
         free_tmp(&counts);
         if (!rc && all) rc = cumo_hip_na_bit_unary("not", z, z);

@@ -571,6 +571,11 @@ void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_t* counts);
  * bit pos%32 onwards, n bits. Returns 1 when launched, 0 when the caller has to take
  * the zero-fill + accumulate route. */
 int  cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, int count_false, uint64_t* out);
+/* Bits from counts: bit pos + i of dst = (counts[i] != 0), or (counts[i] == 0) with zero_is_one; n contiguous
+ * uint64 counts. What all? / any? along axes make of the counts of clear / set bits along them (no counterpart
+ * in the reference, which walks the runs on the host: gen/tmpl_bit/bit_reduce.c:106-146). Bits of dst outside
+ * [pos, pos + n) stay as they are. */
+void cumo_hip_bit_from_counts_kernel_launch(const uint64_t* counts, uint64_t n, int zero_is_one, CUMO_BIT_DIGIT* dst, size_t pos);
 
 /* Row-wise softmax and layer normalisation in one pass (no counterpart in the
  * reference, where they are chains of 5 and 6 array operations,
