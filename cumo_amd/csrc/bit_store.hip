@@ -125,19 +125,22 @@ void launch_reduce_gather(CUMO_BIT_DIGIT* a1, size_t p1, ssize_t s1, size_t* idx
 
 // ---- counts -> bits -----------------------------------------------------------------
 // bit i of the run that starts at bit `pos` of dst = (counts[i] != 0), or (counts[i] == 0) with
-// zero_is_one: what all? / any? along axes make of the counts of clear / set bits. A lane packs one
-// word of the run; the bits of the run's first and last word that lie outside it stay.
+// zero_is_one: what all? / any? along axes make of the counts of clear / set bits. The bits of the
+// run's first and last word that lie outside it stay.
 __global__ __launch_bounds__(kBlock) void bit_from_counts_kernel(const uint64_t* counts, uint64_t n, int zero_is_one, CUMO_BIT_DIGIT* dst, uint64_t pos) {
-    const uint64_t nw = (pos + n + 31) >> 5;
-    for (uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x; w < nw; w += (uint64_t)gridDim.x * kBlock) {
-        uint32_t word = 0u;
-        for (unsigned j = 0; j < 32; ++j) {
-            const uint64_t q = (w << 5) + j;  // bit position in dst
-            if (q < pos || q >= pos + n) continue;
-            const bool zero = counts[q - pos] == 0;
-            if (zero == (zero_is_one != 0)) word |= 1u << j;
+    // lane t of the grid owns bit t of dst (pos < 32): a wave's ballot packs 64 of them, and the lanes at 0 and 32 store the two words
+    const uint64_t span = pos + n;
+    const uint64_t rounds = (span + (uint64_t)gridDim.x * kBlock - 1) / ((uint64_t)gridDim.x * kBlock);
+    for (uint64_t r = 0; r < rounds; ++r) {
+        const uint64_t q = (r * gridDim.x + blockIdx.x) * (uint64_t)kBlock + threadIdx.x;  // whole waves stay together
+        bool on = false;
+        if (q >= pos && q < span) on = (counts[q - pos] == 0) == (zero_is_one != 0);
+        const uint64_t ballot = __ballot(on);
+        const unsigned lane = threadIdx.x & 63;
+        if ((lane & 31) == 0) {
+            const uint64_t w = q >> 5;
+            store_word_masked(dst, w, (uint32_t)(ballot >> lane), run_mask(pos, n, w));
         }
-        store_word_masked(dst, w, word, run_mask(pos, n, w));
     }
 }
 
@@ -307,7 +310,7 @@ extern "C" void cumo_hip_bit_from_counts_kernel_launch(const uint64_t* counts, u
     if (n == 0) return;
     dst += pos / 32;
     pos %= 32;
-    hipLaunchKernelGGL(bit_from_counts_kernel, dim3(grid_for((pos + n + 31) / 32)), dim3(kBlock), 0, current_stream(), counts, n, zero_is_one, dst,
+    hipLaunchKernelGGL(bit_from_counts_kernel, dim3(grid_for(pos + n)), dim3(kBlock), 0, current_stream(), counts, n, zero_is_one, dst,
                        (uint64_t)pos);
     cumo_cuda_runtime_check_kernel_launch();
 }
