@@ -3,7 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--all-configs] [--no-cpu]
 
-Prints ONE JSON line. A "step" is one pass of the headline workload (BASELINE.json
+The last stdout line is ONE compact JSON line (headline, roofline, cpu_baseline and a
+per-op map of fractions of peak); the full per-op tables go to gpurun_out/bench_full.json
+(--full-out). A "step" is one pass of the headline workload (BASELINE.json
 configs[1]: DFloat broadcast add + row reductions) with the inputs already resident
 in HBM: C = A + r; C.sum(axis:1); C.max(axis:1) -- three launches through the
 C-ABI. `value` is algorithmic bytes per step / seconds per step in GB/s, where
@@ -486,8 +488,56 @@ def cpu_baseline_c2(budget_s=12.0):
     }
 
 
+FINAL_LINE_MAX = 6000  # bytes: the last stdout line must stay small enough for any log tail to hold it whole
+
+
+def compact(out):
+    """The result as the last stdout line carries it: every headline field, `roofline` and
+    `cpu_baseline` whole, and of the per-op tables only `op -> fraction of HBM peak`
+    (3 decimals). The full tables go to a file (write_full)."""
+    c = {k: v for k, v in out.items() if k not in ("per_config", "host_io", "host_cost")}
+    if "per_config" in out:
+        c["per_config"] = {name: {o["op"]: round(o["frac_of_peak"], 3) for o in cfg["ops"]}
+                           for name, cfg in out["per_config"].items()}
+    hc = out.get("host_cost")
+    if isinstance(hc, dict) and "launcher_add" in hc:
+        c["host_cost_us"] = {k: hc[k] for k in ("empty_launch", "launcher_add", "add_alloc_free", "sum_alloc_free") if k in hc}
+    return c
+
+
+def final_line(out, full_path=None):
+    """One JSON line of at most FINAL_LINE_MAX bytes. Should the compact form ever outgrow
+    that, the per-op map is dropped first: the headline, roofline and cpu_baseline always fit."""
+    c = compact(out)
+    if full_path:
+        c["full_results"] = full_path
+    line = json.dumps(c)
+    if len(line) > FINAL_LINE_MAX:
+        c.pop("per_config", None)
+        c["per_config_omitted"] = "see full_results"
+        line = json.dumps(c)
+    if len(line) > FINAL_LINE_MAX:
+        raise SystemExit("bench: the result line is %d bytes, over the %d-byte limit" % (len(line), FINAL_LINE_MAX))
+    return line
+
+
+def write_full(out, path):
+    """Every table of the run (per-op timings, host transfer rates, host cost) as indented
+    JSON. Returns the path relative to this file's folder, or None when it cannot be written."""
+    try:
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump(out, f, indent=1)
+            f.write("\n")
+        return os.path.relpath(path, ROOT)
+    except OSError:
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--full-out", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"),
+                    help="file that receives the full per-op tables (the last stdout line holds a compact form)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -668,7 +718,8 @@ def main():
         if not args.no_extras:
             out["host_io"] = measure_host_io(lib)
             out["host_cost"] = measure_host_cost()
-    print(json.dumps(out))
+    full_path = write_full(out, args.full_out)
+    print(final_line(out, full_path))
 
 
 if __name__ == "__main__":
