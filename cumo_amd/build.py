@@ -39,39 +39,61 @@ def sources():
     return out
 
 
-def headers_mtime():
-    newest = 0.0
-    for d in (CSRC, os.path.join(ROOT, "include")):
-        for name in os.listdir(d):
-            if name.endswith((".h", ".inc")):
-                newest = max(newest, os.path.getmtime(os.path.join(d, name)))
-    return newest
-
-
-def compile_one(src, force, hdr_mtime):
-    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
-    if not force and os.path.exists(obj):
+def deps_newer_than(obj):
+    """True when the source or any header the object was compiled from (its .d file, written
+    by -MD) is newer than the object, or when that list is missing."""
+    dep = obj + ".d"
+    try:
         m = os.path.getmtime(obj)
-        if m > os.path.getmtime(src) and m > hdr_mtime:
-            return obj, "", 0
+        with open(dep) as f:
+            text = f.read()
+    except OSError:
+        return True
+    text = text.replace("\\\n", " ")
+    files = text.split(":", 1)[1].split() if ":" in text else []
+    if not files:
+        return True
+    for path in files:
+        try:
+            if os.path.getmtime(path) > m:
+                return True
+        except OSError:
+            return True
+    return False
+
+
+def compile_one(src, force):
+    obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+    if not force and not deps_newer_than(obj):
+        return obj, "", 0
+    dep = ["-MD", "-MF", obj + ".d"]
     if src.endswith(".hip"):
-        cmd = [HIPCC] + DEVICE + COMMON + ["-c", "-x", "hip", src, "-o", obj]
+        cmd = [HIPCC] + DEVICE + COMMON + dep + ["-c", "-x", "hip", src, "-o", obj]
     else:
-        cmd = [HIPCC] + COMMON + ["-x", "hip", "--offload-arch=" + ARCH, "-c", src, "-o", obj]
+        cmd = [HIPCC] + COMMON + dep + ["-x", "hip", "--offload-arch=" + ARCH, "-c", src, "-o", obj]
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     log = "\n".join(l for l in p.stdout.splitlines() if "packed-fp32-ops' is not a recognized feature" not in l)
     return obj, log, p.returncode
 
 
+def drop_stale_objects(srcs):
+    """Objects (and their dependency lists) whose source file no longer exists."""
+    keep = {os.path.basename(s) + ".o" for s in srcs}
+    for name in os.listdir(OBJ):
+        base = name[:-2] if name.endswith(".d") else name
+        if base.endswith(".o") and base not in keep:
+            os.remove(os.path.join(OBJ, name))
+
+
 def build(jobs=None, force=False, verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
-    hdr = headers_mtime()
     srcs = sources()
+    drop_stale_objects(srcs)
     objs = []
     failed = False
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        futs = {ex.submit(compile_one, s, force, hdr): s for s in srcs}
+        futs = {ex.submit(compile_one, s, force): s for s in srcs}
         for f in concurrent.futures.as_completed(futs):
             obj, log, rc = f.result()
             if verbose and (log.strip() or rc):

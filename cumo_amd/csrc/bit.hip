@@ -781,6 +781,9 @@ CUMO_DEF_BIT_BINARY(xor, B_XOR)
 CUMO_DEF_BIT_BINARY(eq, B_EQ)
 CUMO_DEF_BIT_UNARY(copy, B_COPY)
 CUMO_DEF_BIT_UNARY(not, B_NOT)
+// Bit#store(Bit): the same word-wise / per-bit copy as `copy`, with the receiver as a3
+// (narray/gen/tmpl_bit/store_bit.c:1-2, store_bit_kernel.cu:21,38)
+CUMO_DEF_BIT_UNARY(store_bit, B_COPY)
 
 #define CUMO_DEF_BIT_COUNT(name, CF)                                                                                          \
     extern "C" void cumo_iter_bit_##name##_index_kernel_launch(size_t p1, char* p2, CUMO_BIT_DIGIT* a1, size_t* idx1,         \

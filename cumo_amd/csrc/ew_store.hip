@@ -71,6 +71,12 @@ CUMO_DEF_FILL(sfloat, float)
 CUMO_DEF_FILL(dfloat, double)
 CUMO_DEF_FILL(int32, int32_t)
 
+// the common new_dim0 template rendered for Bit: one whole word
+extern "C" void cumo_bit_new_dim0_kernel_launch(unsigned int* ptr, unsigned int x) {
+    hipLaunchKernelGGL((set_one_kernel<unsigned int>), dim3(1), dim3(1), 0, current_stream(), ptr, x);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
 // A fill kernel rather than hipMemsetAsync, so that a caller may capture it.
 extern "C" void cumo_hip_memset(void* dst, int byte, size_t n) {
     if (n == 0) return;

@@ -481,6 +481,8 @@ struct BitUnaryRow {
 };
 #define BITU_ROW(op) {#op, cumo_iter_bit_##op##_kernel_launch, cumo_iter_bit_##op##_contiguous_kernel_launch},
 const BitUnaryRow kBitUnary[] = {CUMO_HIP_BIT_UNARY_OPS(BITU_ROW)};
+// Bit#store(Bit) has launchers of its own (gen/tmpl_bit/store_bit.c:1-2)
+const BitUnaryRow kBitStoreBit = {"store_bit", cumo_iter_bit_store_bit_kernel_launch, cumo_iter_bit_store_bit_contiguous_kernel_launch};
 
 template <class Row, size_t N>
 const Row* find_row(const Row (&rows)[N], const char* op) {
@@ -1961,9 +1963,8 @@ int cumo_hip_na_store(cumo_hip_narray_t* dst, const cumo_hip_narray_t* src) {
             opt = &copt;
         }
     } else if (dst->type == CUMO_HIP_BIT) {
-        const BitUnaryRow* row = find_row(kBitUnary, "copy");
         nf.func = iter_bit_unary;  // args: src, dst
-        opt = (void*)row;
+        opt = (void*)&kBitStoreBit;
     } else if (!is_arith(dst->type)) {
         return fail(CUMO_HIP_ERROR_TYPE, "store: destination must be SFloat, DFloat, Int32 or Bit");
     } else if (src->type == CUMO_HIP_BIT) {

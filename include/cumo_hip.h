@@ -189,6 +189,11 @@ size_t* cumo_cuda_runtime_error_item_new(void);
     void cumo_##t##_new_dim0_kernel_launch(c *ptr, c x); \
     void cumo_iter_##t##_store_bit_kernel_launch(cumo_na_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_indexer_t* indexer);
 
+/* Bit has no new_dim0 template of its own, so the generator renders the common one for it
+ * (gen/cogen.rb:37-39 searches tmpl_bit, then tmpl; tmpl/new_dim0_kernel.cu:2-10 with dtype =
+ * BIT_DIGIT): the whole first word of a 0-dim Bit array becomes x. */
+void cumo_bit_new_dim0_kernel_launch(unsigned int *ptr, unsigned int x);
+
 CUMO_HIP_BINARY_OPS_ALL(CUMO_HIP_DECL_BINARY, sfloat, float)
 CUMO_HIP_BINARY_OPS_ALL(CUMO_HIP_DECL_BINARY, dfloat, double)
 CUMO_HIP_BINARY_OPS_ALL(CUMO_HIP_DECL_BINARY, int32, int32_t)
@@ -445,6 +450,11 @@ int cumo_hip_sfloat_sum_noalloc_kernel_launch(cumo_na_reduction_arg_t* arg);
 
 CUMO_HIP_BIT_BINARY_OPS(CUMO_HIP_DECL_BIT_BINARY)
 CUMO_HIP_BIT_UNARY_OPS(CUMO_HIP_DECL_BIT_UNARY)
+/* Bit#store(Bit) (narray/gen/tmpl_bit/store_bit.c:1-2, kernels store_bit_kernel.cu:1-47;
+ * generated for class Bit by gen/spec.rb:125 `store_from "Bit"`): a1 is the source, a3 the
+ * receiver; the contiguous form takes word pointers with bit offsets below 32 and writes
+ * only the n bits it names. */
+CUMO_HIP_DECL_BIT_UNARY(store_bit)
 CUMO_HIP_DECL_BIT_COUNT(count_true)
 CUMO_HIP_DECL_BIT_COUNT(count_false)
 

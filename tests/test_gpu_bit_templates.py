@@ -311,6 +311,86 @@ def test_typed_stridx_store_and_store_array(tname, dtype, ctype):
     free(pz, pidx)
 
 
+@pytest.mark.parametrize("n", [1, 5, 31, 32, 33, 64, 95, 1000, 100003, (1 << 21) + 19])
+def test_bit_store_bit_contiguous(n):
+    # tmpl_bit/store_bit.c:2 / store_bit_kernel.cu:38-47: word pointers + bit offsets below 32,
+    # only the n named bits of the receiver change
+    L = lib()
+    f = L.fn("cumo_iter_bit_store_bit_contiguous_kernel_launch", None, [VP, SZ, VP, SZ, U64])
+    rng = np.random.default_rng(n)
+    for p1, p3 in ((0, 0), (0, 13), (13, 0), (7, 7), (31, 1), (1, 31), (19, 30)):
+        src = rng.integers(0, 2, size=p1 + n + 70).astype(np.uint8)
+        before = rng.integers(0, 2, size=p3 + n + 70).astype(np.uint8)
+        pa, pz = dev(pack(src)), dev(pack(before))
+        L.call(f, pa, p1, pz, p3, n)
+        want = before.copy()
+        want[p3:p3 + n] = src[p1:p1 + n]
+        got = unpack(fetch(pz, (before.size + 31) // 32, np.uint32), before.size)
+        assert (got == want).all(), (n, p1, p3, np.flatnonzero(got != want)[:8])
+        free(pa, pz)
+
+
+def test_bit_store_bit_general_views():
+    # tmpl_bit/store_bit.c:1 / store_bit_kernel.cu:1-19: both operands through their own
+    # stride-or-index entries: reversed, stepped, 2-d with a column index array, broadcast source
+    L = lib()
+    g = L.fn("cumo_iter_bit_store_bit_kernel_launch", None, [P(L.BitIArrayStridx), P(L.BitIArrayStridx), P(L.Indexer)])
+    rng = np.random.default_rng(11)
+
+    def run(shape, spos, ssteps, dpos, dsteps, nsrc, ndst, sidx=None, didx=None):
+        src = rng.integers(0, 2, size=nsrc).astype(np.uint8)
+        before = rng.integers(0, 2, size=ndst).astype(np.uint8)
+        pa, pz = dev(pack(src)), dev(pack(before))
+        a1, a3 = L.BitIArrayStridx(), L.BitIArrayStridx()
+        a1.ptr, a1.pos, a3.ptr, a3.pos = pa, spos, pz, dpos
+        held = []
+        for d in range(len(shape)):
+            for a, steps, idx in ((a1, ssteps, sidx), (a3, dsteps, didx)):
+                if idx is not None and idx[0] == d:
+                    p = dev(idx[1].astype(np.uint64))
+                    held.append(p)
+                    a.stridx[d] = p
+                else:
+                    a.stridx[d] = stride_sdx(steps[d])
+        ix = indexer(shape)
+        L.call(g, C.byref(a1), C.byref(a3), C.byref(ix))
+        want = before.copy()
+        for pos in np.ndindex(*shape):
+            so, do = spos, dpos
+            for d, i in enumerate(pos):
+                so += int(sidx[1][i]) if sidx is not None and sidx[0] == d else ssteps[d] * i
+                do += int(didx[1][i]) if didx is not None and didx[0] == d else dsteps[d] * i
+            want[do] = src[so]
+        got = unpack(fetch(pz, (ndst + 31) // 32, np.uint32), ndst)
+        assert (got == want).all(), (shape, spos, ssteps, dpos, dsteps, np.flatnonzero(got != want)[:8])
+        free(pa, pz, *held)
+
+    for n in (1, 33, 64, 65, 777):
+        run((n,), 3, (1,), 5 + n - 1, (-1,), n + 10, n + 10)               # receiver reversed
+        run((n,), 2 * n + 1, (-2,), 9, (3,), 2 * n + 5, 3 * n + 12)         # source reversed with step 2, receiver step 3
+        run((n,), 17, (0,), 1, (1,), 40, n + 40)                            # one source bit broadcast
+    run((37, 45), 4, (100, 2), 11, (45, 1), 37 * 100 + 20, 37 * 45 + 30)    # 2-d, rows of the receiver end to end at offset 11
+    run((6, 41), 7, (200, 0), 3, (300, 0), 7 + 6 * 200, 3 + 6 * 300,        # index arrays along the columns of both
+        sidx=(1, (np.arange(41) * 4 + 1) % 190), didx=(1, (np.arange(41) * 7 + 2)))
+    run((3, 4, 5, 6, 7), 0, (840, 210, 42, 7, 1), 6, (900, 215, 43, 7, 1), 2520, 2800)   # 5-d (past the unrolled cases)
+
+
+def test_bit_store_bit_empty():
+    L = lib()
+    f = L.fn("cumo_iter_bit_store_bit_contiguous_kernel_launch", None, [VP, SZ, VP, SZ, U64])
+    g = L.fn("cumo_iter_bit_store_bit_kernel_launch", None, [P(L.BitIArrayStridx), P(L.BitIArrayStridx), P(L.Indexer)])
+    before = np.array([0xdeadbeef, 0x01234567], dtype=np.uint32)
+    pa, pz = dev(before), dev(before)
+    L.call(f, pa, 3, pz, 5, 0)
+    a1, a3 = L.BitIArrayStridx(), L.BitIArrayStridx()
+    a1.ptr, a3.ptr = pa, pz
+    a1.stridx[0] = a3.stridx[0] = stride_sdx(1)
+    ix = indexer((0,))
+    L.call(g, C.byref(a1), C.byref(a3), C.byref(ix))
+    assert (fetch(pz, 2, np.uint32) == before).all()
+    free(pa, pz)
+
+
 # ---- the reference's own cases, through the mirror ---------------------------------------------
 def test_reversed_bit_views_all_any_and_store():
     # test/narray_test.rb:2725-2746
