@@ -154,6 +154,8 @@ def config_ops(name, cumo, host):
             ("mask=E>0.5", lambda e: e.__setitem__("mask", e["E"] > 0.5), 4 * nv + nv // 8, nv),
             ("mask.count_true", lambda e: e.__setitem__("cnt", e["mask"].count_true()), nv // 8 + 8, nv),
             ("I[(0..-1).step(3),true].copy", lambda e: e.__setitem__("Ic", e["I"][::3].copy()), 2 * 4 * rows * i.shape[1], rows * i.shape[1]),
+            # not an op of the config: the same transposed view copied with no arithmetic, the ceiling for E0
+            ("tcopy=V.copy (ceiling of exp(V))", lambda e: e.__setitem__("Vc", e["V"].copy()), 8 * nv, nv),
         ]
     if name == "c5":
         s, x = host["S"], host["X"]
