@@ -23,10 +23,16 @@ hipStream_t current_stream();
 // keep per-stream words in a fixed device array (tickets) index it with this.
 constexpr int kStreamSlots = 64;
 int stream_slot(hipStream_t stream);
-void stream_slot_release(hipStream_t stream);
+int stream_slot_release(hipStream_t stream);  // the number it held, or -1
 
 // pool.cpp: files everything the pool holds for a drained stream under the null stream.
 void pool_retire_stream(hipStream_t stream);
+
+// scan.hip: the regions of look-back words that streams keep from launch to launch. Dropped for
+// a stream slot when its (drained) stream is retired, and all of them by free_all_blocks.
+void scan_chain_words_drop_slot(int slot);
+void scan_chain_words_drop_all();
+size_t scan_chain_words_held_bytes();
 
 // Device address of the reduction ticket words of a stream slot (zero between launches),
 // nullptr after reporting an error. reduce_tickets.hip.
@@ -50,6 +56,27 @@ bool force_wide_indices();
 // touched. CUMO_HIP_NT=0 / 1 (read once) forces the answer.
 constexpr uint64_t kStreamNtBytes = 48ull << 20;
 bool stream_past_caches(uint64_t bytes);
+
+// A kernel that waits for another block's word (the hand-over words of a split reduction, the
+// look-back of a one-pass scan, the totals of a one-launch mulsum) waits a bounded number of
+// looks. One that gives up cannot produce its result: it counts the event and raises the
+// pinned host word, and the next point where the host waits for the device
+// (wait_trouble_check) reports CUMO_HIP_ERROR_RUNTIME, the way a rejected element is
+// reported through the pinned error flag (reference: cuda/runtime.c:22-47).
+struct WaitCtl {
+    uint32_t limit_scale;    // 0: give up at the first failed look (test knob); 1: the kernels' own limits
+    uint32_t reserved;
+    uint32_t* host_flag;     // pinned, device-mapped host word
+    uint32_t gave_up[4];     // counts by family: see WaitFamily
+};
+enum WaitFamily { WAIT_REDUCE = 0, WAIT_SCAN = 1, WAIT_MULSUM = 2 };
+// Device address of the block (allocated and filled on the first call; one per process),
+// nullptr after reporting an error.
+WaitCtl* wait_ctl();
+// Host: reports and clears a raised give-up word. False when one was raised.
+bool wait_trouble_check();
+// Compute units of the current device (queried once).
+int device_compute_units();
 
 static inline bool hip_ok(hipError_t status, const char* what) {
     if (status == hipSuccess) return true;

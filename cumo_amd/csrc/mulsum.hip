@@ -11,6 +11,7 @@
 // scheduling. Products and sums are in the element type, unfused, as the macros
 // write them (types/real_accum_kernel.h:6-10, xint_macro_kernel.h:44).
 #include "common.h"
+#include "wait_ctl.h"
 
 namespace cumo_hip {
 namespace {
@@ -69,7 +70,8 @@ __device__ __forceinline__ T ms_block_sum(T acc) {
 // NT: non-temporal loads, for runs that do not fit the last-level cache anyway
 template <class T, bool NANF, int VEC, bool NT>
 __global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1, const char* p2, int64_t s1, int64_t s2, uint64_t n,
-                                                                  uint64_t chunk, T* partial, T* out, uint64_t* words, uint32_t launch) {
+                                                                  uint64_t chunk, T* partial, T* out, uint64_t* words, uint32_t launch,
+                                                                  WaitCtl* wait) {
     constexpr int W = (int)(sizeof(T) / 4);
     uint32_t block = blockIdx.x;
     if (words) {
@@ -86,7 +88,12 @@ __global__ __launch_bounds__(kMsBlock) void mulsum_partial_kernel(const char* p1
                     const uint64_t* slot = words + (size_t)i * W + k;
                     uint64_t x = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     uint32_t looks = 0;
-                    while ((uint32_t)(x >> 32) != launch && ++looks < (1u << 24)) {
+                    const uint32_t limit = wait_limit(wait, 1u << 24);
+                    while ((uint32_t)(x >> 32) != launch) {
+                        if (++looks > limit) {
+                            wait_gave_up(wait, WAIT_MULSUM);  // the total is not valid; the host is told
+                            break;
+                        }
                         __builtin_amdgcn_s_sleep(4);
                         x = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
@@ -300,6 +307,7 @@ void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, 
     // launch number again), else to scratch from the pool and a second launch
     T* partial = nullptr;
     uint64_t* words = nullptr;
+    WaitCtl* wait = nullptr;
     uint32_t launch = 0;
     if (grid > 1) {
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
@@ -307,7 +315,8 @@ void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, 
             (void)hipGetLastError();
             capturing = hipStreamCaptureStatusActive;
         }
-        if (capturing == hipStreamCaptureStatusNone && grid * (sizeof(T) / 4) <= 8192) words = red_handover_words(stream_slot(stream), &launch);
+        if (capturing == hipStreamCaptureStatusNone && grid * (sizeof(T) / 4) <= 8192 && (wait = wait_ctl()) != nullptr)
+            words = red_handover_words(stream_slot(stream), &launch);
         if (!words) {
             partial = reinterpret_cast<T*>(cumo_cuda_runtime_malloc(sizeof(T) * grid));
             if (!partial) return;
@@ -316,9 +325,9 @@ void mulsum_reduce_launch(char* p1, char* p2, char* p3, ssize_t s1, ssize_t s2, 
     const bool nt = stream_past_caches(2 * n * sizeof(T));
     const dim3 g((unsigned)(words ? grid + 1 : grid)), b(kMsBlock);
     T* out = reinterpret_cast<T*>(p3);
-    if (vec && nt) hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, true>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch);
-    else if (vec) hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, false>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch);
-    else hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1, false>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch);
+    if (vec && nt) hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, true>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch, wait);
+    else if (vec) hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, VEC, false>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch, wait);
+    else hipLaunchKernelGGL((mulsum_partial_kernel<T, NANF, 1, false>), g, b, 0, stream, p1, p2, (int64_t)s1, (int64_t)s2, n, chunk, partial, out, words, launch, wait);
     if (partial) {
         hipLaunchKernelGGL((mulsum_combine_kernel<T>), dim3(1), dim3(kMsBlock), 0, stream, (const T*)partial, grid, out);
         cumo_cuda_runtime_free(reinterpret_cast<char*>(partial));

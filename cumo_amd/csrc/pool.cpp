@@ -371,8 +371,12 @@ void cumo_hip_pool_free_all_blocks(void) {
         std::unique_lock<std::mutex> lock(p.mu);
         rc = p.release_unsplit(false, nullptr);
     }
+    // memory the library holds outside the pool's books: the scans' kept look-back words
+    scan_chain_words_drop_all();
     if (rc < 0) report_hip_error((hipError_t)(-rc), "hipFree");
 }
+
+size_t cumo_hip_pool_held_outside_bytes(void) { return scan_chain_words_held_bytes(); }
 
 void cumo_hip_pool_free_all_blocks_stream(void* hip_stream) {
     Pool& p = g_pool;

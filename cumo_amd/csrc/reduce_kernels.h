@@ -43,6 +43,7 @@
 
 #include "common.h"
 #include "plan.h"
+#include "wait_ctl.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -494,6 +495,7 @@ struct CombineImpl {
 struct RedScratch {
     char* ptr;
     size_t bytes;
+    mutable size_t used;   // set by the launch: bytes of ptr that its kernels write and read (0: none)
 };
 
 static inline unsigned red_grid_cap() {
@@ -723,6 +725,7 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
             if (fixed) {
                 if (scratch_bytes > fixed->bytes) return -1;
                 p.partial = fixed->ptr;
+                fixed->used = scratch_bytes;
             } else {
                 p.partial = cumo_cuda_runtime_malloc(scratch_bytes);
                 if (!p.partial) return 1;  // the pool has reported it
@@ -794,11 +797,17 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
         (void)hipGetLastError();
         capturing = hipStreamCaptureStatusActive;
     }
-    if (!fixed && red_poll_enabled() && capturing == hipStreamCaptureStatusNone && plan.out_total <= 256 &&
+    // The waiting blocks (one per output, started first) may take at most half of what the device
+    // certainly keeps resident beside them (two blocks of this size per compute unit): the blocks
+    // they wait for then always find room. With fewer compute units than this build was tuned for
+    // (a partitioned device) fewer outputs qualify.
+    const uint64_t poll_outputs_max = (uint64_t)device_compute_units() < 256 ? (uint64_t)device_compute_units() : 256;
+    if (!fixed && red_poll_enabled() && capturing == hipStreamCaptureStatusNone && plan.out_total <= poll_outputs_max &&
         plan.out_total * (uint64_t)p.n_split * (sizeof(Acc) / 4) <= kRsHandoverWords) {
         uint32_t launch = 0;
         uint64_t* words = red_handover_words(stream_slot(stream), &launch);
-        if (words != nullptr) {
+        p.wait = words != nullptr ? wait_ctl() : nullptr;
+        if (words != nullptr && p.wait != nullptr) {
             const dim3 g((unsigned)(plan.out_total * p.n_split + plan.out_total));
             if (nt) hipLaunchKernelGGL((red_srow_poll_kernel<Impl, V, true>), g, b, 0, stream, p, impl, words, launch);
             else hipLaunchKernelGGL((red_srow_poll_kernel<Impl, V, false>), g, b, 0, stream, p, impl, words, launch);
@@ -827,6 +836,7 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
     if (fixed) {
         if (scratch_bytes > fixed->bytes) return -1;
         p.partial = fixed->ptr;
+        fixed->used = scratch_bytes;
     } else {
         p.partial = cumo_cuda_runtime_malloc(scratch_bytes);
         if (!p.partial) return 1;  // the pool has reported it
@@ -893,6 +903,7 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     if (fixed) {
         if (sizeof(Acc) * n_partial > fixed->bytes) return false;
         partial = reinterpret_cast<Acc*>(fixed->ptr);
+        fixed->used = sizeof(Acc) * n_partial;
     } else {
         partial = reinterpret_cast<Acc*>(cumo_cuda_runtime_malloc(sizeof(Acc) * n_partial));
         if (!partial) return true;  // the pool has reported it

@@ -23,11 +23,15 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 std::mutex g_lock;
 char* g_scratch_ptr[kMaxDevices];  // per device: address of that device's copy of `scratch`
 
-// The current device's copy of the array; nullptr after reporting an error.
-char* scratch_of_current_device() {
+thread_local size_t t_last_used = 0;
+
+// The current device's copy of the array; nullptr after reporting an error, whose kind goes to *kind.
+char* scratch_of_current_device(int* kind) {
     int dev = -1;
+    *kind = CUMO_HIP_ERROR_RUNTIME;
     if (!hip_ok(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
     if (dev < 0 || dev >= kMaxDevices) {
+        *kind = CUMO_HIP_ERROR_ARGUMENT;
         report_error(CUMO_HIP_ERROR_ARGUMENT, 0, "cumo_hip_sfloat_sum_noalloc_kernel_launch: device ordinal out of range");
         return nullptr;
     }
@@ -47,24 +51,30 @@ char* scratch_of_current_device() {
         report_hip_error(st, "hipGetSymbolAddress(scratch)");
         return nullptr;
     }
+    *kind = CUMO_HIP_OK;
     return p;
 }
 
 }  // namespace
 
 extern "C" int cumo_hip_sfloat_sum_noalloc_kernel_launch(cumo_na_reduction_arg_t* arg) {
+    t_last_used = 0;
     if (arg == nullptr) {
         report_error(CUMO_HIP_ERROR_ARGUMENT, 0, "cumo_hip_sfloat_sum_noalloc_kernel_launch: arg is NULL");
         return CUMO_HIP_ERROR_ARGUMENT;
     }
-    char* p = scratch_of_current_device();
-    if (p == nullptr) return CUMO_HIP_ERROR_RUNTIME;
-    const RedScratch fixed = {p, kScratchBytes};
+    int kind = CUMO_HIP_OK;
+    char* p = scratch_of_current_device(&kind);
+    if (p == nullptr) return kind;
+    const RedScratch fixed = {p, kScratchBytes, 0};
     if (!reduce_launch(arg, nullptr, SumImpl<float, float, false, false>{0.0f}, 0, &fixed)) {
         report_error(CUMO_HIP_ERROR_ARGUMENT, 0,
                      "cumo_hip_sfloat_sum_noalloc_kernel_launch: the partial sums of this reduction do not fit the fixed "
                      "scratch array (CUMO_HIP_NOALLOC_SCRATCH_BYTES); use cumo_sfloat_sum_kernel_launch");
         return CUMO_HIP_ERROR_ARGUMENT;
     }
+    t_last_used = fixed.used;
     return CUMO_HIP_OK;
 }
+
+extern "C" size_t cumo_hip_sfloat_sum_noalloc_scratch_used(void) { return t_last_used; }

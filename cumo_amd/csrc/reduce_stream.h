@@ -49,6 +49,7 @@ struct RedSParams {
     int32_t index_mode;    // what accumulate() gets as idx: 1 = position along the axis, 2 = element offset from `in`
     char* partial;         // split form: n_out * n_split accumulators
     uint32_t* tickets;     // split form: n_out + n_out * ceil(n_split / group) words, zero between launches
+    WaitCtl* wait;         // hand-over form: where a wait that gives up reports it
 };
 
 template <class In, int VEC, bool NT>
@@ -256,7 +257,18 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
         // this block counts in. Blocks count in on their group's ticket; the last of a
         // group counts in on the output's ticket; the last there finds every
         // accumulator of the output in memory. Tickets go back to zero on the way.
+        // What orders the publication before the count:
+        //  * the hardware: rs_publish stores with agent scope, which on this device writes through
+        //    the compute die's second-level cache to the memory all dies share, and the wait below
+        //    returns when those stores are acknowledged; the ticket add is issued after that;
+        //  * the compiler: the fence. At workgroup scope it costs nothing beyond that same wait,
+        //    but no memory operation may be moved across it.
+        // A release on the ticket add itself (agent scope) would be the textbook form; on this
+        // device it also writes back the whole second-level cache of the die, once per block:
+        // measured on T.sum() of 2^25 SFloat with tickets, 25.2 -> 107 us. The emitted order
+        // (store sc1 ... s_waitcnt vmcnt(0) ... atomic add) is pinned by tests/test_emitted_ordering.py.
         rs_publish<Acc>(p.partial + (size_t)vrow * sizeof(Acc), acc);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0): the stores are acknowledged
         const uint32_t groups = (p.n_split + p.group - 1) / p.group;
         const uint32_t g = i_split / p.group;
@@ -354,13 +366,12 @@ __device__ __attribute__((noinline)) typename Impl::Acc rs_exact_refold_wave(con
 // instead of store, acknowledgement, two tickets in turn, fence and loads (C3 T.sum() on fresh
 // operands: 25.0 -> 22.4 us; a sum of 4 MiB: 5.9 -> 4.0 us). A streaming block never waits for
 // anything, so the waiting blocks (which the dispatcher starts first) cannot hold the others up;
-// a wait gives up after kRsPollLimit looks (the count of that is kept).
+// a wait gives up after kRsPollLimit looks, counts that and raises the host's give-up word (wait_ctl.h).
 constexpr uint32_t kRsHandoverWords = 8192;
 constexpr uint32_t kRsPollLimit = 1u << 24;
-__device__ uint32_t g_red_poll_gave_up;
 
 template <class Acc>
-__device__ __forceinline__ Acc rs_await(const uint64_t* slot, uint32_t launch) {
+__device__ __forceinline__ Acc rs_await(const uint64_t* slot, uint32_t launch, WaitCtl* ctl) {
     constexpr int W = sizeof(Acc) / 4;
     union U {
         Acc a;
@@ -371,13 +382,14 @@ __device__ __forceinline__ Acc rs_await(const uint64_t* slot, uint32_t launch) {
 #pragma unroll
     for (int i = 0; i < W; ++i) x[i] = __hip_atomic_load(slot + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     uint32_t looks = 0;
+    const uint32_t limit = wait_limit(ctl, kRsPollLimit);
     for (;;) {
         bool all = true;
 #pragma unroll
         for (int i = 0; i < W; ++i) all = all && (uint32_t)(x[i] >> 32) == launch;
         if (all) break;
-        if (++looks > kRsPollLimit) {
-            __hip_atomic_fetch_add(&g_red_poll_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (++looks > limit) {
+            wait_gave_up(ctl, WAIT_REDUCE);
             break;
         }
         __builtin_amdgcn_s_sleep(4);
@@ -438,7 +450,7 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
         typedef typename Impl::Exact Exact;
         static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
         Acc total = impl.identity();
-        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(mine + (size_t)k * W, launch), total);
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), total);
         rs_group_combine(impl, total, 8, wave_slots);
         if (threadIdx.x == 0) s_need = impl.needs_exact(total) ? 1 : 0;
         __syncthreads();
@@ -446,14 +458,14 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
             const Exact ex = impl.exact();
             __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
             typename Exact::Acc e = ex.identity();
-            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_await<Acc>(mine + (size_t)k * W, launch), (int64_t)k, e);
+            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), (int64_t)k, e);
             rs_group_combine(ex, e, 8, exact_slots);
             total = impl.from_exact(e);
         }
         if (threadIdx.x == 0) impl.store(total, p.out + o_a, nullptr);
     } else {
         Acc total = impl.identity();
-        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(mine + (size_t)k * W, launch), total);
+        for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), total);
         rs_group_combine(impl, total, 8, wave_slots);
         if (threadIdx.x == 0) impl.store(total, p.out + o_a, (Impl::NOUT > 1) ? (p.out2 + o_b) : nullptr);
     }

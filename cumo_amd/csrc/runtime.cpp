@@ -83,11 +83,98 @@ int stream_slot(hipStream_t stream) {
     return free_slot;
 }
 
-void stream_slot_release(hipStream_t stream) {
+int stream_slot_release(hipStream_t stream) {
     std::lock_guard<std::mutex> hold(g_slot_lock);
+    int held = -1;
     for (int i = 0; i < kStreamSlots; ++i) {
-        if (g_slot_used[i] && g_slot_stream[i] == stream) g_slot_used[i] = false;
+        if (g_slot_used[i] && g_slot_stream[i] == stream) {
+            g_slot_used[i] = false;
+            held = i;
+        }
     }
+    return held;
+}
+
+int device_compute_units() {
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        return cus;
+    }();
+    return n;
+}
+
+// The give-up word and counters of the kernels' bounded waits. The flag is pinned host memory
+// the device writes through; the block the kernels read sits in device memory.
+static std::mutex g_wait_lock;
+static WaitCtl* g_wait_dev = nullptr;
+static std::atomic<uint32_t*> g_wait_flag{nullptr};
+
+WaitCtl* wait_ctl() {
+    std::lock_guard<std::mutex> hold(g_wait_lock);
+    if (g_wait_dev) return g_wait_dev;
+    void* flag = nullptr;
+    if (hipHostMalloc(&flag, 64, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    std::memset(flag, 0, 64);
+    void* dev = nullptr;
+    if (hipMalloc(&dev, sizeof(WaitCtl)) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipHostFree(flag);
+        return nullptr;
+    }
+    WaitCtl init;
+    std::memset(&init, 0, sizeof(init));
+    // CUMO_HIP_WAIT_LIMIT=0 (read once, for tests): every wait gives up at its first failed look
+    const char* e = std::getenv("CUMO_HIP_WAIT_LIMIT");
+    init.limit_scale = (e && e[0] == '0') ? 0u : 1u;
+    init.host_flag = (uint32_t*)flag;
+    if (hipMemcpy(dev, &init, sizeof(init), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(dev);
+        (void)hipHostFree(flag);
+        return nullptr;
+    }
+    g_wait_flag.store((uint32_t*)flag);
+    g_wait_dev = (WaitCtl*)dev;
+    return g_wait_dev;
+}
+
+static int wait_counts_read(uint32_t out[4]) {
+    WaitCtl* dev;
+    {
+        std::lock_guard<std::mutex> hold(g_wait_lock);
+        dev = g_wait_dev;
+    }
+    out[0] = out[1] = out[2] = out[3] = 0;
+    if (!dev) return 0;  // no kernel with a wait was ever launched
+    WaitCtl now;
+    if (hipMemcpy(&now, dev, sizeof(now), hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    for (int i = 0; i < 4; ++i) out[i] = now.gave_up[i];
+    return 0;
+}
+
+bool wait_trouble_check() {
+    uint32_t* flag = g_wait_flag.load();   // set once, before any kernel can write it
+    if (!flag || *(volatile uint32_t*)flag == 0) return true;
+    *(volatile uint32_t*)flag = 0;
+    uint32_t c[4];
+    char msg[256];
+    if (wait_counts_read(c) == 0)
+        std::snprintf(msg, sizeof(msg), "a kernel gave up waiting for another block's partial result; the results of that launch are not valid "
+                      "(give-ups so far: reductions %u, scans %u, mulsum %u)", c[0], c[1], c[2]);
+    else
+        std::snprintf(msg, sizeof(msg), "a kernel gave up waiting for another block's partial result; the results of that launch are not valid");
+    report_error(CUMO_HIP_ERROR_RUNTIME, 0, msg);
+    return false;
 }
 
 }  // namespace cumo_hip
@@ -95,6 +182,11 @@ void stream_slot_release(hipStream_t stream) {
 using namespace cumo_hip;
 
 extern "C" {
+
+int cumo_hip_wait_give_ups(uint32_t counts[4]) {
+    if (!counts) return -1;
+    return wait_counts_read(counts);
+}
 
 void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler) { g_handler.store(handler); }
 
@@ -121,13 +213,20 @@ void* cumo_hip_stream_create(void) {
     return (void*)st;
 }
 
+// What the library keeps per stream (its slot of ticket and hand-over words, the look-back words
+// of its scans, its arena of the pool) is given up; the stream itself stays the caller's.
+void cumo_hip_stream_release(void* hip_stream) {
+    if (!hip_stream) return;
+    // what the stream still has queued may use its slot's words: drain it first
+    hip_ok(hipStreamSynchronize((hipStream_t)hip_stream), "hipStreamSynchronize");
+    scan_chain_words_drop_slot(stream_slot_release((hipStream_t)hip_stream));
+    pool_retire_stream((hipStream_t)hip_stream);
+}
+
 void cumo_hip_stream_destroy(void* hip_stream) {
     if (!hip_stream) return;
     if (t_stream == (hipStream_t)hip_stream) t_stream = nullptr;
-    // what the stream still has queued may use its slot's words: drain it first
-    hip_ok(hipStreamSynchronize((hipStream_t)hip_stream), "hipStreamSynchronize");
-    stream_slot_release((hipStream_t)hip_stream);
-    pool_retire_stream((hipStream_t)hip_stream);
+    cumo_hip_stream_release(hip_stream);
     hip_ok(hipStreamDestroy((hipStream_t)hip_stream), "hipStreamDestroy");
 }
 
@@ -140,7 +239,9 @@ int cumo_hip_device_count(void) {
     return n;
 }
 
-void cumo_hip_synchronize(void) { hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize"); }
+void cumo_hip_synchronize(void) {
+    if (hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize")) wait_trouble_check();
+}
 
 void cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n) {
     if (n == 0) return;
@@ -151,7 +252,7 @@ void cumo_hip_memcpy_h2d(void* dst, const void* src, size_t n) {
 void cumo_hip_memcpy_d2h(void* dst, const void* src, size_t n) {
     if (n == 0) return;
     if (!hip_ok(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, t_stream), "hipMemcpyAsync(d2h)")) return;
-    hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+    if (hip_ok(hipStreamSynchronize(t_stream), "hipStreamSynchronize")) wait_trouble_check();
 }
 
 // reference: cuda/runtime.c:16-20
@@ -184,6 +285,7 @@ int* cumo_cuda_runtime_error_flag_new(void) {
 
 bool cumo_cuda_runtime_error_flag_get(int* flag) {
     if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return false;
+    wait_trouble_check();
     return flag && (*(volatile int*)flag != 0);
 }
 

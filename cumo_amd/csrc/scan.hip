@@ -25,6 +25,7 @@
 // totals through LDS. Everything is in a fixed order, so results do not change
 // from launch to launch.
 #include "common.h"
+#include "wait_ctl.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -304,17 +305,20 @@ __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const char* in, 
 // launch to launch (chain_words_acquire below), so nothing is cleared: what an earlier launch
 // left carries another number, and the ticket word just counts on (a launch takes exactly one
 // ticket per block; the host knows where it stood). A wait gives up after kChainSpinLimit polls
-// (it cannot be reached while every tile before this one has a running block); the count
-// of such give-ups is kept in g_scan_chain_gave_up.
+// (it cannot be reached while every tile before this one has a running block); it then counts
+// that and raises the host's give-up word (wait_ctl.h), so the next point where the host waits
+// for the device reports the launch as failed.
+// The ticket is a relaxed add on purpose: it hands out tile numbers and publishes nothing; what
+// a tile publishes travels whole in its tagged words.
 constexpr uint32_t kChainSpinLimit = 1u << 22;
 constexpr uint64_t kChainMaxTiles = 64ull * 64ull * 64ull;
-__device__ uint32_t g_scan_chain_gave_up;
 
 template <class T>
 struct ScanChain {
     static constexpr int W = (int)(sizeof(T) / 4);
     static constexpr int SUB = 64 / (int)sizeof(T) / 2;        // sub-tiles of the block-wide scan per tile: 64 KiB of elements
     static constexpr int TILE = kScanTile * SUB;
+    WaitCtl* wait;     // where a look-back that gives up reports it
     uint32_t* ticket;
     uint64_t* tile;    // [n_tiles * W]
     uint64_t* group;   // [n_groups * W]
@@ -410,13 +414,15 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
     const uint64_t* py = c.group + (size_t)(sg * 64u + lane) * W;
     const uint64_t* pz = c.super + (size_t)lane * W;
     uint32_t polls = 0;
+    const uint32_t spin_limit = wait_limit(c.wait, kChainSpinLimit);
     if (t > 0) {
         // the last word that the tile before this one publishes
         const uint64_t* latest = pos > 0 ? c.tile + (size_t)(t - 1) * W + (W - 1)
                                          : (gpos > 0 ? c.group + (size_t)(g - 1) * W + (W - 1) : c.super + (size_t)(sg - 1) * W + (W - 1));
         if (lane == 0) {
+            // (running out of looks here is not yet a failure: the loop below looks again and reports)
             while ((uint32_t)(__hip_atomic_load(latest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != c.flag) {
-                if (++polls > kChainSpinLimit) break;
+                if (++polls > spin_limit) break;
                 __builtin_amdgcn_s_sleep(16);
             }
         }
@@ -457,8 +463,8 @@ __device__ __forceinline__ void chain_look_back(const ScanChain<T>& c, uint32_t 
             }
         }
         if (__ballot(need_x || need_y || need_z) == 0) break;
-        if (++polls > kChainSpinLimit) {
-            if (lane == 0) __hip_atomic_fetch_add(&g_scan_chain_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (++polls > spin_limit) {
+            if (lane == 0) wait_gave_up(c.wait, WAIT_SCAN);
             break;
         }
         __builtin_amdgcn_s_sleep(16);
@@ -860,9 +866,12 @@ int scan_chain_launch(const char* p1, char* p2, ssize_t s1, ssize_t s2, uint64_t
     if (s1 != (ssize_t)sizeof(T) || s2 != (ssize_t)sizeof(T) || (((uintptr_t)p1 | (uintptr_t)p2) & 15) != 0) return -1;
     const uint64_t n_groups = (n_tiles + 63) / 64, n_supers = (n_groups + 63) / 64;
     const uint64_t words = kChainHead + (n_tiles + n_groups + n_supers) * W;
+    WaitCtl* wait = wait_ctl();
+    if (wait == nullptr) return -1;  // nowhere to report a wait that gives up: the form without waits
     ChainWords cw;
     if (!chain_words_acquire(stream, words, (uint32_t)n_tiles, &cw)) return (int)hipErrorOutOfMemory;
     ScanChain<T> c;
+    c.wait = wait;
     c.ticket = reinterpret_cast<uint32_t*>(cw.ws);
     c.tile = cw.ws + kChainHead;
     c.group = c.tile + n_tiles * W;
@@ -1097,6 +1106,7 @@ constexpr uint32_t kColsChainFan = 8;
 template <class T>
 struct ScanColsChain {
     static constexpr int W = (int)(sizeof(T) / 4);
+    WaitCtl* wait;     // where a look-back that gives up reports it
     uint32_t* ticket;
     uint64_t* tile;    // [strip][level][column][W]
     uint64_t* group;   // [strip][group][column][W]
@@ -1112,10 +1122,11 @@ struct ScanColsChain {
 // once (eight-byte types: four, then three; seven would not fit the registers beside the tile),
 // asked for again until they are there, then folded in order. False when count is 0.
 template <class T, class Op>
-__device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t stride, uint32_t count, uint32_t flag, T& out) {
+__device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t stride, uint32_t count, uint32_t flag, WaitCtl* ctl, T& out) {
     constexpr int W = ScanColsChain<T>::W;
     constexpr uint32_t N = kColsChainFan - 1, C = sizeof(T) == 8 ? 4 : N;
     uint32_t polls = 0;
+    const uint32_t spin_limit = wait_limit(ctl, kChainSpinLimit);
     bool has = false;
 #pragma unroll
     for (uint32_t c0 = 0; c0 < N; c0 += C) {
@@ -1132,8 +1143,8 @@ __device__ __forceinline__ bool cols_chain_gather(const uint64_t* base, size_t s
 #pragma unroll
                 for (int h = 0; h < W; ++h) all = all && (uint32_t)(x[i][h] >> 32) == flag;
             if (all) break;
-            if (++polls > kChainSpinLimit) {
-                __hip_atomic_fetch_add(&g_scan_chain_gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (++polls > spin_limit) {
+                wait_gave_up(ctl, WAIT_SCAN);
                 break;
             }
             __builtin_amdgcn_s_sleep(8);
@@ -1258,7 +1269,7 @@ __global__ __launch_bounds__(NW * 64) void scan_cols_chain_kernel(ScanColsParams
         count = 0;
     }
     T xs = T();
-    const bool xh = cols_chain_gather<T, Op>(from, cw, count, c.flag, xs);
+    const bool xh = cols_chain_gather<T, Op>(from, cw, count, c.flag, c.wait, xs);
     if (role == 0) {
         if (xh) gt = Op::apply(xs, gt);  // the group's total so far
         if (pos == kColsChainFan - 1) chain_publish<T>(c.group + (((size_t)ps * c.n_groups + g) * SW + col) * W, gt, c.flag);
@@ -1362,9 +1373,12 @@ bool scan_cols_chain_launch(ScanColsParams& p, hipStream_t stream) {
     if (n_tiles < 16 || n_tiles > 0x7fffffffull) return false;
     const uint64_t n_groups = (depth + F - 1) / F, n_supers = (n_groups + F - 1) / F;
     const uint64_t words = kChainHead + all_strips * (depth + n_groups + n_supers) * SW * W;
+    WaitCtl* wait = wait_ctl();
+    if (wait == nullptr) return false;  // nowhere to report a wait that gives up: the form without waits
     ChainWords cw;
     if (!chain_words_acquire(stream, words, (uint32_t)n_tiles, &cw)) return true;
     ScanColsChain<T> c;
+    c.wait = wait;
     c.ticket = reinterpret_cast<uint32_t*>(cw.ws);
     c.tile = cw.ws + kChainHead;
     c.flag = cw.flag;
@@ -1504,6 +1518,51 @@ void scan_rows_dispatch(int prod, int nan, const ScanRowsParams& p, hipStream_t 
 }
 
 }  // namespace
+
+// The kept regions go back to the driver when their stream is retired and when the caller asks
+// the pool to give back what it holds (they are not the pool's blocks -- they must outlive a
+// launch without being handed to anybody else -- but they are memory the library holds:
+// up to kChainKeptWords * 8 bytes per stream that has run a one-pass scan).
+// The stream of the slot must have finished its work.
+void scan_chain_words_drop_slot(int slot) {
+    if (slot < 0 || slot >= kStreamSlots) return;
+    std::lock_guard<std::mutex> hold(g_chain_lock);
+    for (int dev = 0; dev < kChainDevices; ++dev) {
+        ChainRegion& r = g_chain_region[dev][slot];
+        if (!r.ptr) continue;
+        if (hipFree(r.ptr) != hipSuccess) (void)hipGetLastError();
+        r = ChainRegion{nullptr, 0, 0, 0};
+    }
+}
+
+// every region, after waiting for the device (a launch that still uses one may be queued)
+void scan_chain_words_drop_all() {
+    std::lock_guard<std::mutex> hold(g_chain_lock);
+    bool any = false;
+    for (int dev = 0; dev < kChainDevices && !any; ++dev)
+        for (int slot = 0; slot < kStreamSlots && !any; ++slot) any = g_chain_region[dev][slot].ptr != nullptr;
+    if (!any) return;
+    if (hipDeviceSynchronize() != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    for (int dev = 0; dev < kChainDevices; ++dev)
+        for (int slot = 0; slot < kStreamSlots; ++slot) {
+            ChainRegion& r = g_chain_region[dev][slot];
+            if (!r.ptr) continue;
+            if (hipFree(r.ptr) != hipSuccess) (void)hipGetLastError();
+            r = ChainRegion{nullptr, 0, 0, 0};
+        }
+}
+
+size_t scan_chain_words_held_bytes() {
+    std::lock_guard<std::mutex> hold(g_chain_lock);
+    size_t total = 0;
+    for (int dev = 0; dev < kChainDevices; ++dev)
+        for (int slot = 0; slot < kStreamSlots; ++slot) total += (size_t)g_chain_region[dev][slot].cap * sizeof(uint64_t);
+    return total;
+}
+
 }  // namespace cumo_hip
 
 using namespace cumo_hip;

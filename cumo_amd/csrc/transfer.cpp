@@ -256,7 +256,11 @@ int transfer(bool to_host, void* dst, const void* src, size_t n) {
     if (to_host) to_host_locked(s, st, (char*)dst, (const char*)src, n, &err);
     else from_host_locked(s, st, (char*)dst, (const char*)src, n, &err);
     s->mu.unlock();
-    if (err.ok()) return CUMO_HIP_OK;
+    if (err.ok()) {
+        // the device has been waited for: a kernel that gave up a bounded wait is reported here
+        if (to_host && !wait_trouble_check()) return CUMO_HIP_ERROR_RUNTIME;
+        return CUMO_HIP_OK;
+    }
     (void)hipGetLastError();  // reported here; must not show up again at the next launch check
     report_hip_error(err.st, err.what);  // may not return
     return err.st == hipErrorOutOfMemory ? CUMO_HIP_ERROR_OUT_OF_MEMORY : CUMO_HIP_ERROR_RUNTIME;

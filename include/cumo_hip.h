@@ -426,6 +426,9 @@ CUMO_HIP_DECL_REDUCE_PAIR(dfloat, minmax_nan)
  * last call's partial sums. */
 #define CUMO_HIP_NOALLOC_SCRATCH_BYTES (256u << 10)
 int cumo_hip_sfloat_sum_noalloc_kernel_launch(cumo_na_reduction_arg_t* arg);
+/* bytes of the fixed array that this thread's last call of the launcher above handed to its
+ * kernels (0: the reduction needed no partial sums, or the call was refused) */
+size_t cumo_hip_sfloat_sum_noalloc_scratch_used(void);
 
 /* ------------------------------------------------------------------------
  * 5. Bit launchers: narray/gen/tmpl_bit/binary_kernel.cu:1-52 (host
@@ -555,6 +558,20 @@ void cumo_hip_set_error_handler(cumo_hip_error_handler_t handler);
  * NULL, receives a pointer to a thread-local string. */
 int cumo_hip_last_error(const char** message);
 
+/* Kernels that finish in one launch what the reference does in two (a split reduction whose
+ * last block folds the partial results, one-pass scans, the one-launch mulsum; the reference's
+ * forms are include/cumo/reduce_kernel.h:395-611 and gen/tmpl/cum_kernel.cu:51-76) let a block
+ * wait for words that other blocks of the same launch publish, for a bounded number of looks.
+ * A wait that runs out cannot produce its result. It is reported the way the reference
+ * reports trouble inside a kernel (the pinned flag that the host reads after a device sync,
+ * cuda/runtime.c:22-47): the next call that waits for the device -- cumo_hip_synchronize,
+ * cumo_hip_memcpy_d2h, cumo_hip_copy_to_host, cumo_cuda_runtime_error_flag_get -- reports
+ * CUMO_HIP_ERROR_RUNTIME through the handler / cumo_hip_last_error. This call returns how
+ * often it has happened since the process started: counts[0] reductions, counts[1] scans,
+ * counts[2] mulsum, counts[3] unused. Returns 0, or -1 when the counts cannot be read.
+ * (It waits for the device.) No counterpart in the reference. */
+int cumo_hip_wait_give_ups(uint32_t counts[4]);
+
 /* count_true / count_false along axes in one launch (no counterpart in the
  * reference, whose ndloop walks every output on the host and launches one run at a
  * time, narray/ndloop.c:1569-1613 under gen/tmpl_bit/bit_count.c:9-36). The loop is
@@ -678,6 +695,13 @@ void* cumo_hip_get_stream(void);
  * null stream if it was this one */
 void* cumo_hip_stream_create(void);
 void  cumo_hip_stream_destroy(void* hip_stream);
+/* For a stream the caller created with its own HIP binding and passed to cumo_hip_set_stream:
+ * call this before destroying it (it waits for the stream). The library keeps a little state
+ * per stream it has seen (one of 64 slots of ticket / hand-over words, the look-back words of
+ * one-pass scans, an arena of the pool); a stream that goes away without this call keeps its
+ * slot, and once all 64 are taken further streams run split reductions and scans in their
+ * slower two-launch forms. cumo_hip_stream_destroy does the same for streams made here. */
+void  cumo_hip_stream_release(void* hip_stream);
 int   cumo_hip_device_count(void);
 void  cumo_hip_synchronize(void);
 /* events on the current stream, for callers that time launches */
@@ -704,7 +728,11 @@ int   cumo_hip_copy_from_host(void* dst_device, const void* src_host, size_t n);
  * Returns CUMO_HIP_OK or an error kind; never raises. */
 int    cumo_hip_pool_malloc(size_t size, void* hip_stream, void** ptr);
 int    cumo_hip_pool_free(void* ptr);                       /* CUMO_HIP_ERROR_ARGUMENT if the pool does not own ptr */
-void   cumo_hip_pool_free_all_blocks(void);
+void   cumo_hip_pool_free_all_blocks(void);   /* also drops the scans' kept look-back words (waits for the device if any are held) */
+/* device memory the library holds outside the pool's books: the look-back words that each
+ * stream keeps from one one-pass scan to the next (at most 64 MiB per stream, sized by the
+ * largest scan it has run). free_all_blocks and cumo_hip_stream_release give it back. */
+size_t cumo_hip_pool_held_outside_bytes(void);
 void   cumo_hip_pool_free_all_blocks_stream(void* hip_stream);
 /* files everything the pool holds for a stream (free or in use) under the null stream; the
  * stream must have finished its work. cumo_hip_stream_destroy calls it. */

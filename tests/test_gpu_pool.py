@@ -127,3 +127,43 @@ def test_two_streams_share_the_pool_without_mixing_results():
         L.cumo_hip_synchronize()
         L.cumo_hip_stream_destroy(own)
     _lib.check()
+
+
+def test_look_back_words_of_scans_are_counted_and_given_back():
+    """One-pass scans keep a region of words per stream outside the pool's books. It shows in
+    cumo_hip_pool_held_outside_bytes, goes back to the driver with free_all_blocks and when
+    the stream is released, and later scans on the stream still give the right answer."""
+    import cumo_amd
+    from cumo_amd import _lib
+    L = _lib.lib
+    held = _lib.fn("cumo_hip_pool_held_outside_bytes", C.c_size_t, [])
+    release = _lib.fn("cumo_hip_stream_release", None, [C.c_void_p])
+    assert held() == 0                      # (the fixture has just called free_all_blocks)
+    n = (1 << 22) + 5
+    hx = np.random.default_rng(5).integers(-3, 4, n).astype(np.float32)
+    want = np.cumsum(hx.astype(np.float64)).astype(np.float32)   # small integers: exact in any order
+    x = cumo_amd.SFloat.cast(hx)
+    assert (x.cumsum().to_numpy() == want).all()
+    on_null = held()
+    assert on_null > 0
+    own = L.cumo_hip_stream_create()
+    assert own
+    try:
+        cumo_amd.synchronize()
+        L.cumo_hip_set_stream(own)
+        assert (x.cumsum().to_numpy() == want).all()
+        assert held() > on_null             # a second region, for the second stream
+        cumo_amd.synchronize()
+        release(own)                        # the caller keeps the stream, the library forgets it
+        assert held() == on_null
+        assert (x.cumsum().to_numpy() == want).all()   # the stream is taken up again from nothing
+        assert held() > on_null
+        cumo_amd.synchronize()
+    finally:
+        L.cumo_hip_set_stream(None)
+        L.cumo_hip_stream_destroy(own)
+    assert held() == on_null
+    cumo_amd.MemoryPool.free_all_blocks()
+    assert held() == 0
+    assert (x.cumsum().to_numpy() == want).all()
+    _lib.check()
