@@ -871,6 +871,7 @@ extern "C" void cumo_hip_bit_count_nd_kernel_launch(const cumo_hip_bit_count_nd_
     const int L = d->out_ndim - 1;
     const bool down_columns = d->red_ndim == 1 && d->out_ndim >= 1 && d->in_out_step[L] == 1;
     if (!down_columns && bit_count_rows_reduce(d)) return;
+    if (down_columns && bit_count_cols_words_launch(d)) return;   // rows on word boundaries: one launch, no zero-fill
     if (d->overwrite) {
         size_t outs = 1;
         for (int k = 0; k < d->out_ndim; ++k) outs *= d->out_shape[k];

@@ -44,6 +44,9 @@ uint64_t* red_handover_words(int slot, uint32_t* launch_number);
 // the loop is not one they take (the caller then uses the Bit kernels' own forms).
 int bit_count_run_reduce(CUMO_BIT_DIGIT* a, size_t pos, uint64_t n, int count_false, uint64_t* out);
 int bit_count_rows_reduce(const cumo_hip_bit_count_nd_t* counts);  // (stores the counts when counts->overwrite, adds them otherwise)
+// Bit counts down the rows of a matrix whose rows start on word boundaries (bit_count_cols.hip): 1 when
+// launched (stored or added as counts->overwrite says), 0 when the loop is not one it takes.
+int bit_count_cols_words_launch(const cumo_hip_bit_count_nd_t* counts);
 
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)

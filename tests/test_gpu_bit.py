@@ -303,3 +303,55 @@ def test_counts_of_very_long_runs(n):
             assert int(d.count_false()) == int(v.size - v.sum()), (lo, cut)
     ones = cumo_amd.Bit.cast(np.ones(n, dtype=np.uint8))
     assert int(ones.count_true()) == n and int(ones.count_false()) == 0 and ones.all_p() and not ones.none_p()
+
+
+def test_counts_down_columns_of_word_aligned_rows():
+    """Rows that start on word boundaries take the carry-save form (a lane per 32, 64 or 128
+    columns, blocks of a column group folded through scratch by the last one in): one, two
+    and four words per lane, a last word that is partly columns, several stretches of 240
+    rows per wave, many planes, and both ways of writing the result -- stored over whatever
+    was there, and added onto it -- through the launcher itself."""
+    import ctypes as C
+    import cumo_amd
+    from cumo_amd import _lib
+    rng = np.random.default_rng(615)
+    for shape in [(4096, 32768), (5000, 8192 + 64), (3000, 16384 + 64), (777, 4096 + 40), (600, 2500, 256), (3, 9000, 640), (65, 96), (2, 128),
+                  (100, 1 << 17)]:
+        h = (rng.random(shape) < 0.6).astype(np.uint8)
+        h[..., 1] = 1
+        h[..., 2] = 0
+        b = cumo_amd.Bit.cast(h)
+        nd = len(shape)
+        want = h.sum(axis=nd - 2, dtype=np.uint64)
+        assert (np.asarray(b.count_true(axis=nd - 2).to_numpy()) == want).all(), shape
+        assert (np.asarray(b.count_false(axis=nd - 2).to_numpy()) == shape[nd - 2] - want).all(), shape
+        if nd == 2:
+            v = b[1::2, 64:]                  # every other row, from the third word on
+            assert (np.asarray(v.count_true(axis=0).to_numpy()) == h[1::2, 64:].sum(axis=0, dtype=np.uint64)).all(), shape
+
+    # the launcher with hand-built arguments: counts ADDED onto what the results hold
+    MAXD = 12
+
+    class CountNd(C.Structure):
+        _fields_ = [("out_ndim", C.c_int), ("red_ndim", C.c_int), ("out_shape", C.c_size_t * MAXD), ("red_shape", C.c_size_t * MAXD),
+                    ("in_out_step", C.c_ssize_t * MAXD), ("in_red_step", C.c_ssize_t * MAXD), ("out_step", C.c_ssize_t * MAXD),
+                    ("in_", C.c_void_p), ("pos", C.c_size_t), ("out", C.c_void_p), ("count_false", C.c_int), ("overwrite", C.c_int)]
+
+    f = _lib.fn("cumo_hip_bit_count_nd_kernel_launch", None, [C.POINTER(CountNd)])
+    rows, cols = 3001, 4096 + 64
+    h = (rng.random((rows, cols)) < 0.5).astype(np.uint8)
+    b = cumo_amd.Bit.cast(h)
+    start = np.arange(cols, dtype=np.uint64) * 3 + 7
+    for overwrite in (0, 1):
+        for count_false in (0, 1):
+            out = cumo_amd.UInt64.cast(start)
+            d = CountNd()
+            d.out_ndim, d.red_ndim = 1, 1
+            d.out_shape[0], d.red_shape[0] = cols, rows
+            d.in_out_step[0], d.in_red_step[0], d.out_step[0] = 1, cols, 8
+            d.in_, d.pos, d.out = b._buf.ptr, 0, out._buf.ptr
+            d.count_false, d.overwrite = count_false, overwrite
+            _lib.call(f, C.byref(d))
+            counts = (rows - h.sum(axis=0, dtype=np.uint64)) if count_false else h.sum(axis=0, dtype=np.uint64)
+            want = counts if overwrite else counts + start
+            assert (out.to_numpy() == want).all(), (overwrite, count_false)
