@@ -1491,10 +1491,13 @@ static inline bool ew_lean_rows_enabled() {
 
 // in1/in2 may be NULL (NIN < 2 or the scalar form). out_bit is non-NULL for a
 // Bit result, in which case out is ignored.
-template <class Op>
+// HEAVY_CALL (a compile-time choice, so that the kernels it rules out are never built): a function
+// with many instructions per element -- capped grids, and no lean two-rows-per-lane form.
+template <class Op, bool HEAVY_CALL = false>
 static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t* in2, const cumo_na_iarray_t* out,
                       const cumo_na_bit_iarray_t* out_bit, const cumo_na_indexer_t* indexer, typename Op::S sv, int use_scalar,
-                      int* flag, bool heavy = false) {
+                      int* flag) {
+    constexpr bool heavy = HEAVY_CALL;
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;
@@ -1751,9 +1754,9 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     // Matrix with rows of an odd length (op) a second two-dimensional operand: flat over the matrix
     // and the result, the other operand addressed by row and column (see ew_flat_period_kernel).
     if constexpr (!Op::BIT_OUT && Op::NIN == 2 && std::is_same<A, B>::value && sizeof(A) == sizeof(R) && (sizeof(A) == 4 || sizeof(A) == 8) &&
-                  !op_is_heavy<Op>::value && !op_has_rare<Op>::value) {
+                  !op_is_heavy<Op>::value && !op_has_rare<Op>::value && !heavy) {
         constexpr int V = 16 / (int)sizeof(A);
-        if ((n == 2 || n == 3) && nops == 3 && use_scalar == 0 && !heavy && !force_scalar && !force_wide_indices() && (kp.inner % V) != 0 && kp.inner >= 64 &&
+        if ((n == 2 || n == 3) && nops == 3 && use_scalar == 0 && !force_scalar && !force_wide_indices() && (kp.inner % V) != 0 && kp.inner >= 64 &&
             plan.total < 0x7fffffffull) {
             const int64_t es = (int64_t)sizeof(A);
             auto one_run = [&](int sl) {
@@ -1889,7 +1892,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     } while (0);
                 // large two-dimensional arrays of a cheap function: the lean form, two rows per lane
                 const uint64_t lean_tiles = ctiles * ((kp.rows + 2 * ty - 1) / (2 * ty));
-                if (n == 2 && nt && !heavy && Op::NIN >= 1 && rp.walk[0] && lean_tiles <= ew_grid_max() && ew_lean_rows_enabled()) {
+                if constexpr (!heavy) if (n == 2 && nt && Op::NIN >= 1 && rp.walk[0] && lean_tiles <= ew_grid_max() && ew_lean_rows_enabled()) {
                     EwR2LeanParams lp;
                     std::memset(&lp, 0, sizeof(lp));
                     for (int k = 0; k < 3; ++k) { lp.ptr[k] = rp.ptr[k]; lp.rstep[k] = rp.rstep[k]; }
