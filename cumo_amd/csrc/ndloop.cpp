@@ -1524,8 +1524,7 @@ int where_single_run(const LP& lp, int invert, int rtype, const char* x, ssize_t
     if (nb > sizeof(host_counts) / sizeof(host_counts[0])) return fail(CUMO_HIP_ERROR_ARGUMENT, "where: more block counts than expected");
     uint64_t* counts = reinterpret_cast<uint64_t*>(cumo_cuda_runtime_malloc(nb * sizeof(uint64_t)));
     if (!counts) return CUMO_HIP_ERROR_OUT_OF_MEMORY;
-    cumo_hip_bit_where_count_kernel_launch((CUMO_BIT_DIGIT*)in.ptr, in.bitpos, in.step[0], n, invert, counts);
-    int rc = cumo_hip_copy_to_host(host_counts, counts, nb * sizeof(uint64_t));
+    int rc = cumo_hip_bit_where_count_to_host((CUMO_BIT_DIGIT*)in.ptr, in.bitpos, in.step[0], n, invert, counts, host_counts);
     uint64_t n_hit = 0;
     for (size_t b = 0; b < nb; ++b) n_hit += host_counts[b];
     bool allocated = false;

@@ -115,7 +115,8 @@ __device__ __forceinline__ uint32_t wh_block_exscan32(uint32_t v, uint32_t* tota
 }
 
 __global__ __launch_bounds__(kWhBlock) void where_count_kernel(const CUMO_BIT_DIGIT* a, uint64_t p, int64_t s, const size_t* idx, uint64_t n,
-                                                               int contiguous, int invert, uint64_t nchunks, uint64_t cpb, uint64_t* block_sums) {
+                                                               int contiguous, int invert, uint64_t nchunks, uint64_t cpb, uint64_t* block_sums,
+                                                               uint64_t* host_sums) {
     uint64_t start = (uint64_t)blockIdx.x * cpb;
     if (start > nchunks) start = nchunks;
     const uint64_t end = (nchunks - start < cpb) ? nchunks : start + cpb;
@@ -123,7 +124,12 @@ __global__ __launch_bounds__(kWhBlock) void where_count_kernel(const CUMO_BIT_DI
     for (uint64_t c = start + threadIdx.x; c < end; c += kWhBlock) cnt += (uint64_t)__popc(wh_chunk(a, p, s, idx, n, c, contiguous, invert));
     uint64_t total;
     wh_block_exscan(cnt, &total);
-    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+    if (threadIdx.x == 0) {
+        block_sums[blockIdx.x] = total;
+        // a copy straight into the caller's pinned host memory: the host then only has to wait for
+        // the stream, not for a copy queued behind the kernel
+        if (host_sums) host_sums[blockIdx.x] = total;
+    }
 }
 
 // block_sums[b] becomes the output position of block b's first hit; *running moves on
@@ -222,7 +228,7 @@ void where_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, size_t* idx, uint64_t 
     const int contiguous = (idx == nullptr && s == 1) ? 1 : 0;
     hipStream_t st = current_stream();
     hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)idx, n, contiguous,
-                       invert, nchunks, cpb, block_sums);
+                       invert, nchunks, cpb, block_sums, (uint64_t*)nullptr);
     hipLaunchKernelGGL(where_scan_kernel, dim3(1), dim3(kWhBlock), 0, st, block_sums, nblocks, running);
 #define WH_SCATTER(ES)                                                                                                                      \
     hipLaunchKernelGGL((where_scatter_kernel<MODE, ES, false>), dim3((unsigned)nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s,     \
@@ -324,8 +330,30 @@ void cumo_hip_bit_where_count_kernel_launch(CUMO_BIT_DIGIT* a, size_t p, ssize_t
     if (n == 0) return;
     const WhGeometry g = wh_geometry(n);
     hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, current_stream(), a, (uint64_t)p, (int64_t)s,
-                       (const size_t*)nullptr, n, s == 1 ? 1 : 0, invert, g.nchunks, g.cpb, counts);
+                       (const size_t*)nullptr, n, s == 1 ? 1 : 0, invert, g.nchunks, g.cpb, counts, (uint64_t*)nullptr);
     cumo_cuda_runtime_check_kernel_launch();
+}
+
+// The same, and the counts on the host when the call returns (it waits for the stream): the kernel
+// writes them into pinned host memory of the calling thread as well, so no copy is queued behind
+// it. host_counts: cumo_hip_bit_where_blocks(n) words of ordinary host memory.
+int cumo_hip_bit_where_count_to_host(CUMO_BIT_DIGIT* a, size_t p, ssize_t s, uint64_t n, int invert, uint64_t* counts, uint64_t* host_counts) {
+    if (n == 0) return CUMO_HIP_OK;
+    const WhGeometry g = wh_geometry(n);
+    static thread_local uint64_t* pinned = nullptr;   // kWhMaxBlocks words, kept for the thread's lifetime
+    if (pinned == nullptr) {
+        void* m = nullptr;
+        if (!hip_ok(hipHostMalloc(&m, kWhMaxBlocks * sizeof(uint64_t), hipHostMallocMapped | hipHostMallocPortable), "hipHostMalloc")) return CUMO_HIP_ERROR_RUNTIME;
+        pinned = static_cast<uint64_t*>(m);
+    }
+    hipStream_t st = current_stream();
+    hipLaunchKernelGGL(where_count_kernel, dim3((unsigned)g.nblocks), dim3(kWhBlock), 0, st, a, (uint64_t)p, (int64_t)s, (const size_t*)nullptr, n,
+                       s == 1 ? 1 : 0, invert, g.nchunks, g.cpb, counts, pinned);
+    cumo_cuda_runtime_check_kernel_launch();
+    if (!hip_ok(hipStreamSynchronize(st), "hipStreamSynchronize")) return CUMO_HIP_ERROR_RUNTIME;
+    if (!wait_trouble_check()) return CUMO_HIP_ERROR_RUNTIME;
+    std::memcpy(host_counts, pinned, g.nblocks * sizeof(uint64_t));
+    return CUMO_HIP_OK;
 }
 
 // x == NULL: out[o] = the position in the run of the o-th hit, as an elmsz-byte integer (4 or 8);

@@ -647,6 +647,11 @@ int cumo_hip_mulsum_rows_kernel_launch(int type, int nan, const cumo_hip_mulsum_
  * cumo_bit_where_kernel_launch were five. invert: the clear bits are the hits. */
 size_t cumo_hip_bit_where_blocks(uint64_t n);
 void cumo_hip_bit_where_count_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, int invert, uint64_t *counts);
+/* count, and the counts in host_counts[0 .. blocks - 1] when the call returns: the kernel also writes
+ * them to pinned host memory of the calling thread, and the call waits for the stream (the one
+ * synchronisation that sizing the result costs, tmpl_bit/where.c:13-28) instead of queueing a copy
+ * behind the kernel. Returns CUMO_HIP_OK or an error kind. */
+int  cumo_hip_bit_where_count_to_host(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, int invert, uint64_t *counts, uint64_t *host_counts);
 void cumo_hip_bit_where_place_kernel_launch(CUMO_BIT_DIGIT *a, size_t p, ssize_t s, uint64_t n, int invert, const uint64_t *counts,
                                             const char *x, ssize_t sx, size_t elmsz, char *out);
 
