@@ -225,13 +225,22 @@ def config_ops(name, cumo, host):
             ("A.cumsum(axis:1)", lambda e: e.__setitem__("c1", e["x"].cumsum(axis=1)), 2 * nb, n),
             ("A.cumsum(axis:0)", lambda e: e.__setitem__("c0", e["x"].cumsum(axis=0)), 2 * nb, n),
         ]
-    if name == "bit":
-        # Bit arrays of 2^29 bits (64 MiB) and the stores between Bit and SFloat [8192,4096]
-        a, b, x = host["a"], host["b"], host["x"]
-        env = {"a": cumo.Bit.cast(a), "b": cumo.Bit.cast(b), "x": cumo.SFloat.cast(x)}
-        env["m"] = env["x"] > 0.0
-        n, nx = a.size, x.size
+    if name in ("bit", "bit_large"):
+        # Bit arrays of 2^29 bits (64 MiB; 2^31 bits, 256 MiB, for bit_large) and the stores between Bit and SFloat [8192,4096]
+        a, b, x = host["a"], host["b"], host.get("x")
+        env = {"a": cumo.Bit.cast(a), "b": cumo.Bit.cast(b)}
+        env["t"] = env["a"] | ~env["a"]
+        n = a.size
         rows, cols = a.shape
+        casts = []
+        if x is not None:
+            env["x"] = cumo.SFloat.cast(x)
+            env["m"] = env["x"] > 0.0
+            nx = x.size
+            casts = [
+                ("SFloat.cast(m) (Bit -> SFloat)", lambda e: e.__setitem__("f", e["m"]._cast_to(cumo.SFloat)), nx // 8 + 4 * nx, nx),
+                ("Bit.cast(x) (SFloat -> Bit)", lambda e: e.__setitem__("g", e["x"]._cast_to(cumo.Bit)), nx // 8 + 4 * nx, nx),
+            ]
         return env, [
             ("a & b", lambda e: e.__setitem__("c", e["a"] & e["b"]), 3 * n // 8, n),
             ("~a", lambda e: e.__setitem__("c", ~e["a"]), 2 * n // 8, n),
@@ -239,10 +248,9 @@ def config_ops(name, cumo, host):
             ("a.count_true", lambda e: e.__setitem__("k", e["a"].count_true()), n // 8, n),
             ("a.count_true(axis:1)", lambda e: e.__setitem__("k1", e["a"].count_true(axis=1)), n // 8 + 8 * rows, n),
             ("a.count_true(axis:0)", lambda e: e.__setitem__("k0", e["a"].count_true(axis=0)), n // 8 + 8 * cols, n),
-            ("a.all?(axis:1)", lambda e: e.__setitem__("p", e["a"].all_p(axis=1)), n // 8, n),
-            ("SFloat.cast(m) (Bit -> SFloat)", lambda e: e.__setitem__("f", e["m"]._cast_to(cumo.SFloat)), nx // 8 + 4 * nx, nx),
-            ("Bit.cast(x) (SFloat -> Bit)", lambda e: e.__setitem__("g", e["x"]._cast_to(cumo.Bit)), nx // 8 + 4 * nx, nx),
-        ]
+            # on an array with every bit set: a row of `a` is decided by its first words and the kernel stops reading it there
+            ("t.all?(axis:1) (t all set: every word is read)", lambda e: e.__setitem__("p", e["t"].all_p(axis=1)), n // 8, n),
+        ] + casts
     if name == "nmath":
         # NMath beyond exp / sqrt, the Float power and the scans on 2^26 elements (256 MiB SFloat,
         # 512 MiB DFloat per array); arguments positive so that every function is defined
@@ -278,6 +286,13 @@ def inputs_bit(shape=(16384, 32768)):
             "x": rng.standard_normal((8192, 4096), dtype=np.float32)}
 
 
+def inputs_bit_large(shape=(32768, 65536)):
+    # (bits unpacked from random bytes: 2^31 draws of one bit each would take most of a minute)
+    rng = np.random.default_rng(9)
+    n = shape[0] * shape[1]
+    return {k: np.unpackbits(np.frombuffer(rng.bytes(n // 8), dtype=np.uint8)).reshape(shape) for k in ("a", "b")}
+
+
 def inputs_nmath(n=1 << 26):
     rng = np.random.default_rng(6)
     return {"x": rng.uniform(0.05, 3.0, n).astype(np.float32)}
@@ -286,7 +301,7 @@ def inputs_nmath(n=1 << 26):
 HOST_INPUTS = {
     "c1": inputs_c1, "c1_large": lambda: inputs_c1(1 << 26), "c2": inputs_c2, "c3": inputs_c3, "c4": inputs_c4, "c5": inputs_c5,
     "c2_large": lambda: inputs_c2(8192), "c3_large": lambda: inputs_c3((256, 512, 1024)), "next": inputs_next,
-    "nmath": inputs_nmath, "odd": inputs_odd, "bit": inputs_bit,
+    "nmath": inputs_nmath, "odd": inputs_odd, "bit": inputs_bit, "bit_large": inputs_bit_large,
 }
 WORKLOAD_TEXT = {
     "c1": "C1 SFloat axpy + full sum, n=2^20",
@@ -296,6 +311,7 @@ WORKLOAD_TEXT = {
     "next": "operations beside the five configs on SFloat [8192,4096]: mulsum, clip, maximum, integer power, cumsum, where, a[mask], row gather and scatter through index arrays",
     "odd": "the hot-path operations on SFloat [8192,4095]: rows that are not a whole number of 128-bit vectors and start off 16-byte boundaries",
     "bit": "Bit [16384,32768] (64 MiB): logic on whole arrays and on windows, counts of the whole, along rows and down columns, all?; stores between Bit and SFloat [8192,4096]",
+    "bit_large": "the Bit logic and counts at [32768,65536] (256 MiB), where a launch's fixed start and drain weigh a quarter of what they do at 64 MiB",
     "nmath": "NMath functions, Float power and cumsum on 2^26 elements (SFloat 256 MiB, DFloat 512 MiB per array), arguments uniform in [0.05, 3)",
     "c2": "C2 DFloat broadcast add + row reduce: A f64 [4096,4096] + r [1,4096]; C.sum(axis:1); C.max(axis:1)",
     "c3": "C3 SFloat axis reductions on [64,512,1024]",
@@ -544,7 +560,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all-configs", action="store_true", help="measure every op of all five configs with full iteration counts")
-    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next,nmath,odd,bit)")
+    ap.add_argument("--configs", default="", help="comma-separated subset for per_config (c1,c1_large,c2,c2_large,c3,c3_large,c4,c5,next,nmath,odd,bit,bit_large)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--rotated-only", action="store_true",
@@ -700,7 +716,7 @@ def main():
 
     per_config = {}
     if not args.no_per_config:
-        names = [c for c in args.configs.split(",") if c] or ["c1", "c2", "c3", "c4", "c5", "c1_large", "c2_large", "c3_large", "next", "nmath", "odd", "bit"]
+        names = [c for c in args.configs.split(",") if c] or ["c1", "c2", "c3", "c4", "c5", "c1_large", "c2_large", "c3_large", "next", "nmath", "odd", "bit", "bit_large"]
         iters, warm = (30, 5) if args.all_configs else (7, 2)
         for name in names:
             per_config[name] = {"workload": WORKLOAD_TEXT[name], "ops": measure_config(name, cumo_amd, lib, iters, warm, not args.rotated_only)}

@@ -9,7 +9,9 @@
 // the block through LDS, and each block adds its total once. Integer addition
 // commutes, so the answer does not depend on the order the blocks arrive in.
 #include "bit_common.h"
+#include "div31.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -57,18 +59,47 @@ __global__ __launch_bounds__(kBlock) void bit_contiguous_kernel(const CUMO_BIT_D
     }
 }
 
-// 128 bits of `a` from bit position q on (q >= 0): one 128-bit load from a 4-byte boundary, and the
-// word after it when q is not at the start of a word. The caller has checked that all of it is there.
+// 128 bits of `a` from bit position q on (q >= 0): one 128-bit load from a 4-byte boundary and, when q is not
+// at the start of a word, the word after it, funnel-shifted. Nothing that looks at a loaded word sits under a
+// branch: that would make the caller wait for one operand's words before it asks for the next operand's. The
+// caller has checked that all the bits are there. Every lane of a wave that is switched on calls it together.
+struct Raw128 {
+    uint32_t v __attribute__((ext_vector_type(4)));
+    uint32_t e;
+    unsigned sh;
+    bool own;  // the fifth word is the lane's own load (e); otherwise it is the next lane's first word
+};
+// what the next lane (within a row of sixteen) holds in `x`; `otherwise` where there is no such lane or it is switched off
+__device__ __forceinline__ uint32_t next_lane(uint32_t x, uint32_t otherwise) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)otherwise, (int)x, 0x101 /* row_shl:1 */, 0xf, 0xf, false);
+}
+template <bool NT>
+__device__ __forceinline__ Raw128 raw128_load(const CUMO_BIT_DIGIT* a, uint64_t q) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    Raw128 r;
+    const uint64_t w = q >> 5;
+    r.sh = (unsigned)(q & 31);
+    r.v = NT ? __builtin_nontemporal_load(reinterpret_cast<const u4*>(a + w)) : *reinterpret_cast<const u4*>(a + w);
+    // The word after the four is the first of the next lane's four when that lane reads the 128 bits that follow
+    // these; a lane whose neighbour reads elsewhere (or is the last of its sixteen, or sits this out) loads the
+    // word itself. A load per lane would cost the memory pipeline a fifth of what the vectors cost it.
+    const uint64_t q_after = q + 128;
+    const uint32_t qlo = (uint32_t)q, qhi = (uint32_t)(q >> 32);
+    r.own = next_lane(qlo, qlo) != (uint32_t)q_after || next_lane(qhi, ~qhi) != (uint32_t)(q_after >> 32);
+    r.e = 0;
+    if (r.sh != 0 && r.own) r.e = a[w + 4];
+    return r;
+}
+// (kept apart from the loads so that a caller can ask for all its operands' words before it shifts the first)
+__device__ __forceinline__ uint4 raw128_bits(const Raw128& r) {
+    const uint32_t from_next = next_lane(r.v.x, 0u);
+    const uint32_t e = r.own ? r.e : from_next;
+    return make_uint4(__builtin_amdgcn_alignbit(r.v.y, r.v.x, r.sh), __builtin_amdgcn_alignbit(r.v.z, r.v.y, r.sh),
+                      __builtin_amdgcn_alignbit(r.v.w, r.v.z, r.sh), __builtin_amdgcn_alignbit(e, r.v.w, r.sh));
+}
 template <bool NT>
 __device__ __forceinline__ uint4 bits128_at(const CUMO_BIT_DIGIT* a, uint64_t q) {
-    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-    const uint64_t w = q >> 5;
-    const unsigned sh = (unsigned)(q & 31);
-    const u4 x = NT ? __builtin_nontemporal_load(reinterpret_cast<const u4*>(a + w)) : *reinterpret_cast<const u4*>(a + w);
-    if (sh == 0) return make_uint4(x.x, x.y, x.z, x.w);
-    const uint32_t e = a[w + 4];
-    const unsigned up = 32 - sh;
-    return make_uint4((x.x >> sh) | (x.y << up), (x.y >> sh) | (x.z << up), (x.z >> sh) | (x.w << up), (x.w >> sh) | (e << up));
+    return raw128_bits(raw128_load<NT>(a, q));
 }
 
 // The same, four output words per lane. The output vectors are the 16-byte aligned ones (`lead` = words
@@ -190,6 +221,257 @@ __global__ __launch_bounds__(kBlock) void bit_rows_kernel(const CUMO_BIT_DIGIT* 
     }
 }
 
+// The same views when the result's rows follow one another without a gap (a fresh result always does): the
+// result is then one run of bits, and a lane takes one 16-byte aligned vector of its words, wherever the rows
+// fall in it. It finds the row and the column of the vector's first bit (one multiplication by the reciprocal of
+// the row length, corrected by at most one) and reads 128 bits of each source from there; a vector that a row
+// ends in, or whose sources end within reach, is put together word by word from the two rows it spans (rows are
+// at least 128 bits long here). Stores are whole aligned vectors but for the run's first and last word.
+constexpr int kFlatOuter = 6;
+struct BitFlatRows {
+    int nouter;                  // outer dimensions after merging, outermost first
+    uint32_t rows;
+    uint32_t shape[kFlatOuter];
+    Div31 dv[kFlatOuter];
+    int64_t s1[kFlatOuter], s2[kFlatOuter];
+    uint64_t inner, total, nw1, nw2;
+    double inv_inner;
+};
+
+__device__ __forceinline__ void flat_row_col(const BitFlatRows& nd, uint64_t e, uint32_t& r, uint64_t& c) {
+    uint64_t q = (uint64_t)((double)e * nd.inv_inner);  // within one of e / inner: e < 2^52
+    int64_t rem = (int64_t)e - (int64_t)(q * nd.inner);
+    if (rem < 0) {
+        --q;
+        rem += (int64_t)nd.inner;
+    } else if (rem >= (int64_t)nd.inner) {
+        ++q;
+        rem -= (int64_t)nd.inner;
+    }
+    r = (uint32_t)q;
+    c = (uint64_t)rem;
+}
+
+__device__ __forceinline__ void flat_row_pos(const BitFlatRows& nd, uint32_t r, int64_t& q1, int64_t& q2) {
+    uint32_t q = r;
+    for (int d = nd.nouter - 1; d > 0; --d) {
+        const uint32_t up = div31(q, nd.dv[d]);
+        const uint32_t i = q - up * nd.shape[d];
+        q = up;
+        q1 += (int64_t)i * nd.s1[d];
+        q2 += (int64_t)i * nd.s2[d];
+    }
+    q1 += (int64_t)q * nd.s1[0];
+    q2 += (int64_t)q * nd.s2[0];
+}
+
+// 32 bits of both sources for the result's elements e ... e + 31 (bit b = element e + b; bits of elements outside
+// [0, total) come out as anything: the caller masks them)
+template <bool BINARY>
+__device__ __forceinline__ void flat_src_words(const CUMO_BIT_DIGIT* a1, uint64_t p1, const CUMO_BIT_DIGIT* a2, uint64_t p2, const BitFlatRows& nd,
+                                               int64_t e, uint32_t& x, uint32_t& y) {
+    const uint64_t ec = e < 0 ? 0 : (uint64_t)e;
+    const unsigned shift = (unsigned)(ec - (uint64_t)e);  // e + shift = ec
+    x = y = 0;
+    if (ec >= nd.total) return;
+    uint32_t r;
+    uint64_t c;
+    flat_row_col(nd, ec, r, c);
+    int64_t q1 = (int64_t)p1, q2 = (int64_t)p2;
+    flat_row_pos(nd, r, q1, q2);
+    x = bits_at(a1, q1 + (int64_t)c, nd.nw1);
+    if (BINARY) y = bits_at(a2, q2 + (int64_t)c, nd.nw2);
+    const uint64_t avail = nd.inner - c;
+    if (avail < 32) {
+        const uint32_t keep = low_bits((unsigned)avail);
+        x &= keep;
+        y &= keep;
+        if (r + 1 < nd.rows) {
+            int64_t n1 = (int64_t)p1, n2 = (int64_t)p2;
+            flat_row_pos(nd, r + 1, n1, n2);
+            x |= bits_at(a1, n1, nd.nw1) << avail;
+            if (BINARY) y |= bits_at(a2, n2, nd.nw2) << avail;
+        }
+    }
+    x <<= shift;
+    y <<= shift;
+}
+
+template <int OP, bool BINARY, bool NT>
+__global__ __launch_bounds__(kBlock) void bit_rows_flat_kernel(const CUMO_BIT_DIGIT* a1, uint64_t p1, const CUMO_BIT_DIGIT* a2, uint64_t p2,
+                                                               CUMO_BIT_DIGIT* a3, uint64_t p3, unsigned lead, BitFlatRows nd) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint64_t nw3 = (p3 + nd.total + 31) >> 5;
+    const uint64_t nvec = (nw3 + lead + 3) >> 2;
+    const uint64_t endbit = p3 + nd.total;
+    // the row and column of a lane's vector come from a division once; from then on they move by what the grid's
+    // step is in rows and columns (the two lanes whose order is changed below divide every time)
+    bool have_rc = false;
+    uint32_t r = 0;
+    uint64_t c = 0;
+    const uint64_t step_bits = ((uint64_t)gridDim.x * kBlock) << 7;
+    const uint32_t step_r = (uint32_t)(step_bits / nd.inner);
+    const uint64_t step_c = step_bits - (uint64_t)step_r * nd.inner;
+    for (uint64_t it = (uint64_t)blockIdx.x * kBlock + threadIdx.x; it < nvec; it += (uint64_t)gridDim.x * kBlock) {
+        if (have_rc) {
+            r += step_r;
+            c += step_c;
+            if (c >= nd.inner) {
+                c -= nd.inner;
+                ++r;
+            }
+        }
+        // the run's last vector goes first (with the first one, in the launch's first wave): the two are put together word by
+        // word, a chain of loads that would otherwise stand alone at the end of the launch
+        const uint64_t v = it == 0 ? nvec - 1 : it - 1;
+        const int64_t w0 = (int64_t)(v << 2) - (int64_t)lead;
+        const bool whole = w0 >= 1 && (uint64_t)w0 + 4 <= nw3 - 1;
+        if (whole) {
+            if (!have_rc) {
+                flat_row_col(nd, ((uint64_t)w0 << 5) - p3, r, c);
+                have_rc = it >= 2;
+            }
+            int64_t q1 = (int64_t)p1, q2 = (int64_t)p2;
+            flat_row_pos(nd, r, q1, q2);
+            q1 += (int64_t)c;
+            q2 += (int64_t)c;
+            bool ok = ((uint64_t)q1 >> 5) + 5 <= nd.nw1 && (!BINARY || ((uint64_t)q2 >> 5) + 5 <= nd.nw2);
+            // a row ends inside the vector: its first `mine` bits are row r's, the rest the start of row r + 1, read as the
+            // 128 bits that have that start at bit `mine`
+            const bool split = c + 128 > nd.inner;
+            const unsigned mine = split ? (unsigned)(nd.inner - c) : 128u;
+            int64_t n1 = (int64_t)p1, n2 = (int64_t)p2;
+            if (split) {
+                flat_row_pos(nd, r + 1, n1, n2);
+                n1 -= (int64_t)mine;
+                n2 -= (int64_t)mine;
+                ok = ok && n1 >= 0 && ((uint64_t)n1 >> 5) + 5 <= nd.nw1 && (!BINARY || (n2 >= 0 && ((uint64_t)n2 >> 5) + 5 <= nd.nw2));
+            }
+            if (ok) {
+                // every load of the vector is asked for before the first is looked at
+                const Raw128 rx = raw128_load<NT>(a1, (uint64_t)q1);
+                Raw128 none;
+                none.v = 0;
+                none.e = 0;
+                none.sh = 0;
+                none.own = true;
+                Raw128 ry = none, rxn = none, ryn = none;  // (not copies of rx: a copy would wait for its words)
+                if (BINARY) ry = raw128_load<NT>(a2, (uint64_t)q2);
+                if (split) {
+                    rxn = raw128_load<NT>(a1, (uint64_t)n1);
+                    if (BINARY) ryn = raw128_load<NT>(a2, (uint64_t)n2);
+                }
+                uint4 x = raw128_bits(rx);
+                uint4 y = BINARY ? raw128_bits(ry) : make_uint4(0u, 0u, 0u, 0u);
+                if (split) {
+                    const uint4 xn = raw128_bits(rxn);
+                    const uint32_t m0 = low_bits(mine), m1 = mine > 32 ? low_bits(mine - 32) : 0u, m2 = mine > 64 ? low_bits(mine - 64) : 0u,
+                                   m3 = mine > 96 ? low_bits(mine - 96) : 0u;
+                    x = make_uint4((x.x & m0) | (xn.x & ~m0), (x.y & m1) | (xn.y & ~m1), (x.z & m2) | (xn.z & ~m2), (x.w & m3) | (xn.w & ~m3));
+                    if (BINARY) {
+                        const uint4 yn = raw128_bits(ryn);
+                        y = make_uint4((y.x & m0) | (yn.x & ~m0), (y.y & m1) | (yn.y & ~m1), (y.z & m2) | (yn.z & ~m2), (y.w & m3) | (yn.w & ~m3));
+                    }
+                }
+                u4 z;
+                z.x = bit_apply<OP>(x.x, y.x);
+                z.y = bit_apply<OP>(x.y, y.y);
+                z.z = bit_apply<OP>(x.z, y.z);
+                z.w = bit_apply<OP>(x.w, y.w);
+                if (NT) __builtin_nontemporal_store(z, reinterpret_cast<u4*>(a3 + w0));
+                else *reinterpret_cast<u4*>(a3 + w0) = z;
+                continue;
+            }
+        }
+        for (int64_t ww = w0 < 0 ? 0 : w0; ww < w0 + 4 && (uint64_t)ww < nw3; ++ww) {
+            const uint64_t w = (uint64_t)ww;
+            uint32_t x, y;
+            flat_src_words<BINARY>(a1, p1, a2, p2, nd, (int64_t)(w << 5) - (int64_t)p3, x, y);
+            const uint32_t z = bit_apply<OP>(x, y);
+            const unsigned lo = (w == 0) ? (unsigned)p3 : 0u;
+            const unsigned hi = ((w + 1) << 5) <= endbit ? 32u : (unsigned)(endbit - (w << 5));
+            const uint32_t mask = low_bits(hi) & ~low_bits(lo);
+            if (mask == 0xffffffffu) a3[w] = z;
+            else a3[w] = (z & mask) | (a3[w] & ~mask);
+        }
+    }
+}
+
+// The most blocks a launch of the vector kernels gets. A lane per vector, in blocks that come and go, keeps memory
+// busier than fewer blocks whose lanes loop (measured on 64 and 256 MiB operands: 0.73 -> 0.74 and 0.70 -> 0.80 of
+// peak for a & b, more where the sources are shifted), so the bound only guards the grid's size.
+// CUMO_HIP_BIT_VEC_GRID (read once) sets it in blocks per compute unit.
+unsigned bit_vec_grid_cap() {
+    static int64_t cap = -1;
+    if (cap < 0) {
+        const char* e = std::getenv("CUMO_HIP_BIT_VEC_GRID");
+        const long mult = e ? std::atol(e) : 0;
+        cap = mult >= 1 && mult <= (1 << 14) ? (int64_t)kNumCU * mult : (int64_t)1 << 22;
+    }
+    return (unsigned)cap;
+}
+
+// the flat form of the row kernel, for operands bit_rows_launch has vetted (strides only, innermost step 1,
+// no position below zero); false when the result's rows do not follow one another or the shape is outside its limits
+template <int OP, bool BINARY>
+bool bit_rows_flat_launch(cumo_na_bit_iarray_stridx_t* const* ops, const cumo_na_indexer_t* indexer, const uint64_t* reach) {
+    const int n = indexer->ndim;
+    const uint64_t inner = indexer->shape[n - 1];
+    if (inner < 128) return false;
+    uint64_t rows = 1;
+    int64_t want = (int64_t)inner;
+    for (int d = n - 2; d >= 0; --d) {
+        if ((int64_t)CUMO_SDX_GET_STRIDE(ops[2]->stridx[d]) != want && indexer->shape[d] != 1) return false;
+        want *= (int64_t)indexer->shape[d];
+        rows *= indexer->shape[d];
+    }
+    if (rows == 0 || rows >= (1ull << 31) || rows * inner >= (1ull << 52)) return false;
+    BitFlatRows nd;
+    std::memset(&nd, 0, sizeof(nd));
+    // outer dimensions, merged where both sources step through two of them as through one
+    int m = 0;
+    for (int d = 0; d < n - 1; ++d) {
+        if (indexer->shape[d] == 1) continue;
+        const int64_t t1 = (int64_t)CUMO_SDX_GET_STRIDE(ops[0]->stridx[d]), t2 = (int64_t)CUMO_SDX_GET_STRIDE(ops[1]->stridx[d]);
+        if (m > 0 && nd.s1[m - 1] == t1 * (int64_t)indexer->shape[d] && nd.s2[m - 1] == t2 * (int64_t)indexer->shape[d]) {
+            nd.shape[m - 1] *= (uint32_t)indexer->shape[d];
+            nd.s1[m - 1] = t1;
+            nd.s2[m - 1] = t2;
+            continue;
+        }
+        if (m == kFlatOuter) return false;
+        nd.shape[m] = (uint32_t)indexer->shape[d];
+        nd.s1[m] = t1;
+        nd.s2[m] = t2;
+        ++m;
+    }
+    if (m == 0) {  // a single row
+        nd.shape[0] = 1;
+        m = 1;
+    }
+    for (int d = 0; d < m; ++d) nd.dv[d] = div31_make(nd.shape[d]);
+    nd.nouter = m;
+    nd.rows = (uint32_t)rows;
+    nd.inner = inner;
+    nd.total = rows * inner;
+    nd.inv_inner = 1.0 / (double)inner;
+    nd.nw1 = reach[0];
+    nd.nw2 = reach[1];
+    CUMO_BIT_DIGIT* a3 = ops[2]->ptr + ops[2]->pos / 32;
+    const uint64_t p3 = ops[2]->pos % 32;
+    const uint64_t nw3 = (p3 + nd.total + 31) >> 5;
+    const unsigned lead = (unsigned)(((uintptr_t)a3 % 16) / sizeof(CUMO_BIT_DIGIT));
+    const dim3 g(grid_for((nw3 + lead + 3) / 4, bit_vec_grid_cap())), b(kBlock);
+    if (stream_past_caches(nw3 * 4 * (BINARY ? 3 : 2)))
+        hipLaunchKernelGGL((bit_rows_flat_kernel<OP, BINARY, true>), g, b, 0, current_stream(), (const CUMO_BIT_DIGIT*)ops[0]->ptr, (uint64_t)ops[0]->pos,
+                           (const CUMO_BIT_DIGIT*)ops[1]->ptr, (uint64_t)ops[1]->pos, a3, p3, lead, nd);
+    else
+        hipLaunchKernelGGL((bit_rows_flat_kernel<OP, BINARY, false>), g, b, 0, current_stream(), (const CUMO_BIT_DIGIT*)ops[0]->ptr, (uint64_t)ops[0]->pos,
+                           (const CUMO_BIT_DIGIT*)ops[1]->ptr, (uint64_t)ops[1]->pos, a3, p3, lead, nd);
+    cumo_cuda_runtime_check_kernel_launch();
+    return true;
+}
+
 // launches the row form when the operands allow it; false: the caller uses the bit-by-bit kernel
 template <int OP, bool BINARY>
 bool bit_rows_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_t* a2, cumo_na_bit_iarray_stridx_t* a3, cumo_na_indexer_t* indexer) {
@@ -234,6 +516,7 @@ bool bit_rows_launch(cumo_na_bit_iarray_stridx_t* a1, cumo_na_bit_iarray_stridx_
     }
     nd.nw1 = reach[0];
     nd.nw2 = reach[1];
+    if (bit_rows_flat_launch<OP, BINARY>(ops, indexer, reach)) return true;
     hipLaunchKernelGGL((bit_rows_kernel<OP, BINARY>), dim3(grid_for(nd.items, kNumCU * 32)), dim3(kBlock), 0, current_stream(),
                        (const CUMO_BIT_DIGIT*)ops[0]->ptr, (uint64_t)ops[0]->pos, (const CUMO_BIT_DIGIT*)ops[1]->ptr, (uint64_t)ops[1]->pos, a3->ptr,
                        (uint64_t)a3->pos, nd);
@@ -470,7 +753,7 @@ void launch_contiguous(CUMO_BIT_DIGIT* a1, size_t p1, CUMO_BIT_DIGIT* a2, size_t
     const uint64_t nw3 = (p3 + n + 31) >> 5;
     if (nw3 >= 64 && p1 < 32 && p2 < 32 && p3 < 32) {
         const unsigned lead = (unsigned)(((uintptr_t)a3 % 16) / sizeof(CUMO_BIT_DIGIT));
-        const dim3 g(grid_for((nw3 + lead + 3) / 4, kNumCU * 16)), b(kBlock);
+        const dim3 g(grid_for((nw3 + lead + 3) / 4, bit_vec_grid_cap())), b(kBlock);
         if (stream_past_caches(nw3 * 4 * (BINARY ? 3 : 2)))
             hipLaunchKernelGGL((bit_contiguous_vec_kernel<OP, BINARY, true>), g, b, 0, current_stream(), a1, (uint64_t)p1, a2, (uint64_t)p2, a3,
                                (uint64_t)p3, n, lead);

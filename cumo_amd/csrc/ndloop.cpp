@@ -2324,6 +2324,24 @@ int cumo_hip_na_bit_reduce(const char* op, const cumo_hip_narray_t* x, unsigned 
         rc = cumo_hip_na_fill(z, all ? 1.0 : 0.0);
         if (rc || total_of(x) == 0) return rc;
     }
+    if (by_counts && lp.reduce_dim == 1 && lp.ndim >= 2 && lp.args[0].step[lp.ndim - 1] == 1) {
+        // rows that start on words, results that are consecutive bits: one launch from the rows to the packed bits
+        const int nkeep = lp.ndim - 1;
+        bool rows_ok = true;
+        uint64_t nrows = lp.n[nkeep - 1];
+        for (int d = nkeep - 2; d >= 0 && rows_ok; d--) {
+            rows_ok = lp.args[0].step[d] == lp.args[0].step[d + 1] * (ssize_t)lp.n[d + 1];
+            nrows *= lp.n[d];
+        }
+        ssize_t zs = 1;
+        for (int d = nkeep - 1; d >= 0 && rows_ok; d--) {
+            rows_ok = lp.args[1].step[d] == zs;
+            zs *= (ssize_t)lp.n[d];
+        }
+        if (rows_ok && cumo_hip_bit_anyall_rows_kernel_launch((CUMO_BIT_DIGIT*)lp.args[0].ptr, lp.args[0].bitpos, nrows, lp.args[0].step[nkeep - 1],
+                                                              lp.n[lp.ndim - 1], all ? 1 : 0, (CUMO_BIT_DIGIT*)lp.args[1].ptr, lp.args[1].bitpos))
+            return CUMO_HIP_OK;
+    }
     if (by_counts) {
         NA counts;
         std::memset(&counts, 0, sizeof(counts));

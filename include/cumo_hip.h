@@ -603,6 +603,13 @@ int  cumo_hip_bit_count_run_store_kernel_launch(CUMO_BIT_DIGIT* a, size_t pos, u
  * in the reference, which walks the runs on the host: gen/tmpl_bit/bit_reduce.c:106-146). Bits of dst outside
  * [pos, pos + n) stay as they are. */
 void cumo_hip_bit_from_counts_kernel_launch(const uint64_t* counts, uint64_t n, int zero_is_one, CUMO_BIT_DIGIT* dst, size_t pos);
+/* all? (all != 0) or any? of each of `rows` runs of n bits, run r at bit pos + r * row_step of `in`, into bit
+ * out_pos + r of `out`, in one launch; pos and row_step must be multiples of 32. Returns 1 when launched, 0 when
+ * the shape is one the caller should hand to the counts instead (short or few runs, unaligned rows). The
+ * reference launches one reduction per run from a walk on the host (gen/tmpl_bit/bit_reduce.c:106-146). Bits of
+ * out outside [out_pos, out_pos + rows) stay as they are. */
+int  cumo_hip_bit_anyall_rows_kernel_launch(CUMO_BIT_DIGIT* in, size_t pos, uint64_t rows, int64_t row_step, uint64_t n, int all,
+                                            CUMO_BIT_DIGIT* out, size_t out_pos);
 
 /* Row-wise softmax and layer normalisation in one pass (no counterpart in the
  * reference, where they are chains of 5 and 6 array operations,

@@ -142,7 +142,7 @@ def test_rows_of_bits_in_views_word_by_word():
     such a view leaves every bit around it as it was."""
     import cumo_amd
     rng = np.random.default_rng(611)
-    for shape in [(70, 131), (5, 4099), (300, 33), (9, 7, 67), (64, 64), (33, 1000)]:
+    for shape in [(70, 131), (5, 4099), (300, 33), (9, 7, 67), (64, 64), (33, 1000), (6, 5, 300), (3, 4, 5, 129), (600, 4097)]:
         ha = rng.integers(0, 2, size=shape).astype(np.uint8)
         hb = rng.integers(0, 2, size=shape).astype(np.uint8)
         a, b = cumo_amd.Bit.cast(ha), cumo_amd.Bit.cast(hb)
@@ -171,6 +171,22 @@ def test_rows_of_bits_in_views_word_by_word():
             z[key] = a[src_key]
             hz[key] = ha[src_key]
             assert (z.to_numpy() == hz).all(), (shape, key)
+
+
+def test_windows_of_a_large_matrix_into_a_fresh_result():
+    """Rows of 32767 bits that follow one another in the result while the sources' rows are 32768 apart:
+    the result is written as one run of whole vectors (past the size from which stores bypass the
+    caches), a row ending inside one vector in four."""
+    import cumo_amd
+    rng = np.random.default_rng(619)
+    shape = (4100, 32768)
+    ha = np.unpackbits(np.frombuffer(rng.bytes(shape[0] * shape[1] // 8), dtype=np.uint8)).reshape(shape)
+    hb = np.unpackbits(np.frombuffer(rng.bytes(shape[0] * shape[1] // 8), dtype=np.uint8)).reshape(shape)
+    a, b = cumo_amd.Bit.cast(ha), cumo_amd.Bit.cast(hb)
+    assert ((a[:, 1:] ^ b[:, :-1]).to_numpy() == (ha[:, 1:] ^ hb[:, :-1])).all()
+    assert ((a[::-1, 5:] & b[:, :-5]).to_numpy() == (ha[::-1, 5:] & hb[:, :-5])).all()
+    assert ((~a[1:, 31:-1]).to_numpy() == 1 - ha[1:, 31:-1]).all()
+    assert (a[::2, 7:].copy().to_numpy() == ha[::2, 7:]).all()
 
 
 @pytest.mark.parametrize("n", [2048, 2049, 5000, 100003, (1 << 22) + 77])
@@ -355,3 +371,63 @@ def test_counts_down_columns_of_word_aligned_rows():
             counts = (rows - h.sum(axis=0, dtype=np.uint64)) if count_false else h.sum(axis=0, dtype=np.uint64)
             want = counts if overwrite else counts + start
             assert (out.to_numpy() == want).all(), (overwrite, count_false)
+
+
+def test_all_any_along_word_aligned_rows():
+    """all? / any? / none? along rows that start on word boundaries go from the rows to the packed
+    result in one launch: whole 128-bit vectors and single words per lane, a last word that is partly
+    row, rows decided at their first and at their last bit, kept dimensions that merge, rows of a view
+    taken backwards and every other one, and a result that starts inside a word (the launcher itself:
+    the bits around the result stay)."""
+    import ctypes as C
+    import cumo_amd
+    from cumo_amd import _lib
+    rng = np.random.default_rng(617)
+
+    def rows_of(shape):
+        # mostly rows of ones / zeros, so that all? and any? both have both answers; a few decided by one bit
+        h = np.empty(shape, dtype=np.uint8)
+        flat = h.reshape(-1, shape[-1])
+        kind = rng.integers(0, 6, size=flat.shape[0])
+        flat[:] = (kind % 2)[:, None]
+        for k, col in ((2, 0), (3, 0), (4, -1), (5, -1)):
+            flat[kind == k, col] ^= 1
+        mid = rng.integers(0, shape[-1], size=flat.shape[0])
+        pick = rng.random(flat.shape[0]) < 0.2
+        flat[pick, mid[pick]] ^= 1
+        return h
+
+    def check(dv, hv, what):
+        ax = hv.ndim - 1
+        assert (dv.all_p(axis=ax).to_numpy() == hv.all(axis=ax)).all(), what
+        assert (dv.any_p(axis=ax).to_numpy() == hv.any(axis=ax)).all(), what
+        assert (dv.none_p(axis=ax).to_numpy() == ~hv.any(axis=ax)).all(), what
+
+    for shape in [(4096, 4096), (5000, 8192 + 32), (4100, 32768), (4200, 8192), (70, 100, 4096 + 64), (9000, 4096), (4097, 1 << 16)]:
+        h = rows_of(shape)
+        b = cumo_amd.Bit.cast(h)
+        check(b, h, shape)
+        for key in ((Ellipsis, slice(0, 5000)), (Ellipsis, slice(64, None)), (slice(None, None, -1),), (slice(None, None, 2), Ellipsis, slice(32, 32 + 4100)),
+                    (Ellipsis, slice(96, 96 + 4099))):
+            hv, dv = h[key], b[key]
+            if hv.shape[-1] >= 4096:
+                check(dv, hv, (shape, key))
+
+    f = _lib.fn("cumo_hip_bit_anyall_rows_kernel_launch", C.c_int,
+                [C.c_void_p, C.c_size_t, C.c_uint64, C.c_int64, C.c_uint64, C.c_int, C.c_void_p, C.c_size_t])
+    rows, cols = 4101, 4096 + 32
+    h = rows_of((rows, cols))
+    b = cumo_amd.Bit.cast(h)
+    for out_pos in (0, 5, 31, 37):
+        for all_ in (0, 1):
+            before = (rng.random(out_pos + rows + 70) < 0.5).astype(np.uint8)
+            out = cumo_amd.Bit.cast(before)
+            took = _lib.call(f, b._buf.ptr, 32 * 0, rows, cols, cols - 7, all_, out._buf.ptr, out_pos)
+            assert took == 1
+            want = before.copy()
+            hv = h[:, :cols - 7]
+            want[out_pos:out_pos + rows] = hv.all(axis=1) if all_ else hv.any(axis=1)
+            assert (out.to_numpy() == want).all(), (out_pos, all_)
+    # shapes it leaves to the counts
+    assert _lib.call(f, b._buf.ptr, 3, rows, cols, 4096, 1, out._buf.ptr, 0) == 0
+    assert _lib.call(f, b._buf.ptr, 0, 100, cols, 4096, 1, out._buf.ptr, 0) == 0
