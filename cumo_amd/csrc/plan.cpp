@@ -266,7 +266,21 @@ void plan_reduce(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out
             // the general kernels take: 41 -> 29 us).
             int bits = 0;
             if (s > 16) {
-                bits = 2;
+                // a second launch folds: the block is as wide as the outputs allow (up to 256 vectors, 4 KiB of every
+                // row it reads), what is left of its 256 lanes shares the axis, and the axis is cut across enough
+                // blocks to fill the device (1024 of them) while a lane's part of it keeps 32 positions
+                // (at least four blocks side by side where that leaves them 64 vectors: the fold of more than
+                // 256 parts costs more than the wider block gains)
+                uint64_t wide = 64;
+                while (wide < 256 && wide * 8 <= threads) wide <<= 1;
+                while (wide > 16 && wide / 2 >= threads) wide >>= 1;
+                while ((256u >> bits) > wide) ++bits;
+                const uint64_t col_blocks = (threads + wide - 1) / wide;
+                uint64_t parts = ((uint64_t)kNumCU * 4 + col_blocks - 1) / col_blocks;
+                if (parts > (fits >> bits)) parts = fits >> bits;
+                if (parts > 1024) parts = 1024;
+                if (parts < 1) parts = 1;
+                s = parts << bits;
             } else {
                 while (bits < 4 && (2ull << bits) <= s) ++bits;
             }

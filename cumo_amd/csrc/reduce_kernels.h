@@ -716,12 +716,14 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
         uint64_t grid = (groups + per_block - 1) / per_block;
         if (plan.n_split > 1) {
             // The axis is cut across blocks as well: accumulators to scratch, a second launch folds them.
-            if (p.lsplit_bits == 0 || grid > 65535) return 0;
+            if (grid > 65535) return 0;
             const uint64_t bchunk = (plan.red_total + (uint64_t)plan.n_split - 1) / (uint64_t)plan.n_split;
             const uint64_t n_split = (plan.red_total + bchunk - 1) / bchunk;  // no part is empty
             if (n_split < 2 || n_split > 65535) return 0;
             p.n_split = (uint32_t)n_split;
-            const uint64_t scratch_bytes = sizeof(Acc) * plan.out_total * n_split;
+            p.chunk = bchunk;
+            const size_t parts_row = rs_parts_row(p.n_out, p.out_inner, V);
+            const uint64_t scratch_bytes = sizeof(Acc) * parts_row * n_split;
             if (fixed) {
                 if (scratch_bytes > fixed->bytes) return -1;
                 p.partial = fixed->ptr;
@@ -734,13 +736,15 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
             if (nt) hipLaunchKernelGGL((red_scol_kernel<Impl, V, true, true, 4, true>), g2, b, 0, stream, p, impl);
             else hipLaunchKernelGGL((red_scol_kernel<Impl, V, false, true, 4, true>), g2, b, 0, stream, p, impl);
             cumo_cuda_runtime_check_kernel_launch();
-            RedKParams kp;
-            red_fill_params(&kp, plan, arg, out2, index_mode);
-            kp.tpr_bits = 0;
-            kp.lsplit_bits = 0;
-            kp.n_split = n_split;
-            kp.chunk = bchunk;
-            red_fold_partials<Impl>(plan, kp, reinterpret_cast<Acc*>(p.partial), impl, stream);
+            // the fold: as many lanes to a group of outputs as give each at most eight parts (a group's 16 bytes of every
+            // part next to its neighbours': at least four groups side by side)
+            RedSParams pf = p;
+            pf.lsplit_bits = 0;
+            while (pf.lsplit_bits < 6 && (8ull << pf.lsplit_bits) < n_split) ++pf.lsplit_bits;
+            const uint64_t fold_groups = (uint64_t)kRedBlock >> pf.lsplit_bits;
+            const dim3 gf((unsigned)((parts_row / V + fold_groups - 1) / fold_groups));
+            hipLaunchKernelGGL((red_fold_parts_kernel<Impl, V>), gf, b, 0, stream, pf, impl);
+            cumo_cuda_runtime_check_kernel_launch();
             if (!fixed) cumo_cuda_runtime_free(p.partial);
             return 1;
         }

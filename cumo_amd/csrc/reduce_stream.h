@@ -42,6 +42,7 @@ struct RedSParams {
     uint32_t n_out;        // outputs
     uint32_t out_inner;    // extent of the inner output dimension (= n_out when there is one dimension)
     uint32_t n_split;      // split form: blocks per output
+    uint64_t chunk;        // column form cut across blocks: positions of the axis a block takes 
     uint32_t group;        // split form: blocks that count in on one first-level ticket
     uint32_t tstride;      // split form: words between two tickets (tickets in one cache line serialise in one memory channel)
     uint32_t tpr_bits;     // row form: 2^tpr_bits lanes share an output
@@ -322,6 +323,84 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
     }
 }
 
+// Second launch of the column form cut across blocks: folds partial[part][output] (rows of rs_parts_row
+// accumulators) into the results. 2^p.lsplit_bits lanes share a group of VEC outputs, each with a run of its
+// parts in axis order, up to eight of them in flight, and combine pairwise through LDS, earlier parts on the left.
+__host__ __device__ __forceinline__ size_t rs_parts_row(uint32_t n_out, uint32_t out_inner, int vec) {
+    const uint32_t gpo = (out_inner + vec - 1) / vec;
+    return (size_t)gpo * vec * (n_out / out_inner);
+}
+
+template <class Impl, int VEC>
+__global__ __launch_bounds__(kRedBlock) void red_fold_parts_kernel(RedSParams p, Impl impl) {
+    typedef typename Impl::Acc Acc;
+    constexpr int B = 8;
+    __shared__ Acc slots[kRedBlock][VEC];
+    const unsigned pbits = p.lsplit_bits;
+    const unsigned PG = 1u << pbits, OV = (unsigned)kRedBlock >> pbits;
+    const unsigned ov = threadIdx.x & (OV - 1), pg = threadIdx.x >> (8u - pbits);
+    const size_t row = rs_parts_row(p.n_out, p.out_inner, VEC);
+    const uint32_t o = (blockIdx.x * OV + ov) * VEC;   // the group's first output (groups are whole here: 1-D outputs, or out_inner a multiple of VEC)
+    const bool ok = o < p.n_out;
+    const uint32_t per = (p.n_split + PG - 1) / PG;
+    const uint32_t k0 = pg * per < p.n_split ? pg * per : p.n_split;
+    const uint32_t k1 = k0 + per < p.n_split ? k0 + per : p.n_split;
+    const Acc* base = reinterpret_cast<const Acc*>(p.partial) + (ok ? o : 0);
+    Acc total[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) total[j] = impl.identity();
+    for (uint32_t k = k0; k < k1; k += B) {
+        Acc v[B][VEC];
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const uint32_t kk = k + b < k1 ? k + b : k1 - 1;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[b][j] = base[(size_t)kk * row + j];
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b)
+            if (k + b < k1) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) impl.combine(v[b][j], total[j]);
+            }
+    }
+    for (unsigned stride = 1; stride < PG; stride <<= 1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) slots[threadIdx.x][j] = total[j];
+        __syncthreads();
+        if ((pg & (2 * stride - 1)) == 0 && pg + stride < PG) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) impl.combine(slots[(pg + stride) * OV + ov][j], total[j]);
+        }
+        __syncthreads();
+    }
+    if (pg != 0 || !ok) return;
+    if constexpr (has_exact<Impl>::value) {
+        // the parts are plain values in axis order: where the fast fold cannot tell which of two equal
+        // values came first, the exact rule over the same values
+        typedef typename Impl::Exact Exact;
+        const Exact ex = impl.exact();
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            if (impl.needs_exact(total[j])) {
+                typename Exact::Acc e = ex.identity();
+                for (uint32_t k = 0; k < p.n_split; ++k) ex.accumulate(base[(size_t)k * row + j], (int64_t)k, e);
+                total[j] = impl.from_exact(e);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        const uint32_t oj = o + j;
+        if (oj >= p.n_out) break;
+        const uint32_t q0 = p.out_inner == p.n_out ? 0u : oj / p.out_inner;
+        const uint32_t q1 = oj - q0 * p.out_inner;
+        const int64_t a = (int64_t)q0 * p.out_step[0] + (int64_t)q1 * p.out_step[1];
+        const int64_t b2 = (Impl::NOUT > 1) ? (int64_t)q0 * p.out2_step[0] + (int64_t)q1 * p.out2_step[1] : 0;
+        impl.store(total[j], p.out + a, (Impl::NOUT > 1) ? (p.out2 + b2) : nullptr);
+    }
+}
+
 // The exact second fold by ONE wave over the tiles that a whole block (tpr_bits 8) folded: the
 // tiles first, first + every, ... of kRedBlock * VEC * kRsUnroll elements each, every vector of
 // them taken by one of the 64 lanes. For the streaming blocks of the kernel below, where only
@@ -475,8 +554,8 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
 // U: positions of the axis a lane has in flight (more when the outputs alone give too few lanes
 // to keep the memory system busy: a block still reads 4 KiB runs of every row it touches).
 // PARTIAL: the axis is also cut across blocks, p.n_split ways (blockIdx.y says which part this
-// block has); a block leaves its accumulators in p.partial[output * n_split + part] and a second
-// launch folds them. Blocks stay 128 or 256 vectors wide that way however few the outputs are.
+// block has); a block leaves its accumulators in p.partial[part][output] and a second launch
+// (red_fold_parts_kernel) folds them. Blocks stay 128 or 256 vectors wide that way however few the outputs are.
 template <class Impl, int VEC, bool NT, bool LOCAL, int U, bool PARTIAL = false>
 __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl impl) {
     typedef typename Impl::In In;
@@ -496,7 +575,7 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
     // this block's stretch of the axis, then this lane's part of it
     uint64_t b0 = 0, b1 = p.n;
     if (PARTIAL) {
-        const uint64_t bchunk = (p.n + p.n_split - 1) / p.n_split;
+        const uint64_t bchunk = p.chunk;
         b0 = (uint64_t)blockIdx.y * bchunk;
         if (b0 > p.n) b0 = p.n;
         b1 = b0 + bchunk;
@@ -593,11 +672,17 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
             __syncthreads();
         }
         if (PARTIAL) {
+            // partial[part][output], a part's outputs padded to whole groups: the lanes of a block write one run
             if (ok && s == 0) {
-                Acc* partial = reinterpret_cast<Acc*>(p.partial);
+                Acc* mine = reinterpret_cast<Acc*>(p.partial) + (size_t)blockIdx.y * ((size_t)gpo * VEC * (p.n_out / p.out_inner)) + i_out0;
+                if (i_out0 == own0) {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j)
-                    if (i_out0 + j >= own0) partial[(size_t)(i_out0 + j) * p.n_split + blockIdx.y] = acc[j];
+                    for (int j = 0; j < VEC; ++j) mine[j] = acc[j];
+                } else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (i_out0 + j >= own0) mine[j] = acc[j];
+                }
             }
             continue;
         }

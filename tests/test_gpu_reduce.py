@@ -248,7 +248,7 @@ def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((700, 24), 0), ((3, 700, 24), 1), ((40000, 8), 0), ((2, 5000, 3), 1), ((130, 1024), 0),
                                         ((3000, 1000), 0), ((4096, 520), 0), ((2, 2100, 516), 1), ((3000, 1001), 0), ((700, 4095), 0),
-                                        ((40, 70001), 0), ((5000, 259), 0),
+                                        ((40, 70001), 0), ((5000, 259), 0), ((70000, 64), 0), ((8192, 1028), 0),
                                         ((3, 700, 67), 1), ((5, 64, 1023), 1), ((2, 2100, 517), 1), ((9, 130, 259), 1), ((64, 40, 131), 1),
                                         ((300, 20, 33), 1)])
 def test_few_outputs_across_memory_share_the_axis_inside_a_block(tname, dt, shape, axis):
