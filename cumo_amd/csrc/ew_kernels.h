@@ -31,12 +31,21 @@
 #include "common.h"
 #include "plan.h"
 #include "div31.h"
+#include "ew_ops.h"
 
 #include <cstdlib>
 #include <type_traits>
 #include <cstring>
 
 namespace cumo_hip {
+
+// An operator that reads the LDS tables of ew_ops.h declares USES_TABLES; every kernel here fills them first.
+template <class O, class = void> struct op_uses_tables { static constexpr bool value = false; };
+template <class O> struct op_uses_tables<O, decltype((void)O::USES_TABLES)> { static constexpr bool value = O::USES_TABLES; };
+template <class Op>
+__device__ __forceinline__ void ew_op_prepare() {
+    if constexpr (op_uses_tables<Op>::value) float_tables_prepare();
+}
 
 constexpr int kEwBlock = 256;
 constexpr int kEwUnroll = 4;
@@ -275,6 +284,7 @@ __device__ __forceinline__ void ew_row_offsets(const EwKParams& p, uint64_t row,
 //   __device__ bool operator()(A x, B y, R& z) const   -- false: reject the element (do not store, raise flag)
 template <class Op, int VEC>
 __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, typename Op::S sv) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;
@@ -467,6 +477,7 @@ __device__ __forceinline__ int64_t ew_period_row(const EwPeriod& pr, uint32_t q)
 template <class Op, int VEC, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_flat_period_kernel(const char* __restrict__ pfull, const char* __restrict__ pper,
                                                                   char* __restrict__ pz, uint32_t n, EwPeriod pr, int* flag, Op op) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     typedef typename Op::R R;
     static_assert(Op::NIN == 2, "two inputs");
@@ -558,6 +569,8 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
     // Every vector is evaluated, loaded or not (an absent one holds zeros and is not stored):
     // with no branch around the arithmetic the compiler interleaves the elements of all the
     // lane's vectors, which the long dependent chains of the NMath functions need.
+    // (the tables of an operator that reads them are filled after the loads have gone out)
+    ew_op_prepare<Op>();
     R zv[UNR][VEC];
     bool ok[UNR];
     if constexpr (op_has_rare<Op>::value) {
@@ -567,23 +580,37 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
         A xe[UNR * VEC];
         B ye[UNR * VEC];
         bool any = false;
+        // which operand the scalar stands for is the same for every element: with it known at compile time
+        // (three copies of the arithmetic under one uniform switch) the scalar's share of the arithmetic is
+        // done once and no element selects its operands. Only where the arithmetic is what bounds the kernel.
+        auto arithmetic = [&](auto mode) {
+            constexpr int SM = decltype(mode)::value;
 #pragma unroll
-        for (int u = 0; u < UNR; ++u) {
-            ok[u] = true;
+            for (int u = 0; u < UNR; ++u) {
+                ok[u] = true;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                A x = xv[u][j];
-                B y = B();
-                if (TWO) {
-                    if (use_scalar == 0) y = yv[u][j];
-                    else if (use_scalar == 1) y = (B)sv;
-                    else { y = (B)x; x = (A)sv; }
+                for (int j = 0; j < VEC; ++j) {
+                    A x = xv[u][j];
+                    B y = B();
+                    if (TWO) {
+                        const int sm = SM >= 0 ? SM : use_scalar;
+                        if (sm == 0) y = yv[u][j];
+                        else if (sm == 1) y = (B)sv;
+                        else { y = (B)x; x = (A)sv; }
+                    }
+                    xe[u * VEC + j] = x;
+                    ye[u * VEC + j] = y;
+                    op.fast(x, y, zv[u][j]);
+                    any = any || op.rare(x, y);
                 }
-                xe[u * VEC + j] = x;
-                ye[u * VEC + j] = y;
-                op.fast(x, y, zv[u][j]);
-                any = any || op.rare(x, y);
             }
+        };
+        if constexpr (TWO && op_uses_tables<Op>::value) {
+            if (use_scalar == 0) arithmetic(std::integral_constant<int, 0>{});
+            else if (use_scalar == 1) arithmetic(std::integral_constant<int, 1>{});
+            else arithmetic(std::integral_constant<int, 2>{});
+        } else {
+            arithmetic(std::integral_constant<int, -1>{});
         }
         if (any) {
 #pragma clang loop unroll(disable)
@@ -658,6 +685,7 @@ template <class Op, int VEC, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_kernel(const char* __restrict__ px, const char* __restrict__ py,
                                                                CUMO_BIT_DIGIT* __restrict__ pz, uint64_t n, int use_scalar, Op op,
                                                                typename Op::S sv) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     typedef typename Op::B B;
     constexpr int NIN = Op::NIN;
@@ -729,6 +757,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_kernel(const char* __res
 template <class Op, int VEC, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_period_kernel(const char* __restrict__ pfull, const char* __restrict__ pper,
                                                                       CUMO_BIT_DIGIT* __restrict__ pz, uint32_t n, EwPeriod pr, Op op) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     static_assert(Op::NIN == 2, "two inputs");
     constexpr int UNR = 4;
@@ -829,6 +858,7 @@ struct EwR2Params {
 // the caches, so it is read with plain loads while the full-size operands stream past.
 template <class Op, int VEC, int NTM>
 __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op, typename Op::S sv) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;
@@ -998,6 +1028,7 @@ __device__ __forceinline__ void ew_rows2_lean_body(const EwR2LeanParams& p, Op o
 
 template <class Op, int VEC, int NTM>
 __global__ __launch_bounds__(kEwBlock) void ew_rows2_lean_kernel(EwR2LeanParams p, Op op, typename Op::S sv) {
+    ew_op_prepare<Op>();
     const unsigned TX = 1u << p.tx_bits;
     const unsigned tx = threadIdx.x & (TX - 1);
     const unsigned ty = threadIdx.x >> p.tx_bits;
@@ -1119,6 +1150,7 @@ __device__ __forceinline__ void ew_tile_at(const EwTParams& p, uint64_t tile, ui
 // fresh operands: 58 us with plain accesses, 50 us with non-temporal ones).
 template <class Op, int TF, int TG, bool PREFETCH, int TRMODE, bool NT>
 __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p, Op op, typename Op::S sv) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;
@@ -1377,6 +1409,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_transpose_vec_kernel(EwTParams p,
 // The element-wise form, for operands that do not tolerate 128-bit accesses.
 template <class Op, int TG>
 __global__ __launch_bounds__(kEwBlock) void ew_transpose_kernel(EwTParams p, Op op, typename Op::S sv) {
+    ew_op_prepare<Op>();
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;

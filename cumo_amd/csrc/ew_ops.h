@@ -55,6 +55,65 @@ __device__ __forceinline__ double int_to_double(int k) {
     return __hiloint2double(0x43300000, (int)((uint32_t)k ^ 0x80000000u)) - 4503601774854144.0;
 }
 
+// ---- table-driven log2 and exp2 (for results that are rounded to float) ------------------
+// 64 entries {1 / c, log2 c} for the logarithm and 32 values 2^(j/32) for the exponential take
+// the place of a division and of half a polynomial each (float_tables.inc, written by
+// make_float_tables.py, says how they are laid out). On the device the tables live in LDS: an
+// operator that reads them declares USES_TABLES, and a kernel that runs such an operator
+// calls float_tables_prepare() with all its threads before the first element.
+#include "float_tables.inc"
+constexpr int kFloatTableDoubles = 128 + 32;
+#ifdef CUMO_HIP_HOST_CHECK
+static const double kFloatTablesHost[kFloatTableDoubles] = {CUMO_HIP_LOG2_TABLE, CUMO_HIP_EXP2_TABLE};
+inline const double* float_tables() { return kFloatTablesHost; }
+#else
+__device__ const double kFloatTablesDevice[kFloatTableDoubles] = {CUMO_HIP_LOG2_TABLE, CUMO_HIP_EXP2_TABLE};
+__device__ __forceinline__ double* float_tables_lds() {
+    __shared__ double tables[kFloatTableDoubles];
+    return tables;
+}
+__device__ __forceinline__ const double* float_tables() { return float_tables_lds(); }
+__device__ __forceinline__ void float_tables_prepare() {
+    double* t = float_tables_lds();
+    for (unsigned i = threadIdx.x; i < (unsigned)kFloatTableDoubles; i += blockDim.x) t[i] = kFloatTablesDevice[i];
+    __syncthreads();
+}
+#endif
+// log2(x) for a positive, finite, normal double to 2^-44 relative (also next to 1, where the
+// entry {1, 0} leaves the polynomial alone): 8 multiply-adds and one 16-byte table read.
+__device__ __forceinline__ double log2_by_table(double x, const double* tab) {
+    const uint32_t hx = (uint32_t)__double2hiint(x);
+    const uint32_t t = hx - 0x3fe6a000u;
+    const int k = (int)t >> 20;
+    const uint32_t i = (t >> 14) & 63u;
+    const double m = __hiloint2double((int)(hx - (t & 0xfff00000u)), __double2loint(x));
+    const double invc = tab[2 * i], logc = tab[2 * i + 1];
+    const double z = __builtin_fma(m, invc, -1.0);
+    double p = CUMO_HIP_LOG2_L6;
+    p = __builtin_fma(p, z, CUMO_HIP_LOG2_L5);
+    p = __builtin_fma(p, z, CUMO_HIP_LOG2_L4);
+    p = __builtin_fma(p, z, CUMO_HIP_LOG2_L3);
+    p = __builtin_fma(p, z, CUMO_HIP_LOG2_L2);
+    p = __builtin_fma(p, z, CUMO_HIP_LOG2_L1);
+    return __builtin_fma(z, p, logc + int_to_double(k));
+}
+// 2^e for -1000 < e < 1000 to 2^-39 relative: e = (32 q + j) / 32 + r with |r| <= 1/64 from one
+// addition of 1.5 * 2^47 (whose last mantissa bit is worth 1/32), 2^(j/32) from the table with
+// q added to its exponent field, 2^r from four multiply-adds.
+__device__ __forceinline__ double exp2_by_table(double e, const double* tab) {
+    const double big = 211106232532992.0;  // 1.5 * 2^47
+    const double t0 = e + big;
+    const uint32_t ki = (uint32_t)__double2loint(t0);
+    const double r = e - (t0 - big);
+    const double sj = tab[128 + (ki & 31u)];
+    const double s = __hiloint2double((int)((uint32_t)__double2hiint(sj) + (uint32_t)(((int)ki >> 5) << 20)), __double2loint(sj));
+    double p = CUMO_HIP_EXP2_E4;
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2_E3);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2_E2);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2_E1);
+    return __builtin_fma(s * r, p, s);
+}
+
 #define CUMO_HIP_OP_COMMON(TA, TB, TR, NIN_, BIT_, CHK_) \
     typedef TA A; typedef TB B; typedef TR R; typedef TA S; \
     static constexpr int NIN = NIN_; static constexpr bool BIT_OUT = BIT_; static constexpr bool CHECKED = CHK_;
@@ -360,7 +419,8 @@ __device__ __forceinline__ double log1p_core(double u) {
     // c / w: c is below 2^-53 w, so the term only counts where u is small, and there 1 / w = 1 - u
     // will do (past u = 2^-10 it is below 2^-43 of the answer, past 1 it is left out)
     const double um = (u < 1.0) ? u : 1.0;
-    return __builtin_fma(c, 1.0 - um, log_core_for_float<0>(w));
+    // the logarithm from the table-driven core (2^-44 relative, next to 1 as well), times ln 2
+    return __builtin_fma(c, 1.0 - um, 6.93147180559945286227e-01 * log2_by_table(w, float_tables()));
 }
 __device__ __forceinline__ float asinh_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);
@@ -598,9 +658,16 @@ CUMO_HIP_TRIG_OP(OpTan, 2, tan((double)x))
 CUMO_HIP_OWN_OP(OpAsin, asin_acos_float_rounded_once<false>, asin((double)x))
 CUMO_HIP_OWN_OP(OpAcos, asin_acos_float_rounded_once<true>, acos((double)x))
 CUMO_HIP_OWN_OP(OpAtan, atan_float_rounded_once, atan((double)x))
-CUMO_HIP_OWN_OP(OpAsinh, asinh_float_rounded_once, asinh((double)x))
-CUMO_HIP_OWN_OP(OpAcosh, acosh_float_rounded_once, acosh((double)x))
-CUMO_HIP_OWN_OP(OpAtanh, atanh_float_rounded_once, atanh((double)x))
+#define CUMO_HIP_OWN_OP_WITH_TABLES(NAME, FEXPR, DEXPR)                                                                     \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
+        static constexpr bool USES_TABLES = sizeof(T) == 4;                                                                 \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const {                                                    \
+            if constexpr (sizeof(T) == 4) z = (T)FEXPR((float)x);                                                           \
+            else z = (T)(DEXPR);                                                                                            \
+            return true; } };
+CUMO_HIP_OWN_OP_WITH_TABLES(OpAsinh, asinh_float_rounded_once, asinh((double)x))
+CUMO_HIP_OWN_OP_WITH_TABLES(OpAcosh, acosh_float_rounded_once, acosh((double)x))
+CUMO_HIP_OWN_OP_WITH_TABLES(OpAtanh, atanh_float_rounded_once, atanh((double)x))
 // the host macro guards x == 0 (types/float_macro.h:113); the reference's device
 // macro does not and answers NaN there, which Numo does not
 __device__ __attribute__((noinline)) float sinc_by_the_library(float xf) { return (float)(sin((double)xf) / (double)xf); }
@@ -636,18 +703,20 @@ struct OpIAbs { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, true)
 // ---- pow, maximum/minimum, clip ----------------------------------------------
 // Float ** float: the host macro's pow in double, rounded once
 // (reference: types/float_macro.h m_pow; device types/float_macro_kernel.h:36).
-// SFloat: for a positive finite base and a finite exponent, exp(y log x) in double with the
-// logarithm good to 2^-50 (|y log x| stays below 110 wherever the float answer is neither 0 nor
-// infinite, so the exponent's error stays below 2^-42) and the exp of the core above; everything
+// SFloat: for a positive finite base and a finite exponent, 2^(y log2 x) in double from the two
+// table-driven cores above: the logarithm is good to 2^-44 relative and |y log2 x| stays below 160
+// wherever the float answer is neither 0 nor infinite, so the exponent is off by less than 2^-36
+// and the result by less than 2^-12 of a float's last place before the one rounding; everything
 // else (zero, negative, infinite or NaN base, infinite or NaN exponent: the sign, domain and
 // limit rules) is the device library's pow.
 // kept out of line: inlined next to every element it would spread the few instructions
 // that run over many times their size of instructions that almost never do
 __device__ __attribute__((noinline)) float pow_by_the_library(float xf, float yf) { return (float)pow((double)xf, (double)yf); }
 __device__ __forceinline__ float pow_fast(float xf, float yf) {
-    double p = (double)yf * log_core_for_float<0, true>((double)xf);
-    p = __builtin_fmin(__builtin_fmax(p, -110.0), 90.0);  // (a NaN only comes from a rare argument)
-    return (float)exp_core_for_float<false>(p);
+    const double* tab = float_tables();
+    double e = (double)yf * log2_by_table((double)xf, tab);
+    e = __builtin_fmin(__builtin_fmax(e, -160.0), 130.0);  // (a NaN only comes from a rare argument)
+    return (float)exp2_by_table(e, tab);
 }
 __device__ __forceinline__ bool pow_is_rare(float xf, float yf) { return !(__float_as_uint(xf) - 1u < 0x7f7fffffu && __builtin_fabsf(yf) < INFINITY); }
 __device__ __forceinline__ float pow_float_rounded_once(float xf, float yf) {
@@ -658,6 +727,7 @@ __device__ __forceinline__ float pow_float_rounded_once(float xf, float yf) {
 }
 template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) static constexpr bool HEAVY = true;
     static constexpr bool HAS_RARE = sizeof(T) == 4;
+    static constexpr bool USES_TABLES = sizeof(T) == 4;
     __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
         if constexpr (sizeof(T) == 4) z = (T)pow_float_rounded_once((float)x, (float)y);
         else z = (T)pow((double)x, (double)y);

@@ -1,0 +1,68 @@
+"""Writes float_tables.inc: the tables and polynomial coefficients of the table-driven
+log2 / exp2 cores in ew_ops.h (SFloat power, asinh, acosh, atanh).
+
+    python cumo_amd/csrc/make_float_tables.py > cumo_amd/csrc/float_tables.inc
+
+log2: the argument's high word minus 0x3fe6a000 gives the binade k (bits 20 and up), the
+interval i (bits 14..19) and, with the binade taken off, a mantissa m in [0.70703125,
+1.4140625). Interval i holds the m whose high word lies in [0x3fe6a000 + i 2^14, + 2^14);
+its entry is {invc, logc} with invc = 1 / (the interval's midpoint) rounded to double and
+logc = -log2(invc) of that rounded value, so that log2 m = logc + log2(1 + z) with
+z = m invc - 1, |z| <= 2^-7. 1.0 is the midpoint of interval 37 (0x3ff00000 - 0x3fe6a000 =
+37.5 * 2^14): its entry is {1, 0} exactly, so arguments next to 1 lose nothing.
+exp2: 2^(j/32), j = 0..31.
+Coefficients are the Taylor ones (the intervals are short enough: the remainders are
+z^6 / 7 relative for log2(1 + z) and (r ln 2)^5 / 120 for 2^r, |r| <= 1/64)."""
+import struct
+
+import mpmath as mp
+
+mp.mp.prec = 200
+OFFH = 0x3FE6A000
+
+
+def dbl(hi, lo=0):
+    return struct.unpack("<d", struct.pack("<Q", (hi << 32) | lo))[0]
+
+
+def to_double(x):
+    return float(mp.nstr(x, 40))  # correctly rounded through the decimal string (40 digits >> 17)
+
+
+def main():
+    rows = []
+    for i in range(64):
+        lo_hi, up_hi = OFFH + (i << 14), OFFH + ((i + 1) << 14)
+
+        def real(h):  # the mantissa value of a high word after the binade is taken off
+            t = h - OFFH
+            return mp.mpf(dbl(h - (t & 0xFFF00000)))  # (t < 2^20 here: nothing is taken off)
+        # interval bounds as reals: a bound in the upper binade is the double with that high word
+        a, b = mp.mpf(dbl(lo_hi)), mp.mpf(dbl(up_hi))
+        c = (a + b) / 2
+        if a < 1 < b:
+            assert i == 37
+            invc, logc = 1.0, 0.0
+        else:
+            invc = to_double(1 / c)
+            logc = to_double(-mp.log(mp.mpf(invc), 2))
+        zmax = max(abs(a * mp.mpf(invc) - 1), abs(b * mp.mpf(invc) - 1))
+        assert zmax <= mp.mpf(2) ** -7 * (1 + mp.mpf(2) ** -20), (i, zmax)
+        rows.append((invc, logc))
+    print("// written by make_float_tables.py; do not edit")
+    print("#define CUMO_HIP_LOG2_TABLE \\")
+    print(", \\\n".join("    %s, %s" % (float.hex(a), float.hex(b)) for a, b in rows))
+    print("#define CUMO_HIP_EXP2_TABLE \\")
+    ex = [to_double(mp.mpf(2) ** (mp.mpf(j) / 32)) for j in range(32)]
+    print(", \\\n".join("    " + ", ".join(float.hex(v) for v in ex[k:k + 4]) for k in range(0, 32, 4)))
+    ln2 = mp.log(2)
+    print("// log2(1 + z) = z (L1 + L2 z + ... + L6 z^5)")
+    for n in range(1, 7):
+        print("#define CUMO_HIP_LOG2_L%d %s" % (n, float.hex(to_double(mp.mpf((-1) ** (n + 1)) / (n * ln2)))))
+    print("// 2^r = 1 + r (E1 + E2 r + E3 r^2 + E4 r^3)")
+    for n in range(1, 5):
+        print("#define CUMO_HIP_EXP2_E%d %s" % (n, float.hex(to_double(ln2 ** n / mp.factorial(n)))))
+
+
+if __name__ == "__main__":
+    main()

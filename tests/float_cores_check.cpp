@@ -6,6 +6,8 @@
 //
 //   float_cores_check vectors <file>   reads "name type n" blocks of arguments (hex bit
 //                                      patterns), prints the results as hex bit patterns
+//   float_cores_check pow <n>          n random (base, exponent) pairs through the SFloat power's arithmetic against
+//                                      (float)glibc pow; prints pairs tried, mismatches and the largest difference in ulps
 //   float_cores_check sweep <stride>   every stride-th float bit pattern through each SFloat
 //                                      core against (float)glibc((double)x); prints, per
 //                                      function, patterns tried, mismatches and the largest
@@ -77,6 +79,41 @@ int main(int argc, char** argv) {
             }
             std::printf("%s %llu %llu %lld\n", c.name, (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
         }
+        return 0;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "pow") == 0) {
+        // n random (base, exponent) pairs: bases over every positive float, exponents spread so that results span the
+        // float range (and beyond), then bases next to 1 with large exponents; against (float)pow((double)x, (double)y)
+        const uint64_t n = std::strtoull(argv[2], nullptr, 10);
+        uint64_t state = 0x9e3779b97f4a7c15ull, tried = 0, bad = 0;
+        int64_t worst = 0;
+        auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+        for (uint64_t it = 0; it < n; ++it) {
+            const uint64_t a = next(), b = next();
+            float x, y;
+            if (it % 3 == 0) {
+                uint32_t u = (uint32_t)(a % 0x7f800000u); if (u == 0) u = 1; std::memcpy(&x, &u, 4);
+                const double lg = std::log2((double)x);
+                const double target = ((double)(b % 2000001) / 1000000.0 - 1.0) * 155.0;   // wanted log2 of the result
+                y = (float)(lg != 0.0 ? target / lg : (double)(b % 1000));
+            } else if (it % 3 == 1) {
+                x = 1.0f + ((float)(int64_t)(a % 4000001) - 2000000.0f) * 1.0e-7f * (float)((a >> 32) % 100 + 1);
+                y = ((float)(int64_t)(b % 2000001) - 1000000.0f) * (float)((b >> 40) % 1000 + 1) * 1.0e-4f;
+            } else {
+                x = (float)(a % 1000003) / 1000.0f + 1.0e-3f;
+                y = ((float)(int64_t)(b % 200001) - 100000.0f) / 5000.0f;
+            }
+            if (pow_is_rare(x, y)) continue;
+            const float got = pow_fast(x, y), want = (float)std::pow((double)x, (double)y);
+            ++tried;
+            uint32_t gu, wu; std::memcpy(&gu, &got, 4); std::memcpy(&wu, &want, 4);
+            if (gu == wu) continue;
+            ++bad;
+            int64_t d = (got != got || want != want) ? (1 << 30) : ordered(got) - ordered(want);
+            if (d < 0) d = -d;
+            if (d > worst) worst = d;
+        }
+        std::printf("pow %llu %llu %lld\n", (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
         return 0;
     }
     if (argc >= 3 && std::strcmp(argv[1], "vectors") == 0) {
