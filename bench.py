@@ -386,11 +386,27 @@ def measure_config(name, cumo, lib, iters, warmup, replay_too=True):
         rot = per_set[:k]
         state = [0]
 
+        # where / a[mask] size their own result: every timed call gets an empty result descriptor, as a caller's
+        # would be, and the result of the set's previous turn is released after it (replaying the recorded call as it
+        # stands would hand the library a result of the right length, which no caller has before the call)
+        sizing = ("cumo_hip_na_where", "cumo_hip_na_mask")
+        owned = [[None] * len(r) for r in rot]
+        first = {}  # (set, call) -> the result the recorded call allocated (the mirror's array owns it)
+
         def rotated(times):
             j = state[0]
             for _ in range(times):
-                for f, a in rot[j]:
-                    f(*a)
+                for c, (f, a) in enumerate(rot[j]):
+                    if f.__name__ in sizing:
+                        z = a[-1]._obj
+                        first.setdefault((j, c), z.ptr)
+                        z.ptr = None
+                        f(*a)
+                        if owned[j][c]:
+                            lib.cumo_cuda_runtime_free(owned[j][c])
+                        owned[j][c] = z.ptr
+                    else:
+                        f(*a)
                 j = j + 1 if j + 1 < k else 0
             state[0] = j
             _lib.check()
@@ -405,6 +421,12 @@ def measure_config(name, cumo, lib, iters, warmup, replay_too=True):
                 rotated(batch)
                 lib.cumo_hip_synchronize()
         ts = sorted(timer.time(lambda: rotated(batch)) / batch for _ in range(iters))
+        for row_owned in owned:
+            for ptr in row_owned:
+                if ptr:
+                    lib.cumo_cuda_runtime_free(ptr)
+        for (j, c), ptr in first.items():
+            rot[j][c][1][-1]._obj.ptr = ptr  # the replay leg below writes into the recorded result again
         del keep
         med, best = ts[len(ts) // 2], ts[0]
         row_replay = {}
