@@ -530,6 +530,70 @@ struct MinMaxImpl {
     }
 };
 
+// Both ends by value alone, for the answers that do not depend on which of two equal elements came
+// first: ptp always (a zero's sign drops out of hi - lo, and a zero spread is +0 by rule), minmax of
+// integers (equal integers are the same answer). One min and one max per element, no index carried
+// through the fold: the index-carrying form above costs a third of the memory rate on large arrays.
+// NaN is skipped unless an output holds nothing else (the rule without `nan: true`).
+// out_mode: 0 = two outputs (minmax), 1 = max - min (ptp).
+template <class T>
+struct MinMaxValueImpl {
+    typedef T In;
+    struct Acc { T lo; T hi; };
+    static constexpr bool USES_INDEX = false;
+    static constexpr int NOUT = 2;
+    int out_mode;
+    // (the library's fmin / fmax: of a number and a NaN the number, a signalling NaN included)
+    static __device__ __forceinline__ float lower(float a, float b) { return __builtin_fminf(a, b); }
+    static __device__ __forceinline__ double lower(double a, double b) { return __builtin_fmin(a, b); }
+    static __device__ __forceinline__ int32_t lower(int32_t a, int32_t b) { return a < b ? a : b; }
+    static __device__ __forceinline__ float upper(float a, float b) { return __builtin_fmaxf(a, b); }
+    static __device__ __forceinline__ double upper(double a, double b) { return __builtin_fmax(a, b); }
+    static __device__ __forceinline__ int32_t upper(int32_t a, int32_t b) { return a > b ? a : b; }
+    __device__ __forceinline__ Acc identity() const {
+        if (is_float_t<T>::value) return Acc{Lim<T>::skip(), Lim<T>::skip()};
+        return Acc{Lim<T>::highest(), Lim<T>::lowest()};
+    }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        acc.lo = lower(acc.lo, next.lo);
+        acc.hi = upper(acc.hi, next.hi);
+    }
+    __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
+        acc.lo = lower(acc.lo, x);
+        acc.hi = upper(acc.hi, x);
+    }
+    template <int N>
+    __device__ __forceinline__ void accumulate_n(const T (&x)[N], int64_t, Acc& acc) const {
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            acc.lo = lower(acc.lo, x[k]);
+            acc.hi = upper(acc.hi, x[k]);
+        }
+    }
+    static constexpr bool GROUPED = true;
+    template <int U, int N>
+    __device__ __forceinline__ void accumulate_group(const T (&x)[U][N], const int64_t (&)[U], Acc& acc) const {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                acc.lo = lower(acc.lo, x[u][k]);
+                acc.hi = upper(acc.hi, x[u][k]);
+            }
+        }
+    }
+    __device__ __forceinline__ void store(const Acc& acc, char* out, char* out2) const {
+        if (out_mode == 0) {
+            *reinterpret_cast<T*>(out) = acc.lo;
+            *reinterpret_cast<T*>(out2) = acc.hi;
+        } else {
+            T d = spread<T>(acc.hi, acc.lo);
+            if (d == (T)0) d = (T)0;  // (+0) - (-0) and the like: +0 (types/real_accum.h:406-441)
+            *reinterpret_cast<T*>(out) = d;
+        }
+    }
+};
+
 }  // namespace cumo_hip
 
 #endif
