@@ -326,6 +326,8 @@ struct ArgImpl {
         if (better || (acc.value == next.value && next.index < acc.index)) acc = next;
     }
     __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{x, (IDX)idx}, acc); }
+    // (an accumulator of the value-only form this is the exact rule of: a plain value, folded as an element at position idx)
+    __device__ __forceinline__ void accumulate_acc(T part, int64_t idx, Acc& acc) const { accumulate(part, idx, acc); }
     // N later elements at once. The block's extreme costs one max/min per element;
     // only a block that beats the accumulator is looked at again, to find where its
     // extreme first occurs, and then merged with one combine. An equal value never
@@ -494,6 +496,11 @@ struct MinMaxImpl {
         acc.hi = One{h.value, h.index};
     }
     __device__ __forceinline__ void accumulate(T x, int64_t idx, Acc& acc) const { combine(Acc{One{x, idx}, One{x, idx}}, acc); }
+    // (an accumulator {lo, hi} of the value-only form this is the exact rule of, folded as one element per end at position idx)
+    template <class P>
+    __device__ __forceinline__ void accumulate_acc(const P& part, int64_t idx, Acc& acc) const {
+        combine(Acc{One{part.lo, idx}, One{part.hi, idx}}, acc);
+    }
     template <int N>
     __device__ __forceinline__ void accumulate_n(const T (&x)[N], int64_t idx0, Acc& acc) const {
         // each end runs its own block rule
@@ -536,13 +543,20 @@ struct MinMaxImpl {
 // through the fold: the index-carrying form above costs a third of the memory rate on large arrays.
 // NaN is skipped unless an output holds nothing else (the rule without `nan: true`).
 // out_mode: 0 = two outputs (minmax), 1 = max - min (ptp).
-template <class T>
+template <class T, bool EXACT_ZEROS = false>
 struct MinMaxValueImpl {
     typedef T In;
     struct Acc { T lo; T hi; };
     static constexpr bool USES_INDEX = false;
     static constexpr int NOUT = 2;
+    // EXACT_ZEROS (float minmax): an end that comes out as a zero may be +0 or -0 depending on which came first;
+    // the kernels that know this protocol then go over the output again with the index-carrying rule
+    typedef MinMaxImpl<T, false> Exact;
+    static constexpr bool HAS_EXACT = EXACT_ZEROS && is_float_t<T>::value;
     int out_mode;
+    __device__ __forceinline__ bool needs_exact(const Acc& acc) const { return acc.lo == (T)0 || acc.hi == (T)0; }
+    __host__ __device__ __forceinline__ Exact exact() const { return Exact{out_mode}; }
+    __device__ __forceinline__ Acc from_exact(const typename Exact::Acc& e) const { return Acc{e.lo.value, e.hi.value}; }
     // (the library's fmin / fmax: of a number and a NaN the number, a signalling NaN included)
     static __device__ __forceinline__ float lower(float a, float b) { return __builtin_fminf(a, b); }
     static __device__ __forceinline__ double lower(double a, double b) { return __builtin_fmin(a, b); }

@@ -921,6 +921,19 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
     return true;
 }
 
+// A form that only the lean kernels run (an accumulator their exact protocol knows and the general kernels' does
+// not) where they take the reduction, the other form through everything else.
+template <class Fast, class Slow>
+static bool reduce_launch_lean_or(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Fast fast, Slow slow, int slow_index_mode) {
+    if (arg->out_indexer.total_size == 0) return true;
+    ReducePlan plan;
+    plan_reduce(arg, out2, (int)sizeof(typename Fast::In), (int)sizeof(typename Fast::Acc), &plan, true);
+    if (plan.kind == RED_EMPTY) return true;
+    const int taken = red_stream_launch(plan, arg, out2, fast, 0, nullptr, current_stream());
+    if (taken != 0) return taken > 0;
+    return reduce_launch(arg, out2, slow, slow_index_mode);
+}
+
 }  // namespace cumo_hip
 
 #endif

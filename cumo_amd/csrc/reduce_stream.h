@@ -297,10 +297,9 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
     const int64_t o_a = (int64_t)o0 * p.out_step[0] + (int64_t)o1 * p.out_step[1];
     const int64_t o_b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)o1 * p.out2_step[1] : 0;
     if constexpr (has_exact<Impl>::value) {
-        // the accumulators are plain values in axis order: the fast fold first, and only where
+        // the accumulators are values in axis order: the fast fold first, and only where
         // it cannot decide (which of two equal values came first) the exact rule over the same values
         typedef typename Impl::Exact Exact;
-        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
         Acc total = impl.identity();
         for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), total);
         rs_group_combine(impl, total, 8, wave_slots);
@@ -310,11 +309,11 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_split_kernel(RedSParams p,
             const Exact ex = impl.exact();
             __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
             typename Exact::Acc e = ex.identity();
-            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), (int64_t)k, e);
+            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate_acc(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), (int64_t)k, e);
             rs_group_combine(ex, e, 8, exact_slots);
             total = impl.from_exact(e);
         }
-        if (threadIdx.x == 0) impl.store(total, p.out + o_a, nullptr);
+        if (threadIdx.x == 0) impl.store(total, p.out + o_a, (Impl::NOUT > 1) ? (p.out2 + o_b) : nullptr);
     } else {
         Acc total = impl.identity();
         for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_fetch<Acc>(mine + (size_t)k * sizeof(Acc)), total);
@@ -384,7 +383,7 @@ __global__ __launch_bounds__(kRedBlock) void red_fold_parts_kernel(RedSParams p,
         for (int j = 0; j < VEC; ++j) {
             if (impl.needs_exact(total[j])) {
                 typename Exact::Acc e = ex.identity();
-                for (uint32_t k = 0; k < p.n_split; ++k) ex.accumulate(base[(size_t)k * row + j], (int64_t)k, e);
+                for (uint32_t k = 0; k < p.n_split; ++k) ex.accumulate_acc(base[(size_t)k * row + j], (int64_t)k, e);
                 total[j] = impl.from_exact(e);
             }
         }
@@ -527,7 +526,6 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
     const int64_t o_b = (Impl::NOUT > 1) ? (int64_t)o0 * p.out2_step[0] + (int64_t)o1 * p.out2_step[1] : 0;
     if constexpr (has_exact<Impl>::value) {
         typedef typename Impl::Exact Exact;
-        static_assert(sizeof(Acc) == sizeof(In), "an impl with an exact fallback keeps a plain value");
         Acc total = impl.identity();
         for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), total);
         rs_group_combine(impl, total, 8, wave_slots);
@@ -537,11 +535,11 @@ __global__ __launch_bounds__(kRedBlock) void red_srow_poll_kernel(RedSParams p, 
             const Exact ex = impl.exact();
             __shared__ typename Exact::Acc exact_slots[kRedBlock / 64];
             typename Exact::Acc e = ex.identity();
-            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), (int64_t)k, e);
+            for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) ex.accumulate_acc(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), (int64_t)k, e);
             rs_group_combine(ex, e, 8, exact_slots);
             total = impl.from_exact(e);
         }
-        if (threadIdx.x == 0) impl.store(total, p.out + o_a, nullptr);
+        if (threadIdx.x == 0) impl.store(total, p.out + o_a, (Impl::NOUT > 1) ? (p.out2 + o_b) : nullptr);
     } else {
         Acc total = impl.identity();
         for (uint32_t k = threadIdx.x; k < p.n_split; k += kRedBlock) impl.combine(rs_await<Acc>(mine + (size_t)k * W, launch, p.wait), total);
@@ -662,7 +660,7 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
                         typedef typename Impl::Exact Exact;
                         const Exact ex = impl.exact();
                         typename Exact::Acc e = ex.identity();
-                        for (unsigned k = 0; k < SB; ++k) ex.accumulate(part[k * CPB + c][j], (int64_t)k, e);
+                        for (unsigned k = 0; k < SB; ++k) ex.accumulate_acc(part[k * CPB + c][j], (int64_t)k, e);
                         acc[j] = impl.from_exact(e);
                     } else {
                         for (unsigned k = 1; k < SB; ++k) impl.combine(part[k * CPB + c][j], acc[j]);

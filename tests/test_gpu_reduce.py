@@ -214,7 +214,8 @@ def test_dfloat_kahan_sum():
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((300, 77), 1), ((300, 77), 0), ((5, 20000), 1), ((20000, 5), 0), ((3000001,), None),
-                                        ((64, 33, 40), (0, 2)), ((6, 70000), 1), ((2, 3, 4096), 2)])
+                                        ((64, 33, 40), (0, 2)), ((6, 70000), 1), ((2, 3, 4096), 2), ((3000, 1000), 0), ((70000, 64), 0),
+                                        ((8192, 260), 0)])
 def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
     # Numo's sequential loop only replaces on a strict comparison (real_accum.h:217-278), so of
     # +0 and -0 the earlier one is the answer. Every output here ends on a zero, with both signs
@@ -235,6 +236,21 @@ def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
         if want.size >= 100:
             zeros = want[want == 0]
             assert np.signbit(zeros).any() and not np.signbit(zeros).all(), "the inputs are meant to produce both signs"
+        # minmax answers the same zero at that end, and the other end as min / max alone do
+        if not isinstance(axis, tuple):
+            lo, hi = (np.asarray(v.to_numpy() if hasattr(v, "to_numpy") else v, dtype=dt) for v in d.minmax(axis=axis))
+            assert_bits_equal(lo, np.asarray(oracle.reduce("min", h, axis=axis), dtype=dt), "minmax lo %r axis %r" % (shape, axis))
+            assert_bits_equal(hi, np.asarray(oracle.reduce("max", h, axis=axis), dtype=dt), "minmax hi %r axis %r" % (shape, axis))
+    # both ends zero: every element a zero of either sign
+    hz = np.where(sign, dt(-0.0), dt(0.0)).astype(dt)
+    dz = cls.cast(hz)
+    if not isinstance(axis, tuple):
+        lo, hi = (np.asarray(v.to_numpy() if hasattr(v, "to_numpy") else v, dtype=dt) for v in dz.minmax(axis=axis))
+        assert_bits_equal(lo, np.asarray(oracle.reduce("min", hz, axis=axis), dtype=dt), "minmax of zeros, lo")
+        assert_bits_equal(hi, np.asarray(oracle.reduce("max", hz, axis=axis), dtype=dt), "minmax of zeros, hi")
+        spread = dz.ptp(axis=axis)
+        spread = np.asarray(spread.to_numpy() if hasattr(spread, "to_numpy") else spread, dtype=dt)
+        assert (spread == 0).all() and not np.signbit(spread).any()
     # NaN in the mix: skipped unless the output holds nothing else
     h = (mag * dt(-1.0)).astype(dt)
     h[zero] = np.nan
