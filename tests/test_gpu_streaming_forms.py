@@ -10,7 +10,10 @@ run on the ordinary suites' small inputs in child processes:
   CUMO_HIP_SCAN_COLS_CHAIN=0  long runs across memory scanned in two passes over segments;
   CUMO_HIP_SCAN_KEEP_WORDS=0  the one-pass scans with their words from the pool, cleared by a kernel
                            before each launch (what a stream under capture gets);
-  CUMO_HIP_EW_LEAN_ROWS=0  (with CUMO_HIP_NT=1) the general row kernel in its non-temporal forms.
+  CUMO_HIP_EW_LEAN_ROWS=0  (with CUMO_HIP_NT=1) the general row kernel in its non-temporal forms;
+  CUMO_HIP_BIT_VEC_GRID=1  (with CUMO_HIP_NT=1) the Bit vector kernels with one block per compute unit, whose lanes
+                           then loop over the result's vectors (what an array beyond 2^37 bits gets) and carry a
+                           vector's row and column from turn to turn.
 Each child runs the same parity tests against the oracle as the main suite does."""
 import os
 import subprocess
@@ -74,3 +77,10 @@ def test_one_pass_scans_with_cleared_words_from_the_pool():
 
 def test_one_long_run_by_blocks_of_four_waves():
     run_child({"CUMO_HIP_SCAN_CHAIN_WAVES": "4"}, ["tests/test_gpu_adjacent.py::test_one_long_run_in_one_pass"])
+
+
+def test_bit_vector_kernels_with_lanes_that_loop():
+    run_child({"CUMO_HIP_BIT_VEC_GRID": "1", "CUMO_HIP_NT": "1"},
+              ["tests/test_gpu_bit.py::test_rows_of_bits_in_views_word_by_word", "tests/test_gpu_bit.py::test_long_runs_of_bits_by_whole_vectors",
+               "tests/test_gpu_bit.py::test_windows_of_a_large_matrix_into_a_fresh_result", "tests/test_gpu_bit.py::test_long_arrays_and_views",
+               "tests/test_gpu_bit.py::test_all_any_along_word_aligned_rows"])
