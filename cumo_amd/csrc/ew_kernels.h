@@ -168,6 +168,12 @@ __device__ __forceinline__ void ew_load(const char* base, int64_t istep, int64_t
         T v = *reinterpret_cast<const T*>(base);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = v;
+    } else if (VEC > 1 && istep < 0) {
+        // the row runs backwards in memory: the vector that ends at this column's element, turned round
+        T rev[VEC];
+        raw_load<T, VEC, NT>(base - (col + (VEC - 1)) * (int64_t)sizeof(T), rev);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = rev[VEC - 1 - j];
     } else if (VEC > 1) {
         const char* p = base + col * (int64_t)sizeof(T);
         raw_load<T, VEC, NT>(p, out);
@@ -843,7 +849,7 @@ struct EwR2Params {
     int64_t rstep[3];    // byte step from one row to the next (0: the operand repeats)
     int64_t ostep[3];    // three dimensions: byte step along outer (rstep is then the step along mid)
     uint32_t mid;        // three dimensions: extent of mid; 0 for two dimensions
-    int walk[3];         // 1: contiguous along inner, 0: constant along inner
+    int walk[3];         // 1: contiguous along inner, 0: constant along inner, 2 (inputs): contiguous, backwards in memory
     uint32_t rows;
     uint32_t inner_vecs; // inner / VEC
     uint32_t col_tiles;
@@ -893,8 +899,13 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
         R zv[VEC];
         if (NIN >= 1) {
             const char* a = p.ptr[0] + roff[0];
-            if (p.walk[0]) {
+            if (p.walk[0] == 1) {
                 raw_load<A, VEC, (NTM & 1) != 0>(a + (uint64_t)cv * (VEC * sizeof(A)), xv);
+            } else if (p.walk[0] == 2) {
+                A rev[VEC];
+                raw_load<A, VEC, (NTM & 1) != 0>(a - ((int64_t)cv * VEC + (VEC - 1)) * (int64_t)sizeof(A), rev);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) xv[j] = rev[VEC - 1 - j];
             } else {
                 const A v = *reinterpret_cast<const A*>(a);
 #pragma unroll
@@ -903,8 +914,13 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows2_kernel(EwR2Params p, Op op,
         }
         if (two_arrays) {
             const char* a = p.ptr[1] + roff[1];
-            if (p.walk[1]) {
+            if (p.walk[1] == 1) {
                 raw_load<B, VEC, (NTM & 2) != 0>(a + (uint64_t)cv * (VEC * sizeof(B)), yv);
+            } else if (p.walk[1] == 2) {
+                B rev[VEC];
+                raw_load<B, VEC, (NTM & 2) != 0>(a - ((int64_t)cv * VEC + (VEC - 1)) * (int64_t)sizeof(B), rev);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) yv[j] = rev[VEC - 1 - j];
             } else {
                 const B v = *reinterpret_cast<const B*>(a);
 #pragma unroll
@@ -1883,6 +1899,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             const int64_t is = plan.step[o][n - 1];
             if (is == es) rp.walk[sl] = 1;
             else if (is == 0 && sl != 2) rp.walk[sl] = 0;
+            else if (is == -es && sl != 2 && es >= 4) rp.walk[sl] = 2;
             else r2 = false;
             rp.ptr[sl] = const_cast<char*>(ops[o].ptr);
             rp.rstep[sl] = plan.step[o][n - 2];
@@ -1925,7 +1942,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     } while (0);
                 // large two-dimensional arrays of a cheap function: the lean form, two rows per lane
                 const uint64_t lean_tiles = ctiles * ((kp.rows + 2 * ty - 1) / (2 * ty));
-                if constexpr (!heavy) if (n == 2 && nt && Op::NIN >= 1 && rp.walk[0] && lean_tiles <= ew_grid_max() && ew_lean_rows_enabled()) {
+                if constexpr (!heavy) if (n == 2 && nt && Op::NIN >= 1 && rp.walk[0] == 1 && rp.walk[1] != 2 && lean_tiles <= ew_grid_max() && ew_lean_rows_enabled()) {
                     EwR2LeanParams lp;
                     std::memset(&lp, 0, sizeof(lp));
                     for (int k = 0; k < 3; ++k) { lp.ptr[k] = rp.ptr[k]; lp.rstep[k] = rp.rstep[k]; }

@@ -146,10 +146,13 @@ void plan_elementwise(int ndim, const size_t* shape, int nops, const EwOperand* 
                 continue;
             }
             if (st[o][L] == 0) { if (o == out) ok = false; continue; }
-            if (st[o][L] != es) { ok = false; break; }
+            // an input that runs backwards along the rows is read by vectors too (the row kernel turns a vector's
+            // elements round); its vectors start wherever the view's last element puts them: element alignment
+            const bool backwards = o != out && es >= 4 && st[o][L] == -(int64_t)es && !loose;
+            if (st[o][L] != es && !backwards) { ok = false; break; }
             int align = vec * es;
             if (align > 16) align = 16;
-            if (loose && o != out && es >= 4) align = es;
+            if ((loose && o != out && es >= 4) || backwards) align = es;
             if (((uintptr_t)ops[o].ptr % align) != 0) { ok = false; break; }
             for (int d = 0; d < L; ++d) if (st[o][d] % align) { ok = false; break; }
         }

@@ -212,6 +212,39 @@ def test_three_dimensions_with_an_operand_repeating_along_one(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_rows_that_run_backwards_in_memory(tname, dt):
+    """An input whose rows are reversed (x[true, (-1..0)], fliplr) is read by 128-bit vectors from the vector that ends
+    at the lane's column, its elements turned round: one operand or both, against forward operands, a row vector, a
+    scalar on either side, three dimensions, rows that are not a whole number of vectors (the general row kernel),
+    windows that start inside a vector, a comparison into Bit."""
+    rng = np.random.default_rng(104)
+    cls = cls_of(tname)
+    def rnd(*shape):
+        return (rng.integers(-50, 50, size=shape) if dt == np.int32 else rng.standard_normal(shape)).astype(dt)
+    for shape in [(70, 256), (33, 1000), (9, 520), (40, 1001), (5, 7, 64), (3, 20, 131)]:
+        a, b = rnd(*shape), rnd(*shape)
+        da, db = cls.cast(a), cls.cast(b)
+        r = rnd(*((1,) * (len(shape) - 1) + (shape[-1],)))
+        dr = cls.cast(r)
+        rev = (Ellipsis, slice(None, None, -1))
+        both = (slice(None, None, -1),) + (slice(None),) * (len(shape) - 2) + (slice(None, None, -1),)
+        win = (Ellipsis, slice(shape[-1] - 3, 1, -1))
+        with np.errstate(all="ignore"):
+            assert_bits_equal((da[rev] + db).to_numpy(), oracle.binary("add", np.ascontiguousarray(a[rev]), b), "rev + fwd %r" % (shape,))
+            assert_bits_equal((da - db[rev]).to_numpy(), oracle.binary("sub", a, np.ascontiguousarray(b[rev])), "fwd - rev %r" % (shape,))
+            assert_bits_equal((da[rev] * db[rev]).to_numpy(), oracle.binary("mul", np.ascontiguousarray(a[rev]), np.ascontiguousarray(b[rev])), "rev * rev")
+            assert_bits_equal((da[both] - db[rev]).to_numpy(), oracle.binary("sub", np.ascontiguousarray(a[both]), np.ascontiguousarray(b[rev])), "both - rev")
+            assert_bits_equal((da[rev] + dr).to_numpy(), oracle.binary("add", np.ascontiguousarray(a[rev]), r), "rev + row vector")
+            assert_bits_equal((da + dr[rev]).to_numpy(), oracle.binary("add", a, np.ascontiguousarray(r[rev])), "fwd + reversed row vector")
+            assert_bits_equal((da[rev] + 3).to_numpy(), oracle.binary("add", np.ascontiguousarray(a[rev]), np.asarray(3, dtype=dt)), "rev + scalar")
+            assert_bits_equal((7 - da[rev]).to_numpy(), oracle.binary("sub", np.asarray(7, dtype=dt), np.ascontiguousarray(a[rev])), "scalar - rev")
+            assert_bits_equal((da[win] * db[win]).to_numpy(), oracle.binary("mul", np.ascontiguousarray(a[win]), np.ascontiguousarray(b[win])), "windows")
+            assert_bits_equal(da[rev].copy().to_numpy(), np.ascontiguousarray(a[rev]), "copy of rev")
+            assert ((da[rev] > db).to_numpy() == (a[rev] > b)).all(), "rev > fwd into Bit %r" % (shape,)
+            assert (da[rev].gt(db[both]).to_numpy() == (a[rev] > b[both])).all() if hasattr(da, "gt") else True
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
 def test_inputs_that_start_off_a_16_byte_boundary(tname, dt):
     """Slices that begin at an odd column (rows and flat runs whose length is still a whole number of
     128-bit accesses): the lean kernels read them with 128-bit loads on 4- or 8-byte boundaries."""

@@ -28,6 +28,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ELEMENTWISE = ["tests/test_gpu_elementwise.py::test_float_binary_over_views", "tests/test_gpu_elementwise.py::test_broadcast_shapes",
                "tests/test_gpu_elementwise.py::test_three_dimensions_with_an_operand_repeating_along_one",
                "tests/test_gpu_elementwise.py::test_inputs_that_start_off_a_16_byte_boundary",
+               "tests/test_gpu_elementwise.py::test_rows_that_run_backwards_in_memory",
                "tests/test_gpu_elementwise.py::test_many_dims_and_permuted_views", "tests/test_gpu_elementwise.py::test_sizes_and_tails",
                "tests/test_gpu_elementwise.py::test_unary_and_rounding", "tests/test_gpu_elementwise.py::test_int32_arithmetic",
                "tests/test_gpu_elementwise.py::test_int32_error_flags", "tests/test_gpu_elementwise.py::test_casts_and_copies",
