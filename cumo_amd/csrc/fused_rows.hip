@@ -9,9 +9,11 @@
 // launches); here a row is read once into registers, reduced across the lanes that
 // share it with wave64 shuffles (and four LDS slots when a block shares it), and the
 // result written once: 2 x the array. Every elementwise step is the same single
-// IEEE operation the separate launches perform (float subtraction, the exp and sqrt
-// that are the double-precision functions rounded once, float division), so results
-// differ from the chain only through the order of the two row sums.
+// IEEE operation the separate launches perform (float subtraction, the sqrt that is
+// the double-precision function rounded once, float division); the SFloat softmax's
+// exponential is the double-precision 2^(x log2 e) of the table-driven core rounded
+// once, which differs from NMath.exp's float in the last place at about one argument
+// in 10^4. Results differ from the chain through that and the order of the two row sums.
 //
 // The reference has no such entry point; the host layer (cumo_hip_na_softmax /
 // cumo_hip_na_layernorm) uses these for contiguous rows of up to 16384 elements and
@@ -63,7 +65,15 @@ __device__ __forceinline__ T fr_allreduce(T v, F f) {
 }
 
 template <class T> __device__ __forceinline__ T fr_exp(T x);
-template <> __device__ __forceinline__ float fr_exp<float>(float x) { return exp_float_rounded_once(x); }
+// SFloat: 2^(x log2 e) from the table-driven core of ew_ops.h (2^-39 relative before the rounding to float; the
+// element operator's polynomial form is good to 2^-50, which a softmax, divided by a sum of 2^-24 terms, cannot
+// show): eight double operations fewer an element in a kernel that the exponential's arithmetic bounds.
+// A NaN passes through the arithmetic; the clamp keeps the exponent in the core's range.
+template <> __device__ __forceinline__ float fr_exp<float>(float x) {
+    float xc = (x < -105.0f) ? -105.0f : x;
+    xc = (xc > 89.0f) ? 89.0f : xc;
+    return (float)exp2_by_table(1.44269504088896338700e+00 * (double)xc, float_tables());
+}
 template <> __device__ __forceinline__ double fr_exp<double>(double x) { return exp(x); }
 template <class T> __device__ __forceinline__ T fr_sqrt(T x) { return (T)sqrt((double)x); }
 
@@ -113,6 +123,7 @@ __global__ __launch_bounds__(kFrBlock) void fused_rows_kernel(FusedRowsParams p)
     const unsigned lane_r = threadIdx.x % TPR;
     const unsigned row_in_block = threadIdx.x / TPR;
     const uint64_t n_row_blocks = (p.rows + RPB - 1) / RPB;
+    if constexpr (MODE == 0 && sizeof(T) == 4) float_tables_prepare();  // (the SFloat softmax reads the 2^x table)
     for (uint64_t rb = blockIdx.x; rb < n_row_blocks; rb += gridDim.x) {
         const uint64_t row = rb * RPB + row_in_block;
         const bool row_ok = row < p.rows;
