@@ -1550,6 +1550,53 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
     typedef typename Op::A A;
     typedef typename Op::B B;
     typedef typename Op::R R;
+    // A Bit result from an input that walks another dimension fastest than the result does (a comparison of a
+    // transposed view): the tile-transposing kernels write typed results only, and lanes along the result's bits would
+    // read such an input one element per cache line. The input is first copied into the result's order (the typed
+    // store, which transposes through LDS), then compared from there: [8192,4096] SFloat x.transpose > 0, 370 -> 75 us.
+    if constexpr (Op::BIT_OUT && Op::NIN >= 1 && (sizeof(A) == 4 || sizeof(A) == 8)) {
+        const cumo_na_iarray_t* ins[2] = {in1, (Op::NIN >= 2 && use_scalar == 0 && sizeof(B) == sizeof(A)) ? in2 : nullptr};
+        const int nd = indexer->ndim;
+        int F = -1;
+        for (int d = 0; d < nd; ++d)
+            if (indexer->shape[d] >= 16 && out_bit->step[d] == 1) F = d;
+        bool stage[2] = {false, false};
+        if (F >= 0 && indexer->total_size >= 65536 && nd <= CUMO_NA_MAX_DIMENSION) {
+            for (int k = 0; k < 2; ++k) {
+                if (!ins[k]) continue;
+                const int64_t sf = (int64_t)ins[k]->step[F];
+                if (sf == 0 || sf == (int64_t)sizeof(A) || sf == -(int64_t)sizeof(A)) continue;
+                for (int d = 0; d < nd; ++d) {
+                    const int64_t sd = (int64_t)ins[k]->step[d];
+                    if (d != F && indexer->shape[d] >= 16 && (sd == (int64_t)sizeof(A) || sd == -(int64_t)sizeof(A))) stage[k] = true;
+                }
+            }
+        }
+        if (stage[0] || stage[1]) {
+            cumo_na_iarray_t tmp[2];
+            char* held[2] = {nullptr, nullptr};
+            bool ok = true;
+            for (int k = 0; k < 2 && ok; ++k) {
+                if (!stage[k]) continue;
+                held[k] = cumo_cuda_runtime_malloc(indexer->total_size * sizeof(A));
+                if (!held[k]) { ok = false; break; }   // (the pool has reported it)
+                tmp[k].ptr = held[k];
+                ssize_t s = (ssize_t)sizeof(A);
+                for (int d = nd - 1; d >= 0; --d) {
+                    tmp[k].step[d] = s;
+                    s *= (ssize_t)indexer->shape[d];
+                }
+                cumo_na_indexer_t ix = *indexer;
+                if (sizeof(A) == 4) cumo_iter_int32_store_int32_kernel_launch(&tmp[k], const_cast<cumo_na_iarray_t*>(ins[k]), &ix);
+                else cumo_iter_dfloat_store_dfloat_kernel_launch(&tmp[k], const_cast<cumo_na_iarray_t*>(ins[k]), &ix);
+            }
+            if (ok)
+                ew_launch<Op, HEAVY_CALL>(op, stage[0] ? &tmp[0] : in1, stage[1] ? &tmp[1] : in2, out, out_bit, indexer, sv, use_scalar, flag);
+            for (int k = 0; k < 2; ++k)
+                if (held[k]) cumo_cuda_runtime_free(held[k]);
+            return;
+        }
+    }
     EwOperand ops[3];
     int slot[3];
     int nops = 0;

@@ -497,6 +497,30 @@ def test_compare_into_bit(tname, dt, op):
             assert (getattr(dx, op)(wide[:, ::2]).to_numpy() == oracle.compare(op, hx, hy)).all(), (shape, op, "view")
 
 
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_compare_of_transposed_views_into_bit(tname, dt):
+    """A comparison whose input walks another dimension fastest than the result's bits do is copied into the result's
+    order first (from 65536 elements on): one or both operands transposed, against a scalar, a row that repeats, three
+    dimensions permuted two ways, a NaN among the values."""
+    rng = np.random.default_rng(111)
+    cls = cls_of(tname)
+    hx = rng.integers(-3, 4, size=(300, 420)).astype(dt)
+    hy = rng.integers(-3, 4, size=(420, 300)).astype(dt)
+    if dt != np.int32:
+        hx[5, 7] = np.nan
+    dx, dy = cls.cast(hx), cls.cast(hy)
+    for op in ("gt", "eq", "le"):
+        assert (getattr(dx.transpose(), op)(dy).to_numpy() == oracle.compare(op, hx.T, hy)).all(), op
+        assert (getattr(dy, op)(dx.transpose()).to_numpy() == oracle.compare(op, hy, hx.T)).all(), op
+        assert (getattr(dx.transpose(), op)(0).to_numpy() == oracle.compare(op, hx.T, 0)).all(), op
+        assert (getattr(dx.transpose(), op)(dy[0]).to_numpy() == oracle.compare(op, hx.T, hy[0])).all(), op
+        assert (getattr(dx.transpose()[::2, 1:], op)(dy[::2, 1:]).to_numpy() == oracle.compare(op, hx.T[::2, 1:], hy[::2, 1:])).all(), op
+    ht = rng.integers(-3, 4, size=(20, 70, 64)).astype(dt)
+    dtn = cls.cast(ht)
+    for perm in ((0, 2, 1), (2, 1, 0), (1, 2, 0)):
+        assert (dtn.transpose(*perm).gt(1).to_numpy() == oracle.compare("gt", ht.transpose(perm), 1)).all(), perm
+
+
 @pytest.mark.parametrize("tname,dt", FLOATS)
 def test_float_classification(tname, dt):
     cls = cls_of(tname)
