@@ -96,6 +96,47 @@ def test_float_reductions_every_axis(tname, dt, view):
     assert_bits_equal(dv.min_index().to_numpy(), oracle.reduce("min_index", np.ascontiguousarray(hv)))
 
 
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_reductions_along_an_axis_that_strides_through_memory(tname, dt):
+    """Full and partial reductions of transposed and permuted views of 65536 elements or more, where the reduce
+    axis' lanes would stride through memory: the view is copied into its own order first. Ties, both zeros and
+    positions answer in the view's order."""
+    rng = np.random.default_rng(207)
+    cls = cls_of(tname)
+    if dt == np.int32:
+        h2 = rng.integers(-50, 50, size=(300, 260)).astype(dt)
+        h3 = rng.integers(-50, 50, size=(40, 50, 64)).astype(dt)
+    else:
+        h2 = (rng.integers(-8, 8, size=(300, 260)) / 4.0).astype(dt)
+        h3 = (rng.integers(-8, 8, size=(40, 50, 64)) / 4.0).astype(dt)
+        h2[h2 == 0] = np.where(rng.random(int((h2 == 0).sum())) < 0.5, dt(-0.0), dt(0.0))
+        h2 = np.minimum(h2, dt(0.0))       # the maximum is a zero: which one depends on the view's order
+    d2, d3 = cls.cast(h2), cls.cast(h3)
+    cases = [(d2.transpose(), h2.T, None), (d2.transpose(), h2.T, 1), (d2.transpose()[::2, 3:], h2.T[::2, 3:], None),
+             (d3.transpose(2, 1, 0), h3.transpose(2, 1, 0), None), (d3.transpose(2, 1, 0), h3.transpose(2, 1, 0), (1, 2)),
+             (d3.transpose(1, 2, 0), h3.transpose(1, 2, 0), (0, 2)), (d3.transpose(0, 2, 1), h3.transpose(0, 2, 1), 2)]
+    for dv, hv, axis in cases:
+        hv = np.ascontiguousarray(hv)
+        what = "%r axis %r" % (hv.shape, axis)
+        for name in ("min", "max", "sum", "argmin", "argmax", "ptp"):
+            got = getattr(dv, name)(axis=axis)
+            got = np.asarray(got.to_numpy() if hasattr(got, "to_numpy") else got)
+            want = np.asarray(oracle.reduce(name, hv, axis=axis))
+            assert_bits_equal(got.astype(want.dtype), want, "%s %s" % (name, what))
+        lo, hi = (np.asarray(v.to_numpy() if hasattr(v, "to_numpy") else v, dtype=dt) for v in dv.minmax(axis=axis))
+        assert_bits_equal(lo, np.asarray(oracle.reduce("min", hv, axis=axis), dtype=dt), "minmax lo " + what)
+        assert_bits_equal(hi, np.asarray(oracle.reduce("max", hv, axis=axis), dtype=dt), "minmax hi " + what)
+        if dt != np.int32:
+            n = red_n(hv.shape, axis)
+            want = oracle.reduce("var", hv, axis=axis)
+            got = dv.var(axis=axis)
+            got = np.asarray(got.to_numpy() if hasattr(got, "to_numpy") else got)
+            assert_reduction_close(got, want, n, np.abs(want) + 1e-30, "var " + what)
+        got = dv.max_index(axis=axis)
+        got = np.asarray(got.to_numpy() if hasattr(got, "to_numpy") else got)
+        assert_bits_equal(got, np.asarray(oracle.reduce("max_index", hv, axis=axis)).astype(got.dtype), "max_index " + what)
+
+
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((1000003,), None), ((7, 100000), 1), ((100000, 7), 0), ((3, 40000, 5), 1),
                                         ((64, 64, 64), (0, 2)), ((2, 3), None), ((1,), None), ((70000, 3), 1),
