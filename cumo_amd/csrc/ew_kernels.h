@@ -42,9 +42,12 @@ namespace cumo_hip {
 // An operator that reads the LDS tables of ew_ops.h declares USES_TABLES; every kernel here fills them first.
 template <class O, class = void> struct op_uses_tables { static constexpr bool value = false; };
 template <class O> struct op_uses_tables<O, decltype((void)O::USES_TABLES)> { static constexpr bool value = O::USES_TABLES; };
+template <class O, class = void> struct op_uses_pair_table { static constexpr bool value = false; };
+template <class O> struct op_uses_pair_table<O, decltype((void)O::USES_PAIR_TABLE)> { static constexpr bool value = O::USES_PAIR_TABLE; };
 template <class Op>
 __device__ __forceinline__ void ew_op_prepare() {
     if constexpr (op_uses_tables<Op>::value) float_tables_prepare();
+    if constexpr (op_uses_pair_table<Op>::value) exp_pair_table_prepare();
 }
 
 constexpr int kEwBlock = 256;

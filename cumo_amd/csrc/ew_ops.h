@@ -114,6 +114,8 @@ __device__ __forceinline__ double exp2_by_table(double e, const double* tab) {
     return __builtin_fma(s * r, p, s);
 }
 
+#include "dd_cores.h"
+
 #define CUMO_HIP_OP_COMMON(TA, TB, TR, NIN_, BIT_, CHK_) \
     typedef TA A; typedef TB B; typedef TR R; typedef TA S; \
     static constexpr int NIN = NIN_; static constexpr bool BIT_OUT = BIT_; static constexpr bool CHECKED = CHK_;
@@ -626,9 +628,17 @@ __device__ __forceinline__ float erfc_float_rounded_once(float xf) {
             if constexpr (sizeof(T) == 4) z = (T)FEXPR((float)x);                                                           \
             else z = (T)(DEXPR);                                                                                            \
             return true; } };
-CUMO_HIP_OWN_OP(OpTanh, tanh_float_rounded_once, tanh((double)x))
-CUMO_HIP_OWN_OP(OpSinh, sinh_float_rounded_once, sinh((double)x))
-CUMO_HIP_OWN_OP(OpCosh, cosh_float_rounded_once, cosh((double)x))
+// (DFloat: the cores of dd_cores.h, which read the table of 2^(j/32) as pairs)
+#define CUMO_HIP_OWN_OP_WITH_PAIR_TABLE(NAME, FEXPR, DEXPR)                                                                 \
+    template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
+        static constexpr bool USES_PAIR_TABLE = sizeof(T) == 8;                                                             \
+        __device__ __forceinline__ bool operator()(T x, T, T& z) const {                                                    \
+            if constexpr (sizeof(T) == 4) z = (T)FEXPR((float)x);                                                           \
+            else z = (T)(DEXPR);                                                                                            \
+            return true; } };
+CUMO_HIP_OWN_OP_WITH_PAIR_TABLE(OpTanh, tanh_float_rounded_once, tanh_double((double)x))
+CUMO_HIP_OWN_OP_WITH_PAIR_TABLE(OpSinh, sinh_float_rounded_once, sinh_double((double)x))
+CUMO_HIP_OWN_OP_WITH_PAIR_TABLE(OpCosh, cosh_float_rounded_once, cosh_double((double)x))
 CUMO_HIP_OWN_OP(OpExpm1, expm1_float_rounded_once, (x == 0) ? (double)x : expm1((double)x))  // the library answers +0 for -0
 
 // (not HEAVY: with the short polynomial a lane's single vector keeps up with memory, and the transposed

@@ -63,6 +63,24 @@ def main():
     for n in range(1, 5):
         print("#define CUMO_HIP_EXP2_E%d %s" % (n, float.hex(to_double(ln2 ** n / mp.factorial(n)))))
 
+    # DFloat hyperbolic functions: e^a = 2^(k/32) e^r with a = k (ln 2 / 32) + r; 2^(j/32) as a double and what is
+    # left of it, ln 2 / 32 as a 42-bit double (k times it is exact for k < 2^11) and what is left of it
+    print("// 2^(j/32) = hi + lo, j = 0..31")
+    print("#define CUMO_HIP_EXPDD_TABLE \\")
+    dd = []
+    for j in range(32):
+        v = mp.mpf(2) ** (mp.mpf(j) / 32)
+        hi = to_double(v)
+        lo = to_double(v - mp.mpf(hi))
+        dd.append((hi, lo))
+    print(", \\\n".join("    %s, %s" % (float.hex(a), float.hex(b)) for a, b in dd))
+    step = ln2 / 32
+    hi = mp.ldexp(mp.floor(mp.ldexp(step, 6 + 41)), -(6 + 41))  # step < 2^-5: 42 bits from 2^-6 down
+    assert mp.mpf(2) ** -6 <= hi < mp.mpf(2) ** -5
+    print("#define CUMO_HIP_LN2_32_HI %s" % float.hex(float(hi)))
+    print("#define CUMO_HIP_LN2_32_LO %s" % float.hex(to_double(step - hi)))
+    print("#define CUMO_HIP_32_LN2 %s" % float.hex(to_double(32 / ln2)))
+
 
 if __name__ == "__main__":
     main()

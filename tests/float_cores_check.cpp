@@ -52,7 +52,8 @@ static const Core32 kCores32[] = {
     {"erfc", erfc_float_rounded_once, erfc},  {"sinc", sinc_float_rounded_once, sinc_ref},
 };
 struct Core64 { const char* name; F64 f; };
-static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>}};
+static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>},
+                                  {"tanh", tanh_double}, {"sinh", sinh_double}, {"cosh", cosh_double}};
 
 static int64_t ordered(float f) { int32_t i; std::memcpy(&i, &f, 4); return i < 0 ? (int64_t)INT32_MIN - i : i; }
 
@@ -78,6 +79,41 @@ int main(int argc, char** argv) {
                 if (d > worst) worst = d;
             }
             std::printf("%s %llu %llu %lld\n", c.name, (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
+        }
+        return 0;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "dsweep") == 0) {
+        // n random doubles per DFloat core (magnitudes spread evenly over the exponents from 2^-40 up to the function's
+        // range, both signs, then arguments next to the ends of the ranges) against the long double function, whose
+        // own error is 2^-11 ulp of a double; prints, per function, arguments tried and the largest error in ulps
+        const uint64_t n = std::strtoull(argv[2], nullptr, 10);
+        struct CoreL { const char* name; F64 f; long double (*ref)(long double); double top; };
+        const CoreL cores[] = {{"tanh", tanh_double, tanhl, 40.0}, {"sinh", sinh_double, sinhl, 710.4}, {"cosh", cosh_double, coshl, 710.4}};
+        for (const CoreL& c : cores) {
+            uint64_t state = 0x9e3779b97f4a7c15ull;
+            auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+            double worst = 0.0, worst_x = 0.0;
+            for (uint64_t it = 0; it < n; ++it) {
+                const uint64_t a = next(), b = next();
+                double x;
+                if (it % 4 != 3) {
+                    const double lo_e = -40.0, hi_e = std::log2(c.top);
+                    const double e = lo_e + (hi_e - lo_e) * (double)(a >> 11) * 0x1p-53;
+                    x = std::exp2(e) * (1.0 + (double)(b >> 12) * 0x1p-52 * 1e-3);
+                } else {
+                    x = c.top * (double)(a >> 11) * 0x1p-53;   // evenly over the range: mostly large arguments
+                }
+                if (x > c.top) x = c.top;
+                if (b & 1) x = -x;
+                const double got = c.f(x);
+                const long double want = c.ref((long double)x);
+                int ex;
+                std::frexp((double)want, &ex);
+                const long double ulp = std::ldexp(1.0L, ex - 53);
+                const double err = (double)(fabsl((long double)got - want) / ulp);
+                if (err > worst) { worst = err; worst_x = x; }
+            }
+            std::printf("%s %llu %.4f %a\n", c.name, (unsigned long long)n, worst, worst_x);
         }
         return 0;
     }

@@ -103,7 +103,7 @@ def cores(tmp_path_factory):
 
 SFLOAT_CORES = ("exp", "log", "log2", "log10", "log1p", "tanh", "sinh", "cosh", "expm1", "asinh", "acosh", "atanh", "sin", "cos", "tan",
                 "atan", "erf", "asin", "acos", "erfc", "sinc")
-DFLOAT_CORES = ("log", "log2", "log10")
+DFLOAT_CORES = ("log", "log2", "log10", "tanh", "sinh", "cosh")
 
 
 def test_device_algorithms_on_the_host_against_vectors(vec, cores, tmp_path):
@@ -133,6 +133,16 @@ def test_device_algorithms_on_the_host_against_vectors(vec, cores, tmp_path):
             # evaluated in double to 2^-40 or better and rounded once: the correctly rounded float
             # itself, bar the rare argument whose exact value lies that close to a rounding boundary
             assert (d > 0).sum() <= 1, (name, int((d > 0).sum()))
+
+
+def test_device_dfloat_hyperbolic_algorithms_against_long_double(cores):
+    """tanh, sinh, cosh of DFloat carry their exponential as a pair of doubles: the result's one rounding and little else."""
+    n = 200000000 if os.environ.get("CUMO_EXHAUSTIVE") else 2000000
+    out = subprocess.run([cores, "dsweep", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
+    assert [line.split()[0] for line in out] == ["tanh", "sinh", "cosh"]
+    for line in out:
+        name, tried, worst, where = line.split()
+        assert int(tried) == n and float(worst) <= 0.52, line
 
 
 def test_device_sfloat_algorithms_against_glibc_over_float_bit_patterns(cores):
