@@ -9,21 +9,36 @@
 // Included by ew_ops.h, inside namespace cumo_hip, after the tables of float_tables.inc.
 #pragma once
 
-constexpr int kExpPairTableDoubles = 64;
+constexpr int kExpPairTableDoubles = 64;    // 2^(j/32) as pairs
+constexpr int kLog2PairTableDoubles = 384;  // {invc, logc head, logc tail} for 128 intervals
 #ifdef CUMO_HIP_HOST_CHECK
-static const double kExpPairTableHost[kExpPairTableDoubles] = {CUMO_HIP_EXPDD_TABLE};
-inline const double* exp_pair_table() { return kExpPairTableHost; }
+static const double kPairTablesHost[kExpPairTableDoubles + kLog2PairTableDoubles] = {CUMO_HIP_EXPDD_TABLE, CUMO_HIP_LOG2DD_TABLE};
+inline const double* exp_pair_table() { return kPairTablesHost; }
+inline const double* log2_pair_table() { return kPairTablesHost + kExpPairTableDoubles; }
 #else
-__device__ const double kExpPairTableDevice[kExpPairTableDoubles] = {CUMO_HIP_EXPDD_TABLE};
+__device__ const double kPairTablesDevice[kExpPairTableDoubles + kLog2PairTableDoubles] = {CUMO_HIP_EXPDD_TABLE, CUMO_HIP_LOG2DD_TABLE};
 __device__ __forceinline__ double* exp_pair_table_lds() {
     __shared__ double table[kExpPairTableDoubles];
     return table;
 }
+__device__ __forceinline__ double* log2_pair_table_lds() {
+    __shared__ double table[kLog2PairTableDoubles];
+    return table;
+}
 __device__ __forceinline__ const double* exp_pair_table() { return exp_pair_table_lds(); }
+__device__ __forceinline__ const double* log2_pair_table() { return log2_pair_table_lds(); }
 // with all threads of the block, before the first element
 __device__ __forceinline__ void exp_pair_table_prepare() {
     double* t = exp_pair_table_lds();
-    for (unsigned i = threadIdx.x; i < (unsigned)kExpPairTableDoubles; i += blockDim.x) t[i] = kExpPairTableDevice[i];
+    for (unsigned i = threadIdx.x; i < (unsigned)kExpPairTableDoubles; i += blockDim.x) t[i] = kPairTablesDevice[i];
+    __syncthreads();
+}
+// (the power reads both tables)
+__device__ __forceinline__ void pow_pair_tables_prepare() {
+    double* t = exp_pair_table_lds();
+    double* l = log2_pair_table_lds();
+    for (unsigned i = threadIdx.x; i < (unsigned)kExpPairTableDoubles; i += blockDim.x) t[i] = kPairTablesDevice[i];
+    for (unsigned i = threadIdx.x; i < (unsigned)kLog2PairTableDoubles; i += blockDim.x) l[i] = kPairTablesDevice[kExpPairTableDoubles + i];
     __syncthreads();
 }
 #endif
@@ -134,4 +149,80 @@ __device__ __forceinline__ double cosh_double(double x) {
     exact_sum(eh, qh, sh, sl);
     const double y = 0.5 * (sh + (sl + (el + ql)));
     return down ? y * 4.0 : y;
+}
+
+// ---- DFloat power -------------------------------------------------------------------------
+// x^y = 2^(y log2 x) for a positive, finite, normal x and a finite y, with log2 x and the product carried as pairs:
+// a result within 2^-53 needs the exponent within 2^-58 or so, and the exponent reaches 1075.
+//   log2 x = k + logc + log2(1 + z): the high word minus 0x3fe69000 gives the binade k, the interval (128 of them; 1.0
+//   is the midpoint of one, whose entry is {1, 0, 0}) and a mantissa m in [0.7003, 1.4006); z = m invc - 1 is exact
+//   because invc has 8 bits or fewer; k + logc's head is exact because the head lies on a grid of 2^-42;
+//   log2(1 + z) = z (A1 + a1) + z^2 (A2 + a2) + z^3 (L3 + ... + L10 z^7): the first two products as pairs, the rest
+//   (below 2^-15 of the first) in double. |z| < 0.00585: what is left out is below 2^-70 of the first term.
+__device__ __forceinline__ void log2_pair(double x, const double* tab, double& lh, double& ll) {
+    const uint32_t hx = (uint32_t)__double2hiint(x);
+    const uint32_t t = hx - 0x3fe69000u;
+    const int k = (int)t >> 20;
+    const uint32_t i = (t >> 13) & 127u;
+    const double m = __hiloint2double((int)(hx - (t & 0xfff00000u)), __double2loint(x));
+    const double invc = tab[3 * i], ch = tab[3 * i + 1], cl = tab[3 * i + 2];
+    const double z = __builtin_fma(m, invc, -1.0);
+    const double p1 = z * CUMO_HIP_LOG2DD_A1;
+    const double p1e = __builtin_fma(z, CUMO_HIP_LOG2DD_a1, __builtin_fma(z, CUMO_HIP_LOG2DD_A1, -p1));
+    const double z2 = z * z;
+    const double z2e = __builtin_fma(z, z, -z2);
+    const double p2 = z2 * CUMO_HIP_LOG2DD_A2;
+    const double p2e = __builtin_fma(z2e, CUMO_HIP_LOG2DD_A2, __builtin_fma(z2, CUMO_HIP_LOG2DD_a2, __builtin_fma(z2, CUMO_HIP_LOG2DD_A2, -p2)));
+    double q = CUMO_HIP_LOG2DD_L10;
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L9);
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L8);
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L7);
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L6);
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L5);
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L4);
+    q = __builtin_fma(q, z, CUMO_HIP_LOG2DD_L3);
+    const double p3 = (z2 * z) * q;
+    // the exact sums in their short form: each left operand is zero or the larger one
+    const double base = int_to_double(k) + ch;
+    const double s1 = base + p1;
+    const double s1e = p1 - (s1 - base);
+    const double s2 = s1 + p2;
+    const double s2e = p2 - (s2 - s1);
+    const double rest = ((s1e + s2e) + (p1e + p2e)) + (p3 + cl);
+    lh = s2 + rest;
+    ll = (s2 - lh) + rest;
+}
+// 2^(eh + el) for |eh| <= 1100, |el| tiny: eh = (32 q + j) / 32 + r, 2^(j/32) as a pair from the table, 2^r - 1 from
+// seven terms, the exponent q through ldexp (which also rounds a subnormal result and overflows to infinity)
+__device__ __forceinline__ double exp2_of_pair(double eh, double el, const double* tab) {
+    const double big = 211106232532992.0;  // 1.5 * 2^47: the last mantissa bit is worth 1/32
+    const double t0 = eh + big;
+    const uint32_t ki = (uint32_t)__double2loint(t0);
+    const double r = (eh - (t0 - big)) + el;
+    double p = CUMO_HIP_EXP2DD_F7;
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2DD_F6);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2DD_F5);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2DD_F4);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2DD_F3);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2DD_F2);
+    p = __builtin_fma(p, r, CUMO_HIP_EXP2DD_F1);
+    p *= r;
+    const uint32_t j = ki & 31u;
+    const double th = tab[2 * j], tl = tab[2 * j + 1];
+    return ldexp(th + __builtin_fma(th, p, tl), (int)ki >> 5);
+}
+__device__ __forceinline__ double pow_double_fast(double x, double y) {
+    double lh, ll;
+    log2_pair(x, log2_pair_table(), lh, ll);
+    double eh = y * lh;
+    double el = __builtin_fma(y, ll, __builtin_fma(y, lh, -eh));
+    // beyond the double range either way (also an infinite product, whose remainder is not a number)
+    const bool far = !(__builtin_fabs(eh) <= 1100.0);
+    eh = far ? __builtin_copysign(1100.0, eh) : eh;
+    el = far ? 0.0 : el;
+    return exp2_of_pair(eh, el, exp_pair_table());
+}
+// every other argument (zero, negative, subnormal, infinite or NaN base; infinite or NaN exponent) goes to the library
+__device__ __forceinline__ bool pow_double_is_rare(double x, double y) {
+    return !((uint32_t)__double2hiint(x) - 0x00100000u < 0x7fe00000u && __builtin_fabs(y) < (double)INFINITY);
 }

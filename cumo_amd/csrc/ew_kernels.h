@@ -44,10 +44,13 @@ template <class O, class = void> struct op_uses_tables { static constexpr bool v
 template <class O> struct op_uses_tables<O, decltype((void)O::USES_TABLES)> { static constexpr bool value = O::USES_TABLES; };
 template <class O, class = void> struct op_uses_pair_table { static constexpr bool value = false; };
 template <class O> struct op_uses_pair_table<O, decltype((void)O::USES_PAIR_TABLE)> { static constexpr bool value = O::USES_PAIR_TABLE; };
+template <class O, class = void> struct op_uses_pow_pair_tables { static constexpr bool value = false; };
+template <class O> struct op_uses_pow_pair_tables<O, decltype((void)O::USES_POW_PAIR_TABLES)> { static constexpr bool value = O::USES_POW_PAIR_TABLES; };
 template <class Op>
 __device__ __forceinline__ void ew_op_prepare() {
     if constexpr (op_uses_tables<Op>::value) float_tables_prepare();
     if constexpr (op_uses_pair_table<Op>::value) exp_pair_table_prepare();
+    if constexpr (op_uses_pow_pair_tables<Op>::value) pow_pair_tables_prepare();
 }
 
 constexpr int kEwBlock = 256;
@@ -614,7 +617,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
                 }
             }
         };
-        if constexpr (TWO && op_uses_tables<Op>::value) {
+        if constexpr (TWO && (op_uses_tables<Op>::value || op_uses_pow_pair_tables<Op>::value)) {
             if (use_scalar == 0) arithmetic(std::integral_constant<int, 0>{});
             else if (use_scalar == 1) arithmetic(std::integral_constant<int, 1>{});
             else arithmetic(std::integral_constant<int, 2>{});

@@ -736,16 +736,26 @@ __device__ __forceinline__ float pow_float_rounded_once(float xf, float yf) {
     if (pow_is_rare(xf, yf)) z = pow_by_the_library(xf, yf);
     return z;
 }
+// DFloat: the same split with log2 x and y log2 x carried as pairs of doubles (dd_cores.h); a subnormal base goes to the
+// library too.
+__device__ __attribute__((noinline)) double pow_double_by_the_library(double x, double y) { return pow(x, y); }
 template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) static constexpr bool HEAVY = true;
-    static constexpr bool HAS_RARE = sizeof(T) == 4;
+    static constexpr bool HAS_RARE = true;
     static constexpr bool USES_TABLES = sizeof(T) == 4;
+    static constexpr bool USES_POW_PAIR_TABLES = sizeof(T) == 8;
     __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
-        if constexpr (sizeof(T) == 4) z = (T)pow_float_rounded_once((float)x, (float)y);
-        else z = (T)pow((double)x, (double)y);
+        fast(x, y, z);
+        if (rare(x, y)) z = slow(x, y);
         return true; }
-    __device__ __forceinline__ void fast(T x, T y, T& z) const { z = (T)pow_fast((float)x, (float)y); }
-    __device__ __forceinline__ bool rare(T x, T y) const { return pow_is_rare((float)x, (float)y); }
-    __device__ __forceinline__ T slow(T x, T y) const { return (T)pow_by_the_library((float)x, (float)y); } };
+    __device__ __forceinline__ void fast(T x, T y, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)pow_fast((float)x, (float)y);
+        else z = (T)pow_double_fast((double)x, (double)y); }
+    __device__ __forceinline__ bool rare(T x, T y) const {
+        if constexpr (sizeof(T) == 4) return pow_is_rare((float)x, (float)y);
+        else return pow_double_is_rare((double)x, (double)y); }
+    __device__ __forceinline__ T slow(T x, T y) const {
+        if constexpr (sizeof(T) == 4) return (T)pow_by_the_library((float)x, (float)y);
+        else return (T)pow_double_by_the_library((double)x, (double)y); } };
 
 // Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
 // element type for small exponents, pow() beyond 64, the reciprocal for negative ones.

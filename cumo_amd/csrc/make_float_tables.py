@@ -81,6 +81,52 @@ def main():
     print("#define CUMO_HIP_LN2_32_LO %s" % float.hex(to_double(step - hi)))
     print("#define CUMO_HIP_32_LN2 %s" % float.hex(to_double(32 / ln2)))
 
+    # DFloat power: log2 x as a pair. 128 intervals by the high word minus 0x3fe69000 (1.0 is the midpoint of interval
+    # 75, whose entry is {1, 0, 0}); invc has so few bits (7 after the point below 1, 8 above: what the interval's
+    # width leaves room for) that z = m invc - 1 is exact in one multiply-add; logc = -log2(invc) as a head on a
+    # grid of 2^-42 (so that binade + head is exact) and a tail.
+    off = 0x3FE69000
+    print("// {invc, logc head, logc tail} for the 128 intervals of the DFloat power's log2")
+    print("#define CUMO_HIP_LOG2DD_TABLE \\")
+    rows = []
+    worst = mp.mpf(0)
+    for i in range(128):
+        lo_hi, up_hi = off + (i << 13), off + ((i + 1) << 13)
+        a, b = mp.mpf(dbl(lo_hi)), mp.mpf(dbl(up_hi))
+        if a < 1 < b:
+            assert i == 75
+            rows.append((1.0, 0.0, 0.0))
+            worst = max(worst, 1 - a, b - 1)
+            continue
+        below = b <= 1
+        f = 7 if below else 8
+        c = (a + b) / 2
+        j = int(mp.nint(mp.ldexp(1 / c, f)))
+        invc = mp.ldexp(mp.mpf(j), -f)
+        zmax = max(abs(a * invc - 1), abs(b * invc - 1))
+        # z is a multiple of 2^(e - 52 - f), e the exponent of m (-1 below 1): it must fit 53 bits
+        e = -1 if below else 0
+        assert mp.log(zmax, 2) + 52 + f - e <= 53, (i, zmax)
+        worst = max(worst, zmax)
+        logc = -mp.log(invc, 2)
+        head = mp.ldexp(mp.nint(mp.ldexp(logc, 42)), -42)
+        tail = to_double(logc - head)
+        rows.append((float(invc), float(head), tail))
+        assert mp.mpf(float(head)) == head
+    print(", \\\n".join("    %s, %s, %s" % tuple(float.hex(v) for v in r) for r in rows))
+    print("// largest |z|: %s" % mp.nstr(worst, 8))
+    print("// log2(1 + z) = z ((A1 + a1) + (A2 + a2) z + L3 z^2 + ... + L10 z^9)")
+    for n in (1, 2):
+        v = mp.mpf((-1) ** (n + 1)) / (n * ln2)
+        hi = to_double(v)
+        print("#define CUMO_HIP_LOG2DD_A%d %s" % (n, float.hex(hi)))
+        print("#define CUMO_HIP_LOG2DD_a%d %s" % (n, float.hex(to_double(v - mp.mpf(hi)))))
+    for n in range(3, 11):
+        print("#define CUMO_HIP_LOG2DD_L%d %s" % (n, float.hex(to_double(mp.mpf((-1) ** (n + 1)) / (n * ln2)))))
+    print("// 2^r = 1 + r (F1 + F2 r + ... + F7 r^6), |r| <= 1/64")
+    for n in range(1, 8):
+        print("#define CUMO_HIP_EXP2DD_F%d %s" % (n, float.hex(to_double(ln2 ** n / mp.factorial(n)))))
+
 
 if __name__ == "__main__":
     main()

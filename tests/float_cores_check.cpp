@@ -117,6 +117,55 @@ int main(int argc, char** argv) {
         }
         return 0;
     }
+    if (argc >= 3 && std::strcmp(argv[1], "dpow") == 0) {
+        // n random (base, exponent) pairs through the DFloat power's arithmetic against the long double function: bases
+        // over every positive normal double with exponents that spread the results over the double range and past
+        // both of its ends, bases next to 1 with exponents up to 2^40, and everyday pairs; prints pairs tried and the
+        // largest error in ulps (of a normal result: a subnormal one is rounded twice, by the arithmetic and by ldexp)
+        const uint64_t n = std::strtoull(argv[2], nullptr, 10);
+        uint64_t state = 0x9e3779b97f4a7c15ull;
+        auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+        double worst = 0.0, worst_x = 0.0, worst_y = 0.0, worst_sub = 0.0;
+        uint64_t wrong_ends = 0;
+        for (uint64_t it = 0; it < n; ++it) {
+            const uint64_t a = next(), b = next();
+            double x, y;
+            const double u = (double)(b >> 11) * 0x1p-53;   // [0, 1)
+            if (it % 3 == 0) {
+                uint64_t bits = 0x0010000000000000ull + a % (0x7ff0000000000000ull - 0x0010000000000000ull);
+                std::memcpy(&x, &bits, 8);
+                const double lg = std::log2(x);
+                const double target = (2.0 * u - 1.0) * 1090.0;
+                y = lg != 0.0 ? target / lg : u * 1000.0;
+            } else if (it % 3 == 1) {
+                const double d = std::exp2(-1.0 - 50.0 * (double)(a >> 11) * 0x1p-53);   // distance from 1: 2^-51 .. 2^-1
+                x = (a & 1) ? 1.0 + d : 1.0 - d;
+                const double lg = std::log2(x);
+                y = (2.0 * u - 1.0) * 1090.0 / lg;
+                if (!(std::fabs(y) < 0x1p40)) y = (2.0 * u - 1.0) * 0x1p40;
+            } else {
+                x = 0.01 + 100.0 * (double)(a >> 11) * 0x1p-53;
+                y = (2.0 * u - 1.0) * 20.0;
+            }
+            if (pow_double_is_rare(x, y)) continue;
+            const double got = pow_double_fast(x, y);
+            const long double want = powl((long double)x, (long double)y);
+            if (want > 1.7976931348623157e308L * (1.0L + 0x1p-54L) || want < 0x1p-1076L) {
+                // past the ends: infinity above; zero (or the smallest subnormal next to the boundary) below
+                if (want > 1.7976931348623157e308L ? got != INFINITY : got > 4.9406564584124654e-324) ++wrong_ends;
+                continue;
+            }
+            int ex;
+            std::frexp((double)want, &ex);
+            const bool sub = ex < -1021;
+            const long double ulp = std::ldexp(1.0L, sub ? -1074 : ex - 53);
+            const double err = (double)(fabsl((long double)got - want) / ulp);
+            if (sub) { if (err > worst_sub) worst_sub = err; }
+            else if (err > worst) { worst = err; worst_x = x; worst_y = y; }
+        }
+        std::printf("pow %llu %.4f %.4f %llu %a %a\n", (unsigned long long)n, worst, worst_sub, (unsigned long long)wrong_ends, worst_x, worst_y);
+        return 0;
+    }
     if (argc >= 3 && std::strcmp(argv[1], "pow") == 0) {
         // n random (base, exponent) pairs: bases over every positive float, exponents spread so that results span the
         // float range (and beyond), then bases next to 1 with large exponents; against (float)pow((double)x, (double)y)

@@ -377,6 +377,46 @@ def test_nmath_two_args(tname, dt):
     assert_bits_equal(cls.cast(x).copysign(cls.cast(y)).to_numpy(), oracle.binary("copysign", x, y))
 
 
+def test_dfloat_power_of_arrays_with_every_kind_of_argument():
+    """DFloat ** DFloat: positive normal bases with finite exponents take the library's own arithmetic (log2 of the base
+    and its product with the exponent as pairs of doubles), every other argument the device library's pow. Both
+    against the host's pow: within 2 ulp (each side is within 1 of the true value) and equal where the rules decide
+    (signs, zeros, infinities, NaN, results beyond the range at either end)."""
+    import cumo_amd
+    rng = np.random.default_rng(108)
+    n = 200000
+    x = np.exp(rng.uniform(-700, 700, n))
+    y = rng.uniform(-1, 1, n) * 1080.0 / np.abs(np.log2(x))            # results over the whole range and past both ends
+    x[::5] = 1.0 + rng.uniform(-1, 1, x[::5].size) * np.exp2(rng.uniform(-50, -2, x[::5].size))
+    y[::5] = rng.uniform(-1, 1, y[::5].size) * np.exp2(rng.uniform(0, 40, y[::5].size))
+    x[1::5] = rng.uniform(0.01, 100, x[1::5].size)
+    y[1::5] = rng.uniform(-20, 20, y[1::5].size)
+    x[2::11] = -x[2::11]
+    y[2::22] = np.round(y[2::22])                                        # negative bases with whole exponents
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 5e-324, 2.2250738585072014e-308, 1.7976931348623157e308, 0.5, 2.0, 3.0])
+    x[3::101] = rng.choice(special, x[3::101].size)
+    y[4::103] = rng.choice(special, y[4::103].size)
+    y[5::107] = rng.choice(np.array([0.5, 2.0, 3.0, -1.0, 1.0, 0.0]), y[5::107].size)
+    with np.errstate(all="ignore"):
+        want = oracle.binary("pow", x, y)
+    got = (cumo_amd.DFloat.cast(x) ** cumo_amd.DFloat.cast(y)).to_numpy()
+    ruled = ~np.isfinite(want) | (want == 0) | ~np.isfinite(got) | (got == 0)
+    # (a result that rounds to the largest double or to a subnormal next to zero may fall on either side of the end)
+    edge = ruled & np.isfinite(x) & np.isfinite(y) & (x > 0) & (
+        (np.abs(want) >= 1.7976931348623157e308) | (np.abs(got) >= 1.7976931348623157e308) | ((np.abs(want) <= 1e-323) & (np.abs(got) <= 1e-323)))
+    strict = ruled & ~edge
+    assert_bits_equal(got[strict], want[strict], "rule-decided results")
+    assert_ulp(got[~ruled], want[~ruled], 2, "dfloat pow")
+    # one exponent for the whole array, and one base
+    for e in (2.5, -0.75, 1.0 / 3.0, 0.0, 7.0):
+        with np.errstate(all="ignore"):
+            want = oracle.binary("pow", x, e)
+        got = (cumo_amd.DFloat.cast(x) ** e).to_numpy()
+        ok = np.isfinite(want) & (want != 0) & np.isfinite(got) & (got != 0)
+        assert_ulp(got[ok], want[ok], 2, "dfloat pow %r" % e)
+        assert (np.isnan(got) == np.isnan(want)).all() and (np.isinf(got) == np.isinf(want))[~np.isnan(want) & (np.abs(want) < 1e308)].all()
+
+
 def test_int32_arithmetic():
     rng = np.random.default_rng(107)
     cls = cls_of("int32")

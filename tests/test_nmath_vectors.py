@@ -145,6 +145,16 @@ def test_device_dfloat_hyperbolic_algorithms_against_long_double(cores):
         assert int(tried) == n and float(worst) <= 0.52, line
 
 
+def test_device_dfloat_power_against_long_double(cores):
+    """x ** y of DFloat for a positive normal base and a finite exponent: log2 x and y log2 x as pairs of doubles."""
+    n = 300000000 if os.environ.get("CUMO_EXHAUSTIVE") else 3000000
+    name, tried, worst, worst_subnormal, wrong_ends, _, _ = subprocess.run(
+        [cores, "dpow", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.split()
+    assert name == "pow" and int(tried) == n
+    # (a subnormal result is rounded twice: by the arithmetic and by the scaling)
+    assert float(worst) <= 0.54 and float(worst_subnormal) <= 1.0 and int(wrong_ends) == 0
+
+
 def test_device_sfloat_algorithms_against_glibc_over_float_bit_patterns(cores):
     stride = 1 if os.environ.get("CUMO_EXHAUSTIVE") else 1021
     out = subprocess.run([cores, "sweep", str(stride)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
