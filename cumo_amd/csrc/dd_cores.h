@@ -11,10 +11,14 @@
 
 constexpr int kExpPairTableDoubles = 64;    // 2^(j/32) as pairs
 constexpr int kLog2PairTableDoubles = 384;  // {invc, logc head, logc tail} for 128 intervals
+constexpr int kErfcRowDoubles = 3 + CUMO_HIP_ERFC_DEGREE;   // {centre, g head, g tail, a1 ... }
+constexpr int kErfcTableDoubles = 45 * kErfcRowDoubles;
 #ifdef CUMO_HIP_HOST_CHECK
 static const double kPairTablesHost[kExpPairTableDoubles + kLog2PairTableDoubles] = {CUMO_HIP_EXPDD_TABLE, CUMO_HIP_LOG2DD_TABLE};
+static const double kErfcTableHost[kErfcTableDoubles] = {CUMO_HIP_ERFC_TABLE};
 inline const double* exp_pair_table() { return kPairTablesHost; }
 inline const double* log2_pair_table() { return kPairTablesHost + kExpPairTableDoubles; }
+inline const double* erfc_table() { return kErfcTableHost; }
 #else
 __device__ const double kPairTablesDevice[kExpPairTableDoubles + kLog2PairTableDoubles] = {CUMO_HIP_EXPDD_TABLE, CUMO_HIP_LOG2DD_TABLE};
 __device__ __forceinline__ double* exp_pair_table_lds() {
@@ -25,8 +29,14 @@ __device__ __forceinline__ double* log2_pair_table_lds() {
     __shared__ double table[kLog2PairTableDoubles];
     return table;
 }
+__device__ const double kErfcTableDevice[kErfcTableDoubles] = {CUMO_HIP_ERFC_TABLE};
+__device__ __forceinline__ double* erfc_table_lds() {
+    __shared__ double table[kErfcTableDoubles];
+    return table;
+}
 __device__ __forceinline__ const double* exp_pair_table() { return exp_pair_table_lds(); }
 __device__ __forceinline__ const double* log2_pair_table() { return log2_pair_table_lds(); }
+__device__ __forceinline__ const double* erfc_table() { return erfc_table_lds(); }
 // with all threads of the block, before the first element
 __device__ __forceinline__ void exp_pair_table_prepare() {
     double* t = exp_pair_table_lds();
@@ -39,6 +49,14 @@ __device__ __forceinline__ void pow_pair_tables_prepare() {
     double* l = log2_pair_table_lds();
     for (unsigned i = threadIdx.x; i < (unsigned)kExpPairTableDoubles; i += blockDim.x) t[i] = kPairTablesDevice[i];
     for (unsigned i = threadIdx.x; i < (unsigned)kLog2PairTableDoubles; i += blockDim.x) l[i] = kPairTablesDevice[kExpPairTableDoubles + i];
+    __syncthreads();
+}
+// (erfc reads the exponential's table and its own)
+__device__ __forceinline__ void erfc_tables_prepare() {
+    double* t = exp_pair_table_lds();
+    double* g = erfc_table_lds();
+    for (unsigned i = threadIdx.x; i < (unsigned)kExpPairTableDoubles; i += blockDim.x) t[i] = kPairTablesDevice[i];
+    for (unsigned i = threadIdx.x; i < (unsigned)kErfcTableDoubles; i += blockDim.x) g[i] = kErfcTableDevice[i];
     __syncthreads();
 }
 #endif
@@ -225,4 +243,75 @@ __device__ __forceinline__ double pow_double_fast(double x, double y) {
 // every other argument (zero, negative, subnormal, infinite or NaN base; infinite or NaN exponent) goes to the library
 __device__ __forceinline__ bool pow_double_is_rare(double x, double y) {
     return !((uint32_t)__double2hiint(x) - 0x00100000u < 0x7fe00000u && __builtin_fabs(y) < (double)INFINITY);
+}
+
+// ---- DFloat erfc --------------------------------------------------------------------------
+// erfc|x| = e^(-x^2) g(|x|), g(x) = e^(x^2) erfc(x), which varies slowly: 1 at 0, 1 / (x sqrt(pi)) far out.
+//   x^2 exactly as a pair (one multiply-add for the product's rounding error), the exponential of its negative as a
+//   pair (the reduction and table of expm1_pair; 2^128 times too large, so that 2^m stays a normal number down to the
+//   smallest subnormal result: ldexp at the end takes the 128 off and rounds a subnormal result);
+//   g from the Taylor series about the centre c of |x|'s interval (centres 0, 1/4 ... 1 below 1.125, eight intervals a
+//   binade from there: |x| - c is exact and at most an eighth, or a sixteenth of c): g(c) as a pair plus d times a
+//   polynomial of degree 15 in double, whose rounding shows as 0.07 ulp at most;
+//   the product of the two pairs rounded once; erfc(-|x|) = 2 - erfc|x|, the subtraction exact before its rounding.
+// The reference calls the CUDA library's erfc (ext/cumo/include/cumo/types/float_macro_kernel.h:120).
+__device__ __forceinline__ void exp_pair_scaled_up(double ah, double al, const double* tab, double& hi, double& lo) {
+    const double big = 6755399441055744.0;  // 1.5 * 2^52
+    const double t0 = __builtin_fma(ah, CUMO_HIP_32_LN2, big);
+    const uint32_t ki = (uint32_t)__double2loint(t0);
+    const double kd = t0 - big;
+    const double rh = __builtin_fma(-kd, CUMO_HIP_LN2_32_HI, ah);
+    const double tail = kd * CUMO_HIP_LN2_32_LO;
+    // (al is not small beside the reduction's own remainder: it joins r before the polynomial sees it)
+    const double r0 = rh - tail;
+    const double rl0 = ((rh - r0) - tail) + al;
+    const double r = r0 + rl0;
+    const double rl = (r0 - r) + rl0;
+    double q = 1.0 / 5040.0;
+    q = __builtin_fma(q, r, 1.0 / 720.0);
+    q = __builtin_fma(q, r, 1.0 / 120.0);
+    q = __builtin_fma(q, r, 1.0 / 24.0);
+    q = __builtin_fma(q, r, 1.0 / 6.0);
+    q = __builtin_fma(q, r, 0.5);
+    const double pl = __builtin_fma(r * r, q, rl);  // e^r - 1 - r
+    const uint32_t j = ki & 31u;
+    const int m = ((int)ki >> 5) + 128;
+    const double scale = __hiloint2double((m + 1023) << 20, 0);
+    const double sh = tab[2 * j] * scale, sl = tab[2 * j + 1] * scale;
+    const double p = sh * r;
+    const double pe = __builtin_fma(sh, r, -p);
+    const double s1 = sh + p;
+    const double rest = (p - (s1 - sh)) + (__builtin_fma(sh, pl, pe) + __builtin_fma(sl, 1.0 + r, 0.0));
+    hi = s1 + rest;
+    lo = (s1 - hi) + rest;
+}
+__device__ __forceinline__ double erfc_double(double x) {
+    const double* tab = erfc_table();
+    double a = __builtin_fabs(x);
+    a = __builtin_fmin(a, 27.5);   // beyond 27.3 the answer is 0 (a NaN becomes 27.5 here and is put back at the end)
+    // the interval: the nearest quarter below 1.125, the binade and three mantissa bits above
+    const uint32_t near = (uint32_t)__double2loint(__builtin_fma(a, 4.0, 6755399441055744.0)) & 7u;
+    const uint32_t far = 5u + (((uint32_t)__double2hiint(a) - 0x3ff00000u) >> 17);
+    const double* row = tab + (a < 1.125 ? near : far) * (uint32_t)kErfcRowDoubles;
+    const double d = a - row[0];
+    double p = row[2 + CUMO_HIP_ERFC_DEGREE];
+#pragma unroll
+    for (int n = CUMO_HIP_ERFC_DEGREE - 1; n >= 1; --n) p = __builtin_fma(p, d, row[2 + n]);
+    const double gt = __builtin_fma(d, p, row[2]);
+    const double gh = row[1] + gt;
+    const double gl = (row[1] - gh) + gt;
+    const double xh = a * a;
+    const double xl = __builtin_fma(a, a, -xh);
+    double eh, el;
+    exp_pair_scaled_up(-xh, -xl, exp_pair_table(), eh, el);
+    const double ph = eh * gh;
+    const double pe = __builtin_fma(eh, gl, __builtin_fma(el, gh, __builtin_fma(eh, gh, -ph)));
+    const double rh = ph + pe;
+    const double rl = (ph - rh) + pe;
+    const double yh = ldexp(rh, -128), yl = ldexp(rl, -128);
+    // 2 - (yh + yl) for a negative argument
+    const double s = 2.0 - yh;
+    const double below = s + (((2.0 - s) - yh) - yl);
+    const double y = (x < 0.0) ? below : yh;
+    return (x != x) ? x : y;
 }

@@ -46,11 +46,18 @@ template <class O, class = void> struct op_uses_pair_table { static constexpr bo
 template <class O> struct op_uses_pair_table<O, decltype((void)O::USES_PAIR_TABLE)> { static constexpr bool value = O::USES_PAIR_TABLE; };
 template <class O, class = void> struct op_uses_pow_pair_tables { static constexpr bool value = false; };
 template <class O> struct op_uses_pow_pair_tables<O, decltype((void)O::USES_POW_PAIR_TABLES)> { static constexpr bool value = O::USES_POW_PAIR_TABLES; };
+template <class O, class = void> struct op_uses_erfc_tables { static constexpr bool value = false; };
+template <class O> struct op_uses_erfc_tables<O, decltype((void)O::USES_ERFC_TABLES)> { static constexpr bool value = O::USES_ERFC_TABLES; };
+template <class Op> struct op_fills_tables {
+    static constexpr bool value = op_uses_tables<Op>::value || op_uses_pair_table<Op>::value || op_uses_pow_pair_tables<Op>::value ||
+                                  op_uses_erfc_tables<Op>::value;
+};
 template <class Op>
 __device__ __forceinline__ void ew_op_prepare() {
     if constexpr (op_uses_tables<Op>::value) float_tables_prepare();
     if constexpr (op_uses_pair_table<Op>::value) exp_pair_table_prepare();
     if constexpr (op_uses_pow_pair_tables<Op>::value) pow_pair_tables_prepare();
+    if constexpr (op_uses_erfc_tables<Op>::value) erfc_tables_prepare();
 }
 
 constexpr int kEwBlock = 256;
@@ -562,7 +569,15 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
     constexpr int NIN = Op::NIN;
     constexpr bool TWO = (NIN == 2);
     constexpr int UNR = op_is_heavy<Op>::value ? 2 : 1;
-    const uint64_t i0 = ((uint64_t)blockIdx.x * (kEwBlock * UNR) + threadIdx.x) * VEC;
+    // An operator with tables to fill takes several tiles per block (the launcher's grid is smaller than the number
+    // of tiles; tile t goes to block t mod the grid), so that one filling serves them all; every other operator
+    // gets a block per tile and runs the body once.
+    constexpr bool LOOPS = op_fills_tables<Op>::value;
+    const uint64_t tiles = LOOPS ? (n + (uint64_t)(kEwBlock * UNR * VEC) - 1) / (uint64_t)(kEwBlock * UNR * VEC) : 0;
+    uint64_t tile = blockIdx.x;
+    bool first_tile = true;
+    do {
+    const uint64_t i0 = (tile * (kEwBlock * UNR) + threadIdx.x) * VEC;
     const bool two_arrays = TWO && use_scalar == 0;
     A xv[UNR][VEC];
     B yv[UNR][VEC];
@@ -581,8 +596,9 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
     // Every vector is evaluated, loaded or not (an absent one holds zeros and is not stored):
     // with no branch around the arithmetic the compiler interleaves the elements of all the
     // lane's vectors, which the long dependent chains of the NMath functions need.
-    // (the tables of an operator that reads them are filled after the loads have gone out)
-    ew_op_prepare<Op>();
+    // (the tables of an operator that reads them are filled after the first tile's loads have gone out)
+    if (first_tile) ew_op_prepare<Op>();
+    first_tile = false;
     R zv[UNR][VEC];
     bool ok[UNR];
     if constexpr (op_has_rare<Op>::value) {
@@ -682,6 +698,8 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
             else if (flag) *flag = 1;
         }
     }
+    tile += gridDim.x;
+    } while (LOOPS && tile < tiles);
 }
 
 // ---------------------------------------------------------------------------
@@ -1527,6 +1545,17 @@ static inline unsigned ew_grid_cap() {
 // Largest x extent of a grid.
 static inline uint64_t ew_grid_max() { return 0x7fffffffull; }
 
+// Blocks of a flat launch whose operator fills tables in LDS (CUMO_HIP_EW_TABLE_BLOCKS; 12 per compute unit)
+static inline unsigned ew_table_op_blocks() {
+    static unsigned blocks = 0;
+    if (blocks == 0) {
+        const char* e = std::getenv("CUMO_HIP_EW_TABLE_BLOCKS");
+        const long v = e ? std::strtol(e, nullptr, 10) : 0;
+        blocks = v > 0 ? (unsigned)v : (unsigned)kNumCU * 12;
+    }
+    return blocks;
+}
+
 // Non-temporal accesses once an operation touches more than the caches could keep for
 // the next operation anyway. Measured with every launch on fresh operands (the state a
 // long computation is in): a 1R+1W operation over 2 x 128 MiB runs at 72-73% of the HBM
@@ -1928,7 +1957,9 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         const uint64_t per_block = (uint64_t)kEwBlock * fvec * (op_is_heavy<Op>::value ? 2 : 1);
         const uint64_t blocks = (kp.inner + per_block - 1) / per_block;
         if (flat && blocks <= ew_grid_max()) {
-            const dim3 g((unsigned)blocks);
+            // (an operator that fills tables: at most a dozen blocks per compute unit, which then take a tile after the other)
+            const uint64_t looping = (uint64_t)ew_table_op_blocks();
+            const dim3 g((unsigned)((op_fills_tables<Op>::value && blocks > looping) ? looping : blocks));
             if (fvec == 4) {
                 if (nt) hipLaunchKernelGGL((ew_flat_kernel<Op, 4, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
                 else hipLaunchKernelGGL((ew_flat_kernel<Op, 4, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);

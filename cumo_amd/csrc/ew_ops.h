@@ -689,7 +689,14 @@ __device__ __forceinline__ float sinc_float_rounded_once(float xf) {
 }
 CUMO_HIP_OWN_OP(OpSinc, sinc_float_rounded_once, (x == 0) ? 1.0 : (sin((double)x) / (double)x))
 CUMO_HIP_OWN_OP(OpErf, erf_float_rounded_once, erf((double)x))
-CUMO_HIP_OWN_OP_WITH_TABLES(OpErfc, erfc_float_rounded_once, erfc((double)x))
+// (DFloat: erfc_double of dd_cores.h, which reads its interval table and the exponential's)
+template <class T> struct OpErfc { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
+    static constexpr bool USES_TABLES = sizeof(T) == 4;
+    static constexpr bool USES_ERFC_TABLES = sizeof(T) == 8;
+    __device__ __forceinline__ bool operator()(T x, T, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)erfc_float_rounded_once((float)x);
+        else z = (T)erfc_double((double)x);
+        return true; } };
 
 #define CUMO_HIP_IUN(NAME, EXPR) \
     struct NAME { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false) \

@@ -53,7 +53,7 @@ static const Core32 kCores32[] = {
 };
 struct Core64 { const char* name; F64 f; };
 static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>},
-                                  {"tanh", tanh_double}, {"sinh", sinh_double}, {"cosh", cosh_double}};
+                                  {"tanh", tanh_double}, {"sinh", sinh_double}, {"cosh", cosh_double}, {"erfc", erfc_double}};
 
 static int64_t ordered(float f) { int32_t i; std::memcpy(&i, &f, 4); return i < 0 ? (int64_t)INT32_MIN - i : i; }
 
@@ -88,7 +88,8 @@ int main(int argc, char** argv) {
         // own error is 2^-11 ulp of a double; prints, per function, arguments tried and the largest error in ulps
         const uint64_t n = std::strtoull(argv[2], nullptr, 10);
         struct CoreL { const char* name; F64 f; long double (*ref)(long double); double top; };
-        const CoreL cores[] = {{"tanh", tanh_double, tanhl, 40.0}, {"sinh", sinh_double, sinhl, 710.4}, {"cosh", cosh_double, coshl, 710.4}};
+        const CoreL cores[] = {{"tanh", tanh_double, tanhl, 40.0}, {"sinh", sinh_double, sinhl, 710.4}, {"cosh", cosh_double, coshl, 710.4},
+                               {"erfc", erfc_double, erfcl, 26.5}};
         for (const CoreL& c : cores) {
             uint64_t state = 0x9e3779b97f4a7c15ull;
             auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };

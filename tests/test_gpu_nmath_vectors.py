@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ONE = ("sqrt cbrt log log2 log10 exp exp2 exp10 sin cos tan asin acos atan sinh cosh tanh "
        "asinh acosh atanh sinc erf erfc log1p expm1").split()
 TWO = ("atan2", "hypot", "pow")
-DEVICE_BOUND = {("erfc", "f64"): 2}
+DEVICE_BOUND = {}
 
 
 @pytest.fixture(scope="module")

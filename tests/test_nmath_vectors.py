@@ -103,7 +103,7 @@ def cores(tmp_path_factory):
 
 SFLOAT_CORES = ("exp", "log", "log2", "log10", "log1p", "tanh", "sinh", "cosh", "expm1", "asinh", "acosh", "atanh", "sin", "cos", "tan",
                 "atan", "erf", "asin", "acos", "erfc", "sinc")
-DFLOAT_CORES = ("log", "log2", "log10", "tanh", "sinh", "cosh")
+DFLOAT_CORES = ("log", "log2", "log10", "tanh", "sinh", "cosh", "erfc")
 
 
 def test_device_algorithms_on_the_host_against_vectors(vec, cores, tmp_path):
@@ -135,14 +135,15 @@ def test_device_algorithms_on_the_host_against_vectors(vec, cores, tmp_path):
             assert (d > 0).sum() <= 1, (name, int((d > 0).sum()))
 
 
-def test_device_dfloat_hyperbolic_algorithms_against_long_double(cores):
-    """tanh, sinh, cosh of DFloat carry their exponential as a pair of doubles: the result's one rounding and little else."""
+def test_device_dfloat_hyperbolic_and_erfc_algorithms_against_long_double(cores):
+    """tanh, sinh, cosh and erfc of DFloat carry their exponential as a pair of doubles: the result's one rounding and little else."""
     n = 200000000 if os.environ.get("CUMO_EXHAUSTIVE") else 2000000
     out = subprocess.run([cores, "dsweep", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
-    assert [line.split()[0] for line in out] == ["tanh", "sinh", "cosh"]
+    assert [line.split()[0] for line in out] == ["tanh", "sinh", "cosh", "erfc"]
     for line in out:
         name, tried, worst, where = line.split()
-        assert int(tried) == n and float(worst) <= 0.52, line
+        # (erfc: the series' first-order term is rounded in double, and subnormal results are rounded twice)
+        assert int(tried) == n and float(worst) <= (0.8 if name == "erfc" else 0.52), line
 
 
 def test_device_dfloat_power_against_long_double(cores):
