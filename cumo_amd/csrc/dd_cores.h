@@ -177,10 +177,10 @@ __device__ __forceinline__ double cosh_double(double x) {
 //   because invc has 8 bits or fewer; k + logc's head is exact because the head lies on a grid of 2^-42;
 //   log2(1 + z) = z (A1 + a1) + z^2 (A2 + a2) + z^3 (L3 + ... + L10 z^7): the first two products as pairs, the rest
 //   (below 2^-15 of the first) in double. |z| < 0.00585: what is left out is below 2^-70 of the first term.
-__device__ __forceinline__ void log2_pair(double x, const double* tab, double& lh, double& ll) {
+__device__ __forceinline__ void log2_pair(double x, const double* tab, double& lh, double& ll, int more_binades = 0) {
     const uint32_t hx = (uint32_t)__double2hiint(x);
     const uint32_t t = hx - 0x3fe69000u;
-    const int k = (int)t >> 20;
+    const int k = ((int)t >> 20) + more_binades;   // (log2 of 2^more x)
     const uint32_t i = (t >> 13) & 127u;
     const double m = __hiloint2double((int)(hx - (t & 0xfff00000u)), __double2loint(x));
     const double invc = tab[3 * i], ch = tab[3 * i + 1], cl = tab[3 * i + 2];
@@ -313,5 +313,116 @@ __device__ __forceinline__ double erfc_double(double x) {
     const double s = 2.0 - yh;
     const double below = s + (((2.0 - s) - yh) - yl);
     const double y = (x < 0.0) ? below : yh;
+    return (x != x) ? x : y;
+}
+
+// ---- DFloat log1p, asinh, acosh, atanh ------------------------------------------------------
+// Each is the logarithm of a quantity u that is built as a pair (uh + ul, |ul| within a few units in uh's last place):
+// ln u = ln 2 * log2 uh + ul / uh, the first term from log2_pair (good to 2^-66 of its value, next to 1 included) times
+// ln 2 as a pair, and one rounding at the end. The reference calls the CUDA library's functions
+// (ext/cumo/include/cumo/types/float_macro_kernel.h:107-118).
+__device__ __forceinline__ double ln_of_pair(double uh, double ul, int more_binades = 0) {
+    double lh, ll;
+    log2_pair(uh, log2_pair_table(), lh, ll, more_binades);
+    const double ln2h = 0x1.62e42fefa39efp-1, ln2l = 0x1.abc9e3b39803fp-56;
+    const double ph = lh * ln2h;
+    const double pe = __builtin_fma(ll, ln2h, __builtin_fma(lh, ln2l, __builtin_fma(lh, ln2h, -ph)));
+    return ph + __builtin_fma(ul, rcp_refined(uh), pe);
+}
+// a + b exactly as s + e for |a| >= |b| (or a == 0)
+__device__ __forceinline__ void exact_sum_ordered(double a, double b, double& s, double& e) {
+    s = a + b;
+    e = b - (s - a);
+}
+// sqrt(wh + wl) as a pair for a positive normal wh: the refined estimate, then what its square leaves of w, exactly
+__device__ __forceinline__ void sqrt_pair(double wh, double wl, double& sh, double& sl) {
+#ifdef CUMO_HIP_HOST_CHECK
+    sh = sqrt(wh);
+    const double half_over = 0.5 / sh;
+#else
+    const double y = __builtin_amdgcn_rsq(wh);
+    const double g = wh * y;
+    sh = __builtin_fma(__builtin_fma(-g, g, wh) * 0.5, y, g);
+    const double half_over = 0.5 * y;
+#endif
+    sl = (__builtin_fma(-sh, sh, wh) + wl) * half_over;
+}
+// log1p: u = 1 + x exactly as a pair; below 2^-54 the answer is x itself (the sign of a zero included)
+__device__ __forceinline__ double log1p_double(double x) {
+    double uh, ul;
+    exact_sum(1.0, x, uh, ul);
+    const bool fine = uh >= 2.2250738585072014e-308 && uh < (double)INFINITY;   // (x > -1, finite)
+    double y = ln_of_pair(fine ? uh : 1.0, fine ? ul : 0.0);
+    y = (__builtin_fabs(x) < 0x1p-54) ? x : y;
+    y = (x == -1.0) ? (double)-INFINITY : y;
+    y = (x < -1.0) ? (double)NAN : y;
+    y = (x == (double)INFINITY) ? x : y;
+    return (x != x) ? x : y;
+}
+// asinh|x| = ln(1 + v), v = |x| + x^2 / (1 + sqrt(1 + x^2)), every step a pair; beyond 2^500 (where x^2 would leave the
+// range) ln(2|x|); below 2^-28 x itself
+__device__ __forceinline__ double asinh_double(double x) {
+    const double a = __builtin_fabs(x);
+    const bool huge = !(a <= 0x1p500);   // (a NaN too: it is put back at the end)
+    const double am = huge ? 1.0 : a;
+    const double x2h = am * am;
+    const double x2l = __builtin_fma(am, am, -x2h);
+    double wh, wl, sh, sl, dh, dl, qh, ql, vh, vl, uh, ul;
+    exact_sum(1.0, x2h, wh, wl);
+    sqrt_pair(wh, wl + x2l, sh, sl);
+    exact_sum_ordered(sh, 1.0, dh, dl);
+    pair_quotient_pair(x2h, x2l, dh, dl + sl, qh, ql);
+    exact_sum_ordered(am, qh, vh, vl);
+    exact_sum(1.0, vh, uh, ul);
+    ul += vl + ql;
+    const bool far = huge && a < (double)INFINITY;
+    double y = ln_of_pair(far ? a : uh, far ? 0.0 : ul, far ? 1 : 0);
+    y = (a < 0x1p-28) ? a : y;
+    y = (a == (double)INFINITY) ? a : y;
+    y = __builtin_copysign(y, x);
+    return (x != x) ? x : y;
+}
+// acosh x = ln(x + sqrt(x^2 - 1)), x^2 - 1 exactly as a pair; beyond 2^500 ln(2x)
+__device__ __forceinline__ double acosh_double(double x) {
+    const bool huge = !(x <= 0x1p500);
+    const bool inside = x >= 1.0;
+    const double am = (huge || !inside) ? 1.0 : x;
+    const double x2h = am * am;
+    const double x2l = __builtin_fma(am, am, -x2h);
+    double wh, wl, sh, sl, uh, ul;
+    exact_sum_ordered(x2h, -1.0, wh, wl);
+    wl += x2l;
+    // (x next to 1: the head may cancel to nothing while the tail does not)
+    const double w0 = wh + wl;
+    const double w1 = (wh - w0) + wl;
+    const bool none = !(w0 > 0.0);
+    sqrt_pair(none ? 1.0 : w0, none ? 0.0 : w1, sh, sl);
+    sh = none ? 0.0 : sh;
+    sl = none ? 0.0 : sl;
+    exact_sum_ordered(am, sh, uh, ul);
+    ul += sl;
+    const bool far = huge && x < (double)INFINITY;
+    double y = ln_of_pair(far ? x : uh, far ? 0.0 : ul, far ? 1 : 0);
+    y = (x == (double)INFINITY) ? x : y;
+    y = (x < 1.0) ? (double)NAN : y;
+    return (x != x) ? x : y;
+}
+// atanh|x| = ln((1 + |x|) / (1 - |x|)) / 2, numerator, denominator and quotient as pairs; below 2^-28 x itself
+__device__ __forceinline__ double atanh_double(double x) {
+    const double a = __builtin_fabs(x);
+    const bool inside = a < 1.0;
+    const double am = inside ? a : 0.5;
+    double nh, nl, dh, dl, qh, ql;
+    exact_sum_ordered(1.0, am, nh, nl);
+    exact_sum_ordered(1.0, -am, dh, dl);
+    pair_quotient_pair(nh, nl, dh, dl, qh, ql);
+    // (the quotient's head and tail overlap by a few bits: ln_of_pair's u wants them apart)
+    const double uh = qh + ql;
+    const double ul = (qh - uh) + ql;
+    double y = 0.5 * ln_of_pair(uh, ul);
+    y = (a < 0x1p-28) ? a : y;
+    y = (a == 1.0) ? (double)INFINITY : y;
+    y = (a > 1.0) ? (double)NAN : y;
+    y = __builtin_copysign(y, x);
     return (x != x) ? x : y;
 }

@@ -340,10 +340,12 @@ __device__ __forceinline__ float log1p_float_rounded_once(float xf) {
 CUMO_HIP_LOG_OP(OpLog, 0)
 CUMO_HIP_LOG_OP(OpLog2, 2)
 CUMO_HIP_LOG_OP(OpLog10, 10)
+// (DFloat: log1p_double of dd_cores.h, which reads the table of the power's logarithm)
 template <class T> struct OpLog1p { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;
+    static constexpr bool USES_POW_PAIR_TABLES = sizeof(T) == 8;
     __device__ __forceinline__ bool operator()(T x, T, T& z) const {
         if constexpr (sizeof(T) == 4) z = (T)log1p_float_rounded_once((float)x);
-        else z = (x == 0) ? x : (T)log1p((double)x);  // the library answers +0 for -0
+        else z = (T)log1p_double((double)x);
         return true; } };
 
 // exp(x) - 1 for x inside [-745, 709] and a result that is rounded to float, from the reduction
@@ -669,16 +671,18 @@ CUMO_HIP_TRIG_OP(OpTan, 2, tan((double)x))
 CUMO_HIP_OWN_OP(OpAsin, asin_acos_float_rounded_once<false>, asin((double)x))
 CUMO_HIP_OWN_OP(OpAcos, asin_acos_float_rounded_once<true>, acos((double)x))
 CUMO_HIP_OWN_OP(OpAtan, atan_float_rounded_once, atan((double)x))
+// (DFloat: the cores of dd_cores.h, which read the table of the power's logarithm)
 #define CUMO_HIP_OWN_OP_WITH_TABLES(NAME, FEXPR, DEXPR)                                                                     \
     template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \
         static constexpr bool USES_TABLES = sizeof(T) == 4;                                                                 \
+        static constexpr bool USES_POW_PAIR_TABLES = sizeof(T) == 8;                                                        \
         __device__ __forceinline__ bool operator()(T x, T, T& z) const {                                                    \
             if constexpr (sizeof(T) == 4) z = (T)FEXPR((float)x);                                                           \
             else z = (T)(DEXPR);                                                                                            \
             return true; } };
-CUMO_HIP_OWN_OP_WITH_TABLES(OpAsinh, asinh_float_rounded_once, asinh((double)x))
-CUMO_HIP_OWN_OP_WITH_TABLES(OpAcosh, acosh_float_rounded_once, acosh((double)x))
-CUMO_HIP_OWN_OP_WITH_TABLES(OpAtanh, atanh_float_rounded_once, atanh((double)x))
+CUMO_HIP_OWN_OP_WITH_TABLES(OpAsinh, asinh_float_rounded_once, asinh_double((double)x))
+CUMO_HIP_OWN_OP_WITH_TABLES(OpAcosh, acosh_float_rounded_once, acosh_double((double)x))
+CUMO_HIP_OWN_OP_WITH_TABLES(OpAtanh, atanh_float_rounded_once, atanh_double((double)x))
 // the host macro guards x == 0 (types/float_macro.h:113); the reference's device
 // macro does not and answers NaN there, which Numo does not
 __device__ __attribute__((noinline)) float sinc_by_the_library(float xf) { return (float)(sin((double)xf) / (double)xf); }

@@ -53,7 +53,8 @@ static const Core32 kCores32[] = {
 };
 struct Core64 { const char* name; F64 f; };
 static const Core64 kCores64[] = {{"log", log_double<0>}, {"log2", log_double<2>}, {"log10", log_double<10>},
-                                  {"tanh", tanh_double}, {"sinh", sinh_double}, {"cosh", cosh_double}, {"erfc", erfc_double}};
+                                  {"tanh", tanh_double}, {"sinh", sinh_double}, {"cosh", cosh_double}, {"erfc", erfc_double},
+                                  {"log1p", log1p_double}, {"asinh", asinh_double}, {"acosh", acosh_double}, {"atanh", atanh_double}};
 
 static int64_t ordered(float f) { int32_t i; std::memcpy(&i, &f, 4); return i < 0 ? (int64_t)INT32_MIN - i : i; }
 
@@ -89,7 +90,8 @@ int main(int argc, char** argv) {
         const uint64_t n = std::strtoull(argv[2], nullptr, 10);
         struct CoreL { const char* name; F64 f; long double (*ref)(long double); double top; };
         const CoreL cores[] = {{"tanh", tanh_double, tanhl, 40.0}, {"sinh", sinh_double, sinhl, 710.4}, {"cosh", cosh_double, coshl, 710.4},
-                               {"erfc", erfc_double, erfcl, 26.5}};
+                               {"erfc", erfc_double, erfcl, 26.5}, {"log1p", log1p_double, log1pl, 1e300}, {"asinh", asinh_double, asinhl, 1e300},
+                               {"acosh", acosh_double, acoshl, 1e300}, {"atanh", atanh_double, atanhl, 1.0}};
         for (const CoreL& c : cores) {
             uint64_t state = 0x9e3779b97f4a7c15ull;
             auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
@@ -97,7 +99,7 @@ int main(int argc, char** argv) {
             for (uint64_t it = 0; it < n; ++it) {
                 const uint64_t a = next(), b = next();
                 double x;
-                if (it % 4 != 3) {
+                if (it % 4 != 3 || c.top > 1e10) {
                     const double lo_e = -40.0, hi_e = std::log2(c.top);
                     const double e = lo_e + (hi_e - lo_e) * (double)(a >> 11) * 0x1p-53;
                     x = std::exp2(e) * (1.0 + (double)(b >> 12) * 0x1p-52 * 1e-3);
@@ -105,7 +107,11 @@ int main(int argc, char** argv) {
                     x = c.top * (double)(a >> 11) * 0x1p-53;   // evenly over the range: mostly large arguments
                 }
                 if (x > c.top) x = c.top;
-                if (b & 1) x = -x;
+                const bool is = std::strcmp(c.name, "acosh") == 0;
+                if (is) x = 1.0 + x;                                     // 1 + 2^-40 ... : the domain of acosh
+                else if (std::strcmp(c.name, "atanh") == 0) { if (x >= 1.0) x = 1.0 - 0x1p-53 * (double)(1 + (a & 0xffff)); }
+                else if (std::strcmp(c.name, "log1p") == 0 && (b & 1) && x >= 1.0) x = 1.0 - 0x1p-53 * (double)(1 + (a & 0xffff));
+                if ((b & 1) && !is) x = -x;
                 const double got = c.f(x);
                 const long double want = c.ref((long double)x);
                 int ex;

@@ -103,7 +103,7 @@ def cores(tmp_path_factory):
 
 SFLOAT_CORES = ("exp", "log", "log2", "log10", "log1p", "tanh", "sinh", "cosh", "expm1", "asinh", "acosh", "atanh", "sin", "cos", "tan",
                 "atan", "erf", "asin", "acos", "erfc", "sinc")
-DFLOAT_CORES = ("log", "log2", "log10", "tanh", "sinh", "cosh", "erfc")
+DFLOAT_CORES = ("log", "log2", "log10", "tanh", "sinh", "cosh", "erfc", "log1p", "asinh", "acosh", "atanh")
 
 
 def test_device_algorithms_on_the_host_against_vectors(vec, cores, tmp_path):
@@ -135,11 +135,12 @@ def test_device_algorithms_on_the_host_against_vectors(vec, cores, tmp_path):
             assert (d > 0).sum() <= 1, (name, int((d > 0).sum()))
 
 
-def test_device_dfloat_hyperbolic_and_erfc_algorithms_against_long_double(cores):
-    """tanh, sinh, cosh and erfc of DFloat carry their exponential as a pair of doubles: the result's one rounding and little else."""
+def test_device_dfloat_algorithms_on_pairs_against_long_double(cores):
+    """tanh, sinh, cosh and erfc of DFloat carry their exponential as a pair of doubles, log1p and the inverse hyperbolic
+    functions the argument of their logarithm: the result's one rounding and little else."""
     n = 200000000 if os.environ.get("CUMO_EXHAUSTIVE") else 2000000
     out = subprocess.run([cores, "dsweep", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
-    assert [line.split()[0] for line in out] == ["tanh", "sinh", "cosh", "erfc"]
+    assert [line.split()[0] for line in out] == ["tanh", "sinh", "cosh", "erfc", "log1p", "asinh", "acosh", "atanh"]
     for line in out:
         name, tried, worst, where = line.split()
         # (erfc: the series' first-order term is rounded in double, and subnormal results are rounded twice)
