@@ -261,7 +261,7 @@ def config_ops(name, cumo, host):
         ops = []
         for fname in ("log", "sin", "cos", "tan", "tanh", "erf", "asinh", "atan", "exp", "sqrt", "log1p", "sinh", "erfc", "cbrt"):
             ops.append(("NMath.%s(SFloat)" % fname, (lambda f: lambda e: e.__setitem__("r", getattr(NM, f)(e["xs"])))(fname), 8 * n, n))
-        for fname in ("log", "sin", "tanh", "erf", "exp", "sqrt"):
+        for fname in ("log", "sin", "tanh", "erf", "exp", "sqrt", "erfc", "asinh", "log1p"):
             ops.append(("NMath.%s(DFloat)" % fname, (lambda f: lambda e: e.__setitem__("rd", getattr(NM, f)(e["xd"])))(fname), 16 * n, n))
         ops += [
             ("SFloat**2.5", lambda e: e.__setitem__("r", e["xs"] ** 2.5), 8 * n, n),

@@ -12,7 +12,7 @@
 constexpr int kExpPairTableDoubles = 64;    // 2^(j/32) as pairs
 constexpr int kLog2PairTableDoubles = 384;  // {invc, logc head, logc tail} for 128 intervals
 constexpr int kErfcRowDoubles = 3 + CUMO_HIP_ERFC_DEGREE;   // {centre, g head, g tail, a1 ... }
-constexpr int kErfcTableDoubles = 45 * kErfcRowDoubles;
+constexpr int kErfcTableDoubles = CUMO_HIP_ERFC_ROWS * kErfcRowDoubles;
 #ifdef CUMO_HIP_HOST_CHECK
 static const double kPairTablesHost[kExpPairTableDoubles + kLog2PairTableDoubles] = {CUMO_HIP_EXPDD_TABLE, CUMO_HIP_LOG2DD_TABLE};
 static const double kErfcTableHost[kErfcTableDoubles] = {CUMO_HIP_ERFC_TABLE};
@@ -250,9 +250,9 @@ __device__ __forceinline__ bool pow_double_is_rare(double x, double y) {
 //   x^2 exactly as a pair (one multiply-add for the product's rounding error), the exponential of its negative as a
 //   pair (the reduction and table of expm1_pair; 2^128 times too large, so that 2^m stays a normal number down to the
 //   smallest subnormal result: ldexp at the end takes the 128 off and rounds a subnormal result);
-//   g from the Taylor series about the centre c of |x|'s interval (centres 0, 1/4 ... 1 below 1.125, eight intervals a
-//   binade from there: |x| - c is exact and at most an eighth, or a sixteenth of c): g(c) as a pair plus d times a
-//   polynomial of degree 15 in double, whose rounding shows as 0.07 ulp at most;
+//   g from the Taylor series about the centre c of |x|'s interval (centres 0, 1/16 ... 1 below 1 + 1/32, 32 intervals a
+//   binade from there: |x| - c is exact and at most 1/32, or 1/64 of c): g(c) as a pair plus d times a polynomial of
+//   degree 9 in double, whose rounding shows as 0.02 ulp at most;
 //   the product of the two pairs rounded once; erfc(-|x|) = 2 - erfc|x|, the subtraction exact before its rounding.
 // The reference calls the CUDA library's erfc (ext/cumo/include/cumo/types/float_macro_kernel.h:120).
 __device__ __forceinline__ void exp_pair_scaled_up(double ah, double al, const double* tab, double& hi, double& lo) {
@@ -289,10 +289,10 @@ __device__ __forceinline__ double erfc_double(double x) {
     const double* tab = erfc_table();
     double a = __builtin_fabs(x);
     a = __builtin_fmin(a, 27.5);   // beyond 27.3 the answer is 0 (a NaN becomes 27.5 here and is put back at the end)
-    // the interval: the nearest quarter below 1.125, the binade and three mantissa bits above
-    const uint32_t near = (uint32_t)__double2loint(__builtin_fma(a, 4.0, 6755399441055744.0)) & 7u;
-    const uint32_t far = 5u + (((uint32_t)__double2hiint(a) - 0x3ff00000u) >> 17);
-    const double* row = tab + (a < 1.125 ? near : far) * (uint32_t)kErfcRowDoubles;
+    // the interval: the nearest sixteenth below 1 + 1/32, the binade and five mantissa bits above
+    const uint32_t near = (uint32_t)__double2loint(__builtin_fma(a, 16.0, 6755399441055744.0)) & 31u;
+    const uint32_t far = 17u + (((uint32_t)__double2hiint(a) - 0x3ff00000u) >> 15);
+    const double* row = tab + (a < 1.03125 ? near : far) * (uint32_t)kErfcRowDoubles;
     const double d = a - row[0];
     double p = row[2 + CUMO_HIP_ERFC_DEGREE];
 #pragma unroll

@@ -48,6 +48,13 @@ template <class O, class = void> struct op_uses_pow_pair_tables { static constex
 template <class O> struct op_uses_pow_pair_tables<O, decltype((void)O::USES_POW_PAIR_TABLES)> { static constexpr bool value = O::USES_POW_PAIR_TABLES; };
 template <class O, class = void> struct op_uses_erfc_tables { static constexpr bool value = false; };
 template <class O> struct op_uses_erfc_tables<O, decltype((void)O::USES_ERFC_TABLES)> { static constexpr bool value = O::USES_ERFC_TABLES; };
+template <class O, class = void> struct op_is_heavy { static constexpr bool value = false; };
+template <class O> struct op_is_heavy<O, decltype((void)O::HEAVY)> { static constexpr bool value = O::HEAVY; };
+// Vectors a lane of the flat kernel takes: two for the functions with long chains of dependent operations (their
+// elements are evaluated side by side), one for everything else.
+template <class Op> struct ew_flat_vectors_per_lane {
+    static constexpr int value = op_is_heavy<Op>::value ? 2 : 1;
+};
 template <class Op> struct op_fills_tables {
     static constexpr bool value = op_uses_tables<Op>::value || op_uses_pair_table<Op>::value || op_uses_pow_pair_tables<Op>::value ||
                                   op_uses_erfc_tables<Op>::value;
@@ -461,8 +468,6 @@ __global__ __launch_bounds__(kEwBlock) void ew_rows_kernel(EwKParams p, Op op, t
 // vectors, a block apart, so that one vector's loads are in flight while the other
 // is computed (measured on the SFloat exp of 2^27 elements: 168 us against 178 us;
 // for a plain copy the single vector is ahead, 164 us against 175 us).
-template <class O, class = void> struct op_is_heavy { static constexpr bool value = false; };
-template <class O> struct op_is_heavy<O, decltype((void)O::HEAVY)> { static constexpr bool value = O::HEAVY; };
 // Ops that declare HAS_RARE offer fast / rare / slow beside operator() (see ew_ops.h).
 template <class O, class = void> struct op_has_rare { static constexpr bool value = false; };
 template <class O> struct op_has_rare<O, decltype((void)O::HAS_RARE)> { static constexpr bool value = O::HAS_RARE; };
@@ -568,7 +573,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
     typedef typename Op::R R;
     constexpr int NIN = Op::NIN;
     constexpr bool TWO = (NIN == 2);
-    constexpr int UNR = op_is_heavy<Op>::value ? 2 : 1;
+    constexpr int UNR = ew_flat_vectors_per_lane<Op>::value;
     // An operator with tables to fill takes several tiles per block (the launcher's grid is smaller than the number
     // of tiles; tile t goes to block t mod the grid), so that one filling serves them all; every other operator
     // gets a block per tile and runs the body once.
@@ -1954,7 +1959,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         // stores one 128-bit vector and a wave one contiguous KiB, rather than two vectors 32 bytes apart
         // (SFloat [8192,4096] -> DFloat: 89.7 -> 62.4 us).
         const int fvec = (sizeof(R) > sizeof(A) && vec == 4) ? 2 : vec;
-        const uint64_t per_block = (uint64_t)kEwBlock * fvec * (op_is_heavy<Op>::value ? 2 : 1);
+        const uint64_t per_block = (uint64_t)kEwBlock * fvec * ew_flat_vectors_per_lane<Op>::value;
         const uint64_t blocks = (kp.inner + per_block - 1) / per_block;
         if (flat && blocks <= ew_grid_max()) {
             // (an operator that fills tables: at most a dozen blocks per compute unit, which then take a tile after the other)

@@ -128,19 +128,20 @@ def main():
         print("#define CUMO_HIP_EXP2DD_F%d %s" % (n, float.hex(to_double(ln2 ** n / mp.factorial(n)))))
 
     # DFloat erfc: g(x) = e^(x^2) erfc(x) by its Taylor series about the centre of the argument's interval: centres
-    # 0, 1/4, ..., 1 for x < 1.125 (within 1/8 of each), then eight intervals a binade up to 32 (the centre is the
-    # midpoint); per interval {c, g(c) as head and tail, a1 ... a16}. From g' = 2 x g - 2 / sqrt(pi):
+    # 0, 1/16, ..., 1 for x < 1 + 1/32 (within 1/32 of each), then 32 intervals a binade up to 32 (the centre is the
+    # midpoint); per interval {c, g(c) as head and tail, a1 ... a10}. From g' = 2 x g - 2 / sqrt(pi):
     # a1 = 2 c a0 - 2 / sqrt(pi), a(n+1) = (2 c a(n) + 2 a(n-1)) / (n + 1) (run forwards at 1200 bits: the recurrence
     # loses some 150 of them at the far end)
     mp.mp.prec = 1200
-    degree = 16
-    spans = [(mp.mpf(i) / 4, max(mp.mpf(0), mp.mpf(i) / 4 - mp.mpf(1) / 8), mp.mpf(i) / 4 + mp.mpf(1) / 8) for i in range(5)]
+    degree = 10
+    spans = [(mp.mpf(i) / 16, max(mp.mpf(0), mp.mpf(i) / 16 - mp.mpf(1) / 32), mp.mpf(i) / 16 + mp.mpf(1) / 32) for i in range(17)]
     for e in range(5):
-        for j in range(8):
-            lo, hi = mp.mpf(2) ** e * (1 + mp.mpf(j) / 8), mp.mpf(2) ** e * (1 + mp.mpf(j + 1) / 8)
+        for j in range(32):
+            lo, hi = mp.mpf(2) ** e * (1 + mp.mpf(j) / 32), mp.mpf(2) ** e * (1 + mp.mpf(j + 1) / 32)
             spans.append(((lo + hi) / 2, lo, hi))
     print("// {c, g(c) head, g(c) tail, a1 .. a%d} for the %d intervals of the DFloat erfc" % (degree, len(spans)))
     print("#define CUMO_HIP_ERFC_DEGREE %d" % degree)
+    print("#define CUMO_HIP_ERFC_ROWS %d" % len(spans))
     print("#define CUMO_HIP_ERFC_TABLE \\")
     lines = []
     worst = mp.mpf(0)
@@ -157,7 +158,7 @@ def main():
             got = mp.mpf(row[1]) + mp.mpf(row[2]) + sum(mp.mpf(row[2 + n]) * d ** n for n in range(1, degree + 1))
             worst = max(worst, abs(got / (mp.exp(x * x) * mp.erfc(x)) - 1))
         lines.append("    " + ", ".join(float.hex(v) for v in row))
-    assert worst < mp.mpf(2) ** -55, worst   # (the coefficients' own rounding included; the series alone is good to 2^-67)
+    assert worst < mp.mpf(2) ** -55, worst   # (the coefficients' own rounding included; the series alone is good to 2^-63)
     print(", \\\n".join(lines))
     print("// largest error of the rounded series at the interval ends: 2^%s" % mp.nstr(mp.log(worst, 2), 5))
     mp.mp.prec = 200
