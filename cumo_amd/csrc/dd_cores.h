@@ -1,11 +1,15 @@
-// DFloat tanh, sinh and cosh from an exponential carried as a pair of doubles (a value and what
-// is left of it), so that the one rounding of the result is the only one that shows: about 60
-// double operations an element where the device library's versions, which work on such pairs
-// throughout, take some 300. The reference calls the CUDA library's tanh / sinh / cosh
-// (ext/cumo/include/cumo/types/float_macro_kernel.h:101-106).
+// DFloat functions whose error would show if they were evaluated in double alone: tanh, sinh, cosh and erfc (an
+// exponential), x ** y (a logarithm times the exponent, then an exponential), log1p, asinh, acosh and atanh (the
+// logarithm of a sum, root or quotient). A double has nothing wider to be evaluated in, so the one quantity that
+// matters is carried as a pair of doubles (a value and what is left of it) through exact sums (two-sum), exact
+// products (the multiply-add's remainder) and quotients corrected by their exact remainder, and everything else stays
+// in double: 60 to 120 double operations an element where the device library's versions, which work on pairs
+// throughout, take about 300. The reference calls the CUDA library's functions
+// (ext/cumo/include/cumo/types/float_macro_kernel.h:36,101-120).
 //
-// Every step is an IEEE operation except the reciprocal estimate, which only enters through a
-// correction term; a CPU build (CUMO_HIP_HOST_CHECK) computes the same up to that.
+// Every step is an IEEE operation except the reciprocal and reciprocal square root estimates, which only enter
+// through correction terms; a CPU build (CUMO_HIP_HOST_CHECK) computes the same up to that, and
+// tests/float_cores_check.cpp runs it against the long double functions.
 // Included by ew_ops.h, inside namespace cumo_hip, after the tables of float_tables.inc.
 #pragma once
 
@@ -281,7 +285,7 @@ __device__ __forceinline__ void exp_pair_scaled_up(double ah, double al, const d
     const double p = sh * r;
     const double pe = __builtin_fma(sh, r, -p);
     const double s1 = sh + p;
-    const double rest = (p - (s1 - sh)) + (__builtin_fma(sh, pl, pe) + __builtin_fma(sl, 1.0 + r, 0.0));
+    const double rest = (p - (s1 - sh)) + __builtin_fma(sl, 1.0 + r, __builtin_fma(sh, pl, pe));
     hi = s1 + rest;
     lo = (s1 - hi) + rest;
 }

@@ -8,6 +8,10 @@
 //                                      patterns), prints the results as hex bit patterns
 //   float_cores_check pow <n>          n random (base, exponent) pairs through the SFloat power's arithmetic against
 //                                      (float)glibc pow; prints pairs tried, mismatches and the largest difference in ulps
+//   float_cores_check dsweep <n>       n random doubles through each DFloat core that works on pairs of doubles (tanh sinh
+//                                      cosh erfc log1p asinh acosh atanh) against the long double function; prints, per
+//                                      function, arguments tried, the largest error in ulps and where it was
+//   float_cores_check dpow <n>         n random (base, exponent) pairs through the DFloat power's arithmetic against powl
 //   float_cores_check sweep <stride>   every stride-th float bit pattern through each SFloat
 //                                      core against (float)glibc((double)x); prints, per
 //                                      function, patterns tried, mismatches and the largest
