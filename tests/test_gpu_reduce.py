@@ -138,6 +138,38 @@ def test_reductions_along_an_axis_that_strides_through_memory(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+@pytest.mark.parametrize("shape", [(4096, 1023), (4096, 1022), (2048, 1021), (4098, 1023), (4097, 1023), (1024, 4095)])
+def test_column_sums_of_rows_that_are_not_whole_vectors(tname, dt, shape):
+    """sum / mean / prod (and the nan forms of the first two) down the columns of a contiguous matrix whose rows are not
+    whole 16-byte vectors, a few thousand columns wide: the axis is cut across blocks and a second launch folds the parts."""
+    rng = np.random.default_rng(208)
+    cls = cls_of(tname)
+    h = rng.uniform(-1, 1, size=shape).astype(dt)
+    h[rng.random(shape) < 0.001] = np.nan
+    hn = np.where(np.isnan(h), dt(0.25), h)
+    n = shape[0]
+    for src, names in ((hn, ("sum", "mean")), (h, ("sum", "mean"))):
+        d = cls.cast(src)
+        for name in names:
+            nan = src is h
+            want = exact_reduce(name, hn if not nan else np.where(np.isnan(h), 0, h), 0)
+            if nan and name == "mean":
+                want = want * n / np.maximum((~np.isnan(h)).sum(axis=0), 1)
+            got = getattr(d, name)(axis=0, nan=True).to_numpy() if nan else getattr(d, name)(axis=0).to_numpy()
+            scale = abs_sum(hn, 0) / (n if name == "mean" else 1)
+            assert_reduction_close(got, want.astype(dt), n, scale, "%s nan=%r %r" % (name, nan, shape))
+        if src is h:
+            # without nan: true a NaN anywhere in the column is the answer
+            got = d.sum(axis=0).to_numpy()
+            assert (np.isnan(got) == np.isnan(h).any(axis=0)).all()
+    # products of numbers next to 1, so that 4096 of them stay in range
+    hp = (1.0 + rng.uniform(-1, 1, size=shape) * 1e-3).astype(dt)
+    want = np.prod(hp.astype(np.longdouble), axis=0)
+    got = cls.cast(hp).prod(axis=0).to_numpy()
+    assert_reduction_close(got, want.astype(dt), n, np.abs(want).astype(np.float64), "prod %r" % (shape,))
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((1000003,), None), ((7, 100000), 1), ((100000, 7), 0), ((3, 40000, 5), 1),
                                         ((64, 64, 64), (0, 2)), ((2, 3), None), ((1,), None), ((70000, 3), 1),
                                         ((5, 8192), 1), ((4096, 33), 0), ((33, 4096), 0), ((3, 2000003), 1), ((130, 40000), 1), ((260, 30000), 1)])
