@@ -47,3 +47,26 @@ def test_device_against_correctly_rounded_vectors(vec, name):
             again = getattr(cumo_amd.NMath, name)(v).to_numpy()
             same = (again == got) | (np.isnan(again) & np.isnan(got))
             assert same.all(), name
+
+
+def test_table_functions_over_many_tiles(vec):
+    """The functions that fill tables in LDS take their tiles a block after the other in a capped grid: the vectors'
+    arguments repeated over some 300 tiles (or 5000, past the cap) give the vectors' answers at every repetition."""
+    import cumo_amd
+    for fmt, cls, names in (("f32", cumo_amd.SFloat, ("asinh", "acosh", "atanh", "erfc")),
+                            ("f64", cumo_amd.DFloat, ("tanh", "sinh", "cosh", "erfc", "log1p", "asinh", "acosh", "atanh"))):
+        for name in names:
+            x = vec["%s_%s_x" % (name, fmt)]
+            small = getattr(cumo_amd.NMath, name)(cls.cast(x)).to_numpy()
+            for reps in (431, 7919 if name in ("erfc", "asinh") else 0):
+                if not reps:
+                    continue
+                big = getattr(cumo_amd.NMath, name)(cls.cast(np.tile(x, reps))).to_numpy().reshape(reps, x.size)
+                same = (big == small[None, :]) | (np.isnan(big) & np.isnan(small)[None, :])
+                assert same.all(), (name, fmt, reps)
+    for fmt, cls in (("f32", cumo_amd.SFloat), ("f64", cumo_amd.DFloat)):
+        x, y = vec["pow_%s_x" % fmt], vec["pow_%s_y" % fmt]
+        small = (cls.cast(x) ** cls.cast(y)).to_numpy()
+        big = (cls.cast(np.tile(x, 4001)) ** cls.cast(np.tile(y, 4001))).to_numpy().reshape(4001, x.size)
+        same = (big == small[None, :]) | (np.isnan(big) & np.isnan(small)[None, :])
+        assert same.all(), ("pow", fmt)

@@ -85,3 +85,12 @@ def test_bit_vector_kernels_with_lanes_that_loop():
               ["tests/test_gpu_bit.py::test_rows_of_bits_in_views_word_by_word", "tests/test_gpu_bit.py::test_long_runs_of_bits_by_whole_vectors",
                "tests/test_gpu_bit.py::test_windows_of_a_large_matrix_into_a_fresh_result", "tests/test_gpu_bit.py::test_long_arrays_and_views",
                "tests/test_gpu_bit.py::test_all_any_along_word_aligned_rows"])
+
+
+def test_table_operators_with_blocks_that_take_many_tiles():
+    """Operators that fill tables in LDS run a capped grid whose blocks take a tile after the other: with two blocks every
+    block loops wherever a launch has three tiles or more."""
+    run_child({"CUMO_HIP_EW_TABLE_BLOCKS": "2"},
+              ["tests/test_gpu_nmath_vectors.py", "tests/test_gpu_elementwise.py::test_nmath",
+               "tests/test_gpu_elementwise.py::test_dfloat_power_of_arrays_with_every_kind_of_argument",
+               "tests/test_gpu_adjacent.py::test_float_pow_parity"])
