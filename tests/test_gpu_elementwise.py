@@ -377,6 +377,47 @@ def test_nmath_two_args(tname, dt):
     assert_bits_equal(cls.cast(x).copysign(cls.cast(y)).to_numpy(), oracle.binary("copysign", x, y))
 
 
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_slices_whose_rows_are_not_whole_vectors(tname, dt):
+    """Functions of slices that drop a column (rows of an odd length that start anywhere), their differences, a slice and
+    a scalar, a slice and a row or column vector, three dimensions: the result is one run and every input is addressed
+    by row and column, a 128-bit load wherever a result vector lies inside one row."""
+    import cumo_amd
+    rng = np.random.default_rng(109)
+    cls = cls_of(tname)
+    if dt == np.int32:
+        h = rng.integers(-1000, 1000, size=(300, 260)).astype(dt)
+        h3 = rng.integers(-1000, 1000, size=(6, 50, 131)).astype(dt)
+    else:
+        h = rng.standard_normal((300, 260)).astype(dt)
+        h3 = rng.standard_normal((6, 50, 131)).astype(dt)
+    d, d3 = cls.cast(h), cls.cast(h3)
+    pairs = [(d[:, 1:], h[:, 1:]), (d[:, :-1], h[:, :-1]), (d[1:, 2:-1], h[1:, 2:-1]), (d[::2, 3:], h[::2, 3:]),
+             (d3[:, :, 1:], h3[:, :, 1:]), (d3[1:, ::2, :-2], h3[1:, ::2, :-2])]
+    for dv, hv in pairs:
+        what = "%r" % (hv.shape,)
+        assert_bits_equal((-dv).to_numpy(), oracle.unary("minus", hv), "minus " + what)
+        assert_bits_equal(dv.abs().to_numpy(), oracle.unary("abs", hv), "abs " + what)
+        assert_bits_equal((dv * 3).to_numpy(), oracle.binary("mul", hv, 3), "slice * scalar " + what)
+        assert_bits_equal((7 - dv).to_numpy(), oracle.binary("sub", 7, hv, scalar_is_left=True), "scalar - slice " + what)
+        assert_bits_equal(dv.copy().to_numpy(), hv, "copy " + what)
+        if dt != np.int32:
+            assert_ulp(cumo_amd.NMath.exp(dv).to_numpy(), oracle.unary("exp", hv), 1 if dt == np.float32 else 2, "exp " + what)
+            assert_ulp(cumo_amd.NMath.erfc(dv).to_numpy(), oracle.unary("erfc", hv), 1 if dt == np.float32 else 3, "erfc " + what)
+    # two slices of one array, a slice and a row vector, a slice and a column vector
+    assert_bits_equal((d[:, 1:] - d[:, :-1]).to_numpy(), oracle.binary("sub", h[:, 1:], h[:, :-1]), "difference along rows")
+    assert_bits_equal((d[1:, 1:] + d[:-1, :-1]).to_numpy(), oracle.binary("add", h[1:, 1:], h[:-1, :-1]), "diagonal neighbours")
+    assert_bits_equal((d3[:, :, 1:] - d3[:, :, :-1]).to_numpy(), oracle.binary("sub", h3[:, :, 1:], h3[:, :, :-1]), "three dimensions")
+    assert_bits_equal((d[:, 1:] + d[0:1, 1:]).to_numpy(), oracle.binary("add", h[:, 1:], h[0:1, 1:]), "slice + row vector")
+    assert_bits_equal((d[:, 1:] * d[:, 0:1]).to_numpy(), oracle.binary("mul", h[:, 1:], h[:, 0:1]), "slice * column vector")
+    if dt == np.int32:
+        # a rejected element (division by zero) in a slice: the flag is raised, the other elements are stored
+        z = h.copy()
+        z[5, 7] = 0
+        with pytest.raises(ZeroDivisionError):
+            (d[:, 1:] / cls.cast(z)[:, 1:]).to_numpy()
+
+
 def test_dfloat_power_of_arrays_with_every_kind_of_argument():
     """DFloat ** DFloat: positive normal bases with finite exponents take the library's own arithmetic (log2 of the base
     and its product with the exponent as pairs of doubles), every other argument the device library's pow. Both
