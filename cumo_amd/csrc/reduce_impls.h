@@ -108,6 +108,10 @@ struct SumImpl {
     static constexpr bool USES_INDEX = false;
     static constexpr int NOUT = 1;
     TA divisor;
+    // results have the input's type: a reduction may go through results of its own (rows first, then the rows' results),
+    // the division only at the end
+    static constexpr bool OWN_RESULTS = sizeof(T) == sizeof(TA);
+    SumImpl before_the_last() const { return SumImpl{(TA)0}; }
     __device__ __forceinline__ Acc identity() const { return PROD ? (TA)1 : (TA)0; }
     __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
         if (SKIP_NAN && isnan_t(x)) return;
@@ -439,6 +443,9 @@ struct ValueExtremeImpl {
     static constexpr bool USES_INDEX = false;
     static constexpr int NOUT = 1;
     static constexpr bool HAS_EXACT = is_float_t<T>::value;
+    // (rows first, then the rows' results: the zero that comes first in a row, then the row that comes first)
+    static constexpr bool OWN_RESULTS = true;
+    ValueExtremeImpl before_the_last() const { return *this; }
     static __device__ __forceinline__ float pick(float a, float b) { return IS_MAX ? __builtin_fmaxf(a, b) : __builtin_fminf(a, b); }
     static __device__ __forceinline__ double pick(double a, double b) { return IS_MAX ? __builtin_fmax(a, b) : __builtin_fmin(a, b); }
     static __device__ __forceinline__ int32_t pick(int32_t a, int32_t b) { return IS_MAX ? (a > b ? a : b) : (a < b ? a : b); }

@@ -862,6 +862,9 @@ static int red_stream_launch(const ReducePlan& plan, const cumo_na_reduction_arg
 // With `fixed` the partial results of a split reduction go to the caller's device memory
 // instead (fixed->ptr, fixed->bytes): nothing is allocated or released, and a reduction
 // whose partial results do not fit is refused (returns false, nothing launched).
+template <class I, class = void> struct reduces_own_results { static constexpr bool value = false; };
+template <class I> struct reduces_own_results<I, decltype((void)I::OWN_RESULTS)> { static constexpr bool value = I::OWN_RESULTS; };
+
 template <class Impl>
 static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarray_t* out2, Impl impl, int index_mode,
                           const RedScratch* fixed = nullptr) {
@@ -909,6 +912,52 @@ static bool reduce_launch(const cumo_na_reduction_arg_t* arg, const cumo_na_iarr
                 cumo_cuda_runtime_free(copy);
                 return done;
             }
+        }
+    }
+    // One result over a view whose rows run along memory but do not follow one another (x[true, 1..-1].sum): the rows
+    // first, each with the lanes of the row kernels, into a scratch vector, then the vector. Only where a result can
+    // stand in for the elements it came from. SFloat [8192,4095] of [8192,4096]: sum 55 -> 27 us.
+    if constexpr (reduces_own_results<Impl>::value) {
+        const int64_t es = (int64_t)sizeof(In);
+        const int nr = plan.red_ndim;
+        if (fixed == nullptr && out2 == nullptr && plan.out_total == 1 && nr >= 2 && nr <= CUMO_NA_MAX_DIMENSION && plan.in_red_step[nr - 1] == es &&
+            plan.red_shape[nr - 1] >= 64 && plan.red_total >= 65536) {
+            const uint64_t inner = plan.red_shape[nr - 1], rows = plan.red_total / inner;
+            char* partial = cumo_cuda_runtime_malloc(rows * sizeof(In));
+            if (!partial) return true;  // the pool has reported it
+            // the outer reduce dimensions are the first launch's output dimensions, their results one run
+            cumo_na_reduction_arg_t a1;
+            std::memset(&a1, 0, sizeof(a1));
+            a1.in.ptr = arg->in.ptr;
+            a1.out.ptr = partial;
+            ssize_t run = (ssize_t)es;
+            for (int d = nr - 2; d >= 0; --d) {
+                a1.in.step[d] = (ssize_t)plan.in_red_step[d];
+                a1.in_indexer.shape[d] = plan.red_shape[d];
+                a1.out.step[d] = run;
+                a1.out_indexer.shape[d] = plan.red_shape[d];
+                run *= (ssize_t)plan.red_shape[d];
+            }
+            a1.in.step[nr - 1] = (ssize_t)es;
+            a1.in_indexer.shape[nr - 1] = inner;
+            a1.in_indexer.ndim = (unsigned char)nr;
+            a1.in_indexer.total_size = rows * inner;
+            a1.out_indexer.ndim = (unsigned char)(nr - 1);
+            a1.out_indexer.total_size = rows;
+            reduce_launch(&a1, nullptr, impl.before_the_last(), index_mode);
+            cumo_na_reduction_arg_t a2;
+            std::memset(&a2, 0, sizeof(a2));
+            a2.in.ptr = partial;
+            a2.in.step[0] = (ssize_t)es;
+            a2.in_indexer.ndim = 1;
+            a2.in_indexer.shape[0] = rows;
+            a2.in_indexer.total_size = rows;
+            a2.out.ptr = arg->out.ptr;
+            a2.out_indexer.ndim = 0;
+            a2.out_indexer.total_size = 1;
+            const bool done = reduce_launch(&a2, nullptr, impl, index_mode);
+            cumo_cuda_runtime_free(partial);
+            return done;
         }
     }
     {

@@ -24,6 +24,11 @@ def cls_of(name):
     return {"sfloat": cumo_amd.SFloat, "dfloat": cumo_amd.DFloat, "int32": cumo_amd.Int32}[name]
 
 
+def host_value(r):
+    """A reduction's answer as a numpy array (a full reduction answers a number or an array of no dimensions)."""
+    return np.asarray(r.to_numpy() if hasattr(r, "to_numpy") else r)
+
+
 def red_n(shape, axis):
     if axis is None:
         return int(np.prod(shape))
@@ -135,6 +140,51 @@ def test_reductions_along_an_axis_that_strides_through_memory(tname, dt):
         got = dv.max_index(axis=axis)
         got = np.asarray(got.to_numpy() if hasattr(got, "to_numpy") else got)
         assert_bits_equal(got, np.asarray(oracle.reduce("max_index", hv, axis=axis)).astype(got.dtype), "max_index " + what)
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_one_result_over_views_whose_rows_do_not_follow_one_another(tname, dt):
+    """x[true, 1..-1].sum and its like: a full reduction over a view of 65536 elements or more whose innermost dimension
+    runs along memory while the outer ones do not merge with it goes rows first, then over the rows' results. Sums
+    within the reduction tolerance; min / max exactly, the zero that comes first in the view's order included."""
+    rng = np.random.default_rng(209)
+    cls = cls_of(tname)
+    if dt == np.int32:
+        h2 = rng.integers(-50, 50, size=(300, 260)).astype(dt)
+        h3 = rng.integers(-50, 50, size=(12, 50, 131)).astype(dt)
+    else:
+        h2 = (rng.integers(-8, 8, size=(300, 260)) / 4.0).astype(dt)
+        h3 = (rng.integers(-8, 8, size=(12, 50, 131)) / 4.0).astype(dt)
+    d2, d3 = cls.cast(h2), cls.cast(h3)
+    views = [(d2[:, 1:], h2[:, 1:]), (d2[::-1, :-3], h2[::-1, :-3]), (d3[:, :, 1:], h3[:, :, 1:]), (d3[::2, 1:, 2:-1], h3[::2, 1:, 2:-1]),
+             (d3.transpose(1, 0, 2)[:, :, 3:], h3.transpose(1, 0, 2)[:, :, 3:])]
+    for dv, hv in views:
+        hv = np.ascontiguousarray(hv)
+        what = "%r" % (hv.shape,)
+        n = hv.size
+        for name in ("min", "max"):
+            got = host_value(getattr(dv, name)())
+            assert_bits_equal(got.astype(dt), np.asarray(oracle.reduce(name, hv, axis=None), dtype=dt), "%s %s" % (name, what))
+        if dt != np.int32:
+            for name in ("sum", "mean"):
+                want = exact_reduce(name, hv, None)
+                got = host_value(getattr(dv, name)()).astype(np.float64)
+                scale = abs_sum(hv, None) / (n if name == "mean" else 1)
+                assert_reduction_close(got.astype(dt), want.astype(dt), n, scale, "%s %s" % (name, what))
+    if dt != np.int32:
+        # the zero that comes first: a matrix of zeros of both signs, seen through the slice
+        z = np.where(rng.random((300, 260)) < 0.5, dt(0.0), dt(-0.0)).astype(dt)
+        dz = cls.cast(z)
+        for dv, hv in ((dz[:, 1:], z[:, 1:]), (dz[::-1, 2:], z[::-1, 2:]), (dz[5:, :-1], z[5:, :-1])):
+            hv = np.ascontiguousarray(hv)
+            for name in ("min", "max"):
+                got = host_value(getattr(dv, name)()).astype(dt)
+                assert_bits_equal(got, np.asarray(oracle.reduce(name, hv, axis=None), dtype=dt), "%s of zeros %r" % (name, hv.shape))
+        hp = (1.0 + rng.uniform(-1, 1, size=(300, 260)) * 1e-4).astype(dt)
+        want = np.prod(hp[:, 1:].astype(np.longdouble))
+        got = host_value(cls.cast(hp)[:, 1:].prod()).astype(np.float64)
+        # (every multiplication rounds: n / 2 units in the last place at worst)
+        assert abs(float(got) / float(want) - 1.0) <= hp[:, 1:].size * np.finfo(dt).eps / 2, ("prod", float(got), float(want))
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
