@@ -953,6 +953,87 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_period_kernel(const char
     }
 }
 
+// The same with every input addressed by row and column (see ew_flat_addressed_kernel): a comparison of a slice whose
+// rows are not whole vectors with the scalar or with another slice (x[true, 1..-1] > x[true, 0..-2]; v[1..-1] > v[0..-2]
+// of one dimension is one row), the bits one run. These went element by element: SFloat [8192,4095] of [8192,4096]
+// `> 0` 100 us.
+template <class Op, int VEC, bool NT>
+__global__ __launch_bounds__(kEwBlock) void ew_flat_bit_addressed_kernel(EwAddressed p, CUMO_BIT_DIGIT* __restrict__ pz, int use_scalar, Op op,
+                                                                         typename Op::S sv) {
+    ew_op_prepare<Op>();
+    typedef typename Op::A A;
+    typedef typename Op::B B;
+    constexpr bool TWO = Op::NIN == 2;
+    constexpr int UNR = 4;
+    constexpr unsigned G = 32 / VEC;
+    const uint32_t lane = blockIdx.x * (uint32_t)kEwBlock + threadIdx.x;
+    const uint32_t group = lane / G;
+    const unsigned k = lane % G;
+    const uint64_t first64 = (uint64_t)group * (32 * UNR);  // the group's first element
+    if (first64 >= p.n) return;
+    const uint32_t e0 = (uint32_t)first64 + k * VEC;
+    const bool two_arrays = TWO && use_scalar == 0;
+    if (first64 + 32 * UNR <= p.n) {
+        A xv[UNR][VEC];
+        B yv[UNR][VEC];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const uint32_t e = e0 + 32 * u;
+            const uint32_t q = div31(e, p.div);
+            const uint32_t r = e - q * p.period;
+            const bool inside = r + VEC <= p.period;
+            ew_addressed_fetch<A, VEC>(p, 0, q, r, (uint32_t)VEC, inside, xv[u]);
+            if (two_arrays) {
+                ew_addressed_fetch<B, VEC>(p, 1, q, r, (uint32_t)VEC, inside, yv[u]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) yv[u][j] = B();
+            }
+        }
+        uint32_t words[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            uint32_t bits = 0;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                A x = xv[u][j];
+                B y = yv[u][j];
+                if (TWO) {
+                    if (use_scalar == 1) y = (B)sv;
+                    else if (use_scalar == 2) { y = (B)x; x = (A)sv; }
+                }
+                uint32_t z = 0;
+                op(x, y, z);
+                bits |= (z ? 1u : 0u) << j;
+            }
+            words[u] = ew_gather_word<VEC>(bits);
+        }
+        if (k == 0) *reinterpret_cast<u32x4*>(pz + (size_t)group * UNR) = u32x4{words[0], words[1], words[2], words[3]};
+        return;
+    }
+    // the ragged end: at most 32 * UNR - 1 elements in the whole launch
+    for (int u = 0; u < UNR; ++u) {
+        for (int j = 0; j < VEC; ++j) {
+            const uint64_t e = (uint64_t)e0 + 32 * u + j;
+            if (e >= p.n) continue;
+            const uint32_t q = div31((uint32_t)e, p.div);
+            const uint32_t r = (uint32_t)e - q * p.period;
+            A x = *reinterpret_cast<const A*>(p.in[0] + ew_addressed_row(p, 0, q) + (int64_t)r * p.s_inner[0]);
+            B y = B();
+            if (two_arrays) y = *reinterpret_cast<const B*>(p.in[1] + ew_addressed_row(p, 1, q) + (int64_t)r * p.s_inner[1]);
+            if (TWO) {
+                if (use_scalar == 1) y = (B)sv;
+                else if (use_scalar == 2) { y = (B)x; x = (A)sv; }
+            }
+            uint32_t z = 0;
+            op(x, y, z);
+            const uint32_t bit = 1u << (e & 31);
+            if (z) atomicOr(&pz[e >> 5], bit);
+            else atomicAnd(&pz[e >> 5], ~bit);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Two-dimensional kernel for typed results: rows x inner, every operand either
 // walks the inner dimension contiguously or is constant along it (a column
@@ -1968,6 +2049,50 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                             const dim3 g((unsigned)pblocks);
                             if (nt) hipLaunchKernelGGL((ew_flat_bit_period_kernel<Op, VB, true>), g, b, 0, stream, kp.ptr[full], kp.ptr[per], dst, total, pr, op);
                             else hipLaunchKernelGGL((ew_flat_bit_period_kernel<Op, VB, false>), g, b, 0, stream, kp.ptr[full], kp.ptr[per], dst, total, pr, op);
+                            cumo_cuda_runtime_check_kernel_launch();
+                            return;
+                        }
+                    }
+                }
+            }
+            // every input addressed by row and column, the bits one run (comparisons of slices whose rows are not whole
+            // vectors, with one another or with the scalar; one dimension is one row)
+            if constexpr (Op::NIN == 1 || (Op::NIN == 2 && std::is_same<A, B>::value)) {
+                const int ob = nops - 1;
+                bool bits_one_run = n <= 3 && plan.step[ob][n - 1] == 1;
+                if (n >= 2) bits_one_run = bits_one_run && plan.step[ob][n - 2] == (int64_t)kp.inner;
+                if (n == 3) bits_one_run = bits_one_run && plan.step[ob][0] == (int64_t)kp.inner * (int64_t)plan.shape[1];
+                if (bits_one_run && vec == 1 && !force_scalar && !force_wide_indices() && plan.total < 0x7fffffffull && plan.total >= 16384 &&
+                    kp.inner >= 64 && (out_bit->pos % 128) == 0 && ((uintptr_t)out_bit->ptr % 16) == 0) {
+                    const int64_t es = (int64_t)sizeof(A);
+                    bool fits = true;
+                    for (int o = 0; o + 1 < nops && fits; ++o) {
+                        const int sl = slot[o];
+                        fits = (kp.istep[sl] == es || kp.istep[sl] == 0) && ((uintptr_t)kp.ptr[sl] % (uintptr_t)es) == 0;
+                    }
+                    if (fits) {
+                        EwAddressed pa;
+                        std::memset(&pa, 0, sizeof(pa));
+                        for (int o = 0; o + 1 < nops; ++o) {
+                            const int sl = slot[o];
+                            pa.in[sl] = kp.ptr[sl];
+                            pa.s_outer[sl] = n >= 2 ? kp.ostep[sl][n - 2] : 0;
+                            pa.s_inner[sl] = kp.istep[sl];
+                            pa.s_outermost[sl] = n == 3 ? kp.ostep[sl][0] : 0;
+                        }
+                        pa.n = (uint32_t)plan.total;
+                        pa.period = (uint32_t)kp.inner;
+                        pa.div = div31_make(pa.period);
+                        pa.mid = n == 3 ? (uint32_t)plan.shape[1] : 0u;
+                        pa.div_mid = div31_make(n == 3 ? (uint32_t)plan.shape[1] : 1u);
+                        const uint64_t pgroups = ((uint64_t)pa.n + 127) / 128;
+                        const uint64_t pblocks = (pgroups * (32 / VB) + kEwBlock - 1) / kEwBlock;
+                        if (pblocks <= ew_grid_max()) {
+                            const bool nt = stream_past_caches((uint64_t)pa.n * sizeof(A) * (uint64_t)(nops - 1));
+                            CUMO_BIT_DIGIT* dst = reinterpret_cast<CUMO_BIT_DIGIT*>(const_cast<char*>(ops[nops - 1].ptr)) + out_bit->pos / 32;
+                            const dim3 g((unsigned)pblocks);
+                            if (nt) hipLaunchKernelGGL((ew_flat_bit_addressed_kernel<Op, VB, true>), g, b, 0, stream, pa, dst, use_scalar, op, sv);
+                            else hipLaunchKernelGGL((ew_flat_bit_addressed_kernel<Op, VB, false>), g, b, 0, stream, pa, dst, use_scalar, op, sv);
                             cumo_cuda_runtime_check_kernel_launch();
                             return;
                         }

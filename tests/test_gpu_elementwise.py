@@ -410,6 +410,21 @@ def test_slices_whose_rows_are_not_whole_vectors(tname, dt):
     assert_bits_equal((d3[:, :, 1:] - d3[:, :, :-1]).to_numpy(), oracle.binary("sub", h3[:, :, 1:], h3[:, :, :-1]), "three dimensions")
     assert_bits_equal((d[:, 1:] + d[0:1, 1:]).to_numpy(), oracle.binary("add", h[:, 1:], h[0:1, 1:]), "slice + row vector")
     assert_bits_equal((d[:, 1:] * d[:, 0:1]).to_numpy(), oracle.binary("mul", h[:, 1:], h[:, 0:1]), "slice * column vector")
+    # comparisons into Bit: the bits are one run, every input is addressed
+    v = (rng.integers(-3, 3, size=70001)).astype(dt)
+    dv1 = cls.cast(v)
+    for dx, hx, dy, hy, what in ((d[:, 1:], h[:, 1:], d[:, :-1], h[:, :-1], "two slices"), (dv1[1:], v[1:], dv1[:-1], v[:-1], "one dimension"),
+                                 (d3[:, :, 1:], h3[:, :, 1:], d3[:, :, :-1], h3[:, :, :-1], "three dimensions"),
+                                 (d[:, 1:], h[:, 1:], d[0:1, 1:], h[0:1, 1:], "slice against row vector")):
+        assert_bits_equal((dx > dy).to_numpy(), (hx > hy).astype(np.uint8), "gt " + what)
+        assert_bits_equal(dx.eq(dy).to_numpy(), (hx == hy).astype(np.uint8), "eq " + what)
+        assert_bits_equal((dx <= dy).to_numpy(), (hx <= hy).astype(np.uint8), "le " + what)
+        assert_bits_equal((dx > 0).to_numpy(), (hx > 0).astype(np.uint8), "gt scalar " + what)
+        assert_bits_equal(dx.ne(1).to_numpy(), (hx != 1).astype(np.uint8), "ne scalar " + what)
+    if dt != np.int32:
+        hn = h.copy()
+        hn[rng.random(h.shape) < 0.1] = np.nan
+        assert_bits_equal(cls.cast(hn)[:, 1:].isnan().to_numpy(), np.isnan(hn[:, 1:]).astype(np.uint8), "isnan of a slice")
     if dt == np.int32:
         # a rejected element (division by zero) in a slice: the flag is raised, the other elements are stored
         z = h.copy()
