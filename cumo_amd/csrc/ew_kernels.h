@@ -2147,14 +2147,15 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
 
     // A result that is one run of rows that are not whole vectors, every input a two-dimensional view that runs along
     // its rows or is constant along them (see ew_flat_addressed_kernel): what would otherwise go element by element.
-    if constexpr (!Op::BIT_OUT && (Op::NIN == 1 || (Op::NIN == 2 && std::is_same<A, B>::value)) && sizeof(A) == sizeof(R) &&
+    // (a result of another width than the inputs, a cast, too: the lane's vector is the result's)
+    if constexpr (!Op::BIT_OUT && (Op::NIN == 1 || (Op::NIN == 2 && std::is_same<A, B>::value)) && (sizeof(R) == 4 || sizeof(R) == 8) &&
                   (sizeof(A) == 4 || sizeof(A) == 8)) {
-        constexpr int V = 16 / (int)sizeof(A);
+        constexpr int V = 16 / (int)sizeof(R);
         if ((n == 2 || n == 3) && lean_vec == 1 && !force_scalar && !force_wide_indices() && (kp.inner % V) != 0 && kp.inner >= 64 &&
             plan.total < 0x7fffffffull && plan.total >= 16384) {
-            const int64_t es = (int64_t)sizeof(A);
-            bool fits = kp.istep[2] == es && kp.ostep[2][n - 2] == es * (int64_t)kp.inner && ((uintptr_t)kp.ptr[2] % 16) == 0;
-            if (n == 3) fits = fits && kp.ostep[2][0] == es * (int64_t)kp.inner * (int64_t)plan.shape[1];
+            const int64_t es = (int64_t)sizeof(A), rs = (int64_t)sizeof(R);
+            bool fits = kp.istep[2] == rs && kp.ostep[2][n - 2] == rs * (int64_t)kp.inner && ((uintptr_t)kp.ptr[2] % 16) == 0;
+            if (n == 3) fits = fits && kp.ostep[2][0] == rs * (int64_t)kp.inner * (int64_t)plan.shape[1];
             for (int o = 0; o + 1 < nops && fits; ++o) {
                 const int sl = slot[o];
                 fits = (kp.istep[sl] == es || kp.istep[sl] == 0) && ((uintptr_t)kp.ptr[sl] % (uintptr_t)es) == 0;
@@ -2177,7 +2178,7 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 pa.div_mid = div31_make(n == 3 ? (uint32_t)plan.shape[1] : 1u);
                 const uint64_t blocks = ((uint64_t)pa.n + (uint64_t)kEwBlock * V - 1) / ((uint64_t)kEwBlock * V);
                 if (blocks <= ew_grid_max()) {
-                    const bool nt = stream_past_caches((uint64_t)nops * pa.n * sizeof(A));
+                    const bool nt = stream_past_caches((uint64_t)pa.n * ((uint64_t)(nops - 1) * sizeof(A) + sizeof(R)));
                     const dim3 g((unsigned)blocks);
                     if (nt) hipLaunchKernelGGL((ew_flat_addressed_kernel<Op, V, true>), g, b, 0, stream, pa, use_scalar, flag, op, sv);
                     else hipLaunchKernelGGL((ew_flat_addressed_kernel<Op, V, false>), g, b, 0, stream, pa, use_scalar, flag, op, sv);

@@ -410,6 +410,15 @@ def test_slices_whose_rows_are_not_whole_vectors(tname, dt):
     assert_bits_equal((d3[:, :, 1:] - d3[:, :, :-1]).to_numpy(), oracle.binary("sub", h3[:, :, 1:], h3[:, :, :-1]), "three dimensions")
     assert_bits_equal((d[:, 1:] + d[0:1, 1:]).to_numpy(), oracle.binary("add", h[:, 1:], h[0:1, 1:]), "slice + row vector")
     assert_bits_equal((d[:, 1:] * d[:, 0:1]).to_numpy(), oracle.binary("mul", h[:, 1:], h[:, 0:1]), "slice * column vector")
+    # casts of slices: the result's vectors are whole, the input's elements of another width
+    import cumo_amd
+    for target, tdt in ((cumo_amd.DFloat, np.float64), (cumo_amd.SFloat, np.float32), (cumo_amd.Int32, np.int32)):
+        if tdt == dt:
+            continue
+        src = h if dt == np.int32 or tdt != np.int32 else np.trunc(h * 10).astype(dt)
+        dsrc = cls.cast(src)
+        assert_bits_equal(target.cast(dsrc[:, 1:]).to_numpy(), src[:, 1:].astype(tdt), "cast of a slice to %s" % tdt.__name__)
+        assert_bits_equal(target.cast(dsrc[::2, 2:-1]).to_numpy(), src[::2, 2:-1].astype(tdt), "cast of a slice to %s" % tdt.__name__)
     # comparisons into Bit: the bits are one run, every input is addressed
     v = (rng.integers(-3, 3, size=70001)).astype(dt)
     dv1 = cls.cast(v)
