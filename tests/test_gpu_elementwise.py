@@ -392,7 +392,7 @@ def test_slices_whose_rows_are_not_whole_vectors(tname, dt):
         h = rng.standard_normal((300, 260)).astype(dt)
         h3 = rng.standard_normal((6, 50, 131)).astype(dt)
     d, d3 = cls.cast(h), cls.cast(h3)
-    pairs = [(d[:, 1:], h[:, 1:]), (d[:, :-1], h[:, :-1]), (d[1:, 2:-1], h[1:, 2:-1]), (d[::2, 3:], h[::2, 3:]),
+    pairs = [(d[:, 1:], h[:, 1:]), (d[:, :-1], h[:, :-1]), (d[1:, 2:-1], h[1:, 2:-1]), (d[::2, 3:], h[::2, 3:]), (d[::-1, 1:], h[::-1, 1:]),
              (d3[:, :, 1:], h3[:, :, 1:]), (d3[1:, ::2, :-2], h3[1:, ::2, :-2])]
     for dv, hv in pairs:
         what = "%r" % (hv.shape,)
