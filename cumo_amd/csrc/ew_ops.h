@@ -130,8 +130,7 @@ CUMO_HIP_FBIN(OpMul, x * y)
 CUMO_HIP_FBIN(OpDiv, x / y)
 CUMO_HIP_FBIN(OpFMod, fmod((double)x, (double)y))
 CUMO_HIP_FBIN(OpCopysign, copysign((double)x, (double)y))
-CUMO_HIP_FBIN(OpAtan2, atan2((double)x, (double)y))
-CUMO_HIP_FBIN(OpHypot, hypot((double)x, (double)y))
+// (OpAtan2 and OpHypot: further down, beside the cores they share with atan)
 // the second operand arrives in the float type and converts to int (types/float_macro_kernel.h:122)
 CUMO_HIP_FBIN(OpLdexp, ldexp((double)x, (int)y))
 
@@ -671,6 +670,65 @@ CUMO_HIP_TRIG_OP(OpTan, 2, tan((double)x))
 CUMO_HIP_OWN_OP(OpAsin, asin_acos_float_rounded_once<false>, asin((double)x))
 CUMO_HIP_OWN_OP(OpAcos, asin_acos_float_rounded_once<true>, acos((double)x))
 CUMO_HIP_OWN_OP(OpAtan, atan_float_rounded_once, atan((double)x))
+// SFloat atan2(y, x) for finite arguments that are not zero, with atan's polynomial: the quotient's reduction is done on
+// numerator and denominator (t = |y| / |x| up to tan(pi/8), (|y| - |x|) / (|y| + |x|) plus pi/4 up to tan(3 pi/8),
+// -|x| / |y| plus pi/2 above; the sums are exact or good to 2^-53 in double), pi minus that for a negative x, y's sign.
+// Every other argument (a zero, an infinity, a NaN: the rules about signs and quadrants) is the device library's atan2.
+// (reference: types/float_macro_kernel.h m_atan2 -> atan2)
+__device__ __attribute__((noinline)) float atan2_by_the_library(float yf, float xf) { return (float)atan2((double)yf, (double)xf); }
+__device__ __forceinline__ float atan2_fast(float yf, float xf) {
+    const double ay = (double)__builtin_fabsf(yf), ax = (double)__builtin_fabsf(xf);
+    const bool mid = ay > 0.41421356237309503 * ax, top = ay > 2.4142135623730951 * ax;
+    const double num = top ? -ax : (mid ? ay - ax : ay);
+    const double den = top ? ay : (mid ? ay + ax : ax);
+    const double off = top ? 1.57079632679489655800e+00 : (mid ? 7.85398163397448278999e-01 : 0.0);
+    const double t = num * rcp_refined(den);
+    const double z = t * t;
+    double p = 0.033038827515269494;
+    p = __builtin_fma(p, z, -0.06032248119994454);
+    p = __builtin_fma(p, z, 0.07605969344616582);
+    p = __builtin_fma(p, z, -0.09084239163280672);
+    p = __builtin_fma(p, z, 0.11110827992295265);
+    p = __builtin_fma(p, z, -0.1428570834807845);
+    p = __builtin_fma(p, z, 0.19999999952417688);
+    p = __builtin_fma(p, z, -0.33333333333270726);
+    double r = off + __builtin_fma(t * z, p, t);
+    r = (xf < 0.0f) ? 3.14159265358979311600e+00 - r : r;
+    return __builtin_copysignf((float)r, yf);
+}
+// (finite and not zero, both)
+__device__ __forceinline__ bool atan2_is_rare(float yf, float xf) {
+    return !(__float_as_uint(__builtin_fabsf(yf)) - 1u < 0x7f7fffffu && __float_as_uint(__builtin_fabsf(xf)) - 1u < 0x7f7fffffu);
+}
+__device__ __forceinline__ float atan2_float_rounded_once(float yf, float xf) {
+    float z = atan2_fast(yf, xf);
+    if (atan2_is_rare(yf, xf)) z = atan2_by_the_library(yf, xf);
+    return z;
+}
+template <class T> struct OpAtan2 { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) static constexpr bool HEAVY = true;
+    static constexpr bool HAS_RARE = sizeof(T) == 4;
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)atan2_float_rounded_once((float)x, (float)y);
+        else z = (T)atan2((double)x, (double)y);
+        return true; }
+    __device__ __forceinline__ void fast(T x, T y, T& z) const { z = (T)atan2_fast((float)x, (float)y); }
+    __device__ __forceinline__ bool rare(T x, T y) const { return atan2_is_rare((float)x, (float)y); }
+    __device__ __forceinline__ T slow(T x, T y) const { return (T)atan2_by_the_library((float)x, (float)y); } };
+// SFloat hypot: x^2 + y^2 cannot leave the double range and is good to 2^-53 there; one refined square root. An
+// infinity on either side answers infinity, whatever the other is (types/float_macro_kernel.h m_hypot -> hypot).
+__device__ __forceinline__ float hypot_float_rounded_once(float xf, float yf) {
+    const double x = (double)xf, y = (double)yf;
+    const double s = __builtin_fma(x, x, y * y);
+    float r = (float)sqrt_refined((s > 0.0) ? s : 1.0);
+    r = (s == 0.0) ? 0.0f : r;
+    r = (s != s) ? (float)s : r;
+    return (__builtin_fabsf(xf) == INFINITY || __builtin_fabsf(yf) == INFINITY) ? INFINITY : r;
+}
+template <class T> struct OpHypot { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)hypot_float_rounded_once((float)x, (float)y);
+        else z = (T)hypot((double)x, (double)y);
+        return true; } };
 // (DFloat: the cores of dd_cores.h, which read the table of the power's logarithm)
 #define CUMO_HIP_OWN_OP_WITH_TABLES(NAME, FEXPR, DEXPR)                                                                     \
     template <class T> struct NAME { CUMO_HIP_OP_COMMON(T, T, T, 1, false, false) static constexpr bool HEAVY = true;       \

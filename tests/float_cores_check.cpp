@@ -12,6 +12,7 @@
 //                                      cosh erfc log1p asinh acosh atanh) against the long double function; prints, per
 //                                      function, arguments tried, the largest error in ulps and where it was
 //   float_cores_check dpow <n>         n random (base, exponent) pairs through the DFloat power's arithmetic against powl
+//   float_cores_check two <n>          n random pairs through the SFloat atan2 and hypot against (float)glibc in double
 //   float_cores_check sweep <stride>   every stride-th float bit pattern through each SFloat
 //                                      core against (float)glibc((double)x); prints, per
 //                                      function, patterns tried, mismatches and the largest
@@ -125,6 +126,52 @@ int main(int argc, char** argv) {
                 if (err > worst) { worst = err; worst_x = x; }
             }
             std::printf("%s %llu %.4f %a\n", c.name, (unsigned long long)n, worst, worst_x);
+        }
+        return 0;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "two") == 0) {
+        // n random pairs of floats through the SFloat atan2 (finite arguments that are not zero: the others are the
+        // library's) and hypot (every argument) against (float)glibc((double)., (double).): magnitudes spread over every
+        // float exponent, over neighbouring exponents (where the quotient's reduction changes form), and special values
+        // for hypot; prints, per function, pairs tried, mismatches and the largest difference in ulps
+        const uint64_t n = std::strtoull(argv[2], nullptr, 10);
+        for (int which = 0; which < 2; ++which) {
+            uint64_t state = 0x9e3779b97f4a7c15ull, tried = 0, bad = 0;
+            int64_t worst = 0;
+            auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+            const uint32_t special[] = {0u, 0x80000000u, 0x7f800000u, 0xff800000u, 0x7fc00000u, 1u, 0x007fffffu, 0x7f7fffffu, 0x3f800000u};
+            for (uint64_t it = 0; it < n; ++it) {
+                const uint64_t a = next(), b = next();
+                uint32_t ux = (uint32_t)a, uy = (uint32_t)b;
+                if (it % 2 == 1) {
+                    // exponents within two of each other
+                    const uint32_t ex = (ux >> 23) & 0xffu;
+                    const uint32_t ey = (uint32_t)((int)ex + (int)((b >> 40) % 5) - 2) & 0xffu;
+                    uy = (uy & 0x807fffffu) | (ey << 23);
+                }
+                if (which == 1 && it % 97 == 0) ux = special[(a >> 33) % 9];
+                if (which == 1 && it % 89 == 0) uy = special[(b >> 33) % 9];
+                float x, y; std::memcpy(&x, &ux, 4); std::memcpy(&y, &uy, 4);
+                float got, want;
+                if (which == 0) {
+                    if (atan2_is_rare(y, x)) continue;
+                    got = atan2_fast(y, x);
+                    want = (float)std::atan2((double)y, (double)x);
+                } else {
+                    got = hypot_float_rounded_once(x, y);
+                    want = (float)std::hypot((double)x, (double)y);
+                }
+                ++tried;
+                if (got != got && want != want) continue;
+                uint32_t gu, wu; std::memcpy(&gu, &got, 4); std::memcpy(&wu, &want, 4);
+                if (gu == wu) continue;
+                ++bad;
+                if (got != got || want != want) { worst = 1 << 30; continue; }
+                int64_t d = ordered(got) - ordered(want);
+                if (d < 0) d = -d;
+                if (d > worst) worst = d;
+            }
+            std::printf("%s %llu %llu %lld\n", which == 0 ? "atan2" : "hypot", (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
         }
         return 0;
     }

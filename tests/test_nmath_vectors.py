@@ -147,6 +147,16 @@ def test_device_dfloat_algorithms_on_pairs_against_long_double(cores):
         assert int(tried) == n and float(worst) <= (0.8 if name == "erfc" else 0.52), line
 
 
+def test_device_sfloat_atan2_and_hypot_against_glibc_in_double(cores):
+    n = 500000000 if os.environ.get("CUMO_EXHAUSTIVE") else 5000000
+    out = subprocess.run([cores, "two", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
+    assert [line.split()[0] for line in out] == ["atan2", "hypot"]
+    for line in out:
+        name, tried, bad, worst = line.split()
+        # evaluated in double to 2^-43 and rounded once: the rare argument next to a rounding boundary may differ by an ulp
+        assert int(tried) >= n * 9 // 10 and int(bad) <= int(tried) >> 17 and int(worst) <= 1, line
+
+
 def test_device_dfloat_power_against_long_double(cores):
     """x ** y of DFloat for a positive normal base and a finite exponent: log2 x and y log2 x as pairs of doubles."""
     n = 300000000 if os.environ.get("CUMO_EXHAUSTIVE") else 3000000
