@@ -3,7 +3,9 @@
 // n / d = (n * M) >> (31 + s) for every n < 2^31 (Granlund and Montgomery, "Division
 // by invariant integers using multiplication", with N = 31).
 #pragma once
+#ifndef CUMO_HIP_HOST_CHECK  // (a CPU build of the element functions defines the qualifiers away)
 #include <hip/hip_runtime.h>
+#endif
 
 #include <cstdint>
 

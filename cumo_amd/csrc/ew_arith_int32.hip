@@ -26,8 +26,28 @@ using namespace cumo_hip;
 CUMO_DEF_BINARY(add, OpIAdd)
 CUMO_DEF_BINARY(sub, OpISub)
 CUMO_DEF_BINARY(mul, OpIMul)
-CUMO_DEF_BINARY(div, OpIDiv)
-CUMO_DEF_BINARY(mod, OpIMod)
+// div, mod: the array forms and the form with the scalar on the left as the others; an array by one divisor that is not
+// zero goes by multiplication (OpIDivBy), nothing there can be rejected
+#define CUMO_DEF_DIVISION(name, OP, OPBY)                                                                            \
+    extern "C" void cumo_iter_int32_##name##_kernel_launch(cumo_na_iarray_t* a1, cumo_na_iarray_t* a2,               \
+                                                           cumo_na_iarray_t* a3, cumo_na_indexer_t* indexer,         \
+                                                           int* divzero) {                                           \
+        ew_launch(OP{}, a1, a2, a3, nullptr, indexer, (int32_t)0, 0, divzero);                                       \
+    }                                                                                                                \
+    extern "C" void cumo_iter_int32_##name##_s_kernel_launch(cumo_na_iarray_t* a1, int32_t sv, cumo_na_iarray_t* a3, \
+                                                             cumo_na_indexer_t* indexer, int* divzero,               \
+                                                             int scalar_is_left) {                                   \
+        if (!scalar_is_left && sv != 0) {                                                                            \
+            OPBY op;                                                                                                 \
+            op.d = sv;                                                                                               \
+            op.magic = div31_make(sv < 0 ? 0u - (uint32_t)sv : (uint32_t)sv);                                        \
+            ew_launch(op, a1, nullptr, a3, nullptr, indexer, (int32_t)0, 0, nullptr);                                \
+            return;                                                                                                  \
+        }                                                                                                            \
+        ew_launch(OP{}, a1, nullptr, a3, nullptr, indexer, sv, scalar_is_left ? 2 : 1, divzero);                     \
+    }
+CUMO_DEF_DIVISION(div, OpIDiv, OpIDivBy)
+CUMO_DEF_DIVISION(mod, OpIMod, OpIModBy)
 CUMO_DEF_BINARY(bit_and, OpIAnd)
 CUMO_DEF_BINARY(bit_or, OpIOr)
 CUMO_DEF_BINARY(bit_xor, OpIXor)

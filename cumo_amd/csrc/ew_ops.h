@@ -19,6 +19,8 @@
 #include <stdint.h>
 #include <float.h>
 
+#include "div31.h"
+
 namespace cumo_hip {
 
 // 1 / x to about one ulp (v_rcp_f32); only used where that is more than enough
@@ -158,6 +160,24 @@ struct OpIMod { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 2, false, true)
     __device__ __forceinline__ bool operator()(int32_t x, int32_t y, int32_t& z) const {
         if (y == 0) return false;
         z = (y == -1) ? 0 : x % y;
+        return true; } };
+
+// Division and remainder by one divisor for the whole launch (array / 7, array % 7), the divisor neither 0 nor the
+// element being rejected: the quotient of the magnitudes by a multiplication and a shift (div31.h: exact up to 2^31,
+// which is the magnitude of the smallest Int32), the sign put back; the remainder from the quotient. Truncating, as
+// the C operators the reference's macros use (types/int_macro_kernel.h m_div, m_mod); every result wraps like theirs.
+struct OpIDivBy { CUMO_HIP_OP_COMMON(int32_t, int32_t, int32_t, 1, false, false)
+    Div31 magic;
+    int32_t d;
+    __device__ __forceinline__ uint32_t quotient(int32_t x) const {
+        const uint32_t ax = x < 0 ? 0u - (uint32_t)x : (uint32_t)x;
+        const uint32_t q = div31(ax, magic);
+        return ((x ^ d) < 0) ? 0u - q : q;
+    }
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t, int32_t& z) const { z = (int32_t)quotient(x); return true; } };
+struct OpIModBy : OpIDivBy {
+    __device__ __forceinline__ bool operator()(int32_t x, int32_t, int32_t& z) const {
+        z = (int32_t)((uint32_t)x - quotient(x) * (uint32_t)d);
         return true; } };
 
 // ---- unary -----------------------------------------------------------------

@@ -1030,8 +1030,9 @@ int cumo_hip_na_binary_s(const char* op, const cumo_hip_narray_t* x, double sv, 
     if (rc) return rc;
     const BinaryRow* row = find_row(kBinary, op);
     if (!row || !binary_has(row, x->type, true)) return no_method(op);
-    BinaryOpt opt = {row, x->type, true, sv, scalar_is_left ? 1 : 0,
-                     x->type == CUMO_HIP_INT32 && (!std::strcmp(op, "div") || !std::strcmp(op, "mod")), false};
+    // (an Int32 array divided by one divisor that is not zero rejects nothing: no flag, and no wait for it)
+    const bool divides = x->type == CUMO_HIP_INT32 && (!std::strcmp(op, "div") || !std::strcmp(op, "mod"));
+    BinaryOpt opt = {row, x->type, true, sv, scalar_is_left ? 1 : 0, divides && (scalar_is_left || (int32_t)sv == 0), false};
     cumo_hip_ndfunc_t nf = {iter_binary, 0, 1, 1, {x->type, 0}};
     const NA* in[1] = {x};
     NA* out[1] = {z};

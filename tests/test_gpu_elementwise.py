@@ -517,6 +517,27 @@ def test_int32_arithmetic():
     assert_bits_equal(r.to_numpy(), hx.astype(np.float64) * 0.5)
 
 
+def test_int32_division_and_remainder_by_one_divisor():
+    """array / d and array % d with one divisor for the whole launch go by multiplication and shift: every divisor
+    kind (small, powers of two and their neighbours, the extremes, negative), dividends next to multiples and at the
+    ends of the range; truncating, wrapping where C's would overflow; views; a zero divisor still raises."""
+    import cumo_amd
+    rng = np.random.default_rng(110)
+    x = rng.integers(-2**31, 2**31, size=(257, 129), dtype=np.int64).astype(np.int32)
+    x.flat[:6] = [0, 1, -1, 2**31 - 1, -2**31, -2**31 + 1]
+    dx = cumo_amd.Int32.cast(x)
+    for d in (1, -1, 2, -2, 3, 7, -7, 10, 255, 256, 257, 65536, 1000003, 2**30 - 1, 2**30, 2**30 + 1, 2**31 - 2, 2**31 - 1, -2**31, -2**31 + 1):
+        near = (np.arange(-30, 30, dtype=np.int64)[:, None] * d + np.arange(-1, 2)[None, :]).reshape(-1)
+        near = near[(near >= -2**31) & (near < 2**31)].astype(np.int32)
+        for h, dv in ((x, dx), (near, cumo_amd.Int32.cast(near)), (x[::2, 1:], dx[::2, 1:]), (x.T, dx.transpose())):
+            assert_bits_equal((dv / d).to_numpy(), oracle.binary("div", h, d), "div by %d" % d)
+            assert_bits_equal((dv % d).to_numpy(), oracle.binary("mod", h, d), "mod by %d" % d)
+    with pytest.raises(ZeroDivisionError):
+        (dx / 0).to_numpy()
+    with pytest.raises(ZeroDivisionError):
+        (dx % 0).to_numpy()
+
+
 def test_int32_error_flags():
     # reference: test/narray_test.rb:4887-4905 -- the flag raises, also through views,
     # and the rejected element is left alone
