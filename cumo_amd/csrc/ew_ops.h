@@ -130,7 +130,7 @@ CUMO_HIP_FBIN(OpAdd, x + y)
 CUMO_HIP_FBIN(OpSub, x - y)
 CUMO_HIP_FBIN(OpMul, x * y)
 CUMO_HIP_FBIN(OpDiv, x / y)
-CUMO_HIP_FBIN(OpFMod, fmod((double)x, (double)y))
+// (OpFMod: further down, with its SFloat core)
 CUMO_HIP_FBIN(OpCopysign, copysign((double)x, (double)y))
 // (OpAtan2 and OpHypot: further down, beside the cores they share with atan)
 // the second operand arrives in the float type and converts to int (types/float_macro_kernel.h:122)
@@ -734,6 +734,38 @@ template <class T> struct OpAtan2 { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
     __device__ __forceinline__ void fast(T x, T y, T& z) const { z = (T)atan2_fast((float)x, (float)y); }
     __device__ __forceinline__ bool rare(T x, T y) const { return atan2_is_rare((float)x, (float)y); }
     __device__ __forceinline__ T slow(T x, T y) const { return (T)atan2_by_the_library((float)x, (float)y); } };
+// SFloat remainder x % y (the C fmod: the sign of x, exact) where the quotient stays below 2^29: its integer part from
+// a refined reciprocal (off by one at most, next to a whole number), taken off in one multiply-add, which is exact there
+// (29 + 24 bits), and put right by one addition or subtraction of |y|. Larger quotients, a zero divisor, infinities and
+// NaN are the device library's fmod (reference: types/float_macro_kernel.h m_mod -> fmod).
+__device__ __attribute__((noinline)) float fmod_by_the_library(float xf, float yf) { return (float)fmod((double)xf, (double)yf); }
+__device__ __forceinline__ float fmod_fast(float xf, float yf) {
+    const double ax = (double)__builtin_fabsf(xf), ay = (double)__builtin_fabsf(yf);
+    const double q = __builtin_trunc(ax * rcp_refined(ay));
+    double r = __builtin_fma(-q, ay, ax);
+    r = (r < 0.0) ? r + ay : r;
+    r = (r >= ay) ? r - ay : r;
+    return __builtin_copysignf((float)r, xf);
+}
+__device__ __forceinline__ bool fmod_is_rare(float xf, float yf) {
+    const float ax = __builtin_fabsf(xf), ay = __builtin_fabsf(yf);
+    // (false for a NaN on either side, a zero or infinite divisor, an infinite dividend)
+    return !(ax < 536870912.0f * ay && ay < INFINITY && ax < INFINITY);
+}
+__device__ __forceinline__ float fmod_float(float xf, float yf) {
+    float z = fmod_fast(xf, yf);
+    if (fmod_is_rare(xf, yf)) z = fmod_by_the_library(xf, yf);
+    return z;
+}
+template <class T> struct OpFMod { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false)
+    static constexpr bool HAS_RARE = sizeof(T) == 4;
+    __device__ __forceinline__ bool operator()(T x, T y, T& z) const {
+        if constexpr (sizeof(T) == 4) z = (T)fmod_float((float)x, (float)y);
+        else z = (T)fmod((double)x, (double)y);
+        return true; }
+    __device__ __forceinline__ void fast(T x, T y, T& z) const { z = (T)fmod_fast((float)x, (float)y); }
+    __device__ __forceinline__ bool rare(T x, T y) const { return fmod_is_rare((float)x, (float)y); }
+    __device__ __forceinline__ T slow(T x, T y) const { return (T)fmod_by_the_library((float)x, (float)y); } };
 // SFloat hypot: x^2 + y^2 cannot leave the double range and is good to 2^-53 there; one refined square root. An
 // infinity on either side answers infinity, whatever the other is (types/float_macro_kernel.h m_hypot -> hypot).
 __device__ __forceinline__ float hypot_float_rounded_once(float xf, float yf) {

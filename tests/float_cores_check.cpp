@@ -135,7 +135,7 @@ int main(int argc, char** argv) {
         // float exponent, over neighbouring exponents (where the quotient's reduction changes form), and special values
         // for hypot; prints, per function, pairs tried, mismatches and the largest difference in ulps
         const uint64_t n = std::strtoull(argv[2], nullptr, 10);
-        for (int which = 0; which < 2; ++which) {
+        for (int which = 0; which < 3; ++which) {
             uint64_t state = 0x9e3779b97f4a7c15ull, tried = 0, bad = 0;
             int64_t worst = 0;
             auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
@@ -157,6 +157,18 @@ int main(int argc, char** argv) {
                     if (atan2_is_rare(y, x)) continue;
                     got = atan2_fast(y, x);
                     want = (float)std::atan2((double)y, (double)x);
+                } else if (which == 2) {
+                    // (quotients of every size up to the limit: the divisor's exponent up to 29 below the dividend's)
+                    if (it % 2 == 0) {
+                        const uint32_t ex = (ux >> 23) & 0xffu;
+                        const uint32_t ey = (uint32_t)((int)ex - (int)((b >> 40) % 31)) & 0xffu;
+                        uy = (uy & 0x807fffffu) | (ey << 23);
+                        std::memcpy(&y, &uy, 4);
+                    }
+                    if (it % 5 == 0) { y = (float)(1 + (b >> 50) % 7); x = y * (float)(int)((a >> 40) % 100000) + ((it % 10 == 0) ? 0.0f : y * 0x1p-20f); }
+                    if (fmod_is_rare(x, y)) continue;
+                    got = fmod_fast(x, y);
+                    want = std::fmod(x, y);
                 } else {
                     got = hypot_float_rounded_once(x, y);
                     want = (float)std::hypot((double)x, (double)y);
@@ -171,7 +183,7 @@ int main(int argc, char** argv) {
                 if (d < 0) d = -d;
                 if (d > worst) worst = d;
             }
-            std::printf("%s %llu %llu %lld\n", which == 0 ? "atan2" : "hypot", (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
+            std::printf("%s %llu %llu %lld\n", which == 0 ? "atan2" : (which == 1 ? "hypot" : "fmod"), (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
         }
         return 0;
     }

@@ -517,6 +517,31 @@ def test_int32_arithmetic():
     assert_bits_equal(r.to_numpy(), hx.astype(np.float64) * 0.5)
 
 
+@pytest.mark.parametrize("tname,dt", FLOATS)
+def test_float_remainder_with_every_kind_of_argument(tname, dt):
+    """x % y of floats is the C fmod, exact: quotients small and beyond 2^29, whole-number quotients and their
+    neighbours, subnormals, zeros of both signs on either side, infinities, NaN; arrays and one divisor."""
+    import cumo_amd
+    rng = np.random.default_rng(111)
+    cls = cls_of(tname)
+    n = 100000
+    x = (rng.standard_normal(n) * np.exp2(rng.uniform(-20, 40, n))).astype(dt)
+    y = (rng.standard_normal(n) * np.exp2(rng.uniform(-20, 10, n))).astype(dt)
+    k = rng.integers(-1000, 1000, n)
+    x[::3] = (y[::3].astype(np.float64) * k[::3]).astype(dt)                          # whole-number quotients (as far as the product is exact)
+    x[1::7] = np.nextafter(x[1::7], dt(0))
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, np.finfo(dt).tiny / 4, np.finfo(dt).max, 1.5], dtype=dt)
+    x[5::101] = rng.choice(special, x[5::101].size)
+    y[7::103] = rng.choice(special, y[7::103].size)
+    with np.errstate(all="ignore"):
+        want = oracle.binary("mod", x, y)
+    assert_bits_equal((cls.cast(x) % cls.cast(y)).to_numpy(), want, "array % array")
+    for d in (1.0, 1.5, -0.75, 6.283185307179586, 1e-30, 3e38 if dt == np.float32 else 1e300):
+        with np.errstate(all="ignore"):
+            want = oracle.binary("mod", x, d)
+        assert_bits_equal((cls.cast(x) % d).to_numpy(), want, "array %% %r" % d)
+
+
 def test_int32_division_and_remainder_by_one_divisor():
     """array / d and array % d with one divisor for the whole launch go by multiplication and shift: every divisor
     kind (small, powers of two and their neighbours, the extremes, negative), dividends next to multiples and at the

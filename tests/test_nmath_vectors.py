@@ -147,14 +147,16 @@ def test_device_dfloat_algorithms_on_pairs_against_long_double(cores):
         assert int(tried) == n and float(worst) <= (0.8 if name == "erfc" else 0.52), line
 
 
-def test_device_sfloat_atan2_and_hypot_against_glibc_in_double(cores):
+def test_device_sfloat_atan2_hypot_and_remainder_against_glibc(cores):
     n = 500000000 if os.environ.get("CUMO_EXHAUSTIVE") else 5000000
     out = subprocess.run([cores, "two", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
-    assert [line.split()[0] for line in out] == ["atan2", "hypot"]
+    assert [line.split()[0] for line in out] == ["atan2", "hypot", "fmod"]
     for line in out:
         name, tried, bad, worst = line.split()
-        # evaluated in double to 2^-43 and rounded once: the rare argument next to a rounding boundary may differ by an ulp
-        assert int(tried) >= n * 9 // 10 and int(bad) <= int(tried) >> 17 and int(worst) <= 1, line
+        # evaluated in double to 2^-43 and rounded once: the rare argument next to a rounding boundary may differ by an ulp;
+        # the remainder is exact (and its arithmetic covers the quotients below 2^29: a part of the random pairs)
+        assert int(tried) >= (n // 10 if name == "fmod" else n * 9 // 10), line
+        assert int(bad) <= (0 if name == "fmod" else int(tried) >> 17) and int(worst) <= 1, line
 
 
 def test_device_dfloat_power_against_long_double(cores):
