@@ -17,6 +17,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 #include <float.h>
 
 namespace cumo_hip {
@@ -150,22 +152,30 @@ struct MeanNanImpl {
 template <class T, bool SKIP_NAN>
 struct RmsImpl {
     typedef T In;
-    struct Acc { T sum; int64_t n; };
+    // (the count rides along only where NaNs are skipped: otherwise it is the axis' length, and the accumulator is
+    // as small as the sum's)
+    struct Counted { T sum; int64_t n; };
+    struct Plain { T sum; };
+    typedef typename std::conditional<SKIP_NAN, Counted, Plain>::type Acc;
     static constexpr bool USES_INDEX = false;
     static constexpr int NOUT = 1;
     T count;
-    __device__ __forceinline__ Acc identity() const { return Acc{(T)0, 0}; }
+    __device__ __forceinline__ Acc identity() const { Acc a = Acc(); a.sum = (T)0; return a; }
     __device__ __forceinline__ void accumulate(T x, int64_t, Acc& acc) const {
-        if (SKIP_NAN) {
+        if constexpr (SKIP_NAN) {
             if (isnan_t(x)) return;
             acc.n += 1;
         }
         acc.sum += x * x;
     }
     CUMO_HIP_ACCUMULATE_N_BY_ELEMENT
-    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const { acc.sum += next.sum; acc.n += next.n; }
+    __device__ __forceinline__ void combine(const Acc& next, Acc& acc) const {
+        acc.sum += next.sum;
+        if constexpr (SKIP_NAN) acc.n += next.n;
+    }
     __device__ __forceinline__ void store(const Acc& acc, char* out, char*) const {
-        const T n = SKIP_NAN ? (T)acc.n : count;
+        T n = count;
+        if constexpr (SKIP_NAN) n = (T)acc.n;
         *reinterpret_cast<T*>(out) = (T)sqrt((double)(acc.sum / n));
     }
 };
@@ -221,6 +231,34 @@ struct MomentsImpl {
             m2 = m2 + d * d;
         }
         combine(Acc{(T)N, mb, m2}, acc);
+    }
+    // U positions of VEC neighbouring outputs at once (the column form: a lane's outputs have all seen the same
+    // number of positions): each output's own two passes over its U values, and one merge each with the ONE weight
+    // U / (n + U) that the count gives all of them (one division a step instead of one an output).
+    static constexpr bool COLUMNS_TOGETHER = !SKIP_NAN;
+    template <int U, int VEC>
+    __device__ __forceinline__ void accumulate_columns(const T (&x)[U][VEC], Acc (&acc)[VEC]) const {
+        const T n = acc[0].n;
+        const T n_new = n + (T)U;
+        const T w = (T)U / n_new;
+        const T nw = n * w;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            T s = x[0][j];
+#pragma unroll
+            for (int u = 1; u < U; ++u) s = s + x[u][j];
+            const T mb = s * ((T)1 / (T)U);
+            T m2 = (T)0;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const T d = x[u][j] - mb;
+                m2 = m2 + d * d;
+            }
+            const T delta = mb - acc[j].mean;
+            acc[j].mean = acc[j].mean + delta * w;
+            acc[j].m2 += m2 + delta * delta * nw;
+            acc[j].n = n_new;
+        }
     }
     // U blocks of N at once: the same two passes over all U * N values, one merge (and one
     // division) for all of them.

@@ -29,6 +29,11 @@ constexpr int kRsGroup = 32;            // blocks that count in on one first-lev
 constexpr int kRsOneLevel = 128;        // up to this many blocks per output count in on a single ticket
 constexpr uint32_t kRsTicketWords = 16384;  // ticket words per stream slot
 
+// An Impl whose accumulate_columns<U, VEC>(x[U][VEC], acc[VEC]) folds U positions of VEC neighbouring outputs at once,
+// all of which have seen the same number of positions before
+template <class I, class = void> struct folds_columns_together { static constexpr bool value = false; };
+template <class I> struct folds_columns_together<I, decltype((void)I::COLUMNS_TOGETHER)> { static constexpr bool value = I::COLUMNS_TOGETHER; };
+
 struct RedSParams {
     const char* in;
     char* out;
@@ -610,12 +615,17 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
             __builtin_amdgcn_sched_barrier(0);  // all loads of the step issued before the first fold
             if (i0 + U <= end && p.index_mode != 2) {
                 // a whole block of consecutive positions along the axis for each output
+                if constexpr (folds_columns_together<Impl>::value) {
+                    // (the lane's outputs have had the same positions so far: what depends on the count alone is worked out once)
+                    impl.template accumulate_columns<U, VEC>(x, acc);
+                } else {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    In t[U];
+                    for (int j = 0; j < VEC; ++j) {
+                        In t[U];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) t[u] = x[u][j];
-                    impl.template accumulate_n<U>(t, (int64_t)i0, acc[j]);
+                        for (int u = 0; u < U; ++u) t[u] = x[u][j];
+                        impl.template accumulate_n<U>(t, (int64_t)i0, acc[j]);
+                    }
                 }
             } else {
 #pragma unroll
