@@ -445,22 +445,39 @@ __device__ __forceinline__ double log1p_core(double u) {
     // the logarithm from the table-driven core (2^-44 relative, next to 1 as well), times ln 2
     return __builtin_fma(c, 1.0 - um, 6.93147180559945286227e-01 * log2_by_table(w, float_tables()));
 }
+// asinh|x| = log(a + sqrt(1 + a^2)) directly from 2^-11 on: with the square root good to 2^-52 (a second refining
+// step) the sum is off by 2^-52 next to 1, where the answer is about a, so by 2^-41 of the answer at most; the
+// logarithm's table has 1.0 as the midpoint of an interval, so a sum next to 1 loses nothing. Below 2^-11
+// a - a^3 / 6 (the next term is below 2^-44 of a). This saves the reciprocal and the lost-bits bookkeeping of
+// the log1p form: 47 -> 39 vector instructions an element.
 __device__ __forceinline__ float asinh_float_rounded_once(float xf) {
     const float af = __builtin_fabsf(xf);
     const double a = (double)af;
     const double a2 = a * a;
-    const double u = __builtin_fma(a2, rcp_refined(1.0 + sqrt_refined(1.0 + a2)), a);
-    float y = (float)log1p_core(u);       // NaN travels through; an infinity gives NaN here and is put right below
-    y = (af < 1.862645149230957e-09f) ? af : y;
+    const double w = 1.0 + a2;
+#ifdef CUMO_HIP_HOST_CHECK
+    const double s = sqrt(w);
+#else
+    const double r = __builtin_amdgcn_rsq(w);
+    double s = w * r;
+    s = __builtin_fma(__builtin_fma(-s, s, w) * 0.5, r, s);
+    s = __builtin_fma(__builtin_fma(-s, s, w) * 0.5, r, s);
+#endif
+    // (the table-driven logarithm works on the argument's bits: a NaN comes back in through a - a, which is NaN for an infinity too)
+    const double big = __builtin_fma(6.93147180559945286227e-01, log2_by_table(a + s, float_tables()), a - a);
+    const double small = __builtin_fma(a2 * a, -1.0 / 6.0, a);
+    float y = (float)((af < 4.8828125e-04f) ? small : big);   // NaN travels through; an infinity gives NaN here and is put right below
     y = (af == INFINITY) ? INFINITY : y;
     return __builtin_copysignf(y, xf);
 }
+// acosh x = log(x + sqrt((x - 1)(x + 1))): both factors and their product are exact in double, so the square root
+// is good to 2^-44 of itself next to 1 as well, where it is the answer's leading term.
 __device__ __forceinline__ float acosh_float_rounded_once(float xf) {
     const float xc = (xf < 1.0f) ? 1.0f : xf;  // keeps the square root's argument in range; a NaN stays
-    const double t = (double)xc - 1.0;
-    const double q = __builtin_fma(t, t, 2.0 * t);
-    const double u = t + ((q > 0.0) ? sqrt_refined(q) : 0.0);   // a NaN gives 0 here and comes back through t
-    float y = (float)log1p_core(u);
+    const double x = (double)xc;
+    const double q = (x - 1.0) * (x + 1.0);
+    const double u = x + ((q > 0.0) ? sqrt_refined(q) : 0.0);   // a NaN gives 0 here and comes back through x
+    float y = (float)__builtin_fma(6.93147180559945286227e-01, log2_by_table(u, float_tables()), x - x);   // (a NaN comes back in through x - x)
     y = (xf < 1.0f) ? NAN : y;
     y = (xf == INFINITY) ? INFINITY : y;
     return y;
