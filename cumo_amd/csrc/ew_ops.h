@@ -895,6 +895,40 @@ template <class T> struct OpPow { CUMO_HIP_OP_COMMON(T, T, T, 2, false, false) s
         if constexpr (sizeof(T) == 4) return (T)pow_by_the_library((float)x, (float)y);
         else return (T)pow_double_by_the_library((double)x, (double)y); } };
 
+// SFloat ** y for one exponent that is a whole number of halves, up to 32 either way (x ** 0.5, x ** -1.5, x ** 2.5,
+// x ** 3.0): the whole part by squaring and multiplying, the half by one refined square root, a negative exponent by one
+// division, all in double (whose range holds every intermediate whose result a float can hold; beyond it the float
+// answer is 0 or infinite either way) and rounded to float once. The rules of pow for the arguments that arithmetic
+// would get wrong are spelt out: with an exponent that is not whole a zero base counts as +0 and -inf as +inf
+// (a negative base answers NaN through the square root); x ** 0 is 1 whatever x is.
+// (NEG, a negative exponent, at compile time: left to run time the compiler evaluates the division for every element
+// and then picks, 25 issue slots an element)
+template <bool NEG>
+struct OpPowHalves { CUMO_HIP_OP_COMMON(float, float, float, 1, false, false)
+    int twice;   // 2 y (negative exactly when NEG)
+    __device__ __forceinline__ bool operator()(float xf, float, float& z) const {
+        const unsigned m = (unsigned)(twice < 0 ? -twice : twice);
+        const bool half = (m & 1u) != 0;
+        double x = (double)xf;
+        if (half) {
+            x = (xf == 0.0f) ? 0.0 : x;
+            x = (xf == -INFINITY) ? (double)INFINITY : x;
+        }
+        double r = 1.0, b = x;
+        for (unsigned q = m >> 1; q != 0; q >>= 1) {   // (the same turns for every lane)
+            if (q & 1u) r *= b;
+            b *= b;
+        }
+        if (half) {
+            const bool inside = x > 0.0 && x < (double)INFINITY;
+            double s = sqrt_refined(inside ? x : 1.0);
+            s = inside ? s : ((x == 0.0 || x == (double)INFINITY) ? x : (double)NAN);   // (a NaN base fails every comparison)
+            r *= s;
+        }
+        if (NEG) r = 1.0 / r;
+        z = (float)r;
+        return true; } };
+
 // Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
 // element type for small exponents, pow() beyond 64, the reciprocal for negative ones.
 // (out of line: inlined at every element, the library's pow took 66 registers of a kernel that needs 10)

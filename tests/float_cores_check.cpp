@@ -12,6 +12,7 @@
 //                                      cosh erfc log1p asinh acosh atanh) against the long double function; prints, per
 //                                      function, arguments tried, the largest error in ulps and where it was
 //   float_cores_check dpow <n>         n random (base, exponent) pairs through the DFloat power's arithmetic against powl
+//   float_cores_check halves <stride>  every stride-th float through the SFloat power by whole numbers of halves against (float)glibc pow
 //   float_cores_check two <n>          n random pairs through the SFloat atan2 and hypot against (float)glibc in double
 //   float_cores_check sweep <stride>   every stride-th float bit pattern through each SFloat
 //                                      core against (float)glibc((double)x); prints, per
@@ -234,6 +235,40 @@ int main(int argc, char** argv) {
             else if (err > worst) { worst = err; worst_x = x; worst_y = y; }
         }
         std::printf("pow %llu %.4f %.4f %llu %a %a\n", (unsigned long long)n, worst, worst_sub, (unsigned long long)wrong_ends, worst_x, worst_y);
+        return 0;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "halves") == 0) {
+        // every stride-th float bit pattern through the SFloat power for exponents that are whole numbers of halves
+        // against (float)glibc pow in double; prints, per exponent, patterns tried, mismatches and the largest difference in ulps
+        const uint32_t stride = (uint32_t)std::strtoul(argv[2], nullptr, 10);
+        const int twices[] = {0, 1, -1, 2, -2, 3, -3, 4, -4, 5, -5, 6, 7, 15, -15, 20, 32, 33, -33, 63, 64, -64};
+        for (int twice : twices) {
+            OpPowHalves<true> down;
+            OpPowHalves<false> up;
+            down.twice = up.twice = twice;
+            const double y = 0.5 * twice;
+            uint64_t tried = 0, bad = 0;
+            int64_t worst = 0;
+            for (uint64_t b = 0; b < (1ull << 32); b += stride) {
+                uint32_t u = (uint32_t)b;
+                float x; std::memcpy(&x, &u, 4);
+                float got = 0.0f;
+                if (twice < 0) down(x, 0.0f, got);
+                else up(x, 0.0f, got);
+                const float want = (float)std::pow((double)x, y);
+                ++tried;
+                if (got != got && want != want) continue;
+                uint32_t gu, wu; std::memcpy(&gu, &got, 4); std::memcpy(&wu, &want, 4);
+                if (gu == wu) continue;
+                ++bad;
+                if (got != got || want != want) { worst = 1 << 30; continue; }
+                if (got == want) { if (worst < 1) worst = 1; continue; }  // +0 against -0
+                int64_t d = ordered(got) - ordered(want);
+                if (d < 0) d = -d;
+                if (d > worst) worst = d;
+            }
+            std::printf("%g %llu %llu %lld\n", y, (unsigned long long)tried, (unsigned long long)bad, (long long)worst);
+        }
         return 0;
     }
     if (argc >= 3 && std::strcmp(argv[1], "pow") == 0) {

@@ -159,6 +159,17 @@ def test_device_sfloat_atan2_hypot_and_remainder_against_glibc(cores):
         assert int(bad) <= (0 if name == "fmod" else int(tried) >> 17) and int(worst) <= 1, line
 
 
+def test_device_sfloat_power_by_whole_numbers_of_halves_against_glibc(cores):
+    """x ** y for one exponent that is a whole number of halves goes by squarings, multiplications and one square root
+    in double: every float bit pattern of the stride, the rules for zeros, infinities, negative bases and NaN included."""
+    stride = 1 if os.environ.get("CUMO_EXHAUSTIVE") else 4099
+    out = subprocess.run([cores, "halves", str(stride)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
+    assert len(out) == 22
+    for line in out:
+        y, tried, bad, worst = line.split()
+        assert int(tried) >= (1 << 32) // stride and int(bad) <= int(tried) >> 17 and int(worst) <= 1, line
+
+
 def test_device_dfloat_power_against_long_double(cores):
     """x ** y of DFloat for a positive normal base and a finite exponent: log2 x and y log2 x as pairs of doubles."""
     n = 300000000 if os.environ.get("CUMO_EXHAUSTIVE") else 3000000
