@@ -264,7 +264,9 @@ def config_ops(name, cumo, host):
         for fname in ("log", "sin", "tanh", "erf", "exp", "sqrt", "erfc", "asinh", "log1p"):
             ops.append(("NMath.%s(DFloat)" % fname, (lambda f: lambda e: e.__setitem__("rd", getattr(NM, f)(e["xd"])))(fname), 16 * n, n))
         ops += [
+            # (2.5 is a whole number of halves: squarings and a square root; 2.7 takes the general power)
             ("SFloat**2.5", lambda e: e.__setitem__("r", e["xs"] ** 2.5), 8 * n, n),
+            ("SFloat**2.7", lambda e: e.__setitem__("r", e["xs"] ** 2.7), 8 * n, n),
             ("DFloat**2.5", lambda e: e.__setitem__("rd", e["xd"] ** 2.5), 16 * n, n),
             ("SFloat.cumsum (one run of 2^26)", lambda e: e.__setitem__("r", e["xs"].cumsum()), 8 * n, n),
             ("SFloat[8192,8192].cumsum(axis:0)", lambda e: e.__setitem__("r2", e["xs2"].cumsum(axis=0)), 8 * n, n),
