@@ -430,3 +430,40 @@ __device__ __forceinline__ double atanh_double(double x) {
     y = __builtin_copysign(y, x);
     return (x != x) ? x : y;
 }
+
+// ---- DFloat ** y for one exponent that is a whole number of halves, up to 8 either way ---------------------
+// (x ** 0.5, x ** -1.5, x ** 2.5): the whole part by squarings and multiplications of pairs (the first square is exact),
+// the half by sqrt_pair, a negative exponent by a reciprocal corrected with its exact remainder, one rounding at the
+// end. For bases between 2^-100 and 2^100 (no intermediate leaves the normal range there); every other base is the
+// device library's pow, out of line.
+__device__ __forceinline__ void pair_product(double ah, double al, double bh, double bl, double& ph, double& pl) {
+    const double p = ah * bh;
+    const double e = __builtin_fma(ah, bl, __builtin_fma(al, bh, __builtin_fma(ah, bh, -p)));
+    ph = p + e;
+    pl = (p - ph) + e;
+}
+template <bool NEG>
+__device__ __forceinline__ double pow_halves_double_fast(double x, int twice) {
+    const unsigned m = (unsigned)(twice < 0 ? -twice : twice);
+    double rh = 1.0, rl = 0.0, bh = x, bl = 0.0;
+    for (unsigned q = m >> 1; q != 0; q >>= 1) {   // (the same turns for every lane)
+        if (q & 1u) pair_product(rh, rl, bh, bl, rh, rl);
+        if (q > 1u) pair_product(bh, bl, bh, bl, bh, bl);
+    }
+    if (m & 1u) {
+        double sh, sl;
+        sqrt_pair(x, 0.0, sh, sl);
+        pair_product(rh, rl, sh, sl, rh, rl);
+    }
+    if (NEG) {
+        // 1 / (rh + rl): the estimate's remainder, exactly, times the estimate again
+        const double q = rcp_refined(rh);
+        const double left = __builtin_fma(-q, rl, __builtin_fma(-q, rh, 1.0));
+        return __builtin_fma(left, q, q);
+    }
+    return rh + rl;
+}
+__device__ __forceinline__ bool pow_halves_double_is_rare(double x) {
+    // positive, between 2^-100 and 2^100 (a NaN fails)
+    return !(x >= 0x1p-100 && x <= 0x1p100);
+}

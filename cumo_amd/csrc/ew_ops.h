@@ -929,6 +929,19 @@ struct OpPowHalves { CUMO_HIP_OP_COMMON(float, float, float, 1, false, false)
         z = (float)r;
         return true; } };
 
+// DFloat ** y for one exponent that is a whole number of halves up to 8 either way (dd_cores.h)
+template <bool NEG>
+struct OpPowHalvesD { CUMO_HIP_OP_COMMON(double, double, double, 1, false, false) static constexpr bool HEAVY = true;
+    static constexpr bool HAS_RARE = true;
+    int twice;   // 2 y (negative exactly when NEG)
+    __device__ __forceinline__ bool operator()(double x, double, double& z) const {
+        fast(x, 0.0, z);
+        if (rare(x, 0.0)) z = slow(x, 0.0);
+        return true; }
+    __device__ __forceinline__ void fast(double x, double, double& z) const { z = pow_halves_double_fast<NEG>(x, twice); }
+    __device__ __forceinline__ bool rare(double x, double) const { return pow_halves_double_is_rare(x); }
+    __device__ __forceinline__ double slow(double x, double) const { return pow_double_by_the_library(x, 0.5 * (double)twice); } };
+
 // Float ** Int32 (reference: types/float_macro_kernel.h:125-149): products in the
 // element type for small exponents, pow() beyond 64, the reciprocal for negative ones.
 // (out of line: inlined at every element, the library's pow took 66 registers of a kernel that needs 10)

@@ -237,6 +237,31 @@ int main(int argc, char** argv) {
         std::printf("pow %llu %.4f %.4f %llu %a %a\n", (unsigned long long)n, worst, worst_sub, (unsigned long long)wrong_ends, worst_x, worst_y);
         return 0;
     }
+    if (argc >= 3 && std::strcmp(argv[1], "dhalves") == 0) {
+        // n random bases between 2^-100 and 2^100 through the DFloat power for every exponent that is a whole number of
+        // halves up to 8 either way, against powl; prints, per exponent, bases tried and the largest error in ulps
+        const uint64_t n = std::strtoull(argv[2], nullptr, 10);
+        for (int twice = -16; twice <= 16; ++twice) {
+            if (twice == 0) continue;
+            uint64_t state = 0x9e3779b97f4a7c15ull;
+            auto next = [&state]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+            double worst = 0.0;
+            for (uint64_t it = 0; it < n; ++it) {
+                const uint64_t a = next(), b = next();
+                const double e = (it % 2) ? 200.0 * (double)(a >> 11) * 0x1p-53 - 100.0 : 4.0 * (double)(a >> 11) * 0x1p-53 - 2.0;
+                double x = std::exp2(std::floor(e)) * (1.0 + (double)(b >> 12) * 0x1p-52);
+                if (pow_halves_double_is_rare(x)) continue;
+                const double got = twice < 0 ? pow_halves_double_fast<true>(x, twice) : pow_halves_double_fast<false>(x, twice);
+                const long double want = powl((long double)x, 0.5L * twice);
+                int ex;
+                std::frexp((double)want, &ex);
+                const double err = (double)(fabsl((long double)got - want) / std::ldexp(1.0L, ex - 53));
+                if (err > worst) worst = err;
+            }
+            std::printf("%g %llu %.4f\n", 0.5 * twice, (unsigned long long)n, worst);
+        }
+        return 0;
+    }
     if (argc >= 3 && std::strcmp(argv[1], "halves") == 0) {
         // every stride-th float bit pattern through the SFloat power for exponents that are whole numbers of halves
         // against (float)glibc pow in double; prints, per exponent, patterns tried, mismatches and the largest difference in ulps

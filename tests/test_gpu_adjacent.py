@@ -82,6 +82,31 @@ def test_maximum_minimum_parity(tname, dt):
 
 
 @pytest.mark.parametrize("tname,dt", FLOATS)
+def test_float_pow_by_whole_numbers_of_halves(tname, dt):
+    """array ** y for one exponent that is a whole number of halves (squarings, multiplications, one square root on
+    the device) against pow: ordinary bases, bases at the ends of the range, zeros, infinities, negatives and NaN."""
+    cls = cls_of(tname)
+    rng = np.random.default_rng(47)
+    ulp = 1 if dt == np.float32 else 2
+    info = np.finfo(dt)
+    ordinary = np.exp2(rng.uniform(-20.0, 20.0, size=5000)).astype(dt)
+    ends = np.concatenate([np.exp2(rng.uniform(info.minexp - 20, info.minexp + 30, size=500)),
+                           np.exp2(rng.uniform(info.maxexp - 30, info.maxexp - 0.001, size=500))]).astype(dt)
+    special = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 2.0, -8.0, -0.25, info.tiny, info.max,
+                        info.smallest_subnormal], dtype=dt)
+    hx = np.concatenate([ordinary, ends, special, -ordinary[:100]])
+    x = cls.cast(hx)
+    for twice in range(-17, 18):
+        e = 0.5 * twice
+        with np.errstate(all="ignore"):
+            assert_ulp((x ** e).to_numpy(), oracle.binary("pow", hx, e), ulp, ("array **", e))
+    hm = ordinary.reshape(50, 100)
+    with np.errstate(all="ignore"):
+        assert_ulp((cls.cast(hm)[:, 1:] ** 1.5).to_numpy(), oracle.binary("pow", np.ascontiguousarray(hm[:, 1:]), 1.5), ulp)
+        assert_ulp((cls.cast(hm).transpose() ** -2.5).to_numpy(), oracle.binary("pow", np.ascontiguousarray(hm.T), -2.5), ulp)
+
+
+@pytest.mark.parametrize("tname,dt", FLOATS)
 def test_float_pow_parity(tname, dt):
     cls = cls_of(tname)
     import cumo_amd

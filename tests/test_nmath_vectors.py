@@ -170,6 +170,15 @@ def test_device_sfloat_power_by_whole_numbers_of_halves_against_glibc(cores):
         assert int(tried) >= (1 << 32) // stride and int(bad) <= int(tried) >> 17 and int(worst) <= 1, line
 
 
+def test_device_dfloat_power_by_whole_numbers_of_halves_against_long_double(cores):
+    n = 20000000 if os.environ.get("CUMO_EXHAUSTIVE") else 200000
+    out = subprocess.run([cores, "dhalves", str(n)], check=True, stdout=subprocess.PIPE, text=True).stdout.strip().split("\n")
+    assert len(out) == 32
+    for line in out:
+        y, tried, worst = line.split()
+        assert int(tried) == n and float(worst) <= 0.51, line
+
+
 def test_device_dfloat_power_against_long_double(cores):
     """x ** y of DFloat for a positive normal base and a finite exponent: log2 x and y log2 x as pairs of doubles."""
     n = 300000000 if os.environ.get("CUMO_EXHAUSTIVE") else 3000000
