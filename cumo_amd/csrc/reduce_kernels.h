@@ -442,22 +442,54 @@ __global__ __launch_bounds__(kRedBlock) void red_col_local_kernel(RedKParams p, 
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[j] = impl.identity();
         }
+        // the SB parts of a group meet pairwise through LDS, neighbours first, the earlier part on the left
+        Acc own[has_exact<Impl>::value ? VEC : 1];
+        if constexpr (has_exact<Impl>::value) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) own[j] = acc[j];
+        }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = acc[j];
         __syncthreads();
+        for (unsigned d = 1; d < SB; d <<= 1) {
+            if ((s & (2u * d - 1u)) == 0) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) impl.combine(part[(s + d) * CPB + c][j], acc[j]);
+                if (2u * d < SB) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = acc[j];
+                }
+            }
+            __syncthreads();
+        }
+        if constexpr (has_exact<Impl>::value) {
+            // folded by value; an output that may have lost which of two equal parts came first is folded
+            // again from the lanes' own parts, plain values in axis order, with the exact rule
+            bool again = false;
+            if (ok && s == 0) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) again = again || impl.needs_exact(acc[j]);
+            }
+            if (__syncthreads_or(again ? 1 : 0)) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = own[j];
+                __syncthreads();
+                if (ok && s == 0) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        if (!impl.needs_exact(acc[j])) continue;
+                        typedef typename Impl::Exact Exact;
+                        const Exact ex = impl.exact();
+                        typename Exact::Acc e = ex.identity();
+                        for (unsigned k = 0; k < SB; ++k) ex.accumulate(part[k * CPB + c][j], (int64_t)k, e);
+                        acc[j] = impl.from_exact(e);
+                    }
+                }
+            }
+        }
         if (ok && s == 0) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                if constexpr (has_exact<Impl>::value) {
-                    // the parts are plain values in axis order: fold them with the exact rule
-                    typedef typename Impl::Exact Exact;
-                    const Exact ex = impl.exact();
-                    typename Exact::Acc e = ex.identity();
-                    for (unsigned k = 0; k < SB; ++k) ex.accumulate(part[k * CPB + c][j], (int64_t)k, e);
-                    acc[j] = impl.from_exact(e);
-                } else {
-                    for (unsigned k = 1; k < SB; ++k) impl.combine(part[k * CPB + c][j], acc[j]);
-                }
                 const uint64_t i_out = i_out0 + j;
                 if (PARTIAL) {
                     partial[i_out * p.n_split + i_split] = acc[j];

@@ -659,25 +659,55 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
             }
         }
         if constexpr (LOCAL) {
+            // The SB parts of an output group meet pairwise through LDS, neighbours first and the earlier part
+            // on the left: log2 SB rounds in which every left-hand lane works, where one lane folding all the
+            // parts one after the other waited for SB reads of LDS in a row while the rest of the block idled
+            // (blocks start and end together here, so nothing else covers that time).
+            Acc own[has_exact<Impl>::value ? VEC : 1];
+            if constexpr (has_exact<Impl>::value) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) own[j] = acc[j];
+            }
 #pragma unroll
             for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = acc[j];
             __syncthreads();
-            if (s == 0) {
+            for (unsigned d = 1; d < SB; d <<= 1) {
+                if ((s & (2u * d - 1u)) == 0) {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    if constexpr (has_exact<Impl>::value) {
-                        // the parts are plain values in axis order: fold them with the exact rule
-                        typedef typename Impl::Exact Exact;
-                        const Exact ex = impl.exact();
-                        typename Exact::Acc e = ex.identity();
-                        for (unsigned k = 0; k < SB; ++k) ex.accumulate_acc(part[k * CPB + c][j], (int64_t)k, e);
-                        acc[j] = impl.from_exact(e);
-                    } else {
-                        for (unsigned k = 1; k < SB; ++k) impl.combine(part[k * CPB + c][j], acc[j]);
+                    for (int j = 0; j < VEC; ++j) impl.combine(part[(s + d) * CPB + c][j], acc[j]);
+                    if (2u * d < SB) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = acc[j];
                     }
                 }
+                __syncthreads();
             }
-            __syncthreads();
+            if constexpr (has_exact<Impl>::value) {
+                // folded by value; an output that may have lost which of two equal parts came first is folded
+                // again from the lanes' own parts, plain values in axis order, with the exact rule
+                bool again = false;
+                if (s == 0) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) again = again || impl.needs_exact(acc[j]);
+                }
+                if (__syncthreads_or(again ? 1 : 0)) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) part[threadIdx.x][j] = own[j];
+                    __syncthreads();
+                    if (s == 0) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) {
+                            if (!impl.needs_exact(acc[j])) continue;
+                            typedef typename Impl::Exact Exact;
+                            const Exact ex = impl.exact();
+                            typename Exact::Acc e = ex.identity();
+                            for (unsigned k = 0; k < SB; ++k) ex.accumulate_acc(part[k * CPB + c][j], (int64_t)k, e);
+                            acc[j] = impl.from_exact(e);
+                        }
+                    }
+                    __syncthreads();
+                }
+            }
         }
         if (PARTIAL) {
             // partial[part][output], a part's outputs padded to whole groups: the lanes of a block write one run

@@ -338,7 +338,7 @@ def test_dfloat_kahan_sum():
 @pytest.mark.parametrize("tname,dt", FLOATS)
 @pytest.mark.parametrize("shape,axis", [((300, 77), 1), ((300, 77), 0), ((5, 20000), 1), ((20000, 5), 0), ((3000001,), None),
                                         ((64, 33, 40), (0, 2)), ((6, 70000), 1), ((2, 3, 4096), 2), ((3000, 1000), 0), ((70000, 64), 0),
-                                        ((8192, 260), 0)])
+                                        ((8192, 260), 0), ((4, 512, 256), 1), ((3, 130, 64), 1)])
 def test_min_max_keep_the_zero_that_came_first(tname, dt, shape, axis):
     # Numo's sequential loop only replaces on a strict comparison (real_accum.h:217-278), so of
     # +0 and -0 the earlier one is the answer. Every output here ends on a zero, with both signs
