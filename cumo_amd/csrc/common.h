@@ -48,6 +48,11 @@ int bit_count_rows_reduce(const cumo_hip_bit_count_nd_t* counts);  // (stores th
 // launched (stored or added as counts->overwrite says), 0 when the loop is not one it takes.
 int bit_count_cols_words_launch(const cumo_hip_bit_count_nd_t* counts);
 
+// x op y (op: 0 + 1 - 2 * 3 /) for two contiguous, 16-byte aligned runs of n elements of different types
+// (SFloat / DFloat / Int32), converted to the result's type on the way in, into z of that type (ew_mixed.hip).
+// False when the pair of types or the alignment is not one it takes; nothing is launched then.
+bool mixed_flat_binary(int op, int ta, const char* x, int tb, const char* y, char* z, uint64_t n);
+
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)
 // stand aside. For tests: the wide paths otherwise only run on arrays beyond 2^32 elements.

@@ -1,0 +1,94 @@
+// Arithmetic on two arrays of different element types, each one contiguous run, in one launch: every
+// element is converted to the result's type on the way in, exactly as the cast the reference makes first
+// would convert it (narray/gen/tmpl/binary.c:38-97 upcasts, then runs the result type's loop), and the
+// result type's + - * / is applied. The cast into a temporary array -- a write and a read of the wider
+// type for every element -- is what this saves: SFloat + DFloat moves 20 bytes an element instead of 36.
+// Other layouts keep the two steps.
+#include "common.h"
+#include "cumo_hip_ndloop.h"
+#include "ew_kernels.h"
+
+namespace cumo_hip {
+namespace {
+
+constexpr int kMxBlock = 256, kMxVec = 4;
+
+template <int OP, class T>
+__device__ __forceinline__ T mixed_apply(T a, T b) {
+    if (OP == 0) return a + b;
+    if (OP == 1) return a - b;
+    if (OP == 2) return a * b;
+    return a / b;
+}
+
+template <int OP, class TA, class TB, class TR, bool NT, int kMxUnr>
+__global__ __launch_bounds__(kMxBlock) void ew_mixed_flat_kernel(const char* __restrict__ px, const char* __restrict__ py,
+                                                                 char* __restrict__ pz, uint64_t n) {
+    const uint64_t i0 = ((uint64_t)blockIdx.x * (kMxBlock * kMxUnr) + threadIdx.x) * kMxVec;
+    TA xv[kMxUnr][kMxVec];
+    TB yv[kMxUnr][kMxVec];
+    bool whole[kMxUnr];
+#pragma unroll
+    for (int u = 0; u < kMxUnr; ++u) {
+        const uint64_t i = i0 + (uint64_t)u * (kMxBlock * kMxVec);
+        whole[u] = i + kMxVec <= n;
+        if (whole[u]) {
+            raw_load<TA, kMxVec, NT>(px + i * sizeof(TA), xv[u]);
+            raw_load<TB, kMxVec, NT>(py + i * sizeof(TB), yv[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kMxUnr; ++u) {
+        const uint64_t i = i0 + (uint64_t)u * (kMxBlock * kMxVec);
+        if (whole[u]) {
+            TR zv[kMxVec];
+#pragma unroll
+            for (int j = 0; j < kMxVec; ++j) zv[j] = mixed_apply<OP, TR>((TR)xv[u][j], (TR)yv[u][j]);
+            raw_store<TR, kMxVec, NT>(pz + i * sizeof(TR), zv);
+        } else if (i < n) {
+            // the run's last elements, fewer than a vector
+            for (uint64_t k = i; k < n; ++k)
+                reinterpret_cast<TR*>(pz)[k] = mixed_apply<OP, TR>((TR) reinterpret_cast<const TA*>(px)[k], (TR) reinterpret_cast<const TB*>(py)[k]);
+        }
+    }
+}
+
+template <int OP, class TA, class TB, class TR>
+void mixed_launch(const char* x, const char* y, char* z, uint64_t n) {
+    constexpr int kMxUnr = sizeof(TR) == 8 ? 2 : 4;   // vectors of four elements a lane has in flight per operand
+    const uint64_t per_block = (uint64_t)kMxBlock * kMxUnr * kMxVec;
+    const dim3 g((unsigned)((n + per_block - 1) / per_block)), b(kMxBlock);
+    const bool nt = stream_past_caches(n * (sizeof(TA) + sizeof(TB) + sizeof(TR)));
+    if (nt) hipLaunchKernelGGL((ew_mixed_flat_kernel<OP, TA, TB, TR, true, kMxUnr>), g, b, 0, current_stream(), x, y, z, n);
+    else hipLaunchKernelGGL((ew_mixed_flat_kernel<OP, TA, TB, TR, false, kMxUnr>), g, b, 0, current_stream(), x, y, z, n);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+template <int OP>
+bool mixed_by_types(int ta, int tb, const char* x, const char* y, char* z, uint64_t n) {
+    // the result's type is the wider float of the two (gen/def/{sfloat,dfloat,int32}.rb: Int32 with SFloat is SFloat)
+    if (ta == CUMO_HIP_SFLOAT && tb == CUMO_HIP_DFLOAT) mixed_launch<OP, float, double, double>(x, y, z, n);
+    else if (ta == CUMO_HIP_DFLOAT && tb == CUMO_HIP_SFLOAT) mixed_launch<OP, double, float, double>(x, y, z, n);
+    else if (ta == CUMO_HIP_INT32 && tb == CUMO_HIP_SFLOAT) mixed_launch<OP, int32_t, float, float>(x, y, z, n);
+    else if (ta == CUMO_HIP_SFLOAT && tb == CUMO_HIP_INT32) mixed_launch<OP, float, int32_t, float>(x, y, z, n);
+    else if (ta == CUMO_HIP_INT32 && tb == CUMO_HIP_DFLOAT) mixed_launch<OP, int32_t, double, double>(x, y, z, n);
+    else if (ta == CUMO_HIP_DFLOAT && tb == CUMO_HIP_INT32) mixed_launch<OP, double, int32_t, double>(x, y, z, n);
+    else return false;
+    return true;
+}
+
+}  // namespace
+
+bool mixed_flat_binary(int op, int ta, const char* x, int tb, const char* y, char* z, uint64_t n) {
+    if (n == 0 || n >= ((uint64_t)1 << 43)) return false;  // (the grid's x dimension: 2^31 blocks of 2^12 elements)
+    if ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15u) != 0) return false;
+    switch (op) {
+        case 0: return mixed_by_types<0>(ta, tb, x, y, z, n);
+        case 1: return mixed_by_types<1>(ta, tb, x, y, z, n);
+        case 2: return mixed_by_types<2>(ta, tb, x, y, z, n);
+        case 3: return mixed_by_types<3>(ta, tb, x, y, z, n);
+    }
+    return false;
+}
+
+}  // namespace cumo_hip

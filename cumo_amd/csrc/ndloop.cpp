@@ -21,6 +21,7 @@
 // No function here keeps a C++ object with a destructor alive across a call
 // that may report an error: the installed handler may leave with longjmp.
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.h"
@@ -995,6 +996,53 @@ int check_arith(const NA* x) {
 
 unsigned all_dims(const NA* x) { return x->ndim ? ((1u << x->ndim) - 1u) : 0u; }
 
+// + - * / of two arrays of different types that have one shape and are one contiguous run each, into a fresh
+// result or a given contiguous one of the higher type: one launch that converts on the way in, instead of a cast
+// into a temporary array and the higher type's own launch (ew_mixed.hip). *taken says whether it has seen to the
+// operation (launched it, or failed to allocate the result: the error kind is returned then).
+int mixed_one_launch(const char* op, const NA* x, const NA* y, int up, NA* z, bool* taken) {
+    *taken = false;
+    int code;
+    if (!std::strcmp(op, "add")) code = 0;
+    else if (!std::strcmp(op, "sub")) code = 1;
+    else if (!std::strcmp(op, "mul")) code = 2;
+    else if (!std::strcmp(op, "div") && is_float(up)) code = 3;
+    else return CUMO_HIP_OK;
+    static const bool off = [] {
+        const char* e = std::getenv("CUMO_HIP_MIXED_ONE_LAUNCH");   // =0: always cast first (for tests)
+        return e && e[0] == '0';
+    }();
+    if (off || !z || x->ndim != y->ndim || x->ndim < 1) return CUMO_HIP_OK;
+    for (int d = 0; d < x->ndim; d++)
+        if (x->shape[d] != y->shape[d]) return CUMO_HIP_OK;
+    const size_t n = total_of(x);
+    if (n == 0 || !is_contiguous(x) || !is_contiguous(y)) return CUMO_HIP_OK;
+    const char* px = x->ptr + x->offset;
+    const char* py = y->ptr + y->offset;
+    if ((((uintptr_t)px | (uintptr_t)py) & 15u) != 0) return CUMO_HIP_OK;
+    const bool fresh = z->ptr == NULL;
+    if (!fresh) {
+        if (z->type != up || z->ndim != x->ndim || !is_contiguous(z) || (((uintptr_t)(z->ptr + z->offset)) & 15u) != 0) return CUMO_HIP_OK;
+        for (int d = 0; d < x->ndim; d++)
+            if (z->shape[d] != x->shape[d]) return CUMO_HIP_OK;
+    } else {
+        const int rc = cumo_hip_na_alloc(z, up, x->ndim, x->shape);
+        if (rc != CUMO_HIP_OK) {
+            *taken = true;
+            return rc;
+        }
+    }
+    if (cumo_hip::mixed_flat_binary(code, x->type, px, y->type, py, z->ptr + z->offset, n)) {
+        *taken = true;
+        return CUMO_HIP_OK;
+    }
+    if (fresh) {
+        cumo_cuda_runtime_free(z->ptr);
+        z->ptr = NULL;
+    }
+    return CUMO_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1006,6 +1054,11 @@ int cumo_hip_na_binary(const char* op, const cumo_hip_narray_t* x, const cumo_hi
     const BinaryRow* row = find_row(kBinary, op);
     const int up = upcast(x->type, y->type);
     if (!row || !binary_has(row, up, false)) return no_method(op);
+    if (x->type != y->type) {
+        bool taken = false;
+        rc = mixed_one_launch(op, x, y, up, z, &taken);
+        if (taken) return rc;
+    }
     NA tx, ty;
     const NA *ux, *uy;
     rc = cast_operand(x, up, &tx, &ux);

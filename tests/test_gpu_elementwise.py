@@ -604,6 +604,53 @@ def test_casts_and_copies(src, dst):
         assert r.type_name == (src if rank[src] > rank[dst] else dst)
 
 
+MIXED_PAIRS = [("sfloat", "dfloat"), ("dfloat", "sfloat"), ("int32", "sfloat"), ("sfloat", "int32"), ("int32", "dfloat"), ("dfloat", "int32")]
+
+
+@pytest.mark.parametrize("ta,tb", MIXED_PAIRS)
+def test_arithmetic_on_two_element_types(ta, tb):
+    """x op y for arrays of different types answers what casting both to the higher type and then running that type's
+    operation answers, bit for bit (gen/tmpl/binary.c:38-97): two contiguous arrays of one shape go through one launch
+    that converts on the way in; views, repeated operands and starts off a 16-byte boundary cast first."""
+    npdt = {"sfloat": np.float32, "dfloat": np.float64, "int32": np.int32}
+    rank = {"int32": 0, "sfloat": 1, "dfloat": 2}
+    up = ta if rank[ta] > rank[tb] else tb
+    rng = np.random.default_rng(613)
+
+    def draw(t, shape):
+        if t == "int32":
+            v = rng.integers(-(1 << 30), 1 << 30, size=shape).astype(np.int32)   # beyond 2^24: the conversion to float rounds
+            v[v == 0] = 7
+            return v
+        return ((rng.standard_normal(shape) + 3.0) * 10.0 ** rng.integers(-3, 4, size=shape)).astype(npdt[t])
+
+    for shape in [(1,), (5,), (4096,), (4099,), (33, 65), (3, 5, 128), ((1 << 20) + 3,), (2048, 4096)]:
+        hx, hy = draw(ta, shape), draw(tb, shape)
+        x, y = cls_of(ta).cast(hx), cls_of(tb).cast(hy)
+        ux, uy = hx.astype(npdt[up]), hy.astype(npdt[up])
+        for op in ("add", "sub", "mul", "div"):
+            r = getattr(x, PYOP[op])(y)
+            assert r.type_name == up and tuple(r.shape) == tuple(shape)
+            with np.errstate(all="ignore"):
+                assert_bits_equal(r.to_numpy(), oracle.binary(op, ux, uy), (op, shape))
+            # the same through the higher type's own operation on arrays cast beforehand
+            assert_bits_equal(r.to_numpy(), getattr(cls_of(up).cast(x), PYOP[op])(cls_of(up).cast(y)).to_numpy(), (op, shape, "cast first"))
+    # layouts that cast first: a start off a 16-byte boundary, a transposed operand, a repeated row, a strided slice
+    hx, hy = draw(ta, (130, 260)), draw(tb, (130, 260))
+    x, y = cls_of(ta).cast(hx), cls_of(tb).cast(hy)
+    cases = [(x.reshape(130 * 260)[1:], y.reshape(130 * 260)[:-1], hx.reshape(-1)[1:], hy.reshape(-1)[:-1]),
+             (x[:, 1:], y[:, :-1], hx[:, 1:], hy[:, :-1]),
+             (x, y[:1, :], hx, hy[:1, :]),
+             (x[::2], y[1::2], hx[::2], hy[1::2])]
+    hs, ht = draw(ta, (260, 130)), None
+    cases.append((cls_of(ta).cast(hs).transpose(), y, hs.T, hy))
+    for dx, dy, ax, ay in cases:
+        for op in ("add", "mul", "div"):
+            with np.errstate(all="ignore"):
+                want = oracle.binary(op, np.ascontiguousarray(ax).astype(npdt[up]), np.ascontiguousarray(np.broadcast_to(ay, ax.shape)).astype(npdt[up]))
+            assert_bits_equal(getattr(dx, PYOP[op])(dy).to_numpy(), want, (op, ax.shape))
+
+
 def test_fill_and_store_into_views():
     cls = cls_of("sfloat")
     a = cls.zeros(6, 8)
