@@ -167,6 +167,7 @@ _sig = {
     "cumo_hip_make_reduction_arg": (None, [P(Loop), P(ReductionArg)]),
     "cumo_hip_na_binary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_binary_s": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
+    "cumo_hip_na_binary_fs": (C.c_int, [C.c_char_p, P(NArrayDesc), C.c_double, C.c_int, P(NArrayDesc)]),
     "cumo_hip_na_unary": (C.c_int, [C.c_char_p, P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_pow": (C.c_int, [P(NArrayDesc), P(NArrayDesc), P(NArrayDesc)]),
     "cumo_hip_na_pow_s": (C.c_int, [P(NArrayDesc), C.c_double, C.c_int, C.c_int, P(NArrayDesc)]),

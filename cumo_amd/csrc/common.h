@@ -52,6 +52,8 @@ int bit_count_cols_words_launch(const cumo_hip_bit_count_nd_t* counts);
 // (SFloat / DFloat / Int32), converted to the result's type on the way in, into z of that type (ew_mixed.hip).
 // False when the pair of types or the alignment is not one it takes; nothing is launched then.
 bool mixed_flat_binary(int op, int ta, const char* x, int tb, const char* y, char* z, uint64_t n);
+// the same for a contiguous Int32 run and one DFloat number (on the left when scalar_is_left), into a DFloat run
+bool mixed_flat_binary_s(int op, const char* x, double sv, bool scalar_is_left, char* z, uint64_t n);
 
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)

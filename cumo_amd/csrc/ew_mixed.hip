@@ -11,7 +11,10 @@
 namespace cumo_hip {
 namespace {
 
-constexpr int kMxBlock = 256, kMxVec = 4;
+constexpr int kMxBlock = 256;
+// elements a vector: the result's 16 bytes (a lane's store is one 128-bit access next to its neighbours'; with four DFloat
+// results a lane, every store instruction of a wave wrote every other 16 bytes of its span: SFloat + DFloat 0.69 of peak)
+template <class TR> struct MxVec { static constexpr int value = 16 / (int)sizeof(TR); };
 
 template <int OP, class T>
 __device__ __forceinline__ T mixed_apply(T a, T b) {
@@ -24,6 +27,7 @@ __device__ __forceinline__ T mixed_apply(T a, T b) {
 template <int OP, class TA, class TB, class TR, bool NT, int kMxUnr>
 __global__ __launch_bounds__(kMxBlock) void ew_mixed_flat_kernel(const char* __restrict__ px, const char* __restrict__ py,
                                                                  char* __restrict__ pz, uint64_t n) {
+    constexpr int kMxVec = MxVec<TR>::value;
     const uint64_t i0 = ((uint64_t)blockIdx.x * (kMxBlock * kMxUnr) + threadIdx.x) * kMxVec;
     TA xv[kMxUnr][kMxVec];
     TB yv[kMxUnr][kMxVec];
@@ -55,12 +59,54 @@ __global__ __launch_bounds__(kMxBlock) void ew_mixed_flat_kernel(const char* __r
 
 template <int OP, class TA, class TB, class TR>
 void mixed_launch(const char* x, const char* y, char* z, uint64_t n) {
-    constexpr int kMxUnr = sizeof(TR) == 8 ? 2 : 4;   // vectors of four elements a lane has in flight per operand
+    constexpr int kMxUnr = 4, kMxVec = MxVec<TR>::value;   // vectors a lane has in flight per operand
     const uint64_t per_block = (uint64_t)kMxBlock * kMxUnr * kMxVec;
     const dim3 g((unsigned)((n + per_block - 1) / per_block)), b(kMxBlock);
     const bool nt = stream_past_caches(n * (sizeof(TA) + sizeof(TB) + sizeof(TR)));
     if (nt) hipLaunchKernelGGL((ew_mixed_flat_kernel<OP, TA, TB, TR, true, kMxUnr>), g, b, 0, current_stream(), x, y, z, n);
     else hipLaunchKernelGGL((ew_mixed_flat_kernel<OP, TA, TB, TR, false, kMxUnr>), g, b, 0, current_stream(), x, y, z, n);
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+// Int32 array op one DFloat number (a Ruby Float meets an Int32 array: the array is computed in DFloat,
+// gen/def/int32.rb upcast table), the number on the right or, with LEFT, on the left.
+template <int OP, bool LEFT, bool NT>
+__global__ __launch_bounds__(kMxBlock) void ew_mixed_scalar_kernel(const char* __restrict__ px, double sv, char* __restrict__ pz, uint64_t n) {
+    constexpr int U = 4, kMxVec = MxVec<double>::value;
+    const uint64_t i0 = ((uint64_t)blockIdx.x * (kMxBlock * U) + threadIdx.x) * kMxVec;
+    int32_t xv[U][kMxVec];
+    bool whole[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t i = i0 + (uint64_t)u * (kMxBlock * kMxVec);
+        whole[u] = i + kMxVec <= n;
+        if (whole[u]) raw_load<int32_t, kMxVec, NT>(px + i * sizeof(int32_t), xv[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t i = i0 + (uint64_t)u * (kMxBlock * kMxVec);
+        if (whole[u]) {
+            double zv[kMxVec];
+#pragma unroll
+            for (int j = 0; j < kMxVec; ++j)
+                zv[j] = LEFT ? mixed_apply<OP, double>(sv, (double)xv[u][j]) : mixed_apply<OP, double>((double)xv[u][j], sv);
+            raw_store<double, kMxVec, NT>(pz + i * sizeof(double), zv);
+        } else if (i < n) {
+            for (uint64_t k = i; k < n; ++k) {
+                const double x = (double)reinterpret_cast<const int32_t*>(px)[k];
+                reinterpret_cast<double*>(pz)[k] = LEFT ? mixed_apply<OP, double>(sv, x) : mixed_apply<OP, double>(x, sv);
+            }
+        }
+    }
+}
+
+template <int OP, bool LEFT>
+void mixed_scalar_launch(const char* x, double sv, char* z, uint64_t n) {
+    const uint64_t per_block = (uint64_t)kMxBlock * 4 * MxVec<double>::value;
+    const dim3 g((unsigned)((n + per_block - 1) / per_block)), b(kMxBlock);
+    const bool nt = stream_past_caches(n * (sizeof(int32_t) + sizeof(double)));
+    if (nt) hipLaunchKernelGGL((ew_mixed_scalar_kernel<OP, LEFT, true>), g, b, 0, current_stream(), x, sv, z, n);
+    else hipLaunchKernelGGL((ew_mixed_scalar_kernel<OP, LEFT, false>), g, b, 0, current_stream(), x, sv, z, n);
     cumo_cuda_runtime_check_kernel_launch();
 }
 
@@ -80,13 +126,29 @@ bool mixed_by_types(int ta, int tb, const char* x, const char* y, char* z, uint6
 }  // namespace
 
 bool mixed_flat_binary(int op, int ta, const char* x, int tb, const char* y, char* z, uint64_t n) {
-    if (n == 0 || n >= ((uint64_t)1 << 43)) return false;  // (the grid's x dimension: 2^31 blocks of 2^12 elements)
+    if (n == 0 || n >= ((uint64_t)1 << 42)) return false;  // (the grid's x dimension: 2^31 blocks of 2^11 elements or more)
     if ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15u) != 0) return false;
     switch (op) {
         case 0: return mixed_by_types<0>(ta, tb, x, y, z, n);
         case 1: return mixed_by_types<1>(ta, tb, x, y, z, n);
         case 2: return mixed_by_types<2>(ta, tb, x, y, z, n);
         case 3: return mixed_by_types<3>(ta, tb, x, y, z, n);
+    }
+    return false;
+}
+
+bool mixed_flat_binary_s(int op, const char* x, double sv, bool scalar_is_left, char* z, uint64_t n) {
+    if (n == 0 || n >= ((uint64_t)1 << 42)) return false;
+    if ((((uintptr_t)x | (uintptr_t)z) & 15u) != 0) return false;
+    switch (op * 2 + (scalar_is_left ? 1 : 0)) {
+        case 0: mixed_scalar_launch<0, false>(x, sv, z, n); return true;
+        case 1: mixed_scalar_launch<0, true>(x, sv, z, n); return true;
+        case 2: mixed_scalar_launch<1, false>(x, sv, z, n); return true;
+        case 3: mixed_scalar_launch<1, true>(x, sv, z, n); return true;
+        case 4: mixed_scalar_launch<2, false>(x, sv, z, n); return true;
+        case 5: mixed_scalar_launch<2, true>(x, sv, z, n); return true;
+        case 6: mixed_scalar_launch<3, false>(x, sv, z, n); return true;
+        case 7: mixed_scalar_launch<3, true>(x, sv, z, n); return true;
     }
     return false;
 }

@@ -1094,6 +1094,51 @@ int cumo_hip_na_binary_s(const char* op, const cumo_hip_narray_t* x, double sv, 
     return rc;
 }
 
+// x op sv for a number that is a Ruby Float: a float array keeps its type, an Int32 array is computed in DFloat
+// (the upcast table of gen/def/int32.rb) -- in one launch that converts on the way in where the array is one
+// contiguous, aligned run and the operation is + - * /, through a DFloat copy of the array otherwise.
+int cumo_hip_na_binary_fs(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z) {
+    int rc = check_arith(x);
+    if (rc) return rc;
+    if (x->type != CUMO_HIP_INT32) return cumo_hip_na_binary_s(op, x, sv, scalar_is_left, z);
+    const BinaryRow* row = find_row(kBinary, op);
+    if (!row || !binary_has(row, CUMO_HIP_DFLOAT, true)) return no_method(op);
+    int code = -1;
+    if (!std::strcmp(op, "add")) code = 0;
+    else if (!std::strcmp(op, "sub")) code = 1;
+    else if (!std::strcmp(op, "mul")) code = 2;
+    else if (!std::strcmp(op, "div")) code = 3;
+    static const bool off = [] {
+        const char* e = std::getenv("CUMO_HIP_MIXED_ONE_LAUNCH");
+        return e && e[0] == '0';
+    }();
+    const size_t n = total_of(x);
+    if (code >= 0 && !off && z && x->ndim >= 1 && n > 0 && is_contiguous(x) && (((uintptr_t)(x->ptr + x->offset)) & 15u) == 0) {
+        const bool fresh = z->ptr == NULL;
+        bool fits = true;
+        if (!fresh) {
+            fits = z->type == CUMO_HIP_DFLOAT && z->ndim == x->ndim && is_contiguous(z) && (((uintptr_t)(z->ptr + z->offset)) & 15u) == 0;
+            for (int d = 0; fits && d < x->ndim; d++) fits = z->shape[d] == x->shape[d];
+        } else {
+            rc = cumo_hip_na_alloc(z, CUMO_HIP_DFLOAT, x->ndim, x->shape);
+            if (rc) return rc;
+        }
+        if (fits) {
+            if (cumo_hip::mixed_flat_binary_s(code, x->ptr + x->offset, sv, scalar_is_left != 0, z->ptr + z->offset, n)) return CUMO_HIP_OK;
+            if (fresh) {
+                cumo_cuda_runtime_free(z->ptr);
+                z->ptr = NULL;
+            }
+        }
+    }
+    NA tx;
+    const NA* ux;
+    rc = cast_operand(x, CUMO_HIP_DFLOAT, &tx, &ux);
+    if (!rc) rc = cumo_hip_na_binary_s(op, ux, sv, scalar_is_left, z);
+    free_tmp(&tx);
+    return rc;
+}
+
 // x ** y for two arrays (gen/tmpl/pow.c:117-190,200-215): the result has the higher
 // type of the two; an Int32 exponent array takes the repeated-product form.
 int cumo_hip_na_pow(const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z) {

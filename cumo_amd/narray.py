@@ -651,6 +651,11 @@ class _Numeric(NArray):
         z = NArrayDesc()
         if isinstance(other, numbers.Number):
             # reference: gen/tmpl/binary.c:184-209 -- the number rides in the launch
+            if isinstance(other, float) and not self.is_float and op in ("add", "sub", "mul", "div"):
+                # (the library moves the array to DFloat: in the same launch where it is one contiguous run)
+                x = self._desc()
+                return _run(_L.cumo_hip_na_binary_fs, op.encode(), C.byref(x), float(other), 1 if scalar_is_left else 0,
+                            C.byref(z), results=(z,))
             x = self._scalar_operand(other)._desc()
             return _run(_L.cumo_hip_na_binary_s, op.encode(), C.byref(x), float(other), 1 if scalar_is_left else 0,
                         C.byref(z), results=(z,))

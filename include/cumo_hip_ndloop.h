@@ -158,6 +158,11 @@ void cumo_hip_make_reduction_arg(const cumo_hip_loop_t* lp, cumo_na_reduction_ar
 int cumo_hip_na_binary(const char* op, const cumo_hip_narray_t* x, const cumo_hip_narray_t* y, cumo_hip_narray_t* z);
 /* z = x op sv (or sv op x when scalar_is_left); the scalar rides in the launch. */
 int cumo_hip_na_binary_s(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z);
+/* The same for a number that is a Ruby Float: a float array keeps its type, an Int32 array
+ * answers DFloat (reference: the upcast table of gen/def/int32.rb:22-23 through
+ * gen/tmpl/binary.c:184-209, which casts the array first; here one launch converts on
+ * the way in where the array is one contiguous run). */
+int cumo_hip_na_binary_fs(const char* op, const cumo_hip_narray_t* x, double sv, int scalar_is_left, cumo_hip_narray_t* z);
 /* z = op(x): minus reciprocal sign square abs floor round ceil trunc rint bit_not.
  * Int32 reciprocal / abs report CUMO_HIP_ERROR_ZERO_DIVISION / CUMO_HIP_ERROR_ARGUMENT
  * for 1/0 and |INT_MIN| (reference: gen/tmpl/unary.c:76-119, unary2.c). */

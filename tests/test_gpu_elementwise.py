@@ -651,6 +651,37 @@ def test_arithmetic_on_two_element_types(ta, tb):
             assert_bits_equal(getattr(dx, PYOP[op])(dy).to_numpy(), want, (op, ax.shape))
 
 
+def test_int32_array_with_a_float_number_answers_dfloat():
+    """An Int32 array meeting a Ruby Float is computed in DFloat (gen/def/int32.rb:22-23): the bits of casting the array
+    first and running DFloat's scalar form, for contiguous arrays (one launch) and for views (cast first)."""
+    import cumo_amd
+    rng = np.random.default_rng(617)
+    for shape in [(1,), (7,), (4096,), (4101,), (33, 65), ((1 << 20) + 1,), (2048, 2048)]:
+        h = rng.integers(-(1 << 31), 1 << 31, size=shape).astype(np.int32)
+        h[h == 0] = 3
+        d = cumo_amd.Int32.cast(h)
+        hd = h.astype(np.float64)
+        for op in ("add", "sub", "mul", "div"):
+            for sv in (2.5, -1.0 / 3.0):
+                r = getattr(d, PYOP[op])(sv)
+                assert isinstance(r, cumo_amd.DFloat) and tuple(r.shape) == tuple(shape)
+                assert_bits_equal(r.to_numpy(), oracle.binary(op, hd, sv), (op, shape, sv))
+                r = getattr(d, RPYOP[op])(sv)
+                assert isinstance(r, cumo_amd.DFloat)
+                assert_bits_equal(r.to_numpy(), oracle.binary(op, sv, hd, scalar_is_left=True), (op, shape, sv, "number on the left"))
+    h = rng.integers(-1000, 1000, size=(130, 260)).astype(np.int32)
+    h[h == 0] = 3
+    d = cumo_amd.Int32.cast(h)
+    for dv, hv in ((d[:, 1:], h[:, 1:]), (d.transpose(), h.T), (d[::2, ::3], h[::2, ::3]), (d.reshape(130 * 260)[1:], h.reshape(-1)[1:])):
+        hd = np.ascontiguousarray(hv).astype(np.float64)
+        assert_bits_equal((dv * 0.3).to_numpy(), oracle.binary("mul", hd, 0.3))
+        assert_bits_equal((2.5 / dv).to_numpy(), oracle.binary("div", 2.5, hd, scalar_is_left=True))
+    # an integer number keeps the array Int32; other operations with a Float still answer DFloat
+    assert isinstance(d * 3, cumo_amd.Int32)
+    assert isinstance(d % 2.5, cumo_amd.DFloat)
+    assert_bits_equal((d % 2.5).to_numpy(), oracle.binary("mod", h.astype(np.float64), 2.5))
+
+
 def test_fill_and_store_into_views():
     cls = cls_of("sfloat")
     a = cls.zeros(6, 8)
