@@ -55,6 +55,9 @@ bool mixed_flat_binary(int op, int ta, const char* x, int tb, const char* y, cha
 // the same for a contiguous Int32 run and one DFloat number (on the left when scalar_is_left), into a DFloat run
 bool mixed_flat_binary_s(int op, const char* x, double sv, bool scalar_is_left, char* z, uint64_t n);
 
+// x cmp y (cmp: 0 == 1 != 2 > 3 >= 4 < 5 <=) for two such runs into the bits of z from its first word on
+bool mixed_flat_compare(int cmp, int ta, const char* x, int tb, const char* y, CUMO_BIT_DIGIT* z, uint64_t n);
+
 // CUMO_HIP_FORCE_WIDE=1 (read once): every launch takes the 64-bit index arithmetic of the
 // general kernels, whatever the array's size, and the lean kernels (which are 32-bit only)
 // stand aside. For tests: the wide paths otherwise only run on arrays beyond 2^32 elements.

@@ -7,6 +7,7 @@
 #include "common.h"
 #include "cumo_hip_ndloop.h"
 #include "ew_kernels.h"
+#include "ew_ops.h"
 
 namespace cumo_hip {
 namespace {
@@ -123,7 +124,63 @@ bool mixed_by_types(int ta, int tb, const char* x, const char* y, char* z, uint6
     return true;
 }
 
+// Comparisons of two arrays of different element types into Bit: the flat Bit kernel of ew_kernels.h (four elements a
+// lane, a group of eight lanes gathers a word, four words stored as one access) with an operator that converts both
+// sides to the higher type first, as the cast the reference makes would (gen/tmpl/cond_binary.c:1-55).
+template <int CMP, class TA, class TB, class TU>
+struct OpCmpMixed { CUMO_HIP_OP_COMMON(TA, TB, uint32_t, 2, true, false)
+    __device__ __forceinline__ bool operator()(TA xa, TB yb, uint32_t& z) const {
+        const TU x = (TU)xa, y = (TU)yb;
+        bool r;
+        if (CMP == 0) r = x == y;
+        else if (CMP == 1) r = x != y;
+        else if (CMP == 2) r = x > y;
+        else if (CMP == 3) r = x >= y;
+        else if (CMP == 4) r = x < y;
+        else r = x <= y;
+        z = r ? 1u : 0u;
+        return true; } };
+
+template <int CMP, class TA, class TB, class TU>
+void mixed_compare_launch(const char* x, const char* y, CUMO_BIT_DIGIT* z, uint64_t n) {
+    typedef OpCmpMixed<CMP, TA, TB, TU> Op;
+    constexpr int VB = 4;
+    const uint64_t groups = (n + 127) / 128;
+    const uint64_t blocks = (groups * (32 / VB) + kEwBlock - 1) / kEwBlock;
+    const dim3 g((unsigned)blocks), b(kEwBlock);
+    const bool nt = stream_past_caches(n * (sizeof(TA) + sizeof(TB)));
+    if (nt) hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, true>), g, b, 0, current_stream(), x, y, z, n, 0, Op{}, TA());
+    else hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, false>), g, b, 0, current_stream(), x, y, z, n, 0, Op{}, TA());
+    cumo_cuda_runtime_check_kernel_launch();
+}
+
+template <int CMP>
+bool mixed_compare_by_types(int ta, int tb, const char* x, const char* y, CUMO_BIT_DIGIT* z, uint64_t n) {
+    if (ta == CUMO_HIP_SFLOAT && tb == CUMO_HIP_DFLOAT) mixed_compare_launch<CMP, float, double, double>(x, y, z, n);
+    else if (ta == CUMO_HIP_DFLOAT && tb == CUMO_HIP_SFLOAT) mixed_compare_launch<CMP, double, float, double>(x, y, z, n);
+    else if (ta == CUMO_HIP_INT32 && tb == CUMO_HIP_SFLOAT) mixed_compare_launch<CMP, int32_t, float, float>(x, y, z, n);
+    else if (ta == CUMO_HIP_SFLOAT && tb == CUMO_HIP_INT32) mixed_compare_launch<CMP, float, int32_t, float>(x, y, z, n);
+    else if (ta == CUMO_HIP_INT32 && tb == CUMO_HIP_DFLOAT) mixed_compare_launch<CMP, int32_t, double, double>(x, y, z, n);
+    else if (ta == CUMO_HIP_DFLOAT && tb == CUMO_HIP_INT32) mixed_compare_launch<CMP, double, int32_t, double>(x, y, z, n);
+    else return false;
+    return true;
+}
+
 }  // namespace
+
+bool mixed_flat_compare(int cmp, int ta, const char* x, int tb, const char* y, CUMO_BIT_DIGIT* z, uint64_t n) {
+    if (n == 0 || n >= ((uint64_t)1 << 40)) return false;
+    if ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15u) != 0) return false;
+    switch (cmp) {
+        case 0: return mixed_compare_by_types<0>(ta, tb, x, y, z, n);
+        case 1: return mixed_compare_by_types<1>(ta, tb, x, y, z, n);
+        case 2: return mixed_compare_by_types<2>(ta, tb, x, y, z, n);
+        case 3: return mixed_compare_by_types<3>(ta, tb, x, y, z, n);
+        case 4: return mixed_compare_by_types<4>(ta, tb, x, y, z, n);
+        case 5: return mixed_compare_by_types<5>(ta, tb, x, y, z, n);
+    }
+    return false;
+}
 
 bool mixed_flat_binary(int op, int ta, const char* x, int tb, const char* y, char* z, uint64_t n) {
     if (n == 0 || n >= ((uint64_t)1 << 42)) return false;  // (the grid's x dimension: 2^31 blocks of 2^11 elements or more)

@@ -1043,6 +1043,48 @@ int mixed_one_launch(const char* op, const NA* x, const NA* y, int up, NA* z, bo
     return CUMO_HIP_OK;
 }
 
+// == != > >= < <= of two such arrays into a fresh Bit result (or a given whole contiguous one) the same way
+int mixed_compare_one_launch(const char* op, const NA* x, const NA* y, NA* z, bool* taken) {
+    *taken = false;
+    static const char* const names[6] = {"eq", "ne", "gt", "ge", "lt", "le"};
+    int code = -1;
+    for (int k = 0; k < 6; k++)
+        if (!std::strcmp(op, names[k])) code = k;
+    static const bool off = [] {
+        const char* e = std::getenv("CUMO_HIP_MIXED_ONE_LAUNCH");
+        return e && e[0] == '0';
+    }();
+    if (code < 0 || off || !z || x->ndim != y->ndim || x->ndim < 1) return CUMO_HIP_OK;
+    for (int d = 0; d < x->ndim; d++)
+        if (x->shape[d] != y->shape[d]) return CUMO_HIP_OK;
+    const size_t n = total_of(x);
+    if (n == 0 || !is_contiguous(x) || !is_contiguous(y)) return CUMO_HIP_OK;
+    const char* px = x->ptr + x->offset;
+    const char* py = y->ptr + y->offset;
+    if ((((uintptr_t)px | (uintptr_t)py) & 15u) != 0) return CUMO_HIP_OK;
+    const bool fresh = z->ptr == NULL;
+    if (!fresh) {
+        if (z->type != CUMO_HIP_BIT || z->ndim != x->ndim || z->offset != 0 || !is_contiguous(z) || (((uintptr_t)z->ptr) & 15u) != 0) return CUMO_HIP_OK;
+        for (int d = 0; d < x->ndim; d++)
+            if (z->shape[d] != x->shape[d]) return CUMO_HIP_OK;
+    } else {
+        const int rc = cumo_hip_na_alloc(z, CUMO_HIP_BIT, x->ndim, x->shape);
+        if (rc != CUMO_HIP_OK) {
+            *taken = true;
+            return rc;
+        }
+    }
+    if (cumo_hip::mixed_flat_compare(code, x->type, px, y->type, py, reinterpret_cast<CUMO_BIT_DIGIT*>(z->ptr), n)) {
+        *taken = true;
+        return CUMO_HIP_OK;
+    }
+    if (fresh) {
+        cumo_cuda_runtime_free(z->ptr);
+        z->ptr = NULL;
+    }
+    return CUMO_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -2000,6 +2042,11 @@ int cumo_hip_na_compare(const char* op, const cumo_hip_narray_t* x, const cumo_h
     const CondRow* row = find_row(kCond, op);
     const int up = upcast(x->type, y->type);
     if (!row || !cond_has(row, up)) return no_method(op);
+    if (x->type != y->type) {
+        bool taken = false;
+        rc = mixed_compare_one_launch(op, x, y, z, &taken);
+        if (taken) return rc;
+    }
     NA tx, ty;
     const NA *ux, *uy;
     rc = cast_operand(x, up, &tx, &ux);

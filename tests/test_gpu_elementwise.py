@@ -651,6 +651,45 @@ def test_arithmetic_on_two_element_types(ta, tb):
             assert_bits_equal(getattr(dx, PYOP[op])(dy).to_numpy(), want, (op, ax.shape))
 
 
+@pytest.mark.parametrize("ta,tb", MIXED_PAIRS)
+def test_comparisons_of_two_element_types(ta, tb):
+    """x cmp y for arrays of different types compares in the higher type (an Int32 beyond 2^24 is rounded to SFloat
+    first, as the cast the reference makes rounds it): contiguous arrays in one launch, views through the cast."""
+    npdt = {"sfloat": np.float32, "dfloat": np.float64, "int32": np.int32}
+    rank = {"int32": 0, "sfloat": 1, "dfloat": 2}
+    up = npdt[ta if rank[ta] > rank[tb] else tb]
+    rng = np.random.default_rng(619)
+
+    def draw(t, shape):
+        if t == "int32":
+            v = rng.integers(-4, 5, size=shape).astype(np.int32)
+            big = rng.random(shape) < 0.1
+            v[big] = 16777217 + rng.integers(-2, 3, size=shape)[big]     # around 2^24 + 1: not all representable in float
+            return v
+        v = rng.integers(-4, 5, size=shape).astype(npdt[t])
+        big = rng.random(shape) < 0.1
+        v[big] = np.asarray(16777217 + rng.integers(-2, 3, size=shape), dtype=npdt[t])[big]
+        if shape != (1,):
+            v.reshape(-1)[1] = np.nan
+        return v
+
+    for shape in [(1,), (31,), (128,), (129,), (1000,), (4096,), (37, 65), (3, 5, 96), ((1 << 20) + 77,), (2048, 4096)]:
+        hx, hy = draw(ta, shape), draw(tb, shape)
+        x, y = cls_of(ta).cast(hx), cls_of(tb).cast(hy)
+        for op in ("eq", "ne", "gt", "ge", "lt", "le"):
+            got = getattr(x, op)(y)
+            assert tuple(got.shape) == tuple(shape)
+            with np.errstate(all="ignore"):
+                want = oracle.compare(op, hx.astype(up), hy.astype(up))
+            assert (got.to_numpy() == want).all(), (op, shape)
+    hx, hy = draw(ta, (130, 260)), draw(tb, (130, 260))
+    x, y = cls_of(ta).cast(hx), cls_of(tb).cast(hy)
+    for dx, dy, ax, ay in ((x[:, 1:], y[:, :-1], hx[:, 1:], hy[:, :-1]), (x, y[:1, :], hx, hy[:1, :]), (x.transpose(), y.transpose(), hx.T, hy.T)):
+        for op in ("eq", "gt", "le"):
+            want = oracle.compare(op, np.ascontiguousarray(ax).astype(up), np.ascontiguousarray(np.broadcast_to(ay, ax.shape)).astype(up))
+            assert (getattr(dx, op)(dy).to_numpy() == want).all(), (op, ax.shape)
+
+
 def test_int32_array_with_a_float_number_answers_dfloat():
     """An Int32 array meeting a Ruby Float is computed in DFloat (gen/def/int32.rb:22-23): the bits of casting the array
     first and running DFloat's scalar form, for contiguous arrays (one launch) and for views (cast first)."""
