@@ -95,7 +95,8 @@ def inputs_c4(n=8192):
 def inputs_next(shape=(8192, 4096)):
     rng = np.random.default_rng(5)
     return {"x": rng.standard_normal(shape, dtype=np.float32), "y": rng.standard_normal(shape, dtype=np.float32),
-            "rows": rng.integers(0, shape[0], shape[0]), "perm": rng.permutation(shape[0])}
+            "rows": rng.integers(0, shape[0], shape[0]), "perm": rng.permutation(shape[0]),
+            "d": rng.standard_normal(shape), "i": rng.integers(-1000, 1000, size=shape).astype(np.int32)}
 
 
 def inputs_c5(s_shape=(32, 16, 512, 512), x_shape=(8192, 4096)):
@@ -183,6 +184,8 @@ def config_ops(name, cumo, host):
         x, y = host["x"], host["y"]
         env = {"x": cumo.SFloat.cast(x), "y": cumo.SFloat.cast(y), "b": cumo.SFloat.cast(y)}
         env["mask"] = env["x"] > 0.5
+        env["d"] = cumo.DFloat.cast(host["d"])
+        env["i"] = cumo.Int32.cast(host["i"])
         env["rows"] = host["rows"]
         env["perm"] = host["perm"]
         n, nb = x.size, x.nbytes
@@ -201,6 +204,10 @@ def config_ops(name, cumo, host):
             ("x[rows,true] (gather)", lambda e: e.__setitem__("g", e["x"][e["rows"]]), 2 * nb + 8 * r, n),
             ("x[perm,true] (gather, every row once)", lambda e: e.__setitem__("g", e["x"][e["perm"]]), 2 * nb + 8 * r, n),
             ("b[perm,true]=x (scatter)", lambda e: e["b"].__setitem__(e["perm"], e["x"]), 2 * nb + 8 * r, n),
+            # two element types: the bytes the operation is defined over (each input once, the result once)
+            ("x+d (SFloat+DFloat)", lambda e: e.__setitem__("xd", e["x"] + e["d"]), 5 * nb, n),
+            ("i*0.5 (Int32 by Float)", lambda e: e.__setitem__("ih", e["i"] * 0.5), 3 * nb, n),
+            ("x>d into Bit", lambda e: e.__setitem__("xgd", e["x"] > e["d"]), 3 * nb + n // 8, n),
         ]
     if name == "odd":
         # the hot-path operations on a matrix whose rows are not a whole number of 128-bit vectors (4095 SFloat:
@@ -310,7 +317,7 @@ WORKLOAD_TEXT = {
     "c1_large": "C1 at n=2^26 (256 MiB per array)",
     "c2_large": "C2 at 8192 x 8192 (512 MiB per matrix)",
     "c3_large": "C3 at [256,512,1024] (512 MiB)",
-    "next": "operations beside the five configs on SFloat [8192,4096]: mulsum, clip, maximum, integer power, cumsum, where, a[mask], row gather and scatter through index arrays",
+    "next": "operations beside the five configs on SFloat [8192,4096]: mulsum, clip, maximum, integer power, cumsum, where, a[mask], row gather and scatter through index arrays, arithmetic and comparison of two element types",
     "odd": "the hot-path operations on SFloat [8192,4095]: rows that are not a whole number of 128-bit vectors and start off 16-byte boundaries",
     "bit": "Bit [16384,32768] (64 MiB): logic on whole arrays and on windows, counts of the whole, along rows and down columns, all?; stores between Bit and SFloat [8192,4096]",
     "bit_large": "the Bit logic and counts at [32768,65536] (256 MiB), where a launch's fixed start and drain weigh a quarter of what they do at 64 MiB",
