@@ -118,15 +118,23 @@ def _reduce_mask(ndim, axis):
 
 
 def _is_index_array(k):
+    # (a Bit array in a key of several entries selects the positions where it is set: narray/index.c:160-165)
     if isinstance(k, (list, np.ndarray, range)):
         return True
-    return isinstance(k, NArray) and type(k).__name__ != "Bit"
+    return isinstance(k, NArray)
 
 
 def _index_positions(k, n):
     """Positions one index array selects in a dimension of n elements, as the
     reference parses them on the host (narray/index.c:112-142,201-233): 1-D,
     negative values count from the end, out of range raises IndexError."""
+    if isinstance(k, NArray) and type(k).__name__ == "Bit":
+        # a Bit array stands for the positions where it is set (narray/index.c:156-166)
+        if k.ndim != 1:
+            raise IndexError("should be 1-d NArray")
+        if k.size != n:
+            raise IndexError("Bit-NArray size mismatch")
+        k = k.where()
     arr = np.asarray(k.to_numpy() if isinstance(k, NArray) else (list(k) if isinstance(k, range) else k))
     if arr.size == 0:
         return np.zeros(0, dtype=np.uint64)
@@ -306,8 +314,8 @@ class NArray:
     def __setitem__(self, key, value):
         """a[key] = value: a store into the view, or a scatter when the key holds
         index arrays (reference: gen/tmpl/aset.c, narray/ndloop.c:1316)."""
-        if isinstance(key, NArray) and type(key).__name__ == "Bit":
-            raise TypeError("store through a mask is outside this path")
+        if isinstance(key, NArray) and type(key).__name__ == "Bit" and (key.ndim != 1 or self.ndim != 1):
+            raise TypeError("a store through a mask of several dimensions is outside this path")
         key = self._expand_key(key)
         if any(_is_index_array(k) for k in key):
             return self._scatter(key, value)

@@ -365,3 +365,41 @@ def test_gather_of_more_than_two_to_the_31_elements():
     assert int(whole.sum(dtype=np.uint64)) == outer * int(want_row.sum(dtype=np.uint64))
     assert (whole.reshape(outer, inner)[::4099] == want_row).all()
     free(psrc, pidx, pbuf)
+
+
+@pytest.mark.parametrize("tname,dt", [("SFloat", np.float32), ("DFloat", np.float64), ("Int32", np.int32)])
+def test_a_bit_array_as_the_index_of_one_dimension(tname, dt):
+    """A 1-D Bit array among the keys selects the positions where it is set (narray/index.c:156-166 turns it into
+    its `where`); the literals are test/narray_test.rb:373-375. A store through such a key scatters."""
+    import cumo_amd
+    cls = getattr(cumo_amd, tname)
+    h = np.array([[1, 2, 3], [5, 7, 11]], dtype=dt)
+    a = cls.cast(h)
+    assert a[a[:, 2] < 5, :].to_numpy().tolist() == [[1, 2, 3]]
+    assert a[:, a[1, :] > 5].to_numpy().tolist() == [[2, 3], [7, 11]]
+    if dt == np.int32:
+        assert a[:, (a[0, :] % 2).eq(1)].to_numpy().tolist() == [[1, 3], [5, 11]]
+    with pytest.raises(IndexError):
+        a[:, a[:, 0] > 0]          # two bits for a dimension of three: "Bit-NArray size mismatch"
+    rng = np.random.default_rng(631)
+    hx = rng.integers(-50, 50, size=(300, 517)).astype(dt)
+    x = cls.cast(hx)
+    rows, cols = hx[:, 3] > 0, hx[7, :] < 10
+    assert_bits_equal(x[x[:, 3] > 0, :].to_numpy(), hx[rows, :])
+    assert_bits_equal(x[:, x[7, :] < 10].to_numpy(), hx[:, cols])
+    assert_bits_equal(x[x[:, 3] > 0, x[7, :] < 10].to_numpy(), hx[np.ix_(rows, cols)])
+    # stores: rows picked by a mask, and a 1-D array through its own mask
+    want = hx.copy()
+    want[rows, :] = 0
+    x[x[:, 3] > 0, :] = 0
+    assert_bits_equal(x.to_numpy(), want)
+    hv = rng.integers(-50, 50, size=70001).astype(dt)
+    v = cls.cast(hv)
+    neg = v < 0
+    v[neg] = 7
+    wantv = hv.copy()
+    wantv[hv < 0] = 7
+    assert_bits_equal(v.to_numpy(), wantv)
+    v[v.eq(7)] = cls.cast(np.arange(int((wantv == 7).sum()), dtype=dt))
+    wantv[wantv == 7] = np.arange(int((wantv == 7).sum()), dtype=dt)
+    assert_bits_equal(v.to_numpy(), wantv)
