@@ -420,6 +420,32 @@ struct ArgImpl {
         }
         combine(Acc{v, (IDX)(idx0 + first)}, acc);
     }
+    // U consecutive positions (idx0, idx0 + 1, ...) of N neighbouring outputs, every position later than what the
+    // accumulators hold, without a branch: the column kernels' lanes each have outputs of their own, and with a test
+    // per output some lane of the wave nearly always takes the long way. What combine() decides for a later
+    // element: a better number wins; a NaN wins over a number (NAN_WINS) or loses to it; nothing seen yet loses to anything.
+    static constexpr bool COLUMNS_BY_POSITION = true;
+    template <int U, int N>
+    __device__ __forceinline__ void accumulate_columns_by_position(const T (&x)[U][N], int64_t idx0, Acc (&acc)[N]) const {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                const T v = x[u][j];
+                const bool better = IS_MAX ? (acc[j].value < v) : (acc[j].value > v);   // false with a NaN on either side
+                const bool first = acc[j].index == kNone;
+                bool take;
+                if (is_float_t<T>::value) {
+                    const bool an = isnan_t(acc[j].value), nn = isnan_t(v);
+                    take = NAN_WINS ? (better || (nn && !an) || first) : (better || (an && (!nn || first)));
+                } else {
+                    take = better || first;
+                }
+                acc[j].value = take ? v : acc[j].value;
+                acc[j].index = take ? (IDX)(idx0 + u) : acc[j].index;
+            }
+        }
+    }
     // U blocks of N at once (all later than what the accumulator holds): when no
     // element of any of them can change the accumulator, one comparison says so.
     static constexpr bool GROUPED = true;

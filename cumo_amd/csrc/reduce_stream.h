@@ -34,6 +34,11 @@ constexpr uint32_t kRsTicketWords = 16384;  // ticket words per stream slot
 template <class I, class = void> struct folds_columns_together { static constexpr bool value = false; };
 template <class I> struct folds_columns_together<I, decltype((void)I::COLUMNS_TOGETHER)> { static constexpr bool value = I::COLUMNS_TOGETHER; };
 
+// An Impl whose accumulate_columns_by_position<U, VEC>(x[U][VEC], first position, acc[VEC]) folds U consecutive
+// positions of VEC neighbouring outputs without a branch
+template <class I, class = void> struct folds_columns_by_position { static constexpr bool value = false; };
+template <class I> struct folds_columns_by_position<I, decltype((void)I::COLUMNS_BY_POSITION)> { static constexpr bool value = I::COLUMNS_BY_POSITION; };
+
 struct RedSParams {
     const char* in;
     char* out;
@@ -618,6 +623,8 @@ __global__ __launch_bounds__(kRedBlock) void red_scol_kernel(RedSParams p, Impl 
                 if constexpr (folds_columns_together<Impl>::value) {
                     // (the lane's outputs have had the same positions so far: what depends on the count alone is worked out once)
                     impl.template accumulate_columns<U, VEC>(x, acc);
+                } else if constexpr (folds_columns_by_position<Impl>::value) {
+                    impl.template accumulate_columns_by_position<U, VEC>(x, (int64_t)i0, acc);
                 } else {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
