@@ -668,6 +668,11 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(const char* __restric
     // of tiles; tile t goes to block t mod the grid), so that one filling serves them all; every other operator
     // gets a block per tile and runs the body once.
     constexpr bool LOOPS = op_fills_tables<Op>::value;
+    if (TWO && (use_scalar & 4)) {
+        // the scalar operand is an array of one element (x - x.mean): py points at it, the rest is the scalar form
+        sv = *reinterpret_cast<const typename Op::S*>(py);
+        use_scalar &= 3;
+    }
     const uint64_t tiles = LOOPS ? (n + (uint64_t)(kEwBlock * UNR * VEC) - 1) / (uint64_t)(kEwBlock * UNR * VEC) : 0;
     uint64_t tile = blockIdx.x;
     bool first_tile = true;
@@ -817,6 +822,11 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_bit_kernel(const char* __res
     constexpr bool TWO = (NIN == 2);
     constexpr int UNR = 4;
     constexpr unsigned G = 32 / VEC;
+    if (TWO && (use_scalar & 4)) {
+        // the scalar operand is an array of one element: py points at it, the rest is the scalar form
+        sv = *reinterpret_cast<const typename Op::S*>(py);
+        use_scalar &= 3;
+    }
     const uint64_t lane = (uint64_t)blockIdx.x * kEwBlock + threadIdx.x;
     const uint64_t group = lane / G;
     const unsigned k = (unsigned)(lane % G);
@@ -1999,10 +2009,24 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         constexpr int VB = 16 / (int)sizeof(A);
         bool flat = n == 1 && vec == VB && (Op::NIN < 2 || sizeof(B) == sizeof(A)) && plan.step[nops - 1][0] == 1 &&
                     (out_bit->pos % 128) == 0 && ((uintptr_t)out_bit->ptr % 16) == 0;
+        int one_element = -1;   // the slot of an input that is an array of a single element (x.eq(x.max)): read as the scalar
         for (int o = 0; o + 1 < nops && flat; ++o) {
             const int sl = slot[o];
             const int64_t es = sl == 0 ? (int64_t)sizeof(A) : (int64_t)sizeof(B);
+            if (Op::NIN == 2 && std::is_same<A, B>::value && std::is_same<typename Op::S, A>::value && use_scalar == 0 &&
+                plan.step[o][0] == 0 && one_element < 0 && ((uintptr_t)ops[o].ptr % sizeof(A)) == 0) {
+                one_element = sl;
+                continue;
+            }
             flat = plan.step[o][0] == es;
+        }
+        const char* flat_px = kp.ptr[0];
+        const char* flat_py = kp.ptr[1];
+        int flat_scalar = use_scalar;
+        if (flat && one_element >= 0) {
+            flat_px = kp.ptr[1 - one_element];
+            flat_py = kp.ptr[one_element];
+            flat_scalar = (one_element == 1 ? 1 : 2) | 4;
         }
         if constexpr (VB == 4 || VB == 2) {
             const uint64_t groups = (kp.inner + 127) / 128;
@@ -2011,8 +2035,8 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
                 const bool nt = stream_past_caches(kp.inner * sizeof(A) * (uint64_t)(nops - 1));
                 CUMO_BIT_DIGIT* dst = reinterpret_cast<CUMO_BIT_DIGIT*>(const_cast<char*>(ops[nops - 1].ptr)) + out_bit->pos / 32;
                 const dim3 g((unsigned)blocks);
-                if (nt) hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], dst, kp.inner, use_scalar, op, sv);
-                else hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], dst, kp.inner, use_scalar, op, sv);
+                if (nt) hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, true>), g, b, 0, stream, flat_px, flat_py, dst, kp.inner, flat_scalar, op, sv);
+                else hipLaunchKernelGGL((ew_flat_bit_kernel<Op, VB, false>), g, b, 0, stream, flat_px, flat_py, dst, kp.inner, flat_scalar, op, sv);
                 cumo_cuda_runtime_check_kernel_launch();
                 return;
             }
@@ -2207,12 +2231,27 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
         }
         const bool nt = stream_past_caches(bytes);
 
-        // every operand one contiguous run
+        // every operand one contiguous run -- or one of two inputs an array of a single element (x - x.mean,
+        // x / x.sum): the kernel reads it from memory and goes on as the scalar form does
         bool flat = n == 1;
+        int one_element = -1;   // the slot of such an input
         for (int o = 0; o < nops && flat; ++o) {
             const int sl = slot[o];
             const int64_t es = sl == 0 ? (int64_t)sizeof(A) : (sl == 1 ? (int64_t)sizeof(B) : (int64_t)sizeof(R));
+            if (Op::NIN == 2 && std::is_same<A, B>::value && std::is_same<typename Op::S, A>::value && use_scalar == 0 && sl != 2 &&
+                plan.step[o][0] == 0 && one_element < 0 && ((uintptr_t)ops[o].ptr % sizeof(A)) == 0) {
+                one_element = sl;
+                continue;
+            }
             flat = plan.step[o][0] == es;
+        }
+        const char* flat_px = kp.ptr[0];
+        const char* flat_py = kp.ptr[1];
+        int flat_scalar = use_scalar;
+        if (flat && one_element >= 0) {
+            flat_px = kp.ptr[1 - one_element];   // the array
+            flat_py = kp.ptr[one_element];       // the element that stands for the scalar
+            flat_scalar = (one_element == 1 ? 1 : 2) | 4;
         }
         // A result wider than the input (SFloat or Int32 -> DFloat): two elements per lane, so that a lane
         // stores one 128-bit vector and a wave one contiguous KiB, rather than two vectors 32 bytes apart
@@ -2225,11 +2264,11 @@ static void ew_launch(Op op, const cumo_na_iarray_t* in1, const cumo_na_iarray_t
             const uint64_t looping = (uint64_t)ew_table_op_blocks();
             const dim3 g((unsigned)((op_fills_tables<Op>::value && blocks > looping) ? looping : blocks));
             if (fvec == 4) {
-                if (nt) hipLaunchKernelGGL((ew_flat_kernel<Op, 4, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
-                else hipLaunchKernelGGL((ew_flat_kernel<Op, 4, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
+                if (nt) hipLaunchKernelGGL((ew_flat_kernel<Op, 4, true>), g, b, 0, stream, flat_px, flat_py, kp.ptr[2], kp.inner, flat_scalar, flag, op, sv);
+                else hipLaunchKernelGGL((ew_flat_kernel<Op, 4, false>), g, b, 0, stream, flat_px, flat_py, kp.ptr[2], kp.inner, flat_scalar, flag, op, sv);
             } else {
-                if (nt) hipLaunchKernelGGL((ew_flat_kernel<Op, 2, true>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
-                else hipLaunchKernelGGL((ew_flat_kernel<Op, 2, false>), g, b, 0, stream, kp.ptr[0], kp.ptr[1], kp.ptr[2], kp.inner, use_scalar, flag, op, sv);
+                if (nt) hipLaunchKernelGGL((ew_flat_kernel<Op, 2, true>), g, b, 0, stream, flat_px, flat_py, kp.ptr[2], kp.inner, flat_scalar, flag, op, sv);
+                else hipLaunchKernelGGL((ew_flat_kernel<Op, 2, false>), g, b, 0, stream, flat_px, flat_py, kp.ptr[2], kp.inner, flat_scalar, flag, op, sv);
             }
             cumo_cuda_runtime_check_kernel_launch();
             return;

@@ -604,6 +604,53 @@ def test_casts_and_copies(src, dst):
         assert r.type_name == (src if rank[src] > rank[dst] else dst)
 
 
+@pytest.mark.parametrize("tname,dt", FLOATS + [("int32", np.int32)])
+def test_an_operand_that_is_an_array_of_one_element(tname, dt):
+    """x - x.mean, x / x.sum, m - x, x.eq(x.max): an array of a single element (of no dimension or of size one) on either
+    side of a contiguous array is read by the kernel as the scalar form's number is; the bits of the broadcast."""
+    cls = cls_of(tname)
+    rng = np.random.default_rng(641)
+    for shape in [(1,), (5,), (4096,), (4099,), (37, 65), (3, 5, 128), ((1 << 20) + 3,), (1024, 4096)]:
+        if dt == np.int32:
+            hx = rng.integers(-1000, 1000, size=shape).astype(dt)
+            hx[hx == 0] = 5
+        else:
+            hx = (rng.standard_normal(shape) * 8).astype(dt)
+            hx[hx == 0] = 5
+        x = cls.cast(hx)
+        ones = [(x.max(), hx.max()), (cls.cast(np.array([3], dtype=dt)), dt(3)), (cls.cast(np.array([[-7]], dtype=dt)).reshape(*([1] * len(shape))), dt(-7))]
+        for m, hm in ones:
+            hmv = np.full(shape, hm, dtype=dt)
+            for op in ("add", "sub", "mul", "div"):
+                got = getattr(x, PYOP[op])(m)
+                assert tuple(got.shape) == tuple(shape), (op, shape)
+                assert_bits_equal(got.to_numpy(), oracle.binary(op, hx, hmv), (op, shape, "element on the right"))
+                got = getattr(m, PYOP[op])(x)
+                assert tuple(got.shape) == tuple(shape), (op, shape)
+                assert_bits_equal(got.to_numpy(), oracle.binary(op, hmv, hx), (op, shape, "element on the left"))
+            for op in ("eq", "gt", "le"):
+                assert (getattr(x, op)(m).to_numpy() == oracle.compare(op, hx, hmv)).all(), (op, shape)
+                assert (getattr(m, op)(x).to_numpy() == oracle.compare(op, hmv, hx)).all(), (op, shape, "left")
+        if dt != np.int32:
+            import cumo_amd
+            m = cls.cast(np.array([2.5], dtype=dt))
+            assert_ulp((x.abs() ** m).to_numpy(), oracle.binary("pow", np.abs(hx), np.full(shape, 2.5, dtype=dt)), 2)
+            assert_bits_equal(cls.maximum(x, m).to_numpy(), np.maximum(hx, dt(2.5)))
+    # views of the array keep their own paths and answer the same
+    hx = (rng.integers(-50, 50, size=(130, 260))).astype(dt)
+    hx[hx == 0] = 5
+    x = cls.cast(hx)
+    m = x.max()
+    for dv, hv in ((x[:, 1:], hx[:, 1:]), (x.transpose(), hx.T), (x[::2, ::3], hx[::2, ::3])):
+        hv = np.ascontiguousarray(hv)
+        assert_bits_equal((dv - m).to_numpy(), oracle.binary("sub", hv, np.full(hv.shape, hx.max(), dtype=dt)))
+        assert_bits_equal((m - dv).to_numpy(), oracle.binary("sub", np.full(hv.shape, hx.max(), dtype=dt), hv))
+    if dt == np.int32:
+        import cumo_amd
+        with pytest.raises(ZeroDivisionError):
+            x / cls.cast(np.array([0], dtype=dt))
+
+
 MIXED_PAIRS = [("sfloat", "dfloat"), ("dfloat", "sfloat"), ("int32", "sfloat"), ("sfloat", "int32"), ("int32", "dfloat"), ("dfloat", "int32")]
 
 
